@@ -1,0 +1,240 @@
+"""CPU oracle for the quantized-inference path -- TEST INFRASTRUCTURE ONLY.
+
+ctypes front end of ``oracle/liboracle.so`` (built from ``quant_oracle.c`` by
+``make -C oracle``).  Only tests, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import this module; the product
+(``torch_musa_amd``) never does.
+
+All arrays are numpy, C-contiguous.  Quantized values travel as ``uint8``
+(``is_signed=False``) or ``int8`` (``is_signed=True``) arrays.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile liboracle.so with gcc (a no-op when it is already there)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE] + (["-B"] if force else []),
+                              stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.orc_max_threads.restype = C.c_int
+        _lib.orc_choose_qparams.restype = C.c_int
+    return _lib
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _qdtype(is_signed: bool):
+    return np.int8 if is_signed else np.uint8
+
+
+def _as_bytes(q: np.ndarray) -> np.ndarray:
+    q = np.ascontiguousarray(q)
+    assert q.dtype in (np.uint8, np.int8), q.dtype
+    return q
+
+
+def max_threads() -> int:
+    return int(lib().orc_max_threads())
+
+
+def quantize_per_tensor(x, scale, zp, is_signed=False, nthreads=1):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    q = np.empty(x.shape, dtype=_qdtype(is_signed))
+    lib().orc_quantize_per_tensor(_p(x), C.c_int64(x.size), C.c_double(scale),
+                                  C.c_int64(zp), C.c_int(is_signed), _p(q),
+                                  C.c_int(nthreads))
+    return q
+
+
+def dequantize_per_tensor(q, scale, zp, nthreads=1):
+    q = _as_bytes(q)
+    r = np.empty(q.shape, dtype=np.float32)
+    lib().orc_dequantize_per_tensor(_p(q), C.c_int64(q.size), C.c_double(scale),
+                                    C.c_int64(zp), C.c_int(q.dtype == np.int8),
+                                    _p(r), C.c_int(nthreads))
+    return r
+
+
+def _outer_c_inner(shape, axis):
+    axis = axis % len(shape)
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    return outer, int(shape[axis]), inner
+
+
+def quantize_per_channel(x, scales, zps, axis, is_signed=False):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    scales = np.ascontiguousarray(scales, dtype=np.float64)
+    zps = np.ascontiguousarray(zps, dtype=np.int64)
+    outer, c, inner = _outer_c_inner(x.shape, axis)
+    assert scales.size == c and zps.size == c
+    q = np.empty(x.shape, dtype=_qdtype(is_signed))
+    lib().orc_quantize_per_channel(_p(x), C.c_int64(outer), C.c_int64(c),
+                                   C.c_int64(inner), _p(scales), _p(zps),
+                                   C.c_int(is_signed), _p(q))
+    return q
+
+
+def dequantize_per_channel(q, scales, zps, axis):
+    q = _as_bytes(q)
+    scales = np.ascontiguousarray(scales, dtype=np.float64)
+    zps = np.ascontiguousarray(zps, dtype=np.int64)
+    outer, c, inner = _outer_c_inner(q.shape, axis)
+    r = np.empty(q.shape, dtype=np.float32)
+    lib().orc_dequantize_per_channel(_p(q), C.c_int64(outer), C.c_int64(c),
+                                     C.c_int64(inner), _p(scales), _p(zps),
+                                     C.c_int(q.dtype == np.int8), _p(r))
+    return r
+
+
+def minmax(x, nthreads=1):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    mn, mx = C.c_float(), C.c_float()
+    lib().orc_minmax(_p(x), C.c_int64(x.size), C.byref(mn), C.byref(mx),
+                     C.c_int(nthreads))
+    return float(mn.value), float(mx.value)
+
+
+def choose_qparams(mn, mx, is_signed=False, reduce_range=False):
+    """-> (scale: float (double precision), zero_point: int)."""
+    qmin, qmax = (-128, 127) if is_signed else (0, 255)
+    s, z = C.c_double(), C.c_int32()
+    rc = lib().orc_choose_qparams(C.c_float(mn), C.c_float(mx), C.c_int32(qmin),
+                                  C.c_int32(qmax), C.c_int(reduce_range),
+                                  C.byref(s), C.byref(z))
+    if rc != 0:
+        raise ValueError("min must be <= max")
+    return float(s.value), int(z.value)
+
+
+def linear_acc32(xq, wq, nthreads=1):
+    xq = _as_bytes(xq)
+    wq = np.ascontiguousarray(wq, dtype=np.int8)
+    m, k = xq.shape
+    n, k2 = wq.shape
+    assert k == k2
+    acc = np.empty((m, n), dtype=np.int32)
+    lib().orc_linear_acc32(_p(xq), C.c_int(xq.dtype == np.int8), _p(wq),
+                           C.c_int64(m), C.c_int64(n), C.c_int64(k), _p(acc),
+                           C.c_int(nthreads))
+    return acc
+
+
+def weight_colsum(wq):
+    wq = np.ascontiguousarray(wq, dtype=np.int8)
+    n = wq.shape[0]
+    k = wq.size // n
+    out = np.empty(n, dtype=np.int32)
+    lib().orc_weight_colsum(_p(wq), C.c_int64(n), C.c_int64(k), _p(out))
+    return out
+
+
+def requantize(acc, colsum, x_zp, x_scale, w_scales, bias, out_scale, out_zp,
+               out_signed=False, relu=False):
+    acc = np.ascontiguousarray(acc, dtype=np.int32)
+    m, n = acc.shape
+    colsum = np.ascontiguousarray(colsum, dtype=np.int32)
+    w_scales = np.ascontiguousarray(np.atleast_1d(w_scales), dtype=np.float64)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    y = np.empty((m, n), dtype=_qdtype(out_signed))
+    lib().orc_requantize(_p(acc), C.c_int64(m), C.c_int64(n), _p(colsum),
+                         C.c_int64(x_zp), C.c_double(x_scale), _p(w_scales),
+                         C.c_int64(w_scales.size), _p(b) if b is not None else None,
+                         C.c_double(out_scale), C.c_int64(out_zp),
+                         C.c_int(out_signed), C.c_int(relu), _p(y))
+    return y
+
+
+def linear(xq, x_scale, x_zp, wq, w_scales, bias, out_scale, out_zp,
+           out_signed=None, relu=False, nthreads=1):
+    """quantized::linear on 2-D ``xq`` [M,K] and ``wq`` [N,K] (zero point 0)."""
+    xq = _as_bytes(xq)
+    wq = np.ascontiguousarray(wq, dtype=np.int8)
+    if out_signed is None:
+        out_signed = xq.dtype == np.int8
+    m, k = xq.shape
+    n = wq.shape[0]
+    w_scales = np.ascontiguousarray(np.atleast_1d(w_scales), dtype=np.float64)
+    assert w_scales.size in (1, n)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    y = np.empty((m, n), dtype=_qdtype(out_signed))
+    lib().orc_linear(_p(xq), C.c_int(xq.dtype == np.int8), _p(wq), C.c_int64(m),
+                     C.c_int64(n), C.c_int64(k), C.c_int64(x_zp),
+                     C.c_double(x_scale), _p(w_scales), C.c_int64(w_scales.size),
+                     _p(b) if b is not None else None, C.c_double(out_scale),
+                     C.c_int64(out_zp), C.c_int(out_signed), C.c_int(relu), _p(y),
+                     C.c_int(nthreads))
+    return y
+
+
+def conv_out_hw(h, w, kh, kw, stride, padding, dilation):
+    oh = (h + 2 * padding[0] - dilation[0] * (kh - 1) - 1) // stride[0] + 1
+    ow = (w + 2 * padding[1] - dilation[1] * (kw - 1) - 1) // stride[1] + 1
+    return oh, ow
+
+
+def conv2d_acc32(x_nhwc, w_ohwi, stride, padding, dilation, groups, x_zp,
+                 nthreads=1):
+    x = _as_bytes(x_nhwc)
+    w = np.ascontiguousarray(w_ohwi, dtype=np.int8)
+    b, h, wd, ic = x.shape
+    oc, kh, kw, icg = w.shape
+    assert icg * groups == ic and oc % groups == 0
+    oh, ow = conv_out_hw(h, wd, kh, kw, stride, padding, dilation)
+    acc = np.empty((b, oh, ow, oc), dtype=np.int32)
+    lib().orc_conv2d_acc32(_p(x), C.c_int(x.dtype == np.int8), _p(w),
+                           *[C.c_int64(v) for v in (b, h, wd, ic, oc, kh, kw,
+                                                    stride[0], stride[1],
+                                                    padding[0], padding[1],
+                                                    dilation[0], dilation[1],
+                                                    groups, x_zp)],
+                           _p(acc), C.c_int(nthreads))
+    return acc
+
+
+def conv2d(x_nhwc, x_scale, x_zp, w_ohwi, w_scales, bias, stride, padding,
+           dilation, groups, out_scale, out_zp, out_signed=None, relu=False,
+           nthreads=1):
+    """quantized::conv2d on NHWC ``x`` and OHWI ``w``; returns NHWC bytes."""
+    x = _as_bytes(x_nhwc)
+    w = np.ascontiguousarray(w_ohwi, dtype=np.int8)
+    if out_signed is None:
+        out_signed = x.dtype == np.int8
+    b, h, wd, ic = x.shape
+    oc, kh, kw, icg = w.shape
+    assert icg * groups == ic and oc % groups == 0
+    oh, ow = conv_out_hw(h, wd, kh, kw, stride, padding, dilation)
+    w_scales = np.ascontiguousarray(np.atleast_1d(w_scales), dtype=np.float64)
+    assert w_scales.size in (1, oc)
+    bb = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    y = np.empty((b, oh, ow, oc), dtype=_qdtype(out_signed))
+    lib().orc_conv2d(_p(x), C.c_int(x.dtype == np.int8), _p(w),
+                     *[C.c_int64(v) for v in (b, h, wd, ic, oc, kh, kw,
+                                              stride[0], stride[1], padding[0],
+                                              padding[1], dilation[0],
+                                              dilation[1], groups, x_zp)],
+                     C.c_double(x_scale), _p(w_scales), C.c_int64(w_scales.size),
+                     _p(bb) if bb is not None else None, C.c_double(out_scale),
+                     C.c_int64(out_zp), C.c_int(out_signed), C.c_int(relu), _p(y),
+                     C.c_int(nthreads))
+    return y

@@ -1,0 +1,225 @@
+"""Seeded test cases shared by the golden-vector generator and the tests.
+
+Every input is rebuilt from a numpy seed, so fixtures only have to hold the
+expected outputs (plus a CRC of each rebuilt input, so a change in numpy's
+random stream is reported as such and not as a parity failure).
+
+Shapes, scales and zero points replay the reference's own quantized tests:
+  tests/unittest/quantized/test_quantized_ops.py:25-99   (quantize cases)
+  tests/unittest/quantized/test_quantized_linear.py:14-49 (linear shapes)
+  tests/unittest/quantized/test_quantized_conv.py:14-80   (conv configs)
+plus the C1 parity configuration (x [128,1024], W [1024,1024] per channel,
+bias, output scale 0.05 / zero point 128) and adversarial cases the reference
+leaves out (exact ties, tail lengths, extreme zero points, clamping).
+"""
+from __future__ import annotations
+
+import zlib
+
+import numpy as np
+
+
+def crc(a: np.ndarray) -> int:
+    return zlib.crc32(np.ascontiguousarray(a).tobytes()) & 0xFFFFFFFF
+
+
+def randn(seed: int, shape, std: float = 1.0) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+
+def absmax_scale(x: np.ndarray, div: float = 128.0) -> float:
+    # float(x.abs().max() / 2**7) as in the reference tests: an fp32 division
+    return float(np.float32(np.abs(x).max()) / np.float32(div))
+
+
+# --------------------------------------------------------------------------
+# per-tensor quantize / dequantize
+# --------------------------------------------------------------------------
+def quantize_per_tensor_cases():
+    """-> list of dict(name, x, scale, zp, signed)."""
+    out = []
+    for i, shape in enumerate([(2, 3, 4), (2, 3, 4, 5), (2, 16, 32, 32)]):
+        x = randn(100 + i, shape)
+        for signed in (False, True):
+            out.append(dict(name=f"ref_shape{i}_{'s8' if signed else 'u8'}", x=x,
+                            scale=absmax_scale(x), zp=0 if signed else 128,
+                            signed=signed))
+    # exact ties: x = (k + 0.5) * scale with a power-of-two scale
+    k = np.arange(-300, 300, dtype=np.float32)
+    for signed in (False, True):
+        out.append(dict(name=f"ties_{'s8' if signed else 'u8'}",
+                        x=((k + np.float32(0.5)) * np.float32(0.25)).astype(np.float32),
+                        scale=0.25, zp=-3 if signed else 7, signed=signed))
+    # the fbgemm comment's example where x*inv and x/scale differ
+    out.append(dict(name="inv_vs_div", x=np.array([0.273939937], dtype=np.float32),
+                    scale=float(np.float32(0.00214854861)), zp=0, signed=False))
+    # tail lengths around vector widths
+    for n in list(range(1, 20)) + [63, 64, 65, 255, 256, 257, 1023, 1025, 4095,
+                                   4096, 4097, 4098, 4099]:
+        x = randn(1000 + n, (n,), std=3.0)
+        out.append(dict(name=f"tail_{n}", x=x, scale=0.05, zp=100, signed=False))
+    # clamping at both ends and extreme zero points
+    x = randn(77, (4099,), std=40.0)
+    out.append(dict(name="clamp_u8_zp0", x=x, scale=0.1, zp=0, signed=False))
+    out.append(dict(name="clamp_u8_zp255", x=x, scale=0.1, zp=255, signed=False))
+    out.append(dict(name="clamp_s8_zpm128", x=x, scale=0.1, zp=-128, signed=True))
+    out.append(dict(name="clamp_s8_zp127", x=x, scale=0.1, zp=127, signed=True))
+    # scale that is not exactly representable + large magnitudes
+    x = randn(78, (3001,), std=1000.0)
+    out.append(dict(name="big_values", x=x, scale=7.3, zp=13, signed=False))
+    return out
+
+
+def dynamic_qparams_cases():
+    """(min, max) pairs for ChooseQuantizationParams, each x reduce_range."""
+    pairs = [(-1.0, 1.0), (0.0, 6.0), (-5.0, 0.0), (0.5, 3.0), (-3.0, -0.5),
+             (0.0, 0.0), (-1e-9, 1e-9), (-1e-4, 3e-4), (0.0, 1e-3), (-2e-3, 0.0),
+             (-50.0, 50.0), (-49.71, 50.33), (-3.4e37, 3.4e37), (-0.1, 25.4),
+             (-12.7, 12.8), (-1.0, 254.0), (-1e-7, 2.0)]
+    for i in range(12):
+        x = randn(300 + i, (64,), std=10.0 ** (i % 4 - 1))
+        pairs.append((float(x.min()), float(x.max())))
+    return [(np.float32(a), np.float32(b)) for a, b in pairs]
+
+
+def dynamic_tensor_cases():
+    out = []
+    for i, shape in enumerate([(2, 3, 4), (2, 3, 4, 5), (2, 16, 32, 32)]):
+        out.append(dict(name=f"dyn_shape{i}", x=randn(200 + i, shape)))
+    x = randn(210, (70001,), std=3.0)
+    x[::101] = 50.0
+    x[7::103] = -50.0
+    out.append(dict(name="dyn_outliers", x=x))
+    out.append(dict(name="dyn_positive", x=np.abs(randn(211, (1000,))) + np.float32(0.5)))
+    return out
+
+
+# --------------------------------------------------------------------------
+# per-channel quantize / dequantize
+# --------------------------------------------------------------------------
+def quantize_per_channel_cases():
+    out = []
+    out.append(dict(name="ref_2x3_axis0", x=randn(400, (2, 3)),
+                    scales=np.array([0.1, 0.01]), zps=np.array([10, 1]), axis=0,
+                    signed=False))
+    out.append(dict(name="ref_5d_axis3", x=randn(401, (2, 3, 4, 5, 6)),
+                    scales=np.array([0.1] * 5), zps=np.array([1] * 5), axis=3,
+                    signed=False))
+    x = randn(402, (37, 19), std=0.02)
+    s = (np.abs(x).max(axis=1) / 127.0).astype(np.float64)
+    out.append(dict(name="weight_axis0_s8", x=x, scales=s, zps=np.zeros(37, np.int64),
+                    axis=0, signed=True))
+    x = randn(403, (4, 6, 5, 3))
+    out.append(dict(name="axis1_u8", x=x,
+                    scales=np.array([0.013, 0.1, 0.5, 0.02, 0.3, 0.07]),
+                    zps=np.array([0, 255, 128, 3, 77, 200]), axis=1, signed=False))
+    out.append(dict(name="last_axis_s8", x=x, scales=np.array([0.011, 0.2, 0.05]),
+                    zps=np.array([-128, 127, 0]), axis=3, signed=True))
+    # float64 scales that are not fp32-representable (pins the double multiply
+    # in per-channel dequantize)
+    x = randn(404, (8, 301))
+    out.append(dict(name="double_scales", x=x,
+                    scales=np.array([0.1, 1 / 3, 0.0123456789, 2 / 7, 0.7, 0.05,
+                                     1e-2 / 3, 0.9]),
+                    zps=np.array([1, 2, 3, 4, 5, 6, 7, 8]), axis=0, signed=False))
+    return out
+
+
+# --------------------------------------------------------------------------
+# quantized::linear
+# --------------------------------------------------------------------------
+def _int_inputs(seed, m, n, k, x_signed):
+    rng = np.random.default_rng(seed)
+    if x_signed:
+        xq = rng.integers(-128, 128, size=(m, k), dtype=np.int8)
+    else:
+        xq = rng.integers(0, 256, size=(m, k), dtype=np.uint8)
+    wq = rng.integers(-127, 128, size=(n, k), dtype=np.int8)
+    bias = (rng.standard_normal(n, dtype=np.float32)).astype(np.float32)
+    return xq, wq, bias
+
+
+def linear_cases():
+    """Integer-domain cases: list of dict(name, xq, wq, bias, x_scale, x_zp,
+    w_scales, out_scale, out_zp, relu). Weight zero points are 0."""
+    out = []
+    spec = [
+        # name, M, N, K, per_channel, bias, relu, x_zp
+        ("ref_8x128_512", 8, 512, 128, False, False, False, 128),
+        ("ref_8x128_512_relu", 8, 512, 128, False, False, True, 128),
+        ("ref_80x128_512", 80, 512, 128, False, False, False, 120),
+        ("pc_bias", 33, 70, 96, True, True, False, 131),
+        ("pc_bias_relu", 33, 70, 96, True, True, True, 0),
+        ("pt_bias", 17, 40, 64, False, True, False, 255),
+        ("odd_k", 5, 9, 37, True, True, False, 17),
+        ("one_row", 1, 256, 512, True, True, False, 127),
+        ("wide", 3, 1031, 48, True, False, False, 64),
+    ]
+    for i, (name, m, n, k, pc, has_bias, relu, x_zp) in enumerate(spec):
+        xq, wq, bias = _int_inputs(500 + i, m, n, k, False)
+        rng = np.random.default_rng(900 + i)
+        x_scale = float(np.float32(0.02 + 0.01 * i))
+        if pc:
+            w_scales = (0.001 + 0.002 * rng.random(n)).astype(np.float32).astype(np.float64)
+        else:
+            w_scales = np.array([float(np.float32(0.0031))])
+        # output scale so that roughly +-3 sigma of the result spans the range
+        sigma = np.sqrt(k) * 74.0 * 74.0 * x_scale * float(np.mean(w_scales))
+        out_scale = float(np.float32(3.0 * sigma / 128.0))
+        out.append(dict(name=name, xq=xq, wq=wq, bias=bias * np.float32(sigma) if has_bias else None,
+                        x_scale=x_scale, x_zp=x_zp, w_scales=w_scales,
+                        out_scale=out_scale, out_zp=128 if not relu else 10,
+                        relu=relu))
+    return out
+
+
+def c1_case():
+    """BASELINE config 1: x fp32 [128,1024] ~N(0,1) -> dynamic quint8;
+    W fp32 [1024,1024] ~N(0,0.02) -> per-channel symmetric qint8
+    (scale_c = absmax_c / 127); bias fp32 [1024]; out scale 0.05, zp 128."""
+    x = randn(41, (128, 1024))
+    w = randn(42, (1024, 1024), std=0.02)
+    bias = randn(43, (1024,))
+    w_scales = (np.abs(w).max(axis=1).astype(np.float32) / np.float32(127.0)).astype(np.float64)
+    return dict(x=x, w=w, bias=bias, w_scales=w_scales, out_scale=0.05, out_zp=128)
+
+
+# --------------------------------------------------------------------------
+# quantized::conv2d  (logical NCHW shapes; tensors are built NHWC / OHWI)
+# --------------------------------------------------------------------------
+def conv_cases():
+    spec = [
+        # name, B, IC, H, W, OC, k, stride, pad, dil, groups, bias, relu, per_channel
+        ("ref_32to64_k3", 2, 32, 16, 16, 64, 3, 1, 1, 1, 1, False, False, False),
+        ("ref_32to64_k3_relu", 2, 32, 16, 16, 64, 3, 1, 1, 1, 1, False, True, False),
+        ("ref_3to32_k3s2_bias_relu", 2, 3, 16, 16, 32, 3, 2, 1, 1, 1, True, True, False),
+        ("ref_64to32_g32_relu", 2, 64, 16, 16, 32, 3, 2, 1, 1, 32, False, True, False),
+        ("ref_3to32_k7s2p3_bias", 8, 3, 32, 32, 32, 7, 2, 3, 1, 1, True, False, False),
+        ("pc_64to64_k3_bias", 2, 64, 14, 14, 64, 3, 1, 1, 1, 1, True, False, True),
+        ("pc_16to48_k1", 3, 16, 9, 11, 48, 1, 1, 0, 1, 1, True, False, True),
+        ("pc_32to32_k3_dil2", 1, 32, 13, 13, 32, 3, 1, 2, 2, 1, True, True, True),
+        ("pc_groups2", 2, 32, 10, 10, 64, 3, 1, 1, 1, 2, True, False, True),
+    ]
+    out = []
+    for i, (name, b, ic, h, w, oc, k, s, p, d, g, has_bias, relu, pc) in enumerate(spec):
+        rng = np.random.default_rng(700 + i)
+        x_zp = int(rng.integers(0, 200))
+        xq = rng.integers(0, 256, size=(b, h, w, ic), dtype=np.uint8)
+        wq = rng.integers(-127, 128, size=(oc, k, k, ic // g), dtype=np.int8)
+        bias = rng.standard_normal(oc, dtype=np.float32)
+        x_scale = float(np.float32(0.03))
+        if pc:
+            w_scales = (0.001 + 0.002 * rng.random(oc)).astype(np.float32).astype(np.float64)
+        else:
+            w_scales = np.array([float(np.float32(0.0027))])
+        kk = k * k * (ic // g)
+        sigma = np.sqrt(kk) * 74.0 * 74.0 * x_scale * float(np.mean(w_scales))
+        out_scale = float(np.float32(3.0 * sigma / 128.0))
+        out.append(dict(name=name, xq=xq, wq=wq,
+                        bias=bias * np.float32(sigma) if has_bias else None,
+                        x_scale=x_scale, x_zp=x_zp, w_scales=w_scales,
+                        stride=(s, s), padding=(p, p), dilation=(d, d), groups=g,
+                        out_scale=out_scale, out_zp=128 if not relu else 5,
+                        relu=relu))
+    return out

@@ -1,0 +1,157 @@
+"""Writes tests/golden/golden.npz: expected outputs of PyTorch's CPU quantized
+ops (engine 'fbgemm') for the seeded cases in tests/cases.py.
+
+PyTorch's CPU ops are the numerics the reference's own tests compare against
+(torch_musa/testing/base_test_tool.py:814-825); they are a third-party
+dependency of the reference, not part of it, and are installed here.  Nothing
+from the reference tree is imported or executed.
+
+Run from the repo root:   python tests/golden/make_golden.py
+The fixture holds only outputs, scalars and CRCs of the rebuilt inputs.
+"""
+from __future__ import annotations
+
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+import cases  # noqa: E402
+
+
+def qdtype(signed):
+    return torch.qint8 if signed else torch.quint8
+
+
+def put_dq(g, k, dq):
+    """Dequantized values must match exactly, so a CRC pins them; small arrays
+    are also kept in full to make a mismatch readable."""
+    g[k + "/dq_crc"] = np.uint32(cases.crc(dq))
+    if dq.size <= 2048:
+        g[k + "/dq"] = dq
+
+
+def main():
+    torch.backends.quantized.engine = "fbgemm"
+    torch.set_num_threads(4)
+    g = {}
+    meta = {"torch": torch.__version__, "engine": torch.backends.quantized.engine}
+
+    # ---- per-tensor quantize / dequantize --------------------------------
+    for c in cases.quantize_per_tensor_cases():
+        x = torch.from_numpy(c["x"])
+        q = torch.quantize_per_tensor(x, c["scale"], c["zp"], qdtype(c["signed"]))
+        k = "qpt/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/q"] = q.int_repr().numpy()
+        put_dq(g, k, q.dequantize().numpy())
+
+    # ---- dynamic qparams -------------------------------------------------
+    pairs = cases.dynamic_qparams_cases()
+    res = []
+    for mn, mx in pairs:
+        for rr in (False, True):
+            x = torch.tensor([mn, mx], dtype=torch.float32)
+            s, z = torch._choose_qparams_per_tensor(x, rr)
+            res.append((float(mn), float(mx), float(rr), float(s), float(z)))
+    g["dynq/pairs"] = np.array(res, dtype=np.float64)
+    for c in cases.dynamic_tensor_cases():
+        x = torch.from_numpy(c["x"])
+        for rr in (False, True):
+            q = torch.quantize_per_tensor_dynamic(x, torch.quint8, rr)
+            k = f"dyn/{c['name']}/rr{int(rr)}"
+            g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+            g[k + "/scale"] = np.float64(q.q_scale())
+            g[k + "/zp"] = np.int64(q.q_zero_point())
+            g[k + "/q"] = q.int_repr().numpy()
+
+    # ---- per-channel -----------------------------------------------------
+    for c in cases.quantize_per_channel_cases():
+        x = torch.from_numpy(c["x"])
+        q = torch.quantize_per_channel(x, torch.from_numpy(c["scales"].astype(np.float64)),
+                                       torch.from_numpy(c["zps"].astype(np.int64)),
+                                       c["axis"], qdtype(c["signed"]))
+        k = "qpc/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/q"] = q.int_repr().numpy()
+        put_dq(g, k, q.dequantize().numpy())
+
+    # ---- quantized::linear (integer-domain cases) ------------------------
+    def make_w(wq, w_scales, axis_len):
+        wt = torch.from_numpy(wq)
+        if len(w_scales) == 1:
+            return torch._make_per_tensor_quantized_tensor(wt, float(w_scales[0]), 0)
+        return torch._make_per_channel_quantized_tensor(
+            wt, torch.from_numpy(w_scales.astype(np.float64)),
+            torch.zeros(axis_len, dtype=torch.int64), 0)
+
+    for c in cases.linear_cases():
+        xq = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["xq"]),
+                                                     c["x_scale"], c["x_zp"])
+        w = make_w(c["wq"], c["w_scales"], c["wq"].shape[0])
+        b = None if c["bias"] is None else torch.from_numpy(c["bias"])
+        packed = torch.ops.quantized.linear_prepack(w, b)
+        op = torch.ops.quantized.linear_relu if c["relu"] else torch.ops.quantized.linear
+        y = op(xq, packed, c["out_scale"], c["out_zp"])
+        k = "lin/" + c["name"]
+        g[k + "/xq_crc"] = np.uint32(cases.crc(c["xq"]))
+        g[k + "/wq_crc"] = np.uint32(cases.crc(c["wq"]))
+        g[k + "/out_scale"] = np.float64(c["out_scale"])
+        g[k + "/y"] = y.int_repr().numpy()
+
+    # ---- C1 ---------------------------------------------------------------
+    c1 = cases.c1_case()
+    x = torch.from_numpy(c1["x"])
+    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+    wq = torch.quantize_per_channel(torch.from_numpy(c1["w"]),
+                                    torch.from_numpy(c1["w_scales"]),
+                                    torch.zeros(1024, dtype=torch.int64), 0, torch.qint8)
+    packed = torch.ops.quantized.linear_prepack(wq, torch.from_numpy(c1["bias"]))
+    y = torch.ops.quantized.linear(xq, packed, c1["out_scale"], c1["out_zp"])
+    g["c1/x_crc"] = np.uint32(cases.crc(c1["x"]))
+    g["c1/w_crc"] = np.uint32(cases.crc(c1["w"]))
+    g["c1/x_scale"] = np.float64(xq.q_scale())
+    g["c1/x_zp"] = np.int64(xq.q_zero_point())
+    g["c1/xq_crc"] = np.uint32(cases.crc(xq.int_repr().numpy()))
+    g["c1/wq_crc"] = np.uint32(cases.crc(wq.int_repr().numpy()))
+    g["c1/y"] = y.int_repr().numpy()
+    g["c1/y_dq_crc"] = np.uint32(cases.crc(y.dequantize().numpy()))
+    # engines agree on C1 (recorded, so a later engine drift is visible)
+    for eng in ("x86", "onednn"):
+        if eng in torch.backends.quantized.supported_engines:
+            torch.backends.quantized.engine = eng
+            p2 = torch.ops.quantized.linear_prepack(wq, torch.from_numpy(c1["bias"]))
+            y2 = torch.ops.quantized.linear(xq, p2, c1["out_scale"], c1["out_zp"])
+            meta[f"c1_mismatch_{eng}"] = int((y2.int_repr() != y.int_repr()).sum())
+    torch.backends.quantized.engine = "fbgemm"
+
+    # ---- quantized::conv2d -------------------------------------------------
+    for c in cases.conv_cases():
+        x_nchw = torch.from_numpy(c["xq"]).permute(0, 3, 1, 2)  # channels-last view
+        xq = torch._make_per_tensor_quantized_tensor(x_nchw, c["x_scale"], c["x_zp"])
+        w_oihw = torch.from_numpy(c["wq"]).permute(0, 3, 1, 2).contiguous()
+        w = make_w(w_oihw.numpy(), c["w_scales"], w_oihw.shape[0])
+        b = None if c["bias"] is None else torch.from_numpy(c["bias"])
+        packed = torch.ops.quantized.conv2d_prepack(w, b, list(c["stride"]),
+                                                    list(c["padding"]),
+                                                    list(c["dilation"]), c["groups"])
+        op = torch.ops.quantized.conv2d_relu if c["relu"] else torch.ops.quantized.conv2d
+        y = op(xq, packed, c["out_scale"], c["out_zp"])
+        k = "conv/" + c["name"]
+        g[k + "/xq_crc"] = np.uint32(cases.crc(c["xq"]))
+        g[k + "/wq_crc"] = np.uint32(cases.crc(c["wq"]))
+        g[k + "/out_scale"] = np.float64(c["out_scale"])
+        # NHWC bytes
+        g[k + "/y"] = y.int_repr().permute(0, 2, 3, 1).contiguous().numpy()
+
+    g["meta"] = np.array(repr(meta))
+    path = os.path.join(HERE, "golden.npz")
+    np.savez_compressed(path, **g)
+    print("wrote", path, os.path.getsize(path), "bytes;", len(g), "arrays;", meta)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,105 @@
+"""The CPU oracle against golden vectors written by PyTorch's CPU quantized ops
+(tests/golden/make_golden.py).  Bit-exact for quantize, dequantize, qparams and
+accumulators; the requantised uint8 of linear/conv must also be exact here
+because the oracle restates fbgemm's scalar output stage and the fixtures were
+produced by its vector one -- a difference would show an order-of-operations
+mistake (the two agree on every element of these cases)."""
+import numpy as np
+import pytest
+
+import cases
+import oracle
+
+
+def _check_crc(golden, key, arr):
+    assert int(golden[key]) == cases.crc(arr), (
+        f"{key}: rebuilt input differs from the one the fixture was made from "
+        "(numpy random stream changed?)")
+
+
+@pytest.mark.parametrize("c", cases.quantize_per_tensor_cases(), ids=lambda c: c["name"])
+def test_quantize_dequantize_per_tensor(golden, c):
+    k = "qpt/" + c["name"]
+    _check_crc(golden, k + "/x_crc", c["x"])
+    q = oracle.quantize_per_tensor(c["x"], c["scale"], c["zp"], c["signed"])
+    np.testing.assert_array_equal(q, golden[k + "/q"])
+    dq = oracle.dequantize_per_tensor(q, c["scale"], c["zp"])
+    assert cases.crc(dq) == int(golden[k + "/dq_crc"])
+    if k + "/dq" in golden:
+        np.testing.assert_array_equal(dq, golden[k + "/dq"])
+
+
+def test_choose_qparams_pairs(golden):
+    rows = golden["dynq/pairs"]
+    assert len(rows) == 2 * len(cases.dynamic_qparams_cases())
+    for mn, mx, rr, s, z in rows:
+        so, zo = oracle.choose_qparams(np.float32(mn), np.float32(mx), False, bool(rr))
+        assert so == s and zo == int(z), (mn, mx, rr, so, s, zo, z)
+
+
+@pytest.mark.parametrize("c", cases.dynamic_tensor_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("rr", [False, True])
+def test_quantize_per_tensor_dynamic(golden, c, rr):
+    k = f"dyn/{c['name']}/rr{int(rr)}"
+    _check_crc(golden, k + "/x_crc", c["x"])
+    mn, mx = oracle.minmax(c["x"])
+    assert mn == float(c["x"].min()) and mx == float(c["x"].max())
+    s, z = oracle.choose_qparams(mn, mx, False, rr)
+    assert s == float(golden[k + "/scale"]) and z == int(golden[k + "/zp"])
+    q = oracle.quantize_per_tensor(c["x"], s, z, False)
+    np.testing.assert_array_equal(q, golden[k + "/q"])
+
+
+@pytest.mark.parametrize("c", cases.quantize_per_channel_cases(), ids=lambda c: c["name"])
+def test_quantize_dequantize_per_channel(golden, c):
+    k = "qpc/" + c["name"]
+    _check_crc(golden, k + "/x_crc", c["x"])
+    q = oracle.quantize_per_channel(c["x"], c["scales"], c["zps"], c["axis"], c["signed"])
+    np.testing.assert_array_equal(q, golden[k + "/q"])
+    dq = oracle.dequantize_per_channel(q, c["scales"], c["zps"], c["axis"])
+    assert cases.crc(dq) == int(golden[k + "/dq_crc"])
+    if k + "/dq" in golden:
+        np.testing.assert_array_equal(dq, golden[k + "/dq"])
+
+
+@pytest.mark.parametrize("c", cases.linear_cases(), ids=lambda c: c["name"])
+def test_linear(golden, c):
+    k = "lin/" + c["name"]
+    _check_crc(golden, k + "/xq_crc", c["xq"])
+    _check_crc(golden, k + "/wq_crc", c["wq"])
+    assert float(golden[k + "/out_scale"]) == c["out_scale"]
+    y = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"],
+                      c["bias"], c["out_scale"], c["out_zp"], relu=c["relu"])
+    want = golden[k + "/y"]
+    assert 0 < np.count_nonzero((want > 0) & (want < 255)), "degenerate case"
+    np.testing.assert_array_equal(y, want)
+
+
+def test_c1(golden):
+    c1 = cases.c1_case()
+    _check_crc(golden, "c1/x_crc", c1["x"])
+    _check_crc(golden, "c1/w_crc", c1["w"])
+    mn, mx = oracle.minmax(c1["x"])
+    s, z = oracle.choose_qparams(mn, mx, False, False)
+    assert s == float(golden["c1/x_scale"]) and z == int(golden["c1/x_zp"])
+    xq = oracle.quantize_per_tensor(c1["x"], s, z, False)
+    assert cases.crc(xq) == int(golden["c1/xq_crc"])
+    wq = oracle.quantize_per_channel(c1["w"], c1["w_scales"], np.zeros(1024, np.int64), 0, True)
+    assert cases.crc(wq) == int(golden["c1/wq_crc"])
+    y = oracle.linear(xq, s, z, wq, c1["w_scales"], c1["bias"], c1["out_scale"], c1["out_zp"])
+    np.testing.assert_array_equal(y, golden["c1/y"])
+    dq = oracle.dequantize_per_tensor(y, c1["out_scale"], c1["out_zp"])
+    assert cases.crc(dq) == int(golden["c1/y_dq_crc"])
+
+
+@pytest.mark.parametrize("c", cases.conv_cases(), ids=lambda c: c["name"])
+def test_conv2d(golden, c):
+    k = "conv/" + c["name"]
+    _check_crc(golden, k + "/xq_crc", c["xq"])
+    _check_crc(golden, k + "/wq_crc", c["wq"])
+    y = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                      c["stride"], c["padding"], c["dilation"], c["groups"],
+                      c["out_scale"], c["out_zp"], relu=c["relu"])
+    want = golden[k + "/y"]
+    assert y.shape == want.shape
+    np.testing.assert_array_equal(y, want)

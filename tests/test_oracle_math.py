@@ -1,0 +1,188 @@
+"""The CPU oracle against what the mathematics fixes, independently of any
+fixture: exact rational rounding, brute force over all codes, exact int64
+matmul, closed-form special cases of the output stage, conv == GEMM on im2col."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+import oracle
+
+
+def _rne(fr: Fraction) -> int:
+    fl = fr.numerator // fr.denominator
+    rem = fr - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        return fl + 1
+    return fl
+
+
+@pytest.mark.parametrize("signed", [False, True])
+def test_quantize_matches_exact_rational_rounding(signed):
+    # power-of-two scale: x*inv is exact in fp32, so the result is RNE of the
+    # exact quotient, shifted and clamped.
+    rng = np.random.default_rng(1)
+    x = (rng.integers(-4000, 4000, size=5000).astype(np.float32) / np.float32(8.0))
+    scale, zp = 0.5, (-5 if signed else 9)
+    q = oracle.quantize_per_tensor(x, scale, zp, signed)
+    lo, hi = (-128, 127) if signed else (0, 255)
+    want = [min(hi, max(lo, _rne(Fraction(float(v)) / Fraction(scale)) + zp)) for v in x]
+    np.testing.assert_array_equal(q.astype(np.int64), np.array(want))
+
+
+def test_ties_round_to_even_not_away():
+    x = np.array([0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5], dtype=np.float32)
+    q = oracle.quantize_per_tensor(x, 1.0, 10, False)
+    np.testing.assert_array_equal(q, np.array([10, 12, 12, 14, 10, 8, 8], dtype=np.uint8))
+
+
+def test_multiply_by_reciprocal_not_divide():
+    # fbgemm's documented example: x*inv gives 127.5 -> 128, x/scale gives 127
+    q = oracle.quantize_per_tensor(np.array([0.273939937], np.float32),
+                                   float(np.float32(0.00214854861)), 0, False)
+    assert int(q[0]) == 128
+
+
+@pytest.mark.parametrize("signed", [False, True])
+def test_dequantize_all_codes_and_roundtrip(signed):
+    codes = np.arange(-128, 128, dtype=np.int8) if signed else np.arange(256, dtype=np.uint8)
+    for scale, zp in [(0.1, 3), (0.0143444, 127 if not signed else -7), (1 / 3, 0)]:
+        r = oracle.dequantize_per_tensor(codes, scale, zp)
+        want = (np.float32(scale) * (codes.astype(np.int32) - zp).astype(np.float32)).astype(np.float32)
+        np.testing.assert_array_equal(r, want)
+        # every code is a fixed point of dequantize -> quantize
+        back = oracle.quantize_per_tensor(r, scale, zp, signed)
+        np.testing.assert_array_equal(back, codes)
+
+
+def test_per_channel_reduces_to_per_tensor():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((5, 7, 3), dtype=np.float32)
+    scales = np.array([0.02, 0.3, 0.011, 0.07, 0.5, 0.09, 0.013])
+    zps = np.array([0, 255, 7, 128, 64, 1, 200])
+    q = oracle.quantize_per_channel(x, scales, zps, 1, False)
+    for c in range(7):
+        np.testing.assert_array_equal(
+            q[:, c, :], oracle.quantize_per_tensor(x[:, c, :], scales[c], zps[c], False))
+    dq = oracle.dequantize_per_channel(q, scales, zps, 1)
+    want = ((q.astype(np.float32) - zps.astype(np.float32)[None, :, None]).astype(np.float64)
+            * scales[None, :, None]).astype(np.float32)
+    np.testing.assert_array_equal(dq, want)
+
+
+def test_choose_qparams_invariants():
+    rng = np.random.default_rng(3)
+    for _ in range(300):
+        a, b = np.sort(rng.standard_normal(2).astype(np.float32) * np.float32(10.0 ** rng.integers(-3, 3)))
+        for rr in (False, True):
+            s, z = oracle.choose_qparams(a, b, False, rr)
+            qmax = 127 if rr else 255
+            assert s > 0 and 0 <= z <= qmax
+            # zero is exactly representable
+            assert oracle.dequantize_per_tensor(np.array([z], np.uint8), s, z)[0] == 0.0
+            # closed form of the scale when no cut-off applies
+            lo, hi = min(float(a), 0.0), max(float(b), 0.0)
+            if (hi - lo) / qmax >= 6.1e-5:
+                assert s == (hi - lo) / qmax
+    assert oracle.choose_qparams(0.0, 0.0)[0] == 0.1  # degenerate range fallback
+    with pytest.raises(ValueError):
+        oracle.choose_qparams(1.0, -1.0)
+
+
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_linear_acc32_is_exact_integer_matmul(x_signed):
+    rng = np.random.default_rng(4)
+    m, n, k = 13, 29, 257
+    x = rng.integers(-128, 128, (m, k), dtype=np.int8) if x_signed else rng.integers(0, 256, (m, k), dtype=np.uint8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc = oracle.linear_acc32(x, w)
+    np.testing.assert_array_equal(acc.astype(np.int64), x.astype(np.int64) @ w.astype(np.int64).T)
+    np.testing.assert_array_equal(oracle.weight_colsum(w), w.astype(np.int64).sum(axis=1))
+    # worst-case magnitudes stay inside int32 for K this small
+    xmax = np.full((1, k), -128 if x_signed else 255, dtype=x.dtype)
+    wmin = np.full((1, k), -128, dtype=np.int8)
+    assert int(oracle.linear_acc32(xmax, wmin)[0, 0]) == int(xmax[0, 0]) * -128 * k
+
+
+def test_requantize_special_cases():
+    rng = np.random.default_rng(5)
+    acc = rng.integers(-400, 400, (6, 9)).astype(np.int32)
+    colsum = rng.integers(-50, 50, 9).astype(np.int32)
+    # multiplier exactly 1 (x_scale*w_scale == out_scale), no bias:
+    #   y = clamp(acc - x_zp*colsum + out_zp)
+    y = oracle.requantize(acc, colsum, 3, 0.5, [0.25], None, 0.125, 100)
+    want = np.clip(acc.astype(np.int64) - 3 * colsum + 100, 0, 255)
+    np.testing.assert_array_equal(y.astype(np.int64), want)
+    # relu raises the lower clamp to the zero point
+    y = oracle.requantize(acc, colsum, 3, 0.5, [0.25], None, 0.125, 100, relu=True)
+    np.testing.assert_array_equal(y.astype(np.int64), np.clip(want, 100, 255))
+    # signed output range
+    y = oracle.requantize(acc, colsum, 0, 0.5, [0.25], None, 0.125, -3, out_signed=True)
+    np.testing.assert_array_equal(y.astype(np.int64),
+                                  np.clip(acc.astype(np.int64) - 3, -128, 127))
+    # power-of-two multiplier 1/4 with exact halves -> ties to even
+    acc2 = np.array([[2, 6, 10, -2, -6, 1, 3]], dtype=np.int32)
+    y = oracle.requantize(acc2, np.zeros(7, np.int32), 0, 0.5, [0.5], None, 1.0, 100)
+    np.testing.assert_array_equal(y[0], np.array([100, 102, 102, 100, 98, 100, 101], np.uint8))
+    # bias enters as bias / (x_scale*w_scale) BEFORE the multiply:
+    #   bias = 3*atw exactly  ->  same as adding 3 to the accumulator
+    atw = 0.5 * 0.25
+    y_b = oracle.requantize(acc, colsum, 3, 0.5, [0.25], np.full(9, 3 * atw, np.float32), 0.125, 100)
+    np.testing.assert_array_equal(y_b.astype(np.int64),
+                                  np.clip(acc.astype(np.int64) - 3 * colsum + 103, 0, 255))
+    # per-channel scales pick the column's own multiplier
+    ws = np.array([0.25 * 2.0 ** (j % 3) for j in range(9)])
+    y_pc = oracle.requantize(acc, np.zeros(9, np.int32), 0, 0.5, ws, None, 0.125, 0)
+    want_pc = np.clip(acc.astype(np.int64) * (2 ** (np.arange(9) % 3))[None, :], 0, 255)
+    np.testing.assert_array_equal(y_pc.astype(np.int64), want_pc)
+
+
+def _im2col(x, kh, kw, stride, padding, dilation, x_zp):
+    b, h, w, c = x.shape
+    oh, ow = oracle.conv_out_hw(h, w, kh, kw, stride, padding, dilation)
+    cols = np.zeros((b, oh, ow, kh, kw, c), dtype=np.int64)
+    for i in range(oh):
+        for j in range(ow):
+            for a in range(kh):
+                for e in range(kw):
+                    ih = i * stride[0] - padding[0] + a * dilation[0]
+                    iw = j * stride[1] - padding[1] + e * dilation[1]
+                    if 0 <= ih < h and 0 <= iw < w:
+                        cols[:, i, j, a, e, :] = x[:, ih, iw, :].astype(np.int64) - x_zp
+    return cols.reshape(b * oh * ow, kh * kw * c), (b, oh, ow)
+
+
+@pytest.mark.parametrize("stride,padding,dilation", [((1, 1), (1, 1), (1, 1)),
+                                                     ((2, 1), (0, 2), (1, 2)),
+                                                     ((3, 2), (2, 0), (2, 1))])
+def test_conv_acc32_equals_gemm_on_im2col(stride, padding, dilation):
+    rng = np.random.default_rng(6)
+    x = rng.integers(0, 256, (2, 9, 8, 5), dtype=np.uint8)
+    w = rng.integers(-128, 128, (7, 3, 3, 5), dtype=np.int8)
+    acc = oracle.conv2d_acc32(x, w, stride, padding, dilation, 1, 77)
+    cols, (b, oh, ow) = _im2col(x, 3, 3, stride, padding, dilation, 77)
+    want = cols @ w.reshape(7, -1).astype(np.int64).T
+    np.testing.assert_array_equal(acc.reshape(-1, 7).astype(np.int64), want)
+
+
+def test_conv_groups_are_independent_convs():
+    rng = np.random.default_rng(7)
+    x = rng.integers(0, 256, (1, 6, 6, 8), dtype=np.uint8)
+    w = rng.integers(-128, 128, (6, 3, 3, 4), dtype=np.int8)   # groups=2: 2x(4 -> 3)
+    acc = oracle.conv2d_acc32(x, w, (1, 1), (1, 1), (1, 1), 2, 9)
+    for g in range(2):
+        part = oracle.conv2d_acc32(np.ascontiguousarray(x[..., 4 * g:4 * g + 4]),
+                                   np.ascontiguousarray(w[3 * g:3 * g + 3]),
+                                   (1, 1), (1, 1), (1, 1), 1, 9)
+        np.testing.assert_array_equal(acc[..., 3 * g:3 * g + 3], part)
+
+
+def test_conv_1x1_is_linear():
+    rng = np.random.default_rng(8)
+    x = rng.integers(0, 256, (2, 5, 4, 16), dtype=np.uint8)
+    w = rng.integers(-127, 128, (12, 1, 1, 16), dtype=np.int8)
+    ws = 0.001 + 0.002 * rng.random(12)
+    bias = rng.standard_normal(12).astype(np.float32)
+    yc = oracle.conv2d(x, 0.03, 50, w, ws, bias, (1, 1), (0, 0), (1, 1), 1, 0.08, 120)
+    yl = oracle.linear(x.reshape(-1, 16), 0.03, 50, w.reshape(12, 16), ws, bias, 0.08, 120)
+    np.testing.assert_array_equal(yc.reshape(-1, 12), yl)
