@@ -1,0 +1,233 @@
+/*
+ * tmq -- quantized-inference kernels for AMD MI355X (gfx950), C ABI.
+ *
+ * This is the whole device boundary of the library: raw device pointers, sizes,
+ * scalars and a HIP stream go in, a status code comes out.  No entry point
+ * allocates, frees, synchronises the device or touches global mutable state, so
+ * all of them are asynchronous on `stream`, re-entrant, and callable from
+ * several host threads on different streams.  Every buffer (inputs, outputs,
+ * packed weights, workspaces) is owned by the caller.
+ *
+ * Each entry point names the interface of the reference (MooreThreads
+ * torch_musa, paths relative to its tree) that it replaces.
+ *
+ * Numerics are those of PyTorch's CPU quantized ops (fbgemm):
+ *   quantize      q = clamp(rne(fl(x * fl(1/fl(scale)))) + zp, qmin, qmax)
+ *   dequantize    r = fl(fl(scale) * float(q - zp))
+ *   linear/conv   exact int32 accumulation, then per output channel n
+ *                   raw  = acc - x_zp * sum_k W[n][k]
+ *                   v    = float(raw) (+ fl(bias[n] / atw[n]))
+ *                   q    = clamp(rne(fl(v * mult[n])) + out_zp, lo, qmax)
+ *                 atw[n] = fl(fl(x_scale) * fl(w_scale[n])), mult[n] = fl(atw[n] / fl(out_scale)),
+ *                 lo = relu ? max(out_zp, qmin) : qmin.
+ * rne = round half to even, fl = round to fp32.
+ */
+#ifndef TMQ_H_
+#define TMQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TMQ_VERSION 100
+
+/* A hipStream_t, passed as an opaque pointer so that this header needs no HIP
+ * include. NULL is the default stream. */
+typedef void* tmq_stream_t;
+
+enum tmq_status {
+  TMQ_OK = 0,
+  TMQ_ERR_INVALID_ARGUMENT = 1, /* null pointer, negative size, bad enum value */
+  TMQ_ERR_UNSUPPORTED = 2,      /* well-formed request outside what is built */
+  TMQ_ERR_WORKSPACE = 3,        /* workspace missing or too small */
+  TMQ_ERR_LAUNCH = 4,           /* the HIP runtime refused the launch */
+  TMQ_ERR_ALIGNMENT = 5         /* pointer or leading dimension not aligned */
+};
+
+/* Static, human readable text for a status code. */
+const char* tmq_status_string(int status);
+int tmq_version(void);
+
+/* ---------------------------------------------------------------------------
+ * Affine quantizer, per tensor.
+ * Replaces torch_musa/csrc/aten/quantized/musa/AffineQuantizer.mu:99-143
+ * (quantize_tensor_per_tensor_affine_musa) and :145-179
+ * (dequantize_tensor_per_tensor_affine_musa), the functions registered on
+ * quantize_tensor_per_tensor_affine_stub / dequantize_..._stub (:340-357).
+ * `x`/`r` are dense fp32, `q` is one byte per element in the same order
+ * (uint8 when q_signed == 0, two's-complement int8 otherwise). n >= 0.
+ * ------------------------------------------------------------------------- */
+int tmq_quantize_per_tensor(const float* x, void* q, int64_t n, double scale,
+                            int64_t zero_point, int q_signed, tmq_stream_t stream);
+int tmq_dequantize_per_tensor(const void* q, float* r, int64_t n, double scale,
+                              int64_t zero_point, int q_signed, tmq_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Range calibration for quantize_per_tensor_dynamic.
+ * Replaces the two full reductions + host round trips behind
+ * torch_musa/csrc/aten/ops/musa_functions.yaml:3515-3519
+ * (aten::quantize_per_tensor_dynamic -> x.min().item(), x.max().item()).
+ *
+ * tmq_minmax writes {min, max} of x[0..n) to minmax[0..1] (device memory).
+ * `workspace` must hold tmq_minmax_workspace_bytes(n) bytes of device memory.
+ * n == 0 yields {+inf, -inf}.
+ * ------------------------------------------------------------------------- */
+size_t tmq_minmax_workspace_bytes(int64_t n);
+int tmq_minmax(const float* x, int64_t n, float* minmax, void* workspace,
+               size_t workspace_bytes, tmq_stream_t stream);
+
+/* Quantization parameters as the device-side chain keeps them. */
+typedef struct tmq_qparams {
+  double scale;       /* as ChooseQuantizationParams returns it */
+  int32_t zero_point;
+  int32_t reserved;
+} tmq_qparams;
+
+/* Device-side ChooseQuantizationParams (ATen/native/quantized/cpu/QuantUtils.h:
+ * 71-187 with preserve_sparsity = force_scale_power_of_two = false): reads
+ * minmax[0..1] on the device, writes *qparams on the device, so that
+ * tmq_quantize_per_tensor_dev can follow on the same stream without a host
+ * round trip. */
+int tmq_choose_qparams_dev(const float* minmax, int q_signed, int reduce_range,
+                           tmq_qparams* qparams, tmq_stream_t stream);
+/* Same as tmq_quantize_per_tensor with scale / zero point read from device
+ * memory at kernel run time. */
+int tmq_quantize_per_tensor_dev(const float* x, void* q, int64_t n,
+                                const tmq_qparams* qparams, int q_signed,
+                                tmq_stream_t stream);
+/* Host-side ChooseQuantizationParams, same arithmetic (pure CPU, no GPU call). */
+int tmq_choose_qparams_host(float min, float max, int q_signed, int reduce_range,
+                            double* scale, int32_t* zero_point);
+
+/* ---------------------------------------------------------------------------
+ * Affine quantizer, per channel.
+ * Replaces AffineQuantizer.mu:181-224 (quantize_tensor_per_channel_affine_musa)
+ * and :226-257 (dequantize_tensor_per_channel_affine_musa).
+ * The tensor is viewed as [outer, channels, inner] with the quantization axis
+ * in the middle; scales (double) and zero_points (int64) are device arrays of
+ * `channels` entries, the types the dispatch stub hands over.
+ * ------------------------------------------------------------------------- */
+int tmq_quantize_per_channel(const float* x, void* q, int64_t outer,
+                             int64_t channels, int64_t inner, const double* scales,
+                             const int64_t* zero_points, int q_signed,
+                             tmq_stream_t stream);
+int tmq_dequantize_per_channel(const void* q, float* r, int64_t outer,
+                               int64_t channels, int64_t inner, const double* scales,
+                               const int64_t* zero_points, int q_signed,
+                               tmq_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * quantized::linear weights.
+ * Replaces PackedLinearWeightMudnn::prepack
+ * (torch_musa/csrc/aten/quantized/mudnn/LinearPrepack.cpp:11-37), which keeps
+ * the [N,K] int8 weight as is for muDNN.  Here the weight is re-tiled once into
+ * the order the int8 MFMA kernels stream it in:
+ *   packed[nb][kc][r][b] = W[16*nb + r][16*kc + b],  r,b in [0,16)
+ * nb < ceil(N/16), kc < tmq_linear_packed_kchunks(K) (K rounded up to 128),
+ * zero filled outside W.  colsum[n] = sum_k W[n][k] (int32) is produced in the
+ * same pass; the epilogue needs it for the activation zero point.
+ * ------------------------------------------------------------------------- */
+int64_t tmq_linear_packed_kchunks(int64_t K);
+int64_t tmq_linear_packed_bytes(int64_t N, int64_t K);
+int tmq_linear_prepack(const int8_t* w, int64_t N, int64_t K, int64_t ldw,
+                       void* packed, int32_t* colsum, tmq_stream_t stream);
+/* Inverse re-tiling (packed -> [N,K] row major), for round-trip checks. */
+int tmq_linear_unpack(const void* packed, int64_t N, int64_t K, int8_t* w,
+                      int64_t ldw, tmq_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * quantized::linear / quantized::linear_relu.
+ * Replaces PackedLinearWeightMudnn::apply_impl_helper
+ * (torch_musa/csrc/aten/quantized/mudnn/Linear.cpp:16-65: muDNN
+ * MatMul::RunWithBiasAdd with SetTranspose(false,true), then a separate relu_).
+ * Y[M,N] = requant(X[M,K] . W[N,K]^T + bias), everything fused in one kernel.
+ * ------------------------------------------------------------------------- */
+typedef struct tmq_linear_desc {
+  int64_t M, N, K;
+  const void* x;         /* [M,K] bytes, row pitch ldx (elements) */
+  int64_t ldx;
+  int32_t x_signed;      /* 0: quint8 activations, 1: qint8 */
+  int32_t x_zero_point;
+  float x_scale;
+  const void* w_packed;  /* from tmq_linear_prepack */
+  const int32_t* w_colsum; /* [N] */
+  const float* w_scales;   /* [N] (per channel) or [1] (per tensor) */
+  int32_t w_per_channel;   /* 0: w_scales[0] for every n */
+  int32_t relu;            /* 1: lower clamp is the output zero point */
+  const float* bias;       /* [N] fp32 or NULL */
+  float out_scale;
+  int32_t out_zero_point;
+  int32_t out_signed;      /* 0: quint8 output, 1: qint8 */
+  int32_t reserved;
+  void* y;                 /* [M,N] bytes, row pitch ldy */
+  int64_t ldy;
+} tmq_linear_desc;
+
+int tmq_linear(const tmq_linear_desc* desc, tmq_stream_t stream);
+
+/* Raw accumulators acc[m][n] = sum_k X[m][k] * W[n][k] as int32 (row pitch
+ * ldacc), from the same MFMA main loop, for bit-exactness checks.  Uses
+ * M, N, K, x, ldx, x_signed, w_packed, w_colsum of `desc`. */
+int tmq_linear_acc32(const tmq_linear_desc* desc, int32_t* acc, int64_t ldacc,
+                     tmq_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * quantized::conv2d weights.
+ * Replaces PackedConvWeightMudnn<2>::prepack
+ * (torch_musa/csrc/aten/quantized/mudnn/ConvPrepack.cpp:10-92), which permutes
+ * OIHW to OHWI.  Input here is already OHWI ([OC, KH, KW, IC/groups] int8,
+ * dense); per group g it is re-tiled like a linear weight with
+ * N = OC/groups rows and K = KH*KW*ICg columns where every (kh,kw) tap is
+ * padded to a multiple of 16 input channels:
+ *   k = (kh*KW + kw) * roundup(ICg,16) + ic.
+ * colsum[oc] = sum of all weights of output channel oc.
+ * ------------------------------------------------------------------------- */
+typedef struct tmq_conv2d_geom {
+  int64_t B, H, W, IC; /* activations, NHWC */
+  int64_t OC, KH, KW;  /* weights, OHWI with IC/groups innermost */
+  int64_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, groups;
+} tmq_conv2d_geom;
+
+int64_t tmq_conv2d_packed_bytes(const tmq_conv2d_geom* g);
+int tmq_conv2d_prepack(const int8_t* w_ohwi, const tmq_conv2d_geom* g, void* packed,
+                       int32_t* colsum, tmq_stream_t stream);
+/* OH / OW as reference mudnn/Conv.cpp:20-36 computes them. */
+int tmq_conv2d_out_hw(const tmq_conv2d_geom* g, int64_t* OH, int64_t* OW);
+
+/* ---------------------------------------------------------------------------
+ * quantized::conv2d / conv2d_relu, NHWC implicit GEMM.
+ * Replaces PackedConvWeightMudnn<2>::apply_impl_helper
+ * (torch_musa/csrc/aten/quantized/mudnn/Conv.cpp:38-133: muDNN
+ * Convolution::RunFusion on NHWC tensors).
+ * x is [B,H,W,IC] bytes dense, y is [B,OH,OW,OC] bytes dense.
+ * ------------------------------------------------------------------------- */
+typedef struct tmq_conv2d_desc {
+  tmq_conv2d_geom geom;
+  const void* x;
+  int32_t x_signed;
+  int32_t x_zero_point;
+  float x_scale;
+  int32_t w_per_channel;
+  const void* w_packed;
+  const int32_t* w_colsum; /* [OC] */
+  const float* w_scales;   /* [OC] or [1] */
+  const float* bias;       /* [OC] or NULL */
+  float out_scale;
+  int32_t out_zero_point;
+  int32_t out_signed;
+  int32_t relu;
+  void* y;
+} tmq_conv2d_desc;
+
+int tmq_conv2d(const tmq_conv2d_desc* desc, tmq_stream_t stream);
+/* Zero-point-corrected accumulators, [B,OH,OW,OC] int32:
+ * acc = sum over in-image taps of (x - x_zp) * w. */
+int tmq_conv2d_acc32(const tmq_conv2d_desc* desc, int32_t* acc, tmq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TMQ_H_ */

@@ -1,0 +1,68 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol that
+include/tmq.h declares, and its host-only entry points agree with the oracle.
+No kernel is launched here."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+import cases
+import oracle
+from torch_musa_amd import cabi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_in_header():
+    text = open(os.path.join(ROOT, "include", "tmq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tmq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_list_agree():
+    assert _declared_in_header() == sorted(cabi.DECLARED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = cabi.lib()
+    for name in _declared_in_header():
+        assert hasattr(lib, name), f"{name} is declared in include/tmq.h but not exported"
+    assert lib.tmq_version() == 100
+    assert lib.tmq_status_string(0) == b"ok"
+    assert lib.tmq_status_string(3) != lib.tmq_status_string(4)
+
+
+def test_struct_sizes_match_the_header():
+    # natural alignment on x86-64: see include/tmq.h
+    import ctypes as C
+    assert C.sizeof(cabi.QParams) == 16
+    assert C.sizeof(cabi.LinearDesc) == 128
+    assert C.sizeof(cabi.Conv2dGeom) == 14 * 8
+    assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8
+
+
+def test_packed_size_arithmetic():
+    lib = cabi.lib()
+    assert lib.tmq_linear_packed_kchunks(1) == 8
+    assert lib.tmq_linear_packed_kchunks(128) == 8
+    assert lib.tmq_linear_packed_kchunks(129) == 16
+    assert lib.tmq_linear_packed_bytes(11008, 4096) == 11008 * 4096
+    assert lib.tmq_linear_packed_bytes(17, 130) == 2 * 16 * 256
+    g = cabi.conv_geom((32, 56, 56, 64), (64, 3, 3), (1, 1), (1, 1), (1, 1), 1)
+    assert cabi.conv_out_hw(g) == (56, 56)
+    assert lib.tmq_conv2d_packed_bytes(g) == 4 * 40 * 256  # K = 576 -> 640 padded
+    g2 = cabi.conv_geom((8, 32, 32, 3), (32, 7, 7), (2, 2), (3, 3), (1, 1), 1)
+    assert cabi.conv_out_hw(g2) == (16, 16)
+
+
+def test_host_choose_qparams_matches_oracle(golden):
+    for mn, mx in cases.dynamic_qparams_cases():
+        for rr in (False, True):
+            for signed in (False, True):
+                assert cabi.choose_qparams_host(float(mn), float(mx), signed, rr) == \
+                    oracle.choose_qparams(mn, mx, signed, rr)
+    for mn, mx, rr, s, z in golden["dynq/pairs"]:
+        assert cabi.choose_qparams_host(mn, mx, False, bool(rr)) == (s, int(z))
+    with pytest.raises(cabi.TmqError):
+        cabi.choose_qparams_host(1.0, -1.0, False, False)

@@ -1,0 +1,116 @@
+"""GPU parity of quantized::conv2d (NHWC implicit GEMM) through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle
+from gpu_util import dev, host, say
+
+pytestmark = pytest.mark.gpu
+
+LSB_TOL = 1
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from torch_musa_amd import cabi as m
+    assert torch.cuda.is_available()
+    m.lib()
+    return m
+
+
+def _check(y, want, what):
+    d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+    assert d.max() <= LSB_TOL, f"{what}: max diff {d.max()}"
+    assert d.max() == 0, f"{what}: {np.count_nonzero(d)} of {d.size} bytes differ by 1 LSB"
+
+
+def _run(cabi, c):
+    g = cabi.conv_geom(c["xq"].shape, c["wq"].shape, c["stride"], c["padding"], c["dilation"],
+                       c["groups"])
+    pw = cabi.PackedConv2d(dev(c["wq"]), g)
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    x = dev(c["xq"])
+    y = cabi.conv2d(x, pw, g, c["x_scale"], c["x_zp"], ws, b, c["out_scale"], c["out_zp"],
+                    relu=c["relu"])
+    acc = cabi.conv2d_acc32(x, pw, g, c["x_zp"])
+    return host(y), host(acc), pw
+
+
+@pytest.mark.parametrize("c", cases.conv_cases(), ids=lambda c: c["name"])
+def test_conv_cases(cabi, golden, c):
+    say("conv", c["name"])
+    y, acc, pw = _run(cabi, c)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                 c["groups"], c["x_zp"]))
+    np.testing.assert_array_equal(host(pw.colsum),
+                                  c["wq"].reshape(c["wq"].shape[0], -1).astype(np.int64).sum(1))
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"])
+    _check(y, want, "vs oracle")
+    _check(y, golden["conv/" + c["name"] + "/y"], "vs golden")
+
+
+def _conv_case(b, h, w, ic, oc, k, s, p, d, g, seed, x_signed=False, relu=False):
+    rng = np.random.default_rng(seed)
+    xq = (rng.integers(-128, 128, (b, h, w, ic), dtype=np.int8) if x_signed
+          else rng.integers(0, 256, (b, h, w, ic), dtype=np.uint8))
+    wq = rng.integers(-127, 128, (oc, k, k, ic // g), dtype=np.int8)
+    ws = (0.001 + 0.002 * rng.random(oc)).astype(np.float32).astype(np.float64)
+    kk = k * k * (ic // g)
+    sigma = np.sqrt(kk) * 74.0 * 74.0 * 0.03 * float(ws.mean())
+    return dict(xq=xq, wq=wq, bias=rng.standard_normal(oc).astype(np.float32) * np.float32(sigma),
+                x_scale=0.03, x_zp=-9 if x_signed else 60, w_scales=ws, stride=(s, s),
+                padding=(p, p), dilation=(d, d), groups=g,
+                out_scale=float(np.float32(3 * sigma / 128)), out_zp=4 if x_signed else 128,
+                relu=relu)
+
+
+@pytest.mark.parametrize("spec", [
+    (2, 20, 20, 64, 64, 3, 1, 1, 1, 1),      # C5's channel geometry, small image
+    (1, 30, 30, 128, 160, 3, 2, 1, 1, 1),    # OC > 64 -> 128x128 tiles when large
+    (4, 64, 64, 16, 256, 3, 1, 1, 1, 1),     # many rows, 128x128 tiles
+    (5, 120, 120, 16, 32, 3, 1, 0, 1, 1),    # > 65536 rows -> 256x64 tiles
+    (2, 17, 13, 48, 24, 5, 2, 2, 1, 1),      # ragged everything
+    (2, 16, 16, 64, 96, 3, 1, 1, 1, 2),      # two groups on the MFMA path
+    (2, 15, 15, 32, 40, 3, 1, 2, 2, 1),      # dilation
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_mfma_shapes(cabi, spec, x_signed):
+    say("conv mfma", spec, x_signed)
+    c = _conv_case(*spec, seed=sum(spec), x_signed=x_signed, relu=x_signed)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                 c["groups"], c["x_zp"], nthreads=8))
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "mfma conv")
+
+
+def test_c5_full_size(cabi):
+    """BASELINE config 5: [32,56,56,64] (x) [64,3,3,64], stride 1, pad 1."""
+    say("C5 full size")
+    rng = np.random.default_rng(55)
+    xf = np.maximum(rng.standard_normal((32, 56, 56, 64), dtype=np.float32), 0)
+    wf = rng.standard_normal((64, 3, 3, 64), dtype=np.float32) * np.float32(0.05)
+    xs, xz = oracle.choose_qparams(float(xf.min()), float(xf.max()))
+    assert xz == 0
+    xq = oracle.quantize_per_tensor(xf, xs, xz, False, nthreads=8)
+    ws = (np.abs(wf).reshape(64, -1).max(axis=1) / np.float32(127.0)).astype(np.float64)
+    wq = oracle.quantize_per_channel(wf, ws, np.zeros(64, np.int64), 0, True)
+    c = dict(xq=xq, wq=wq, bias=rng.standard_normal(64).astype(np.float32), x_scale=xs, x_zp=xz,
+             w_scales=ws, stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1,
+             out_scale=0.02, out_zp=128, relu=False)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(xq, wq, (1, 1), (1, 1), (1, 1), 1, xz, nthreads=8))
+    want = oracle.conv2d(xq, xs, xz, wq, ws, c["bias"], (1, 1), (1, 1), (1, 1), 1, 0.02, 128,
+                         nthreads=8)
+    assert 0.2 < np.mean((want > 0) & (want < 255))
+    _check(y, want, "C5")

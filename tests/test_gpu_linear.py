@@ -1,0 +1,208 @@
+"""GPU parity of quantized::linear through the C ABI.
+
+int32 accumulators: bit-exact against the oracle (exact integer matmul).
+Requantised bytes: the stated bar is 1 LSB; the epilogue restates the oracle's
+operation order, so the tests also report (and require) exact equality against
+the oracle, and stay within 1 LSB of the golden vectors of PyTorch's CPU op."""
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle
+from gpu_util import dev, host, say
+
+pytestmark = pytest.mark.gpu
+
+LSB_TOL = 1  # north-star tolerance for requantised int8/uint8 outputs
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from torch_musa_amd import cabi as m
+    assert torch.cuda.is_available()
+    m.lib()
+    yield m
+    m.force_linear_config(-1)
+
+
+def _run(cabi, c, cfg=-1, x=None):
+    xq = c["xq"] if x is None else x
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    cabi.force_linear_config(cfg)
+    try:
+        y = cabi.linear(dev(xq), pw, c["x_scale"], c["x_zp"], ws, b, c["out_scale"], c["out_zp"],
+                        relu=c["relu"])
+        acc = cabi.linear_acc32(dev(xq), pw)
+    finally:
+        cabi.force_linear_config(-1)
+    return host(y), host(acc), pw
+
+
+def _check(y, want, what):
+    d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+    assert d.max() <= LSB_TOL, f"{what}: max diff {d.max()}"
+    assert d.max() == 0, f"{what}: {np.count_nonzero(d)} of {d.size} bytes differ by 1 LSB"
+
+
+@pytest.mark.parametrize("c", cases.linear_cases(), ids=lambda c: c["name"])
+def test_linear_cases(cabi, golden, c):
+    say("lin", c["name"], c["xq"].shape, c["wq"].shape)
+    y, acc, pw = _run(cabi, c)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]))
+    np.testing.assert_array_equal(host(pw.colsum), oracle.weight_colsum(c["wq"]))
+    np.testing.assert_array_equal(host(pw.unpack()), c["wq"])
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"])
+    _check(y, want, "vs oracle")
+    _check(y, golden["lin/" + c["name"] + "/y"], "vs golden")
+
+
+def _tile_case(m, n, k, seed, x_signed=False, relu=False, bias=True, per_channel=True):
+    rng = np.random.default_rng(seed)
+    xq = (rng.integers(-128, 128, (m, k), dtype=np.int8) if x_signed
+          else rng.integers(0, 256, (m, k), dtype=np.uint8))
+    wq = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    ws = (0.001 + 0.002 * rng.random(n if per_channel else 1)).astype(np.float32).astype(np.float64)
+    x_scale = 0.02
+    sigma = np.sqrt(k) * 74.0 * 74.0 * x_scale * float(ws.mean())
+    return dict(xq=xq, wq=wq, bias=(rng.standard_normal(n).astype(np.float32) * np.float32(sigma)) if bias else None,
+                x_scale=x_scale, x_zp=-5 if x_signed else 121, w_scales=ws,
+                out_scale=float(np.float32(3 * sigma / 128)), out_zp=-3 if x_signed else 128,
+                relu=relu)
+
+
+# every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 9])
+@pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168)])
+def test_tile_configs(cabi, cfg, shape):
+    say("tile cfg", cfg, shape)
+    c = _tile_case(*shape, seed=cfg * 10 + shape[0])
+    y, acc, _ = _run(cabi, c, cfg)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"])
+    _check(y, want, f"cfg {cfg}")
+
+
+@pytest.mark.parametrize("x_signed,relu,bias,pc", [(True, False, True, True), (True, True, False, False),
+                                                   (False, True, True, False), (False, False, False, True)])
+def test_dtype_and_epilogue_variants(cabi, x_signed, relu, bias, pc):
+    say("variants", x_signed, relu, bias, pc)
+    c = _tile_case(150, 200, 256, seed=99, x_signed=x_signed, relu=relu, bias=bias, per_channel=pc)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"])
+    assert want.dtype == (np.int8 if x_signed else np.uint8) and y.dtype == want.dtype
+    _check(y, want, "variant")
+
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_decode_shapes(cabi, m):
+    """BASELINE config 4: M in {1,4,16}, K = N = 4096."""
+    say("decode", m)
+    c = _tile_case(m, 4096, 4096, seed=40 + m)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], nthreads=8)
+    _check(y, want, "decode")
+
+
+@pytest.mark.parametrize("m,n,k", [(3, 50, 100), (16, 16, 64), (9, 130, 4096 + 64), (16, 17, 16)])
+def test_decode_ragged(cabi, m, n, k):
+    say("decode ragged", m, n, k)
+    c = _tile_case(m, n, k, seed=m * n)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"])
+    _check(y, want, "decode ragged")
+
+
+def test_row_strided_and_unaligned_activations(cabi):
+    say("strided x")
+    c = _tile_case(70, 90, 128, seed=5)
+    big = np.zeros((70, 160), dtype=np.uint8)
+    big[:, :128] = c["xq"]
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    ws, b = dev(c["w_scales"].astype(np.float32)), dev(c["bias"])
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"])
+    xb = dev(big)
+    y = cabi.linear(xb[:, :128], pw, c["x_scale"], c["x_zp"], ws, b, c["out_scale"], c["out_zp"])
+    _check(host(y), want, "ldx=160")
+    big2 = np.zeros((70, 131), dtype=np.uint8)      # rows not 16-byte aligned -> plain kernel
+    big2[:, 3:] = c["xq"]
+    y = cabi.linear(dev(big2)[:, 3:], pw, c["x_scale"], c["x_zp"], ws, b, c["out_scale"], c["out_zp"])
+    _check(host(y), want, "unaligned rows")
+
+
+def test_empty_batch(cabi):
+    c = _tile_case(4, 32, 64, seed=1)
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    x = torch.empty((0, 64), dtype=torch.uint8, device="cuda")
+    y = cabi.linear(x, pw, 0.1, 0, dev(c["w_scales"].astype(np.float32)), None, 0.1, 0)
+    assert tuple(y.shape) == (0, 32)
+
+
+def test_c1_golden(cabi, golden):
+    """BASELINE config 1 end to end on the device: dynamic quantize of x,
+    per-channel quantize of W, prepack, linear."""
+    say("C1")
+    c1 = cases.c1_case()
+    x = dev(c1["x"].reshape(-1))
+    qp = cabi.choose_qparams_dev(cabi.minmax(x), False, False)
+    s, z = cabi.read_qparams(qp)
+    assert s == float(golden["c1/x_scale"]) and z == int(golden["c1/x_zp"])
+    xq = cabi.quantize_per_tensor_dev(x, qp, False).reshape(128, 1024)
+    assert cases.crc(host(xq)) == int(golden["c1/xq_crc"])
+    wq = cabi.quantize_per_channel(dev(c1["w"]), dev(c1["w_scales"]),
+                                   torch.zeros(1024, dtype=torch.int64, device="cuda"), 0, True)
+    assert cases.crc(host(wq)) == int(golden["c1/wq_crc"])
+    pw = cabi.PackedLinear(wq)
+    y = cabi.linear(xq, pw, s, z, dev(c1["w_scales"].astype(np.float32)), dev(c1["bias"]),
+                    c1["out_scale"], c1["out_zp"])
+    acc = cabi.linear_acc32(xq, pw)
+    np.testing.assert_array_equal(host(acc), oracle.linear_acc32(host(xq), host(wq), nthreads=8))
+    _check(host(y), golden["c1/y"], "C1 vs golden")
+    dq = cabi.dequantize_per_tensor(y, c1["out_scale"], c1["out_zp"])
+    assert cases.crc(host(dq)) == int(golden["c1/y_dq_crc"])
+
+
+def test_c3_full_size(cabi):
+    """BASELINE config 3 (M=4096, K=4096, N=11008): oracle parity on sampled
+    rows, and the all-ones identity acc[m][n] = colsum[n] on the whole output."""
+    M, K, N = 4096, 4096, 11008
+    say("C3 full size")
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    w = rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)
+    mn, mx = oracle.minmax(x, nthreads=8)
+    s, z = oracle.choose_qparams(mn, mx)
+    xq = cabi.quantize_per_tensor(dev(x.reshape(-1)), s, z, False).reshape(M, K)
+    ws = (np.abs(w).max(axis=1) / np.float32(127.0)).astype(np.float64)
+    wq = cabi.quantize_per_channel(dev(w), dev(ws), torch.zeros(N, dtype=torch.int64, device="cuda"), 0, True)
+    bias = rng.standard_normal(N, dtype=np.float32)
+    pw = cabi.PackedLinear(wq)
+    out_scale, out_zp = 0.02, 128
+    y = cabi.linear(xq, pw, s, z, dev(ws.astype(np.float32)), dev(bias), out_scale, out_zp)
+    acc = cabi.linear_acc32(xq, pw)
+    rows = np.array([0, 1, 255, 256, 1023, 2048, 4000, 4095])
+    xq_h, wq_h = host(xq[torch.from_numpy(rows).cuda()]), host(wq)
+    np.testing.assert_array_equal(host(acc[torch.from_numpy(rows).cuda()]),
+                                  oracle.linear_acc32(xq_h, wq_h, nthreads=8))
+    want = oracle.linear(xq_h, s, z, wq_h, ws, bias, out_scale, out_zp, nthreads=8)
+    got = host(y[torch.from_numpy(rows).cuda()])
+    assert 0.2 < np.mean((got > 0) & (got < 255)), "output saturated: test would prove nothing"
+    _check(got, want, "C3 rows")
+    # every tile of the output: activations of all ones reproduce the column sums
+    ones = torch.ones((M, K), dtype=torch.uint8, device="cuda")
+    acc1 = cabi.linear_acc32(ones, pw)
+    assert torch.equal(acc1, pw.colsum[None, :].expand(M, N))
+    # the GEMM is linear in x: acc(x) + acc(255 - x) = 255 * colsum
+    acc2 = cabi.linear_acc32(255 - xq, pw)
+    assert torch.equal(acc + acc2, 255 * pw.colsum[None, :].expand(M, N))

@@ -1,0 +1,155 @@
+"""GPU parity of the affine quantizer kernels, through the C ABI, against the
+CPU oracle and the golden vectors.  Everything here is bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle
+from gpu_util import dev, host, say
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from torch_musa_amd import cabi as m
+    assert torch.cuda.is_available()
+    m.lib()
+    return m
+
+
+@pytest.mark.parametrize("c", cases.quantize_per_tensor_cases(), ids=lambda c: c["name"])
+def test_quantize_dequantize_per_tensor(cabi, golden, c):
+    say("qpt", c["name"])
+    x = dev(c["x"].reshape(-1))
+    q = cabi.quantize_per_tensor(x, c["scale"], c["zp"], c["signed"])
+    want = oracle.quantize_per_tensor(c["x"], c["scale"], c["zp"], c["signed"]).reshape(-1)
+    np.testing.assert_array_equal(host(q), want)
+    np.testing.assert_array_equal(host(q).view(np.uint8), golden["qpt/" + c["name"] + "/q"].reshape(-1).view(np.uint8))
+    r = cabi.dequantize_per_tensor(q, c["scale"], c["zp"])
+    np.testing.assert_array_equal(host(r), oracle.dequantize_per_tensor(want, c["scale"], c["zp"]))
+    assert cases.crc(host(r)) == int(golden["qpt/" + c["name"] + "/dq_crc"])
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3])
+@pytest.mark.parametrize("n", [1, 5, 17, 1000, 4099])
+def test_unaligned_pointers(cabi, offset, n):
+    say("unaligned", offset, n)
+    x_full = cases.randn(5000 + n, (n + offset,), std=3.0)
+    xd = dev(x_full)[offset:]              # x is 4-byte but not 16-byte aligned
+    qbuf = torch.zeros(n + offset + 8, dtype=torch.uint8, device="cuda")
+    qv = qbuf[offset:offset + n]           # q is not 4-byte aligned
+    cabi.quantize_per_tensor_into(xd, qv, 0.05, 100, False)
+    want = oracle.quantize_per_tensor(x_full[offset:], 0.05, 100, False)
+    np.testing.assert_array_equal(host(qv), want)
+    assert int(qbuf[:offset].sum()) == 0 and int(qbuf[offset + n:].sum()) == 0  # no stray writes
+    rbuf = torch.zeros(n + offset + 8, dtype=torch.float32, device="cuda")
+    rv = rbuf[offset:offset + n]
+    cabi.dequantize_per_tensor_into(qv, rv, 0.05, 100)
+    np.testing.assert_array_equal(host(rv), oracle.dequantize_per_tensor(want, 0.05, 100))
+    assert float(rbuf[:offset].abs().sum()) == 0 and float(rbuf[offset + n:].abs().sum()) == 0
+
+
+def test_empty_and_bad_arguments(cabi):
+    x = torch.empty(0, dtype=torch.float32, device="cuda")
+    assert cabi.quantize_per_tensor(x, 0.1, 0, False).numel() == 0
+    x = torch.zeros(4, dtype=torch.float32, device="cuda")
+    with pytest.raises(cabi.TmqError):
+        cabi.quantize_per_tensor(x, 0.1, 256, False)     # zero point outside quint8
+    with pytest.raises(cabi.TmqError):
+        cabi.quantize_per_tensor(x, 0.1, -129, True)
+
+
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 5, 63, 1024, 2049, 8191, 70001, 2 ** 22 + 3])
+@pytest.mark.parametrize("offset", [0, 1])
+def test_minmax(cabi, n, offset):
+    say("minmax", n, offset)
+    x = cases.randn(600 + n % 97, (n + offset,), std=2.0)
+    got = host(cabi.minmax(dev(x)[offset:]))
+    if n == 0:
+        assert got[0] == np.inf and got[1] == -np.inf
+    else:
+        assert got[0] == x[offset:].min() and got[1] == x[offset:].max()
+
+
+@pytest.mark.parametrize("c", cases.dynamic_tensor_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("rr", [False, True])
+def test_dynamic_chain_on_device(cabi, golden, c, rr):
+    """min/max -> qparams -> quantize without leaving the device."""
+    say("dyn", c["name"], rr)
+    k = f"dyn/{c['name']}/rr{int(rr)}"
+    x = dev(c["x"].reshape(-1))
+    mm = cabi.minmax(x)
+    qp = cabi.choose_qparams_dev(mm, False, rr)
+    q = cabi.quantize_per_tensor_dev(x, qp, False)
+    s, z = cabi.read_qparams(qp)
+    assert s == float(golden[k + "/scale"]) and z == int(golden[k + "/zp"])
+    np.testing.assert_array_equal(host(q), golden[k + "/q"].reshape(-1))
+
+
+def test_choose_qparams_dev_matches_oracle(cabi):
+    for mn, mx in cases.dynamic_qparams_cases():
+        for rr in (False, True):
+            for signed in (False, True):
+                mm = dev(np.array([mn, mx], dtype=np.float32))
+                got = cabi.read_qparams(cabi.choose_qparams_dev(mm, signed, rr))
+                assert got == oracle.choose_qparams(mn, mx, signed, rr), (mn, mx, rr, signed)
+
+
+@pytest.mark.parametrize("c", cases.quantize_per_channel_cases(), ids=lambda c: c["name"])
+def test_quantize_dequantize_per_channel(cabi, golden, c):
+    say("qpc", c["name"])
+    k = "qpc/" + c["name"]
+    x = dev(c["x"])
+    scales = dev(c["scales"].astype(np.float64))
+    zps = dev(c["zps"].astype(np.int64))
+    q = cabi.quantize_per_channel(x, scales, zps, c["axis"], c["signed"])
+    np.testing.assert_array_equal(host(q), golden[k + "/q"])
+    r = cabi.dequantize_per_channel(q, scales, zps, c["axis"])
+    want = oracle.dequantize_per_channel(golden[k + "/q"], c["scales"], c["zps"], c["axis"])
+    np.testing.assert_array_equal(host(r), want)
+    assert cases.crc(host(r)) == int(golden[k + "/dq_crc"])
+
+
+def test_per_channel_weight_sized(cabi):
+    """[N,K] weight, axis 0, the shape quantized::linear weights come in."""
+    say("qpc weight 1000x4096")
+    w = cases.randn(31, (1000, 4096), std=0.02)
+    s = (np.abs(w).max(axis=1) / 127.0).astype(np.float64)
+    z = np.zeros(1000, np.int64)
+    q = cabi.quantize_per_channel(dev(w), dev(s), dev(z), 0, True)
+    np.testing.assert_array_equal(host(q), oracle.quantize_per_channel(w, s, z, 0, True))
+
+
+def test_full_size_properties(cabi):
+    """BASELINE config 2 at full size (2**28 fp32): properties that need no
+    full-size oracle run, plus oracle parity on sampled windows."""
+    n = 2 ** 28
+    say("C2 full size", n)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randn(n, device="cuda", generator=g) * 3.0
+    x[::100] = 50.0
+    x[37::100] = -50.0
+    mm = host(cabi.minmax(x))
+    assert mm[0] == -50.0 and mm[1] == 50.0
+    s, z = oracle.choose_qparams(mm[0], mm[1], False, False)
+    q = cabi.quantize_per_tensor(x, s, z, False)
+    r = cabi.dequantize_per_tensor(q, s, z)
+    # round trip error is at most half a step (everything is inside the range)
+    err = (r - x).abs().max().item()
+    assert err <= 0.5 * np.float32(s) * (1 + 1e-5), err
+    # idempotence: dequantized values are fixed points
+    q2 = cabi.quantize_per_tensor(r, s, z, False)
+    assert torch.equal(q, q2)
+    # device-side chain gives the same bytes
+    qp = cabi.choose_qparams_dev(cabi.minmax(x), False, False)
+    assert cabi.read_qparams(qp) == (s, z)
+    assert torch.equal(cabi.quantize_per_tensor_dev(x, qp, False), q)
+    # oracle parity on windows, including the very end of the buffer
+    for start in (0, 123_456_789 // 4 * 4 + 1, n - 2 ** 20):
+        xs = host(x[start:start + 2 ** 20])
+        np.testing.assert_array_equal(host(q[start:start + 2 ** 20]),
+                                      oracle.quantize_per_tensor(xs, s, z, False))
+        np.testing.assert_array_equal(host(r[start:start + 2 ** 20]),
+                                      oracle.dequantize_per_tensor(host(q[start:start + 2 ** 20]), s, z))

@@ -1,0 +1,116 @@
+"""Builds the native libraries in-tree with hipcc (cross-compiles without a GPU).
+
+  libtmq.so       torch-free HIP kernel library behind include/tmq.h
+  libtmq_aten.so  ATen registrations (TORCH_LIBRARY_IMPL + dispatch stubs)
+                  that call libtmq.so
+
+    python -m torch_musa_amd.build [--kernels-only] [--verbose]
+"""
+from __future__ import annotations
+
+import argparse
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+OBJ = os.path.join(PKG, "build")
+LIB_KERNELS = os.path.join(PKG, "libtmq.so")
+LIB_ATEN = os.path.join(PKG, "libtmq_aten.so")
+ARCH = "gfx950"
+
+KERNEL_SOURCES = ["kernels/quantize.hip", "kernels/linear.hip", "kernels/conv2d.hip"]
+ATEN_SOURCES = ["aten/register.cpp"]
+
+# -ffp-contract=off: the requantisation epilogue and the quantizer must round
+# after every fp32 operation, as the CPU ops they mirror do.
+# packed-fp32-ops disabled: never emit v_pk_{add,mul,fma}_f32.
+DEVICE_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC",
+    "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in p.stdout.splitlines()
+                    if "is not a recognized feature for this target" not in l)
+    if p.returncode != 0:
+        raise RuntimeError(f"command failed ({p.returncode}): {' '.join(cmd)}\n{out}")
+    if verbose and out.strip():
+        print(out, flush=True)
+
+
+def _hipcc():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def build_kernels(verbose=False):
+    os.makedirs(OBJ, exist_ok=True)
+    hipcc = _hipcc()
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", os.path.join(CSRC, "kernels")]
+    jobs = []
+    for src in KERNEL_SOURCES:
+        path = os.path.join(CSRC, src)
+        if not os.path.exists(path):
+            continue
+        obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+        jobs.append((obj, [hipcc] + DEVICE_FLAGS + inc + ["-c", path, "-o", obj]))
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
+        list(ex.map(lambda j: _run(j[1], verbose), jobs))
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", LIB_KERNELS]
+         + [j[0] for j in jobs], verbose)
+    return LIB_KERNELS
+
+
+def build_aten(verbose=False):
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    os.makedirs(OBJ, exist_ok=True)
+    hipcc = _hipcc()
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = []
+    for d in ce.include_paths("cuda") if hasattr(ce, "include_paths") else []:
+        inc += ["-isystem", d]
+    inc += ["-I", os.path.join(ROOT, "include")]
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    objs = []
+    for src in ATEN_SOURCES:
+        path = os.path.join(CSRC, src)
+        obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+        _run([hipcc, "-x", "hip", f"--offload-arch={ARCH}", "-O2", "-std=c++17", "-fPIC",
+              "-fvisibility=hidden", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-DUSE_ROCM",
+              "-D__HIP_PLATFORM_AMD__=1", "-Wno-unused-command-line-argument",
+              "-Wno-deprecated-declarations"] + inc + ["-c", path, "-o", obj], verbose)
+        objs.append(obj)
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", LIB_ATEN] + objs
+         + ["-L", PKG, "-ltmq", "-L", tlib, "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10",
+            "-lc10_hip", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}"], verbose)
+    return LIB_ATEN
+
+
+def build_all(verbose=False, kernels_only=False):
+    out = [build_kernels(verbose)]
+    if not kernels_only and all(os.path.exists(os.path.join(CSRC, s)) for s in ATEN_SOURCES):
+        out.append(build_aten(verbose))
+    return out
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--kernels-only", action="store_true")
+    ap.add_argument("--verbose", action="store_true")
+    a = ap.parse_args()
+    for lib in build_all(a.verbose, a.kernels_only):
+        print("built", lib, os.path.getsize(lib), "bytes")
+    sys.exit(0)

@@ -1,0 +1,372 @@
+"""ctypes binding of the C ABI in ``include/tmq.h`` (``libtmq.so``).
+
+Thin by design: device pointers come from ``torch.Tensor.data_ptr()``, the
+stream from ``torch.cuda.current_stream()``; torch is only the allocator here.
+Every wrapper raises ``TmqError`` on a non-zero status.  There is no CPU
+fallback: if ``libtmq.so`` is missing the import of this module's library
+fails loudly.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch  # first: libtmq.so must bind to the HIP runtime torch has loaded
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libtmq.so")
+
+DECLARED_SYMBOLS = [
+    "tmq_status_string", "tmq_version",
+    "tmq_quantize_per_tensor", "tmq_dequantize_per_tensor",
+    "tmq_minmax_workspace_bytes", "tmq_minmax", "tmq_choose_qparams_dev",
+    "tmq_quantize_per_tensor_dev", "tmq_choose_qparams_host",
+    "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
+    "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
+    "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
+    "tmq_conv2d", "tmq_conv2d_acc32",
+]
+
+
+class TmqError(RuntimeError):
+    pass
+
+
+class QParams(C.Structure):
+    _fields_ = [("scale", C.c_double), ("zero_point", C.c_int32), ("reserved", C.c_int32)]
+
+
+class LinearDesc(C.Structure):
+    _fields_ = [
+        ("M", C.c_int64), ("N", C.c_int64), ("K", C.c_int64),
+        ("x", C.c_void_p), ("ldx", C.c_int64),
+        ("x_signed", C.c_int32), ("x_zero_point", C.c_int32), ("x_scale", C.c_float),
+        ("w_packed", C.c_void_p), ("w_colsum", C.c_void_p), ("w_scales", C.c_void_p),
+        ("w_per_channel", C.c_int32), ("relu", C.c_int32),
+        ("bias", C.c_void_p),
+        ("out_scale", C.c_float), ("out_zero_point", C.c_int32),
+        ("out_signed", C.c_int32), ("reserved", C.c_int32),
+        ("y", C.c_void_p), ("ldy", C.c_int64),
+    ]
+
+
+class Conv2dGeom(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in (
+        "B", "H", "W", "IC", "OC", "KH", "KW", "stride_h", "stride_w", "pad_h", "pad_w",
+        "dil_h", "dil_w", "groups")]
+
+
+class Conv2dDesc(C.Structure):
+    _fields_ = [
+        ("geom", Conv2dGeom),
+        ("x", C.c_void_p),
+        ("x_signed", C.c_int32), ("x_zero_point", C.c_int32), ("x_scale", C.c_float),
+        ("w_per_channel", C.c_int32),
+        ("w_packed", C.c_void_p), ("w_colsum", C.c_void_p), ("w_scales", C.c_void_p),
+        ("bias", C.c_void_p),
+        ("out_scale", C.c_float), ("out_zero_point", C.c_int32),
+        ("out_signed", C.c_int32), ("relu", C.c_int32),
+        ("y", C.c_void_p),
+    ]
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise TmqError(f"{LIB_PATH} is missing: build it with `python -m torch_musa_amd.build`")
+        l = C.CDLL(LIB_PATH)
+        l.tmq_status_string.restype = C.c_char_p
+        l.tmq_minmax_workspace_bytes.restype = C.c_size_t
+        l.tmq_minmax_workspace_bytes.argtypes = [C.c_int64]
+        for name in ("tmq_linear_packed_kchunks", "tmq_linear_packed_bytes"):
+            getattr(l, name).restype = C.c_int64
+        l.tmq_linear_packed_kchunks.argtypes = [C.c_int64]
+        l.tmq_linear_packed_bytes.argtypes = [C.c_int64, C.c_int64]
+        l.tmq_conv2d_packed_bytes.restype = C.c_int64
+        l.tmq_conv2d_packed_bytes.argtypes = [C.POINTER(Conv2dGeom)]
+        v = C.c_void_p
+        l.tmq_quantize_per_tensor.argtypes = [v, v, C.c_int64, C.c_double, C.c_int64, C.c_int, v]
+        l.tmq_dequantize_per_tensor.argtypes = [v, v, C.c_int64, C.c_double, C.c_int64, C.c_int, v]
+        l.tmq_minmax.argtypes = [v, C.c_int64, v, v, C.c_size_t, v]
+        l.tmq_choose_qparams_dev.argtypes = [v, C.c_int, C.c_int, v, v]
+        l.tmq_quantize_per_tensor_dev.argtypes = [v, v, C.c_int64, v, C.c_int, v]
+        l.tmq_choose_qparams_host.argtypes = [C.c_float, C.c_float, C.c_int, C.c_int,
+                                              C.POINTER(C.c_double), C.POINTER(C.c_int32)]
+        l.tmq_quantize_per_channel.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, v, v, C.c_int, v]
+        l.tmq_dequantize_per_channel.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, v, v, C.c_int, v]
+        l.tmq_linear_prepack.argtypes = [v, C.c_int64, C.c_int64, C.c_int64, v, v, v]
+        l.tmq_linear_unpack.argtypes = [v, C.c_int64, C.c_int64, v, C.c_int64, v]
+        l.tmq_linear.argtypes = [C.POINTER(LinearDesc), v]
+        l.tmq_linear_acc32.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, v]
+        l.tmq_conv2d_prepack.argtypes = [v, C.POINTER(Conv2dGeom), v, v, v]
+        l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+        l.tmq_conv2d.argtypes = [C.POINTER(Conv2dDesc), v]
+        l.tmq_conv2d_acc32.argtypes = [C.POINTER(Conv2dDesc), v, v]
+        _lib = l
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        raise TmqError(f"{what}: {lib().tmq_status_string(status).decode()} (status {status})")
+
+
+def stream_ptr() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+# ---------------------------------------------------------------------------
+# quantizer
+# ---------------------------------------------------------------------------
+def quantize_per_tensor(x: torch.Tensor, scale: float, zp: int, signed: bool) -> torch.Tensor:
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    q = torch.empty(x.shape, dtype=torch.int8 if signed else torch.uint8, device=x.device)
+    check(lib().tmq_quantize_per_tensor(x.data_ptr(), q.data_ptr(), x.numel(), scale, zp,
+                                        int(signed), stream_ptr()), "tmq_quantize_per_tensor")
+    return q
+
+
+def quantize_per_tensor_into(x, q, scale, zp, signed):
+    check(lib().tmq_quantize_per_tensor(x.data_ptr(), q.data_ptr(), x.numel(), scale, zp,
+                                        int(signed), stream_ptr()), "tmq_quantize_per_tensor")
+
+
+def dequantize_per_tensor(q: torch.Tensor, scale: float, zp: int) -> torch.Tensor:
+    assert q.dtype in (torch.int8, torch.uint8) and q.is_contiguous()
+    r = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    check(lib().tmq_dequantize_per_tensor(q.data_ptr(), r.data_ptr(), q.numel(), scale, zp,
+                                          int(q.dtype == torch.int8), stream_ptr()),
+          "tmq_dequantize_per_tensor")
+    return r
+
+
+def dequantize_per_tensor_into(q, r, scale, zp):
+    check(lib().tmq_dequantize_per_tensor(q.data_ptr(), r.data_ptr(), q.numel(), scale, zp,
+                                          int(q.dtype == torch.int8), stream_ptr()),
+          "tmq_dequantize_per_tensor")
+
+
+def minmax_workspace(device) -> torch.Tensor:
+    return torch.empty(lib().tmq_minmax_workspace_bytes(0), dtype=torch.uint8, device=device)
+
+
+def minmax(x: torch.Tensor, out: torch.Tensor = None, ws: torch.Tensor = None) -> torch.Tensor:
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    if out is None:
+        out = torch.empty(2, dtype=torch.float32, device=x.device)
+    if ws is None:
+        ws = minmax_workspace(x.device)
+    check(lib().tmq_minmax(x.data_ptr(), x.numel(), out.data_ptr(), ws.data_ptr(), ws.numel(),
+                           stream_ptr()), "tmq_minmax")
+    return out
+
+
+def choose_qparams_dev(mm: torch.Tensor, signed: bool, reduce_range: bool) -> torch.Tensor:
+    qp = torch.empty(16, dtype=torch.uint8, device=mm.device)
+    check(lib().tmq_choose_qparams_dev(mm.data_ptr(), int(signed), int(reduce_range),
+                                       qp.data_ptr(), stream_ptr()), "tmq_choose_qparams_dev")
+    return qp
+
+
+def read_qparams(qp: torch.Tensor):
+    raw = bytes(qp.cpu().numpy().tobytes())
+    s = QParams.from_buffer_copy(raw)
+    return float(s.scale), int(s.zero_point)
+
+
+def quantize_per_tensor_dev(x: torch.Tensor, qp: torch.Tensor, signed: bool) -> torch.Tensor:
+    q = torch.empty(x.shape, dtype=torch.int8 if signed else torch.uint8, device=x.device)
+    check(lib().tmq_quantize_per_tensor_dev(x.data_ptr(), q.data_ptr(), x.numel(), qp.data_ptr(),
+                                            int(signed), stream_ptr()),
+          "tmq_quantize_per_tensor_dev")
+    return q
+
+
+def choose_qparams_host(mn: float, mx: float, signed: bool, reduce_range: bool):
+    s, z = C.c_double(), C.c_int32()
+    check(lib().tmq_choose_qparams_host(mn, mx, int(signed), int(reduce_range), C.byref(s),
+                                        C.byref(z)), "tmq_choose_qparams_host")
+    return float(s.value), int(z.value)
+
+
+def _outer_c_inner(shape, axis):
+    axis = axis % len(shape)
+    outer = 1
+    for d in shape[:axis]:
+        outer *= d
+    inner = 1
+    for d in shape[axis + 1:]:
+        inner *= d
+    return outer, shape[axis], inner
+
+
+def quantize_per_channel(x, scales, zps, axis, signed):
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert scales.dtype == torch.float64 and zps.dtype == torch.int64
+    outer, c, inner = _outer_c_inner(tuple(x.shape), axis)
+    q = torch.empty(x.shape, dtype=torch.int8 if signed else torch.uint8, device=x.device)
+    check(lib().tmq_quantize_per_channel(x.data_ptr(), q.data_ptr(), outer, c, inner,
+                                         scales.data_ptr(), zps.data_ptr(), int(signed),
+                                         stream_ptr()), "tmq_quantize_per_channel")
+    return q
+
+
+def dequantize_per_channel(q, scales, zps, axis):
+    assert q.is_contiguous()
+    outer, c, inner = _outer_c_inner(tuple(q.shape), axis)
+    r = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    check(lib().tmq_dequantize_per_channel(q.data_ptr(), r.data_ptr(), outer, c, inner,
+                                           scales.data_ptr(), zps.data_ptr(),
+                                           int(q.dtype == torch.int8), stream_ptr()),
+          "tmq_dequantize_per_channel")
+    return r
+
+
+# ---------------------------------------------------------------------------
+# linear
+# ---------------------------------------------------------------------------
+class PackedLinear:
+    """Device buffers produced by tmq_linear_prepack for one [N,K] int8 weight."""
+
+    def __init__(self, w: torch.Tensor):
+        assert w.dtype == torch.int8 and w.dim() == 2 and w.stride(1) == 1
+        self.N, self.K = w.shape
+        nbytes = lib().tmq_linear_packed_bytes(self.N, self.K)
+        self.packed = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=w.device)
+        self.colsum = torch.empty(max(self.N, 1), dtype=torch.int32, device=w.device)
+        check(lib().tmq_linear_prepack(w.data_ptr(), self.N, self.K, w.stride(0),
+                                       self.packed.data_ptr(), self.colsum.data_ptr(),
+                                       stream_ptr()), "tmq_linear_prepack")
+
+    def unpack(self) -> torch.Tensor:
+        w = torch.empty((self.N, self.K), dtype=torch.int8, device=self.packed.device)
+        check(lib().tmq_linear_unpack(self.packed.data_ptr(), self.N, self.K, w.data_ptr(),
+                                      self.K, stream_ptr()), "tmq_linear_unpack")
+        return w
+
+
+def _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed, relu, y):
+    d = LinearDesc()
+    d.M, d.K = x.shape
+    d.N = pw.N
+    assert d.K == pw.K
+    d.x, d.ldx = x.data_ptr(), x.stride(0)
+    d.x_signed = int(x.dtype == torch.int8)
+    d.x_zero_point, d.x_scale = x_zp, x_scale
+    d.w_packed, d.w_colsum = pw.packed.data_ptr(), pw.colsum.data_ptr()
+    if w_scales is not None:
+        assert w_scales.dtype == torch.float32
+        d.w_scales = w_scales.data_ptr()
+        d.w_per_channel = int(w_scales.numel() > 1)
+    d.relu = int(relu)
+    d.bias = _ptr(bias)
+    d.out_scale, d.out_zero_point, d.out_signed = out_scale, out_zp, int(out_signed)
+    if y is not None:
+        d.y, d.ldy = y.data_ptr(), y.stride(0)
+    return d
+
+
+def linear(x, pw: PackedLinear, x_scale, x_zp, w_scales, bias, out_scale, out_zp,
+           out_signed=None, relu=False, out=None):
+    """x: [M,K] uint8/int8 (row stride free), w_scales: fp32 [N] or [1]."""
+    assert x.dim() == 2 and x.stride(1) == 1
+    if out_signed is None:
+        out_signed = x.dtype == torch.int8
+    y = out if out is not None else torch.empty(
+        (x.shape[0], pw.N), dtype=torch.int8 if out_signed else torch.uint8, device=x.device)
+    d = _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed, relu, y)
+    check(lib().tmq_linear(C.byref(d), stream_ptr()), "tmq_linear")
+    return y
+
+
+def linear_acc32(x, pw: PackedLinear):
+    acc = torch.empty((x.shape[0], pw.N), dtype=torch.int32, device=x.device)
+    d = _linear_desc(x, pw, 1.0, 0, None, None, 1.0, 0, False, False, None)
+    check(lib().tmq_linear_acc32(C.byref(d), acc.data_ptr(), acc.stride(0), stream_ptr()),
+          "tmq_linear_acc32")
+    return acc
+
+
+def force_linear_config(cfg: int) -> None:
+    """Benchmark hook: pin the GEMM tile configuration (-1 = automatic)."""
+    lib().tmq_debug_force_linear_config(C.c_int(cfg))
+
+
+# ---------------------------------------------------------------------------
+# conv2d
+# ---------------------------------------------------------------------------
+def conv_geom(x_shape_nhwc, w_shape_ohwi, stride, padding, dilation, groups) -> Conv2dGeom:
+    g = Conv2dGeom()
+    g.B, g.H, g.W, g.IC = x_shape_nhwc
+    g.OC, g.KH, g.KW = w_shape_ohwi[:3]
+    g.stride_h, g.stride_w = stride
+    g.pad_h, g.pad_w = padding
+    g.dil_h, g.dil_w = dilation
+    g.groups = groups
+    return g
+
+
+def conv_out_hw(g: Conv2dGeom):
+    oh, ow = C.c_int64(), C.c_int64()
+    check(lib().tmq_conv2d_out_hw(C.byref(g), C.byref(oh), C.byref(ow)), "tmq_conv2d_out_hw")
+    return oh.value, ow.value
+
+
+class PackedConv2d:
+    def __init__(self, w_ohwi: torch.Tensor, g: Conv2dGeom):
+        assert w_ohwi.dtype == torch.int8 and w_ohwi.is_contiguous()
+        nbytes = lib().tmq_conv2d_packed_bytes(C.byref(g))
+        if nbytes <= 0:
+            raise TmqError("invalid convolution geometry")
+        self.packed = torch.empty(nbytes, dtype=torch.uint8, device=w_ohwi.device)
+        self.colsum = torch.empty(g.OC, dtype=torch.int32, device=w_ohwi.device)
+        check(lib().tmq_conv2d_prepack(w_ohwi.data_ptr(), C.byref(g), self.packed.data_ptr(),
+                                       self.colsum.data_ptr(), stream_ptr()),
+              "tmq_conv2d_prepack")
+
+
+def _conv_desc(x, pw, g, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed, relu, y):
+    d = Conv2dDesc()
+    d.geom = g
+    d.x = x.data_ptr()
+    d.x_signed = int(x.dtype == torch.int8)
+    d.x_zero_point, d.x_scale = x_zp, x_scale
+    d.w_packed, d.w_colsum = pw.packed.data_ptr(), pw.colsum.data_ptr()
+    if w_scales is not None:
+        d.w_scales = w_scales.data_ptr()
+        d.w_per_channel = int(w_scales.numel() > 1)
+    d.bias = _ptr(bias)
+    d.out_scale, d.out_zero_point, d.out_signed, d.relu = out_scale, out_zp, int(out_signed), int(relu)
+    d.y = _ptr(y)
+    return d
+
+
+def conv2d(x_nhwc, pw: PackedConv2d, g: Conv2dGeom, x_scale, x_zp, w_scales, bias, out_scale,
+           out_zp, out_signed=None, relu=False, out=None):
+    assert x_nhwc.is_contiguous() and tuple(x_nhwc.shape) == (g.B, g.H, g.W, g.IC)
+    if out_signed is None:
+        out_signed = x_nhwc.dtype == torch.int8
+    oh, ow = conv_out_hw(g)
+    y = out if out is not None else torch.empty(
+        (g.B, oh, ow, g.OC), dtype=torch.int8 if out_signed else torch.uint8, device=x_nhwc.device)
+    d = _conv_desc(x_nhwc, pw, g, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed,
+                   relu, y)
+    check(lib().tmq_conv2d(C.byref(d), stream_ptr()), "tmq_conv2d")
+    return y
+
+
+def conv2d_acc32(x_nhwc, pw: PackedConv2d, g: Conv2dGeom, x_zp):
+    oh, ow = conv_out_hw(g)
+    acc = torch.empty((g.B, oh, ow, g.OC), dtype=torch.int32, device=x_nhwc.device)
+    d = _conv_desc(x_nhwc, pw, g, 1.0, x_zp, None, None, 1.0, 0, False, False, None)
+    check(lib().tmq_conv2d_acc32(C.byref(d), acc.data_ptr(), stream_ptr()), "tmq_conv2d_acc32")
+    return acc

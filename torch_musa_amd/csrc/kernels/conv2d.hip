@@ -1,0 +1,283 @@
+// quantized::conv2d for gfx950: NHWC implicit GEMM on the int8 MFMA core.
+//
+// GEMM view per group: rows m = (b, oh, ow) output pixels, columns n = output
+// channels of the group, k = (kh, kw, ic) with every tap padded to a multiple
+// of 16 input channels, so one 16-byte k-chunk is one run of 16 channels of one
+// input pixel -- a single aligned load from the NHWC activation tensor.
+// Taps outside the image are filled with the activation zero point (real value
+// 0), which the accumulator start value then cancels exactly.
+#include "gemm_i8_core.h"
+
+static_assert(sizeof(tmq_conv2d_geom) == 112, "tmq_conv2d_geom layout changed");
+static_assert(sizeof(tmq_conv2d_desc) == 192, "tmq_conv2d_desc layout changed");
+
+namespace tmq {
+namespace {
+
+constexpr int64_t kKPad = 128;
+inline int64_t packed_kchunks(int64_t K) { return (K + kKPad - 1) / kKPad * (kKPad / 16); }
+
+struct ConvShape {
+  int64_t B, H, W, IC, OC, KH, KW, OH, OW;
+  int64_t sh, sw, ph, pw, dh, dw, groups;
+  int64_t ICg, OCg, ICgp, Kp, KC, group_bytes;
+};
+
+int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
+  if (g == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  if (g->B < 0 || g->H <= 0 || g->W <= 0 || g->IC <= 0 || g->OC <= 0 || g->KH <= 0 || g->KW <= 0 ||
+      g->stride_h <= 0 || g->stride_w <= 0 || g->pad_h < 0 || g->pad_w < 0 || g->dil_h <= 0 ||
+      g->dil_w <= 0 || g->groups <= 0)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  if (g->IC % g->groups != 0 || g->OC % g->groups != 0) return TMQ_ERR_INVALID_ARGUMENT;
+  s->B = g->B; s->H = g->H; s->W = g->W; s->IC = g->IC; s->OC = g->OC; s->KH = g->KH; s->KW = g->KW;
+  s->sh = g->stride_h; s->sw = g->stride_w; s->ph = g->pad_h; s->pw = g->pad_w;
+  s->dh = g->dil_h; s->dw = g->dil_w; s->groups = g->groups;
+  s->OH = (g->H + 2 * g->pad_h - g->dil_h * (g->KH - 1) - 1) / g->stride_h + 1;
+  s->OW = (g->W + 2 * g->pad_w - g->dil_w * (g->KW - 1) - 1) / g->stride_w + 1;
+  if (s->OH <= 0 || s->OW <= 0) return TMQ_ERR_INVALID_ARGUMENT;
+  s->ICg = g->IC / g->groups;
+  s->OCg = g->OC / g->groups;
+  s->ICgp = round_up(s->ICg, 16);
+  s->Kp = g->KH * g->KW * s->ICgp;
+  s->KC = packed_kchunks(s->Kp);
+  s->group_bytes = ceil_div(s->OCg, 16) * s->KC * 256;
+  // 32-bit index arithmetic inside the kernels
+  if (g->H > (1 << 24) || g->W > (1 << 24) || g->IC > (1 << 24) || s->Kp > (1 << 30))
+    return TMQ_ERR_UNSUPPORTED;
+  return TMQ_OK;
+}
+
+// One thread per 16-byte packed chunk (group, nb, kc, r).
+__global__ __launch_bounds__(256) void conv_prepack_kernel(const int8_t* __restrict__ w,
+                                                           ConvShape s, int64_t total,
+                                                           uint8_t* __restrict__ packed) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const int64_t per_group = s.group_bytes / 16;
+  const int64_t g = id / per_group, lid = id % per_group;
+  const int r = static_cast<int>(lid & 15);
+  const int64_t kc = (lid >> 4) % s.KC, nb = (lid >> 4) / s.KC;
+  const int64_t n = nb * 16 + r;
+  const int64_t k0 = kc * 16;
+  const int64_t tap = k0 / s.ICgp, ic0 = k0 % s.ICgp;
+  uint32_t words[4] = {0, 0, 0, 0};
+  if (n < s.OCg && tap < s.KH * s.KW) {
+    const int8_t* src = w + ((g * s.OCg + n) * s.KH * s.KW + tap) * s.ICg;
+    for (int b = 0; b < 16; ++b)
+      if (ic0 + b < s.ICg)
+        words[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(src[ic0 + b])) << (8 * (b & 3));
+  }
+  *reinterpret_cast<v4i*>(packed + id * 16) =
+      v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
+          static_cast<int>(words[3])};
+}
+
+__global__ __launch_bounds__(256) void conv_colsum_kernel(const int8_t* __restrict__ w, int64_t OC,
+                                                          int64_t K, int32_t* __restrict__ colsum) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * (256 / kWave) + threadIdx.x / kWave;
+  if (n >= OC) return;
+  int s = 0;
+  for (int64_t i = lane; i < K; i += kWave) s += w[n * K + i];
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, kWave);
+  if (lane == 0) colsum[n] = s;
+}
+
+struct PlainArgs {
+  const uint8_t* x;
+  const uint8_t* w_packed;
+  const int32_t* colsum;
+  const float* w_scales;
+  const float* bias;
+  int32_t w_scale_stride, x_signed, x_zp;
+  float x_scale, out_scale, zp_f, lo_f, hi_f;
+  void* y;
+};
+
+// Direct convolution, one thread per output value: any channel count, any
+// grouping, any alignment.  Accumulates (x - x_zp) * w over in-image taps.
+template <int MODE>
+__global__ __launch_bounds__(256) void conv_plain_kernel(ConvShape s, PlainArgs a) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t rows = s.B * s.OH * s.OW;
+  if (id >= rows * s.OC) return;
+  const int64_t oc = id % s.OC, m = id / s.OC;
+  const int64_t g = oc / s.OCg, n = oc % s.OCg;
+  const int64_t ow = m % s.OW, oh = (m / s.OW) % s.OH, b = m / (s.OW * s.OH);
+  const uint8_t* wp = a.w_packed + g * s.group_bytes;
+  int acc = 0;
+  for (int64_t kh = 0; kh < s.KH; ++kh) {
+    const int64_t ih = oh * s.sh - s.ph + kh * s.dh;
+    if (ih < 0 || ih >= s.H) continue;
+    for (int64_t kw = 0; kw < s.KW; ++kw) {
+      const int64_t iw = ow * s.sw - s.pw + kw * s.dw;
+      if (iw < 0 || iw >= s.W) continue;
+      const uint8_t* xp = a.x + ((b * s.H + ih) * s.W + iw) * s.IC + g * s.ICg;
+      const int64_t kbase = (kh * s.KW + kw) * s.ICgp;
+      for (int64_t ic = 0; ic < s.ICg; ++ic) {
+        const int xv = a.x_signed ? static_cast<int>(static_cast<int8_t>(xp[ic])) : static_cast<int>(xp[ic]);
+        const int64_t k = kbase + ic;
+        const int wv = static_cast<int8_t>(wp[(((n >> 4) * s.KC + (k >> 4)) * 16 + (n & 15)) * 16 + (k & 15)]);
+        acc += (xv - a.x_zp) * wv;
+      }
+    }
+  }
+  if (MODE == kOutAcc32) {
+    static_cast<int32_t*>(a.y)[id] = acc;
+  } else {
+    const float atw = a.x_scale * a.w_scales[oc * a.w_scale_stride];
+    const float mult = atw / a.out_scale;
+    float v = static_cast<float>(acc);
+    if (a.bias != nullptr) v = v + a.bias[oc] / atw;
+    const float ab = v * mult;
+    float r = __builtin_rintf(ab) + a.zp_f;
+    r = __builtin_amdgcn_fmed3f(r, a.lo_f, a.hi_f);
+    static_cast<uint8_t*>(a.y)[id] = static_cast<uint8_t>(static_cast<int>(r));
+  }
+}
+
+template <int BM, int BN, int WM, int WN, int MODE>
+int launch_conv_gemm(const GemmArgs& a, const XConv& xs, hipStream_t s) {
+  const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  gemm_i8_kernel<BM, BN, WM, WN, MODE, XConv>
+      <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
+  return launch_status();
+}
+
+template <int MODE>
+int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
+  ConvShape s;
+  int rc = make_shape(&d->geom, &s);
+  if (rc != TMQ_OK) return rc;
+  const int64_t rows = s.B * s.OH * s.OW;
+  if (rows == 0) return TMQ_OK;
+  if (d->x == nullptr || d->w_packed == nullptr || d->w_colsum == nullptr || out == nullptr)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  if (!aligned(d->w_packed, 16)) return TMQ_ERR_ALIGNMENT;
+  const int qmin = d->out_signed ? -128 : 0, qmax = d->out_signed ? 127 : 255;
+  const int xmin = d->x_signed ? -128 : 0, xmax = d->x_signed ? 127 : 255;
+  if (d->x_zero_point < xmin || d->x_zero_point > xmax) return TMQ_ERR_INVALID_ARGUMENT;
+  if (MODE != kOutAcc32) {
+    if (d->w_scales == nullptr || !(d->x_scale > 0.f) || !(d->out_scale > 0.f))
+      return TMQ_ERR_INVALID_ARGUMENT;
+    if (d->out_zero_point < qmin || d->out_zero_point > qmax) return TMQ_ERR_INVALID_ARGUMENT;
+  }
+  const float zp_f = static_cast<float>(d->out_zero_point);
+  const float lo_f = static_cast<float>(d->relu ? d->out_zero_point : qmin);
+  const float hi_f = static_cast<float>(qmax);
+
+  const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
+  if (!mfma_ok) {
+    PlainArgs p{};
+    p.x = static_cast<const uint8_t*>(d->x);
+    p.w_packed = static_cast<const uint8_t*>(d->w_packed);
+    p.colsum = d->w_colsum;
+    p.w_scales = d->w_scales;
+    p.bias = d->bias;
+    p.w_scale_stride = d->w_per_channel ? 1 : 0;
+    p.x_signed = d->x_signed;
+    p.x_zp = d->x_zero_point;
+    p.x_scale = d->x_scale;
+    p.out_scale = d->out_scale;
+    p.zp_f = zp_f; p.lo_f = lo_f; p.hi_f = hi_f;
+    p.y = out;
+    const int64_t blocks = ceil_div(rows * s.OC, 256);
+    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    conv_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(s, p);
+    return launch_status();
+  }
+
+  XConv xs{};
+  xs.x = static_cast<const uint8_t*>(d->x);
+  xs.H = static_cast<int>(s.H); xs.W = static_cast<int>(s.W); xs.IC = static_cast<int>(s.IC);
+  xs.OH = static_cast<int>(s.OH); xs.OW = static_cast<int>(s.OW);
+  xs.KW = static_cast<int>(s.KW); xs.icb = static_cast<int>(s.ICgp / 16);
+  xs.stride_h = static_cast<int>(s.sh); xs.stride_w = static_cast<int>(s.sw);
+  xs.pad_h = static_cast<int>(s.ph); xs.pad_w = static_cast<int>(s.pw);
+  xs.dil_h = static_cast<int>(s.dh); xs.dil_w = static_cast<int>(s.dw);
+  xs.pad_word = 0x01010101u * static_cast<uint32_t>(static_cast<uint8_t>(d->x_zero_point));
+
+  GemmArgs a{};
+  a.M = rows;
+  a.N = s.OCg;
+  a.K = s.Kp;
+  a.w_kchunks = s.KC;
+  a.colsum = d->w_colsum;
+  a.w_scales = d->w_scales;
+  a.bias = d->bias;
+  a.w_scale_stride = d->w_per_channel ? 1 : 0;
+  a.x_xor = d->x_signed ? 0u : 0x80808080u;
+  a.acc_coef = (d->x_signed ? 0 : 128) - d->x_zero_point;
+  a.x_scale = d->x_scale;
+  a.out_scale = d->out_scale;
+  a.zp_f = zp_f; a.lo_f = lo_f; a.hi_f = hi_f;
+  a.y = out;
+  a.ldy = s.OC;
+  for (int64_t g = 0; g < s.groups; ++g) {
+    a.w_packed = static_cast<const uint8_t*>(d->w_packed) + g * s.group_bytes;
+    a.n_off = static_cast<int32_t>(g * s.OCg);
+    xs.ic_off = static_cast<int>(g * s.ICg);
+    if (s.OCg > 64 && rows >= 128 * 128)
+      rc = launch_conv_gemm<128, 128, 2, 2, MODE>(a, xs, stream);
+    else if (rows >= 256 * 256)
+      rc = launch_conv_gemm<256, 64, 4, 1, MODE>(a, xs, stream);
+    else
+      rc = launch_conv_gemm<64, 64, 2, 2, MODE>(a, xs, stream);
+    if (rc != TMQ_OK) return rc;
+  }
+  return TMQ_OK;
+}
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+TMQ_EXPORT int64_t tmq_conv2d_packed_bytes(const tmq_conv2d_geom* g) {
+  ConvShape s;
+  if (make_shape(g, &s) != TMQ_OK) return 0;
+  return s.groups * s.group_bytes;
+}
+
+TMQ_EXPORT int tmq_conv2d_out_hw(const tmq_conv2d_geom* g, int64_t* OH, int64_t* OW) {
+  ConvShape s;
+  const int rc = make_shape(g, &s);
+  if (rc != TMQ_OK) return rc;
+  if (OH != nullptr) *OH = s.OH;
+  if (OW != nullptr) *OW = s.OW;
+  return TMQ_OK;
+}
+
+TMQ_EXPORT int tmq_conv2d_prepack(const int8_t* w_ohwi, const tmq_conv2d_geom* g, void* packed,
+                                  int32_t* colsum, tmq_stream_t stream) {
+  ConvShape s;
+  const int rc = make_shape(g, &s);
+  if (rc != TMQ_OK) return rc;
+  if (w_ohwi == nullptr || packed == nullptr || colsum == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!aligned(packed, 16)) return TMQ_ERR_ALIGNMENT;
+  hipStream_t hs = as_stream(stream);
+  const int64_t total = s.groups * s.group_bytes / 16;
+  int64_t blocks = ceil_div(total, 256);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  conv_prepack_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, hs>>>(
+      w_ohwi, s, total, static_cast<uint8_t*>(packed));
+  if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  blocks = ceil_div(s.OC, 256 / kWave);
+  conv_colsum_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, hs>>>(
+      w_ohwi, s.OC, s.KH * s.KW * s.ICg, colsum);
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_conv2d(const tmq_conv2d_desc* d, tmq_stream_t stream) {
+  if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  return d->out_signed ? run_conv<kOutS8>(d, d->y, as_stream(stream))
+                       : run_conv<kOutU8>(d, d->y, as_stream(stream));
+}
+
+TMQ_EXPORT int tmq_conv2d_acc32(const tmq_conv2d_desc* d, int32_t* acc, tmq_stream_t stream) {
+  if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  return run_conv<kOutAcc32>(d, acc, as_stream(stream));
+}

@@ -1,0 +1,380 @@
+// quantized::linear for gfx950: weight re-tiling, the MFMA GEMM dispatch, a
+// weight-streaming kernel for decode-sized batches, and a plain kernel for
+// shapes the vector paths do not take (K not a multiple of 16, unaligned rows).
+#include <atomic>
+
+#include "gemm_i8_core.h"
+
+// Layout that non-C++ bindings rely on (natural alignment, x86-64).
+static_assert(sizeof(tmq_linear_desc) == 128, "tmq_linear_desc layout changed");
+static_assert(sizeof(tmq_qparams) == 16, "tmq_qparams layout changed");
+
+namespace tmq {
+namespace {
+
+constexpr int64_t kKPad = 128;  // packed k extent is a multiple of this
+
+__host__ __device__ inline int64_t packed_kchunks(int64_t K) { return (K + kKPad - 1) / kKPad * (kKPad / 16); }
+
+// ---------------------------------------------------------------------------
+// prepack: one thread per 16-byte packed chunk (nb, kc, r)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void prepack_kernel(const int8_t* __restrict__ w, int64_t N,
+                                                      int64_t K, int64_t ldw, int64_t KC,
+                                                      int64_t total, bool vec,
+                                                      uint8_t* __restrict__ packed) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const int r = static_cast<int>(id & 15);
+  const int64_t kc = (id >> 4) % KC;
+  const int64_t nb = (id >> 4) / KC;
+  const int64_t n = nb * 16 + r, k0 = kc * 16;
+  v4i out = {0, 0, 0, 0};
+  if (n < N && k0 < K) {
+    const int8_t* src = w + n * ldw + k0;
+    if (vec && k0 + 16 <= K) {
+      out = ld16(src);
+    } else {
+      uint32_t words[4] = {0, 0, 0, 0};
+      for (int b = 0; b < 16 && k0 + b < K; ++b)
+        words[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(src[b])) << (8 * (b & 3));
+      out = v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
+                static_cast<int>(words[3])};
+    }
+  }
+  *reinterpret_cast<v4i*>(packed + id * 16) = out;
+}
+
+__global__ __launch_bounds__(256) void unpack_kernel(const uint8_t* __restrict__ packed, int64_t N,
+                                                     int64_t K, int64_t ldw, int64_t KC,
+                                                     int8_t* __restrict__ w) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= N * K) return;
+  const int64_t n = id / K, k = id % K;
+  w[n * ldw + k] = static_cast<int8_t>(packed[(((n >> 4) * KC + (k >> 4)) * 16 + (n & 15)) * 16 + (k & 15)]);
+}
+
+// colsum[n] = sum_k W[n][k]; one wavefront per weight row.
+__global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ w, int64_t N,
+                                                     int64_t K, int64_t ldw, bool vec,
+                                                     int32_t* __restrict__ colsum) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * (256 / kWave) + threadIdx.x / kWave;
+  if (n >= N) return;
+  const int8_t* row = w + n * ldw;
+  int s = 0;
+  int64_t k = 0;
+  if (vec) {
+    for (int64_t c = lane; c < K / 16; c += kWave) {
+      const v4i v = ld16(row + c * 16);
+      s = __builtin_amdgcn_sdot4(v.x, 0x01010101, s, false);
+      s = __builtin_amdgcn_sdot4(v.y, 0x01010101, s, false);
+      s = __builtin_amdgcn_sdot4(v.z, 0x01010101, s, false);
+      s = __builtin_amdgcn_sdot4(v.w, 0x01010101, s, false);
+    }
+    k = K / 16 * 16;
+  }
+  for (int64_t i = k + lane; i < K; i += kWave) s += row[i];
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, kWave);
+  if (lane == 0) colsum[n] = s;
+}
+
+// ---------------------------------------------------------------------------
+// Decode-sized batches (M <= 16): the weight is read once, straight from HBM
+// into MFMA operand registers (the packed layout is the 16x16x64 operand
+// order), activations come from L2.  One block per 16 output channels, its
+// four waves split K and reduce through LDS.
+//   D[i][j] of v_mfma_i32_16x16x64_i8: lane l, register r -> i = 4*(l/16)+r
+//   (channel), j = l%16 (activation row).
+// ---------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(256) void linear_decode_kernel(GemmArgs a, XLinear xs) {
+  constexpr int kWaves = 4;
+  constexpr int kBatch = 8;  // 64-byte k-blocks in flight per wave
+  __shared__ int s_part[kWaves][16 * 16];
+  const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
+  const int lr = lane & 15, lc = lane >> 4;
+  const int64_t nb = blockIdx.x;
+  const int64_t KB = ceil_div(a.K, 64);
+  const uint8_t* wp = a.w_packed + nb * a.w_kchunks * 256 + lc * 256 + lr * 16;
+  const bool xrow = lr < a.M;
+  const uint8_t* xp = xs.x + (xrow ? lr : 0) * xs.ldx + lc * 16;
+  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
+                     static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
+  v4i acc = {0, 0, 0, 0};
+  for (int64_t kb0 = wave; kb0 < KB; kb0 += kWaves * kBatch) {
+    v4i wf[kBatch], xf[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t kb = kb0 + u * kWaves;
+      const bool ok = kb < KB;
+      wf[u] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + kb * 1024))
+                 : v4i{0, 0, 0, 0};
+      const bool xok = ok && xrow && (kb * 64 + lc * 16 < a.K);
+      xf[u] = xok ? ld16(xp + kb * 64) : v4i{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], xf[u] ^ xmask, acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) s_part[wave][(4 * lc + r) * 16 + lr] = acc[r];
+  __syncthreads();
+  // 64 threads finish: thread -> (activation row m, channel group of 4)
+  if (t < 64) {
+    const int m = t >> 2, g = t & 3;
+    if (m < a.M) {
+      int raw[4];
+      v4f bdiv, mult;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        const int64_t n = nb * 16 + i;
+        int s = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) s += s_part[w][i * 16 + m];
+        const bool ok = n < a.N;
+        const int64_t np = ok ? n : 0;
+        raw[j] = s + a.acc_coef * a.colsum[np];
+        if (MODE != kOutAcc32) {
+          const float atw = a.x_scale * a.w_scales[np * a.w_scale_stride];
+          mult[j] = atw / a.out_scale;
+          bdiv[j] = a.bias != nullptr ? a.bias[np] / atw : 0.f;
+        }
+      }
+      const int64_t n = nb * 16 + 4 * g;
+      if (MODE == kOutAcc32) {
+        int32_t* dst = static_cast<int32_t*>(a.y) + m * a.ldy + n;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < a.N) dst[j] = raw[j];
+      } else {
+        const uint32_t packed = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+        uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
+        if (n + 3 < a.N && (a.ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 3) == 0) {
+          *reinterpret_cast<uint32_t*>(dst) = packed;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (n + j < a.N) dst[j] = static_cast<uint8_t>(packed >> (8 * j));
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Plain kernel: any K, any alignment.  One thread per (m, group of 4 channels).
+// ---------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear xs, int x_signed) {
+  const int64_t groups = ceil_div(a.N, 4);
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= a.M * groups) return;
+  const int64_t m = id / groups, n = (id % groups) * 4;
+  const uint8_t* xr = xs.x + m * xs.ldx;
+  int raw[4] = {0, 0, 0, 0};
+  for (int64_t k = 0; k < a.K; ++k) {
+    const int xv = x_signed ? static_cast<int>(static_cast<int8_t>(xr[k])) : static_cast<int>(xr[k]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t nn = n + j;  // rows past N are zero in the packed buffer's last block
+      const int wv = static_cast<int8_t>(
+          a.w_packed[(((nn >> 4) * a.w_kchunks + (k >> 4)) * 16 + (nn & 15)) * 16 + (k & 15)]);
+      raw[j] += xv * wv;
+    }
+  }
+  v4f bdiv, mult;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t np = n + j < a.N ? n + j : 0;
+    // plain accumulation used the true activation value, so only -x_zp*colsum is left
+    raw[j] += a.acc_coef * a.colsum[np];
+    if (MODE != kOutAcc32) {
+      const float atw = a.x_scale * a.w_scales[np * a.w_scale_stride];
+      mult[j] = atw / a.out_scale;
+      bdiv[j] = a.bias != nullptr ? a.bias[np] / atw : 0.f;
+    }
+  }
+  if (MODE == kOutAcc32) {
+    int32_t* dst = static_cast<int32_t*>(a.y) + m * a.ldy + n;
+    for (int j = 0; j < 4; ++j)
+      if (n + j < a.N) dst[j] = raw[j];
+  } else {
+    const uint32_t packed = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+    uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
+    for (int j = 0; j < 4; ++j)
+      if (n + j < a.N) dst[j] = static_cast<uint8_t>(packed >> (8 * j));
+  }
+}
+
+// Kernel selection override for benchmarking: -1 = automatic.
+std::atomic<int> g_forced_config{-1};
+
+template <int BM, int BN, int WM, int WN, int MODE>
+int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear>
+      <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
+  return launch_status();
+}
+
+template <int MODE>
+int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec_ok,
+                    hipStream_t s) {
+  const int forced = g_forced_config.load(std::memory_order_relaxed);
+  if (!vec_ok || forced == 9) {
+    // plain kernel accumulates true activation values: undo the +128 share
+    GemmArgs b = a;
+    if (!x_signed) b.acc_coef -= 128;
+    const int64_t work = a.M * ceil_div(a.N, 4);
+    const int64_t blocks = ceil_div(work, 256);
+    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    linear_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(b, xs, x_signed);
+    return launch_status();
+  }
+  if ((a.M <= 16 && forced < 0) || forced == 8) {
+    if (a.M > 16) return TMQ_ERR_UNSUPPORTED;
+    const int64_t blocks = ceil_div(a.N, 16);
+    linear_decode_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(a, xs);
+    return launch_status();
+  }
+  int cfg = forced;
+  if (cfg < 0) {
+    // largest tile that still leaves at least ~2 blocks per CU, else smaller
+    const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
+    if (nblk(256, 256) >= 512)
+      cfg = 0;
+    else if (nblk(128, 128) >= 256)
+      cfg = 1;
+    else
+      cfg = 2;
+  }
+  switch (cfg) {
+    case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
+    case 1: return launch_gemm<128, 128, 2, 2, MODE>(a, xs, s);
+    case 2: return launch_gemm<64, 64, 2, 2, MODE>(a, xs, s);
+    case 3: return launch_gemm<256, 256, 2, 4, MODE>(a, xs, s);
+    case 4: return launch_gemm<128, 256, 2, 2, MODE>(a, xs, s);
+    case 5: return launch_gemm<256, 128, 2, 2, MODE>(a, xs, s);
+    default: return TMQ_ERR_UNSUPPORTED;
+  }
+}
+
+int fill_args(const tmq_linear_desc* d, GemmArgs* a, XLinear* xs, bool* vec_ok) {
+  if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  if (d->M < 0 || d->N < 0 || d->K < 0) return TMQ_ERR_INVALID_ARGUMENT;
+  if (d->M == 0 || d->N == 0) return TMQ_OK;
+  if (d->x == nullptr && d->K > 0) return TMQ_ERR_INVALID_ARGUMENT;
+  if (d->w_packed == nullptr || d->w_colsum == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  if (d->ldx < d->K) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!aligned(d->w_packed, 16)) return TMQ_ERR_ALIGNMENT;
+  a->M = d->M;
+  a->N = d->N;
+  a->K = d->K;
+  a->w_packed = static_cast<const uint8_t*>(d->w_packed);
+  a->w_kchunks = packed_kchunks(d->K);
+  a->colsum = d->w_colsum;
+  a->x_xor = d->x_signed ? 0u : 0x80808080u;
+  a->n_off = 0;
+  xs->x = static_cast<const uint8_t*>(d->x);
+  xs->ldx = d->ldx;
+  *vec_ok = d->K % 16 == 0 && d->ldx % 16 == 0 && aligned(d->x, 16);
+  return TMQ_OK;
+}
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+TMQ_EXPORT int64_t tmq_linear_packed_kchunks(int64_t K) { return K < 0 ? 0 : packed_kchunks(K); }
+
+TMQ_EXPORT int64_t tmq_linear_packed_bytes(int64_t N, int64_t K) {
+  if (N < 0 || K < 0) return 0;
+  return ceil_div(N, 16) * packed_kchunks(K) * 256;
+}
+
+TMQ_EXPORT int tmq_linear_prepack(const int8_t* w, int64_t N, int64_t K, int64_t ldw, void* packed,
+                                  int32_t* colsum, tmq_stream_t stream) {
+  if (N < 0 || K < 0 || ldw < K) return TMQ_ERR_INVALID_ARGUMENT;
+  if (N == 0) return TMQ_OK;
+  if (packed == nullptr || colsum == nullptr || (w == nullptr && K > 0))
+    return TMQ_ERR_INVALID_ARGUMENT;
+  if (!aligned(packed, 16)) return TMQ_ERR_ALIGNMENT;
+  hipStream_t s = as_stream(stream);
+  const int64_t KC = packed_kchunks(K);
+  const int64_t total = ceil_div(N, 16) * KC * 16;
+  const bool vec = aligned(w, 16) && ldw % 16 == 0;
+  if (total > 0) {
+    const int64_t blocks = ceil_div(total, 256);
+    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    prepack_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(
+        w, N, K, ldw, KC, total, vec, static_cast<uint8_t*>(packed));
+    if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  }
+  const int64_t blocks = ceil_div(N, 256 / kWave);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  colsum_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(w, N, K, ldw, vec, colsum);
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_linear_unpack(const void* packed, int64_t N, int64_t K, int8_t* w, int64_t ldw,
+                                 tmq_stream_t stream) {
+  if (N < 0 || K < 0 || ldw < K) return TMQ_ERR_INVALID_ARGUMENT;
+  if (N == 0 || K == 0) return TMQ_OK;
+  if (packed == nullptr || w == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  const int64_t blocks = ceil_div(N * K, 256);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  unpack_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, as_stream(stream)>>>(
+      static_cast<const uint8_t*>(packed), N, K, ldw, packed_kchunks(K), w);
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_linear(const tmq_linear_desc* d, tmq_stream_t stream) {
+  GemmArgs a{};
+  XLinear xs{};
+  bool vec_ok = false;
+  const int rc = fill_args(d, &a, &xs, &vec_ok);
+  if (rc != TMQ_OK || d->M == 0 || d->N == 0) return rc;
+  if (d->y == nullptr || d->w_scales == nullptr || d->ldy < d->N) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!(d->x_scale > 0.f) || !(d->out_scale > 0.f)) return TMQ_ERR_INVALID_ARGUMENT;
+  const int qmin = d->out_signed ? -128 : 0, qmax = d->out_signed ? 127 : 255;
+  if (d->out_zero_point < qmin || d->out_zero_point > qmax) return TMQ_ERR_INVALID_ARGUMENT;
+  a.w_scales = d->w_scales;
+  a.w_scale_stride = d->w_per_channel ? 1 : 0;
+  a.bias = d->bias;
+  a.acc_coef = (d->x_signed ? 0 : 128) - d->x_zero_point;
+  a.x_scale = d->x_scale;
+  a.out_scale = d->out_scale;
+  a.zp_f = static_cast<float>(d->out_zero_point);
+  a.lo_f = static_cast<float>(d->relu ? d->out_zero_point : qmin);
+  a.hi_f = static_cast<float>(qmax);
+  a.y = d->y;
+  a.ldy = d->ldy;
+  hipStream_t s = as_stream(stream);
+  return d->out_signed ? dispatch_linear<kOutS8>(a, xs, d->x_signed, vec_ok, s)
+                       : dispatch_linear<kOutU8>(a, xs, d->x_signed, vec_ok, s);
+}
+
+TMQ_EXPORT int tmq_linear_acc32(const tmq_linear_desc* d, int32_t* acc, int64_t ldacc,
+                                tmq_stream_t stream) {
+  GemmArgs a{};
+  XLinear xs{};
+  bool vec_ok = false;
+  const int rc = fill_args(d, &a, &xs, &vec_ok);
+  if (rc != TMQ_OK || d->M == 0 || d->N == 0) return rc;
+  if (acc == nullptr || ldacc < d->N) return TMQ_ERR_INVALID_ARGUMENT;
+  a.acc_coef = d->x_signed ? 0 : 128;  // undo the x ^ 0x80 shift only
+  a.y = acc;
+  a.ldy = ldacc;
+  return dispatch_linear<kOutAcc32>(a, xs, d->x_signed, vec_ok, as_stream(stream));
+}
+
+// Benchmark hook (not part of the public header): force a kernel
+// configuration, -1 restores automatic selection.
+TMQ_EXPORT void tmq_debug_force_linear_config(int cfg) {
+  g_forced_config.store(cfg, std::memory_order_relaxed);
+}

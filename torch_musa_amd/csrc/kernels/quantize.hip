@@ -1,0 +1,567 @@
+// Affine quantize / dequantize / range calibration for gfx950.
+//
+// All of these are HBM-streaming kernels: 5 bytes of traffic per element for
+// quantize and dequantize (4 + 1), 4 for min/max.  Every wave instruction
+// touches one dense run of memory: a lane moves 16 bytes of fp32 and the
+// matching 4 bytes of codes, so loads and stores are both fully coalesced, and
+// each thread keeps several independent 16-byte accesses in flight.
+//
+// Numerics follow PyTorch's CPU quantizer (fbgemm/QuantUtils.h:67-101,155-158):
+// multiply by the fp32 reciprocal of the fp32 scale, round half to even, add
+// the zero point, clamp.  Compiled with -ffp-contract=off.
+#include <cmath>
+#include <limits>
+
+#include "common.h"
+
+namespace tmq {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 8;  // independent 16-byte accesses per thread
+
+template <bool SIGNED>
+__device__ __forceinline__ int quantize_one(float x, float inv, float zp_f) {
+  constexpr float lo = SIGNED ? -128.f : 0.f;
+  constexpr float hi = SIGNED ? 127.f : 255.f;
+  float t = x * inv;
+  float r = __builtin_rintf(t);  // v_rndne_f32: ties to even
+  // zp_f and every in-range r are small integers, so the sum is exact whenever
+  // it can land inside [lo, hi]; larger magnitudes clamp either way.
+  r = r + zp_f;
+  r = fminf(fmaxf(r, lo), hi);
+  return static_cast<int>(r);
+}
+
+template <bool SIGNED>
+__device__ __forceinline__ uint32_t quantize_four(v4f v, float inv, float zp_f) {
+  uint32_t a = static_cast<uint32_t>(quantize_one<SIGNED>(v.x, inv, zp_f)) & 0xffu;
+  uint32_t b = static_cast<uint32_t>(quantize_one<SIGNED>(v.y, inv, zp_f)) & 0xffu;
+  uint32_t c = static_cast<uint32_t>(quantize_one<SIGNED>(v.z, inv, zp_f)) & 0xffu;
+  uint32_t d = static_cast<uint32_t>(quantize_one<SIGNED>(v.w, inv, zp_f)) & 0xffu;
+  return a | (b << 8) | (c << 16) | (d << 24);
+}
+
+template <bool SIGNED>
+__device__ __forceinline__ float dequantize_one(uint32_t byte, int zp, float scale) {
+  int v = SIGNED ? static_cast<int>(static_cast<int8_t>(byte)) : static_cast<int>(byte);
+  return scale * static_cast<float>(v - zp);
+}
+
+template <bool SIGNED>
+__device__ __forceinline__ v4f dequantize_four(uint32_t w, int zp, float scale) {
+  v4f r;
+  r.x = dequantize_one<SIGNED>(w & 0xffu, zp, scale);
+  r.y = dequantize_one<SIGNED>((w >> 8) & 0xffu, zp, scale);
+  r.z = dequantize_one<SIGNED>((w >> 16) & 0xffu, zp, scale);
+  r.w = dequantize_one<SIGNED>(w >> 24, zp, scale);
+  return r;
+}
+
+// Where the scale / zero point come from: kernel arguments, or device memory
+// written earlier on the stream by choose_qparams_kernel.
+struct QParamsArg {
+  float inv;
+  float zp_f;
+  const tmq_qparams* dev;
+};
+
+__device__ __forceinline__ void resolve(const QParamsArg& a, float& inv, float& zp_f) {
+  if (a.dev != nullptr) {
+    inv = 1.0f / static_cast<float>(a.dev->scale);  // IEEE division
+    zp_f = static_cast<float>(a.dev->zero_point);
+  } else {
+    inv = a.inv;
+    zp_f = a.zp_f;
+  }
+}
+
+// x4/q4 view the first 4*n4 elements; the block with index 0 also converts the
+// n - 4*n4 (< 4) trailing elements one by one.
+template <bool SIGNED>
+__global__ __launch_bounds__(kThreads) void quantize_vec_kernel(
+    const v4f* __restrict__ x4, uint32_t* __restrict__ q4, int64_t n4,
+    const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, QParamsArg qp) {
+  float inv, zp_f;
+  resolve(qp, inv, zp_f);
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+  v4f v[kUnroll];
+  if (base - threadIdx.x + kThreads * kUnroll <= n4) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) v[u] = __builtin_nontemporal_load(&x4[base + u * kThreads]);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      __builtin_nontemporal_store(quantize_four<SIGNED>(v[u], inv, zp_f), &q4[base + u * kThreads]);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < n4) v[u] = x4[i];
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < n4) q4[i] = quantize_four<SIGNED>(v[u], inv, zp_f);
+    }
+  }
+  if (blockIdx.x == 0) {
+    const int64_t i = 4 * n4 + threadIdx.x;
+    if (i < n) q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(x[i], inv, zp_f));
+  }
+}
+
+// Fallback for pointers that are not 16-byte (x) / 4-byte (q) aligned.
+template <bool SIGNED>
+__global__ __launch_bounds__(kThreads) void quantize_scalar_kernel(
+    const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, QParamsArg qp) {
+  float inv, zp_f;
+  resolve(qp, inv, zp_f);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride)
+    q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(x[i], inv, zp_f));
+}
+
+template <bool SIGNED>
+__global__ __launch_bounds__(kThreads) void dequantize_vec_kernel(
+    const uint32_t* __restrict__ q4, v4f* __restrict__ r4, int64_t n4,
+    const uint8_t* __restrict__ q, float* __restrict__ r, int64_t n, float scale, int zp) {
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+  uint32_t w[kUnroll];
+  if (base - threadIdx.x + kThreads * kUnroll <= n4) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) w[u] = __builtin_nontemporal_load(&q4[base + u * kThreads]);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      __builtin_nontemporal_store(dequantize_four<SIGNED>(w[u], zp, scale), &r4[base + u * kThreads]);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < n4) w[u] = q4[i];
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < n4) r4[i] = dequantize_four<SIGNED>(w[u], zp, scale);
+    }
+  }
+  if (blockIdx.x == 0) {
+    const int64_t i = 4 * n4 + threadIdx.x;
+    if (i < n) r[i] = dequantize_one<SIGNED>(q[i], zp, scale);
+  }
+}
+
+template <bool SIGNED>
+__global__ __launch_bounds__(kThreads) void dequantize_scalar_kernel(
+    const uint8_t* __restrict__ q, float* __restrict__ r, int64_t n, float scale, int zp) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride)
+    r[i] = dequantize_one<SIGNED>(q[i], zp, scale);
+}
+
+// ---------------------------------------------------------------------------
+// min / max: persistent grid, 16-byte loads, wavefront butterfly reduction,
+// one {min,max} pair per block, then a one-block second stage.
+// ---------------------------------------------------------------------------
+constexpr int kMinMaxMaxBlocks = 2048;
+
+__device__ __forceinline__ void wave_minmax(float& mn, float& mx) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, off, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+  }
+}
+
+__device__ __forceinline__ void block_minmax_store(float mn, float mx, float* out) {
+  __shared__ float s_mn[kThreads / kWave];
+  __shared__ float s_mx[kThreads / kWave];
+  wave_minmax(mn, mx);
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (lane == 0) {
+    s_mn[wave] = mn;
+    s_mx[wave] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kThreads / kWave; ++w) {
+      mn = fminf(mn, s_mn[w]);
+      mx = fmaxf(mx, s_mx[w]);
+    }
+    out[0] = mn;
+    out[1] = mx;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void minmax_partial_kernel(
+    const v4f* __restrict__ x4, int64_t n4, const float* __restrict__ x, int64_t head,
+    int64_t n, float* __restrict__ partials) {
+  float mn = std::numeric_limits<float>::infinity();
+  float mx = -std::numeric_limits<float>::infinity();
+  const int64_t step = static_cast<int64_t>(gridDim.x) * (kThreads * kUnroll);
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+       base - threadIdx.x < n4; base += step) {
+    v4f v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < n4) v[u] = __builtin_nontemporal_load(&x4[i]);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < n4) {
+        mn = fminf(fminf(mn, v[u].x), fminf(v[u].y, fminf(v[u].z, v[u].w)));
+        mx = fmaxf(fmaxf(mx, v[u].x), fmaxf(v[u].y, fmaxf(v[u].z, v[u].w)));
+      }
+    }
+  }
+  if (blockIdx.x == 0) {
+    // elements before the first 16-byte boundary and after the last full group
+    const int64_t tail0 = head + 4 * n4;
+    const int64_t extra = head + (n - tail0);
+    for (int64_t j = threadIdx.x; j < extra; j += kThreads) {
+      const float v = j < head ? x[j] : x[tail0 + (j - head)];
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+  }
+  block_minmax_store(mn, mx, partials + 2 * blockIdx.x);
+}
+
+__global__ __launch_bounds__(kThreads) void minmax_final_kernel(
+    const float* __restrict__ partials, int count, float* __restrict__ out) {
+  float mn = std::numeric_limits<float>::infinity();
+  float mx = -std::numeric_limits<float>::infinity();
+  for (int i = threadIdx.x; i < count; i += kThreads) {
+    mn = fminf(mn, partials[2 * i]);
+    mx = fmaxf(mx, partials[2 * i + 1]);
+  }
+  block_minmax_store(mn, mx, out);
+}
+
+// ChooseQuantizationParams, shared by host and device
+// (ATen/native/quantized/cpu/QuantUtils.h:71-187).
+__host__ __device__ inline void choose_qparams(float min, float max, int qmin, int qmax,
+                                               bool reduce_range, double* out_scale,
+                                               int32_t* out_zp) {
+  if (reduce_range) {
+    qmin = qmin / 2;
+    qmax = qmax / 2;
+  }
+  min = fminf(min, 0.f);
+  max = fmaxf(max, 0.f);
+  double scale = (static_cast<double>(max) - min) / (qmax - qmin);
+  const float scale_f = static_cast<float>(scale);
+  if (scale_f == 0.0f || __builtin_isinf(1.0f / scale_f)) scale = 0.1;
+  constexpr float kSmall = 6.1e-5f;
+  if (scale < kSmall) {
+    const float org_scale = static_cast<float>(scale);
+    scale = kSmall;
+    if (min == 0.0f) {
+      max = kSmall * (qmax - qmin);
+    } else if (max == 0.0f) {
+      min = -kSmall * (qmax - qmin);
+    } else {
+      const float amplifier = kSmall / org_scale;
+      min *= amplifier;
+      max *= amplifier;
+    }
+  }
+  const double zp_from_min = qmin - min / scale;
+  const double zp_from_max = qmax - max / scale;
+  const double err_min = (qmin < 0 ? -qmin : qmin) - fabs(min / scale);
+  const double err_max = (qmax < 0 ? -qmax : qmax) - fabs(max / scale);
+  const double initial = err_min < err_max ? zp_from_min : zp_from_max;
+  int32_t nudged;
+  if (initial < qmin) {
+    nudged = qmin;
+  } else if (initial > qmax) {
+    nudged = qmax;
+  } else {
+    nudged = static_cast<int32_t>(rint(initial));
+  }
+  *out_scale = scale;
+  *out_zp = nudged;
+}
+
+__global__ void choose_qparams_kernel(const float* __restrict__ minmax, int qmin, int qmax,
+                                      int reduce_range, tmq_qparams* __restrict__ out) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    double s;
+    int32_t z;
+    choose_qparams(minmax[0], minmax[1], qmin, qmax, reduce_range != 0, &s, &z);
+    out->scale = s;
+    out->zero_point = z;
+    out->reserved = 0;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Per-channel kernels over [outer, C, inner].  VEC = 4 when inner % 4 == 0 and
+// the pointers are 16-byte aligned (a group of 4 never straddles a channel).
+// ---------------------------------------------------------------------------
+template <bool SIGNED, int VEC>
+__global__ __launch_bounds__(kThreads) void quantize_pc_kernel(
+    const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, int64_t C, int64_t inner,
+    const double* __restrict__ scales, const int64_t* __restrict__ zps) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads * VEC;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * VEC; i < n;
+       i += stride) {
+    const int64_t c = (i / inner) % C;
+    const float inv = 1.0f / static_cast<float>(scales[c]);
+    const float zp_f = static_cast<float>(zps[c]);
+    if constexpr (VEC == 4) {
+      const v4f v = *reinterpret_cast<const v4f*>(x + i);
+      *reinterpret_cast<uint32_t*>(q + i) = quantize_four<SIGNED>(v, inv, zp_f);
+    } else {
+      q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(x[i], inv, zp_f));
+    }
+  }
+}
+
+template <bool SIGNED>
+__device__ __forceinline__ float dequantize_pc_one(uint32_t byte, float zp_f, double scale) {
+  const int v = SIGNED ? static_cast<int>(static_cast<int8_t>(byte)) : static_cast<int>(byte);
+  const float d = static_cast<float>(v) - zp_f;
+  return static_cast<float>(static_cast<double>(d) * scale);
+}
+
+template <bool SIGNED, int VEC>
+__global__ __launch_bounds__(kThreads) void dequantize_pc_kernel(
+    const uint8_t* __restrict__ q, float* __restrict__ r, int64_t n, int64_t C, int64_t inner,
+    const double* __restrict__ scales, const int64_t* __restrict__ zps) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads * VEC;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * VEC; i < n;
+       i += stride) {
+    const int64_t c = (i / inner) % C;
+    const double scale = scales[c];
+    const float zp_f = static_cast<float>(zps[c]);
+    if constexpr (VEC == 4) {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(q + i);
+      v4f o;
+      o.x = dequantize_pc_one<SIGNED>(w & 0xffu, zp_f, scale);
+      o.y = dequantize_pc_one<SIGNED>((w >> 8) & 0xffu, zp_f, scale);
+      o.z = dequantize_pc_one<SIGNED>((w >> 16) & 0xffu, zp_f, scale);
+      o.w = dequantize_pc_one<SIGNED>(w >> 24, zp_f, scale);
+      *reinterpret_cast<v4f*>(r + i) = o;
+    } else {
+      r[i] = dequantize_pc_one<SIGNED>(q[i], zp_f, scale);
+    }
+  }
+}
+
+inline unsigned grid_for(int64_t work_items, int64_t per_block, int64_t cap) {
+  int64_t g = ceil_div(work_items, per_block);
+  if (g < 1) g = 1;
+  if (g > cap) g = cap;
+  return static_cast<unsigned>(g);
+}
+
+int quantize_launch(const float* x, void* q, int64_t n, QParamsArg qp, int q_signed,
+                    hipStream_t s) {
+  if (n == 0) return TMQ_OK;
+  uint8_t* qb = static_cast<uint8_t*>(q);
+  if (aligned(x, 16) && aligned(q, 4)) {
+    const int64_t n4 = n / 4;
+    const int64_t blocks = n4 == 0 ? 1 : ceil_div(n4, kThreads * kUnroll);
+    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    auto* x4 = reinterpret_cast<const v4f*>(x);
+    auto* q4 = reinterpret_cast<uint32_t*>(q);
+    if (q_signed)
+      quantize_vec_kernel<true><<<dim3(blocks), dim3(kThreads), 0, s>>>(x4, q4, n4, x, qb, n, qp);
+    else
+      quantize_vec_kernel<false><<<dim3(blocks), dim3(kThreads), 0, s>>>(x4, q4, n4, x, qb, n, qp);
+  } else {
+    const unsigned g = grid_for(n, kThreads, 65536);
+    if (q_signed)
+      quantize_scalar_kernel<true><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, qp);
+    else
+      quantize_scalar_kernel<false><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, qp);
+  }
+  return launch_status();
+}
+
+bool zp_in_range(int64_t zp, int q_signed) {
+  return q_signed ? (zp >= -128 && zp <= 127) : (zp >= 0 && zp <= 255);
+}
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+TMQ_EXPORT int tmq_quantize_per_tensor(const float* x, void* q, int64_t n, double scale,
+                                       int64_t zero_point, int q_signed, tmq_stream_t stream) {
+  if (n < 0 || (n > 0 && (x == nullptr || q == nullptr))) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!zp_in_range(zero_point, q_signed)) return TMQ_ERR_INVALID_ARGUMENT;
+  QParamsArg qp;
+  qp.inv = 1.0f / static_cast<float>(scale);
+  qp.zp_f = static_cast<float>(zero_point);
+  qp.dev = nullptr;
+  return quantize_launch(x, q, n, qp, q_signed, as_stream(stream));
+}
+
+TMQ_EXPORT int tmq_quantize_per_tensor_dev(const float* x, void* q, int64_t n,
+                                           const tmq_qparams* qparams, int q_signed,
+                                           tmq_stream_t stream) {
+  if (n < 0 || qparams == nullptr || (n > 0 && (x == nullptr || q == nullptr)))
+    return TMQ_ERR_INVALID_ARGUMENT;
+  QParamsArg qp;
+  qp.inv = 0.f;
+  qp.zp_f = 0.f;
+  qp.dev = qparams;
+  return quantize_launch(x, q, n, qp, q_signed, as_stream(stream));
+}
+
+TMQ_EXPORT int tmq_dequantize_per_tensor(const void* q, float* r, int64_t n, double scale,
+                                         int64_t zero_point, int q_signed, tmq_stream_t stream) {
+  if (n < 0 || (n > 0 && (r == nullptr || q == nullptr))) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!zp_in_range(zero_point, q_signed)) return TMQ_ERR_INVALID_ARGUMENT;
+  if (n == 0) return TMQ_OK;
+  hipStream_t s = as_stream(stream);
+  const float scale_f = static_cast<float>(scale);
+  const int zp = static_cast<int>(zero_point);
+  const uint8_t* qb = static_cast<const uint8_t*>(q);
+  if (aligned(r, 16) && aligned(q, 4)) {
+    const int64_t n4 = n / 4;
+    const int64_t blocks = n4 == 0 ? 1 : ceil_div(n4, kThreads * kUnroll);
+    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    auto* q4 = reinterpret_cast<const uint32_t*>(q);
+    auto* r4 = reinterpret_cast<v4f*>(r);
+    if (q_signed)
+      dequantize_vec_kernel<true><<<dim3(blocks), dim3(kThreads), 0, s>>>(q4, r4, n4, qb, r, n, scale_f, zp);
+    else
+      dequantize_vec_kernel<false><<<dim3(blocks), dim3(kThreads), 0, s>>>(q4, r4, n4, qb, r, n, scale_f, zp);
+  } else {
+    const unsigned g = grid_for(n, kThreads, 65536);
+    if (q_signed)
+      dequantize_scalar_kernel<true><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, scale_f, zp);
+    else
+      dequantize_scalar_kernel<false><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, scale_f, zp);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT size_t tmq_minmax_workspace_bytes(int64_t n) {
+  (void)n;
+  return static_cast<size_t>(kMinMaxMaxBlocks) * 2 * sizeof(float);
+}
+
+TMQ_EXPORT int tmq_minmax(const float* x, int64_t n, float* minmax, void* workspace,
+                          size_t workspace_bytes, tmq_stream_t stream) {
+  if (n < 0 || minmax == nullptr || (n > 0 && x == nullptr)) return TMQ_ERR_INVALID_ARGUMENT;
+  if (workspace == nullptr || workspace_bytes < tmq_minmax_workspace_bytes(n) ||
+      !aligned(workspace, 4))
+    return TMQ_ERR_WORKSPACE;
+  if (!aligned(x, 4)) return TMQ_ERR_ALIGNMENT;
+  hipStream_t s = as_stream(stream);
+  float* partials = static_cast<float*>(workspace);
+  // elements before the first 16-byte boundary are handled one by one
+  int64_t head = 0;
+  if (n > 0) {
+    const uintptr_t mis = reinterpret_cast<uintptr_t>(x) & 15u;
+    head = mis == 0 ? 0 : static_cast<int64_t>((16 - mis) / 4);
+    if (head > n) head = n;
+  }
+  const int64_t n4 = (n - head) / 4;
+  const unsigned g = grid_for(n4, kThreads * kUnroll, kMinMaxMaxBlocks);
+  minmax_partial_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(
+      reinterpret_cast<const v4f*>(x + head), n4, x, head, n, partials);
+  if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  minmax_final_kernel<<<dim3(1), dim3(kThreads), 0, s>>>(partials, static_cast<int>(g), minmax);
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_choose_qparams_dev(const float* minmax, int q_signed, int reduce_range,
+                                      tmq_qparams* qparams, tmq_stream_t stream) {
+  if (minmax == nullptr || qparams == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  choose_qparams_kernel<<<dim3(1), dim3(kWave), 0, as_stream(stream)>>>(
+      minmax, q_signed ? -128 : 0, q_signed ? 127 : 255, reduce_range, qparams);
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_choose_qparams_host(float min, float max, int q_signed, int reduce_range,
+                                       double* scale, int32_t* zero_point) {
+  if (scale == nullptr || zero_point == nullptr || !(min <= max)) return TMQ_ERR_INVALID_ARGUMENT;
+  choose_qparams(min, max, q_signed ? -128 : 0, q_signed ? 127 : 255, reduce_range != 0, scale,
+                 zero_point);
+  return TMQ_OK;
+}
+
+namespace {
+bool pc_args_ok(const void* a, const void* b, int64_t outer, int64_t C, int64_t inner,
+                const double* scales, const int64_t* zps) {
+  if (outer < 0 || C < 0 || inner < 0) return false;
+  const bool empty = outer == 0 || C == 0 || inner == 0;
+  if (!empty && (a == nullptr || b == nullptr || scales == nullptr || zps == nullptr)) return false;
+  return true;
+}
+}  // namespace
+
+TMQ_EXPORT int tmq_quantize_per_channel(const float* x, void* q, int64_t outer, int64_t channels,
+                                        int64_t inner, const double* scales,
+                                        const int64_t* zero_points, int q_signed,
+                                        tmq_stream_t stream) {
+  if (!pc_args_ok(x, q, outer, channels, inner, scales, zero_points))
+    return TMQ_ERR_INVALID_ARGUMENT;
+  const int64_t n = outer * channels * inner;
+  if (n == 0) return TMQ_OK;
+  hipStream_t s = as_stream(stream);
+  uint8_t* qb = static_cast<uint8_t*>(q);
+  const bool vec = inner % 4 == 0 && aligned(x, 16) && aligned(q, 4);
+  const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
+  if (vec) {
+    if (q_signed)
+      quantize_pc_kernel<true, 4><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+    else
+      quantize_pc_kernel<false, 4><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+  } else {
+    if (q_signed)
+      quantize_pc_kernel<true, 1><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+    else
+      quantize_pc_kernel<false, 1><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_dequantize_per_channel(const void* q, float* r, int64_t outer, int64_t channels,
+                                          int64_t inner, const double* scales,
+                                          const int64_t* zero_points, int q_signed,
+                                          tmq_stream_t stream) {
+  if (!pc_args_ok(q, r, outer, channels, inner, scales, zero_points))
+    return TMQ_ERR_INVALID_ARGUMENT;
+  const int64_t n = outer * channels * inner;
+  if (n == 0) return TMQ_OK;
+  hipStream_t s = as_stream(stream);
+  const uint8_t* qb = static_cast<const uint8_t*>(q);
+  const bool vec = inner % 4 == 0 && aligned(r, 16) && aligned(q, 4);
+  const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
+  if (vec) {
+    if (q_signed)
+      dequantize_pc_kernel<true, 4><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+    else
+      dequantize_pc_kernel<false, 4><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+  } else {
+    if (q_signed)
+      dequantize_pc_kernel<true, 1><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+    else
+      dequantize_pc_kernel<false, 1><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT const char* tmq_status_string(int status) {
+  switch (status) {
+    case TMQ_OK: return "ok";
+    case TMQ_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case TMQ_ERR_UNSUPPORTED: return "unsupported configuration";
+    case TMQ_ERR_WORKSPACE: return "workspace missing or too small";
+    case TMQ_ERR_LAUNCH: return "HIP launch failed";
+    case TMQ_ERR_ALIGNMENT: return "pointer or leading dimension not aligned";
+    default: return "unknown status";
+  }
+}
+
+TMQ_EXPORT int tmq_version(void) { return TMQ_VERSION; }
