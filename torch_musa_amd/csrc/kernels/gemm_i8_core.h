@@ -22,8 +22,7 @@
 //               ((row >> 1) ^ (row >> 3)) & 3, so that both the row-major fill
 //               and the column-wise operand reads of any 8 or 16 consecutive
 //               lanes fall into distinct 16-byte bank groups
-// Pipeline per stage: registers -> LDS for stage t+1, global -> registers for
-// stage t+2, MFMAs on stage t, one barrier.
+// Pipeline: see the comment at the software pipeline inside gemm_i8_kernel.
 #pragma once
 
 #include "common.h"
@@ -75,19 +74,20 @@ template <class XSRC>
 struct XLoader;
 
 // One loader per 16-byte chunk slot a thread stages: fixed activation row,
-// k-chunk index `kc` supplied per stage.
+// k-chunk index `kc` supplied per stage.  Loads are never predicated: rows past
+// M are clamped to the last row (their results are never stored) and k-chunks
+// past K to the last chunk (the packed weight is zero there), so that every
+// stage issues the same number of loads and the wait counters stay exact.
 template <>
 struct XLoader<XLinear> {
   const uint8_t* p;
-  bool row_ok;
   __device__ __forceinline__ void init(const XLinear& s, int64_t m, int64_t M) {
-    row_ok = m < M;
-    p = s.x + (row_ok ? m : 0) * s.ldx;
+    p = s.x + (m < M ? m : M - 1) * s.ldx;
   }
   __device__ __forceinline__ v4i load(const XLinear&, int kc, int64_t K) const {
-    const int64_t k = static_cast<int64_t>(kc) * 16;
-    if (row_ok && k < K) return ld16(p + k);
-    return v4i{0, 0, 0, 0};
+    int64_t k = static_cast<int64_t>(kc) * 16;
+    k = k < K ? k : K - 16;
+    return ld16(p + k);
   }
 };
 
@@ -95,10 +95,8 @@ template <>
 struct XLoader<XConv> {
   const uint8_t* img;  // first byte of this row's image (+ group channel offset)
   int ih0, iw0;        // top-left input coordinate of the receptive field
-  bool row_ok;
   __device__ __forceinline__ void init(const XConv& s, int64_t m, int64_t M) {
-    row_ok = m < M;
-    const int64_t mm = row_ok ? m : 0;
+    const int64_t mm = m < M ? m : M - 1;
     const int ow = static_cast<int>(mm % s.OW);
     const int64_t t = mm / s.OW;
     const int oh = static_cast<int>(t % s.OH);
@@ -110,16 +108,17 @@ struct XLoader<XConv> {
   // Out-of-image taps read as the activation zero point, i.e. real value 0.
   __device__ __forceinline__ v4i load(const XConv& s, int kc, int64_t K) const {
     const int pw = static_cast<int>(s.pad_word);
-    const v4i pad = {pw, pw, pw, pw};
-    if (!row_ok || static_cast<int64_t>(kc) * 16 >= K) return pad;
-    const int tap = kc / s.icb;
-    const int blk = kc - tap * s.icb;
+    const int kcc = static_cast<int64_t>(kc) * 16 < K ? kc : 0;
+    const int tap = kcc / s.icb;
+    const int blk = kcc - tap * s.icb;
     const int kh = tap / s.KW;
     const int kw = tap - kh * s.KW;
     const int ih = ih0 + kh * s.dil_h;
     const int iw = iw0 + kw * s.dil_w;
-    if (ih < 0 || ih >= s.H || iw < 0 || iw >= s.W) return pad;
-    return ld16(img + (static_cast<int64_t>(ih) * s.W + iw) * s.IC + blk * 16);
+    const bool inside = ih >= 0 && ih < s.H && iw >= 0 && iw < s.W;
+    const int ihc = inside ? ih : 0, iwc = inside ? iw : 0;
+    const v4i v = ld16(img + (static_cast<int64_t>(ihc) * s.W + iwc) * s.IC + blk * 16);
+    return v4i{inside ? v.x : pw, inside ? v.y : pw, inside ? v.z : pw, inside ? v.w : pw};
   }
 };
 
@@ -148,22 +147,34 @@ __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, v4f 
 }
 
 // BM x BN output tile per block (BM activation rows, BN weight rows),
-// WM x WN waves, each wave (BM/WM) x (BN/WN).
-template <int BM, int BN, int WM, int WN, int MODE, class XSRC>
+// WM x WN waves, each wave (BM/WM) x (BN/WN).  PD = prefetch distance in
+// stages: the global loads of stage t+PD are issued while stage t is being
+// multiplied, so PD-1 stages of 16-byte loads are in flight per thread.
+template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4>
 __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int NT = WM * WN * kWave;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int NW = BN * kChunks / NT;  // 16-byte weight chunks per thread per stage
   constexpr int NX = BM * kChunks / NT;
+  constexpr int NSET = PD - 1;           // register sets holding stages in flight
   static_assert(TM >= 1 && TN >= 1 && NW >= 1 && NX >= 1, "tile too small for the wave grid");
   static_assert(BN * kChunks % NT == 0 && BM * kChunks % NT == 0, "uneven staging");
+  static_assert(PD >= 3, "prefetch distance");
 
-  __shared__ __attribute__((aligned(16))) uint8_t sW[2][kChunks * BN * 16];
-  __shared__ __attribute__((aligned(16))) uint8_t sX[2][BM * kBK];
+  // LDS: two stages of {weights, activations}; the same bytes are reused after
+  // the main loop to transpose the output tile into row-major order.
+  constexpr int kWStage = kChunks * BN * 16, kXStage = BM * kBK;
+  constexpr int kOutPitch = BN + 16;  // bytes; keeps rows 16-byte aligned and off one bank
+  constexpr int kMainBytes = 2 * (kWStage + kXStage);
+  constexpr int kOutBytes = (MODE == kOutAcc32) ? 0 : BM * kOutPitch;
+  constexpr int kTileBytes = kMainBytes > kOutBytes ? kMainBytes : kOutBytes;
+  __shared__ __attribute__((aligned(16))) uint8_t smem[kTileBytes];
   __shared__ __attribute__((aligned(16))) int s_acc0[BN];
   __shared__ __attribute__((aligned(16))) float s_mult[BN];
   __shared__ __attribute__((aligned(16))) float s_bdiv[BN];
+  uint8_t* const sW = smem;                 // [2][kWStage]
+  uint8_t* const sX = smem + 2 * kWStage;   // [2][kXStage]
 
   const int t = threadIdx.x;
   const int lane = t % kWave, wave = t / kWave;
@@ -205,17 +216,16 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     s_bdiv[i] = bdiv;
   }
 
-  // ---- staging assignments
+  // ---- staging assignments (weight rows past N are clamped: never stored)
   const uint8_t* wsrc[NW];
-  bool wok[NW];
   int wdst[NW];
 #pragma unroll
   for (int i = 0; i < NW; ++i) {
     const int id = t + i * NT;
     const int nbl = id >> 6, kcl = (id >> 4) & 3, r = id & 15;
-    const int64_t nb = n0 / 16 + nbl;
-    wok[i] = nb < NB;
-    wsrc[i] = a.w_packed + ((wok[i] ? nb : 0) * a.w_kchunks + kcl) * 256 + r * 16;
+    int64_t nb = n0 / 16 + nbl;
+    nb = nb < NB ? nb : NB - 1;
+    wsrc[i] = a.w_packed + (nb * a.w_kchunks + kcl) * 256 + r * 16;
     wdst[i] = (kcl * BN + nbl * 16 + r) * 16;
   }
   XLoader<XSRC> xl[NX];
@@ -225,33 +235,29 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     const int id = t + i * NT;
     const int row = id >> 2, c = id & 3;
     xl[i].init(xsrc, m0 + row, a.M);
-    xdst[i] = row * kBK + ((c ^ x_swizzle(row)) << 4);
+    xdst[i] = 2 * kWStage + row * kBK + ((c ^ x_swizzle(row)) << 4);
   }
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
 
-  v4i wreg[NW], xreg[NX];
-  auto load_global = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < NW; ++i)
-      wreg[i] = wok[i] ? ld16(wsrc[i] + static_cast<int64_t>(kt) * (kChunks * 256)) : v4i{0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < NX; ++i) xreg[i] = xl[i].load(xsrc, kt * kChunks + (t & 3), a.K);
+  v4i wreg[NSET][NW], xreg[NSET][NX];
+  // k-th global load of a stage (weights first, then activations)
+  auto load_one = [&](int set, int kt, int k) {
+    if (k < NW)
+      wreg[set][k] = ld16(wsrc[k] + static_cast<int64_t>(kt) * (kChunks * 256));
+    else
+      xreg[set][k - NW] = xl[k - NW].load(xsrc, kt * kChunks + (t & 3), a.K);
   };
-  auto store_lds = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < NW; ++i) *reinterpret_cast<v4i*>(&sW[buf][wdst[i]]) = wreg[i];
-#pragma unroll
-    for (int i = 0; i < NX; ++i) *reinterpret_cast<v4i*>(&sX[buf][xdst[i]]) = xreg[i] ^ xmask;
+  // k-th LDS store of a stage
+  auto store_one = [&](int set, int buf, int k) {
+    if (k < NW)
+      *reinterpret_cast<v4i*>(&smem[buf * kWStage + wdst[k]]) = wreg[set][k];
+    else
+      *reinterpret_cast<v4i*>(&smem[buf * kXStage + xdst[k - NW]]) = xreg[set][k - NW] ^ xmask;
   };
-
-  const int KT = static_cast<int>(ceil_div(a.K, kBK));
-  load_global(0);
-  store_lds(0);
-  if (KT > 1) load_global(1);
-  __syncthreads();
 
   // ---- accumulators start at the per-channel offset (see file header)
+  __syncthreads();  // s_acc0 / s_mult / s_bdiv are written
   v16i acc[TN][TM];
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
@@ -263,41 +269,103 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = init;
   }
 
+  // ---- software pipeline.
+  // Stage t of the k loop = 64 k-bytes = two MFMA k-steps.  The schedule of one
+  // stage, written out in issue order with one memory operation per MFMA so
+  // that the matrix pipe never waits for the other pipes:
+  //   first half   MFMAs of k-step 0 (fragments already in registers)
+  //                + LDS reads of the k-step 1 fragments of stage t
+  //                + global loads of stage t+PD into a free register set
+  //   barrier      (stage t+1 is now visible in LDS; buffer t&1 is dead)
+  //   second half  MFMAs of k-step 1
+  //                + LDS reads of the k-step 0 fragments of stage t+1
+  //                + LDS stores of stage t+2 (loaded PD-2 stages ago) into buffer t&1
+  // Stage s lives in register set s % NSET and in LDS buffer s & 1.  Every
+  // operation is unconditional: past the last stage it touches valid memory
+  // and its result is never consumed, so the compiler's count of outstanding
+  // loads stays exact (a predicated load would force it to drain them all).
+  // The scheduling fences keep this order; without them the compiler sinks the
+  // global loads to the end of the stage and loses the prefetch distance.
+  const int KT = static_cast<int>(ceil_div(a.K, kBK));
+  auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };
   const int xswz = x_swizzle(li);
-  for (int kt = 0; kt < KT; ++kt) {
+  v4i wf0[TN], xf0[TM], wf1[TN], xf1[TM];
+  // j-th fragment read of a k-step (weights first, then activations)
+  auto read_one = [&](int buf, int s, int j, v4i(&wf)[TN], v4i(&xf)[TM]) {
+    const int c = 2 * s + half;
+    if (j < TN)
+      wf[j] = ld16(&sW[buf * kWStage + (c * BN + wn0 + j * 32 + li) * 16]);
+    else
+      xf[j - TN] = ld16(&sX[buf * kXStage + (wm0 + (j - TN) * 32 + li) * kBK + ((c ^ xswz) << 4)]);
+  };
+  constexpr int Q = TN * TM;    // MFMAs per k-step
+  constexpr int NF = TN + TM;   // fragment reads per k-step
+  constexpr int NG = NW + NX;   // global loads (and LDS stores) per stage
+  auto stage = [&](int kt, int load_set, int store_set) {
     const int buf = kt & 1;
-    if (kt + 1 < KT) store_lds(buf ^ 1);
-    if (kt + 2 < KT) load_global(kt + 2);
+    const int kload = clampk(kt + PD);
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const int c = 2 * s + half;
-      v4i wf[TN], xf[TM];
+    for (int q = 0; q < Q; ++q) {
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
-        wf[tn] = ld16(&sW[buf][(c * BN + wn0 + tn * 32 + li) * 16]);
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        xf[tm] = ld16(&sX[buf][(wm0 + tm * 32 + li) * kBK + ((c ^ xswz) << 4)]);
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-          acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[tn], xf[tm], acc[tn][tm], 0, 0, 0);
+      for (int o = q * (NF + NG) / Q; o < (q + 1) * (NF + NG) / Q; ++o) {
+        if (o < NF) read_one(buf, 1, o, wf1, xf1);
+        else load_one(load_set, kload, o - NF);
+      }
+      acc[q / TM][q % TM] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf0[q / TM], xf0[q % TM],
+                                                                 acc[q / TM][q % TM], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
-  }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+#pragma unroll
+      for (int o = q * (NF + NG) / Q; o < (q + 1) * (NF + NG) / Q; ++o) {
+        if (o < NF) read_one(buf ^ 1, 0, o, wf0, xf0);
+        else store_one(store_set, buf, o - NF);
+      }
+      acc[q / TM][q % TM] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf1[q / TM], xf1[q % TM],
+                                                                 acc[q / TM][q % TM], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
 
-  // ---- epilogue: lane holds, per 32x32 tile, rows n = 8g + 4*half + j (g,j <4)
-  // of column m = li.
+  // prologue: stages 0 and 1 into LDS, stages 2 .. PD-1 in flight
 #pragma unroll
-  for (int tn = 0; tn < TN; ++tn) {
+  for (int k = 0; k < NG; ++k) load_one(0, 0, k);
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int nl = wn0 + tn * 32 + 8 * g + 4 * half;
-      const int64_t n = n0 + nl;
-      if (n >= a.N) continue;
-      if constexpr (MODE == kOutAcc32) {
-        int32_t* y = static_cast<int32_t*>(a.y);
+  for (int k = 0; k < NG; ++k) load_one(1 % NSET, clampk(1), k);
+#pragma unroll
+  for (int k = 0; k < NG; ++k) store_one(0, 0, k);
+#pragma unroll
+  for (int s = 2; s < PD; ++s)
+#pragma unroll
+    for (int k = 0; k < NG; ++k) load_one(s % NSET, clampk(s), k);
+  // (with NSET == 2 the loads of stage 2 reuse set 0, already stored above)
+#pragma unroll
+  for (int k = 0; k < NG; ++k) store_one(1 % NSET, 1, k);
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < NF; ++j) read_one(0, 0, j, wf0, xf0);
+
+  int kt0 = 0;
+  for (; kt0 + NSET <= KT; kt0 += NSET) {
+#pragma unroll
+    for (int j = 0; j < NSET; ++j) stage(kt0 + j, (j + 1) % NSET, (j + 2) % NSET);
+  }
+#pragma unroll
+  for (int j = 0; j < NSET - 1; ++j)
+    if (kt0 + j < KT) stage(kt0 + j, (j + 1) % NSET, (j + 2) % NSET);
+
+  // ---- epilogue.  A lane holds, per 32x32 MFMA tile, channels
+  // n = 8g + 4*half + j (g, j < 4) of activation row m = li.
+  if constexpr (MODE == kOutAcc32) {
+    int32_t* y = static_cast<int32_t*>(a.y);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int64_t n = n0 + wn0 + tn * 32 + 8 * g + 4 * half;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
           const int64_t m = m0 + wm0 + tm * 32 + li;
@@ -307,29 +375,45 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
           for (int j = 0; j < 4; ++j)
             if (n + j < a.N) dst[j] = acc[tn][tm][4 * g + j];
         }
-      } else {
+      }
+  } else {
+    // Requantise in registers, transpose through LDS, then write whole rows:
+    // 16 bytes per lane, consecutive lanes on consecutive addresses.
+    __syncthreads();  // every wave is done with the operand stages
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int nl = wn0 + tn * 32 + 8 * g + 4 * half;
         const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[nl]);
         const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[nl]);
-        uint8_t* y = static_cast<uint8_t*>(a.y);
-        const bool full = (n + 3 < a.N) && ((a.ldy & 3) == 0) && ((a.n_off & 3) == 0) &&
-                          ((reinterpret_cast<uintptr_t>(y) & 3) == 0);
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
-          const int64_t m = m0 + wm0 + tm * 32 + li;
-          if (m >= a.M) continue;
           int raw[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * g + j];
-          const uint32_t packed = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
-          uint8_t* dst = y + m * a.ldy + a.n_off + n;
-          if (full) {
-            *reinterpret_cast<uint32_t*>(dst) = packed;
-          } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              if (n + j < a.N) dst[j] = static_cast<uint8_t>(packed >> (8 * j));
-          }
+          *reinterpret_cast<uint32_t*>(&smem[(wm0 + tm * 32 + li) * kOutPitch + nl]) =
+              requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
         }
+      }
+    __syncthreads();
+    uint8_t* y = static_cast<uint8_t*>(a.y) + a.n_off;
+    const bool vec_ok = ((a.ldy & 15) == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+    constexpr int kRowChunks = BN / 16;
+#pragma unroll 4
+    for (int id = t; id < BM * kRowChunks; id += NT) {
+      const int row = id / kRowChunks, cc = id % kRowChunks;
+      const int64_t m = m0 + row, n = n0 + cc * 16;
+      if (m >= a.M || n >= a.N) continue;
+      const v4i v = ld16(&smem[row * kOutPitch + cc * 16]);
+      uint8_t* dst = y + m * a.ldy + n;
+      if (vec_ok && n + 16 <= a.N) {
+        *reinterpret_cast<v4i*>(dst) = v;
+      } else {
+        const uint32_t w[4] = {static_cast<uint32_t>(v.x), static_cast<uint32_t>(v.y),
+                               static_cast<uint32_t>(v.z), static_cast<uint32_t>(v.w)};
+        for (int b = 0; b < 16; ++b)
+          if (n + b < a.N) dst[b] = static_cast<uint8_t>(w[b >> 2] >> (8 * (b & 3)));
       }
     }
   }

@@ -281,7 +281,7 @@ int fill_args(const tmq_linear_desc* d, GemmArgs* a, XLinear* xs, bool* vec_ok) 
   a->n_off = 0;
   xs->x = static_cast<const uint8_t*>(d->x);
   xs->ldx = d->ldx;
-  *vec_ok = d->K % 16 == 0 && d->ldx % 16 == 0 && aligned(d->x, 16);
+  *vec_ok = d->K >= 16 && d->K % 16 == 0 && d->ldx % 16 == 0 && aligned(d->x, 16);
   return TMQ_OK;
 }
 
