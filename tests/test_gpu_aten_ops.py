@@ -1,0 +1,255 @@
+"""The operator-level drop-in: torch.quantize_per_*, Tensor.dequantize and
+torch.ops.quantized.{linear,conv2d}* on GPU tensors, written the way the
+reference's own tests are (tests/unittest/quantized/test_quantized_ops.py:25-99,
+test_quantized_linear.py:52-111, test_quantized_conv.py:83-150: run on CPU, run
+on the device, compare int_repr / dequantize / qparams), plus the CPU-op
+semantics the reference's device path does not have (quint8 activations with a
+zero point, per-channel weights)."""
+import numpy as np
+import pytest
+import torch
+import torch.ao.nn.intrinsic.quantized as nniq
+import torch.ao.nn.quantized as nnq
+
+import cases
+from gpu_util import say
+
+pytestmark = pytest.mark.gpu
+
+LSB_TOL = 1
+
+
+@pytest.fixture(scope="module", autouse=True)
+def tmq():
+    import torch_musa_amd
+    assert torch.cuda.is_available() and torch_musa_amd.is_loaded()
+    torch.backends.quantized.engine = "fbgemm"
+    return torch_musa_amd
+
+
+def assert_q_equal(q_gpu, q_cpu, abs_diff=0):
+    """QuantizedComparator of the reference (base_test_tool.py:233-289)."""
+    assert q_gpu.is_cuda and q_gpu.dtype == q_cpu.dtype and q_gpu.shape == q_cpu.shape
+    assert q_gpu.qscheme() == q_cpu.qscheme()
+    if q_cpu.qscheme() in (torch.per_tensor_affine, torch.per_tensor_symmetric):
+        assert q_gpu.q_scale() == q_cpu.q_scale() and q_gpu.q_zero_point() == q_cpu.q_zero_point()
+    else:
+        assert torch.equal(q_gpu.q_per_channel_scales().cpu(), q_cpu.q_per_channel_scales())
+        assert torch.equal(q_gpu.q_per_channel_zero_points().cpu(), q_cpu.q_per_channel_zero_points())
+        assert q_gpu.q_per_channel_axis() == q_cpu.q_per_channel_axis()
+    d = (q_gpu.int_repr().cpu().to(torch.int32) - q_cpu.int_repr().to(torch.int32)).abs().max().item() \
+        if q_cpu.numel() else 0
+    assert d <= abs_diff, f"int_repr differs by {d}"
+    if abs_diff == 0:
+        assert torch.equal(q_gpu.dequantize().cpu(), q_cpu.dequantize())
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4), (2, 3, 4, 5), (2, 16, 32, 32), (0, 4), (7,)])
+@pytest.mark.parametrize("dtype", [torch.quint8, torch.qint8])
+def test_quantize_per_tensor(shape, dtype):
+    say("aten qpt", shape, dtype)
+    torch.manual_seed(41)
+    x = torch.randn(shape)
+    scale = float(x.abs().max() / 2 ** 7) if x.numel() else 0.1
+    zp = 0 if dtype == torch.qint8 else 128
+    assert_q_equal(torch.quantize_per_tensor(x.cuda(), scale, zp, dtype),
+                   torch.quantize_per_tensor(x, scale, zp, dtype))
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4), (2, 3, 4, 5), (2, 16, 32, 32)])
+@pytest.mark.parametrize("reduce_range", [True, False])
+@pytest.mark.parametrize("dtype", [torch.quint8, torch.qint8])
+def test_quantize_per_tensor_dynamic(shape, reduce_range, dtype):
+    say("aten dyn", shape, reduce_range, dtype)
+    torch.manual_seed(42)
+    x = torch.randn(shape) * 3
+    assert_q_equal(torch.quantize_per_tensor_dynamic(x.cuda(), dtype, reduce_range),
+                   torch.quantize_per_tensor_dynamic(x, dtype, reduce_range))
+
+
+def test_memory_format_is_preserved():
+    x = torch.randn(2, 8, 5, 7).contiguous(memory_format=torch.channels_last)
+    q = torch.quantize_per_tensor(x.cuda(), 0.05, 10, torch.quint8)
+    assert q.is_contiguous(memory_format=torch.channels_last)
+    assert_q_equal(q, torch.quantize_per_tensor(x, 0.05, 10, torch.quint8))
+    assert q.dequantize().is_contiguous(memory_format=torch.channels_last)
+    qd = torch.quantize_per_tensor_dynamic(x.cuda(), torch.quint8, False)
+    assert qd.is_contiguous(memory_format=torch.channels_last)
+    assert_q_equal(qd, torch.quantize_per_tensor_dynamic(x, torch.quint8, False))
+
+
+@pytest.mark.parametrize("c", cases.quantize_per_channel_cases(), ids=lambda c: c["name"])
+def test_quantize_per_channel(c):
+    say("aten qpc", c["name"])
+    x = torch.from_numpy(c["x"])
+    s = torch.from_numpy(c["scales"].astype(np.float64))
+    z = torch.from_numpy(c["zps"].astype(np.int64))
+    dt = torch.qint8 if c["signed"] else torch.quint8
+    assert_q_equal(torch.quantize_per_channel(x.cuda(), s.cuda(), z.cuda(), c["axis"], dt),
+                   torch.quantize_per_channel(x, s, z, c["axis"], dt))
+
+
+def test_quantize_per_channel_rejects_bad_zero_point():
+    x = torch.randn(2, 3).cuda()
+    with pytest.raises(RuntimeError):
+        torch.quantize_per_channel(x, torch.tensor([0.1, 0.1]).cuda(), torch.tensor([0, 256]).cuda(), 0,
+                                   torch.quint8)
+
+
+# ---------------------------------------------------------------------------
+# linear
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(8, 128), (8, 10, 128)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_qlinear_reference_flavour(shape, relu):
+    """qint8 activations, per-tensor symmetric qint8 weight, qint8 output, no
+    bias: the configuration of the reference's test_qlinear, same assertion."""
+    say("aten qlinear ref", shape, relu)
+    torch.manual_seed(41)
+    data = torch.randn(shape)
+    module = torch.nn.Linear(128, 512, False)
+    fweight = module.weight.detach()
+    qweight = torch.quantize_per_tensor(fweight, float(fweight.abs().max() / 2 ** 7), 0, torch.qint8)
+    module.weight = torch.nn.Parameter(qweight.dequantize())
+    qmodule = (nniq.LinearReLU if relu else nnq.Linear)(128, 512, False, torch.qint8)
+    qmodule.set_weight_bias(qweight.cuda(), None)
+    qdata = torch.quantize_per_tensor(data, float(data.abs().max() / 2 ** 7), 0, torch.qint8)
+    foutput = module(qdata.dequantize()).detach()
+    out_scale = float(foutput.abs().max() / 2 ** 7)
+    qmodule.scale, qmodule.zero_point = out_scale, 0
+    qoutput = qmodule(qdata.cuda())
+    assert qoutput.dtype == torch.qint8 and tuple(qoutput.shape) == shape[:-1] + (512,)
+    if relu:
+        foutput = torch.relu(foutput)
+    assert (qoutput.dequantize().cpu() - foutput).mean().abs() < 1e-3
+    fq = torch.quantize_per_tensor(foutput, out_scale, 0, torch.qint8)
+    d = (qoutput.int_repr().cpu().to(torch.int32) - fq.int_repr().to(torch.int32)).abs().max()
+    assert d <= LSB_TOL
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("bias", [False, True])
+def test_qlinear_matches_cpu_op(per_channel, relu, bias):
+    """quint8 activations / per-channel weights: the CPU op is the oracle."""
+    say("aten qlinear cpu", per_channel, relu, bias)
+    torch.manual_seed(7)
+    x = torch.randn(3, 17, 256)
+    w = torch.randn(300, 256) * 0.05
+    b = torch.randn(300) if bias else None
+    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+    if per_channel:
+        s = (w.abs().amax(dim=1) / 127).to(torch.float64)
+        wq = torch.quantize_per_channel(w, s, torch.zeros(300, dtype=torch.int64), 0, torch.qint8)
+    else:
+        wq = torch.quantize_per_tensor(w, float(w.abs().max() / 127), 0, torch.qint8)
+    op = torch.ops.quantized.linear_relu if relu else torch.ops.quantized.linear
+    ref = op(xq, torch.ops.quantized.linear_prepack(wq, b), 0.1, 100)
+    packed = torch.ops.quantized.linear_prepack(wq.cuda(), None if b is None else b.cuda())
+    got = op(xq.cuda(), packed, 0.1, 100)
+    assert_q_equal(got, ref, abs_diff=LSB_TOL)
+    n_off = (got.int_repr().cpu() != ref.int_repr()).sum().item()
+    assert n_off == 0, f"{n_off} outputs off by one LSB"
+    # unpack returns what was packed (reference: mudnn/LinearUnpackImpl.cpp:9-12)
+    w2, b2 = torch.ops.quantized.linear_unpack(packed)
+    assert_q_equal(w2, wq)
+    assert (b2 is None) == (b is None) and (b is None or torch.equal(b2.cpu(), b))
+
+
+def test_qlinear_errors():
+    w = torch.quantize_per_tensor(torch.randn(8, 16), 0.1, 3, torch.qint8).cuda()
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.linear_prepack(w, None)                # weight zero point != 0
+    wu = torch.quantize_per_tensor(torch.randn(8, 16), 0.1, 0, torch.quint8).cuda()
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.linear_prepack(wu, None)               # weight dtype
+    w = torch.quantize_per_tensor(torch.randn(8, 16), 0.1, 0, torch.qint8).cuda()
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.linear_prepack(w, torch.zeros(9).cuda())  # bias length
+    packed = torch.ops.quantized.linear_prepack(w, None)
+    x = torch.quantize_per_tensor(torch.randn(4, 15), 0.1, 0, torch.quint8).cuda()
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.linear(x, packed, 0.1, 0)              # feature mismatch
+    x = torch.quantize_per_tensor(torch.randn(4, 16), 0.1, 0, torch.quint8).cuda()
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.linear_dynamic(x.dequantize(), packed)  # apply_dynamic not implemented
+    empty = torch.quantize_per_tensor(torch.randn(0, 16), 0.1, 0, torch.quint8).cuda()
+    assert tuple(torch.ops.quantized.linear(empty, packed, 0.1, 0).shape) == (0, 8)
+
+
+def test_c1_through_the_operators(golden):
+    """BASELINE config 1 with nothing but torch calls on GPU tensors."""
+    say("aten C1")
+    c1 = cases.c1_case()
+    xq = torch.quantize_per_tensor_dynamic(torch.from_numpy(c1["x"]).cuda(), torch.quint8, False)
+    assert xq.q_scale() == float(golden["c1/x_scale"]) and xq.q_zero_point() == int(golden["c1/x_zp"])
+    wq = torch.quantize_per_channel(torch.from_numpy(c1["w"]).cuda(), torch.from_numpy(c1["w_scales"]).cuda(),
+                                    torch.zeros(1024, dtype=torch.int64).cuda(), 0, torch.qint8)
+    packed = torch.ops.quantized.linear_prepack(wq, torch.from_numpy(c1["bias"]).cuda())
+    y = torch.ops.quantized.linear(xq, packed, c1["out_scale"], c1["out_zp"])
+    assert y.dtype == torch.quint8
+    d = np.abs(y.int_repr().cpu().numpy().astype(np.int32) - golden["c1/y"].astype(np.int32))
+    assert d.max() <= LSB_TOL and d.max() == 0
+    assert cases.crc(y.dequantize().cpu().numpy()) == int(golden["c1/y_dq_crc"])
+
+
+# ---------------------------------------------------------------------------
+# conv2d
+# ---------------------------------------------------------------------------
+CONV_CONFIGS = [
+    dict(shape=(2, 32, 16, 16), oc=64, k=3, s=1, p=1, d=1, g=1, bias=False, relu=False),
+    dict(shape=(2, 32, 16, 16), oc=64, k=3, s=1, p=1, d=1, g=1, bias=False, relu=True),
+    dict(shape=(2, 3, 16, 16), oc=32, k=3, s=2, p=1, d=1, g=1, bias=True, relu=True),
+    dict(shape=(2, 64, 16, 16), oc=32, k=3, s=2, p=1, d=1, g=32, bias=False, relu=True),
+    dict(shape=(8, 3, 32, 32), oc=32, k=7, s=2, p=3, d=1, g=1, bias=True, relu=False),
+    dict(shape=(4, 64, 28, 28), oc=64, k=3, s=1, p=1, d=1, g=1, bias=True, relu=False),
+]
+
+
+@pytest.mark.parametrize("cfg", CONV_CONFIGS, ids=lambda c: f"{c['shape']}-{c['oc']}-k{c['k']}g{c['g']}")
+@pytest.mark.parametrize("per_channel", [False, True])
+@pytest.mark.parametrize("channels_last_input", [False, True])
+def test_qconv2d_matches_cpu_op(cfg, per_channel, channels_last_input):
+    """Configurations of the reference's test_qconv2d, through nnq.Conv2d with
+    weights set from outside (test_quantized_conv.py:83-150), against the CPU op."""
+    say("aten qconv", cfg, per_channel, channels_last_input)
+    torch.manual_seed(41)
+    ic = cfg["shape"][1]
+    x = torch.randn(cfg["shape"])
+    if channels_last_input:
+        x = x.contiguous(memory_format=torch.channels_last)
+    w = torch.randn(cfg["oc"], ic // cfg["g"], cfg["k"], cfg["k"]) * 0.1
+    b = torch.randn(cfg["oc"]) if cfg["bias"] else None
+    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+    if per_channel:
+        s = (w.abs().amax(dim=(1, 2, 3)) / 127).to(torch.float64)
+        wq = torch.quantize_per_channel(w, s, torch.zeros(cfg["oc"], dtype=torch.int64), 0, torch.qint8)
+    else:
+        wq = torch.quantize_per_tensor(w, float(w.abs().max() / 127), 0, torch.qint8)
+    cls = nniq.ConvReLU2d if cfg["relu"] else nnq.Conv2d
+    mods = []
+    for dev in ("cpu", "cuda"):
+        m = cls(ic, cfg["oc"], cfg["k"], cfg["s"], cfg["p"], cfg["d"], cfg["g"], cfg["bias"])
+        m.set_weight_bias(wq.to(dev), None if b is None else b.to(dev))
+        m.scale, m.zero_point = 0.25, 90
+        mods.append(m)
+    ref = mods[0](xq)
+    got = mods[1](xq.cuda())
+    assert got.is_contiguous(memory_format=torch.channels_last) or got.numel() == 0
+    assert_q_equal(got, ref, abs_diff=LSB_TOL)
+    n_off = (got.int_repr().cpu() != ref.int_repr()).sum().item()
+    assert n_off == 0, f"{n_off} outputs off by one LSB"
+    w2, b2 = mods[1]._weight_bias()
+    assert_q_equal(w2, wq)
+    assert (b2 is None) == (b is None) and (b is None or torch.equal(b2.cpu(), b))
+
+
+def test_qconv2d_errors():
+    w = torch.quantize_per_tensor(torch.randn(8, 4, 3, 3), 0.1, 5, torch.qint8).cuda()
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.conv2d_prepack(w, None, [1, 1], [0, 0], [1, 1], 1)   # zero point != 0
+    w = torch.quantize_per_tensor(torch.randn(8, 4, 3, 3), 0.1, 0, torch.qint8).cuda()
+    packed = torch.ops.quantized.conv2d_prepack(w, None, [1, 1], [1, 1], [1, 1], 1)
+    x = torch.quantize_per_tensor(torch.randn(1, 5, 8, 8), 0.1, 0, torch.quint8).cuda()
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.conv2d(x, packed, 0.1, 0)                             # channel mismatch

@@ -1,0 +1,64 @@
+"""MI355X-native quantized-inference operators behind PyTorch's own op names.
+
+Importing this package loads two in-tree native libraries:
+
+  libtmq.so        hand-written HIP kernels for gfx950 behind the C ABI of
+                   ``include/tmq.h`` (quantize / dequantize / min-max, int8 MFMA
+                   linear, NHWC implicit-GEMM conv2d)
+  libtmq_aten.so   registrations that put those kernels behind
+                   ``torch.quantize_per_tensor``, ``torch.quantize_per_channel``,
+                   ``torch.quantize_per_tensor_dynamic``, ``Tensor.dequantize`` and
+                   ``torch.ops.quantized.{linear,linear_relu,linear_prepack,
+                   conv2d,conv2d_relu,conv2d_prepack}`` for tensors on the GPU
+
+so that a model written against ``torch.ops.quantized.*`` runs unchanged (the
+counterpart of ``import torch_musa`` for this operator path; reference:
+torch_musa/csrc/aten/quantized).  There is no CPU or eager fallback: if a
+library is missing the import fails.
+"""
+from __future__ import annotations
+
+import os
+import warnings
+
+import torch
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_KERNELS = os.path.join(_PKG, "libtmq.so")
+LIB_ATEN = os.path.join(_PKG, "libtmq_aten.so")
+
+__all__ = ["LIB_KERNELS", "LIB_ATEN", "is_loaded", "load", "quantized_device"]
+
+_loaded = False
+
+
+def load() -> None:
+    """Load the native libraries and register the operators (idempotent)."""
+    global _loaded
+    if _loaded:
+        return
+    for lib in (LIB_KERNELS, LIB_ATEN):
+        if not os.path.exists(lib):
+            raise ImportError(
+                f"{lib} is missing: build the native libraries with "
+                "`python torch_musa_amd/build.py` (there is no fallback path)")
+    with warnings.catch_warnings():
+        # replacing PyTorch's own GPU kernel of aten::quantize_per_tensor_dynamic
+        # is intended; the dispatcher warns about it once
+        warnings.filterwarnings("ignore", message=".*Overriding a previously registered kernel.*")
+        torch.ops.load_library(LIB_ATEN)
+    _loaded = True
+
+
+def is_loaded() -> bool:
+    return _loaded
+
+
+def quantized_device() -> torch.device:
+    """The device the operators run on (PyTorch-ROCm names the GPU "cuda")."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("no MI355X visible: the tmq operators have no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+load()

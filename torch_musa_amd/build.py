@@ -4,7 +4,10 @@
   libtmq_aten.so  ATen registrations (TORCH_LIBRARY_IMPL + dispatch stubs)
                   that call libtmq.so
 
-    python -m torch_musa_amd.build [--kernels-only] [--verbose]
+    python torch_musa_amd/build.py [--kernels-only] [--verbose]
+
+Run it as a script (not with -m): importing the package loads the libraries
+this script is about to produce.
 """
 from __future__ import annotations
 

@@ -78,7 +78,7 @@ def lib() -> C.CDLL:
     global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):
-            raise TmqError(f"{LIB_PATH} is missing: build it with `python -m torch_musa_amd.build`")
+            raise TmqError(f"{LIB_PATH} is missing: build it with `python torch_musa_amd/build.py`")
         l = C.CDLL(LIB_PATH)
         l.tmq_status_string.restype = C.c_char_p
         l.tmq_minmax_workspace_bytes.restype = C.c_size_t
