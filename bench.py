@@ -1,0 +1,290 @@
+"""Benchmark of the quantized-inference operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one quantized::linear at BASELINE config 3 (x quint8 [4096,4096] from
+N(0,1), W qint8 per-channel [11008,4096] from N(0,0.02), fp32 bias, quint8
+output), issued through torch.ops.quantized.linear on tensors that are already
+resident in HBM.  The last line of stdout is one JSON object:
+
+  value / unit     whole-job int8 throughput of those K steps (TOP/s)
+  roofline         the GEMM kernel against the dense int8 MFMA peak, its average
+                   launch duration measured with HIP events on the launch stream
+  cpu_baseline     the CPU oracle (a scalar C port of the reference CPU
+                   numerics, OpenMP over rows) on a bounded sample of the same
+                   workload, on this host's cores
+  secondary        the other BASELINE configs: quantize / dequantize / min-max
+                   over 2**28 fp32 (HBM bound), decode-shaped linear (weight
+                   read bound), conv2d NHWC
+
+Everything here is synthetic data of the BASELINE shapes and distributions
+("N(0,s)" read as standard deviation s).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# Published MI355X peaks used for roofline.frac
+PEAK_INT8_TOPS = 5000.0   # dense int8 MFMA, 5.0 POP/s
+PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (one run each, scaled by the same counters on a plain copy of known size);
+# the runs and the scale factor are in profiles/.  None = not measured yet.
+MEASURED_TRAFFIC = {
+    "linear_c3": None,
+    "quantize_c2": None,
+    "dequantize_c2": None,
+    "minmax_c2": None,
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--skip-secondary", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the quantized operator path is single-device "
+              "(no collectives); run it with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import torch_musa_amd
+    from torch_musa_amd import cabi
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    assert torch_musa_amd.is_loaded()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    torch.manual_seed(41)
+
+    def events_ms(fn, n):
+        """n launches, one HIP event pair each, on the current (launch) stream."""
+        evs = []
+        for _ in range(n):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        return [a.elapsed_time(b) for a, b in evs]
+
+    # ------------------------------------------------------------------ C3
+    M, K, N = 4096, 4096, 11008
+    log(f"[bench] building config 3: M={M} K={K} N={N}")
+    x = torch.randn(M, K, device=dev)
+    w = torch.randn(N, K, device=dev) * 0.02
+    bias = torch.randn(N, device=dev)
+    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+    w_scales = (w.abs().amax(dim=1) / 127.0).to(torch.float64)
+    wq = torch.quantize_per_channel(w, w_scales, torch.zeros(N, dtype=torch.int64, device=dev), 0, torch.qint8)
+    packed = torch.ops.quantized.linear_prepack(wq, bias)
+    # output scale from a calibration pass of the fp32 result, fixed thereafter
+    y_f = torch.nn.functional.linear(xq.dequantize()[:256], wq.dequantize(), bias)
+    out_scale = float((y_f.max() - y_f.min()) / 255.0)
+    out_zp = int(round(float(-y_f.min()) / out_scale))
+    out_zp = max(0, min(255, out_zp))
+    del x, w, y_f
+
+    def step():
+        return torch.ops.quantized.linear(xq, packed, out_scale, out_zp)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    ops = 2.0 * M * N * K
+    value = ops / (ms_per_step * 1e-3) / 1e12
+    kern = events_ms(step, args.steps)
+    kern_ms = sum(kern) / len(kern)
+    achieved = ops / (kern_ms * 1e-3) / 1e12
+    log(f"[bench] linear C3: {ms_per_step*1e3:.1f} us/step wall, {kern_ms*1e3:.1f} us/launch (events), "
+        f"{achieved:.0f} TOP/s")
+    roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": MEASURED_TRAFFIC["linear_c3"],
+                "kernel": "tmq::gemm_i8_kernel", "ops_per_launch": ops,
+                "avg_launch_us": round(kern_ms * 1e3, 2),
+                "algorithmic_bytes_per_launch": M * K + N * K + M * N + 12 * N}
+
+    secondary = {}
+    if not args.skip_secondary:
+        # -------------------------------------------------------------- C2
+        n = 2 ** 28
+        log("[bench] config 2: quantize / dequantize / min-max over 2**28 fp32")
+        xf = torch.randn(n, device=dev) * 3.0
+        idx = torch.randint(0, n, (n // 100,), device=dev)
+        xf[idx] = torch.where(torch.rand(idx.numel(), device=dev) < 0.5, 50.0, -50.0)
+        del idx
+        mm = cabi.minmax(xf).cpu()
+        scale, zp = cabi.choose_qparams_host(float(mm[0]), float(mm[1]), False, False)
+        q = torch.quantize_per_tensor(xf, scale, zp, torch.quint8)
+        ws = cabi.minmax_workspace(dev)
+        mm_out = torch.empty(2, device=dev)
+
+        def hbm(name, fn, bytes_per_launch, key):
+            for _ in range(5):
+                fn()
+            ts = events_ms(fn, 20)
+            avg = sum(ts) / len(ts)
+            gbs = bytes_per_launch / (avg * 1e-3) / 1e9
+            log(f"[bench] {name}: {avg*1e3:.1f} us/launch, {gbs:.0f} GB/s")
+            secondary[name] = {"avg_launch_us": round(avg * 1e3, 2), "value": round(gbs, 1), "unit": "GB/s",
+                               "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                                            "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
+                                            "traffic": MEASURED_TRAFFIC.get(key)},
+                               "algorithmic_bytes_per_launch": bytes_per_launch}
+
+        hbm("quantize_per_tensor_c2", lambda: torch.quantize_per_tensor(xf, scale, zp, torch.quint8), 5 * n,
+            "quantize_c2")
+        hbm("dequantize_c2", lambda: q.dequantize(), 5 * n, "dequantize_c2")
+        hbm("minmax_c2", lambda: cabi.minmax(xf, mm_out, ws), 4 * n, "minmax_c2")
+        hbm("quantize_per_tensor_dynamic_c2", lambda: torch.quantize_per_tensor_dynamic(xf, torch.quint8, False),
+            9 * n, None)
+        del xf, q
+
+        # -------------------------------------------------------------- C4
+        log("[bench] config 4: decode-shaped linear, K=N=4096, cold weights (40 weight sets, HIP graph)")
+        Kd = Nd = 4096
+        sets = 40  # 40 x 16.8 MB > 2 x the 256 MB last-level cache
+        pws = [cabi.PackedLinear(torch.randint(-127, 128, (Nd, Kd), dtype=torch.int8, device=dev))
+               for _ in range(sets)]
+        wsd = torch.rand(Nd, device=dev) * 0.002 + 0.001
+        bd = torch.randn(Nd, device=dev)
+        for Md in (1, 4, 16):
+            xd = torch.randint(0, 256, (Md, Kd), dtype=torch.uint8, device=dev)
+            yd = torch.empty((Md, Nd), dtype=torch.uint8, device=dev)
+
+            def run_sets():
+                for p in pws:
+                    cabi.linear(xd, p, 0.02, 128, wsd, bd, 0.05, 128, out=yd)
+
+            run_sets()
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                run_sets()
+                side.synchronize()
+                with torch.cuda.graph(graph, stream=side):
+                    run_sets()
+            torch.cuda.synchronize()
+            for _ in range(3):
+                graph.replay()
+            ts = events_ms(graph.replay, 10)
+            per = sum(ts) / len(ts) / sets
+            nbytes = Nd * Kd + Md * Kd + Md * Nd + 12 * Nd
+            gbs = nbytes / (per * 1e-3) / 1e9
+            log(f"[bench] decode M={Md}: {per*1e3:.2f} us/launch in a replayed graph, {gbs:.0f} GB/s")
+            secondary[f"linear_decode_m{Md}"] = {
+                "avg_launch_us": round(per * 1e3, 3), "value": round(gbs, 1), "unit": "GB/s",
+                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
+                "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
+                "algorithmic_bytes_per_launch": nbytes}
+        del pws
+
+        # -------------------------------------------------------------- C5
+        log("[bench] config 5: conv2d NHWC [32,56,56,64] x [64,3,3,64]")
+        xc = torch.relu(torch.randn(32, 64, 56, 56, device=dev)).contiguous(memory_format=torch.channels_last)
+        xcq = torch.quantize_per_tensor_dynamic(xc, torch.quint8, False)
+        wc = torch.randn(64, 64, 3, 3, device=dev) * 0.05
+        wcs = (wc.abs().amax(dim=(1, 2, 3)) / 127.0).to(torch.float64)
+        wcq = torch.quantize_per_channel(wc, wcs, torch.zeros(64, dtype=torch.int64, device=dev), 0, torch.qint8)
+        pc = torch.ops.quantized.conv2d_prepack(wcq, torch.randn(64, device=dev), [1, 1], [1, 1], [1, 1], 1)
+        conv = lambda: torch.ops.quantized.conv2d(xcq, pc, 0.05, 0)
+        for _ in range(5):
+            conv()
+        ts = events_ms(conv, 30)
+        avg = sum(ts) / len(ts)
+        cops = 2.0 * 32 * 56 * 56 * 64 * 576
+        cbytes = 2 * 32 * 56 * 56 * 64 + 64 * 576 + 768
+        log(f"[bench] conv2d C5: {avg*1e3:.1f} us/launch, {cops/(avg*1e-3)/1e12:.0f} TOP/s, "
+            f"{cbytes/(avg*1e-3)/1e9:.0f} GB/s")
+        secondary["conv2d_c5"] = {
+            "avg_launch_us": round(avg * 1e3, 2), "value": round(cops / (avg * 1e-3) / 1e12, 1), "unit": "TOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(cops / (avg * 1e-3) / 1e12, 1),
+                         "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                         "frac": round(cops / (avg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "traffic": None},
+            "hbm_frac": round(cbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "algorithmic_bytes_per_launch": cbytes, "ops_per_launch": cops}
+
+    # ------------------------------------------------------------ CPU baseline
+    cpu_baseline = None
+    if not args.skip_cpu:
+        import oracle
+
+        cores = min(os.cpu_count() or 1, 16)
+        rows = M if cores >= 8 else 512  # ~4 s of CPU work on 16 cores
+        xs = xq.int_repr()[:rows].cpu().numpy()
+        ws_h = wq.int_repr().cpu().numpy()
+        wsc = w_scales.cpu().numpy()
+        b_h = bias.cpu().numpy()
+        log(f"[bench] CPU baseline: oracle linear on {rows} of {M} rows, {cores} threads")
+        t0 = time.perf_counter()
+        y_ref = oracle.linear(xs, xq.q_scale(), xq.q_zero_point(), ws_h, wsc, b_h, out_scale, out_zp,
+                              nthreads=cores)
+        dt = time.perf_counter() - t0
+        cpu_tops = 2.0 * rows * N * K / dt / 1e12
+        got = step().int_repr()[:rows].cpu().numpy()
+        max_diff = int(np.abs(got.astype(np.int32) - y_ref.astype(np.int32)).max())
+        log(f"[bench] CPU oracle: {dt:.2f} s, {cpu_tops*1e3:.2f} GOP/s; GPU vs oracle max diff {max_diff} LSB")
+        cpu_baseline = {"value": round(cpu_tops, 5), "unit": "TOP/s", "cores": cores, "kind": "port",
+                        "sample": f"first {rows} of {M} rows of config 3 (all {N} x {K} weights), "
+                                  f"{dt:.1f} s of CPU work", "gpu_vs_oracle_max_lsb": max_diff}
+        # PyTorch's own CPU op (fbgemm) on the same sample, for reference
+        try:
+            torch.backends.quantized.engine = "fbgemm"
+            torch.set_num_threads(cores)
+            xs_q = torch._make_per_tensor_quantized_tensor(torch.from_numpy(xs), xq.q_scale(), xq.q_zero_point())
+            p_cpu = torch.ops.quantized.linear_prepack(wq.cpu(), bias.cpu())
+            torch.ops.quantized.linear(xs_q, p_cpu, out_scale, out_zp)
+            t0 = time.perf_counter()
+            for _ in range(3):
+                torch.ops.quantized.linear(xs_q, p_cpu, out_scale, out_zp)
+            dt2 = (time.perf_counter() - t0) / 3
+            cpu_baseline["torch_cpu_fbgemm"] = {"value": round(2.0 * rows * N * K / dt2 / 1e12, 4),
+                                                "unit": "TOP/s", "threads": cores}
+        except Exception as e:  # the CPU op is extra information only
+            cpu_baseline["torch_cpu_fbgemm"] = {"error": str(e)[:200]}
+
+    out = {
+        "metric": "int8 quantized::linear TOPS (% MFMA peak) + quantize GB/s (% HBM), 1 GPU",
+        "value": round(value, 2), "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "quantized::linear prefill, BASELINE config 3: x quint8 [4096,4096] from N(0,1), "
+                               "W qint8 per-channel [11008,4096] from N(0,0.02), fp32 bias, int32 accumulate, "
+                               "quint8 output", "M": M, "K": K, "N": N,
+                   "api": "torch.ops.quantized.linear on GPU tensors"},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "secondary": secondary,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
