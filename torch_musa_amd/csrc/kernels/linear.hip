@@ -84,14 +84,15 @@ __global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ 
 // Decode-sized batches (M <= 16): the weight is read once, straight from HBM
 // into MFMA operand registers (the packed layout is the 16x16x64 operand
 // order), activations come from L2.  One block per 16 output channels, its
-// four waves split K and reduce through LDS.
+// eight waves split K and reduce through LDS.
 //   D[i][j] of v_mfma_i32_16x16x64_i8: lane l, register r -> i = 4*(l/16)+r
 //   (channel), j = l%16 (activation row).
 // ---------------------------------------------------------------------------
+constexpr int kDecodeWaves = 8;
 template <int MODE>
-__global__ __launch_bounds__(256) void linear_decode_kernel(GemmArgs a, XLinear xs) {
-  constexpr int kWaves = 4;
-  constexpr int kBatch = 8;  // 64-byte k-blocks in flight per wave
+__global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(GemmArgs a, XLinear xs) {
+  constexpr int kWaves = kDecodeWaves;
+  constexpr int kBatch = 8;  // 64-byte k-blocks in flight per wave: 64 KB of weights per block
   __shared__ int s_part[kWaves][16 * 16];
   const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
   const int lr = lane & 15, lc = lane >> 4;
@@ -238,7 +239,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   if ((a.M <= 16 && forced < 0) || forced == 8) {
     if (a.M > 16) return TMQ_ERR_UNSUPPORTED;
     const int64_t blocks = ceil_div(a.N, 16);
-    linear_decode_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(a, xs);
+    linear_decode_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(kDecodeWaves * kWave), 0, s>>>(a, xs);
     return launch_status();
   }
   int cfg = forced;
