@@ -58,6 +58,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-secondary", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy"],
+                    help="run just this kernel --steps times (for rocprofv3 --pmc runs); 'copy' is a plain "
+                         "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the quantized operator path is single-device "
@@ -88,6 +91,26 @@ def main():
         torch.cuda.synchronize()
         return [a.elapsed_time(b) for a, b in evs]
 
+    if args.only in ("quantize", "dequantize", "minmax", "copy"):
+        n = 2 ** 28
+        xf = torch.randn(n, device=dev) * 3.0
+        if args.only == "copy":
+            yf = torch.empty_like(xf)
+            fn = lambda: yf.copy_(xf)
+        elif args.only == "quantize":
+            fn = lambda: torch.quantize_per_tensor(xf, 0.39, 128, torch.quint8)
+        elif args.only == "dequantize":
+            q = torch.quantize_per_tensor(xf, 0.39, 128, torch.quint8)
+            fn = lambda: q.dequantize()
+        else:
+            ws_, mm_ = cabi.minmax_workspace(dev), torch.empty(2, device=dev)
+            fn = lambda: cabi.minmax(xf, mm_, ws_)
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        print(json.dumps({"only": args.only, "launches": args.steps, "elements": n}))
+        return
+
     # ------------------------------------------------------------------ C3
     M, K, N = 4096, 4096, 11008
     log(f"[bench] building config 3: M={M} K={K} N={N}")
@@ -107,6 +130,13 @@ def main():
 
     def step():
         return torch.ops.quantized.linear(xq, packed, out_scale, out_zp)
+
+    if args.only == "linear":
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        print(json.dumps({"only": "linear", "launches": args.steps, "M": M, "K": K, "N": N}))
+        return
 
     for _ in range(args.warmup):
         step()

@@ -69,6 +69,11 @@ struct GemmArgs {
 };
 
 __device__ __forceinline__ v4i ld16(const void* p) { return *reinterpret_cast<const v4i*>(p); }
+// Streaming load: data that this CU reads exactly once (packed weight tiles)
+// should not push reusable lines out of the vector L1.
+__device__ __forceinline__ v4i ld16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+}
 
 template <class XSRC>
 struct XLoader;
@@ -182,8 +187,10 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   const int wm0 = (wave % WM) * WTM;
   const int wn0 = (wave / WM) * WTN;
 
-  // ---- tile assignment: blocks are dealt round-robin to the 8 XCDs; give each
-  // XCD one contiguous run of tiles (row tiles fastest) so its L2 sees reuse.
+  // ---- tile assignment.  Blocks are dealt round-robin to the 8 XCDs, each with
+  // its own L2: give every XCD one contiguous run of the tile sequence, and order
+  // the sequence so that the ~32 tiles an XCD runs at once form a compact patch
+  // (kGroupN channel tiles wide, row tiles next) that shares operand tiles.
   const int64_t tiles_m = ceil_div(a.M, BM), tiles_n = ceil_div(a.N, BN);
   const int64_t nblocks = tiles_m * tiles_n;
   int64_t tile;
@@ -193,8 +200,13 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     const int64_t xcd = bid % 8, within = bid / 8;
     tile = xcd * q + (xcd < rem ? xcd : rem) + within;
   }
-  const int64_t m0 = (tile % tiles_m) * BM;
-  const int64_t n0 = (tile / tiles_m) * BN;
+  constexpr int64_t kGroupN = 4;
+  const int64_t group = tile / (tiles_m * kGroupN);
+  const int64_t gfirst = group * kGroupN;
+  const int64_t gwidth = tiles_n - gfirst < kGroupN ? tiles_n - gfirst : kGroupN;
+  const int64_t in_group = tile - group * (tiles_m * kGroupN);
+  const int64_t m0 = (in_group / gwidth) * BM;
+  const int64_t n0 = (gfirst + in_group % gwidth) * BN;
   const int64_t NB = ceil_div(a.N, 16);
 
   // ---- per-channel constants of this tile's BN output channels
@@ -244,7 +256,7 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   // k-th global load of a stage (weights first, then activations)
   auto load_one = [&](int set, int kt, int k) {
     if (k < NW)
-      wreg[set][k] = ld16(wsrc[k] + static_cast<int64_t>(kt) * (kChunks * 256));
+      wreg[set][k] = ld16_stream(wsrc[k] + static_cast<int64_t>(kt) * (kChunks * 256));
     else
       xreg[set][k - NW] = xl[k - NW].load(xsrc, kt * kChunks + (t & 3), a.K);
   };
