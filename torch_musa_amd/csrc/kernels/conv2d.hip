@@ -43,7 +43,8 @@ int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
   s->KC = packed_kchunks(s->Kp);
   s->group_bytes = ceil_div(s->OCg, 16) * s->KC * 256;
   // 32-bit index arithmetic inside the kernels
-  if (g->H > (1 << 24) || g->W > (1 << 24) || g->IC > (1 << 24) || s->Kp > (1 << 30))
+  if (g->H > (1 << 24) || g->W > (1 << 24) || g->IC > (1 << 24) || s->Kp > (1 << 30) ||
+      g->B * s->OH * s->OW > 0x7fffffff || g->H * g->W * g->IC > 0x3fffffff)
     return TMQ_ERR_UNSUPPORTED;
   return TMQ_OK;
 }

@@ -89,40 +89,98 @@ struct XLoader<XLinear> {
   __device__ __forceinline__ void init(const XLinear& s, int64_t m, int64_t M) {
     p = s.x + (m < M ? m : M - 1) * s.ldx;
   }
-  __device__ __forceinline__ v4i load(const XLinear&, int kc, int64_t K) const {
-    int64_t k = static_cast<int64_t>(kc) * 16;
-    k = k < K ? k : K - 16;
-    return ld16(p + k);
-  }
 };
 
 template <>
 struct XLoader<XConv> {
   const uint8_t* img;  // first byte of this row's image (+ group channel offset)
   int ih0, iw0;        // top-left input coordinate of the receptive field
+  int off0;            // byte offset of (ih0, iw0) inside the image (may be negative)
   __device__ __forceinline__ void init(const XConv& s, int64_t m, int64_t M) {
-    const int64_t mm = m < M ? m : M - 1;
-    const int ow = static_cast<int>(mm % s.OW);
-    const int64_t t = mm / s.OW;
-    const int oh = static_cast<int>(t % s.OH);
-    const int64_t b = t / s.OH;
-    img = s.x + b * (static_cast<int64_t>(s.H) * s.W * s.IC) + s.ic_off;
+    // the host guarantees fewer than 2**31 output pixels and image bytes:
+    // 32-bit divisions and offsets
+    const uint32_t mm = static_cast<uint32_t>(m < M ? m : M - 1);
+    const uint32_t t = mm / static_cast<uint32_t>(s.OW);
+    const int ow = static_cast<int>(mm - t * static_cast<uint32_t>(s.OW));
+    const uint32_t b = t / static_cast<uint32_t>(s.OH);
+    const int oh = static_cast<int>(t - b * static_cast<uint32_t>(s.OH));
+    img = s.x + static_cast<int64_t>(b) * (static_cast<int64_t>(s.H) * s.W * s.IC) + s.ic_off;
     ih0 = oh * s.stride_h - s.pad_h;
     iw0 = ow * s.stride_w - s.pad_w;
+    off0 = (ih0 * s.W + iw0) * s.IC;
   }
-  // Out-of-image taps read as the activation zero point, i.e. real value 0.
-  __device__ __forceinline__ v4i load(const XConv& s, int kc, int64_t K) const {
+};
+
+// Position of a thread's k-chunk (chunk c of stage kt) in the k dimension.
+// Stages are visited in increasing order, so the position advances
+// incrementally instead of being decoded with divisions every stage.
+template <class XSRC>
+struct KCursor;
+
+template <>
+struct KCursor<XLinear> {
+  int kc;
+  int c;
+  __device__ __forceinline__ void init(const XLinear&, int c_) { c = c_; kc = c_; }
+  __device__ __forceinline__ void seek(const XLinear&, int kt) { kc = kt * kChunks + c; }
+  __device__ __forceinline__ v4i load(const XLinear&, const XLoader<XLinear>& row, int64_t K) const {
+    int64_t k = static_cast<int64_t>(kc) * 16;
+    k = k < K ? k : K - 16;
+    return ld16(row.p + k);
+  }
+};
+
+template <>
+struct KCursor<XConv> {
+  int kt_cur, c;
+  int kh, kw, blk;      // tap (kh, kw) and 16-channel block of the current chunk
+  int dh, dw, tapoff;   // the tap's input displacement and its byte offset
+  __device__ __forceinline__ void place(const XConv& s) {
+    dh = kh * s.dil_h;
+    dw = kw * s.dil_w;
+    tapoff = (dh * s.W + dw) * s.IC + blk * 16;
+  }
+  __device__ __forceinline__ void init(const XConv& s, int c_) {
+    c = c_;
+    kt_cur = 0;
+    const int tap = c_ / s.icb;
+    blk = c_ - tap * s.icb;
+    kh = tap / s.KW;
+    kw = tap - kh * s.KW;
+    place(s);
+  }
+  // Advances by at most one stage per call (stages are requested in order, the
+  // last one repeatedly).  Written with selects only: a branch between the
+  // global loads would make the compiler drain all outstanding loads.
+  __device__ __forceinline__ void seek(const XConv& s, int kt) {
+    const bool adv = kt > kt_cur;
+    kt_cur = adv ? kt_cur + 1 : kt_cur;
+    int b = blk + (adv ? kChunks : 0);
+    int w = kw, h = kh;
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+      const bool wrap = b >= s.icb;
+      b -= wrap ? s.icb : 0;
+      w += wrap ? 1 : 0;
+      const bool row = w == s.KW;
+      w = row ? 0 : w;
+      h += row ? 1 : 0;
+    }
+    blk = b;
+    kw = w;
+    kh = h;
+    place(s);
+  }
+  // Out-of-image taps read as the activation zero point, i.e. real value 0;
+  // chunks past K land on taps past the kernel window: any in-bounds address
+  // will do there because the packed weight is zero.
+  __device__ __forceinline__ v4i load(const XConv& s, const XLoader<XConv>& row, int64_t K) const {
     const int pw = static_cast<int>(s.pad_word);
-    const int kcc = static_cast<int64_t>(kc) * 16 < K ? kc : 0;
-    const int tap = kcc / s.icb;
-    const int blk = kcc - tap * s.icb;
-    const int kh = tap / s.KW;
-    const int kw = tap - kh * s.KW;
-    const int ih = ih0 + kh * s.dil_h;
-    const int iw = iw0 + kw * s.dil_w;
-    const bool inside = ih >= 0 && ih < s.H && iw >= 0 && iw < s.W;
-    const int ihc = inside ? ih : 0, iwc = inside ? iw : 0;
-    const v4i v = ld16(img + (static_cast<int64_t>(ihc) * s.W + iwc) * s.IC + blk * 16);
+    const bool in_k = static_cast<int64_t>(kt_cur * kChunks + c) * 16 < K;
+    const bool inside = in_k && static_cast<unsigned>(row.ih0 + dh) < static_cast<unsigned>(s.H) &&
+                        static_cast<unsigned>(row.iw0 + dw) < static_cast<unsigned>(s.W);
+    const int off = inside ? row.off0 + tapoff : 0;
+    const v4i v = ld16(row.img + off);
     return v4i{inside ? v.x : pw, inside ? v.y : pw, inside ? v.z : pw, inside ? v.w : pw};
   }
 };
@@ -249,6 +307,8 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     xl[i].init(xsrc, m0 + row, a.M);
     xdst[i] = 2 * kWStage + row * kBK + ((c ^ x_swizzle(row)) << 4);
   }
+  KCursor<XSRC> kcur;
+  kcur.init(xsrc, t & 3);
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
 
@@ -257,8 +317,10 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   auto load_one = [&](int set, int kt, int k) {
     if (k < NW)
       wreg[set][k] = ld16_stream(wsrc[k] + static_cast<int64_t>(kt) * (kChunks * 256));
-    else
-      xreg[set][k - NW] = xl[k - NW].load(xsrc, kt * kChunks + (t & 3), a.K);
+    else {
+      if (k == NW) kcur.seek(xsrc, kt);
+      xreg[set][k - NW] = kcur.load(xsrc, xl[k - NW], a.K);
+    }
   };
   // k-th LDS store of a stage
   auto store_one = [&](int set, int buf, int k) {
