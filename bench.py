@@ -36,14 +36,16 @@ if ROOT not in sys.path:
 PEAK_INT8_TOPS = 5000.0   # dense int8 MFMA, 5.0 POP/s
 PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (one run each, scaled by the same counters on a plain copy of known size);
-# the runs and the scale factor are in profiles/.  None = not measured yet.
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
+# dispatch, one run each: `rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --only linear --steps 3`).
+# Calibration against a plain 1 GiB device copy (`--only copy`): FETCH_SIZE reads 524 300 for
+# 1 048 576 KiB actually read (factor 2.0), WRITE_SIZE reads 1 048 576 (factor 1.0).
+# Summaries: profiles/hbm_traffic_pmc.md.
 MEASURED_TRAFFIC = {
-    "linear_c3": None,
-    "quantize_c2": None,
-    "dequantize_c2": None,
-    "minmax_c2": None,
+    "linear_c3": int((161_200 * 2.0 + 44_030) * 1024),      # 375 MB: operands re-fetched 5.3x by the 8 L2s
+    "quantize_c2": int((524_300 * 2.0 + 262_100) * 1024),   # 1.342 GB = algorithmic
+    "dequantize_c2": int((131_100 * 2.0 + 1_049_000) * 1024),
+    "minmax_c2": int((524_300 * 2.0 + 64) * 1024),
 }
 
 
@@ -162,6 +164,17 @@ def main():
 
     secondary = {}
     if not args.skip_secondary:
+        # ---------------------------------------------- matrix-pipe ceiling probe
+        log("[bench] int8 MFMA ceiling probe (register-only loop, 256 workgroups)")
+        probe = {}
+        for mode, name in ((0, "zero_operands"), (1, "uniform_random_int8"), (2, "gaussian_int8")):
+            tops_p, ghz_p = cabi.probe_mfma_i8(mode)
+            probe[name] = {"tops": round(tops_p, 1), "shader_ghz": round(ghz_p, 3)}
+            log(f"[bench]   {name}: {tops_p:.0f} TOP/s at {ghz_p:.2f} GHz")
+        secondary["mfma_i8_ceiling_probe"] = probe
+        roofline["power_limited_ceiling_tops"] = probe["gaussian_int8"]["tops"]
+        roofline["frac_of_power_limited_ceiling"] = round(achieved / probe["gaussian_int8"]["tops"], 4)
+
         # -------------------------------------------------------------- C2
         n = 2 ** 28
         log("[bench] config 2: quantize / dequantize / min-max over 2**28 fp32")

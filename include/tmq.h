@@ -2,7 +2,7 @@
  * tmq -- quantized-inference kernels for AMD MI355X (gfx950), C ABI.
  *
  * This is the whole device boundary of the library: raw device pointers, sizes,
- * scalars and a HIP stream go in, a status code comes out.  No entry point
+ * scalars and a HIP stream go in, a status code comes out.  No operator entry point
  * allocates, frees, synchronises the device or touches global mutable state, so
  * all of them are asynchronous on `stream`, re-entrant, and callable from
  * several host threads on different streams.  Every buffer (inputs, outputs,
@@ -226,6 +226,17 @@ int tmq_conv2d(const tmq_conv2d_desc* desc, tmq_stream_t stream);
 /* Zero-point-corrected accumulators, [B,OH,OW,OC] int32:
  * acc = sum over in-image taps of (x - x_zp) * w. */
 int tmq_conv2d_acc32(const tmq_conv2d_desc* desc, int32_t* acc, tmq_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Measurement probe (no counterpart in the reference; used by bench.py only).
+ * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four
+ * waves and reports the sustained rate in TOP/s and the shader clock in GHz.
+ * data_mode 0: zero operands, 1: uniform random bytes, 2: Gaussian int8.
+ * Unlike every other entry point this one synchronises (default stream) and
+ * creates two HIP events; `scratch` is >= 2 KiB of device memory.
+ * ------------------------------------------------------------------------- */
+int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, double* tops,
+                      double* shader_ghz);
 
 #ifdef __cplusplus
 }

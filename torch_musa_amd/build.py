@@ -25,7 +25,8 @@ LIB_KERNELS = os.path.join(PKG, "libtmq.so")
 LIB_ATEN = os.path.join(PKG, "libtmq_aten.so")
 ARCH = "gfx950"
 
-KERNEL_SOURCES = ["kernels/quantize.hip", "kernels/linear.hip", "kernels/conv2d.hip"]
+KERNEL_SOURCES = ["kernels/quantize.hip", "kernels/linear.hip", "kernels/conv2d.hip",
+                  "kernels/probe.hip"]
 ATEN_SOURCES = ["aten/register.cpp"]
 
 # -ffp-contract=off: the requantisation epilogue and the quantizer must round

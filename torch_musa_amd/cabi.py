@@ -26,6 +26,7 @@ DECLARED_SYMBOLS = [
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32",
+    "tmq_probe_mfma_i8",
 ]
 
 
@@ -107,6 +108,8 @@ def lib() -> C.CDLL:
         l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         l.tmq_conv2d.argtypes = [C.POINTER(Conv2dDesc), v]
         l.tmq_conv2d_acc32.argtypes = [C.POINTER(Conv2dDesc), v, v]
+        l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, v, C.POINTER(C.c_double),
+                                        C.POINTER(C.c_double)]
         _lib = l
     return _lib
 
@@ -370,3 +373,16 @@ def conv2d_acc32(x_nhwc, pw: PackedConv2d, g: Conv2dGeom, x_zp):
     d = _conv_desc(x_nhwc, pw, g, 1.0, x_zp, None, None, 1.0, 0, False, False, None)
     check(lib().tmq_conv2d_acc32(C.byref(d), acc.data_ptr(), stream_ptr()), "tmq_conv2d_acc32")
     return acc
+
+
+# ---------------------------------------------------------------------------
+# measurement probe
+# ---------------------------------------------------------------------------
+def probe_mfma_i8(data_mode: int, blocks: int = 256, iters: int = 20000):
+    """-> (TOP/s, shader GHz) of a register-only int8 MFMA loop; synchronises."""
+    scratch = torch.zeros(2048, dtype=torch.uint8, device="cuda")
+    tops, ghz = C.c_double(), C.c_double()
+    torch.cuda.synchronize()
+    check(lib().tmq_probe_mfma_i8(data_mode, blocks, iters, scratch.data_ptr(), C.byref(tops),
+                                  C.byref(ghz)), "tmq_probe_mfma_i8")
+    return float(tops.value), float(ghz.value)

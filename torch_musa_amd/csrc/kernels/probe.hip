@@ -1,0 +1,108 @@
+// Measurement probe: what the int8 matrix pipe sustains on this device when it
+// is fed from registers only, as a function of the operand data.  MI355X is
+// power-limited on this instruction: the shader clock, and with it the
+// throughput, depends on how much the operands toggle.  bench.py reports the
+// probe next to the GEMM figure so that the GEMM can be read against the
+// ceiling the silicon actually reaches, not only against the nominal peak.
+#include "common.h"
+
+namespace tmq {
+namespace {
+
+__device__ __forceinline__ unsigned mix(unsigned x) {
+  x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+  return x;
+}
+
+// four bytes ~ N(0, 37) clamped to int8 (sum of four uniform bytes, scaled)
+__device__ __forceinline__ unsigned gaussian_bytes(unsigned seed) {
+  unsigned out = 0;
+  for (int b = 0; b < 4; ++b) {
+    const unsigned h = mix(seed + 77u * b);
+    int g = 0;
+    for (int u = 0; u < 4; ++u) g += static_cast<int>((h >> (8 * u)) & 0xff) - 128;
+    g >>= 2;
+    g = g > 127 ? 127 : (g < -128 ? -128 : g);
+    out |= static_cast<unsigned>(g & 0xff) << (8 * b);
+  }
+  return out;
+}
+
+// data_mode 0: zeros, 1: uniform random bytes, 2: Gaussian int8 (sigma ~37)
+__global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int data_mode, int* sink,
+                                                         long long* stamps) {
+  v16i acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+  v4i a[4], b[4];
+  const unsigned seed = threadIdx.x * 977u + blockIdx.x * 131071u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      unsigned ra = mix(seed + i * 8 + j), rb = mix(seed + 1000 + i * 8 + j);
+      if (data_mode == 0) ra = rb = 0;
+      if (data_mode == 2) {
+        ra = gaussian_bytes(ra);
+        rb = gaussian_bytes(rb);
+      }
+      a[i][j] = static_cast<int>(ra);
+      b[i][j] = static_cast<int>(rb);
+    }
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i >> 1) & 3], acc[i], 0, 0, 0);
+  }
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[i][r];
+  if (s == 0x7fffffff) sink[threadIdx.x] = s;  // keeps the loop alive
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    stamps[0] = c1 - c0;  // shader clock cycles
+    stamps[1] = w1 - w0;  // 100 MHz ticks
+  }
+}
+
+}  // namespace
+}  // namespace tmq
+
+using namespace tmq;
+
+// Synchronous by design (it is a measurement, not an operator): launches one
+// block of 4 waves per `blocks`, times the second of two launches with HIP
+// events, and reads back the clock counters.  `scratch` is device memory of at
+// least 2 KiB owned by the caller.
+TMQ_EXPORT int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, double* tops,
+                                 double* shader_ghz) {
+  if (data_mode < 0 || data_mode > 2 || blocks <= 0 || iters <= 0 || scratch == nullptr ||
+      tops == nullptr || shader_ghz == nullptr)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  int* sink = static_cast<int*>(scratch);
+  long long* stamps = reinterpret_cast<long long*>(static_cast<char*>(scratch) + 1024);
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return TMQ_ERR_LAUNCH;
+  mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
+  hipEventRecord(e0, nullptr);
+  mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
+  hipEventRecord(e1, nullptr);
+  int rc = hipEventSynchronize(e1) == hipSuccess ? TMQ_OK : TMQ_ERR_LAUNCH;
+  float ms = 0.f;
+  long long host[2] = {0, 1};
+  if (rc == TMQ_OK && (hipEventElapsedTime(&ms, e0, e1) != hipSuccess ||
+                       hipMemcpy(host, stamps, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess))
+    rc = TMQ_ERR_LAUNCH;
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  if (rc != TMQ_OK) return rc;
+  const double ops = 2.0 * 32 * 32 * 32 * 8 * static_cast<double>(iters) * 4 * blocks;
+  *tops = ops / (ms * 1e-3) / 1e12;
+  *shader_ghz = static_cast<double>(host[0]) / (static_cast<double>(host[1]) / 100e6) / 1e9;
+  return TMQ_OK;
+}
