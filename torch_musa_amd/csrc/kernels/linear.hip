@@ -213,11 +213,11 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
 // Kernel selection override for benchmarking: -1 = automatic.
 std::atomic<int> g_forced_config{-1};
 
-template <int BM, int BN, int WM, int WN, int MODE>
+template <int BM, int BN, int WM, int WN, int MODE, int PD = 4>
 int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
   if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear>
+  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear, PD>
       <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
   return launch_status();
 }
@@ -247,7 +247,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     // largest tile that still leaves at least ~2 blocks per CU, else smaller
     const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
     if (nblk(256, 256) >= 512)
-      cfg = 0;
+      cfg = 3;  // 8 waves of 128x64: two waves per SIMD cover each other's waits
     else if (nblk(128, 128) >= 256)
       cfg = 1;
     else
@@ -257,7 +257,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
     case 1: return launch_gemm<128, 128, 2, 2, MODE>(a, xs, s);
     case 2: return launch_gemm<64, 64, 2, 2, MODE>(a, xs, s);
-    case 3: return launch_gemm<256, 256, 2, 4, MODE>(a, xs, s);
+    case 3: return launch_gemm<256, 256, 2, 4, MODE, 3>(a, xs, s);
     case 4: return launch_gemm<128, 256, 2, 2, MODE>(a, xs, s);
     case 5: return launch_gemm<256, 128, 2, 2, MODE>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
