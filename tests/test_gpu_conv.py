@@ -80,10 +80,15 @@ def _conv_case(b, h, w, ic, oc, k, s, p, d, g, seed, x_signed=False, relu=False)
     (2, 15, 15, 32, 40, 3, 1, 2, 2, 1),      # dilation
 ])
 @pytest.mark.parametrize("x_signed", [False, True])
-def test_conv_mfma_shapes(cabi, spec, x_signed):
-    say("conv mfma", spec, x_signed)
+@pytest.mark.parametrize("path", [1, 2], ids=["tiles", "gemm"])
+def test_conv_mfma_shapes(cabi, spec, x_signed, path):
+    say("conv mfma", spec, x_signed, path)
     c = _conv_case(*spec, seed=sum(spec), x_signed=x_signed, relu=x_signed)
-    y, acc, _ = _run(cabi, c)
+    cabi.force_conv_path(path)
+    try:
+        y, acc, _ = _run(cabi, c)
+    finally:
+        cabi.force_conv_path(-1)
     np.testing.assert_array_equal(
         acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
                                  c["groups"], c["x_zp"], nthreads=8))
@@ -91,6 +96,30 @@ def test_conv_mfma_shapes(cabi, spec, x_signed):
                          c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
                          c["out_zp"], relu=c["relu"], nthreads=8)
     _check(y, want, "mfma conv")
+
+
+@pytest.mark.parametrize("spec", [
+    (1, 9, 300, 16, 16, 3, 1, 1, 1, 1),      # wide rows: patches split the width
+    (2, 33, 21, 32, 72, 3, 2, 1, 2, 1),      # stride 2 with dilation 2, OC over two 64-channel tiles
+    (1, 12, 12, 96, 48, 3, 1, 1, 1, 4),      # four groups of 24 in, 12 out -> direct kernel
+    (3, 10, 10, 64, 48, 3, 1, 1, 1, 2),      # groups whose 24 channels break 16-byte stores
+    (1, 14, 14, 128, 64, 3, 1, 1, 1, 1),     # 72 KB weight slice in LDS
+    (1, 14, 14, 256, 64, 3, 1, 1, 1, 1),     # weight slice too large for LDS: implicit GEMM
+    (2, 28, 28, 64, 128, 1, 1, 0, 1, 1),     # 1x1
+    (1, 40, 40, 16, 64, 7, 2, 3, 1, 1),      # 7x7 stride 2
+    (1, 1, 1, 16, 1, 1, 1, 0, 1, 1),         # a single output value
+])
+def test_conv_auto_path_shapes(cabi, spec):
+    say("conv auto", spec)
+    c = _conv_case(*spec, seed=sum(spec) + 1)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                 c["groups"], c["x_zp"], nthreads=8))
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "auto conv")
 
 
 def test_c5_full_size(cabi):

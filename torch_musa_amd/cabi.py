@@ -304,6 +304,12 @@ def force_linear_config(cfg: int) -> None:
     lib().tmq_debug_force_linear_config(C.c_int(cfg))
 
 
+def force_conv_path(path: int) -> None:
+    """Test and benchmark hook: pin the conv2d kernel family
+    (-1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct)."""
+    lib().tmq_debug_force_conv_path(C.c_int(path))
+
+
 # ---------------------------------------------------------------------------
 # conv2d
 # ---------------------------------------------------------------------------

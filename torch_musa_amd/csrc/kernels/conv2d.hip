@@ -6,6 +6,10 @@
 // input pixel -- a single aligned load from the NHWC activation tensor.
 // Taps outside the image are filled with the activation zero point (real value
 // 0), which the accumulator start value then cancels exactly.
+#include <atomic>
+#include <type_traits>
+
+#include "conv_tile.h"
 #include "gemm_i8_core.h"
 
 static_assert(sizeof(tmq_conv2d_geom) == 112, "tmq_conv2d_geom layout changed");
@@ -148,6 +152,87 @@ int launch_conv_gemm(const GemmArgs& a, const XConv& xs, hipStream_t s) {
   return launch_status();
 }
 
+std::atomic<int> g_forced_path{-1};
+std::atomic<int> g_forced_rows{0};   // > 0: patch height of the halo-tiled kernel
+std::atomic<int> g_forced_cols{0};   // > 0: upper bound of its patch width  // -1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct
+
+// Patch shape and LDS layout of the halo-tiled kernel for one problem.
+struct TilePlan {
+  int TH, TW, HH, HW, pitch, KS;
+  int lds_x, lds_t, lds_tab, lds_total;
+};
+
+int lds_limit() {
+  static const int limit = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+      return 0;
+    return v;
+  }();
+  return limit;
+}
+
+// Chooses the patch that minimises a simple time estimate: rounds of blocks
+// over the 256 CUs times (fixed cost + MFMA time of the busiest SIMD + copy
+// time).  Returns false when the weight slice or the smallest halo do not fit.
+bool plan_tiles(const ConvShape& s, TilePlan* best) {
+  const int64_t icb = s.ICg / 16;
+  const int64_t chunks = s.KH * s.KW * icb;
+  const int64_t KS = round_up(ceil_div(chunks, 2), 2);  // <= packed k-chunks / 2 (padded to 8)
+  const int64_t w_bytes = 2048 * KS;
+  const int64_t budget = static_cast<int64_t>(lds_limit()) - 3 * kCtBN * 4 - 256;
+  if (w_bytes > 96 * 1024 || icb > 64) return false;
+  const int64_t pitch = (icb | 1) * 16;
+  const int64_t n_tiles = ceil_div(s.OCg, kCtBN);
+  const int64_t tw_caps[6] = {128, 64, 32, 16, 8, 4};
+  double best_cost = -1.0;
+  for (int64_t cap : tw_caps) {
+    const int forced_cols = g_forced_cols.load(std::memory_order_relaxed);
+    if (forced_cols > 0 && cap != 128) continue;
+    const int64_t TW = forced_cols > 0 ? (s.OW < forced_cols ? s.OW : forced_cols) : (s.OW < cap ? s.OW : cap);
+    const int64_t HWd = (TW - 1) * s.sw + (s.KW - 1) * s.dw + 1;
+    if (HWd * (pitch / 16) > kCtThreads) continue;  // one halo row is copied in one pass of the block
+    const int forced_rows = g_forced_rows.load(std::memory_order_relaxed);
+    for (int64_t TH = 1; TH <= s.OH && TH * TW <= kCtMaxPixels; ++TH) {
+      if (forced_rows > 0 && TH != forced_rows) continue;
+      const int64_t HH = (TH - 1) * s.sh + (s.KH - 1) * s.dh + 1;
+      const int64_t x_bytes = round_up(HH * HWd * pitch, 16);
+      const int64_t total = w_bytes + x_bytes + kCtWaves * kCtTBytes + round_up(8 * (KS + 4), 16);
+      if (total > budget) break;
+      const int64_t blocks = s.B * ceil_div(s.OH, TH) * ceil_div(s.OW, TW) * n_tiles * s.groups;
+      const int64_t MT = ceil_div(TH * TW, 32);
+      const double per_block = 3000.0 + static_cast<double>(ceil_div(MT, 4) * KS * 64) +
+                               static_cast<double>(w_bytes + x_bytes) / 64.0;
+      const double cost = static_cast<double>(ceil_div(blocks, 256)) * per_block;
+      if (best_cost < 0 || cost < best_cost) {
+        best_cost = cost;
+        best->TH = static_cast<int>(TH); best->TW = static_cast<int>(TW);
+        best->HH = static_cast<int>(HH); best->HW = static_cast<int>(HWd);
+        best->pitch = static_cast<int>(pitch); best->KS = static_cast<int>(KS);
+        best->lds_x = static_cast<int>(w_bytes);
+        best->lds_t = static_cast<int>(w_bytes + x_bytes);
+        best->lds_tab = best->lds_t + kCtWaves * kCtTBytes;
+        best->lds_total = static_cast<int>(total);
+      }
+    }
+  }
+  return best_cost >= 0;
+}
+
+template <int MODE>
+int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs& a, hipStream_t stream) {
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&conv_tile_kernel<MODE>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit() - 3 * kCtBN * 4);
+  if (attr != hipSuccess) return TMQ_ERR_LAUNCH;
+  const int64_t bx = s.B * a.tiles_h * a.tiles_w, by = static_cast<int64_t>(a.n_tiles) * s.groups;
+  if (bx > 0x7fffffff || by > 65535) return TMQ_ERR_UNSUPPORTED;
+  conv_tile_kernel<MODE><<<dim3(static_cast<unsigned>(bx), static_cast<unsigned>(by)),
+                           dim3(kCtThreads), p.lds_total, stream>>>(a);
+  return launch_status();
+}
+
 template <int MODE>
 int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
   ConvShape s;
@@ -170,8 +255,10 @@ int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
   const float lo_f = static_cast<float>(d->relu ? d->out_zero_point : qmin);
   const float hi_f = static_cast<float>(qmax);
 
+  const int forced = g_forced_path.load(std::memory_order_relaxed);
   const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
-  if (!mfma_ok) {
+  if ((forced == 1 || forced == 2) && !mfma_ok) return TMQ_ERR_UNSUPPORTED;
+  if (!mfma_ok || forced == 3) {
     PlainArgs p{};
     p.x = static_cast<const uint8_t*>(d->x);
     p.w_packed = static_cast<const uint8_t*>(d->w_packed);
@@ -189,6 +276,53 @@ int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
     conv_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(s, p);
     return launch_status();
+  }
+
+  TilePlan plan;
+  const bool tiles_ok = forced != 2 && plan_tiles(s, &plan);
+  if (forced == 1 && !tiles_ok) return TMQ_ERR_UNSUPPORTED;
+  if (tiles_ok) {
+    ConvTileArgs t{};
+    t.x = static_cast<const uint8_t*>(d->x);
+    t.w_packed = static_cast<const uint8_t*>(d->w_packed);
+    t.colsum = d->w_colsum;
+    t.w_scales = d->w_scales;
+    t.bias = d->bias;
+    t.y = out;
+    t.w_kchunks = s.KC;
+    t.group_bytes = s.group_bytes;
+    t.H = static_cast<int>(s.H); t.W = static_cast<int>(s.W); t.IC = static_cast<int>(s.IC);
+    t.OH = static_cast<int>(s.OH); t.OW = static_cast<int>(s.OW); t.OC = static_cast<int>(s.OC);
+    t.KW = static_cast<int>(s.KW); t.icb = static_cast<int>(s.ICg / 16);
+    t.kchunks = static_cast<int>(s.KH * s.KW * (s.ICg / 16));
+    t.KS = plan.KS;
+    t.sh = static_cast<int>(s.sh); t.sw = static_cast<int>(s.sw);
+    t.ph = static_cast<int>(s.ph); t.pw = static_cast<int>(s.pw);
+    t.dh = static_cast<int>(s.dh); t.dw = static_cast<int>(s.dw);
+    t.ICg = static_cast<int>(s.ICg); t.OCg = static_cast<int>(s.OCg);
+    t.n_tiles = static_cast<int>(ceil_div(s.OCg, kCtBN));
+    t.TH = plan.TH; t.TW = plan.TW; t.HH = plan.HH; t.HW = plan.HW; t.pitch = plan.pitch;
+    t.tiles_h = static_cast<int>(ceil_div(s.OH, plan.TH));
+    t.tiles_w = static_cast<int>(ceil_div(s.OW, plan.TW));
+    t.lds_x = plan.lds_x; t.lds_t = plan.lds_t; t.lds_tab = plan.lds_tab;
+    t.w_scale_stride = d->w_per_channel ? 1 : 0;
+    t.x_xor = d->x_signed ? 0u : 0x80808080u;
+    t.pad_word = 0x01010101u * static_cast<uint32_t>(static_cast<uint8_t>(d->x_zero_point));
+    t.acc_coef = (d->x_signed ? 0 : 128) - d->x_zero_point;
+    t.x_scale = d->x_scale;
+    t.out_scale = d->out_scale;
+    t.zp_f = zp_f; t.lo_f = lo_f; t.hi_f = hi_f;
+    t.ri = plan.HW * (plan.pitch / 16);
+    t.rpp = kCtThreads / t.ri;
+    t.cx = (plan.HH + t.rpp - 1) / t.rpp;
+    t.xstep = static_cast<uint32_t>(t.rpp) * static_cast<uint32_t>(s.W) * static_cast<uint32_t>(s.IC);
+    t.xdstep = t.rpp * t.ri * 16;
+    t.rcp_tw = 1.0f / static_cast<float>(plan.TW);
+    t.rcp_ri = 1.0f / static_cast<float>(t.ri);
+    t.rcp_pslots = 16.0f / static_cast<float>(plan.pitch);
+    t.rcp_icb = 1.0f / static_cast<float>(t.icb);
+    t.rcp_kw = 1.0f / static_cast<float>(s.KW);
+    return launch_conv_tiles<MODE>(s, plan, t, stream);
   }
 
   XConv xs{};
@@ -276,6 +410,16 @@ TMQ_EXPORT int tmq_conv2d(const tmq_conv2d_desc* d, tmq_stream_t stream) {
   if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
   return d->out_signed ? run_conv<kOutS8>(d, d->y, as_stream(stream))
                        : run_conv<kOutU8>(d, d->y, as_stream(stream));
+}
+
+// Test and benchmark hook (not part of the public header): force a kernel
+// family.  -1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct.
+TMQ_EXPORT void tmq_debug_force_conv_path(int path) {
+  g_forced_path.store(path, std::memory_order_relaxed);
+}
+TMQ_EXPORT void tmq_debug_force_conv_tile(int rows, int cols) {
+  g_forced_rows.store(rows, std::memory_order_relaxed);
+  g_forced_cols.store(cols, std::memory_order_relaxed);
 }
 
 TMQ_EXPORT int tmq_conv2d_acc32(const tmq_conv2d_desc* d, int32_t* acc, tmq_stream_t stream) {
