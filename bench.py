@@ -262,17 +262,35 @@ def main():
         for _ in range(5):
             conv()
         ts = events_ms(conv, 30)
-        avg = sum(ts) / len(ts)
+        single = sum(ts) / len(ts)
+        # a ~10 us kernel: one launch between two events mostly times the launch
+        # path, so the figure of merit is 50 launches replayed from a HIP graph
+        reps = 50
+        side = torch.cuda.Stream()
+        cgraph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            conv()
+            side.synchronize()
+            with torch.cuda.graph(cgraph, stream=side):
+                for _ in range(reps):
+                    conv()
+        torch.cuda.synchronize()
+        for _ in range(3):
+            cgraph.replay()
+        ts = events_ms(cgraph.replay, 10)
+        avg = sum(ts) / len(ts) / reps
         cops = 2.0 * 32 * 56 * 56 * 64 * 576
         cbytes = 2 * 32 * 56 * 56 * 64 + 64 * 576 + 768
-        log(f"[bench] conv2d C5: {avg*1e3:.1f} us/launch, {cops/(avg*1e-3)/1e12:.0f} TOP/s, "
-            f"{cbytes/(avg*1e-3)/1e9:.0f} GB/s")
+        log(f"[bench] conv2d C5: {avg*1e3:.1f} us/launch in a replayed graph ({single*1e3:.1f} us as a single "
+            f"launch between events), {cops/(avg*1e-3)/1e12:.0f} TOP/s, {cbytes/(avg*1e-3)/1e9:.0f} GB/s")
         secondary["conv2d_c5"] = {
-            "avg_launch_us": round(avg * 1e3, 2), "value": round(cops / (avg * 1e-3) / 1e12, 1), "unit": "TOP/s",
+            "avg_launch_us": round(avg * 1e3, 2), "single_launch_us": round(single * 1e3, 2),
+            "value": round(cops / (avg * 1e-3) / 1e12, 1), "unit": "TOP/s",
             "roofline": {"bound": "mfma", "achieved": round(cops / (avg * 1e-3) / 1e12, 1),
                          "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": round(cops / (avg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "traffic": None},
             "hbm_frac": round(cbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "method": f"{reps} launches replayed back to back in one HIP graph",
             "algorithmic_bytes_per_launch": cbytes, "ops_per_launch": cops}
 
     # ------------------------------------------------------------ CPU baseline

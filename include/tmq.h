@@ -119,6 +119,22 @@ int tmq_dequantize_per_channel(const void* q, float* r, int64_t outer,
                                const int64_t* zero_points, int q_signed,
                                tmq_stream_t stream);
 
+/* Per channel with float scales and float zero points (qscheme
+ * per_channel_affine_float_qparams): q = clamp(lrintf(x * (1/scale_c) + zp_c)),
+ * r = (float(q) - zp_c) * scale_c, all in fp32; a zero scale quantizes with
+ * inverse 1.  Replaces AffineQuantizer.mu:259-301
+ * (quantize_tensor_per_channel_float_qparams_musa) and :303-336
+ * (dequantize_tensor_per_channel_float_qparams_musa).  scales and zero_points
+ * are device arrays of `channels` floats. */
+int tmq_quantize_per_channel_float_qparams(const float* x, void* q, int64_t outer,
+                                           int64_t channels, int64_t inner,
+                                           const float* scales, const float* zero_points,
+                                           int q_signed, tmq_stream_t stream);
+int tmq_dequantize_per_channel_float_qparams(const void* q, float* r, int64_t outer,
+                                             int64_t channels, int64_t inner,
+                                             const float* scales, const float* zero_points,
+                                             int q_signed, tmq_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * quantized::linear weights.
  * Replaces PackedLinearWeightMudnn::prepack

@@ -107,6 +107,30 @@ def dequantize_per_channel(q, scales, zps, axis):
     return r
 
 
+def quantize_per_channel_float(x, scales, zps, axis, is_signed=False):
+    """float scales / float zero points (per_channel_affine_float_qparams)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    scales = np.ascontiguousarray(scales, dtype=np.float32)
+    zps = np.ascontiguousarray(zps, dtype=np.float32)
+    outer, c, inner = _outer_c_inner(x.shape, axis)
+    assert scales.size == c and zps.size == c
+    q = np.empty(x.shape, dtype=_qdtype(is_signed))
+    lib().orc_quantize_per_channel_float(_p(x), C.c_int64(outer), C.c_int64(c), C.c_int64(inner),
+                                         _p(scales), _p(zps), C.c_int(is_signed), _p(q))
+    return q
+
+
+def dequantize_per_channel_float(q, scales, zps, axis):
+    q = _as_bytes(q)
+    scales = np.ascontiguousarray(scales, dtype=np.float32)
+    zps = np.ascontiguousarray(zps, dtype=np.float32)
+    outer, c, inner = _outer_c_inner(q.shape, axis)
+    r = np.empty(q.shape, dtype=np.float32)
+    lib().orc_dequantize_per_channel_float(_p(q), C.c_int64(outer), C.c_int64(c), C.c_int64(inner),
+                                           _p(scales), _p(zps), C.c_int(q.dtype == np.int8), _p(r))
+    return r
+
+
 def minmax(x, nthreads=1):
     x = np.ascontiguousarray(x, dtype=np.float32)
     mn, mx = C.c_float(), C.c_float()

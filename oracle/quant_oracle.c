@@ -142,6 +142,48 @@ ORC_API void orc_dequantize_per_channel(const uint8_t* q, int64_t outer, int64_t
     }
 }
 
+/* per-channel quantize with float scales and float zero points (qscheme
+ * per_channel_affine_float_qparams).  ATen quantize_val_float_qparams
+ * (torch/include/ATen/native/quantized/AffineQuantizerBase.h:44):
+ *   inv = scale == 0 ? 1.0f : 1.0f / scale;  q = clamp(lrintf(x * inv + zp)),
+ * product and sum each rounded to fp32.  Stands behind reference
+ * AffineQuantizer.mu:259-301, which states the same formula (:291-294). */
+ORC_API void orc_quantize_per_channel_float(const float* x, int64_t outer, int64_t C,
+                                            int64_t inner, const float* scales,
+                                            const float* zps, int is_signed, uint8_t* q) {
+  int64_t qmin, qmax;
+  qrange(is_signed, &qmin, &qmax);
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t c = 0; c < C; ++c) {
+      const float inv = scales[c] == 0.0f ? 1.0f : 1.0f / scales[c];
+      const int64_t base = (o * C + c) * inner;
+      for (int64_t i = 0; i < inner; ++i) {
+        volatile float t = x[base + i] * inv;
+        volatile float u = t + zps[c];
+        int64_t v = (int64_t)lrintf(u);
+        if (v < qmin) v = qmin;
+        if (v > qmax) v = qmax;
+        q[base + i] = (uint8_t)v;
+      }
+    }
+}
+
+/* its inverse: r = (float(q) - zp_c) * scale_c in fp32 (reference
+ * AffineQuantizer.mu:303-336, lambda at :331-333). */
+ORC_API void orc_dequantize_per_channel_float(const uint8_t* q, int64_t outer, int64_t C,
+                                              int64_t inner, const float* scales,
+                                              const float* zps, int is_signed, float* r) {
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t c = 0; c < C; ++c) {
+      const int64_t base = (o * C + c) * inner;
+      for (int64_t i = 0; i < inner; ++i) {
+        int32_t v = is_signed ? (int32_t)(int8_t)q[base + i] : (int32_t)q[base + i];
+        volatile float d = (float)v - zps[c];
+        r[base + i] = d * scales[c];
+      }
+    }
+}
+
 /* global min / max of a float array (the two reductions that
  * quantize_per_tensor_dynamic performs before choosing qparams,
  * reference musa_functions.yaml:3515-3519). NaN-free input assumed. */

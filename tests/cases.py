@@ -126,6 +126,33 @@ def quantize_per_channel_cases():
     return out
 
 
+def quantize_per_channel_float_cases():
+    """float scales / float zero points (qscheme per_channel_affine_float_qparams):
+    embedding-style rows along axis 0, an inner axis, fractional zero points,
+    ties (x * inv + zp exactly halfway) and a zero scale."""
+    out = []
+    x = randn(410, (6, 50))
+    mn, mx = x.min(axis=1), x.max(axis=1)
+    s = ((mx - mn) / 255.0).astype(np.float32)
+    z = (-mn / s).astype(np.float32)
+    out.append(dict(name="rows_minmax_u8", x=x, scales=s, zps=z, axis=0, signed=False))
+    x = randn(411, (3, 5, 8))
+    out.append(dict(name="axis1_u8", x=x, scales=np.array([0.02, 0.5, 0.013, 0.1, 0.25], np.float32),
+                    zps=np.array([0.0, 10.5, 127.25, 3.75, 200.0], np.float32), axis=1, signed=False))
+    out.append(dict(name="last_axis_s8", x=x, scales=np.full(8, 0.05, np.float32),
+                    zps=np.array([-3.5, 0, 1.25, -100, 100, 0.5, -0.5, 7], np.float32), axis=2,
+                    signed=True))
+    # exact ties: scale 0.25 (a power of two) and zp .0 / .5 make x*inv+zp land on k + 0.5
+    k = np.arange(-20, 21, dtype=np.float32)
+    x = np.stack([(k + 0.5) * 0.25, k * 0.25]).astype(np.float32)
+    out.append(dict(name="ties_u8", x=x, scales=np.array([0.25, 0.25], np.float32),
+                    zps=np.array([30.0, 30.5], np.float32), axis=0, signed=False))
+    x = randn(412, (2, 7))
+    out.append(dict(name="zero_scale_u8", x=x * 40, scales=np.array([0.0, 0.5], np.float32),
+                    zps=np.array([100.0, 1.0], np.float32), axis=0, signed=False))
+    return out
+
+
 # --------------------------------------------------------------------------
 # quantized::linear
 # --------------------------------------------------------------------------

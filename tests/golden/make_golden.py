@@ -79,6 +79,17 @@ def main():
         g[k + "/q"] = q.int_repr().numpy()
         put_dq(g, k, q.dequantize().numpy())
 
+    # ---- per-channel, float scales / float zero points --------------------
+    for c in cases.quantize_per_channel_float_cases():
+        x = torch.from_numpy(c["x"])
+        q = torch.quantize_per_channel(x, torch.from_numpy(c["scales"]), torch.from_numpy(c["zps"]),
+                                       c["axis"], qdtype(c["signed"]))
+        assert q.qscheme() == torch.per_channel_affine_float_qparams
+        k = "qpcf/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/q"] = q.int_repr().numpy()
+        put_dq(g, k, q.dequantize().numpy())
+
     # ---- quantized::linear (integer-domain cases) ------------------------
     def make_w(wq, w_scales, axis_len):
         wt = torch.from_numpy(wq)

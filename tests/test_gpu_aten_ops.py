@@ -89,6 +89,19 @@ def test_quantize_per_channel(c):
                    torch.quantize_per_channel(x, s, z, c["axis"], dt))
 
 
+@pytest.mark.parametrize("c", cases.quantize_per_channel_float_cases(), ids=lambda c: c["name"])
+def test_quantize_per_channel_float_qparams(c):
+    say("aten qpcf", c["name"])
+    x = torch.from_numpy(c["x"])
+    s, z = torch.from_numpy(c["scales"]), torch.from_numpy(c["zps"])
+    dt = torch.qint8 if c["signed"] else torch.quint8
+    q_gpu = torch.quantize_per_channel(x.cuda(), s.cuda(), z.cuda(), c["axis"], dt)
+    q_cpu = torch.quantize_per_channel(x, s, z, c["axis"], dt)
+    assert q_gpu.qscheme() == torch.per_channel_affine_float_qparams
+    assert torch.equal(q_gpu.int_repr().cpu(), q_cpu.int_repr())
+    assert torch.equal(q_gpu.dequantize().cpu(), q_cpu.dequantize())
+
+
 def test_quantize_per_channel_rejects_bad_zero_point():
     x = torch.randn(2, 3).cuda()
     with pytest.raises(RuntimeError):

@@ -112,6 +112,37 @@ def test_quantize_dequantize_per_channel(cabi, golden, c):
     assert cases.crc(host(r)) == int(golden[k + "/dq_crc"])
 
 
+@pytest.mark.parametrize("c", cases.quantize_per_channel_float_cases(), ids=lambda c: c["name"])
+def test_quantize_dequantize_per_channel_float_qparams(cabi, golden, c):
+    say("qpcf", c["name"])
+    k = "qpcf/" + c["name"]
+    scales, zps = dev(c["scales"]), dev(c["zps"])
+    q = cabi.quantize_per_channel_float_qparams(dev(c["x"]), scales, zps, c["axis"], c["signed"])
+    np.testing.assert_array_equal(host(q), golden[k + "/q"])
+    np.testing.assert_array_equal(
+        host(q), oracle.quantize_per_channel_float(c["x"], c["scales"], c["zps"], c["axis"], c["signed"]))
+    r = cabi.dequantize_per_channel_float_qparams(q, scales, zps, c["axis"])
+    want = oracle.dequantize_per_channel_float(golden[k + "/q"], c["scales"], c["zps"], c["axis"])
+    np.testing.assert_array_equal(host(r), want)
+    assert cases.crc(host(r)) == int(golden[k + "/dq_crc"])
+
+
+def test_per_channel_float_qparams_embedding_sized(cabi):
+    """[rows, dim] table quantized row-wise, unaligned inner size (scalar path)
+    and an aligned one (vector path)."""
+    for rows, dim in ((1000, 130), (257, 64)):
+        say("qpcf table", rows, dim)
+        w = cases.randn(33 + dim, (rows, dim))
+        mn, mx = w.min(axis=1), w.max(axis=1)
+        s = ((mx - mn) / 255.0).astype(np.float32)
+        z = (-mn / s).astype(np.float32)
+        q = cabi.quantize_per_channel_float_qparams(dev(w), dev(s), dev(z), 0, False)
+        want = oracle.quantize_per_channel_float(w, s, z, 0, False)
+        np.testing.assert_array_equal(host(q), want)
+        r = cabi.dequantize_per_channel_float_qparams(q, dev(s), dev(z), 0)
+        np.testing.assert_array_equal(host(r), oracle.dequantize_per_channel_float(want, s, z, 0))
+
+
 def test_per_channel_weight_sized(cabi):
     """[N,K] weight, axis 0, the shape quantized::linear weights come in."""
     say("qpc weight 1000x4096")

@@ -62,6 +62,18 @@ def test_quantize_dequantize_per_channel(golden, c):
         np.testing.assert_array_equal(dq, golden[k + "/dq"])
 
 
+@pytest.mark.parametrize("c", cases.quantize_per_channel_float_cases(), ids=lambda c: c["name"])
+def test_quantize_dequantize_per_channel_float_qparams(golden, c):
+    k = "qpcf/" + c["name"]
+    _check_crc(golden, k + "/x_crc", c["x"])
+    q = oracle.quantize_per_channel_float(c["x"], c["scales"], c["zps"], c["axis"], c["signed"])
+    np.testing.assert_array_equal(q, golden[k + "/q"])
+    dq = oracle.dequantize_per_channel_float(q, c["scales"], c["zps"], c["axis"])
+    assert cases.crc(dq) == int(golden[k + "/dq_crc"])
+    if k + "/dq" in golden:
+        np.testing.assert_array_equal(dq, golden[k + "/dq"])
+
+
 @pytest.mark.parametrize("c", cases.linear_cases(), ids=lambda c: c["name"])
 def test_linear(golden, c):
     k = "lin/" + c["name"]

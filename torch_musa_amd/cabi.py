@@ -22,6 +22,7 @@ DECLARED_SYMBOLS = [
     "tmq_minmax_workspace_bytes", "tmq_minmax", "tmq_choose_qparams_dev",
     "tmq_quantize_per_tensor_dev", "tmq_choose_qparams_host",
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
+    "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
@@ -100,6 +101,8 @@ def lib() -> C.CDLL:
                                               C.POINTER(C.c_double), C.POINTER(C.c_int32)]
         l.tmq_quantize_per_channel.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, v, v, C.c_int, v]
         l.tmq_dequantize_per_channel.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, v, v, C.c_int, v]
+        l.tmq_quantize_per_channel_float_qparams.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, v, v, C.c_int, v]
+        l.tmq_dequantize_per_channel_float_qparams.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, v, v, C.c_int, v]
         l.tmq_linear_prepack.argtypes = [v, C.c_int64, C.c_int64, C.c_int64, v, v, v]
         l.tmq_linear_unpack.argtypes = [v, C.c_int64, C.c_int64, v, C.c_int64, v]
         l.tmq_linear.argtypes = [C.POINTER(LinearDesc), v]
@@ -297,6 +300,30 @@ def linear_acc32(x, pw: PackedLinear):
     check(lib().tmq_linear_acc32(C.byref(d), acc.data_ptr(), acc.stride(0), stream_ptr()),
           "tmq_linear_acc32")
     return acc
+
+
+def quantize_per_channel_float_qparams(x, scales, zps, axis, signed):
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert scales.dtype == torch.float32 and zps.dtype == torch.float32
+    outer, c, inner = _outer_c_inner(tuple(x.shape), axis)
+    q = torch.empty(x.shape, dtype=torch.int8 if signed else torch.uint8, device=x.device)
+    check(lib().tmq_quantize_per_channel_float_qparams(x.data_ptr(), q.data_ptr(), outer, c, inner,
+                                                       scales.data_ptr(), zps.data_ptr(), int(signed),
+                                                       stream_ptr()),
+          "tmq_quantize_per_channel_float_qparams")
+    return q
+
+
+def dequantize_per_channel_float_qparams(q, scales, zps, axis):
+    assert q.is_contiguous()
+    assert scales.dtype == torch.float32 and zps.dtype == torch.float32
+    outer, c, inner = _outer_c_inner(tuple(q.shape), axis)
+    r = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    check(lib().tmq_dequantize_per_channel_float_qparams(q.data_ptr(), r.data_ptr(), outer, c, inner,
+                                                         scales.data_ptr(), zps.data_ptr(),
+                                                         int(q.dtype == torch.int8), stream_ptr()),
+          "tmq_dequantize_per_channel_float_qparams")
+    return r
 
 
 def force_linear_config(cfg: int) -> None:

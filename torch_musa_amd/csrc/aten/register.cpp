@@ -142,6 +142,54 @@ void dequantize_per_channel_stub(const at::Tensor& q, at::Tensor& r, const at::T
                "tmq_dequantize_per_channel");
 }
 
+// Float scales and float zero points (qscheme per_channel_affine_float_qparams,
+// AffineQuantizer.mu:259-336), with the reference's range check of the zero
+// points (check_zero_points_musa, :23-33) and its host synchronisation.
+struct FloatChannelParams {
+  at::Tensor scales, zps;
+};
+
+FloatChannelParams float_channel_params(const at::Tensor& like, const at::Tensor& scales,
+                                        const at::Tensor& zps, int64_t channels, bool sgn) {
+  TORCH_CHECK(scales.numel() == channels && zps.numel() == channels,
+              "per-channel scales / zero points must have one entry per channel");
+  FloatChannelParams p;
+  p.scales = scales.to(like.device(), at::kFloat).contiguous();
+  p.zps = zps.to(like.device(), at::kFloat).contiguous();
+  const int64_t qmin = sgn ? -128 : 0, qmax = sgn ? 127 : 255;
+  if (channels > 0) {
+    const bool bad = p.zps.lt(qmin).logical_or(p.zps.gt(qmax)).any().item<bool>();
+    TORCH_CHECK(!bad, "per-channel zero point outside the range of the quantized dtype");
+  }
+  return p;
+}
+
+void quantize_per_channel_float_qparams_stub(const at::Tensor& r, at::Tensor& q, const at::Tensor& scales,
+                                             const at::Tensor& zps, int64_t axis) {
+  const bool sgn = is_signed_qtype(q.scalar_type(), "quantize_tensor_per_channel_float_qparams");
+  TORCH_CHECK(r.scalar_type() == at::kFloat, "quantize_tensor_per_channel_float_qparams expects a Float tensor");
+  const c10::OptionalDeviceGuard guard(at::device_of(q));
+  const ChannelView v = channel_view(q, axis);
+  const FloatChannelParams p = float_channel_params(q, scales, zps, v.channels, sgn);
+  check_status(tmq_quantize_per_channel_float_qparams(cptr<float>(r), q.data_ptr(), v.outer, v.channels,
+                                                      v.inner, cptr<float>(p.scales), cptr<float>(p.zps), sgn,
+                                                      current_stream(q)),
+               "tmq_quantize_per_channel_float_qparams");
+}
+
+void dequantize_per_channel_float_qparams_stub(const at::Tensor& q, at::Tensor& r, const at::Tensor& scales,
+                                               const at::Tensor& zps, int64_t axis) {
+  const bool sgn = is_signed_qtype(q.scalar_type(), "dequantize_tensor_per_channel_float_qparams");
+  TORCH_CHECK(r.scalar_type() == at::kFloat, "dequantize_tensor_per_channel_float_qparams writes a Float tensor");
+  const c10::OptionalDeviceGuard guard(at::device_of(q));
+  const ChannelView v = channel_view(q, axis);
+  const FloatChannelParams p = float_channel_params(q, scales, zps, v.channels, sgn);
+  check_status(tmq_dequantize_per_channel_float_qparams(q.data_ptr(), mptr<float>(r), v.outer, v.channels,
+                                                        v.inner, cptr<float>(p.scales), cptr<float>(p.zps), sgn,
+                                                        current_stream(q)),
+               "tmq_dequantize_per_channel_float_qparams");
+}
+
 // The stub objects live in libtorch; overriding their GPU slot at load time is
 // the counterpart of REGISTER_PRIVATEUSE1_DISPATCH in the reference.
 struct StubInstaller {
@@ -150,6 +198,10 @@ struct StubInstaller {
     at::native::dequantize_tensor_per_tensor_affine_stub.set_cuda_dispatch_ptr(&dequantize_per_tensor_stub);
     at::native::quantize_tensor_per_channel_affine_stub.set_cuda_dispatch_ptr(&quantize_per_channel_stub);
     at::native::dequantize_tensor_per_channel_affine_stub.set_cuda_dispatch_ptr(&dequantize_per_channel_stub);
+    at::native::quantize_tensor_per_channel_float_qparams_stub.set_cuda_dispatch_ptr(
+        &quantize_per_channel_float_qparams_stub);
+    at::native::dequantize_tensor_per_channel_float_qparams_stub.set_cuda_dispatch_ptr(
+        &dequantize_per_channel_float_qparams_stub);
   }
 } const g_stub_installer;
 

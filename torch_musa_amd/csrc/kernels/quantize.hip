@@ -361,6 +361,69 @@ __global__ __launch_bounds__(kThreads) void dequantize_pc_kernel(
   }
 }
 
+// Per-channel quantizer with float scales and float zero points
+// (qscheme per_channel_affine_float_qparams): q = clamp(lrintf(x * inv + zp)),
+// inv = 1 / scale (1 when the scale is 0), r = (float(q) - zp) * scale, all fp32.
+template <bool SIGNED>
+__device__ __forceinline__ uint32_t quantize_fq_one(float x, float inv, float zp) {
+  const float t = x * inv;
+  float r = __builtin_rintf(t + zp);
+  r = __builtin_amdgcn_fmed3f(r, SIGNED ? -128.f : 0.f, SIGNED ? 127.f : 255.f);
+  return static_cast<uint32_t>(static_cast<int>(r)) & 0xffu;
+}
+
+template <bool SIGNED, int VEC>
+__global__ __launch_bounds__(kThreads) void quantize_pcf_kernel(
+    const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, int64_t C, int64_t inner,
+    const float* __restrict__ scales, const float* __restrict__ zps) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads * VEC;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * VEC; i < n;
+       i += stride) {
+    const int64_t c = (i / inner) % C;
+    const float sc = scales[c];
+    const float inv = sc == 0.f ? 1.0f : 1.0f / sc;
+    const float zp = zps[c];
+    if constexpr (VEC == 4) {
+      const v4f v = *reinterpret_cast<const v4f*>(x + i);
+      *reinterpret_cast<uint32_t*>(q + i) =
+          quantize_fq_one<SIGNED>(v.x, inv, zp) | (quantize_fq_one<SIGNED>(v.y, inv, zp) << 8) |
+          (quantize_fq_one<SIGNED>(v.z, inv, zp) << 16) | (quantize_fq_one<SIGNED>(v.w, inv, zp) << 24);
+    } else {
+      q[i] = static_cast<uint8_t>(quantize_fq_one<SIGNED>(x[i], inv, zp));
+    }
+  }
+}
+
+template <bool SIGNED>
+__device__ __forceinline__ float dequantize_fq_one(uint32_t byte, float zp, float scale) {
+  const int v = SIGNED ? static_cast<int>(static_cast<int8_t>(byte)) : static_cast<int>(byte);
+  const float d = static_cast<float>(v) - zp;
+  return d * scale;
+}
+
+template <bool SIGNED, int VEC>
+__global__ __launch_bounds__(kThreads) void dequantize_pcf_kernel(
+    const uint8_t* __restrict__ q, float* __restrict__ r, int64_t n, int64_t C, int64_t inner,
+    const float* __restrict__ scales, const float* __restrict__ zps) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads * VEC;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * VEC; i < n;
+       i += stride) {
+    const int64_t c = (i / inner) % C;
+    const float scale = scales[c], zp = zps[c];
+    if constexpr (VEC == 4) {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(q + i);
+      v4f o;
+      o.x = dequantize_fq_one<SIGNED>(w & 0xffu, zp, scale);
+      o.y = dequantize_fq_one<SIGNED>((w >> 8) & 0xffu, zp, scale);
+      o.z = dequantize_fq_one<SIGNED>((w >> 16) & 0xffu, zp, scale);
+      o.w = dequantize_fq_one<SIGNED>(w >> 24, zp, scale);
+      *reinterpret_cast<v4f*>(r + i) = o;
+    } else {
+      r[i] = dequantize_fq_one<SIGNED>(q[i], zp, scale);
+    }
+  }
+}
+
 inline unsigned grid_for(int64_t work_items, int64_t per_block, int64_t cap) {
   int64_t g = ceil_div(work_items, per_block);
   if (g < 1) g = 1;
@@ -557,6 +620,60 @@ TMQ_EXPORT int tmq_dequantize_per_channel(const void* q, float* r, int64_t outer
       dequantize_pc_kernel<true, 1><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
     else
       dequantize_pc_kernel<false, 1><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_quantize_per_channel_float_qparams(const float* x, void* q, int64_t outer,
+                                                      int64_t channels, int64_t inner,
+                                                      const float* scales, const float* zero_points,
+                                                      int q_signed, tmq_stream_t stream) {
+  if (outer < 0 || channels < 0 || inner < 0) return TMQ_ERR_INVALID_ARGUMENT;
+  const int64_t n = outer * channels * inner;
+  if (n == 0) return TMQ_OK;
+  if (x == nullptr || q == nullptr || scales == nullptr || zero_points == nullptr)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  hipStream_t s = as_stream(stream);
+  uint8_t* qb = static_cast<uint8_t*>(q);
+  const bool vec = inner % 4 == 0 && aligned(x, 16) && aligned(q, 4);
+  const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
+  if (vec) {
+    if (q_signed)
+      quantize_pcf_kernel<true, 4><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+    else
+      quantize_pcf_kernel<false, 4><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+  } else {
+    if (q_signed)
+      quantize_pcf_kernel<true, 1><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+    else
+      quantize_pcf_kernel<false, 1><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, channels, inner, scales, zero_points);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_dequantize_per_channel_float_qparams(const void* q, float* r, int64_t outer,
+                                                        int64_t channels, int64_t inner,
+                                                        const float* scales, const float* zero_points,
+                                                        int q_signed, tmq_stream_t stream) {
+  if (outer < 0 || channels < 0 || inner < 0) return TMQ_ERR_INVALID_ARGUMENT;
+  const int64_t n = outer * channels * inner;
+  if (n == 0) return TMQ_OK;
+  if (r == nullptr || q == nullptr || scales == nullptr || zero_points == nullptr)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  hipStream_t s = as_stream(stream);
+  const uint8_t* qb = static_cast<const uint8_t*>(q);
+  const bool vec = inner % 4 == 0 && aligned(r, 16) && aligned(q, 4);
+  const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
+  if (vec) {
+    if (q_signed)
+      dequantize_pcf_kernel<true, 4><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+    else
+      dequantize_pcf_kernel<false, 4><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+  } else {
+    if (q_signed)
+      dequantize_pcf_kernel<true, 1><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
+    else
+      dequantize_pcf_kernel<false, 1><<<dim3(g), dim3(kThreads), 0, s>>>(qb, r, n, channels, inner, scales, zero_points);
   }
   return launch_status();
 }
