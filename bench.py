@@ -116,22 +116,37 @@ def main():
     # ------------------------------------------------------------------ C3
     M, K, N = 4096, 4096, 11008
     log(f"[bench] building config 3: M={M} K={K} N={N}")
-    x = torch.randn(M, K, device=dev)
-    w = torch.randn(N, K, device=dev) * 0.02
-    bias = torch.randn(N, device=dev)
-    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
-    w_scales = (w.abs().amax(dim=1) / 127.0).to(torch.float64)
-    wq = torch.quantize_per_channel(w, w_scales, torch.zeros(N, dtype=torch.int64, device=dev), 0, torch.qint8)
-    packed = torch.ops.quantized.linear_prepack(wq, bias)
-    # output scale from a calibration pass of the fp32 result, fixed thereafter
-    y_f = torch.nn.functional.linear(xq.dequantize()[:256], wq.dequantize(), bias)
-    out_scale = float((y_f.max() - y_f.min()) / 255.0)
-    out_zp = int(round(float(-y_f.min()) / out_scale))
-    out_zp = max(0, min(255, out_zp))
-    del x, w, y_f
+    # Operands rotate over 4 sets (4 x 107 MB of inputs and outputs, more than the
+    # 256 MB last-level cache) so that no step finds its operands cached by the
+    # step before.
+    NSETS = 4
+    xqs, packs = [], []
+    for i in range(NSETS):
+        x = torch.randn(M, K, device=dev)
+        w = torch.randn(N, K, device=dev) * 0.02
+        bias = torch.randn(N, device=dev)
+        xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+        w_scales = (w.abs().amax(dim=1) / 127.0).to(torch.float64)
+        wq = torch.quantize_per_channel(w, w_scales, torch.zeros(N, dtype=torch.int64, device=dev), 0, torch.qint8)
+        xqs.append(xq)
+        packs.append(torch.ops.quantized.linear_prepack(wq, bias))
+        if i == 0:
+            # output scale from a calibration pass of the fp32 result, fixed thereafter
+            y_f = torch.nn.functional.linear(xq.dequantize()[:256], wq.dequantize(), bias)
+            out_scale = float((y_f.max() - y_f.min()) / 255.0)
+            out_zp = int(round(float(-y_f.min()) / out_scale))
+            out_zp = max(0, min(255, out_zp))
+            xq0, wq0, w_scales0, bias0 = xq, wq, w_scales, bias
+            del y_f
+        del x, w
+    xq, wq, w_scales, bias = xq0, wq0, w_scales0, bias0
+    packed = packs[0]
+    counter = [0]
 
     def step():
-        return torch.ops.quantized.linear(xq, packed, out_scale, out_zp)
+        i = counter[0] % NSETS
+        counter[0] += 1
+        return torch.ops.quantized.linear(xqs[i], packs[i], out_scale, out_zp)
 
     if args.only == "linear":
         for _ in range(args.steps):
@@ -160,7 +175,8 @@ def main():
                 "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": MEASURED_TRAFFIC["linear_c3"],
                 "kernel": "tmq::gemm_i8_kernel", "ops_per_launch": ops,
                 "avg_launch_us": round(kern_ms * 1e3, 2),
-                "algorithmic_bytes_per_launch": M * K + N * K + M * N + 12 * N}
+                "algorithmic_bytes_per_launch": M * K + N * K + M * N + 12 * N,
+                "operand_sets_rotated": NSETS}
 
     secondary = {}
     if not args.skip_secondary:
@@ -258,14 +274,28 @@ def main():
         wcs = (wc.abs().amax(dim=(1, 2, 3)) / 127.0).to(torch.float64)
         wcq = torch.quantize_per_channel(wc, wcs, torch.zeros(64, dtype=torch.int64, device=dev), 0, torch.qint8)
         pc = torch.ops.quantized.conv2d_prepack(wcq, torch.randn(64, device=dev), [1, 1], [1, 1], [1, 1], 1)
-        conv = lambda: torch.ops.quantized.conv2d(xcq, pc, 0.05, 0)
+        # 24 input tensors (and as many outputs inside the graph): 309 MB, more than
+        # the last-level cache, so a launch does not find its input cached
+        csets = 24
+        xcqs = [xcq]
+        for _ in range(csets - 1):
+            xf_ = torch.relu(torch.randn(32, 64, 56, 56, device=dev)).contiguous(memory_format=torch.channels_last)
+            xcqs.append(torch.quantize_per_tensor(xf_, xcq.q_scale(), xcq.q_zero_point(), torch.quint8))
+            del xf_
+        assert all(t_.is_contiguous(memory_format=torch.channels_last) for t_ in xcqs)
+        ccount = [0]
+
+        def conv():
+            ccount[0] += 1
+            return torch.ops.quantized.conv2d(xcqs[ccount[0] % csets], pc, 0.05, 0)
+
         for _ in range(5):
             conv()
         ts = events_ms(conv, 30)
         single = sum(ts) / len(ts)
         # a ~10 us kernel: one launch between two events mostly times the launch
         # path, so the figure of merit is 50 launches replayed from a HIP graph
-        reps = 50
+        reps = 2 * csets
         side = torch.cuda.Stream()
         cgraph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
@@ -290,7 +320,7 @@ def main():
                          "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": round(cops / (avg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "traffic": None},
             "hbm_frac": round(cbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-            "method": f"{reps} launches replayed back to back in one HIP graph",
+            "method": f"{reps} launches over {csets} rotating inputs replayed back to back in one HIP graph",
             "algorithmic_bytes_per_launch": cbytes, "ops_per_launch": cops}
 
     # ------------------------------------------------------------ CPU baseline
@@ -310,7 +340,7 @@ def main():
                               nthreads=cores)
         dt = time.perf_counter() - t0
         cpu_tops = 2.0 * rows * N * K / dt / 1e12
-        got = step().int_repr()[:rows].cpu().numpy()
+        got = torch.ops.quantized.linear(xq, packed, out_scale, out_zp).int_repr()[:rows].cpu().numpy()
         max_diff = int(np.abs(got.astype(np.int32) - y_ref.astype(np.int32)).max())
         log(f"[bench] CPU oracle: {dt:.2f} s, {cpu_tops*1e3:.2f} GOP/s; GPU vs oracle max diff {max_diff} LSB")
         cpu_baseline = {"value": round(cpu_tops, 5), "unit": "TOP/s", "cores": cores, "kind": "port",
