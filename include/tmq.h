@@ -244,6 +244,30 @@ int tmq_conv2d(const tmq_conv2d_desc* desc, tmq_stream_t stream);
 int tmq_conv2d_acc32(const tmq_conv2d_desc* desc, int32_t* acc, tmq_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * quantized::conv2d_add / conv2d_add_relu / conv2d_silu / conv2d_add_silu.
+ * Replaces PackedConvWeightMudnn<2>::apply_add, apply_add_relu, apply_add_silu
+ * (torch_musa/csrc/aten/quantized/mudnn/ConvAdd.cpp:11-39) and the SILU mode of
+ * apply_impl_helper (mudnn/Conv.cpp:86-130: residual tensor `add` and
+ * FusedActivationDesc handed to muDNN RunFusion).
+ *   t = (float(acc) + bias/(x_scale*w_scale)) * (x_scale*w_scale/out_scale)
+ *   t += float(accum_q - accum_zero_point) * (accum_scale/out_scale)   if accum
+ *   t  = silu(t*out_scale)/out_scale                                    if activation == 2
+ *   y  = clamp(rne(t) + out_zero_point), lower clamp out_zero_point if relu
+ * accum is [B,OH,OW,OC] bytes dense (NHWC, the output's shape) or NULL.
+ * activation: 0 identity, 1 relu, 2 silu; desc->relu also selects relu.
+ * ------------------------------------------------------------------------- */
+typedef struct tmq_conv2d_post {
+  const void* accum;
+  int32_t accum_signed;
+  int32_t accum_zero_point;
+  float accum_scale;
+  int32_t activation;
+} tmq_conv2d_post;
+
+int tmq_conv2d_fused(const tmq_conv2d_desc* desc, const tmq_conv2d_post* post,
+                     tmq_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Measurement probe (no counterpart in the reference; used by bench.py only).
  * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four
  * waves and reports the sustained rate in TOP/s and the shader clock in GHz.

@@ -262,3 +262,41 @@ def conv2d(x_nhwc, x_scale, x_zp, w_ohwi, w_scales, bias, stride, padding,
                      C.c_int64(out_zp), C.c_int(out_signed), C.c_int(relu), _p(y),
                      C.c_int(nthreads))
     return y
+
+
+_ACT = {"none": 0, "relu": 1, "silu": 2}
+
+
+def conv2d_fused(x_nhwc, x_scale, x_zp, w_ohwi, w_scales, bias, stride, padding, dilation,
+                 groups, out_scale, out_zp, accum=None, accum_scale=1.0, accum_zp=0,
+                 activation="none", out_signed=None, nthreads=1):
+    """conv2d with an optional quantized residual (NHWC bytes, the output's
+    shape) and an activation ("none", "relu", "silu"); returns NHWC bytes."""
+    x = _as_bytes(x_nhwc)
+    w = np.ascontiguousarray(w_ohwi, dtype=np.int8)
+    if out_signed is None:
+        out_signed = x.dtype == np.int8
+    b, h, wd, ic = x.shape
+    oc, kh, kw, icg = w.shape
+    assert icg * groups == ic and oc % groups == 0
+    oh, ow = conv_out_hw(h, wd, kh, kw, stride, padding, dilation)
+    w_scales = np.ascontiguousarray(np.atleast_1d(w_scales), dtype=np.float64)
+    assert w_scales.size in (1, oc)
+    bb = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    aa = None
+    if accum is not None:
+        aa = _as_bytes(accum)
+        assert aa.shape == (b, oh, ow, oc)
+    y = np.empty((b, oh, ow, oc), dtype=_qdtype(out_signed))
+    lib().orc_conv2d_fused(_p(x), C.c_int(x.dtype == np.int8), _p(w),
+                           *[C.c_int64(v) for v in (b, h, wd, ic, oc, kh, kw, stride[0], stride[1],
+                                                    padding[0], padding[1], dilation[0], dilation[1],
+                                                    groups, x_zp)],
+                           C.c_double(x_scale), _p(w_scales), C.c_int64(w_scales.size),
+                           _p(bb) if bb is not None else None,
+                           _p(aa) if aa is not None else None,
+                           C.c_int(aa is not None and aa.dtype == np.int8), C.c_int64(accum_zp),
+                           C.c_double(accum_scale), C.c_int(_ACT[activation]),
+                           C.c_double(out_scale), C.c_int64(out_zp), C.c_int(out_signed), _p(y),
+                           C.c_int(nthreads))
+    return y

@@ -409,3 +409,74 @@ ORC_API void orc_conv2d(const uint8_t* x, int x_signed, const int8_t* w, int64_t
   free(acc);
   free(zero);
 }
+
+/* ------------------------------------------------------------------------- */
+/* Fused residual / activation variants of quantized::conv2d: conv2d_add,
+ * conv2d_add_relu (reference mudnn/ConvAdd.cpp:11-39,63-99), conv2d_silu and
+ * conv2d_add_silu (mudnn/Conv.cpp:278-288).  The reference hands the whole
+ * expression to muDNN's Convolution::RunFusion (mudnn/Conv.cpp:86-130, closed
+ * source); its tests define the result as
+ *   quantize( act( conv(dq(x), dq(w)) + bias + dq(accum) ) )   within 1 LSB
+ * (tests/unittest/quantized/test_quantized_conv.py:159-227, :236-360).
+ * This restatement keeps the plain conv's requantisation and adds the residual
+ * in output-scale units before the single rounding:
+ *   t = (float(raw) + bias/atw) * mult                       (as requant_one)
+ *   t = t + float(qa - za) * amult,  amult = fl(fl(accum_scale) / fl(out_scale))
+ *   silu: r = t * out_scale;  t = (r / (1 + expf(-r))) / out_scale
+ *   q = clamp(rne(t) + out_zp, relu ? out_zp : qmin, qmax)
+ * every operation rounded to fp32.  With no accum and no silu this is exactly
+ * orc_conv2d.  activation: 0 identity, 1 relu, 2 silu. */
+ORC_API void orc_conv2d_fused(const uint8_t* x, int x_signed, const int8_t* w, int64_t B,
+                              int64_t H, int64_t W, int64_t IC, int64_t OC, int64_t KH,
+                              int64_t KW, int64_t sh, int64_t sw, int64_t ph, int64_t pw,
+                              int64_t dh, int64_t dw, int64_t groups, int64_t x_zp,
+                              double x_scale, const double* w_scales, int64_t n_scales,
+                              const float* bias, const uint8_t* accum, int accum_signed,
+                              int64_t accum_zp, double accum_scale, int activation,
+                              double out_scale, int64_t out_zp, int out_signed, uint8_t* y,
+                              int nthreads) {
+  const int64_t OH = (H + 2 * ph - dh * (KH - 1) - 1) / sh + 1;
+  const int64_t OW = (W + 2 * pw - dw * (KW - 1) - 1) / sw + 1;
+  const int64_t rows = B * OH * OW;
+  int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)rows * (size_t)OC);
+  orc_conv2d_acc32(x, x_signed, w, B, H, W, IC, OC, KH, KW, sh, sw, ph, pw, dh, dw,
+                   groups, x_zp, acc, nthreads);
+  int64_t qmin, qmax;
+  qrange(out_signed, &qmin, &qmax);
+  const int64_t lo = activation == 1 ? (out_zp > qmin ? out_zp : qmin) : qmin;
+  const float xs = (float)x_scale, os = (float)out_scale;
+  volatile float amult = (float)accum_scale / os;
+  for (int64_t n = 0; n < OC; ++n) {
+    const float ws = (float)w_scales[n_scales == 1 ? 0 : n];
+    volatile float atw = xs * ws;
+    volatile float mult = atw / os;
+    for (int64_t m = 0; m < rows; ++m) {
+      volatile float raw_f = (float)acc[m * OC + n];
+      if (bias != NULL) {
+        volatile float b = bias[n] / atw;
+        raw_f = raw_f + b;
+      }
+      volatile float t = raw_f * mult;
+      if (accum != NULL) {
+        const int32_t qa = accum_signed ? (int32_t)(int8_t)accum[m * OC + n]
+                                        : (int32_t)accum[m * OC + n];
+        volatile float a = (float)(qa - (int32_t)accum_zp) * amult;
+        t = t + a;
+      }
+      if (activation == 2) {
+        volatile float r = t * os;
+        volatile float e = expf(-r);
+        volatile float d = 1.0f + e;
+        volatile float sl = r / d;
+        t = sl / os;
+      }
+      float r = nearbyintf(t);
+      int64_t q;
+      if (!(r > -2147483648.0f)) q = lo;
+      else if (!(r < 2147483648.0f)) q = qmax;
+      else q = clamp_i64((int64_t)r + out_zp, lo, qmax);
+      y[m * OC + n] = (uint8_t)q;
+    }
+  }
+  free(acc);
+}

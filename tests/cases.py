@@ -250,3 +250,57 @@ def conv_cases():
                         out_scale=out_scale, out_zp=128 if not relu else 5,
                         relu=relu))
     return out
+
+
+# --------------------------------------------------------------------------
+# fused residual / activation variants of quantized::conv2d
+# --------------------------------------------------------------------------
+def conv_fused_cases():
+    """conv2d_add, conv2d_add_relu, conv2d_silu, conv2d_add_silu on float-born
+    data, the way the reference's tests build them (a quantized input, a
+    quantized residual of the output's shape, weights quantized per tensor or
+    per channel)."""
+    spec = [
+        # name, B, IC, H, W, OC, k, stride, pad, groups, bias, per_channel, activation, accum, signed
+        ("add_16to32_k3", 2, 16, 12, 12, 32, 3, 1, 1, 1, True, False, "none", True, False),
+        ("add_relu_32to64_k3s2", 2, 32, 15, 15, 64, 3, 2, 1, 1, True, True, "relu", True, False),
+        ("silu_16to16_k3", 1, 16, 10, 10, 16, 3, 1, 1, 1, False, False, "silu", False, False),
+        ("add_silu_32to48_k1", 2, 32, 9, 7, 48, 1, 1, 0, 1, True, True, "silu", True, False),
+        ("add_groups2_64to64", 2, 64, 8, 8, 64, 3, 1, 1, 2, True, True, "none", True, False),
+        ("add_relu_3to8_k3_direct", 2, 3, 11, 11, 8, 3, 1, 1, 1, True, False, "relu", True, False),
+        ("add_s8_16to24_k3", 2, 16, 10, 10, 24, 3, 1, 1, 1, True, False, "none", True, True),
+        ("add_silu_s8_16to32_k3", 1, 16, 9, 9, 32, 3, 1, 1, 1, False, False, "silu", True, True),
+    ]
+    out = []
+    for i, (name, b, ic, h, w, oc, k, s, p, g, has_bias, pc, act, has_acc, signed) in enumerate(spec):
+        rng = np.random.default_rng(1200 + i)
+        x = rng.standard_normal((b, h, w, ic), dtype=np.float32)
+        wt = rng.standard_normal((oc, k, k, ic // g), dtype=np.float32) * np.float32(0.1)
+        bias = rng.standard_normal(oc, dtype=np.float32) if has_bias else None
+        x_scale = float(np.float32(np.abs(x).max() / 128.0))
+        x_zp = 0 if signed else 128
+        lo, hi = (-128, 127) if signed else (0, 255)
+        xq = np.clip(np.rint(x / np.float32(x_scale)) + x_zp, lo, hi).astype(np.int8 if signed else np.uint8)
+        if pc:
+            w_scales = (np.abs(wt).reshape(oc, -1).max(axis=1) / np.float32(127.0)).astype(np.float64)
+            wq = np.clip(np.rint(wt / w_scales.astype(np.float32)[:, None, None, None]), -127, 127).astype(np.int8)
+        else:
+            w_scales = np.array([float(np.float32(np.abs(wt).max() / 128.0))])
+            wq = np.clip(np.rint(wt / np.float32(w_scales[0])), -127, 127).astype(np.int8)
+        oh = (h + 2 * p - (k - 1) - 1) // s + 1
+        ow = (w + 2 * p - (k - 1) - 1) // s + 1
+        acc = accq = None
+        acc_scale, acc_zp = 1.0, 0
+        if has_acc:
+            acc = rng.standard_normal((b, oh, ow, oc), dtype=np.float32) * np.float32(2.0)
+            acc_scale = float(np.float32(np.abs(acc).max() / 128.0))
+            acc_zp = 0 if signed else 128
+            accq = np.clip(np.rint(acc / np.float32(acc_scale)) + acc_zp, lo, hi).astype(xq.dtype)
+        # spread of conv + residual, for an output scale that uses the range
+        sigma = float(np.sqrt(k * k * (ic // g)) * 0.1 + (2.0 if has_acc else 0.0))
+        out_scale = float(np.float32(3.0 * sigma / 128.0))
+        out.append(dict(name=name, xq=xq, x_scale=x_scale, x_zp=x_zp, wq=wq, w_scales=w_scales, bias=bias,
+                        stride=(s, s), padding=(p, p), dilation=(1, 1), groups=g, accq=accq,
+                        acc_scale=acc_scale, acc_zp=acc_zp, activation=act, out_scale=out_scale,
+                        out_zp=0 if signed else 128, signed=signed))
+    return out

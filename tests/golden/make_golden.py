@@ -139,6 +139,37 @@ def main():
             meta[f"c1_mismatch_{eng}"] = int((y2.int_repr() != y.int_repr()).sum())
     torch.backends.quantized.engine = "fbgemm"
 
+    # ---- fused conv variants: the float pipeline of the reference's tests ----
+    # quantize( act( conv(dq(x), dq(w)) + bias + dq(accum) ) )
+    # (test_quantized_conv.py:159-227, :236-360 of the reference)
+    for c in cases.conv_fused_cases():
+        qd = torch.qint8 if c["signed"] else torch.quint8
+        xq = torch._make_per_tensor_quantized_tensor(
+            torch.from_numpy(c["xq"]).permute(0, 3, 1, 2).contiguous(), c["x_scale"], c["x_zp"])
+        wt = torch.from_numpy(c["wq"]).permute(0, 3, 1, 2).contiguous()
+        if len(c["w_scales"]) == 1:
+            w = torch._make_per_tensor_quantized_tensor(wt, float(c["w_scales"][0]), 0)
+        else:
+            w = torch._make_per_channel_quantized_tensor(
+                wt, torch.from_numpy(c["w_scales"]), torch.zeros(wt.shape[0], dtype=torch.int64), 0)
+        b = None if c["bias"] is None else torch.from_numpy(c["bias"])
+        f = torch.nn.functional.conv2d(xq.dequantize().double(), w.dequantize().double(),
+                                       None if b is None else b.double(), c["stride"], c["padding"],
+                                       c["dilation"], c["groups"])
+        if c["accq"] is not None:
+            aq = torch._make_per_tensor_quantized_tensor(
+                torch.from_numpy(c["accq"]).permute(0, 3, 1, 2).contiguous(), c["acc_scale"], c["acc_zp"])
+            f = f + aq.dequantize().double()
+        if c["activation"] == "relu":
+            f = torch.relu(f)
+        elif c["activation"] == "silu":
+            f = torch.nn.functional.silu(f)
+        y = torch.quantize_per_tensor(f.float(), c["out_scale"], c["out_zp"], qd)
+        k = "convf/" + c["name"]
+        g[k + "/xq_crc"] = np.uint32(cases.crc(c["xq"]))
+        g[k + "/wq_crc"] = np.uint32(cases.crc(c["wq"]))
+        g[k + "/y"] = y.int_repr().permute(0, 2, 3, 1).contiguous().numpy()
+
     # ---- quantized::conv2d -------------------------------------------------
     for c in cases.conv_cases():
         x_nchw = torch.from_numpy(c["xq"]).permute(0, 3, 1, 2)  # channels-last view

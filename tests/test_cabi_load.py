@@ -40,6 +40,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(cabi.LinearDesc) == 128
     assert C.sizeof(cabi.Conv2dGeom) == 14 * 8
     assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8
+    assert C.sizeof(cabi.Conv2dPost) == 24
 
 
 def test_packed_size_arithmetic():

@@ -266,3 +266,48 @@ def test_qconv2d_errors():
     x = torch.quantize_per_tensor(torch.randn(1, 5, 8, 8), 0.1, 0, torch.quint8).cuda()
     with pytest.raises(RuntimeError):
         torch.ops.quantized.conv2d(x, packed, 0.1, 0)                             # channel mismatch
+
+
+# ---------------------------------------------------------------------------
+# fused conv ops (quantized::conv2d_add, conv2d_add_relu, conv2d_silu, conv2d_add_silu)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("c", cases.conv_fused_cases(), ids=lambda c: c["name"])
+def test_conv2d_fused_ops(golden, c):
+    say("aten conv fused", c["name"])
+    qd = torch.qint8 if c["signed"] else torch.quint8
+    xq = torch._make_per_tensor_quantized_tensor(
+        torch.from_numpy(c["xq"]).cuda().permute(0, 3, 1, 2), c["x_scale"], c["x_zp"])
+    wt = torch.from_numpy(c["wq"]).permute(0, 3, 1, 2).contiguous().cuda()
+    if len(c["w_scales"]) == 1:
+        w = torch._make_per_tensor_quantized_tensor(wt, float(c["w_scales"][0]), 0)
+    else:
+        w = torch._make_per_channel_quantized_tensor(
+            wt, torch.from_numpy(c["w_scales"]).cuda(), torch.zeros(wt.shape[0], dtype=torch.int64).cuda(), 0)
+    b = None if c["bias"] is None else torch.from_numpy(c["bias"]).cuda()
+    packed = torch.ops.quantized.conv2d_prepack(w, b, list(c["stride"]), list(c["padding"]),
+                                                list(c["dilation"]), c["groups"])
+    ops = torch.ops.quantized
+    if c["accq"] is not None:
+        aq = torch._make_per_tensor_quantized_tensor(
+            torch.from_numpy(c["accq"]).cuda().permute(0, 3, 1, 2), c["acc_scale"], c["acc_zp"])
+        op = {"none": ops.conv2d_add, "relu": ops.conv2d_add_relu, "silu": ops.conv2d_add_silu}[c["activation"]]
+        y = op(xq, aq, packed, c["out_scale"], c["out_zp"])
+    else:
+        assert c["activation"] == "silu"
+        y = ops.conv2d_silu(xq, packed, c["out_scale"], c["out_zp"])
+    assert y.dtype == qd and y.q_scale() == c["out_scale"] and y.q_zero_point() == c["out_zp"]
+    assert y.is_contiguous(memory_format=torch.channels_last)
+    got = y.int_repr().permute(0, 2, 3, 1).contiguous().cpu().numpy()
+    d = np.abs(got.astype(np.int32) - golden["convf/" + c["name"] + "/y"].astype(np.int32))
+    assert d.max() <= 1 and np.count_nonzero(d) <= 0.003 * d.size
+
+
+def test_conv2d_add_rejects_wrong_accum():
+    w = torch._make_per_tensor_quantized_tensor(torch.zeros(8, 16, 3, 3, dtype=torch.int8).cuda(), 0.1, 0)
+    packed = torch.ops.quantized.conv2d_prepack(w, None, [1, 1], [1, 1], [1, 1], 1)
+    x = torch._make_per_tensor_quantized_tensor(torch.zeros(1, 16, 5, 5, dtype=torch.uint8).cuda(), 0.1, 0)
+    bad = torch._make_per_tensor_quantized_tensor(torch.zeros(1, 8, 4, 4, dtype=torch.uint8).cuda(), 0.1, 0)
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.conv2d_add(x, bad, packed, 0.1, 0)
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.conv2d_add(x, torch.zeros(1, 8, 5, 5).cuda(), packed, 0.1, 0)

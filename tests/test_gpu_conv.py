@@ -143,3 +143,64 @@ def test_c5_full_size(cabi):
                          nthreads=8)
     assert 0.2 < np.mean((want > 0) & (want < 255))
     _check(y, want, "C5")
+
+
+# ---------------------------------------------------------------------------
+# fused residual / activation variants
+# ---------------------------------------------------------------------------
+def _run_fused(cabi, c):
+    g = cabi.conv_geom(c["xq"].shape, c["wq"].shape, c["stride"], c["padding"], c["dilation"],
+                       c["groups"])
+    pw = cabi.PackedConv2d(dev(c["wq"]), g)
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    acc = None if c["accq"] is None else dev(c["accq"])
+    y = cabi.conv2d_fused(dev(c["xq"]), pw, g, c["x_scale"], c["x_zp"], ws, b, c["out_scale"],
+                          c["out_zp"], accum=acc, accum_scale=c["acc_scale"], accum_zp=c["acc_zp"],
+                          activation=c["activation"], out_signed=c["signed"])
+    return host(y)
+
+
+@pytest.mark.parametrize("path", [-1, 2, 3], ids=["auto", "gemm", "direct"])
+@pytest.mark.parametrize("c", cases.conv_fused_cases(), ids=lambda c: c["name"])
+def test_conv_fused(cabi, golden, c, path):
+    say("conv fused", c["name"], path)
+    if path == 2 and (c["xq"].shape[3] // c["groups"]) % 16 != 0:
+        pytest.skip("the MFMA kernels need 16-channel blocks")
+    cabi.force_conv_path(path)
+    try:
+        y = _run_fused(cabi, c)
+    finally:
+        cabi.force_conv_path(-1)
+    want = oracle.conv2d_fused(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                               c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                               c["out_zp"], accum=c["accq"], accum_scale=c["acc_scale"],
+                               accum_zp=c["acc_zp"], activation=c["activation"], out_signed=c["signed"],
+                               nthreads=8)
+    d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+    if c["activation"] == "silu":
+        # expf on the device and on the host may differ in the last bit
+        assert d.max() <= LSB_TOL and np.count_nonzero(d) <= 0.001 * d.size, (d.max(), np.count_nonzero(d))
+    else:
+        assert d.max() == 0, f"{np.count_nonzero(d)} of {d.size} bytes differ (max {d.max()})"
+    dg = np.abs(y.astype(np.int32) - golden["convf/" + c["name"] + "/y"].astype(np.int32))
+    assert dg.max() <= LSB_TOL and np.count_nonzero(dg) <= 0.003 * dg.size
+
+
+def test_conv_fused_c5_sized(cabi):
+    """conv2d_add_relu at BASELINE config 5's size (the residual block of a ResNet stage)."""
+    say("conv fused C5 size")
+    rng = np.random.default_rng(56)
+    xq = rng.integers(0, 256, (32, 56, 56, 64), dtype=np.uint8)
+    wq = rng.integers(-127, 128, (64, 3, 3, 64), dtype=np.int8)
+    accq = rng.integers(0, 256, (32, 56, 56, 64), dtype=np.uint8)
+    ws = (0.001 + 0.002 * rng.random(64)).astype(np.float32).astype(np.float64)
+    bias = rng.standard_normal(64).astype(np.float32)
+    c = dict(xq=xq, wq=wq, accq=accq, w_scales=ws, bias=bias, x_scale=0.02, x_zp=3, stride=(1, 1),
+             padding=(1, 1), dilation=(1, 1), groups=1, out_scale=0.9, out_zp=20, acc_scale=0.35,
+             acc_zp=110, activation="relu", signed=False)
+    y = _run_fused(cabi, c)
+    want = oracle.conv2d_fused(xq, 0.02, 3, wq, ws, bias, (1, 1), (1, 1), (1, 1), 1, 0.9, 20, accum=accq,
+                               accum_scale=0.35, accum_zp=110, activation="relu", nthreads=8)
+    assert 0.2 < np.mean((want > 20) & (want < 255))
+    np.testing.assert_array_equal(y, want)

@@ -115,3 +115,23 @@ def test_conv2d(golden, c):
     want = golden[k + "/y"]
     assert y.shape == want.shape
     np.testing.assert_array_equal(y, want)
+
+
+@pytest.mark.parametrize("c", cases.conv_fused_cases(), ids=lambda c: c["name"])
+def test_conv2d_fused_vs_float_pipeline(golden, c):
+    """The fused variants are defined by the reference's tests as the float
+    pipeline quantize(act(conv(dq x, dq w) + bias + dq accum)) within 1 LSB;
+    the golden file holds that pipeline evaluated in float64."""
+    k = "convf/" + c["name"]
+    _check_crc(golden, k + "/xq_crc", c["xq"])
+    _check_crc(golden, k + "/wq_crc", c["wq"])
+    y = oracle.conv2d_fused(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                            c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                            c["out_zp"], accum=c["accq"], accum_scale=c["acc_scale"],
+                            accum_zp=c["acc_zp"], activation=c["activation"], out_signed=c["signed"])
+    want = golden[k + "/y"]
+    lo, hi = (-128, 127) if c["signed"] else (0, 255)
+    assert 0.5 < np.mean((want > lo) & (want < hi)), "degenerate case"
+    d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+    assert d.max() <= 1
+    assert np.count_nonzero(d) <= 0.002 * d.size, f"{np.count_nonzero(d)} of {d.size} differ"

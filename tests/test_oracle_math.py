@@ -186,3 +186,60 @@ def test_conv_1x1_is_linear():
     yc = oracle.conv2d(x, 0.03, 50, w, ws, bias, (1, 1), (0, 0), (1, 1), 1, 0.08, 120)
     yl = oracle.linear(x.reshape(-1, 16), 0.03, 50, w.reshape(12, 16), ws, bias, 0.08, 120)
     np.testing.assert_array_equal(yc.reshape(-1, 12), yl)
+
+
+# ---------------------------------------------------------------------------
+# fused conv variants: special cases that fix each term of the closed form
+# ---------------------------------------------------------------------------
+def _fused_inputs(seed=5):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 256, (2, 7, 6, 16), dtype=np.uint8)
+    w = rng.integers(-127, 128, (8, 3, 3, 16), dtype=np.int8)
+    ws = (0.001 + 0.002 * rng.random(8)).astype(np.float32).astype(np.float64)
+    bias = rng.standard_normal(8).astype(np.float32)
+    return rng, x, w, ws, bias
+
+
+def test_fused_without_post_ops_is_plain_conv():
+    _, x, w, ws, bias = _fused_inputs()
+    for relu in (False, True):
+        a = oracle.conv2d(x, 0.03, 90, w, ws, bias, (1, 1), (1, 1), (1, 1), 1, 0.4, 100, relu=relu)
+        b = oracle.conv2d_fused(x, 0.03, 90, w, ws, bias, (1, 1), (1, 1), (1, 1), 1, 0.4, 100,
+                                activation="relu" if relu else "none")
+        np.testing.assert_array_equal(a, b)
+
+
+def test_fused_residual_at_its_zero_point_adds_nothing():
+    _, x, w, ws, bias = _fused_inputs()
+    acc = np.full((2, 7, 6, 8), 77, np.uint8)
+    a = oracle.conv2d(x, 0.03, 90, w, ws, bias, (1, 1), (1, 1), (1, 1), 1, 0.4, 100)
+    b = oracle.conv2d_fused(x, 0.03, 90, w, ws, bias, (1, 1), (1, 1), (1, 1), 1, 0.4, 100, accum=acc,
+                            accum_scale=0.123, accum_zp=77)
+    np.testing.assert_array_equal(a, b)
+
+
+def test_fused_zero_weights_pass_the_residual_through():
+    """conv == 0 and accum_scale == out_scale: y = qa - za + zp, clamped; with a
+    scale ratio of 2 the residual's distance from its zero point doubles."""
+    rng, x, w, ws, _ = _fused_inputs()
+    acc = rng.integers(0, 256, (2, 7, 6, 8), dtype=np.uint8)
+    y = oracle.conv2d_fused(x, 0.03, 90, np.zeros_like(w), ws, None, (1, 1), (1, 1), (1, 1), 1, 0.25,
+                            100, accum=acc, accum_scale=0.25, accum_zp=120)
+    np.testing.assert_array_equal(y, np.clip(acc.astype(int) - 120 + 100, 0, 255))
+    y2 = oracle.conv2d_fused(x, 0.03, 90, np.zeros_like(w), ws, None, (1, 1), (1, 1), (1, 1), 1, 0.25,
+                             100, accum=acc, accum_scale=0.5, accum_zp=120, activation="relu")
+    np.testing.assert_array_equal(y2, np.clip(2 * (acc.astype(int) - 120) + 100, 100, 255))
+
+
+def test_fused_silu_of_a_known_value():
+    """One output value at a time: conv == 0, residual r, silu(r) = r / (1 + e^-r)."""
+    _, x, w, ws, _ = _fused_inputs()
+    acc = np.arange(2 * 7 * 6 * 8, dtype=np.int64).reshape(2, 7, 6, 8) % 256
+    acc = acc.astype(np.uint8)
+    s = 0.05
+    y = oracle.conv2d_fused(x, 0.03, 90, np.zeros_like(w), ws, None, (1, 1), (1, 1), (1, 1), 1, s, 30,
+                            accum=acc, accum_scale=s, accum_zp=128, activation="silu")
+    r = (acc.astype(np.float64) - 128) * s
+    want = np.clip(np.rint(r / (1 + np.exp(-r)) / s) + 30, 0, 255)
+    d = np.abs(y.astype(int) - want.astype(int))
+    assert d.max() <= 1 and np.count_nonzero(d) <= 2  # float32 vs float64 at exact ties only

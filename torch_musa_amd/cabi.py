@@ -26,7 +26,7 @@ DECLARED_SYMBOLS = [
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
-    "tmq_conv2d", "tmq_conv2d_acc32",
+    "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_probe_mfma_i8",
 ]
 
@@ -73,6 +73,16 @@ class Conv2dDesc(C.Structure):
     ]
 
 
+class Conv2dPost(C.Structure):
+    _fields_ = [
+        ("accum", C.c_void_p),
+        ("accum_signed", C.c_int32), ("accum_zero_point", C.c_int32), ("accum_scale", C.c_float),
+        ("activation", C.c_int32),
+    ]
+
+
+ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2}
+
 _lib = None
 
 
@@ -111,6 +121,7 @@ def lib() -> C.CDLL:
         l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         l.tmq_conv2d.argtypes = [C.POINTER(Conv2dDesc), v]
         l.tmq_conv2d_acc32.argtypes = [C.POINTER(Conv2dDesc), v, v]
+        l.tmq_conv2d_fused.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(Conv2dPost), v]
         l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, v, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]
         _lib = l
@@ -397,6 +408,30 @@ def conv2d(x_nhwc, pw: PackedConv2d, g: Conv2dGeom, x_scale, x_zp, w_scales, bia
     d = _conv_desc(x_nhwc, pw, g, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed,
                    relu, y)
     check(lib().tmq_conv2d(C.byref(d), stream_ptr()), "tmq_conv2d")
+    return y
+
+
+def conv2d_fused(x_nhwc, pw: PackedConv2d, g: Conv2dGeom, x_scale, x_zp, w_scales, bias, out_scale,
+                 out_zp, accum=None, accum_scale=1.0, accum_zp=0, activation="none", out_signed=None,
+                 out=None):
+    """conv2d + optional quantized residual (NHWC bytes, the output's shape) + activation."""
+    assert x_nhwc.is_contiguous() and tuple(x_nhwc.shape) == (g.B, g.H, g.W, g.IC)
+    if out_signed is None:
+        out_signed = x_nhwc.dtype == torch.int8
+    oh, ow = conv_out_hw(g)
+    y = out if out is not None else torch.empty(
+        (g.B, oh, ow, g.OC), dtype=torch.int8 if out_signed else torch.uint8, device=x_nhwc.device)
+    d = _conv_desc(x_nhwc, pw, g, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed,
+                   False, y)
+    post = Conv2dPost()
+    if accum is not None:
+        assert accum.is_contiguous() and tuple(accum.shape) == (g.B, oh, ow, g.OC)
+        post.accum = accum.data_ptr()
+        post.accum_signed = int(accum.dtype == torch.int8)
+    post.accum_zero_point = int(accum_zp)
+    post.accum_scale = float(accum_scale)
+    post.activation = ACTIVATIONS[activation]
+    check(lib().tmq_conv2d_fused(C.byref(d), C.byref(post), stream_ptr()), "tmq_conv2d_fused")
     return y
 
 

@@ -10,7 +10,9 @@
 //   * quantized::linear / linear_relu / linear_prepack (mudnn/Linear.cpp:134-158,
 //     mudnn/LinearPrepack.cpp:39-57) and quantized::conv2d.new / conv2d_relu.new /
 //     conv2d_prepack (mudnn/Conv.cpp:252-288, mudnn/ConvPrepack.cpp:109-225),
-//     registered on the quantized GPU dispatch key with the upstream schemas.
+//     registered on the quantized GPU dispatch key with the upstream schemas;
+//   * the fused variants quantized::conv2d_add / conv2d_add_relu / conv2d_add_silu
+//     (mudnn/ConvAdd.cpp:63-99) and conv2d_silu.new (mudnn/Conv.cpp:285-287).
 // This file only validates, allocates through the caching allocator and calls
 // the C ABI of include/tmq.h on the current stream; it contains no kernels.
 // Unlike the reference (muDNN: symmetric qint8 only, mudnn/Linear.cpp:80-85,
@@ -411,10 +413,16 @@ struct PackedConvWeightTmq final : public ConvPackedParamsBase<2> {
         padding_(std::move(padding)), dilation_(std::move(dilation)), groups_(groups) {}
 
   at::Tensor apply(const at::Tensor& input, double output_scale, int64_t output_zero_point) override {
-    return apply_impl(input, output_scale, output_zero_point, false);
+    return apply_impl(input, std::nullopt, output_scale, output_zero_point, 0);
+  }
+  // Fused residual / activation variants (mudnn/ConvAdd.cpp:11-39, ActMode::SILU
+  // of mudnn/Conv.cpp:38-133).  activation: 0 identity, 1 relu, 2 silu.
+  at::Tensor apply_fused(const at::Tensor& input, const std::optional<at::Tensor>& accum,
+                         double output_scale, int64_t output_zero_point, int activation) {
+    return apply_impl(input, accum, output_scale, output_zero_point, activation);
   }
   at::Tensor apply_relu(const at::Tensor& input, double output_scale, int64_t output_zero_point) override {
-    return apply_impl(input, output_scale, output_zero_point, true);
+    return apply_impl(input, std::nullopt, output_scale, output_zero_point, 1);
   }
   at::Tensor apply_dynamic(const at::Tensor&, bool) override {
     TORCH_CHECK(false, "apply_dynamic is not implemented for this packed parameter type");
@@ -467,7 +475,8 @@ struct PackedConvWeightTmq final : public ConvPackedParamsBase<2> {
   }
 
  private:
-  at::Tensor apply_impl(const at::Tensor& act, double output_scale, int64_t output_zero_point, bool relu) {
+  at::Tensor apply_impl(const at::Tensor& act, const std::optional<at::Tensor>& accum, double output_scale,
+                        int64_t output_zero_point, int activation) {
     TORCH_CHECK(act.qscheme() == c10::kPerTensorAffine || act.qscheme() == c10::kPerTensorSymmetric,
                 "Conv2d only supports per-tensor quantized activation");
     const bool x_signed = is_signed_qtype(act.scalar_type(), "quantized::conv2d");
@@ -518,9 +527,30 @@ struct PackedConvWeightTmq final : public ConvPackedParamsBase<2> {
     d.out_scale = static_cast<float>(output_scale);
     d.out_zero_point = static_cast<int32_t>(output_zero_point);
     d.out_signed = x_signed;
-    d.relu = relu;
+    d.relu = activation == 1;
     d.y = y.data_ptr();
-    check_status(tmq_conv2d(&d, current_stream(x)), "tmq_conv2d");
+    if (!accum.has_value() && activation != 2) {
+      check_status(tmq_conv2d(&d, current_stream(x)), "tmq_conv2d");
+      return y;
+    }
+    tmq_conv2d_post post{};
+    post.activation = activation;
+    at::Tensor acc_nhwc;  // keeps a channels-last copy alive until the launch is enqueued
+    if (accum.has_value()) {
+      const at::Tensor& a = *accum;
+      TORCH_CHECK(a.is_quantized(), "accum tensor in qconv must be a quantized Tensor");
+      TORCH_CHECK(a.qscheme() == c10::kPerTensorAffine || a.qscheme() == c10::kPerTensorSymmetric,
+                  "quantized::conv2d_add only supports a per-tensor quantized accum");
+      TORCH_CHECK(a.sizes() == y.sizes(), "quantized::conv2d_add: accum has shape ", a.sizes(),
+                  ", the convolution produces ", y.sizes());
+      TORCH_CHECK(a.device() == x.device(), "quantized::conv2d_add: accum on a different device");
+      acc_nhwc = a.contiguous(c10::MemoryFormat::ChannelsLast);
+      post.accum = acc_nhwc.data_ptr();
+      post.accum_signed = is_signed_qtype(a.scalar_type(), "quantized::conv2d_add");
+      post.accum_zero_point = static_cast<int32_t>(a.q_zero_point());
+      post.accum_scale = static_cast<float>(a.q_scale());
+    }
+    check_status(tmq_conv2d_fused(&d, &post, current_stream(x)), "tmq_conv2d_fused");
     return y;
   }
 
@@ -538,6 +568,27 @@ at::Tensor qconv2d_relu_run(at::Tensor act, const c10::intrusive_ptr<ConvPackedP
                             int64_t z) {
   return w->apply_relu(act, s, z);
 }
+PackedConvWeightTmq& tmq_conv(const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w, const char* op) {
+  auto* p = dynamic_cast<PackedConvWeightTmq*>(w.get());
+  TORCH_CHECK(p != nullptr, op, ": the packed weight was not made by quantized::conv2d_prepack on this device");
+  return *p;
+}
+at::Tensor qconv2d_add_run(at::Tensor act, at::Tensor accum, const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w,
+                           double s, int64_t z) {
+  return tmq_conv(w, "quantized::conv2d_add").apply_fused(act, accum, s, z, 0);
+}
+at::Tensor qconv2d_add_relu_run(at::Tensor act, at::Tensor accum,
+                                const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w, double s, int64_t z) {
+  return tmq_conv(w, "quantized::conv2d_add_relu").apply_fused(act, accum, s, z, 1);
+}
+at::Tensor qconv2d_silu_run(at::Tensor act, const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w, double s,
+                            int64_t z) {
+  return tmq_conv(w, "quantized::conv2d_silu").apply_fused(act, std::nullopt, s, z, 2);
+}
+at::Tensor qconv2d_add_silu_run(at::Tensor act, at::Tensor accum,
+                                const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w, double s, int64_t z) {
+  return tmq_conv(w, "quantized::conv2d_add_silu").apply_fused(act, accum, s, z, 2);
+}
 c10::intrusive_ptr<ConvPackedParamsBase<2>> qconv2d_prepack_run(at::Tensor weight, std::optional<at::Tensor> bias,
                                                                 torch::List<int64_t> stride,
                                                                 torch::List<int64_t> padding,
@@ -548,7 +599,25 @@ c10::intrusive_ptr<ConvPackedParamsBase<2>> qconv2d_prepack_run(at::Tensor weigh
 
 }  // namespace
 
+// The two SiLU schemas are not part of upstream PyTorch; the reference adds them
+// by patching ATen's quantized/library.cpp
+// (torch_patches/aten_src_ATen_native_quantized_library.cpp.patch:9,12).  Here
+// they are defined from this library.
+TORCH_LIBRARY_FRAGMENT(quantized, m) {
+  m.def(TORCH_SELECTIVE_SCHEMA(
+      "quantized::conv2d_silu.new(Tensor qx, __torch__.torch.classes.quantized.Conv2dPackedParamsBase "
+      "packed_weight, float output_scale, int output_zero_point) -> Tensor"));
+  m.def(TORCH_SELECTIVE_SCHEMA(
+      "quantized::conv2d_add_silu(Tensor qx, Tensor qaccum, "
+      "__torch__.torch.classes.quantized.Conv2dPackedParamsBase packed_weight, float output_scale, "
+      "int output_zero_point) -> Tensor"));
+}
+
 TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add"), TORCH_FN(qconv2d_add_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add_relu"), TORCH_FN(qconv2d_add_relu_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_silu.new"), TORCH_FN(qconv2d_silu_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add_silu"), TORCH_FN(qconv2d_add_silu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear"), TORCH_FN(qlinear_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear_relu"), TORCH_FN(qlinear_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear_prepack"), TORCH_FN(qlinear_prepack_run));

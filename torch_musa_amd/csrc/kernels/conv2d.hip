@@ -14,6 +14,7 @@
 
 static_assert(sizeof(tmq_conv2d_geom) == 112, "tmq_conv2d_geom layout changed");
 static_assert(sizeof(tmq_conv2d_desc) == 192, "tmq_conv2d_desc layout changed");
+static_assert(sizeof(tmq_conv2d_post) == 24, "tmq_conv2d_post layout changed");
 
 namespace tmq {
 namespace {
@@ -99,6 +100,7 @@ struct PlainArgs {
   int32_t w_scale_stride, x_signed, x_zp;
   float x_scale, out_scale, zp_f, lo_f, hi_f;
   void* y;
+  PostOps post;
 };
 
 // Direct convolution, one thread per output value: any channel count, any
@@ -136,7 +138,20 @@ __global__ __launch_bounds__(256) void conv_plain_kernel(ConvShape s, PlainArgs 
     const float mult = atw / a.out_scale;
     float v = static_cast<float>(acc);
     if (a.bias != nullptr) v = v + a.bias[oc] / atw;
-    const float ab = v * mult;
+    float ab = v * mult;
+    if (a.post.accum != nullptr) {
+      const uint8_t b8 = a.post.accum[id];
+      const int qa = a.post.accum_signed ? static_cast<int>(static_cast<int8_t>(b8)) : static_cast<int>(b8);
+      const float ad = static_cast<float>(qa - a.post.accum_zp) * a.post.amult;
+      ab = ab + ad;
+    }
+    if (a.post.silu) {
+      const float rv = ab * a.post.out_scale;
+      const float e = expf(-rv);
+      const float dd = 1.0f + e;
+      const float sl = rv / dd;
+      ab = sl / a.post.out_scale;
+    }
     float r = __builtin_rintf(ab) + a.zp_f;
     r = __builtin_amdgcn_fmed3f(r, a.lo_f, a.hi_f);
     static_cast<uint8_t*>(a.y)[id] = static_cast<uint8_t>(static_cast<int>(r));
@@ -234,7 +249,7 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
 }
 
 template <int MODE>
-int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
+int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, hipStream_t stream) {
   ConvShape s;
   int rc = make_shape(&d->geom, &s);
   if (rc != TMQ_OK) return rc;
@@ -251,8 +266,27 @@ int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
       return TMQ_ERR_INVALID_ARGUMENT;
     if (d->out_zero_point < qmin || d->out_zero_point > qmax) return TMQ_ERR_INVALID_ARGUMENT;
   }
+  PostOps po{};
+  bool relu = d->relu != 0;
+  if (post != nullptr) {
+    if (MODE == kOutAcc32) return TMQ_ERR_INVALID_ARGUMENT;
+    if (post->activation < 0 || post->activation > 2) return TMQ_ERR_INVALID_ARGUMENT;
+    if (post->activation == 2 && relu) return TMQ_ERR_INVALID_ARGUMENT;
+    relu = relu || post->activation == 1;
+    po.silu = post->activation == 2;
+    po.out_scale = d->out_scale;
+    if (post->accum != nullptr) {
+      const int amin = post->accum_signed ? -128 : 0, amax = post->accum_signed ? 127 : 255;
+      if (!(post->accum_scale > 0.f) || post->accum_zero_point < amin || post->accum_zero_point > amax)
+        return TMQ_ERR_INVALID_ARGUMENT;
+      po.accum = static_cast<const uint8_t*>(post->accum);
+      po.accum_signed = post->accum_signed;
+      po.accum_zp = post->accum_zero_point;
+      po.amult = post->accum_scale / d->out_scale;
+    }
+  }
   const float zp_f = static_cast<float>(d->out_zero_point);
-  const float lo_f = static_cast<float>(d->relu ? d->out_zero_point : qmin);
+  const float lo_f = static_cast<float>(relu ? d->out_zero_point : qmin);
   const float hi_f = static_cast<float>(qmax);
 
   const int forced = g_forced_path.load(std::memory_order_relaxed);
@@ -272,6 +306,7 @@ int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
     p.out_scale = d->out_scale;
     p.zp_f = zp_f; p.lo_f = lo_f; p.hi_f = hi_f;
     p.y = out;
+    p.post = po;
     const int64_t blocks = ceil_div(rows * s.OC, 256);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
     conv_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(s, p);
@@ -317,6 +352,7 @@ int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
     t.cx = (plan.HH + t.rpp - 1) / t.rpp;
     t.xstep = static_cast<uint32_t>(t.rpp) * static_cast<uint32_t>(s.W) * static_cast<uint32_t>(s.IC);
     t.xdstep = t.rpp * t.ri * 16;
+    t.post = po;
     t.rcp_tw = 1.0f / static_cast<float>(plan.TW);
     t.rcp_ri = 1.0f / static_cast<float>(t.ri);
     t.rcp_pslots = 16.0f / static_cast<float>(plan.pitch);
@@ -351,6 +387,7 @@ int run_conv(const tmq_conv2d_desc* d, void* out, hipStream_t stream) {
   a.zp_f = zp_f; a.lo_f = lo_f; a.hi_f = hi_f;
   a.y = out;
   a.ldy = s.OC;
+  a.post = po;
   for (int64_t g = 0; g < s.groups; ++g) {
     a.w_packed = static_cast<const uint8_t*>(d->w_packed) + g * s.group_bytes;
     a.n_off = static_cast<int32_t>(g * s.OCg);
@@ -408,8 +445,15 @@ TMQ_EXPORT int tmq_conv2d_prepack(const int8_t* w_ohwi, const tmq_conv2d_geom* g
 
 TMQ_EXPORT int tmq_conv2d(const tmq_conv2d_desc* d, tmq_stream_t stream) {
   if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
-  return d->out_signed ? run_conv<kOutS8>(d, d->y, as_stream(stream))
-                       : run_conv<kOutU8>(d, d->y, as_stream(stream));
+  return d->out_signed ? run_conv<kOutS8>(d, nullptr, d->y, as_stream(stream))
+                       : run_conv<kOutU8>(d, nullptr, d->y, as_stream(stream));
+}
+
+TMQ_EXPORT int tmq_conv2d_fused(const tmq_conv2d_desc* d, const tmq_conv2d_post* post,
+                                tmq_stream_t stream) {
+  if (d == nullptr || post == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  return d->out_signed ? run_conv<kOutS8>(d, post, d->y, as_stream(stream))
+                       : run_conv<kOutU8>(d, post, d->y, as_stream(stream));
 }
 
 // Test and benchmark hook (not part of the public header): force a kernel
@@ -424,5 +468,5 @@ TMQ_EXPORT void tmq_debug_force_conv_tile(int rows, int cols) {
 
 TMQ_EXPORT int tmq_conv2d_acc32(const tmq_conv2d_desc* d, int32_t* acc, tmq_stream_t stream) {
   if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
-  return run_conv<kOutAcc32>(d, acc, as_stream(stream));
+  return run_conv<kOutAcc32>(d, nullptr, acc, as_stream(stream));
 }

@@ -60,6 +60,7 @@ struct ConvTileArgs {
   int32_t acc_coef;
   float x_scale, out_scale, zp_f, lo_f, hi_f;
   float rcp_tw, rcp_ri, rcp_icb, rcp_kw, rcp_pslots;  // 1 / TW, 1 / ri, 1 / icb, 1 / KW, 16 / pitch
+  PostOps post;
 };
 
 // n / d for n < 2**22 with rcp = 1.0f / d: the float estimate is off by at most
@@ -355,8 +356,18 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
             int raw[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * gq + j];
-            *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) =
-                requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+            uint32_t q4;
+            if (a.post.any()) {
+              const int left = a.OCg - (n0 + nl);
+              const int nvalid = (opix[tm] >= 0 && left > 0) ? (left < 4 ? left : 4) : 0;
+              const uint32_t accw = (a.post.accum != nullptr && nvalid > 0)
+                                        ? load_accum4(a.post, static_cast<int64_t>(opix[tm]) * a.OC + ch0 + nl, nvalid)
+                                        : 0u;
+              q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
+            } else {
+              q4 = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+            }
+            *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) = q4;
           }
         wave_sync_lds();
         // whole pixels leave as 16 bytes per lane: 4 lanes per pixel, 16 pixels per pass

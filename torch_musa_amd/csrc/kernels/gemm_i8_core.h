@@ -36,11 +36,13 @@ enum EpilogueMode { kOutU8 = 0, kOutS8 = 1, kOutAcc32 = 2 };
 
 // Where a tile's activation rows come from.
 struct XLinear {
+  static constexpr bool kPostOps = false;
   const uint8_t* x;
   int64_t ldx;
 };
 
 struct XConv {
+  static constexpr bool kPostOps = true;
   const uint8_t* x;  // NHWC
   int H, W, IC;      // IC = all input channels (row pitch of a pixel)
   int OH, OW;
@@ -48,6 +50,18 @@ struct XConv {
   int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
   int ic_off;        // first input channel of this group
   uint32_t pad_word; // activation zero point replicated in 4 bytes
+};
+
+// Optional work between the requantisation's multiply and its rounding:
+//   t += float(accum_q - accum_zp) * amult     (quantized residual, output-scale units)
+//   t  = silu(t * out_scale) / out_scale
+struct PostOps {
+  const uint8_t* accum;  // bytes laid out like the output, or null
+  int32_t accum_signed, accum_zp;
+  float amult;           // accum_scale / out_scale
+  int32_t silu;
+  float out_scale;
+  __host__ __device__ bool any() const { return accum != nullptr || silu != 0; }
 };
 
 struct GemmArgs {
@@ -66,6 +80,7 @@ struct GemmArgs {
   void* y;               // bytes [M, ldy] or int32 [M, ldy]
   int64_t ldy;
   int32_t n_off;         // conv groups: channel offset of this group in y/params
+  PostOps post;          // all zero for quantized::linear
 };
 
 __device__ __forceinline__ v4i ld16(const void* p) { return *reinterpret_cast<const v4i*>(p); }
@@ -209,6 +224,53 @@ __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, v4f 
   return packed;
 }
 
+// Up to four residual bytes of one output row, starting at byte offset `off`
+// of the residual tensor; `nvalid` of them exist.
+__device__ __forceinline__ uint32_t load_accum4(const PostOps& p, int64_t off, int nvalid) {
+  const uint8_t* src = p.accum + off;
+  if (nvalid >= 4 && (reinterpret_cast<uintptr_t>(src) & 3) == 0)
+    return *reinterpret_cast<const uint32_t*>(src);
+  uint32_t w = 0;
+  for (int j = 0; j < 4; ++j)
+    if (j < nvalid) w |= static_cast<uint32_t>(src[j]) << (8 * j);
+  return w;
+}
+
+// requant4 with the post operations (see PostOps) before the rounding.
+template <int MODE>
+__device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv, v4f mult,
+                                                  const PostOps& p, uint32_t accw, float zp_f,
+                                                  float lo_f, float hi_f) {
+  uint32_t packed = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float v = static_cast<float>(raw[j]);
+    v = v + bdiv[j];
+    float t = v * mult[j];
+    if (p.accum != nullptr) {
+      const uint32_t b = (accw >> (8 * j)) & 0xffu;
+      const int qa = p.accum_signed ? static_cast<int>(static_cast<int8_t>(b)) : static_cast<int>(b);
+      const float a = static_cast<float>(qa - p.accum_zp) * p.amult;
+      t = t + a;
+    }
+    if (p.silu) {
+      const float r = t * p.out_scale;
+      const float e = expf(-r);
+      const float d = 1.0f + e;
+      const float sl = r / d;
+      t = sl / p.out_scale;
+    }
+    float r = __builtin_rintf(t) + zp_f;
+    r = __builtin_amdgcn_fmed3f(r, lo_f, hi_f);
+    if constexpr (MODE == kOutU8) {
+      packed = __builtin_amdgcn_cvt_pk_u8_f32(r, j, packed);
+    } else {
+      packed |= (static_cast<uint32_t>(static_cast<int>(r)) & 0xffu) << (8 * j);
+    }
+  }
+  return packed;
+}
+
 // BM x BN output tile per block (BM activation rows, BN weight rows),
 // WM x WN waves, each wave (BM/WM) x (BN/WN).  PD = prefetch distance in
 // stages: the global loads of stage t+PD are issued while stage t is being
@@ -216,6 +278,7 @@ __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, v4f 
 template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4>
 __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int NT = WM * WN * kWave;
+  constexpr bool kHasPost = XSRC::kPostOps;  // residual / activation epilogue compiled in
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int NW = BN * kChunks / NT;  // 16-byte weight chunks per thread per stage
@@ -466,8 +529,18 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
           int raw[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * g + j];
-          *reinterpret_cast<uint32_t*>(&smem[(wm0 + tm * 32 + li) * kOutPitch + nl]) =
-              requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+          uint32_t q4;
+          if (kHasPost && a.post.any()) {
+            const int64_t m = m0 + wm0 + tm * 32 + li, n = n0 + nl;
+            const int64_t left = a.N - n;
+            const int nvalid = (m < a.M && left > 0) ? (left < 4 ? static_cast<int>(left) : 4) : 0;
+            const uint32_t accw =
+                (a.post.accum != nullptr && nvalid > 0) ? load_accum4(a.post, m * a.ldy + a.n_off + n, nvalid) : 0u;
+            q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
+          } else {
+            q4 = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+          }
+          *reinterpret_cast<uint32_t*>(&smem[(wm0 + tm * 32 + li) * kOutPitch + nl]) = q4;
         }
       }
     __syncthreads();
