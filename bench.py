@@ -342,6 +342,47 @@ def main():
             "method": f"{reps} launches over {csets} rotating inputs replayed back to back in one HIP graph",
             "algorithmic_bytes_per_launch": cbytes, "ops_per_launch": cops}
 
+        # ---------------------------------------- C5 with a fused residual + ReLU
+        log("[bench] config 5 + residual: conv2d_add_relu, same shapes, quantized residual of the output's shape")
+        accs = []
+        for _ in range(csets):
+            af_ = torch.randn(32, 64, 56, 56, device=dev).contiguous(memory_format=torch.channels_last)
+            accs.append(torch.quantize_per_tensor(af_, 0.03, 128, torch.quint8))
+            del af_
+        fcount = [0]
+
+        def conv_add_relu():
+            fcount[0] += 1
+            i = fcount[0] % csets
+            return torch.ops.quantized.conv2d_add_relu(xcqs[i], accs[i], pc, 0.05, 0)
+
+        for _ in range(5):
+            conv_add_relu()
+        fgraph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            conv_add_relu()
+            side.synchronize()
+            with torch.cuda.graph(fgraph, stream=side):
+                for _ in range(reps):
+                    conv_add_relu()
+        torch.cuda.synchronize()
+        for _ in range(3):
+            fgraph.replay()
+        ts = events_ms(fgraph.replay, 10)
+        favg = sum(ts) / len(ts) / reps
+        fbytes = cbytes + 32 * 56 * 56 * 64
+        log(f"[bench] conv2d_add_relu C5: {favg*1e3:.1f} us/launch in a replayed graph, "
+            f"{cops/(favg*1e-3)/1e12:.0f} TOP/s, {fbytes/(favg*1e-3)/1e9:.0f} GB/s")
+        secondary["conv2d_add_relu_c5"] = {
+            "avg_launch_us": round(favg * 1e3, 2), "value": round(cops / (favg * 1e-3) / 1e12, 1), "unit": "TOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(cops / (favg * 1e-3) / 1e12, 1),
+                         "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                         "frac": round(cops / (favg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "traffic": None},
+            "hbm_frac": round(fbytes / (favg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "method": f"{reps} launches over {csets} rotating inputs and residuals replayed in one HIP graph",
+            "algorithmic_bytes_per_launch": fbytes, "ops_per_launch": cops}
+        del accs, xcqs
+
     # ------------------------------------------------------------ CPU baseline
     cpu_baseline = None
     if not args.skip_cpu:

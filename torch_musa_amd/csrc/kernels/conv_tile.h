@@ -281,6 +281,22 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = init;
     }
 
+    // The residual bytes this lane will add (4 consecutive channels per word)
+    // are requested now; they arrive while the k loop runs.
+    uint32_t accw[TM][8];
+    if (a.post.accum != nullptr) {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int nl = (u >> 2) * 32 + 8 * (u & 3) + 4 * half;
+          const int left = a.OCg - (n0 + nl);
+          const int nvalid = (opix[tm] >= 0 && left > 0) ? (left < 4 ? left : 4) : 0;
+          accw[tm][u] = nvalid > 0 ? load_accum4(a.post, static_cast<int64_t>(opix[tm]) * a.OC + ch0 + nl, nvalid)
+                                   : 0u;
+        }
+    }
+
     // Fragments of successive k-steps; the two halves of the wave take the two
     // chunks of the step.  The tap offset of a step is fetched one step ahead.
     // Reading runs two steps past the end (results unused; the addresses stay
@@ -358,12 +374,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
             for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * gq + j];
             uint32_t q4;
             if (a.post.any()) {
-              const int left = a.OCg - (n0 + nl);
-              const int nvalid = (opix[tm] >= 0 && left > 0) ? (left < 4 ? left : 4) : 0;
-              const uint32_t accw = (a.post.accum != nullptr && nvalid > 0)
-                                        ? load_accum4(a.post, static_cast<int64_t>(opix[tm]) * a.OC + ch0 + nl, nvalid)
-                                        : 0u;
-              q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
+              q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw[tm][tn * 4 + gq], a.zp_f, a.lo_f, a.hi_f);
             } else {
               q4 = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
             }
