@@ -242,7 +242,11 @@ def main():
         hbm("minmax_c2", lambda: cabi.minmax(xf, mm_out, ws), 4 * n, "minmax_c2")
         hbm("quantize_per_tensor_dynamic_c2", lambda: torch.quantize_per_tensor_dynamic(xf, torch.quint8, False),
             9 * n, None)
-        del xf, q
+        # elementwise glue on quantized tensors of the same element count
+        q2 = torch.quantize_per_tensor(xf * 0.5, scale, zp, torch.quint8)
+        hbm("quantized_add_2p28", lambda: torch.ops.quantized.add(q, q2, scale * 1.5, zp), 3 * n, None)
+        hbm("quantized_relu_2p28", lambda: torch.relu(q), 2 * n, None)
+        del xf, q, q2
 
         # -------------------------------------------------------------- C4
         log("[bench] config 4: decode-shaped linear, K=N=4096, cold weights (40 weight sets, HIP graph)")

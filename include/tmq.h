@@ -268,6 +268,23 @@ int tmq_conv2d_fused(const tmq_conv2d_desc* desc, const tmq_conv2d_post* post,
                      tmq_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Elementwise kernels on per-tensor quantized tensors (n codes, dense).
+ * tmq_qadd replaces QAdd<kReluFused> / QuantizedAddKernel
+ * (torch_musa/csrc/aten/quantized/musa/BinaryOps.mu:24-99,154-207) with the
+ * arithmetic of PyTorch's CPU quantized::add / add_relu:
+ *   a = fma(float(qa), a_scale, -a_zp*a_scale), b likewise, c = a + b,
+ *   relu: c = max(c, 0), q = clamp(rne(c * (1/out_scale)) + out_zp).
+ * tmq_qrelu replaces ActQuantized<ActMode::RELU>
+ * (torch_musa/csrc/aten/quantized/musa/Activation.mu:165-186,215-220):
+ *   y = max(x, zero_point), scale and zero point unchanged.
+ * ------------------------------------------------------------------------- */
+int tmq_qadd(const void* a, const void* b, void* out, int64_t n, float a_scale,
+             int32_t a_zero_point, float b_scale, int32_t b_zero_point, float out_scale,
+             int32_t out_zero_point, int q_signed, int relu, tmq_stream_t stream);
+int tmq_qrelu(const void* x, void* y, int64_t n, int32_t zero_point, int q_signed,
+              tmq_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Measurement probe (no counterpart in the reference; used by bench.py only).
  * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four
  * waves and reports the sustained rate in TOP/s and the shader clock in GHz.

@@ -300,3 +300,21 @@ def conv2d_fused(x_nhwc, x_scale, x_zp, w_ohwi, w_scales, bias, stride, padding,
                            C.c_double(out_scale), C.c_int64(out_zp), C.c_int(out_signed), _p(y),
                            C.c_int(nthreads))
     return y
+
+
+def qadd(qa, a_scale, a_zp, qb, b_scale, b_zp, out_scale, out_zp, relu=False):
+    """quantized::add / add_relu of two per-tensor quantized tensors (bytes)."""
+    qa, qb = _as_bytes(qa), _as_bytes(qb)
+    assert qa.shape == qb.shape and qa.dtype == qb.dtype
+    out = np.empty(qa.shape, dtype=qa.dtype)
+    lib().orc_qadd(_p(qa), _p(qb), C.c_int64(qa.size), C.c_double(a_scale), C.c_int64(a_zp),
+                   C.c_double(b_scale), C.c_int64(b_zp), C.c_double(out_scale), C.c_int64(out_zp),
+                   C.c_int(qa.dtype == np.int8), C.c_int(relu), _p(out))
+    return out
+
+
+def qrelu(q, zp):
+    q = _as_bytes(q)
+    y = np.empty(q.shape, dtype=q.dtype)
+    lib().orc_qrelu(_p(q), C.c_int64(q.size), C.c_int64(zp), C.c_int(q.dtype == np.int8), _p(y))
+    return y

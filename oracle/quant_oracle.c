@@ -480,3 +480,46 @@ ORC_API void orc_conv2d_fused(const uint8_t* x, int x_signed, const int8_t* w, i
   }
   free(acc);
 }
+
+/* ------------------------------------------------------------------------- */
+/* quantized::add / add_relu on two per-tensor quantized tensors of one shape
+ * (reference musa/BinaryOps.mu:154-207; the reference evaluates
+ * (qa + qb*b_s/a_s)*a_s/out_s in double and clamps the relu variant at 0, not
+ * at the zero point).  Restated from PyTorch's CPU kernel, vector body of
+ * qadd_kernel (ATen/native/quantized/cpu/kernels/QuantizedOpKernels.cpp):
+ *   a = fmaf((float)qa, a_scale, fl(-a_zp * a_scale))
+ *   b = fmaf((float)qb, b_scale, fl(-b_zp * b_scale))
+ *   c = a + b; relu: c = max(c, 0)
+ *   q = clamp(rne(c * fl(1/out_scale)) + out_zp, qmin, qmax)
+ * (the scalar tail of the CPU kernel dequantizes with (q - zp) * scale instead
+ * of the fused form: about 1e-5 of values differ by one between the two). */
+ORC_API void orc_qadd(const uint8_t* qa, const uint8_t* qb, int64_t n, double a_scale,
+                      int64_t a_zp, double b_scale, int64_t b_zp, double out_scale,
+                      int64_t out_zp, int is_signed, int relu, uint8_t* out) {
+  int64_t qmin, qmax;
+  qrange(is_signed, &qmin, &qmax);
+  const float sa = (float)a_scale, sb = (float)b_scale;
+  volatile float pa = -(float)a_zp * sa;
+  volatile float pb = -(float)b_zp * sb;
+  volatile float inv = 1.0f / (float)out_scale;
+  for (int64_t i = 0; i < n; ++i) {
+    const int32_t va = is_signed ? (int32_t)(int8_t)qa[i] : (int32_t)qa[i];
+    const int32_t vb = is_signed ? (int32_t)(int8_t)qb[i] : (int32_t)qb[i];
+    volatile float a = fmaf((float)va, sa, pa);
+    volatile float b = fmaf((float)vb, sb, pb);
+    volatile float c = a + b;
+    if (relu && c < 0.0f) c = 0.0f;
+    volatile float t = c * inv;
+    int64_t q = (int64_t)nearbyintf(t) + out_zp;
+    out[i] = (uint8_t)clamp_i64(q, qmin, qmax);
+  }
+}
+
+/* relu of a per-tensor quantized tensor: y = max(x, zero_point) (reference
+ * musa/Activation.mu:165-186; PyTorch CPU qrelu does the same clamp). */
+ORC_API void orc_qrelu(const uint8_t* x, int64_t n, int64_t zp, int is_signed, uint8_t* y) {
+  for (int64_t i = 0; i < n; ++i) {
+    const int32_t v = is_signed ? (int32_t)(int8_t)x[i] : (int32_t)x[i];
+    y[i] = (uint8_t)(v > zp ? v : (int32_t)zp);
+  }
+}

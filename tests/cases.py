@@ -304,3 +304,28 @@ def conv_fused_cases():
                         acc_scale=acc_scale, acc_zp=acc_zp, activation=act, out_scale=out_scale,
                         out_zp=0 if signed else 128, signed=signed))
     return out
+
+
+# --------------------------------------------------------------------------
+# quantized::add / add_relu and relu of a quantized tensor
+# --------------------------------------------------------------------------
+def qadd_cases():
+    spec = [
+        # name, shape, signed, relu, (a_scale, a_zp), (b_scale, b_zp), (out_scale, out_zp)
+        ("ref_u8", (2, 16, 8, 8), False, False, (0.05, 128), (0.031, 120), (0.07, 128)),
+        ("ref_u8_relu", (2, 16, 8, 8), False, True, (0.05, 128), (0.031, 120), (0.07, 128)),
+        ("s8", (3, 5, 7), True, False, (0.02, 0), (0.045, -3), (0.05, 4)),
+        ("s8_relu", (3, 5, 7), True, True, (0.02, 0), (0.045, -3), (0.05, -20)),
+        ("saturating_u8", (4099,), False, False, (0.1, 10), (0.2, 250), (0.05, 100)),
+        ("odd_sizes_u8_relu", (1, 3, 5, 11), False, True, (0.013, 77), (0.4, 3), (0.11, 9)),
+        ("big_u8", (64, 1031), False, False, (1 / 3, 128), (0.0123456789, 127), (0.21, 101)),
+    ]
+    out = []
+    for i, (name, shape, signed, relu, (sa, za), (sb, zb), (so, zo)) in enumerate(spec):
+        rng = np.random.default_rng(1300 + i)
+        lo, hi = (-128, 128) if signed else (0, 256)
+        dt = np.int8 if signed else np.uint8
+        out.append(dict(name=name, qa=rng.integers(lo, hi, shape).astype(dt),
+                        qb=rng.integers(lo, hi, shape).astype(dt), a_scale=sa, a_zp=za, b_scale=sb,
+                        b_zp=zb, out_scale=so, out_zp=zo, signed=signed, relu=relu))
+    return out

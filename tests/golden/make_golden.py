@@ -170,6 +170,18 @@ def main():
         g[k + "/wq_crc"] = np.uint32(cases.crc(c["wq"]))
         g[k + "/y"] = y.int_repr().permute(0, 2, 3, 1).contiguous().numpy()
 
+    # ---- quantized::add / add_relu, relu ------------------------------------
+    for c in cases.qadd_cases():
+        qa = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["qa"]), c["a_scale"], c["a_zp"])
+        qb = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["qb"]), c["b_scale"], c["b_zp"])
+        op = torch.ops.quantized.add_relu if c["relu"] else torch.ops.quantized.add
+        y = op(qa, qb, c["out_scale"], c["out_zp"])
+        k = "qadd/" + c["name"]
+        g[k + "/qa_crc"] = np.uint32(cases.crc(c["qa"]))
+        g[k + "/qb_crc"] = np.uint32(cases.crc(c["qb"]))
+        g[k + "/y"] = y.int_repr().numpy()
+        g[k + "/relu_a"] = torch.relu(qa).int_repr().numpy()
+
     # ---- quantized::conv2d -------------------------------------------------
     for c in cases.conv_cases():
         x_nchw = torch.from_numpy(c["xq"]).permute(0, 3, 1, 2)  # channels-last view

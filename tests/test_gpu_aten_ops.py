@@ -311,3 +311,33 @@ def test_conv2d_add_rejects_wrong_accum():
         torch.ops.quantized.conv2d_add(x, bad, packed, 0.1, 0)
     with pytest.raises(RuntimeError):
         torch.ops.quantized.conv2d_add(x, torch.zeros(1, 8, 5, 5).cuda(), packed, 0.1, 0)
+
+
+# ---------------------------------------------------------------------------
+# quantized::add / add_relu, relu
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("c", cases.qadd_cases(), ids=lambda c: c["name"])
+def test_quantized_add_ops(golden, c):
+    say("aten qadd", c["name"])
+    qa = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["qa"]).cuda(), c["a_scale"], c["a_zp"])
+    qb = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["qb"]).cuda(), c["b_scale"], c["b_zp"])
+    op = torch.ops.quantized.add_relu if c["relu"] else torch.ops.quantized.add
+    y = op(qa, qb, c["out_scale"], c["out_zp"])
+    assert y.q_scale() == c["out_scale"] and y.q_zero_point() == c["out_zp"] and y.dtype == qa.dtype
+    d = np.abs(y.int_repr().cpu().numpy().astype(np.int32) - golden["qadd/" + c["name"] + "/y"].astype(np.int32))
+    assert d.max() <= 1 and np.count_nonzero(d) <= max(1, d.size // 20000)
+    r = torch.relu(qa)
+    assert r.q_scale() == qa.q_scale() and r.q_zero_point() == qa.q_zero_point()
+    np.testing.assert_array_equal(r.int_repr().cpu().numpy(), golden["qadd/" + c["name"] + "/relu_a"])
+
+
+def test_quantized_add_keeps_channels_last_and_checks_shapes():
+    x = torch.randn(2, 8, 5, 5).contiguous(memory_format=torch.channels_last)
+    qa = torch.quantize_per_tensor(x.cuda(), 0.05, 128, torch.quint8)
+    qb = torch.quantize_per_tensor((x * 0.5).cuda(), 0.04, 120, torch.quint8)
+    y = torch.ops.quantized.add(qa, qb, 0.08, 128)
+    assert y.is_contiguous(memory_format=torch.channels_last)
+    want = torch.ops.quantized.add(qa.cpu(), qb.cpu(), 0.08, 128)
+    assert (y.int_repr().cpu().int() - want.int_repr().int()).abs().max() <= 1
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.add(qa, qb[:, :4], 0.08, 128)

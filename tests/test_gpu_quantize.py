@@ -184,3 +184,45 @@ def test_full_size_properties(cabi):
                                       oracle.quantize_per_tensor(xs, s, z, False))
         np.testing.assert_array_equal(host(r[start:start + 2 ** 20]),
                                       oracle.dequantize_per_tensor(host(q[start:start + 2 ** 20]), s, z))
+
+
+# ---------------------------------------------------------------------------
+# quantized::add / add_relu, relu
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("c", cases.qadd_cases(), ids=lambda c: c["name"])
+def test_qadd_qrelu(cabi, golden, c):
+    say("qadd", c["name"])
+    k = "qadd/" + c["name"]
+    qa, qb = dev(c["qa"]), dev(c["qb"])
+    y = host(cabi.qadd(qa, c["a_scale"], c["a_zp"], qb, c["b_scale"], c["b_zp"], c["out_scale"],
+                       c["out_zp"], relu=c["relu"]))
+    want = oracle.qadd(c["qa"], c["a_scale"], c["a_zp"], c["qb"], c["b_scale"], c["b_zp"], c["out_scale"],
+                       c["out_zp"], relu=c["relu"])
+    np.testing.assert_array_equal(y, want)
+    d = np.abs(y.astype(np.int32) - golden[k + "/y"].astype(np.int32))
+    assert d.max() <= 1 and np.count_nonzero(d) <= max(1, d.size // 20000)
+    np.testing.assert_array_equal(host(cabi.qrelu(qa, c["a_zp"])), golden[k + "/relu_a"])
+
+
+def test_qadd_unaligned_and_large(cabi):
+    """Scalar path (operands off a 16-byte boundary) and a 64 Mi element add."""
+    say("qadd unaligned")
+    rng = np.random.default_rng(77)
+    a = rng.integers(0, 256, 100003, dtype=np.uint8)
+    b = rng.integers(0, 256, 100003, dtype=np.uint8)
+    da, db = dev(a), dev(b)
+    y = torch.empty(100003, dtype=torch.uint8, device="cuda")
+    got = host(cabi.qadd(da[1:], 0.05, 128, db[1:], 0.03, 100, 0.06, 120, relu=True, out=y[1:]))
+    np.testing.assert_array_equal(got, oracle.qadd(a[1:], 0.05, 128, b[1:], 0.03, 100, 0.06, 120, relu=True))
+    say("qadd 2**26")
+    n = 2 ** 26
+    g = torch.Generator(device="cuda").manual_seed(3)
+    ta = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    tb = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    ty = cabi.qadd(ta, 0.05, 128, tb, 0.03, 100, 0.06, 120)
+    for lo in (0, n // 2 - 5000, n - 10000):
+        sl = slice(lo, lo + 10000)
+        np.testing.assert_array_equal(host(ty[sl]), oracle.qadd(host(ta[sl]), 0.05, 128, host(tb[sl]), 0.03, 100, 0.06, 120))
+    # commutes when the operands' quantization parameters are swapped too
+    tz = cabi.qadd(tb, 0.03, 100, ta, 0.05, 128, 0.06, 120)
+    assert torch.equal(ty, tz)

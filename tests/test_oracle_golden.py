@@ -135,3 +135,17 @@ def test_conv2d_fused_vs_float_pipeline(golden, c):
     d = np.abs(y.astype(np.int32) - want.astype(np.int32))
     assert d.max() <= 1
     assert np.count_nonzero(d) <= 0.002 * d.size, f"{np.count_nonzero(d)} of {d.size} differ"
+
+
+@pytest.mark.parametrize("c", cases.qadd_cases(), ids=lambda c: c["name"])
+def test_qadd_and_qrelu(golden, c):
+    k = "qadd/" + c["name"]
+    _check_crc(golden, k + "/qa_crc", c["qa"])
+    _check_crc(golden, k + "/qb_crc", c["qb"])
+    y = oracle.qadd(c["qa"], c["a_scale"], c["a_zp"], c["qb"], c["b_scale"], c["b_zp"], c["out_scale"],
+                    c["out_zp"], relu=c["relu"])
+    # the CPU kernel's scalar tail dequantizes without the fused multiply-add:
+    # a handful of values per 100 000 may differ by one
+    d = np.abs(y.astype(np.int32) - golden[k + "/y"].astype(np.int32))
+    assert d.max() <= 1 and np.count_nonzero(d) <= max(1, d.size // 20000), np.count_nonzero(d)
+    np.testing.assert_array_equal(oracle.qrelu(c["qa"], c["a_zp"]), golden[k + "/relu_a"])

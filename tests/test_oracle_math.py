@@ -243,3 +243,37 @@ def test_fused_silu_of_a_known_value():
     want = np.clip(np.rint(r / (1 + np.exp(-r)) / s) + 30, 0, 255)
     d = np.abs(y.astype(int) - want.astype(int))
     assert d.max() <= 1 and np.count_nonzero(d) <= 2  # float32 vs float64 at exact ties only
+
+
+# ---------------------------------------------------------------------------
+# quantized::add: cases with an exact answer
+# ---------------------------------------------------------------------------
+def test_qadd_equal_power_of_two_scales_is_integer_addition():
+    rng = np.random.default_rng(8)
+    qa = rng.integers(0, 256, 5000, dtype=np.uint8)
+    qb = rng.integers(0, 256, 5000, dtype=np.uint8)
+    y = oracle.qadd(qa, 0.25, 100, qb, 0.25, 90, 0.25, 60)
+    np.testing.assert_array_equal(y, np.clip(qa.astype(int) - 100 + qb.astype(int) - 90 + 60, 0, 255))
+    yr = oracle.qadd(qa, 0.25, 100, qb, 0.25, 90, 0.25, 60, relu=True)
+    np.testing.assert_array_equal(yr, np.clip(np.maximum(qa.astype(int) - 100 + qb.astype(int) - 90, 0) + 60, 0, 255))
+    # output scale twice as coarse: halves, ties to even
+    y2 = oracle.qadd(qa, 0.25, 100, qb, 0.25, 90, 0.5, 60)
+    np.testing.assert_array_equal(y2, np.clip(np.rint((qa.astype(int) - 100 + qb.astype(int) - 90) / 2.0) + 60, 0, 255))
+
+
+def test_qadd_close_to_real_arithmetic():
+    rng = np.random.default_rng(9)
+    qa = rng.integers(-128, 128, 20000).astype(np.int8)
+    qb = rng.integers(-128, 128, 20000).astype(np.int8)
+    y = oracle.qadd(qa, 0.037, -5, qb, 0.11, 17, 0.09, 3)
+    real = (qa.astype(np.float64) + 5) * np.float64(np.float32(0.037)) + (qb.astype(np.float64) - 17) * np.float64(np.float32(0.11))
+    want = np.clip(np.rint(real / np.float64(np.float32(0.09))) + 3, -128, 127)
+    d = np.abs(y.astype(int) - want.astype(int))
+    assert d.max() <= 1 and np.count_nonzero(d) < 100  # fp32 steps: only values next to a rounding boundary move
+
+
+def test_qrelu_is_a_clamp_at_the_zero_point():
+    q = np.arange(256, dtype=np.uint8)
+    np.testing.assert_array_equal(oracle.qrelu(q, 77), np.maximum(q, 77))
+    s = np.arange(-128, 128).astype(np.int8)
+    np.testing.assert_array_equal(oracle.qrelu(s, -5), np.maximum(s, -5))

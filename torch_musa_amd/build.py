@@ -26,7 +26,7 @@ LIB_ATEN = os.path.join(PKG, "libtmq_aten.so")
 ARCH = "gfx950"
 
 KERNEL_SOURCES = ["kernels/quantize.hip", "kernels/linear.hip", "kernels/conv2d.hip",
-                  "kernels/probe.hip"]
+                  "kernels/elementwise.hip", "kernels/probe.hip"]
 ATEN_SOURCES = ["aten/register.cpp"]
 
 # -ffp-contract=off: the requantisation epilogue and the quantizer must round

@@ -27,6 +27,7 @@ DECLARED_SYMBOLS = [
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
+    "tmq_qadd", "tmq_qrelu",
     "tmq_probe_mfma_i8",
 ]
 
@@ -122,6 +123,9 @@ def lib() -> C.CDLL:
         l.tmq_conv2d.argtypes = [C.POINTER(Conv2dDesc), v]
         l.tmq_conv2d_acc32.argtypes = [C.POINTER(Conv2dDesc), v, v]
         l.tmq_conv2d_fused.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(Conv2dPost), v]
+        l.tmq_qadd.argtypes = [v, v, v, C.c_int64, C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_float,
+                               C.c_int32, C.c_int, C.c_int, v]
+        l.tmq_qrelu.argtypes = [v, v, C.c_int64, C.c_int32, C.c_int, v]
         l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, v, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]
         _lib = l
@@ -441,6 +445,26 @@ def conv2d_acc32(x_nhwc, pw: PackedConv2d, g: Conv2dGeom, x_zp):
     d = _conv_desc(x_nhwc, pw, g, 1.0, x_zp, None, None, 1.0, 0, False, False, None)
     check(lib().tmq_conv2d_acc32(C.byref(d), acc.data_ptr(), stream_ptr()), "tmq_conv2d_acc32")
     return acc
+
+
+# ---------------------------------------------------------------------------
+# elementwise
+# ---------------------------------------------------------------------------
+def qadd(qa, a_scale, a_zp, qb, b_scale, b_zp, out_scale, out_zp, relu=False, out=None):
+    assert qa.shape == qb.shape and qa.dtype == qb.dtype and qa.is_contiguous() and qb.is_contiguous()
+    y = out if out is not None else torch.empty_like(qa)
+    check(lib().tmq_qadd(qa.data_ptr(), qb.data_ptr(), y.data_ptr(), qa.numel(), a_scale, a_zp, b_scale,
+                         b_zp, out_scale, out_zp, int(qa.dtype == torch.int8), int(relu), stream_ptr()),
+          "tmq_qadd")
+    return y
+
+
+def qrelu(q, zp, out=None):
+    assert q.is_contiguous()
+    y = out if out is not None else torch.empty_like(q)
+    check(lib().tmq_qrelu(q.data_ptr(), y.data_ptr(), q.numel(), zp, int(q.dtype == torch.int8),
+                          stream_ptr()), "tmq_qrelu")
+    return y
 
 
 # ---------------------------------------------------------------------------

@@ -597,6 +597,50 @@ c10::intrusive_ptr<ConvPackedParamsBase<2>> qconv2d_prepack_run(at::Tensor weigh
                                       std::move(padding), std::move(dilation), groups);
 }
 
+// ---------------------------------------------------------------------------
+// quantized::add / add_relu (musa/BinaryOps.mu:154-207) and relu of a quantized
+// tensor (musa/Activation.mu:165-186,215-220)
+// ---------------------------------------------------------------------------
+at::Tensor qadd_impl(const at::Tensor& qa, const at::Tensor& qb, double output_scale, int64_t output_zero_point,
+                     bool relu) {
+  TORCH_CHECK(qa.qscheme() == c10::kPerTensorAffine, "Only per tensor quantization is supported in Add.");
+  TORCH_CHECK(qa.qscheme() == qb.qscheme(), "Both inputs to Add must have the same quantization scheme.");
+  TORCH_CHECK(qa.scalar_type() == qb.scalar_type(), "Add operands should have same data type.");
+  const bool sgn = is_signed_qtype(qa.scalar_type(), "quantized::add");
+  TORCH_CHECK(qa.sizes() == qb.sizes(),
+              "quantized::add currently expects both input tensors to be the same shape");
+  TORCH_CHECK(qa.device() == qb.device(), "quantized::add: operands on different devices");
+  TORCH_CHECK(output_scale > 0, "quantized::add: output scale must be positive");
+  const c10::OptionalDeviceGuard guard(at::device_of(qa));
+  const auto fmt = qa.suggest_memory_format();
+  const at::Tensor a = qa.contiguous(fmt), b = qb.contiguous(fmt);
+  at::Tensor y = at::_empty_affine_quantized(qa.sizes(), qa.options(), output_scale, output_zero_point, fmt);
+  if (y.numel() == 0) return y;
+  check_status(tmq_qadd(a.data_ptr(), b.data_ptr(), y.data_ptr(), y.numel(), static_cast<float>(a.q_scale()),
+                        static_cast<int32_t>(a.q_zero_point()), static_cast<float>(b.q_scale()),
+                        static_cast<int32_t>(b.q_zero_point()), static_cast<float>(output_scale),
+                        static_cast<int32_t>(output_zero_point), sgn, relu, current_stream(a)),
+               "tmq_qadd");
+  return y;
+}
+at::Tensor qadd_run(at::Tensor qa, at::Tensor qb, double s, int64_t z) { return qadd_impl(qa, qb, s, z, false); }
+at::Tensor qadd_relu_run(at::Tensor qa, at::Tensor qb, double s, int64_t z) { return qadd_impl(qa, qb, s, z, true); }
+
+at::Tensor qrelu_run(const at::Tensor& self) {
+  TORCH_CHECK(self.qscheme() == c10::kPerTensorAffine || self.qscheme() == c10::kPerTensorSymmetric,
+              "we currently only support per-tensor quantized relu, but got ", toString(self.qscheme()));
+  const bool sgn = is_signed_qtype(self.scalar_type(), "relu");
+  const c10::OptionalDeviceGuard guard(at::device_of(self));
+  const auto fmt = self.suggest_memory_format();
+  const at::Tensor x = self.contiguous(fmt);
+  at::Tensor y = at::_empty_affine_quantized(self.sizes(), self.options(), self.q_scale(), self.q_zero_point(), fmt);
+  if (y.numel() == 0) return y;
+  check_status(tmq_qrelu(x.data_ptr(), y.data_ptr(), y.numel(), static_cast<int32_t>(self.q_zero_point()), sgn,
+                         current_stream(x)),
+               "tmq_qrelu");
+  return y;
+}
+
 }  // namespace
 
 // The two SiLU schemas are not part of upstream PyTorch; the reference adds them
@@ -618,6 +662,8 @@ TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add_relu"), TORCH_FN(qconv2d_add_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_silu.new"), TORCH_FN(qconv2d_silu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add_silu"), TORCH_FN(qconv2d_add_silu_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::add"), TORCH_FN(qadd_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::add_relu"), TORCH_FN(qadd_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear"), TORCH_FN(qlinear_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear_relu"), TORCH_FN(qlinear_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear_prepack"), TORCH_FN(qlinear_prepack_run));
@@ -644,6 +690,10 @@ struct MuteOn {
 
 TORCH_LIBRARY_IMPL(aten, CUDA, m) {
   m.impl("quantize_per_tensor_dynamic", TORCH_FN(quantize_per_tensor_dynamic));
+}
+// one kernel instead of PyTorch-ROCm's int_repr / compare / where / re-wrap chain
+TORCH_LIBRARY_IMPL(aten, QuantizedCUDA, m) {
+  m.impl("relu", TORCH_FN(qrelu_run));
 }
 
 namespace {
