@@ -362,24 +362,34 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       uint8_t* y = static_cast<uint8_t*>(a.y);
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
+        // kind 0: residual / SiLU; 1: plain; 2: plain, unsigned output without
+        // ReLU, where the saturating pack conversion is the clamp
+        auto requant_rows = [&](auto kind_tag) {
+          constexpr int KIND = decltype(kind_tag)::value;
 #pragma unroll
-        for (int tn = 0; tn < 2; ++tn)
+          for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
-          for (int gq = 0; gq < 4; ++gq) {
-            const int nl = tn * 32 + 8 * gq + 4 * half;
-            const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[nl]);
-            const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[nl]);
-            int raw[4];
+            for (int gq = 0; gq < 4; ++gq) {
+              const int nl = tn * 32 + 8 * gq + 4 * half;
+              const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[nl]);
+              const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[nl]);
+              int raw[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * gq + j];
-            uint32_t q4;
-            if (a.post.any()) {
-              q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw[tm][tn * 4 + gq], a.zp_f, a.lo_f, a.hi_f);
-            } else {
-              q4 = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+              for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * gq + j];
+              uint32_t q4;
+              if constexpr (KIND == 0)
+                q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw[tm][tn * 4 + gq], a.zp_f, a.lo_f, a.hi_f);
+              else
+                q4 = requant4<MODE, KIND == 1>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+              *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) = q4;
             }
-            *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) = q4;
-          }
+        };
+        if (a.post.any())
+          requant_rows(std::integral_constant<int, 0>{});
+        else if (MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f)
+          requant_rows(std::integral_constant<int, 2>{});
+        else
+          requant_rows(std::integral_constant<int, 1>{});
         wave_sync_lds();
         // whole pixels leave as 16 bytes per lane: 4 lanes per pixel, 16 pixels per pass
 #pragma unroll

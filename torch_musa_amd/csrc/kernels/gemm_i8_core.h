@@ -25,6 +25,8 @@
 // Pipeline: see the comment at the software pipeline inside gemm_i8_kernel.
 #pragma once
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace tmq {
@@ -204,7 +206,9 @@ struct KCursor<XConv> {
 __device__ __forceinline__ int x_swizzle(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
 
 // One requantised byte group: four consecutive channels of one output row.
-template <int MODE>
+// CLAMP = false (unsigned output, bounds 0 and 255 only): the packing
+// conversion v_cvt_pk_u8_f32 already saturates to [0, 255], no separate clamp.
+template <int MODE, bool CLAMP = true>
 __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, v4f mult, float zp_f,
                                              float lo_f, float hi_f) {
   uint32_t packed = 0;
@@ -214,7 +218,7 @@ __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, v4f 
     v = v + bdiv[j];
     const float ab = v * mult[j];
     float r = __builtin_rintf(ab) + zp_f;
-    r = __builtin_amdgcn_fmed3f(r, lo_f, hi_f);
+    if constexpr (CLAMP || MODE != kOutU8) r = __builtin_amdgcn_fmed3f(r, lo_f, hi_f);
     if constexpr (MODE == kOutU8) {
       packed = __builtin_amdgcn_cvt_pk_u8_f32(r, j, packed);
     } else {
@@ -517,6 +521,8 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     // Requantise in registers, transpose through LDS, then write whole rows:
     // 16 bytes per lane, consecutive lanes on consecutive addresses.
     __syncthreads();  // every wave is done with the operand stages
+    auto requant_tile = [&](auto clamp_tag) {
+      constexpr bool CL = decltype(clamp_tag)::value;
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -538,11 +544,17 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
                 (a.post.accum != nullptr && nvalid > 0) ? load_accum4(a.post, m * a.ldy + a.n_off + n, nvalid) : 0u;
             q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
           } else {
-            q4 = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+            q4 = requant4<MODE, CL>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
           }
           *reinterpret_cast<uint32_t*>(&smem[(wm0 + tm * 32 + li) * kOutPitch + nl]) = q4;
         }
       }
+    };
+    // unsigned output without ReLU: the saturating conversion is the clamp
+    if (MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f)
+      requant_tile(std::false_type{});
+    else
+      requant_tile(std::true_type{});
     __syncthreads();
     uint8_t* y = static_cast<uint8_t*>(a.y) + a.n_off;
     const bool vec_ok = ((a.ldy & 15) == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
