@@ -103,6 +103,24 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
   const uint8_t* xp = xs.x + (xrow ? lr : 0) * xs.ldx + lc * 16;
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
+  // The 64 threads that finish a block (thread -> activation row m, channel
+  // group of 4) request their per-channel constants first, so that these
+  // arrive under the weight stream instead of after it.
+  const int fm = t >> 2, fg = t & 3;
+  int c_cs[4] = {0, 0, 0, 0};
+  float c_ws[4] = {1.f, 1.f, 1.f, 1.f}, c_b[4] = {0.f, 0.f, 0.f, 0.f};
+  if (t < 64 && fm < a.M) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t n = nb * 16 + 4 * fg + j;
+      const int64_t np = n < a.N ? n : 0;
+      c_cs[j] = a.colsum[np];
+      if (MODE != kOutAcc32) {
+        c_ws[j] = a.w_scales[np * a.w_scale_stride];
+        if (a.bias != nullptr) c_b[j] = a.bias[np];
+      }
+    }
+  }
   v4i acc = {0, 0, 0, 0};
   for (int64_t kb0 = wave; kb0 < KB; kb0 += kWaves * kBatch) {
     v4i wf[kBatch], xf[kBatch];
@@ -121,28 +139,32 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) s_part[wave][(4 * lc + r) * 16 + lr] = acc[r];
-  __syncthreads();
-  // 64 threads finish: thread -> (activation row m, channel group of 4)
+  // requantisation constants, before the barrier: off the block's critical path
+  v4f bdiv = {0.f, 0.f, 0.f, 0.f}, mult = {0.f, 0.f, 0.f, 0.f};
+  int acc0[4] = {0, 0, 0, 0};
   if (t < 64) {
-    const int m = t >> 2, g = t & 3;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc0[j] = a.acc_coef * c_cs[j];
+      if (MODE != kOutAcc32) {
+        const float atw = a.x_scale * c_ws[j];
+        mult[j] = atw / a.out_scale;
+        bdiv[j] = a.bias != nullptr ? c_b[j] / atw : 0.f;
+      }
+    }
+  }
+  __syncthreads();
+  if (t < 64) {
+    const int m = fm, g = fg;
     if (m < a.M) {
       int raw[4];
-      v4f bdiv, mult;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int i = 4 * g + j;
-        const int64_t n = nb * 16 + i;
         int s = 0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) s += s_part[w][i * 16 + m];
-        const bool ok = n < a.N;
-        const int64_t np = ok ? n : 0;
-        raw[j] = s + a.acc_coef * a.colsum[np];
-        if (MODE != kOutAcc32) {
-          const float atw = a.x_scale * a.w_scales[np * a.w_scale_stride];
-          mult[j] = atw / a.out_scale;
-          bdiv[j] = a.bias != nullptr ? a.bias[np] / atw : 0.f;
-        }
+        raw[j] = s + acc0[j];
       }
       const int64_t n = nb * 16 + 4 * g;
       if (MODE == kOutAcc32) {
