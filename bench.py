@@ -387,6 +387,45 @@ def main():
             "algorithmic_bytes_per_launch": fbytes, "ops_per_launch": cops}
         del accs, xcqs
 
+        # ------------------------- quantized max pooling, the ResNet stem's shape
+        log("[bench] quantized max_pool2d 3x3/2 on [32,64,112,112] channels-last")
+        psets = 12  # 12 x 25.7 MB of input, more than the last-level cache
+        pxs = []
+        for _ in range(psets):
+            pf_ = torch.randn(32, 64, 112, 112, device=dev).contiguous(memory_format=torch.channels_last)
+            pxs.append(torch.quantize_per_tensor(pf_, 0.03, 128, torch.quint8))
+            del pf_
+        pcount = [0]
+
+        def pool():
+            pcount[0] += 1
+            return torch.nn.functional.max_pool2d(pxs[pcount[0] % psets], 3, 2, 1)
+
+        for _ in range(3):
+            pool()
+        pgraph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            pool()
+            side.synchronize()
+            with torch.cuda.graph(pgraph, stream=side):
+                for _ in range(2 * psets):
+                    pool()
+        torch.cuda.synchronize()
+        for _ in range(3):
+            pgraph.replay()
+        ts = events_ms(pgraph.replay, 10)
+        pavg = sum(ts) / len(ts) / (2 * psets)
+        pbytes = 32 * 64 * (112 * 112 + 56 * 56)
+        log(f"[bench] quantized max_pool2d: {pavg*1e3:.1f} us/launch in a replayed graph, {pbytes/(pavg*1e-3)/1e9:.0f} GB/s")
+        secondary["quantized_max_pool2d_stem"] = {
+            "avg_launch_us": round(pavg * 1e3, 2), "value": round(pbytes / (pavg * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "roofline": {"bound": "hbm", "achieved": round(pbytes / (pavg * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": round(pbytes / (pavg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "traffic": None},
+            "method": f"{2 * psets} launches over {psets} rotating inputs replayed in one HIP graph",
+            "algorithmic_bytes_per_launch": pbytes}
+        del pxs
+
     # ------------------------------------------------------------ CPU baseline
     cpu_baseline = None
     if not args.skip_cpu:

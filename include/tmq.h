@@ -284,6 +284,29 @@ int tmq_qadd(const void* a, const void* b, void* out, int64_t n, float a_scale,
 int tmq_qrelu(const void* x, void* y, int64_t n, int32_t zero_point, int q_signed,
               tmq_stream_t stream);
 
+/* Building block of quantized::cat (replaces QuantizedCat / QuantizedCatOut,
+ * torch_musa/csrc/aten/quantized/TensorShape.cpp:335-426, muDNN Concat): one
+ * input viewed as [outer, in_row] codes is written into the output viewed as
+ * [outer, out_row] at column out_col_offset, requantised from the input's to
+ * the output's parameters (a plain copy when they agree):
+ *   r = in_scale * float(q - in_zp);  q' = clamp(rne(r * (1/out_scale)) + out_zp)
+ * i.e. the per-tensor dequantizer followed by the per-tensor quantizer.  For a
+ * concatenation along dim d of contiguous tensors: outer = prod(sizes[:d]),
+ * in_row = size_i[d] * prod(sizes[d+1:]), one call per input. */
+int tmq_qcat_rows(const void* x, void* y, int64_t outer, int64_t in_row, int64_t out_row,
+                  int64_t out_col_offset, float in_scale, int32_t in_zero_point, float out_scale,
+                  int32_t out_zero_point, int q_signed, tmq_stream_t stream);
+
+/* Max pooling over NHWC codes (replaces MaxPool2dQuantized /
+ * QuantizedMaxPool2dImpl, torch_musa/csrc/aten/quantized/Pool.cpp:80-130,178-247,
+ * muDNN Pooling): y[b,oh,ow,c] = max over the window's in-image positions of
+ * x[b,ih,iw,c]; scale and zero point carry over.  OH / OW are the caller's
+ * (floor or ceil mode); every window must overlap the image. */
+int tmq_qmaxpool2d(const void* x, void* y, int64_t B, int64_t H, int64_t W, int64_t C, int32_t kh,
+                   int32_t kw, int32_t stride_h, int32_t stride_w, int32_t pad_h, int32_t pad_w,
+                   int32_t dil_h, int32_t dil_w, int64_t OH, int64_t OW, int q_signed,
+                   tmq_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * Measurement probe (no counterpart in the reference; used by bench.py only).
  * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four

@@ -318,3 +318,33 @@ def qrelu(q, zp):
     y = np.empty(q.shape, dtype=q.dtype)
     lib().orc_qrelu(_p(q), C.c_int64(q.size), C.c_int64(zp), C.c_int(q.dtype == np.int8), _p(y))
     return y
+
+
+def pool_out_size(n, k, s, p, d, ceil_mode):
+    """Output extent of a pooling window sweep (PyTorch's pooling_output_shape)."""
+    out = (n + 2 * p - d * (k - 1) - 1 + (s - 1 if ceil_mode else 0)) // s + 1
+    if ceil_mode and (out - 1) * s >= n + p:
+        out -= 1
+    return out
+
+
+def qmaxpool2d(x_nhwc, kernel, stride, padding, dilation=(1, 1), ceil_mode=False):
+    x = _as_bytes(x_nhwc)
+    b, h, w, c = x.shape
+    oh = pool_out_size(h, kernel[0], stride[0], padding[0], dilation[0], ceil_mode)
+    ow = pool_out_size(w, kernel[1], stride[1], padding[1], dilation[1], ceil_mode)
+    y = np.empty((b, oh, ow, c), dtype=x.dtype)
+    lib().orc_qmaxpool2d(_p(x), *[C.c_int64(v) for v in (b, h, w, c, kernel[0], kernel[1], stride[0],
+                                                        stride[1], padding[0], padding[1], dilation[0],
+                                                        dilation[1], oh, ow)],
+                         C.c_int(x.dtype == np.int8), _p(y))
+    return y
+
+
+def qcat(qs, scales, zps, axis, out_scale, out_zp):
+    """quantized::cat: every input dequantized and requantized to the output's
+    parameters (the composition PyTorch's CPU op performs), then concatenated."""
+    signed = _as_bytes(qs[0]).dtype == np.int8
+    parts = [quantize_per_tensor(dequantize_per_tensor(q, s, z), out_scale, out_zp, signed)
+             for q, s, z in zip(qs, scales, zps)]
+    return np.concatenate(parts, axis=axis)

@@ -523,3 +523,29 @@ ORC_API void orc_qrelu(const uint8_t* x, int64_t n, int64_t zp, int is_signed, u
     y[i] = (uint8_t)(v > zp ? v : (int32_t)zp);
   }
 }
+
+/* Max pooling over NHWC codes: the maximum of the window's in-image codes
+ * (reference Pool.cpp:178-247 hands it to muDNN; PyTorch's CPU
+ * quantized_max_pool2d takes the maximum of the underlying integers). */
+ORC_API void orc_qmaxpool2d(const uint8_t* x, int64_t B, int64_t H, int64_t W, int64_t C,
+                            int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw,
+                            int64_t dh, int64_t dw, int64_t OH, int64_t OW, int is_signed, uint8_t* y) {
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t oh = 0; oh < OH; ++oh)
+      for (int64_t ow = 0; ow < OW; ++ow)
+        for (int64_t c = 0; c < C; ++c) {
+          int32_t m = is_signed ? -128 : 0;
+          for (int64_t i = 0; i < kh; ++i) {
+            const int64_t ih = oh * sh - ph + i * dh;
+            if (ih < 0 || ih >= H) continue;
+            for (int64_t j = 0; j < kw; ++j) {
+              const int64_t iw = ow * sw - pw + j * dw;
+              if (iw < 0 || iw >= W) continue;
+              const uint8_t byte = x[((b * H + ih) * W + iw) * C + c];
+              const int32_t v = is_signed ? (int32_t)(int8_t)byte : (int32_t)byte;
+              if (v > m) m = v;
+            }
+          }
+          y[((b * OH + oh) * OW + ow) * C + c] = (uint8_t)m;
+        }
+}

@@ -329,3 +329,44 @@ def qadd_cases():
                         qb=rng.integers(lo, hi, shape).astype(dt), a_scale=sa, a_zp=za, b_scale=sb,
                         b_zp=zb, out_scale=so, out_zp=zo, signed=signed, relu=relu))
     return out
+
+
+# --------------------------------------------------------------------------
+# quantized::cat and quantized max pooling
+# --------------------------------------------------------------------------
+def qcat_cases():
+    spec = [
+        # name, shapes (differ along axis only), axis, signed, per-input (scale, zp), out (scale, zp)
+        ("same_params_axis1", [(2, 3, 4), (2, 5, 4)], 1, False, [(0.1, 10), (0.1, 10)], (0.1, 10)),
+        ("requant_axis1", [(2, 3, 4), (2, 5, 4), (2, 1, 4)], 1, False, [(0.1, 10), (0.2, 20), (0.05, 0)], (0.15, 30)),
+        ("requant_axis0_s8", [(3, 7), (2, 7)], 0, True, [(0.02, -3), (0.045, 5)], (0.03, 1)),
+        ("last_axis", [(4, 6, 16), (4, 6, 32)], -1, False, [(0.3, 128), (0.11, 100)], (0.2, 120)),
+        ("channels_16aligned", [(2, 16, 5, 5), (2, 32, 5, 5)], 1, False, [(0.07, 77), (0.09, 99)], (0.08, 88)),
+    ]
+    out = []
+    for i, (name, shapes, axis, signed, params, (so, zo)) in enumerate(spec):
+        rng = np.random.default_rng(1400 + i)
+        lo, hi = (-128, 128) if signed else (0, 256)
+        dt = np.int8 if signed else np.uint8
+        out.append(dict(name=name, qs=[rng.integers(lo, hi, sh).astype(dt) for sh in shapes], axis=axis,
+                        scales=[p[0] for p in params], zps=[p[1] for p in params], out_scale=so, out_zp=zo,
+                        signed=signed))
+    return out
+
+
+def qmaxpool_cases():
+    spec = [
+        # name, (B, H, W, C), kernel, stride, padding, dilation, ceil_mode, signed
+        ("k3s2p1_c16", (2, 13, 13, 16), (3, 3), (2, 2), (1, 1), (1, 1), False, False),
+        ("k3s2p1_ceil_c16", (2, 14, 14, 16), (3, 3), (2, 2), (1, 1), (1, 1), True, False),
+        ("k2s2_c5_s8", (3, 8, 10, 5), (2, 2), (2, 2), (0, 0), (1, 1), False, True),
+        ("k3s1p1_dil2_c32", (1, 9, 9, 32), (3, 3), (1, 1), (1, 1), (2, 2), False, False),
+        ("k5x3_s2x1_c7", (2, 11, 6, 7), (5, 3), (2, 1), (2, 1), (1, 1), True, True),
+    ]
+    out = []
+    for i, (name, shape, k, s, p, d, ceil_mode, signed) in enumerate(spec):
+        rng = np.random.default_rng(1500 + i)
+        lo, hi = (-128, 128) if signed else (0, 256)
+        out.append(dict(name=name, x=rng.integers(lo, hi, shape).astype(np.int8 if signed else np.uint8),
+                        kernel=k, stride=s, padding=p, dilation=d, ceil_mode=ceil_mode, signed=signed))
+    return out

@@ -182,6 +182,23 @@ def main():
         g[k + "/y"] = y.int_repr().numpy()
         g[k + "/relu_a"] = torch.relu(qa).int_repr().numpy()
 
+    # ---- quantized::cat, quantized max pooling -------------------------------
+    for c in cases.qcat_cases():
+        qs = [torch._make_per_tensor_quantized_tensor(torch.from_numpy(q), s_, z_)
+              for q, s_, z_ in zip(c["qs"], c["scales"], c["zps"])]
+        y = torch.ops.quantized.cat(qs, c["axis"], c["out_scale"], c["out_zp"])
+        k = "qcat/" + c["name"]
+        g[k + "/q0_crc"] = np.uint32(cases.crc(c["qs"][0]))
+        g[k + "/y"] = y.int_repr().numpy()
+    for c in cases.qmaxpool_cases():
+        xq = torch._make_per_tensor_quantized_tensor(
+            torch.from_numpy(c["x"]).permute(0, 3, 1, 2).contiguous(), 0.1, -7 if c["signed"] else 33)
+        y = torch.nn.functional.max_pool2d(xq, c["kernel"], c["stride"], c["padding"], c["dilation"],
+                                           c["ceil_mode"])
+        k = "qmaxpool/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/y"] = y.int_repr().permute(0, 2, 3, 1).contiguous().numpy()
+
     # ---- quantized::conv2d -------------------------------------------------
     for c in cases.conv_cases():
         x_nchw = torch.from_numpy(c["xq"]).permute(0, 3, 1, 2)  # channels-last view

@@ -341,3 +341,27 @@ def test_quantized_add_keeps_channels_last_and_checks_shapes():
     assert (y.int_repr().cpu().int() - want.int_repr().int()).abs().max() <= 1
     with pytest.raises(RuntimeError):
         torch.ops.quantized.add(qa, qb[:, :4], 0.08, 128)
+
+
+@pytest.mark.parametrize("c", cases.qcat_cases(), ids=lambda c: c["name"])
+def test_quantized_cat_op(golden, c):
+    say("aten qcat", c["name"])
+    qs = [torch._make_per_tensor_quantized_tensor(torch.from_numpy(q).cuda(), s_, z_)
+          for q, s_, z_ in zip(c["qs"], c["scales"], c["zps"])]
+    y = torch.ops.quantized.cat(qs, c["axis"], c["out_scale"], c["out_zp"])
+    assert y.q_scale() == c["out_scale"] and y.q_zero_point() == c["out_zp"]
+    np.testing.assert_array_equal(y.int_repr().cpu().numpy(), golden["qcat/" + c["name"] + "/y"])
+    # scale / zero point default to the first input's
+    y0 = torch.ops.quantized.cat(qs, c["axis"], None, None)
+    assert y0.q_scale() == qs[0].q_scale() and y0.q_zero_point() == qs[0].q_zero_point()
+
+
+@pytest.mark.parametrize("c", cases.qmaxpool_cases(), ids=lambda c: c["name"])
+def test_quantized_max_pool2d_op(golden, c):
+    say("aten qmaxpool", c["name"])
+    zp = -7 if c["signed"] else 33
+    xq = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["x"]).cuda().permute(0, 3, 1, 2), 0.1, zp)
+    y = torch.nn.functional.max_pool2d(xq, c["kernel"], c["stride"], c["padding"], c["dilation"], c["ceil_mode"])
+    assert y.q_scale() == 0.1 and y.q_zero_point() == zp
+    np.testing.assert_array_equal(y.int_repr().permute(0, 2, 3, 1).contiguous().cpu().numpy(),
+                                  golden["qmaxpool/" + c["name"] + "/y"])

@@ -226,3 +226,35 @@ def test_qadd_unaligned_and_large(cabi):
     # commutes when the operands' quantization parameters are swapped too
     tz = cabi.qadd(tb, 0.03, 100, ta, 0.05, 128, 0.06, 120)
     assert torch.equal(ty, tz)
+
+
+# ---------------------------------------------------------------------------
+# quantized::cat, quantized max pooling
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("c", cases.qcat_cases(), ids=lambda c: c["name"])
+def test_qcat(cabi, golden, c):
+    say("qcat", c["name"])
+    y = host(cabi.qcat([dev(q) for q in c["qs"]], c["scales"], c["zps"], c["axis"], c["out_scale"], c["out_zp"]))
+    np.testing.assert_array_equal(y, golden["qcat/" + c["name"] + "/y"])
+    np.testing.assert_array_equal(y, oracle.qcat(c["qs"], c["scales"], c["zps"], c["axis"], c["out_scale"], c["out_zp"]))
+
+
+@pytest.mark.parametrize("c", cases.qmaxpool_cases(), ids=lambda c: c["name"])
+def test_qmaxpool2d(cabi, golden, c):
+    say("qmaxpool", c["name"])
+    want = golden["qmaxpool/" + c["name"] + "/y"]
+    y = host(cabi.qmaxpool2d(dev(c["x"]), c["kernel"], c["stride"], c["padding"], c["dilation"], want.shape[1:3]))
+    np.testing.assert_array_equal(y, want)
+
+
+def test_qmaxpool_resnet_stem_sized(cabi):
+    """[32,112,112,64] -> 3x3 / 2, pad 1: the pooling after a ResNet stem."""
+    say("qmaxpool stem")
+    rng = np.random.default_rng(91)
+    x = rng.integers(0, 256, (32, 112, 112, 64), dtype=np.uint8)
+    y = host(cabi.qmaxpool2d(dev(x), (3, 3), (2, 2), (1, 1), (1, 1), (56, 56)))
+    # separable maximum in numpy: rows then columns over the padded image
+    xp = np.pad(x, ((0, 0), (1, 1), (1, 1), (0, 0)))
+    r = np.maximum(np.maximum(xp[:, 0:-2:2], xp[:, 1:-1:2]), xp[:, 2::2])
+    want = np.maximum(np.maximum(r[:, :, 0:-2:2], r[:, :, 1:-1:2]), r[:, :, 2::2])
+    np.testing.assert_array_equal(y, want[:, :56, :56])

@@ -149,3 +149,19 @@ def test_qadd_and_qrelu(golden, c):
     d = np.abs(y.astype(np.int32) - golden[k + "/y"].astype(np.int32))
     assert d.max() <= 1 and np.count_nonzero(d) <= max(1, d.size // 20000), np.count_nonzero(d)
     np.testing.assert_array_equal(oracle.qrelu(c["qa"], c["a_zp"]), golden[k + "/relu_a"])
+
+
+@pytest.mark.parametrize("c", cases.qcat_cases(), ids=lambda c: c["name"])
+def test_qcat(golden, c):
+    k = "qcat/" + c["name"]
+    _check_crc(golden, k + "/q0_crc", c["qs"][0])
+    y = oracle.qcat(c["qs"], c["scales"], c["zps"], c["axis"], c["out_scale"], c["out_zp"])
+    np.testing.assert_array_equal(y, golden[k + "/y"])
+
+
+@pytest.mark.parametrize("c", cases.qmaxpool_cases(), ids=lambda c: c["name"])
+def test_qmaxpool2d(golden, c):
+    k = "qmaxpool/" + c["name"]
+    _check_crc(golden, k + "/x_crc", c["x"])
+    y = oracle.qmaxpool2d(c["x"], c["kernel"], c["stride"], c["padding"], c["dilation"], c["ceil_mode"])
+    np.testing.assert_array_equal(y, golden[k + "/y"])

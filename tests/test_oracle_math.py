@@ -277,3 +277,27 @@ def test_qrelu_is_a_clamp_at_the_zero_point():
     np.testing.assert_array_equal(oracle.qrelu(q, 77), np.maximum(q, 77))
     s = np.arange(-128, 128).astype(np.int8)
     np.testing.assert_array_equal(oracle.qrelu(s, -5), np.maximum(s, -5))
+
+
+def test_qmaxpool_brute_force_and_global_window():
+    rng = np.random.default_rng(12)
+    x = rng.integers(0, 256, (2, 6, 7, 3), dtype=np.uint8)
+    # a window that covers the whole image is the per-channel maximum
+    y = oracle.qmaxpool2d(x, (6, 7), (6, 7), (0, 0))
+    np.testing.assert_array_equal(y[:, 0, 0, :], x.max(axis=(1, 2)))
+    # 1x1 window, stride 1: identity
+    np.testing.assert_array_equal(oracle.qmaxpool2d(x, (1, 1), (1, 1), (0, 0)), x)
+    # 2x2 / 2 against a reshape-based maximum
+    x2 = x[:, :6, :6, :]
+    want = x2.reshape(2, 3, 2, 3, 2, 3).max(axis=(2, 4))
+    np.testing.assert_array_equal(oracle.qmaxpool2d(x2, (2, 2), (2, 2), (0, 0)), want)
+
+
+def test_qcat_with_equal_parameters_is_concatenation():
+    rng = np.random.default_rng(13)
+    a = rng.integers(0, 256, (2, 3, 4), dtype=np.uint8)
+    b = rng.integers(0, 256, (2, 5, 4), dtype=np.uint8)
+    np.testing.assert_array_equal(oracle.qcat([a, b], [0.1, 0.1], [7, 7], 1, 0.1, 7), np.concatenate([a, b], 1))
+    # scale ratio 2 with zero points 0: codes halve (ties to even)
+    y = oracle.qcat([a], [0.25], [0], 0, 0.5, 0)
+    np.testing.assert_array_equal(y, np.rint(a / 2.0).astype(np.uint8))

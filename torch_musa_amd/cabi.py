@@ -27,7 +27,7 @@ DECLARED_SYMBOLS = [
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
-    "tmq_qadd", "tmq_qrelu",
+    "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d",
     "tmq_probe_mfma_i8",
 ]
 
@@ -126,6 +126,9 @@ def lib() -> C.CDLL:
         l.tmq_qadd.argtypes = [v, v, v, C.c_int64, C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_float,
                                C.c_int32, C.c_int, C.c_int, v]
         l.tmq_qrelu.argtypes = [v, v, C.c_int64, C.c_int32, C.c_int, v]
+        l.tmq_qcat_rows.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int32,
+                                    C.c_float, C.c_int32, C.c_int, v]
+        l.tmq_qmaxpool2d.argtypes = [v, v] + [C.c_int64] * 4 + [C.c_int32] * 8 + [C.c_int64] * 2 + [C.c_int, v]
         l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, v, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]
         _lib = l
@@ -464,6 +467,39 @@ def qrelu(q, zp, out=None):
     y = out if out is not None else torch.empty_like(q)
     check(lib().tmq_qrelu(q.data_ptr(), y.data_ptr(), q.numel(), zp, int(q.dtype == torch.int8),
                           stream_ptr()), "tmq_qrelu")
+    return y
+
+
+def qcat(qs, scales, zps, axis, out_scale, out_zp):
+    """quantized::cat of contiguous tensors along ``axis``."""
+    shape = list(qs[0].shape)
+    axis = axis % len(shape)
+    shape[axis] = sum(q.shape[axis] for q in qs)
+    y = torch.empty(shape, dtype=qs[0].dtype, device=qs[0].device)
+    outer = 1
+    for d in shape[:axis]:
+        outer *= d
+    inner = 1
+    for d in shape[axis + 1:]:
+        inner *= d
+    off = 0
+    for q, s, z in zip(qs, scales, zps):
+        assert q.is_contiguous() and q.dtype == y.dtype
+        row = q.shape[axis] * inner
+        check(lib().tmq_qcat_rows(q.data_ptr(), y.data_ptr(), outer, row, shape[axis] * inner, off, s, z,
+                                  out_scale, out_zp, int(q.dtype == torch.int8), stream_ptr()),
+              "tmq_qcat_rows")
+        off += row
+    return y
+
+
+def qmaxpool2d(x_nhwc, kernel, stride, padding, dilation, out_hw):
+    assert x_nhwc.is_contiguous()
+    b, h, w, c = x_nhwc.shape
+    y = torch.empty((b, out_hw[0], out_hw[1], c), dtype=x_nhwc.dtype, device=x_nhwc.device)
+    check(lib().tmq_qmaxpool2d(x_nhwc.data_ptr(), y.data_ptr(), b, h, w, c, kernel[0], kernel[1], stride[0],
+                               stride[1], padding[0], padding[1], dilation[0], dilation[1], out_hw[0],
+                               out_hw[1], int(x_nhwc.dtype == torch.int8), stream_ptr()), "tmq_qmaxpool2d")
     return y
 
 

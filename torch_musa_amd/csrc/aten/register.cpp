@@ -641,6 +641,92 @@ at::Tensor qrelu_run(const at::Tensor& self) {
   return y;
 }
 
+// ---------------------------------------------------------------------------
+// quantized::cat (TensorShape.cpp:383-426 of the reference) and
+// aten::quantized_max_pool2d (Pool.cpp:178-247)
+// ---------------------------------------------------------------------------
+at::Tensor qcat_run(const c10::List<at::Tensor>& qxs, int64_t dim, std::optional<double> scale,
+                    std::optional<int64_t> zero_point) {
+  TORCH_CHECK(qxs.size() > 0, "quantized::cat expects at least one tensor");
+  const at::Tensor qx0 = qxs[0];
+  if (dim < 0) dim += qx0.dim();
+  TORCH_CHECK(dim >= 0 && dim < qx0.dim(), "Wrong dim: ", dim);
+  TORCH_CHECK(qx0.qscheme() == c10::kPerTensorAffine || qx0.qscheme() == c10::kPerTensorSymmetric,
+              "Quantized cat only supports quantize-per-tensor");
+  const bool sgn = is_signed_qtype(qx0.scalar_type(), "quantized::cat");
+  const double out_scale = scale.has_value() ? *scale : qx0.q_scale();
+  const int64_t out_zp = zero_point.has_value() ? *zero_point : qx0.q_zero_point();
+  TORCH_CHECK(out_scale > 0, "quantized::cat: output scale must be positive");
+  std::vector<int64_t> shape = qx0.sizes().vec();
+  shape[dim] = 0;
+  for (const at::Tensor& qx : qxs) {
+    TORCH_CHECK(qx.scalar_type() == qx0.scalar_type() && qx.dim() == qx0.dim() && qx.device() == qx0.device(),
+                "quantized::cat: all inputs need the dtype, rank and device of the first");
+    TORCH_CHECK(qx.qscheme() == c10::kPerTensorAffine || qx.qscheme() == c10::kPerTensorSymmetric,
+                "Quantized cat only supports quantize-per-tensor");
+    for (int64_t d = 0; d < qx0.dim(); ++d)
+      TORCH_CHECK(d == dim || qx.size(d) == qx0.size(d), "quantized::cat: sizes differ outside dim ", dim);
+    shape[dim] += qx.size(dim);
+  }
+  const c10::OptionalDeviceGuard guard(at::device_of(qx0));
+  at::Tensor y = at::_empty_affine_quantized(shape, qx0.options(), out_scale, out_zp, c10::MemoryFormat::Contiguous);
+  if (y.numel() == 0) return y;
+  int64_t outer = 1, inner = 1;
+  for (int64_t d = 0; d < dim; ++d) outer *= shape[d];
+  for (int64_t d = dim + 1; d < qx0.dim(); ++d) inner *= shape[d];
+  int64_t off = 0;
+  for (const at::Tensor& qx : qxs) {
+    const at::Tensor x = qx.contiguous();
+    const int64_t row = x.size(dim) * inner;
+    check_status(tmq_qcat_rows(x.data_ptr(), y.data_ptr(), outer, row, shape[dim] * inner, off,
+                               static_cast<float>(x.q_scale()), static_cast<int32_t>(x.q_zero_point()),
+                               static_cast<float>(out_scale), static_cast<int32_t>(out_zp), sgn, current_stream(y)),
+                 "tmq_qcat_rows");
+    off += row;
+  }
+  return y;
+}
+
+int64_t pool_out(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d, bool ceil_mode) {
+  int64_t out = (n + 2 * p - d * (k - 1) - 1 + (ceil_mode ? s - 1 : 0)) / s + 1;
+  if (ceil_mode && (out - 1) * s >= n + p) --out;
+  return out;
+}
+
+at::Tensor qmaxpool2d_run(const at::Tensor& input, at::IntArrayRef kernel_size, at::IntArrayRef stride,
+                          at::IntArrayRef padding, at::IntArrayRef dilation, bool ceil_mode) {
+  TORCH_CHECK(input.qscheme() == c10::kPerTensorAffine || input.qscheme() == c10::kPerTensorSymmetric,
+              "MaxPool2dQuantized(): only supports per tensor quantized tensors");
+  const bool sgn = is_signed_qtype(input.scalar_type(), "quantized_max_pool2d");
+  TORCH_CHECK(input.dim() == 3 || input.dim() == 4, "Expecting the input tensor of rank 3 or 4.");
+  TORCH_CHECK(kernel_size.size() == 1 || kernel_size.size() == 2, "quantized_max_pool2d: kernel_size must have 1 or 2 elements");
+  TORCH_CHECK(stride.empty() || stride.size() == 1 || stride.size() == 2, "quantized_max_pool2d: stride must have 0, 1 or 2 elements");
+  TORCH_CHECK(padding.size() == 1 || padding.size() == 2, "quantized_max_pool2d: padding must have 1 or 2 elements");
+  TORCH_CHECK(dilation.size() == 1 || dilation.size() == 2, "quantized_max_pool2d: dilation must have 1 or 2 elements");
+  const int64_t kh = kernel_size[0], kw = kernel_size.size() == 1 ? kh : kernel_size[1];
+  const int64_t sh = stride.empty() ? kh : stride[0], sw = stride.empty() ? kw : (stride.size() == 1 ? sh : stride[1]);
+  const int64_t ph = padding[0], pw = padding.size() == 1 ? ph : padding[1];
+  const int64_t dh = dilation[0], dw = dilation.size() == 1 ? dh : dilation[1];
+  TORCH_CHECK(kh > 0 && kw > 0 && sh > 0 && sw > 0 && dh > 0 && dw > 0 && ph >= 0 && pw >= 0,
+              "quantized_max_pool2d: kernel, stride and dilation must be positive, padding non-negative");
+  TORCH_CHECK(ph <= kh / 2 && pw <= kw / 2, "pad should be at most half of effective kernel size");
+  const c10::OptionalDeviceGuard guard(at::device_of(input));
+  const at::Tensor x4 = input.dim() == 3 ? input.unsqueeze(0) : input;
+  const at::Tensor x = x4.contiguous(c10::MemoryFormat::ChannelsLast);
+  const int64_t B = x.size(0), C = x.size(1), H = x.size(2), W = x.size(3);
+  const int64_t OH = pool_out(H, kh, sh, ph, dh, ceil_mode), OW = pool_out(W, kw, sw, pw, dw, ceil_mode);
+  TORCH_CHECK(OH > 0 && OW > 0, "quantized_max_pool2d: the output would be empty");
+  at::Tensor y = at::_empty_affine_quantized({B, C, OH, OW}, x.options(), input.q_scale(), input.q_zero_point(),
+                                             c10::MemoryFormat::ChannelsLast);
+  if (y.numel() > 0)
+    check_status(tmq_qmaxpool2d(x.data_ptr(), y.data_ptr(), B, H, W, C, static_cast<int32_t>(kh),
+                                static_cast<int32_t>(kw), static_cast<int32_t>(sh), static_cast<int32_t>(sw),
+                                static_cast<int32_t>(ph), static_cast<int32_t>(pw), static_cast<int32_t>(dh),
+                                static_cast<int32_t>(dw), OH, OW, sgn, current_stream(x)),
+                 "tmq_qmaxpool2d");
+  return input.dim() == 3 ? y.squeeze(0) : y;
+}
+
 }  // namespace
 
 // The two SiLU schemas are not part of upstream PyTorch; the reference adds them
@@ -662,6 +748,7 @@ TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add_relu"), TORCH_FN(qconv2d_add_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_silu.new"), TORCH_FN(qconv2d_silu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add_silu"), TORCH_FN(qconv2d_add_silu_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::cat"), TORCH_FN(qcat_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::add"), TORCH_FN(qadd_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::add_relu"), TORCH_FN(qadd_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear"), TORCH_FN(qlinear_run));
@@ -694,6 +781,7 @@ TORCH_LIBRARY_IMPL(aten, CUDA, m) {
 // one kernel instead of PyTorch-ROCm's int_repr / compare / where / re-wrap chain
 TORCH_LIBRARY_IMPL(aten, QuantizedCUDA, m) {
   m.impl("relu", TORCH_FN(qrelu_run));
+  m.impl("quantized_max_pool2d", TORCH_FN(qmaxpool2d_run));
 }
 
 namespace {

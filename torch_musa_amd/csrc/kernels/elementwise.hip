@@ -1,5 +1,6 @@
-// Elementwise kernels on quantized tensors for gfx950: quantized::add /
-// add_relu and relu of a per-tensor quantized tensor.  HBM streaming kernels:
+// Elementwise and data-movement kernels on quantized tensors for gfx950:
+// quantized::add / add_relu, relu, the row requantiser behind quantized::cat
+// and max pooling over NHWC codes.  HBM streaming kernels:
 // a lane moves 16 bytes (16 codes) per access, consecutive lanes touch
 // consecutive addresses, a few independent accesses per thread.
 //
@@ -151,6 +152,123 @@ __global__ __launch_bounds__(kEwThreads) void qrelu_scalar_kernel(const uint8_t*
     y[i] = static_cast<uint8_t>(relu_four<SIGNED>(x[i], zp) & 0xffu);
 }
 
+// ---------------------------------------------------------------------------
+// quantized::cat building block: rows of `in_row` codes are requantised (or
+// copied, when the quantization parameters agree) into a wider output row at a
+// column offset:  y[o][off + j] = Q_out(DQ_in(x[o][j])).
+//   DQ: r = fl(in_scale) * float(q - in_zp)          (the per-tensor dequantizer)
+//   Q : q' = clamp(rne(r * fl(1/out_scale)) + out_zp)  (the per-tensor quantizer)
+// ---------------------------------------------------------------------------
+struct RequantParams {
+  float in_scale, inv_out, out_zp_f;
+  int in_zp;
+  int identity;
+};
+
+template <bool SIGNED>
+__device__ __forceinline__ uint32_t requant_codes4(uint32_t w, const RequantParams& p) {
+  if (p.identity) return w;
+  uint32_t packed = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t byte = (w >> (8 * j)) & 0xffu;
+    const int v = SIGNED ? static_cast<int>(static_cast<int8_t>(byte)) : static_cast<int>(byte);
+    const float r = p.in_scale * static_cast<float>(v - p.in_zp);
+    const float t = r * p.inv_out;
+    float q = __builtin_rintf(t) + p.out_zp_f;
+    if constexpr (SIGNED) {
+      q = __builtin_amdgcn_fmed3f(q, -128.f, 127.f);
+      packed |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xffu) << (8 * j);
+    } else {
+      packed = __builtin_amdgcn_cvt_pk_u8_f32(q, j, packed);
+    }
+  }
+  return packed;
+}
+
+// VEC = 16: rows, offset and pointers are multiples of 16 bytes; VEC = 1 otherwise.
+template <bool SIGNED, int VEC>
+__global__ __launch_bounds__(kEwThreads) void qcat_rows_kernel(const uint8_t* __restrict__ x,
+                                                               uint8_t* __restrict__ y, int64_t outer,
+                                                               int64_t in_row, int64_t out_row, int64_t off,
+                                                               RequantParams p) {
+  const int64_t per_row = in_row / VEC;
+  const int64_t total = outer * per_row;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kEwThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kEwThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t o = i / per_row, j = (i - o * per_row) * VEC;
+    const uint8_t* src = x + o * in_row + j;
+    uint8_t* dst = y + o * out_row + off + j;
+    if constexpr (VEC == 16) {
+      const v4i v = *reinterpret_cast<const v4i*>(src);
+      *reinterpret_cast<v4i*>(dst) =
+          v4i{static_cast<int>(requant_codes4<SIGNED>(v.x, p)), static_cast<int>(requant_codes4<SIGNED>(v.y, p)),
+              static_cast<int>(requant_codes4<SIGNED>(v.z, p)), static_cast<int>(requant_codes4<SIGNED>(v.w, p))};
+    } else {
+      *dst = static_cast<uint8_t>(requant_codes4<SIGNED>(*src, p) & 0xffu);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// max pooling over NHWC codes: the maximum of the window's codes (the scale
+// and zero point carry over; positions outside the image do not take part).
+// VEC = 16: one thread per (output pixel, 16 channels), C % 16 == 0.
+// ---------------------------------------------------------------------------
+struct PoolShape {
+  int64_t B, H, W, C, OH, OW;
+  int kh, kw, sh, sw, ph, pw, dh, dw;
+};
+
+template <bool SIGNED>
+__device__ __forceinline__ uint32_t max_codes4(uint32_t a, uint32_t b) {
+  const uint32_t bias = SIGNED ? 0x80808080u : 0u;
+  const uint32_t ua = a ^ bias, ub = b ^ bias;
+  const us2 me = __builtin_elementwise_max(__builtin_bit_cast(us2, ua & 0x00ff00ffu),
+                                           __builtin_bit_cast(us2, ub & 0x00ff00ffu));
+  const us2 mo = __builtin_elementwise_max(__builtin_bit_cast(us2, (ua >> 8) & 0x00ff00ffu),
+                                           __builtin_bit_cast(us2, (ub >> 8) & 0x00ff00ffu));
+  return (__builtin_bit_cast(uint32_t, me) | (__builtin_bit_cast(uint32_t, mo) << 8)) ^ bias;
+}
+
+template <bool SIGNED, int VEC>
+__global__ __launch_bounds__(kEwThreads) void qmaxpool_kernel(const uint8_t* __restrict__ x,
+                                                              uint8_t* __restrict__ y, PoolShape s) {
+  const int64_t cv = s.C / VEC;
+  const int64_t total = s.B * s.OH * s.OW * cv;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kEwThreads;
+  const uint32_t lowest = SIGNED ? 0x80808080u : 0u;  // the smallest code in every byte
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kEwThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t c = (i % cv) * VEC;
+    int64_t t = i / cv;
+    const int64_t ow = t % s.OW;
+    t /= s.OW;
+    const int64_t oh = t % s.OH, b = t / s.OH;
+    v4i m = {static_cast<int>(lowest), static_cast<int>(lowest), static_cast<int>(lowest), static_cast<int>(lowest)};
+    for (int kh = 0; kh < s.kh; ++kh) {
+      const int64_t ih = oh * s.sh - s.ph + static_cast<int64_t>(kh) * s.dh;
+      if (ih < 0 || ih >= s.H) continue;
+      for (int kw = 0; kw < s.kw; ++kw) {
+        const int64_t iw = ow * s.sw - s.pw + static_cast<int64_t>(kw) * s.dw;
+        if (iw < 0 || iw >= s.W) continue;
+        const uint8_t* src = x + ((b * s.H + ih) * s.W + iw) * s.C + c;
+        if constexpr (VEC == 16) {
+          const v4i v = *reinterpret_cast<const v4i*>(src);
+          m = v4i{static_cast<int>(max_codes4<SIGNED>(m.x, v.x)), static_cast<int>(max_codes4<SIGNED>(m.y, v.y)),
+                  static_cast<int>(max_codes4<SIGNED>(m.z, v.z)), static_cast<int>(max_codes4<SIGNED>(m.w, v.w))};
+        } else {
+          m.x = static_cast<int>(max_codes4<SIGNED>(m.x, *src) & 0xffu) | (m.x & ~0xff);
+        }
+      }
+    }
+    uint8_t* dst = y + ((b * s.OH + oh) * s.OW + ow) * s.C + c;
+    if constexpr (VEC == 16)
+      *reinterpret_cast<v4i*>(dst) = m;
+    else
+      *dst = static_cast<uint8_t>(m.x & 0xff);
+  }
+}
+
 bool zp_ok(int32_t zp, int q_signed) { return q_signed ? (zp >= -128 && zp <= 127) : (zp >= 0 && zp <= 255); }
 
 template <bool SIGNED, bool RELU>
@@ -222,6 +340,75 @@ TMQ_EXPORT int tmq_qrelu(const void* x, void* y, int64_t n, int32_t zero_point, 
       qrelu_scalar_kernel<true><<<grid, block, 0, s>>>(xb, yb, n, zero_point);
     else
       qrelu_scalar_kernel<false><<<grid, block, 0, s>>>(xb, yb, n, zero_point);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_qcat_rows(const void* x, void* y, int64_t outer, int64_t in_row, int64_t out_row,
+                             int64_t out_col_offset, float in_scale, int32_t in_zero_point,
+                             float out_scale, int32_t out_zero_point, int q_signed, tmq_stream_t stream) {
+  if (outer < 0 || in_row < 0 || out_row < in_row || out_col_offset < 0 || out_col_offset + in_row > out_row)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  if (!zp_ok(in_zero_point, q_signed) || !zp_ok(out_zero_point, q_signed) || !(out_scale > 0.f))
+    return TMQ_ERR_INVALID_ARGUMENT;
+  if (outer == 0 || in_row == 0) return TMQ_OK;
+  if (x == nullptr || y == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  RequantParams p;
+  p.in_scale = in_scale;
+  p.inv_out = 1.0f / out_scale;
+  p.out_zp_f = static_cast<float>(out_zero_point);
+  p.in_zp = in_zero_point;
+  p.identity = in_scale == out_scale && in_zero_point == out_zero_point;
+  const bool vec = in_row % 16 == 0 && out_row % 16 == 0 && out_col_offset % 16 == 0 && aligned(x, 16) &&
+                   aligned(y, 16);
+  const int64_t items = outer * (vec ? in_row / 16 : in_row);
+  int64_t g = ceil_div(items, kEwThreads);
+  g = g > (1 << 20) ? (1 << 20) : g;
+  const dim3 grid(static_cast<unsigned>(g)), block(kEwThreads);
+  hipStream_t s = as_stream(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  if (vec) {
+    if (q_signed)
+      qcat_rows_kernel<true, 16><<<grid, block, 0, s>>>(xb, yb, outer, in_row, out_row, out_col_offset, p);
+    else
+      qcat_rows_kernel<false, 16><<<grid, block, 0, s>>>(xb, yb, outer, in_row, out_row, out_col_offset, p);
+  } else {
+    if (q_signed)
+      qcat_rows_kernel<true, 1><<<grid, block, 0, s>>>(xb, yb, outer, in_row, out_row, out_col_offset, p);
+    else
+      qcat_rows_kernel<false, 1><<<grid, block, 0, s>>>(xb, yb, outer, in_row, out_row, out_col_offset, p);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_qmaxpool2d(const void* x, void* y, int64_t B, int64_t H, int64_t W, int64_t C,
+                              int32_t kh, int32_t kw, int32_t stride_h, int32_t stride_w, int32_t pad_h,
+                              int32_t pad_w, int32_t dil_h, int32_t dil_w, int64_t OH, int64_t OW,
+                              int q_signed, tmq_stream_t stream) {
+  if (B < 0 || H <= 0 || W <= 0 || C < 0 || OH < 0 || OW < 0 || kh <= 0 || kw <= 0 || stride_h <= 0 ||
+      stride_w <= 0 || pad_h < 0 || pad_w < 0 || dil_h <= 0 || dil_w <= 0)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  // every window must touch the image, or its maximum is undefined
+  if (OH > 0 && ((OH - 1) * stride_h - pad_h >= H || pad_h > (kh - 1) * dil_h)) return TMQ_ERR_INVALID_ARGUMENT;
+  if (OW > 0 && ((OW - 1) * stride_w - pad_w >= W || pad_w > (kw - 1) * dil_w)) return TMQ_ERR_INVALID_ARGUMENT;
+  const int64_t n = B * OH * OW * C;
+  if (n == 0) return TMQ_OK;
+  if (x == nullptr || y == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  PoolShape s{B, H, W, C, OH, OW, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w};
+  const bool vec = C % 16 == 0 && aligned(x, 16) && aligned(y, 16);
+  int64_t g = ceil_div(vec ? n / 16 : n, kEwThreads);
+  g = g > (1 << 20) ? (1 << 20) : g;
+  const dim3 grid(static_cast<unsigned>(g)), block(kEwThreads);
+  hipStream_t hs = as_stream(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  if (vec) {
+    if (q_signed) qmaxpool_kernel<true, 16><<<grid, block, 0, hs>>>(xb, yb, s);
+    else qmaxpool_kernel<false, 16><<<grid, block, 0, hs>>>(xb, yb, s);
+  } else {
+    if (q_signed) qmaxpool_kernel<true, 1><<<grid, block, 0, hs>>>(xb, yb, s);
+    else qmaxpool_kernel<false, 1><<<grid, block, 0, hs>>>(xb, yb, s);
   }
   return launch_status();
 }
