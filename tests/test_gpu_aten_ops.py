@@ -365,3 +365,84 @@ def test_quantized_max_pool2d_op(golden, c):
     assert y.q_scale() == 0.1 and y.q_zero_point() == zp
     np.testing.assert_array_equal(y.int_repr().permute(0, 2, 3, 1).contiguous().cpu().numpy(),
                                   golden["qmaxpool/" + c["name"] + "/y"])
+
+
+# ---------------------------------------------------------------------------
+# torch.ao modules on the GPU (the reference's tests drive its ops through
+# nnq.Linear / nnq.Conv2d with set_weight_bias, test_quantized_linear.py:58-60)
+# ---------------------------------------------------------------------------
+def test_ao_modules_run_on_gpu_and_round_trip_state():
+    import torch.ao.nn.intrinsic.quantized as nniq
+    import torch.ao.nn.quantized as nnq
+    say("ao modules")
+    torch.manual_seed(3)
+    x = torch.randn(4, 64)
+    w = torch.randn(32, 64) * 0.1
+    b = torch.randn(32)
+    wq = torch.quantize_per_tensor(w, float(w.abs().max()) / 128, 0, torch.qint8)
+    xq = torch.quantize_per_tensor(x, float(x.abs().max()) / 128, 128, torch.quint8)
+    m, mc = nnq.Linear(64, 32), nnq.Linear(64, 32)
+    m.set_weight_bias(wq.cuda(), b.cuda())
+    mc.set_weight_bias(wq, b)
+    for mod in (m, mc):
+        mod.scale, mod.zero_point = 0.1, 128
+    assert torch.equal(m(xq.cuda()).int_repr().cpu(), mc(xq).int_repr())
+    assert torch.equal(m.weight().int_repr().cpu(), wq.int_repr()) and m.bias().is_cuda
+    m2 = nnq.Linear(64, 32)
+    m2.load_state_dict(m.state_dict())
+    assert torch.equal(m2(xq.cuda()).int_repr().cpu(), mc(xq).int_repr())
+
+    xc = torch.randn(2, 16, 9, 9)
+    wc = torch.randn(8, 16, 3, 3) * 0.1
+    bc = torch.randn(8)
+    wcq = torch.quantize_per_tensor(wc, float(wc.abs().max()) / 128, 0, torch.qint8)
+    xcq = torch.quantize_per_tensor(xc, float(xc.abs().max()) / 128, 128, torch.quint8)
+    for cls in (nnq.Conv2d, nniq.ConvReLU2d):
+        g, c = cls(16, 8, 3, padding=1), cls(16, 8, 3, padding=1)
+        g.set_weight_bias(wcq.cuda(), bc.cuda())
+        c.set_weight_bias(wcq, bc)
+        for mod in (g, c):
+            mod.scale, mod.zero_point = 0.05, 128
+        assert torch.equal(g(xcq.cuda()).int_repr().cpu(), c(xcq).int_repr()), cls.__name__
+        wt, bt = g._weight_bias()
+        assert torch.equal(wt.int_repr().cpu(), wcq.int_repr()) and torch.equal(bt.cpu(), bc)
+
+
+def test_residual_block_end_to_end():
+    """conv_relu -> conv_add_relu -> max_pool -> cat with the block's input pooled,
+    all on quantized GPU tensors, against the float pipeline on dequantized values."""
+    import torch.nn.functional as F
+    say("residual block")
+    torch.manual_seed(5)
+    ops = torch.ops.quantized
+    x = torch.relu(torch.randn(2, 32, 16, 16)).contiguous(memory_format=torch.channels_last)
+    xq = torch.quantize_per_tensor(x, float(x.max()) / 255, 0, torch.quint8)
+    ws, ps = [], []
+    for _ in range(2):
+        w = torch.randn(32, 32, 3, 3) * 0.05
+        s = (w.abs().amax(dim=(1, 2, 3)) / 127).double()
+        wq = torch.quantize_per_channel(w, s, torch.zeros(32, dtype=torch.int64), 0, torch.qint8)
+        b = torch.randn(32) * 0.1
+        ws.append((wq, b))
+        ps.append(ops.conv2d_prepack(wq.cuda(), b.cuda(), [1, 1], [1, 1], [1, 1], 1))
+    # float pipeline with a quantize -> dequantize after every op, as the quantized graph does
+    def qdq(t, s, z=0):
+        return torch.quantize_per_tensor(t, s, z, torch.quint8)
+    f1 = torch.relu(F.conv2d(xq.dequantize(), ws[0][0].dequantize(), ws[0][1], 1, 1))
+    s1 = float(f1.max()) / 255
+    q1 = qdq(f1, s1)
+    f2 = torch.relu(F.conv2d(q1.dequantize(), ws[1][0].dequantize(), ws[1][1], 1, 1) + xq.dequantize())
+    s2 = float(f2.max()) / 255
+    q2 = qdq(f2, s2)
+    want = torch.cat([F.max_pool2d(q2.dequantize(), 2), F.max_pool2d(xq.dequantize(), 2)], 1)
+    want_q = qdq(want, s2)
+
+    g = xq.cuda()
+    y1 = ops.conv2d_relu(g, ps[0], s1, 0)
+    y2 = ops.conv2d_add_relu(y1, g, ps[1], s2, 0)
+    y = ops.cat([F.max_pool2d(y2, 2), F.max_pool2d(g, 2)], 1, s2, 0)
+    assert y.shape == want_q.shape
+    d = (y.int_repr().cpu().int() - want_q.int_repr().int()).abs()
+    # one LSB per requantisation boundary crossed; a second-layer value may move
+    # by one more when its input moved
+    assert d.max() <= 2 and (d > 1).float().mean() < 1e-3 and (d > 0).float().mean() < 0.02, (d.max(), (d > 0).float().mean())
