@@ -112,7 +112,9 @@ def test_decode_shapes(cabi, m):
     _check(y, want, "decode")
 
 
-@pytest.mark.parametrize("m,n,k", [(3, 50, 100), (16, 16, 64), (9, 130, 4096 + 64), (16, 17, 16)])
+@pytest.mark.parametrize("m,n,k", [(3, 50, 100), (16, 16, 64), (9, 130, 4096 + 64), (16, 17, 16),
+                                   (17, 48, 256), (32, 4096, 4096), (33, 130, 1024 + 16), (48, 64, 512),
+                                   (64, 1000, 2048)])
 def test_decode_ragged(cabi, m, n, k):
     say("decode ragged", m, n, k)
     c = _tile_case(m, n, k, seed=m * n)

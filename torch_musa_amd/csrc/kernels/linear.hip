@@ -89,27 +89,36 @@ __global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ 
 //   (channel), j = l%16 (activation row).
 // ---------------------------------------------------------------------------
 constexpr int kDecodeWaves = 8;
-template <int MODE>
+constexpr int kDecodeMaxRows = 64;
+constexpr int kDecodeRowsAuto = 64;  // largest M the automatic choice sends here
+// MG = groups of 16 activation rows (M <= 16 * MG): the weight operands are
+// loaded once and multiplied with every group.
+template <int MODE, int MG>
 __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(GemmArgs a, XLinear xs) {
   constexpr int kWaves = kDecodeWaves;
   constexpr int kBatch = 8;  // 64-byte k-blocks in flight per wave: 64 KB of weights per block
-  __shared__ int s_part[kWaves][16 * 16];
+  __shared__ int s_part[kWaves][MG][16 * 16];
   const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
   const int lr = lane & 15, lc = lane >> 4;
   const int64_t nb = blockIdx.x;
   const int64_t KB = ceil_div(a.K, 64);
   const uint8_t* wp = a.w_packed + nb * a.w_kchunks * 256 + lc * 256 + lr * 16;
-  const bool xrow = lr < a.M;
-  const uint8_t* xp = xs.x + (xrow ? lr : 0) * xs.ldx + lc * 16;
+  bool xrow[MG];
+  const uint8_t* xp[MG];
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) {
+    xrow[mg] = mg * 16 + lr < a.M;
+    xp[mg] = xs.x + (xrow[mg] ? mg * 16 + lr : 0) * xs.ldx + lc * 16;
+  }
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
-  // The 64 threads that finish a block (thread -> activation row m, channel
-  // group of 4) request their per-channel constants first, so that these
-  // arrive under the weight stream instead of after it.
+  // The 64 threads that finish a block (thread -> activation row within a
+  // group, channel group of 4) request their per-channel constants first, so
+  // that these arrive under the weight stream instead of after it.
   const int fm = t >> 2, fg = t & 3;
   int c_cs[4] = {0, 0, 0, 0};
   float c_ws[4] = {1.f, 1.f, 1.f, 1.f}, c_b[4] = {0.f, 0.f, 0.f, 0.f};
-  if (t < 64 && fm < a.M) {
+  if (t < 64) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t n = nb * 16 + 4 * fg + j;
@@ -121,24 +130,33 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
       }
     }
   }
-  v4i acc = {0, 0, 0, 0};
+  v4i acc[MG];
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) acc[mg] = v4i{0, 0, 0, 0};
   for (int64_t kb0 = wave; kb0 < KB; kb0 += kWaves * kBatch) {
-    v4i wf[kBatch], xf[kBatch];
+    v4i wf[kBatch], xf[MG][kBatch];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       const int64_t kb = kb0 + u * kWaves;
       const bool ok = kb < KB;
       wf[u] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + kb * 1024))
                  : v4i{0, 0, 0, 0};
-      const bool xok = ok && xrow && (kb * 64 + lc * 16 < a.K);
-      xf[u] = xok ? ld16(xp + kb * 64) : v4i{0, 0, 0, 0};
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) {
+        const bool xok = ok && xrow[mg] && (kb * 64 + lc * 16 < a.K);
+        xf[mg][u] = xok ? ld16(xp[mg] + kb * 64) : v4i{0, 0, 0, 0};
+      }
     }
 #pragma unroll
     for (int u = 0; u < kBatch; ++u)
-      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], xf[u] ^ xmask, acc, 0, 0, 0);
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg)
+        acc[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], xf[mg][u] ^ xmask, acc[mg], 0, 0, 0);
   }
 #pragma unroll
-  for (int r = 0; r < 4; ++r) s_part[wave][(4 * lc + r) * 16 + lr] = acc[r];
+  for (int mg = 0; mg < MG; ++mg)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s_part[wave][mg][(4 * lc + r) * 16 + lr] = acc[mg][r];
   // requantisation constants, before the barrier: off the block's critical path
   v4f bdiv = {0.f, 0.f, 0.f, 0.f}, mult = {0.f, 0.f, 0.f, 0.f};
   int acc0[4] = {0, 0, 0, 0};
@@ -155,15 +173,18 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
   }
   __syncthreads();
   if (t < 64) {
-    const int m = fm, g = fg;
-    if (m < a.M) {
+    const int g = fg;
+#pragma unroll
+    for (int mg = 0; mg < MG; ++mg) {
+      const int64_t m = mg * 16 + fm;
+      if (m >= a.M) continue;
       int raw[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int i = 4 * g + j;
         int s = 0;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) s += s_part[w][i * 16 + m];
+        for (int w = 0; w < kWaves; ++w) s += s_part[w][mg][i * 16 + fm];
         raw[j] = s + acc0[j];
       }
       const int64_t n = nb * 16 + 4 * g;
@@ -258,10 +279,17 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     linear_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(b, xs, x_signed);
     return launch_status();
   }
-  if ((a.M <= 16 && forced < 0) || forced == 8) {
-    if (a.M > 16) return TMQ_ERR_UNSUPPORTED;
+  if ((a.M <= kDecodeRowsAuto && forced < 0) || forced == 8) {
+    if (a.M > kDecodeMaxRows) return TMQ_ERR_UNSUPPORTED;
     const int64_t blocks = ceil_div(a.N, 16);
-    linear_decode_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(kDecodeWaves * kWave), 0, s>>>(a, xs);
+    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(blocks)), block(kDecodeWaves * kWave);
+    switch ((a.M + 15) / 16) {
+      case 1: linear_decode_kernel<MODE, 1><<<grid, block, 0, s>>>(a, xs); break;
+      case 2: linear_decode_kernel<MODE, 2><<<grid, block, 0, s>>>(a, xs); break;
+      case 3: linear_decode_kernel<MODE, 3><<<grid, block, 0, s>>>(a, xs); break;
+      default: linear_decode_kernel<MODE, 4><<<grid, block, 0, s>>>(a, xs); break;
+    }
     return launch_status();
   }
   int cfg = forced;
