@@ -279,32 +279,44 @@ __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv,
 // WM x WN waves, each wave (BM/WM) x (BN/WN).  PD = prefetch distance in
 // stages: the global loads of stage t+PD are issued while stage t is being
 // multiplied, so PD-1 stages of 16-byte loads are in flight per thread.
-template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4>
+//
+// WDMA = true: the weight stages do not pass through registers.  Each wave
+// copies 64 rows x 16 bytes per instruction straight from the packed weight
+// into LDS (global_load_lds_dwordx4), three stages ahead, into one of three
+// weight buffers; only the activations are staged through registers (they
+// need the sign-bit flip on the way).  This halves the LDS store traffic of
+// the loop and frees the weight staging registers.
+template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4, bool WDMA = false>
 __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int NT = WM * WN * kWave;
   constexpr bool kHasPost = XSRC::kPostOps;  // residual / activation epilogue compiled in
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int NW = BN * kChunks / NT;  // 16-byte weight chunks per thread per stage
+  constexpr int NW = WDMA ? 0 : BN * kChunks / NT;  // 16-byte weight chunks per thread per stage
   constexpr int NX = BM * kChunks / NT;
+  constexpr int NWAVES = WM * WN;
+  constexpr int NWI = kChunks * (BN / 64) / NWAVES;  // direct-to-LDS weight copies per wave per stage
+  constexpr int kWBufs = WDMA ? 3 : 2;
+  static_assert(!WDMA || (BN % 64 == 0 && kChunks * (BN / 64) % NWAVES == 0), "weight copies do not divide");
   constexpr int NSET = PD - 1;           // register sets holding stages in flight
-  static_assert(TM >= 1 && TN >= 1 && NW >= 1 && NX >= 1, "tile too small for the wave grid");
+  static_assert(TM >= 1 && TN >= 1 && (WDMA || NW >= 1) && NX >= 1, "tile too small for the wave grid");
   static_assert(BN * kChunks % NT == 0 && BM * kChunks % NT == 0, "uneven staging");
+  static_assert(!WDMA || PD == 4, "the explicit load-counter waits assume prefetch distance 4");
   static_assert(PD >= 3, "prefetch distance");
 
   // LDS: two stages of {weights, activations}; the same bytes are reused after
   // the main loop to transpose the output tile into row-major order.
   constexpr int kWStage = kChunks * BN * 16, kXStage = BM * kBK;
   constexpr int kOutPitch = BN + 16;  // bytes; keeps rows 16-byte aligned and off one bank
-  constexpr int kMainBytes = 2 * (kWStage + kXStage);
+  constexpr int kMainBytes = kWBufs * kWStage + 2 * kXStage;
   constexpr int kOutBytes = (MODE == kOutAcc32) ? 0 : BM * kOutPitch;
   constexpr int kTileBytes = kMainBytes > kOutBytes ? kMainBytes : kOutBytes;
   __shared__ __attribute__((aligned(16))) uint8_t smem[kTileBytes];
   __shared__ __attribute__((aligned(16))) int s_acc0[BN];
   __shared__ __attribute__((aligned(16))) float s_mult[BN];
   __shared__ __attribute__((aligned(16))) float s_bdiv[BN];
-  uint8_t* const sW = smem;                 // [2][kWStage]
-  uint8_t* const sX = smem + 2 * kWStage;   // [2][kXStage]
+  uint8_t* const sW = smem;                      // [kWBufs][kWStage]
+  uint8_t* const sX = smem + kWBufs * kWStage;   // [2][kXStage]
 
   const int t = threadIdx.x;
   const int lane = t % kWave, wave = t / kWave;
@@ -354,8 +366,23 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   }
 
   // ---- staging assignments (weight rows past N are clamped: never stored)
-  const uint8_t* wsrc[NW];
-  int wdst[NW];
+  const uint8_t* wsrc[NW > 0 ? NW : 1];
+  int wdst[NW > 0 ? NW : 1];
+  // direct copies: item it = wave + i*NWAVES -> k-chunk it & 3, 64-row group it >> 2
+  const uint8_t* wdma_src[NWI > 0 ? NWI : 1];
+  int wdma_dst[NWI > 0 ? NWI : 1];
+  if constexpr (WDMA) {
+#pragma unroll
+    for (int i = 0; i < NWI; ++i) {
+      const int it = wave + i * NWAVES;
+      const int kcl = it & 3, rg = it >> 2;
+      const int row = rg * 64 + lane;
+      int64_t nb = n0 / 16 + (row >> 4);
+      nb = nb < NB ? nb : NB - 1;
+      wdma_src[i] = a.w_packed + (nb * a.w_kchunks + kcl) * 256 + (row & 15) * 16;
+      wdma_dst[i] = (kcl * BN + rg * 64) * 16;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < NW; ++i) {
     const int id = t + i * NT;
@@ -372,14 +399,31 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     const int id = t + i * NT;
     const int row = id >> 2, c = id & 3;
     xl[i].init(xsrc, m0 + row, a.M);
-    xdst[i] = 2 * kWStage + row * kBK + ((c ^ x_swizzle(row)) << 4);
+    xdst[i] = kWBufs * kWStage + row * kBK + ((c ^ x_swizzle(row)) << 4);
   }
   KCursor<XSRC> kcur;
   kcur.init(xsrc, t & 3);
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
 
-  v4i wreg[NSET][NW], xreg[NSET][NX];
+  v4i wreg[NSET][NW > 0 ? NW : 1], xreg[NSET][NX];
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  // i-th direct weight copy of stage kt into weight buffer wbuf
+  // Issued through inline assembly on purpose: for the builtin the compiler
+  // assumes that every later LDS read may alias the copy and drains all
+  // outstanding loads (vmcnt(0)) before it, which serialises the pipeline.  The
+  // waits that these copies need are the explicit ones in stage() below.
+  auto dma_one = [&](int kt, int wbuf, int i) {
+    const uint8_t* src = wdma_src[i] + static_cast<int64_t>(kt) * (kChunks * 256);
+    // wave-uniform by construction; the compiler has to be told
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>((lptr_t)(sW + wbuf * kWStage + wdma_dst[i]))));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(src), "s"(dst)
+                 : "memory", "m0");
+  };
   // k-th global load of a stage (weights first, then activations)
   auto load_one = [&](int set, int kt, int k) {
     if (k < NW)
@@ -432,46 +476,71 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   const int xswz = x_swizzle(li);
   v4i wf0[TN], xf0[TM], wf1[TN], xf1[TM];
   // j-th fragment read of a k-step (weights first, then activations)
-  auto read_one = [&](int buf, int s, int j, v4i(&wf)[TN], v4i(&xf)[TM]) {
+  auto read_one = [&](int buf, int wbuf, int s, int j, v4i(&wf)[TN], v4i(&xf)[TM]) {
     const int c = 2 * s + half;
     if (j < TN)
-      wf[j] = ld16(&sW[buf * kWStage + (c * BN + wn0 + j * 32 + li) * 16]);
+      wf[j] = ld16(&sW[wbuf * kWStage + (c * BN + wn0 + j * 32 + li) * 16]);
     else
       xf[j - TN] = ld16(&sX[buf * kXStage + (wm0 + (j - TN) * 32 + li) * kBK + ((c ^ xswz) << 4)]);
   };
   constexpr int Q = TN * TM;    // MFMAs per k-step
   constexpr int NF = TN + TM;   // fragment reads per k-step
   constexpr int NG = NW + NX;   // global loads (and LDS stores) per stage
+  // With WDMA the weight buffer of stage s is s % 3 (wb tracks it), the second
+  // half also issues the direct copies of stage t+3 into buffer t % 3 (dead
+  // since the barrier), and the barrier is preceded by a wait that lets only
+  // this stage's own loads stay outstanding: everything older -- the copies of
+  // stage t+1 among them -- has then landed.
+  int wb = 0;
+  constexpr int kSecond = NF + NG + (WDMA ? NWI : 0);  // operations of the second half
   auto stage = [&](int kt, int load_set, int store_set) {
     const int buf = kt & 1;
     const int kload = clampk(kt + PD);
+    const int wb_cur = WDMA ? wb : buf;
+    const int wb_next = WDMA ? (wb == 2 ? 0 : wb + 1) : (buf ^ 1);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
 #pragma unroll
       for (int o = q * (NF + NG) / Q; o < (q + 1) * (NF + NG) / Q; ++o) {
-        if (o < NF) read_one(buf, 1, o, wf1, xf1);
+        if (o < NF) read_one(buf, wb_cur, 1, o, wf1, xf1);
         else load_one(load_set, kload, o - NF);
       }
       acc[q / TM][q % TM] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf0[q / TM], xf0[q % TM],
                                                                  acc[q / TM][q % TM], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (WDMA) {
+      // at most the loads of this stage and the one before, and the copies issued
+      // half a stage ago, may still be outstanding
+      constexpr int kLeft = 2 * NX + NWI;
+      __builtin_amdgcn_s_waitcnt((kLeft & 15) | ((kLeft >> 4) << 14) | (7 << 4) | (15 << 8));
+    }
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
 #pragma unroll
-      for (int o = q * (NF + NG) / Q; o < (q + 1) * (NF + NG) / Q; ++o) {
-        if (o < NF) read_one(buf ^ 1, 0, o, wf0, xf0);
-        else store_one(store_set, buf, o - NF);
+      for (int o = q * kSecond / Q; o < (q + 1) * kSecond / Q; ++o) {
+        if (o < NF) read_one(buf ^ 1, wb_next, 0, o, wf0, xf0);
+        else if (o < NF + NG) store_one(store_set, buf, o - NF);
+        else dma_one(clampk(kt + 3), wb_cur, o - NF - NG);
       }
       acc[q / TM][q % TM] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf1[q / TM], xf1[q % TM],
                                                                  acc[q / TM][q % TM], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
+    wb = wb_next;
   };
 
-  // prologue: stages 0 and 1 into LDS, stages 2 .. PD-1 in flight
+  // prologue: stages 0 and 1 into LDS, stages 2 .. PD-1 in flight.  The direct
+  // weight copies of stages 0 and 1 go first: the activation stores below wait
+  // for younger loads, which implies that these have landed.
+  if constexpr (WDMA) {
+#pragma unroll
+    for (int i = 0; i < NWI; ++i) dma_one(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NWI; ++i) dma_one(clampk(1), 1, i);
+  }
 #pragma unroll
   for (int k = 0; k < NG; ++k) load_one(0, 0, k);
 #pragma unroll
@@ -485,9 +554,13 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   // (with NSET == 2 the loads of stage 2 reuse set 0, already stored above)
 #pragma unroll
   for (int k = 0; k < NG; ++k) store_one(1 % NSET, 1, k);
+  if constexpr (WDMA) {
+#pragma unroll
+    for (int i = 0; i < NWI; ++i) dma_one(clampk(2), 2, i);
+  }
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < NF; ++j) read_one(0, 0, j, wf0, xf0);
+  for (int j = 0; j < NF; ++j) read_one(0, 0, 0, j, wf0, xf0);
 
   int kt0 = 0;
   for (; kt0 + NSET <= KT; kt0 += NSET) {
@@ -497,6 +570,10 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
 #pragma unroll
   for (int j = 0; j < NSET - 1; ++j)
     if (kt0 + j < KT) stage(kt0 + j, (j + 1) % NSET, (j + 2) % NSET);
+
+  // the last direct copies (past the end of K, never read) must have landed
+  // before the LDS is reused below or handed to another block
+  if constexpr (WDMA) __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
 
   // ---- epilogue.  A lane holds, per 32x32 MFMA tile, channels
   // n = 8g + 4*half + j (g, j < 4) of activation row m = li.

@@ -256,11 +256,11 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
 // Kernel selection override for benchmarking: -1 = automatic.
 std::atomic<int> g_forced_config{-1};
 
-template <int BM, int BN, int WM, int WN, int MODE, int PD = 4>
+template <int BM, int BN, int WM, int WN, int MODE, int PD = 4, bool WDMA = false>
 int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
   if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear, PD>
+  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear, PD, WDMA>
       <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
   return launch_status();
 }
@@ -310,6 +310,8 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 3: return launch_gemm<256, 256, 2, 4, MODE, 3>(a, xs, s);
     case 4: return launch_gemm<128, 256, 2, 2, MODE>(a, xs, s);
     case 5: return launch_gemm<256, 128, 2, 2, MODE>(a, xs, s);
+    case 6: return launch_gemm<256, 256, 2, 4, MODE, 4, true>(a, xs, s);
+    case 7: return launch_gemm<128, 128, 2, 2, MODE, 4, true>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
