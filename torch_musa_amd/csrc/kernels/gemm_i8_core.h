@@ -18,10 +18,13 @@
 // LDS staging (64 k-bytes per stage, two stages):
 //   weights     [k-chunk][row][16 B]      straight copy of the packed layout,
 //                                         lanes read consecutive 16-byte slots
-//   activations [row][64 B], the 16-byte slot index XOR-ed with
-//               ((row >> 1) ^ (row >> 3)) & 3, so that both the row-major fill
-//               and the column-wise operand reads of any 8 or 16 consecutive
-//               lanes fall into distinct 16-byte bank groups
+//   activations [row][64 B], the 16-byte slot index XOR-ed with (row >> 2) & 3:
+//               rows r, r+4, r+8, r+12 start on the same bank and the XOR moves
+//               them to four different 16-byte bank groups.  Measured on the
+//               chip: column-wise ds_read_b128 of 32 rows runs at 224 B/clk per
+//               CU with this swizzle (as fast as consecutive addresses), at
+//               128 B/clk with XORs built from (row >> 1) or (row >> 3), and at
+//               64 B/clk with none
 // Pipeline: see the comment at the software pipeline inside gemm_i8_kernel.
 #pragma once
 
@@ -203,7 +206,7 @@ struct KCursor<XConv> {
 };
 
 // Slot swizzle of the activation stage: see the file header.
-__device__ __forceinline__ int x_swizzle(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
+__device__ __forceinline__ int x_swizzle(int row) { return (row >> 2) & 3; }
 
 // One requantised byte group: four consecutive channels of one output row.
 // CLAMP = false (unsigned output, bounds 0 and 255 only): the packing
@@ -280,35 +283,46 @@ __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv,
 // stages: the global loads of stage t+PD are issued while stage t is being
 // multiplied, so PD-1 stages of 16-byte loads are in flight per thread.
 //
-// WDMA = true: the weight stages do not pass through registers.  Each wave
-// copies 64 rows x 16 bytes per instruction straight from the packed weight
-// into LDS (global_load_lds_dwordx4), three stages ahead, into one of three
-// weight buffers; only the activations are staged through registers (they
-// need the sign-bit flip on the way).  This halves the LDS store traffic of
-// the loop and frees the weight staging registers.
+// WDMA = true (quantized::linear only): no operand passes through registers on
+// its way to LDS.  Each wave copies 1 KB per instruction straight from global
+// memory into LDS (global_load_lds_dwordx4: lane L's 16 bytes land in slot L
+// of the 1 KB destination), kDmaBufs stages ahead, into a ring of kDmaBufs
+// buffers; the sign-bit flip of unsigned activations is applied to the
+// fragments after they are read from LDS.  Register staging costs the matrix
+// pipe about a quarter of its time on this chip: the ds_write_b128 traffic of
+// eight waves, mixed with their fragment reads, backs up the LDS queue and the
+// fragment reads behind it.
 template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4, bool WDMA = false>
-__global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
+__global__ __launch_bounds__(WM* WN* kWave, (WDMA && WM * WN == 4 && (BM / WM) * (BN / WN) <= 128 * 64) ? 2 : 1)
+void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int NT = WM * WN * kWave;
   constexpr bool kHasPost = XSRC::kPostOps;  // residual / activation epilogue compiled in
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int NW = WDMA ? 0 : BN * kChunks / NT;  // 16-byte weight chunks per thread per stage
+  constexpr int NW = BN * kChunks / NT;  // 16-byte weight chunks per thread per stage
   constexpr int NX = BM * kChunks / NT;
   constexpr int NWAVES = WM * WN;
-  constexpr int NWI = kChunks * (BN / 64) / NWAVES;  // direct-to-LDS weight copies per wave per stage
-  constexpr int kWBufs = WDMA ? 3 : 2;
-  static_assert(!WDMA || (BN % 64 == 0 && kChunks * (BN / 64) % NWAVES == 0), "weight copies do not divide");
   constexpr int NSET = PD - 1;           // register sets holding stages in flight
-  static_assert(TM >= 1 && TN >= 1 && (WDMA || NW >= 1) && NX >= 1, "tile too small for the wave grid");
+  static_assert(TM >= 1 && TN >= 1 && NW >= 1 && NX >= 1, "tile too small for the wave grid");
   static_assert(BN * kChunks % NT == 0 && BM * kChunks % NT == 0, "uneven staging");
-  static_assert(!WDMA || PD == 4, "the explicit load-counter waits assume prefetch distance 4");
   static_assert(PD >= 3, "prefetch distance");
+  // direct copies: 1 KB (64 weight rows of one k-chunk, or 16 activation rows) each
+  constexpr int kDmaBufs = PD;
+  constexpr int NDW = kChunks * (BN / 64) / NWAVES;  // weight copies per wave per stage
+  constexpr int NDX = (BM / 16) / NWAVES;            // activation copies per wave per stage
+  constexpr int ND = NDW + NDX;
+  static_assert(!WDMA || std::is_same<XSRC, XLinear>::value, "direct copies need plain activation rows");
+  static_assert(!WDMA || (BN % 64 == 0 && kChunks * (BN / 64) % NWAVES == 0 && BM % 16 == 0 &&
+                          (BM / 16) % NWAVES == 0),
+                "direct copies do not divide among the waves");
+  static_assert(!WDMA || (TN + TM <= TN * TM && ND <= TN * TM), "one LDS read and one copy per MFMA at most");
+  constexpr int kWBufs = WDMA ? kDmaBufs : 2, kXBufs = WDMA ? kDmaBufs : 2;
 
   // LDS: two stages of {weights, activations}; the same bytes are reused after
   // the main loop to transpose the output tile into row-major order.
   constexpr int kWStage = kChunks * BN * 16, kXStage = BM * kBK;
   constexpr int kOutPitch = BN + 16;  // bytes; keeps rows 16-byte aligned and off one bank
-  constexpr int kMainBytes = kWBufs * kWStage + 2 * kXStage;
+  constexpr int kMainBytes = kWBufs * kWStage + kXBufs * kXStage;
   constexpr int kOutBytes = (MODE == kOutAcc32) ? 0 : BM * kOutPitch;
   constexpr int kTileBytes = kMainBytes > kOutBytes ? kMainBytes : kOutBytes;
   __shared__ __attribute__((aligned(16))) uint8_t smem[kTileBytes];
@@ -316,7 +330,7 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   __shared__ __attribute__((aligned(16))) float s_mult[BN];
   __shared__ __attribute__((aligned(16))) float s_bdiv[BN];
   uint8_t* const sW = smem;                      // [kWBufs][kWStage]
-  uint8_t* const sX = smem + kWBufs * kWStage;   // [2][kXStage]
+  uint8_t* const sX = smem + kWBufs * kWStage;   // [kXBufs][kXStage]
 
   const int t = threadIdx.x;
   const int lane = t % kWave, wave = t / kWave;
@@ -346,43 +360,191 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   const int64_t n0 = (gfirst + in_group % gwidth) * BN;
   const int64_t NB = ceil_div(a.N, 16);
 
-  // ---- per-channel constants of this tile's BN output channels
-  for (int i = t; i < BN; i += NT) {
-    const int64_t n = n0 + i;
-    int acc0 = 0;
-    float mult = 0.f, bdiv = 0.f;
-    if (n < a.N) {
-      const int64_t np = n + a.n_off;
-      acc0 = a.acc_coef * a.colsum[np];
-      if (MODE != kOutAcc32) {
-        const float atw = a.x_scale * a.w_scales[np * a.w_scale_stride];
-        mult = atw / a.out_scale;
-        bdiv = a.bias != nullptr ? a.bias[np] / atw : 0.f;
+  // ---- per-channel constants of this tile's BN output channels, then the
+  // accumulators' start value (see file header).  Called once per tile, after
+  // the first operand copies are on their way.
+  v16i acc[TN][TM];
+  auto init_tile = [&]() {
+    for (int i = t; i < BN; i += NT) {
+      const int64_t n = n0 + i;
+      int acc0 = 0;
+      float mult = 0.f, bdiv = 0.f;
+      if (n < a.N) {
+        const int64_t np = n + a.n_off;
+        acc0 = a.acc_coef * a.colsum[np];
+        if (MODE != kOutAcc32) {
+          const float atw = a.x_scale * a.w_scales[np * a.w_scale_stride];
+          mult = atw / a.out_scale;
+          bdiv = a.bias != nullptr ? a.bias[np] / atw : 0.f;
+        }
       }
+      s_acc0[i] = acc0;
+      s_mult[i] = mult;
+      s_bdiv[i] = bdiv;
     }
-    s_acc0[i] = acc0;
-    s_mult[i] = mult;
-    s_bdiv[i] = bdiv;
-  }
-
-  // ---- staging assignments (weight rows past N are clamped: never stored)
-  const uint8_t* wsrc[NW > 0 ? NW : 1];
-  int wdst[NW > 0 ? NW : 1];
-  // direct copies: item it = wave + i*NWAVES -> k-chunk it & 3, 64-row group it >> 2
-  const uint8_t* wdma_src[NWI > 0 ? NWI : 1];
-  int wdma_dst[NWI > 0 ? NWI : 1];
-  if constexpr (WDMA) {
+    __syncthreads();  // s_acc0 / s_mult / s_bdiv are written
 #pragma unroll
-    for (int i = 0; i < NWI; ++i) {
-      const int it = wave + i * NWAVES;
-      const int kcl = it & 3, rg = it >> 2;
-      const int row = rg * 64 + lane;
-      int64_t nb = n0 / 16 + (row >> 4);
-      nb = nb < NB ? nb : NB - 1;
-      wdma_src[i] = a.w_packed + (nb * a.w_kchunks + kcl) * 256 + (row & 15) * 16;
-      wdma_dst[i] = (kcl * BN + rg * 64) * 16;
+    for (int tn = 0; tn < TN; ++tn) {
+      v16i init;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        init[r] = s_acc0[wn0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3)];
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = init;
     }
-  }
+  };
+
+  const int KT = static_cast<int>(ceil_div(a.K, kBK));
+  auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };
+  const int xswz = x_swizzle(li);
+  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
+                     static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
+  v4i wf0[TN], xf0[TM], wf1[TN], xf1[TM];
+  // j-th fragment read of k-step s (weights first, then activations)
+  auto read_one = [&](int wbuf, int xbuf, int s, int j, v4i(&wf)[TN], v4i(&xf)[TM]) {
+    const int c = 2 * s + half;
+    if (j < TN)
+      wf[j] = ld16(&sW[wbuf * kWStage + (c * BN + wn0 + j * 32 + li) * 16]);
+    else
+      xf[j - TN] = ld16(&sX[xbuf * kXStage + (wm0 + (j - TN) * 32 + li) * kBK + ((c ^ xswz) << 4)]);
+  };
+  constexpr int Q = TN * TM;    // MFMAs per k-step
+  constexpr int NF = TN + TM;   // fragment reads per k-step
+  auto mfma = [&](int q, const v4i(&wf)[TN], const v4i(&xf)[TM]) {
+    acc[q / TM][q % TM] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[q / TM], xf[q % TM],
+                                                               acc[q / TM][q % TM], 0, 0, 0);
+  };
+
+  if constexpr (WDMA) {
+    // ---- direct-copy pipeline.  Stage s lives in buffer s % kDmaBufs.  The
+    // schedule of stage t, one LDS or copy operation per MFMA:
+    //   first half   MFMAs of k-step 0 + LDS reads of the k-step 1 fragments
+    //   wait + barrier: stage t+1 has landed for every wave; buffer t % kDmaBufs
+    //                is dead (its last reads were waited for before the barrier)
+    //   second half  MFMAs of k-step 1 + LDS reads of the k-step 0 fragments of
+    //                stage t+1 + this wave's copies of stage t+kDmaBufs into the
+    //                dead buffer
+    // Activation fragments get their sign-bit flip one MFMA ahead of their
+    // first use, so that the flip never sits between a barrier and an MFMA.
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    // Every copy is "uniform 64-bit base + per-lane 32-bit offset" on the global
+    // side and a wave-uniform LDS address in M0 on the other: per stage only the
+    // scalar bases move, no vector instruction is spent on addresses.  The host
+    // keeps 256 rows of either operand within 32 bits of the tile's base.
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t lds0 =
+        __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)smem)));
+    // weight copy i of wave w: k-chunk w & 3, 64-row group (w >> 2) + i * NWAVES / 4
+    static_assert(NWAVES % 4 == 0, "weight copies: one k-chunk per wave");
+    const uint8_t* const wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
+    const int64_t nb_last = NB - 1 - n0 / 16;  // rows past N: clamped, never stored
+    uint32_t wdma_off[NDW];
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) {
+      const int rg = (wave_u >> 2) + i * (NWAVES / 4);
+      int64_t rb = rg * 4 + (lane >> 4);
+      rb = rb < nb_last ? rb : nb_last;
+      wdma_off[i] = static_cast<uint32_t>((rb * a.w_kchunks + (wave_u & 3)) * 256 + (lane & 15) * 16);
+    }
+    const uint32_t wdma_lds = lds0 + ((wave_u & 3) * BN + (wave_u >> 2) * 64) * 16;
+    // activation copy i of wave w: rows 16 (w + i NWAVES) .. + 15, four lanes per
+    // row; the lane of slot sl fetches the k-chunk that the swizzle puts there
+    const uint8_t* const xtile = xsrc.x + m0 * xsrc.ldx;
+    const int64_t m_last = a.M - 1 - m0;
+    const int ktail = static_cast<int>(a.K) - 16 - (KT - 1) * kBK;  // last chunk inside K of the last stage
+    uint32_t xdma_off[NDX], xdma_off_last[NDX];
+#pragma unroll
+    for (int i = 0; i < NDX; ++i) {
+      const int row = (wave_u + i * NWAVES) * 16 + (lane >> 2);
+      const int64_t r = row < m_last ? row : m_last;
+      const int kc = ((lane & 3) ^ x_swizzle(row)) * 16;
+      xdma_off[i] = static_cast<uint32_t>(r * xsrc.ldx + kc);
+      // chunks past K: any valid bytes will do, the packed weight is zero there
+      xdma_off_last[i] = static_cast<uint32_t>(r * xsrc.ldx + (kc < ktail ? kc : ktail));
+    }
+    const uint32_t xdma_lds = lds0 + kWBufs * kWStage + wave_u * 1024;
+    // Issued through inline assembly on purpose: for the builtin the compiler
+    // assumes that every later LDS read may alias the copy and drains all
+    // outstanding loads before it, which serialises the pipeline.  The waits
+    // that these copies need are the explicit ones below.
+    auto dma = [&](const uint8_t* base, uint32_t off, uint32_t lds_dst) {
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(off), "s"(base), "s"(lds_dst)
+                   : "memory", "m0");
+    };
+    // i-th copy of stage kt into buffer b
+    auto dma_one = [&](int kt, int b, int i) {
+      if (i < NDW) {
+        dma(wtile + static_cast<int64_t>(kt) * (kChunks * 256), wdma_off[i],
+            wdma_lds + b * kWStage + i * (NWAVES / 4) * 64 * 16);
+      } else {
+        const int j = i - NDW;
+        dma(xtile + static_cast<int64_t>(kt) * kBK, kt == KT - 1 ? xdma_off_last[j] : xdma_off[j],
+            xdma_lds + b * kXStage + j * NWAVES * 1024);
+      }
+    };
+    auto wait_loads = [&](auto left_tag) {  // s_waitcnt vmcnt(left) only
+      constexpr int kLeft = decltype(left_tag)::value;
+      static_assert(kLeft < 64, "load counter range");
+      __builtin_amdgcn_s_waitcnt((kLeft & 15) | ((kLeft >> 4) << 14) | (7 << 4) | (15 << 8));
+    };
+    auto flip = [&](v4i& f) { f ^= xmask; };
+    // b = kt % kDmaBufs as a compile-time constant
+    auto stage = [&](int kt, int b) {
+      const int bn = (b + 1) % kDmaBufs;
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        if (q < NF) read_one(b, b, 1, q, wf1, xf1);
+        mfma(q, wf0, xf0);
+        if (q + 1 < TM) flip(xf0[q + 1]);
+        if (q == Q - 1) flip(xf1[0]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // only the copies of stages t+2 .. t+kDmaBufs-1 may still be outstanding
+      wait_loads(std::integral_constant<int, (kDmaBufs - 2) * ND>{});
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      const int kload = clampk(kt + kDmaBufs);
+      // copies go to the MFMA slots that carry no sign flip
+      constexpr int kFirstDma = (TM - 1 < Q - 1 - ND) ? TM - 1 : (Q - 1 - ND > 0 ? Q - 1 - ND : 0);
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        if (q < NF) read_one(bn, bn, 0, q, wf0, xf0);
+        if (q >= kFirstDma && q - kFirstDma < ND) dma_one(kload, b, q - kFirstDma);
+        mfma(q, wf1, xf1);
+        if (q + 1 < TM) flip(xf1[q + 1]);
+        if (q == Q - 1) flip(xf0[0]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // prologue: all buffers in flight, stage 0 landed and visible
+#pragma unroll
+    for (int st = 0; st < kDmaBufs; ++st)
+#pragma unroll
+      for (int i = 0; i < ND; ++i) dma_one(clampk(st), st, i);
+    init_tile();
+    wait_loads(std::integral_constant<int, (kDmaBufs - 1) * ND>{});
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NF; ++j) read_one(0, 0, 0, j, wf0, xf0);
+    flip(xf0[0]);
+    int kt0 = 0;
+    for (; kt0 + kDmaBufs <= KT; kt0 += kDmaBufs) {
+#pragma unroll
+      for (int j = 0; j < kDmaBufs; ++j) stage(kt0 + j, j);
+    }
+#pragma unroll
+    for (int j = 0; j < kDmaBufs - 1; ++j)
+      if (kt0 + j < KT) stage(kt0 + j, j);
+    // the last copies (past the end of K, never read) must have landed before
+    // the LDS is reused below or handed to another block
+    wait_loads(std::integral_constant<int, 0>{});
+  } else {
+  init_tile();
+  // ---- staging assignments (weight rows past N are clamped: never stored)
+  const uint8_t* wsrc[NW];
+  int wdst[NW];
 #pragma unroll
   for (int i = 0; i < NW; ++i) {
     const int id = t + i * NT;
@@ -403,27 +565,8 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   }
   KCursor<XSRC> kcur;
   kcur.init(xsrc, t & 3);
-  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
-                     static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
 
-  v4i wreg[NSET][NW > 0 ? NW : 1], xreg[NSET][NX];
-  typedef const __attribute__((address_space(1))) void* gptr_t;
-  typedef __attribute__((address_space(3))) void* lptr_t;
-  // i-th direct weight copy of stage kt into weight buffer wbuf
-  // Issued through inline assembly on purpose: for the builtin the compiler
-  // assumes that every later LDS read may alias the copy and drains all
-  // outstanding loads (vmcnt(0)) before it, which serialises the pipeline.  The
-  // waits that these copies need are the explicit ones in stage() below.
-  auto dma_one = [&](int kt, int wbuf, int i) {
-    const uint8_t* src = wdma_src[i] + static_cast<int64_t>(kt) * (kChunks * 256);
-    // wave-uniform by construction; the compiler has to be told
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(
-        reinterpret_cast<uintptr_t>((lptr_t)(sW + wbuf * kWStage + wdma_dst[i]))));
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :
-                 : "v"(src), "s"(dst)
-                 : "memory", "m0");
-  };
+  v4i wreg[NSET][NW], xreg[NSET][NX];
   // k-th global load of a stage (weights first, then activations)
   auto load_one = [&](int set, int kt, int k) {
     if (k < NW)
@@ -440,19 +583,6 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
     else
       *reinterpret_cast<v4i*>(&smem[buf * kXStage + xdst[k - NW]]) = xreg[set][k - NW] ^ xmask;
   };
-
-  // ---- accumulators start at the per-channel offset (see file header)
-  __syncthreads();  // s_acc0 / s_mult / s_bdiv are written
-  v16i acc[TN][TM];
-#pragma unroll
-  for (int tn = 0; tn < TN; ++tn) {
-    v16i init;
-#pragma unroll
-    for (int r = 0; r < 16; ++r)
-      init[r] = s_acc0[wn0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3)];
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = init;
-  }
 
   // ---- software pipeline.
   // Stage t of the k loop = 64 k-bytes = two MFMA k-steps.  The schedule of one
@@ -471,76 +601,35 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   // loads stays exact (a predicated load would force it to drain them all).
   // The scheduling fences keep this order; without them the compiler sinks the
   // global loads to the end of the stage and loses the prefetch distance.
-  const int KT = static_cast<int>(ceil_div(a.K, kBK));
-  auto clampk = [&](int kt) { return kt < KT ? kt : KT - 1; };
-  const int xswz = x_swizzle(li);
-  v4i wf0[TN], xf0[TM], wf1[TN], xf1[TM];
-  // j-th fragment read of a k-step (weights first, then activations)
-  auto read_one = [&](int buf, int wbuf, int s, int j, v4i(&wf)[TN], v4i(&xf)[TM]) {
-    const int c = 2 * s + half;
-    if (j < TN)
-      wf[j] = ld16(&sW[wbuf * kWStage + (c * BN + wn0 + j * 32 + li) * 16]);
-    else
-      xf[j - TN] = ld16(&sX[buf * kXStage + (wm0 + (j - TN) * 32 + li) * kBK + ((c ^ xswz) << 4)]);
-  };
-  constexpr int Q = TN * TM;    // MFMAs per k-step
-  constexpr int NF = TN + TM;   // fragment reads per k-step
   constexpr int NG = NW + NX;   // global loads (and LDS stores) per stage
-  // With WDMA the weight buffer of stage s is s % 3 (wb tracks it), the second
-  // half also issues the direct copies of stage t+3 into buffer t % 3 (dead
-  // since the barrier), and the barrier is preceded by a wait that lets only
-  // this stage's own loads stay outstanding: everything older -- the copies of
-  // stage t+1 among them -- has then landed.
-  int wb = 0;
-  constexpr int kSecond = NF + NG + (WDMA ? NWI : 0);  // operations of the second half
   auto stage = [&](int kt, int load_set, int store_set) {
     const int buf = kt & 1;
     const int kload = clampk(kt + PD);
-    const int wb_cur = WDMA ? wb : buf;
-    const int wb_next = WDMA ? (wb == 2 ? 0 : wb + 1) : (buf ^ 1);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
 #pragma unroll
       for (int o = q * (NF + NG) / Q; o < (q + 1) * (NF + NG) / Q; ++o) {
-        if (o < NF) read_one(buf, wb_cur, 1, o, wf1, xf1);
+        if (o < NF) read_one(buf, buf, 1, o, wf1, xf1);
         else load_one(load_set, kload, o - NF);
       }
-      acc[q / TM][q % TM] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf0[q / TM], xf0[q % TM],
-                                                                 acc[q / TM][q % TM], 0, 0, 0);
+      mfma(q, wf0, xf0);
       __builtin_amdgcn_sched_barrier(0);
-    }
-    if constexpr (WDMA) {
-      // at most the loads of this stage and the one before, and the copies issued
-      // half a stage ago, may still be outstanding
-      constexpr int kLeft = 2 * NX + NWI;
-      __builtin_amdgcn_s_waitcnt((kLeft & 15) | ((kLeft >> 4) << 14) | (7 << 4) | (15 << 8));
     }
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
 #pragma unroll
-      for (int o = q * kSecond / Q; o < (q + 1) * kSecond / Q; ++o) {
-        if (o < NF) read_one(buf ^ 1, wb_next, 0, o, wf0, xf0);
-        else if (o < NF + NG) store_one(store_set, buf, o - NF);
-        else dma_one(clampk(kt + 3), wb_cur, o - NF - NG);
+      for (int o = q * (NF + NG) / Q; o < (q + 1) * (NF + NG) / Q; ++o) {
+        if (o < NF) read_one(buf ^ 1, buf ^ 1, 0, o, wf0, xf0);
+        else store_one(store_set, buf, o - NF);
       }
-      acc[q / TM][q % TM] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf1[q / TM], xf1[q % TM],
-                                                                 acc[q / TM][q % TM], 0, 0, 0);
+      mfma(q, wf1, xf1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    wb = wb_next;
   };
 
-  // prologue: stages 0 and 1 into LDS, stages 2 .. PD-1 in flight.  The direct
-  // weight copies of stages 0 and 1 go first: the activation stores below wait
-  // for younger loads, which implies that these have landed.
-  if constexpr (WDMA) {
-#pragma unroll
-    for (int i = 0; i < NWI; ++i) dma_one(0, 0, i);
-#pragma unroll
-    for (int i = 0; i < NWI; ++i) dma_one(clampk(1), 1, i);
-  }
+  // prologue: stages 0 and 1 into LDS, stages 2 .. PD-1 in flight
 #pragma unroll
   for (int k = 0; k < NG; ++k) load_one(0, 0, k);
 #pragma unroll
@@ -554,10 +643,6 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
   // (with NSET == 2 the loads of stage 2 reuse set 0, already stored above)
 #pragma unroll
   for (int k = 0; k < NG; ++k) store_one(1 % NSET, 1, k);
-  if constexpr (WDMA) {
-#pragma unroll
-    for (int i = 0; i < NWI; ++i) dma_one(clampk(2), 2, i);
-  }
   __syncthreads();
 #pragma unroll
   for (int j = 0; j < NF; ++j) read_one(0, 0, 0, j, wf0, xf0);
@@ -570,10 +655,7 @@ __global__ __launch_bounds__(WM* WN* kWave) void gemm_i8_kernel(GemmArgs a, XSRC
 #pragma unroll
   for (int j = 0; j < NSET - 1; ++j)
     if (kt0 + j < KT) stage(kt0 + j, (j + 1) % NSET, (j + 2) % NSET);
-
-  // the last direct copies (past the end of K, never read) must have landed
-  // before the LDS is reused below or handed to another block
-  if constexpr (WDMA) __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
+  }
 
   // ---- epilogue.  A lane holds, per 32x32 MFMA tile, channels
   // n = 8g + 4*half + j (g, j < 4) of activation row m = li.

@@ -297,12 +297,15 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     // largest tile that still leaves at least ~2 blocks per CU, else smaller
     const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
     if (nblk(256, 256) >= 512)
-      cfg = 3;  // 8 waves of 128x64: two waves per SIMD cover each other's waits
+      cfg = 6;  // 8 waves of 128x64, operands copied straight into LDS (3 otherwise, see below)
     else if (nblk(128, 128) >= 256)
       cfg = 1;
     else
       cfg = 2;
   }
+  // the direct-copy kernels address 256 rows of either operand with 32-bit offsets
+  const bool dma_ok = xs.ldx <= (int64_t{1} << 23) && a.K <= (int64_t{1} << 23);
+  if ((cfg == 6 || cfg == 7) && !dma_ok) cfg = 3;
   switch (cfg) {
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
     case 1: return launch_gemm<128, 128, 2, 2, MODE>(a, xs, s);
@@ -310,8 +313,8 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 3: return launch_gemm<256, 256, 2, 4, MODE, 3>(a, xs, s);
     case 4: return launch_gemm<128, 256, 2, 2, MODE>(a, xs, s);
     case 5: return launch_gemm<256, 128, 2, 2, MODE>(a, xs, s);
-    case 6: return launch_gemm<256, 256, 2, 4, MODE, 4, true>(a, xs, s);
-    case 7: return launch_gemm<128, 128, 2, 2, MODE, 4, true>(a, xs, s);
+    case 6: return launch_gemm<256, 256, 2, 4, MODE, 3, true>(a, xs, s);
+    case 7: return launch_gemm<128, 128, 2, 2, MODE, 3, true>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
