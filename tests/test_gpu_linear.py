@@ -76,7 +76,7 @@ def _tile_case(m, n, k, seed, x_signed=False, relu=False, bias=True, per_channel
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
 @pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9])
-@pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168)])
+@pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192)])
 def test_tile_configs(cabi, cfg, shape):
     say("tile cfg", cfg, shape)
     c = _tile_case(*shape, seed=cfg * 10 + shape[0])

@@ -529,11 +529,14 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
 #pragma unroll
     for (int j = 0; j < NF; ++j) read_one(0, 0, 0, j, wf0, xf0);
     flip(xf0[0]);
+    // the host sends only K >= kDmaBufs stages here: a loop that always runs
+    // keeps the prologue's fragments out of the way of the register allocator
     int kt0 = 0;
-    for (; kt0 + kDmaBufs <= KT; kt0 += kDmaBufs) {
+    do {
 #pragma unroll
       for (int j = 0; j < kDmaBufs; ++j) stage(kt0 + j, j);
-    }
+      kt0 += kDmaBufs;
+    } while (kt0 + kDmaBufs <= KT);
 #pragma unroll
     for (int j = 0; j < kDmaBufs - 1; ++j)
       if (kt0 + j < KT) stage(kt0 + j, j);

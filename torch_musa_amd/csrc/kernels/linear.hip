@@ -292,20 +292,24 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     }
     return launch_status();
   }
+  // the direct-copy kernels address 256 rows of either operand with 32-bit offsets
+  // and run their three-stage ring at least once around
+  const bool dma_ok = xs.ldx <= (int64_t{1} << 23) && a.K <= (int64_t{1} << 23) && a.K > 2 * kBK;
   int cfg = forced;
   if (cfg < 0) {
-    // largest tile that still leaves at least ~2 blocks per CU, else smaller
+    // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
+    // 256x256 tile (one block per CU) wins once it keeps about two thirds of
+    // the CUs busy, the 128x128 tile (three blocks per CU) down to 64 tiles.
     const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
-    if (nblk(256, 256) >= 512)
-      cfg = 6;  // 8 waves of 128x64, operands copied straight into LDS (3 otherwise, see below)
-    else if (nblk(128, 128) >= 256)
-      cfg = 1;
+    if (nblk(256, 256) >= 160)
+      cfg = 6;  // 8 waves of 128x64, operands copied straight into LDS
+    else if (nblk(128, 128) >= 64)
+      cfg = 7;
     else
       cfg = 2;
   }
-  // the direct-copy kernels address 256 rows of either operand with 32-bit offsets
-  const bool dma_ok = xs.ldx <= (int64_t{1} << 23) && a.K <= (int64_t{1} << 23);
-  if ((cfg == 6 || cfg == 7) && !dma_ok) cfg = 3;
+  if (cfg == 6 && !dma_ok) cfg = 3;
+  if (cfg == 7 && !dma_ok) cfg = 1;
   switch (cfg) {
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
     case 1: return launch_gemm<128, 128, 2, 2, MODE>(a, xs, s);
