@@ -307,6 +307,16 @@ int tmq_qmaxpool2d(const void* x, void* y, int64_t B, int64_t H, int64_t W, int6
                    int32_t dil_h, int32_t dil_w, int64_t OH, int64_t OW, int q_signed,
                    tmq_stream_t stream);
 
+/* Adaptive average pooling over NHWC codes (replaces AdaptiveAvgPool2dQuantized /
+ * QuantizedAvgPool2dImpl, torch_musa/csrc/aten/quantized/Pool.cpp:93-127,132-176,
+ * muDNN Pooling ADAPTIVE_AVGPOOL).  Output pixel (oh, ow) covers input rows
+ * floor(oh*H/OH) .. ceil((oh+1)*H/OH)-1 and the like columns; scale and zero
+ * point carry over:
+ *   acc = sum(q) - zero_point * count;  q' = clamp(rne(float(acc) * (1.0f / count)) + zero_point) */
+int tmq_qadaptive_avgpool2d(const void* x, void* y, int64_t B, int64_t H, int64_t W, int64_t C,
+                            int64_t OH, int64_t OW, int32_t zero_point, int q_signed,
+                            tmq_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * Measurement probe (no counterpart in the reference; used by bench.py only).
  * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four

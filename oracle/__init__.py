@@ -341,6 +341,16 @@ def qmaxpool2d(x_nhwc, kernel, stride, padding, dilation=(1, 1), ceil_mode=False
     return y
 
 
+def qadaptive_avgpool2d(x_nhwc, out_hw, zero_point):
+    """adaptive_avg_pool2d of per-tensor quantized NHWC codes; qparams carry over."""
+    x = _as_bytes(x_nhwc)
+    b, h, w, c = x.shape
+    y = np.empty((b, out_hw[0], out_hw[1], c), dtype=x.dtype)
+    lib().orc_qadaptive_avgpool2d(_p(x), *[C.c_int64(v) for v in (b, h, w, c, out_hw[0], out_hw[1], zero_point)],
+                                  C.c_int(x.dtype == np.int8), _p(y))
+    return y
+
+
 def qcat(qs, scales, zps, axis, out_scale, out_zp):
     """quantized::cat: every input dequantized and requantized to the output's
     parameters (the composition PyTorch's CPU op performs), then concatenated."""

@@ -549,3 +549,34 @@ ORC_API void orc_qmaxpool2d(const uint8_t* x, int64_t B, int64_t H, int64_t W, i
           y[((b * OH + oh) * OW + ow) * C + c] = (uint8_t)m;
         }
 }
+
+/* Adaptive average pooling over NHWC codes (reference Pool.cpp:132-176 hands it
+ * to muDNN; numerics of PyTorch's CPU op, qadaptive_avg_pool2d_nhwc_kernel in
+ * aten/src/ATen/native/quantized/cpu/kernels/QuantizedOpKernels.cpp): window
+ * rows floor(oh*H/OH) .. ceil((oh+1)*H/OH)-1, int32 sum minus zp * count, times
+ * fl(1 / count) in fp32, round half to even, plus zp, clamp. */
+ORC_API void orc_qadaptive_avgpool2d(const uint8_t* x, int64_t B, int64_t H, int64_t W, int64_t C,
+                                     int64_t OH, int64_t OW, int64_t zp, int is_signed, uint8_t* y) {
+  const int32_t lo = is_signed ? -128 : 0, hi = is_signed ? 127 : 255;
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t oh = 0; oh < OH; ++oh) {
+      const int64_t h0 = (oh * H) / OH, h1 = ((oh + 1) * H + OH - 1) / OH;
+      for (int64_t ow = 0; ow < OW; ++ow) {
+        const int64_t w0 = (ow * W) / OW, w1 = ((ow + 1) * W + OW - 1) / OW;
+        const int32_t count = (int32_t)((h1 - h0) * (w1 - w0));
+        const float mult = 1.0f / (float)count;
+        for (int64_t c = 0; c < C; ++c) {
+          int32_t acc = -(int32_t)zp * count;
+          for (int64_t ih = h0; ih < h1; ++ih)
+            for (int64_t iw = w0; iw < w1; ++iw) {
+              const uint8_t byte = x[((b * H + ih) * W + iw) * C + c];
+              acc += is_signed ? (int32_t)(int8_t)byte : (int32_t)byte;
+            }
+          const float v = (float)acc * mult;
+          int32_t q = (int32_t)nearbyintf(v) + (int32_t)zp;
+          q = q < lo ? lo : (q > hi ? hi : q);
+          y[((b * OH + oh) * OW + ow) * C + c] = (uint8_t)q;
+        }
+      }
+    }
+}

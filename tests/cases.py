@@ -370,3 +370,22 @@ def qmaxpool_cases():
         out.append(dict(name=name, x=rng.integers(lo, hi, shape).astype(np.int8 if signed else np.uint8),
                         kernel=k, stride=s, padding=p, dilation=d, ceil_mode=ceil_mode, signed=signed))
     return out
+
+
+def qavgpool_cases():
+    spec = [
+        # name, (B, H, W, C), (OH, OW), zero point, signed
+        ("global_7x7_c64", (2, 7, 7, 64), (1, 1), 120, False),
+        ("ties_4x4_to_2x2_c8", (2, 4, 4, 8), (2, 2), 3, False),
+        ("ragged_13x9_to_5x3_c48", (2, 13, 9, 48), (5, 3), 77, False),
+        ("c7_10x11_to_3x4_s8", (1, 10, 11, 7), (3, 4), -9, True),
+        ("upsample_3x3_to_5x5_c4", (1, 3, 3, 4), (5, 5), 0, False),
+        ("global_14x14_c130_s8", (1, 14, 14, 130), (1, 1), 5, True),
+    ]
+    out = []
+    for i, (name, shape, ohw, zp, signed) in enumerate(spec):
+        rng = np.random.default_rng(1600 + i)
+        lo, hi = (-128, 128) if signed else (0, 256)
+        out.append(dict(name=name, x=rng.integers(lo, hi, shape).astype(np.int8 if signed else np.uint8),
+                        out_hw=ohw, zp=zp, signed=signed))
+    return out

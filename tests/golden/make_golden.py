@@ -199,6 +199,16 @@ def main():
         g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
         g[k + "/y"] = y.int_repr().permute(0, 2, 3, 1).contiguous().numpy()
 
+    for c in cases.qavgpool_cases():
+        xq = torch._make_per_tensor_quantized_tensor(
+            torch.from_numpy(c["x"]).permute(0, 3, 1, 2).contiguous(memory_format=torch.channels_last),
+            0.05, c["zp"])
+        y = torch.nn.functional.adaptive_avg_pool2d(xq, c["out_hw"])
+        assert y.q_scale() == xq.q_scale() and y.q_zero_point() == c["zp"]
+        k = "qavgpool/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/y"] = y.int_repr().permute(0, 2, 3, 1).contiguous().numpy()
+
     # ---- quantized::conv2d -------------------------------------------------
     for c in cases.conv_cases():
         x_nchw = torch.from_numpy(c["xq"]).permute(0, 3, 1, 2)  # channels-last view

@@ -446,3 +446,17 @@ def test_residual_block_end_to_end():
     # one LSB per requantisation boundary crossed; a second-layer value may move
     # by one more when its input moved
     assert d.max() <= 2 and (d > 1).float().mean() < 1e-3 and (d > 0).float().mean() < 0.02, (d.max(), (d > 0).float().mean())
+
+
+@pytest.mark.parametrize("c", cases.qavgpool_cases(), ids=lambda c: c["name"])
+def test_adaptive_avg_pool2d_op(golden, c):
+    say("aten adaptive_avg_pool2d", c["name"])
+    x_nchw = torch.from_numpy(c["x"]).permute(0, 3, 1, 2)
+    xq = torch._make_per_tensor_quantized_tensor(x_nchw.contiguous().cuda(), 0.05, c["zp"])
+    for inp in (xq, xq.contiguous(memory_format=torch.channels_last)):
+        y = torch.nn.functional.adaptive_avg_pool2d(inp, c["out_hw"])
+        assert y.is_quantized and y.q_scale() == 0.05 and y.q_zero_point() == c["zp"]
+        np.testing.assert_array_equal(y.int_repr().permute(0, 2, 3, 1).contiguous().cpu().numpy(),
+                                      golden["qavgpool/" + c["name"] + "/y"])
+    m = torch.nn.AdaptiveAvgPool2d(c["out_hw"])
+    np.testing.assert_array_equal(m(xq).int_repr().cpu().numpy(), y.int_repr().cpu().numpy())

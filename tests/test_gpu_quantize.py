@@ -258,3 +258,20 @@ def test_qmaxpool_resnet_stem_sized(cabi):
     r = np.maximum(np.maximum(xp[:, 0:-2:2], xp[:, 1:-1:2]), xp[:, 2::2])
     want = np.maximum(np.maximum(r[:, :, 0:-2:2], r[:, :, 1:-1:2]), r[:, :, 2::2])
     np.testing.assert_array_equal(y, want[:, :56, :56])
+
+
+@pytest.mark.parametrize("c", cases.qavgpool_cases(), ids=lambda c: c["name"])
+def test_qadaptive_avgpool2d(cabi, golden, c):
+    say("qavgpool", c["name"])
+    want = golden["qavgpool/" + c["name"] + "/y"]
+    y = host(cabi.qadaptive_avgpool2d(dev(c["x"]), c["out_hw"], c["zp"]))
+    np.testing.assert_array_equal(y, want)
+    np.testing.assert_array_equal(y, oracle.qadaptive_avgpool2d(c["x"], c["out_hw"], c["zp"]))
+
+
+def test_qadaptive_avgpool_resnet_head_sized(cabi):
+    # [64, 7, 7, 2048] -> [64, 1, 1, 2048]: bit-exact against the oracle
+    say("qavgpool head")
+    x = np.random.default_rng(5).integers(0, 256, (64, 7, 7, 2048)).astype(np.uint8)
+    y = host(cabi.qadaptive_avgpool2d(dev(x), (1, 1), 128))
+    np.testing.assert_array_equal(y, oracle.qadaptive_avgpool2d(x, (1, 1), 128))

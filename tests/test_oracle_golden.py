@@ -165,3 +165,11 @@ def test_qmaxpool2d(golden, c):
     _check_crc(golden, k + "/x_crc", c["x"])
     y = oracle.qmaxpool2d(c["x"], c["kernel"], c["stride"], c["padding"], c["dilation"], c["ceil_mode"])
     np.testing.assert_array_equal(y, golden[k + "/y"])
+
+
+@pytest.mark.parametrize("c", cases.qavgpool_cases(), ids=lambda c: c["name"])
+def test_qadaptive_avgpool2d(golden, c):
+    k = "qavgpool/" + c["name"]
+    assert int(golden[k + "/x_crc"]) == cases.crc(c["x"])
+    y = oracle.qadaptive_avgpool2d(c["x"], c["out_hw"], c["zp"])
+    np.testing.assert_array_equal(y, golden[k + "/y"])

@@ -301,3 +301,23 @@ def test_qcat_with_equal_parameters_is_concatenation():
     # scale ratio 2 with zero points 0: codes halve (ties to even)
     y = oracle.qcat([a], [0.25], [0], 0, 0.5, 0)
     np.testing.assert_array_equal(y, np.rint(a / 2.0).astype(np.uint8))
+
+
+def test_qadaptive_avgpool_identity_constant_and_exact_means():
+    rng = np.random.default_rng(77)
+    x = rng.integers(0, 256, (2, 6, 5, 9)).astype(np.uint8)
+    # output grid = input grid: every window is one pixel
+    np.testing.assert_array_equal(oracle.qadaptive_avgpool2d(x, (6, 5), 17), x)
+    # a constant image stays constant whatever the windows and the zero point
+    k = np.full((1, 7, 9, 3), 201, np.uint8)
+    np.testing.assert_array_equal(oracle.qadaptive_avgpool2d(k, (3, 4), 250), np.full((1, 3, 4, 3), 201, np.uint8))
+    # 2x2 windows: sums of four codes; exact quarters, ties to even (brute force in integers)
+    x2 = rng.integers(-128, 128, (1, 4, 6, 2)).astype(np.int8)
+    zp = -3
+    s = x2.astype(np.int64).reshape(1, 2, 2, 3, 2, 2).sum(axis=(2, 4)) - 4 * zp
+    q, r = np.divmod(s, 4)
+    want = q + (r > 2) + ((r == 2) & (q % 2 == 1)) + zp       # round half to even of s / 4
+    np.testing.assert_array_equal(oracle.qadaptive_avgpool2d(x2, (2, 3), zp), np.clip(want, -128, 127).astype(np.int8))
+    # window bounds: 10 rows -> 3 outputs use rows [0,4) [3,7) [6,10)
+    ramp = np.arange(10, dtype=np.uint8).reshape(1, 10, 1, 1) * 10
+    np.testing.assert_array_equal(oracle.qadaptive_avgpool2d(ramp, (3, 1), 0).ravel(), [15, 45, 75])

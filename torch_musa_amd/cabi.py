@@ -27,7 +27,7 @@ DECLARED_SYMBOLS = [
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
-    "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d",
+    "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d",
     "tmq_probe_mfma_i8",
 ]
 
@@ -129,6 +129,7 @@ def lib() -> C.CDLL:
         l.tmq_qcat_rows.argtypes = [v, v, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int32,
                                     C.c_float, C.c_int32, C.c_int, v]
         l.tmq_qmaxpool2d.argtypes = [v, v] + [C.c_int64] * 4 + [C.c_int32] * 8 + [C.c_int64] * 2 + [C.c_int, v]
+        l.tmq_qadaptive_avgpool2d.argtypes = [v, v] + [C.c_int64] * 6 + [C.c_int32, C.c_int, v]
         l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, v, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]
         _lib = l
@@ -500,6 +501,16 @@ def qmaxpool2d(x_nhwc, kernel, stride, padding, dilation, out_hw):
     check(lib().tmq_qmaxpool2d(x_nhwc.data_ptr(), y.data_ptr(), b, h, w, c, kernel[0], kernel[1], stride[0],
                                stride[1], padding[0], padding[1], dilation[0], dilation[1], out_hw[0],
                                out_hw[1], int(x_nhwc.dtype == torch.int8), stream_ptr()), "tmq_qmaxpool2d")
+    return y
+
+
+def qadaptive_avgpool2d(x_nhwc, out_hw, zero_point):
+    assert x_nhwc.is_contiguous()
+    b, h, w, c = x_nhwc.shape
+    y = torch.empty((b, out_hw[0], out_hw[1], c), dtype=x_nhwc.dtype, device=x_nhwc.device)
+    check(lib().tmq_qadaptive_avgpool2d(x_nhwc.data_ptr(), y.data_ptr(), b, h, w, c, out_hw[0], out_hw[1],
+                                        zero_point, int(x_nhwc.dtype == torch.int8), stream_ptr()),
+          "tmq_qadaptive_avgpool2d")
     return y
 
 

@@ -727,6 +727,31 @@ at::Tensor qmaxpool2d_run(const at::Tensor& input, at::IntArrayRef kernel_size, 
   return input.dim() == 3 ? y.squeeze(0) : y;
 }
 
+// aten::_adaptive_avg_pool2d on quantized GPU tensors (reference:
+// AdaptiveAvgPool2dQuantized, torch_musa/csrc/aten/quantized/Pool.cpp:132-176).
+// The result keeps the input's scale and zero point and comes back channels-last.
+at::Tensor qadaptive_avgpool2d_run(const at::Tensor& input, c10::SymIntArrayRef output_size_sym) {
+  TORCH_CHECK(input.qscheme() == c10::kPerTensorAffine || input.qscheme() == c10::kPerTensorSymmetric,
+              "AdaptiveAvgPool2dQuantized only supports per tensor quantized tensors");
+  TORCH_CHECK(output_size_sym.size() == 2, "AdaptiveAvgPool2d only supports output with 2-elements");
+  const bool sgn = is_signed_qtype(input.scalar_type(), "adaptive_avg_pool2d");
+  TORCH_CHECK(input.dim() == 3 || input.dim() == 4, "adaptive_avg_pool2d: expected a 3-D or 4-D input");
+  const int64_t OH = output_size_sym[0].expect_int(), OW = output_size_sym[1].expect_int();
+  TORCH_CHECK(OH >= 0 && OW >= 0, "adaptive_avg_pool2d: output sizes must be non-negative");
+  const c10::OptionalDeviceGuard guard(at::device_of(input));
+  const at::Tensor x4 = input.dim() == 3 ? input.unsqueeze(0) : input;
+  TORCH_CHECK(x4.size(2) > 0 && x4.size(3) > 0, "adaptive_avg_pool2d: input spatial sizes must be positive");
+  const at::Tensor x = x4.contiguous(c10::MemoryFormat::ChannelsLast);
+  const int64_t B = x.size(0), C = x.size(1), H = x.size(2), W = x.size(3);
+  at::Tensor y = at::_empty_affine_quantized({B, C, OH, OW}, x.options(), input.q_scale(), input.q_zero_point(),
+                                             c10::MemoryFormat::ChannelsLast);
+  if (y.numel() > 0)
+    check_status(tmq_qadaptive_avgpool2d(x.data_ptr(), y.data_ptr(), B, H, W, C, OH, OW,
+                                         static_cast<int32_t>(input.q_zero_point()), sgn, current_stream(x)),
+                 "tmq_qadaptive_avgpool2d");
+  return input.dim() == 3 ? y.squeeze(0) : y;
+}
+
 }  // namespace
 
 // The two SiLU schemas are not part of upstream PyTorch; the reference adds them
@@ -782,6 +807,7 @@ TORCH_LIBRARY_IMPL(aten, CUDA, m) {
 TORCH_LIBRARY_IMPL(aten, QuantizedCUDA, m) {
   m.impl("relu", TORCH_FN(qrelu_run));
   m.impl("quantized_max_pool2d", TORCH_FN(qmaxpool2d_run));
+  m.impl("_adaptive_avg_pool2d", TORCH_FN(qadaptive_avgpool2d_run));
 }
 
 namespace {

@@ -269,6 +269,62 @@ __global__ __launch_bounds__(kEwThreads) void qmaxpool_kernel(const uint8_t* __r
   }
 }
 
+// Adaptive average pooling: output pixel (oh, ow) averages the input window
+// rows floor(oh*H/OH) .. ceil((oh+1)*H/OH)-1 (likewise columns).  VEC = 4: a
+// thread owns four consecutive channels (one 32-bit word per input pixel).
+template <bool SIGNED, int VEC>
+__global__ __launch_bounds__(kEwThreads) void qadaptive_avgpool_kernel(const uint8_t* __restrict__ x,
+                                                                       uint8_t* __restrict__ y, PoolShape s,
+                                                                       int32_t zp) {
+  const int64_t cv = ceil_div(s.C, static_cast<int64_t>(VEC));
+  const int64_t total = s.B * s.OH * s.OW * cv;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kEwThreads;
+  const float lo = SIGNED ? -128.f : 0.f, hi = SIGNED ? 127.f : 255.f;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kEwThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t c = (i % cv) * VEC;
+    int64_t t = i / cv;
+    const int64_t ow = t % s.OW;
+    t /= s.OW;
+    const int64_t oh = t % s.OH, b = t / s.OH;
+    const int64_t h0 = (oh * s.H) / s.OH, h1 = ceil_div((oh + 1) * s.H, s.OH);
+    const int64_t w0 = (ow * s.W) / s.OW, w1 = ceil_div((ow + 1) * s.W, s.OW);
+    int32_t acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0;
+    for (int64_t ih = h0; ih < h1; ++ih) {
+      const uint8_t* row = x + ((b * s.H + ih) * s.W) * s.C + c;
+      for (int64_t iw = w0; iw < w1; ++iw) {
+        if constexpr (VEC == 4) {
+          const uint32_t w = *reinterpret_cast<const uint32_t*>(row + iw * s.C);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t bte = (w >> (8 * j)) & 0xffu;
+            acc[j] += SIGNED ? static_cast<int32_t>(static_cast<int8_t>(bte)) : static_cast<int32_t>(bte);
+          }
+        } else {
+          const uint8_t bte = row[iw * s.C];
+          acc[0] += SIGNED ? static_cast<int32_t>(static_cast<int8_t>(bte)) : static_cast<int32_t>(bte);
+        }
+      }
+    }
+    const int32_t size = static_cast<int32_t>((h1 - h0) * (w1 - w0));
+    const float mult = 1.0f / static_cast<float>(size);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float v = static_cast<float>(acc[j] - zp * size) * mult;
+      float r = __builtin_rintf(v) + static_cast<float>(zp);
+      r = __builtin_amdgcn_fmed3f(r, lo, hi);
+      packed |= (static_cast<uint32_t>(static_cast<int32_t>(r)) & 0xffu) << (8 * j);
+    }
+    uint8_t* dst = y + ((b * s.OH + oh) * s.OW + ow) * s.C + c;
+    if constexpr (VEC == 4)
+      *reinterpret_cast<uint32_t*>(dst) = packed;
+    else
+      *dst = static_cast<uint8_t>(packed);
+  }
+}
+
 bool zp_ok(int32_t zp, int q_signed) { return q_signed ? (zp >= -128 && zp <= 127) : (zp >= 0 && zp <= 255); }
 
 template <bool SIGNED, bool RELU>
@@ -409,6 +465,34 @@ TMQ_EXPORT int tmq_qmaxpool2d(const void* x, void* y, int64_t B, int64_t H, int6
   } else {
     if (q_signed) qmaxpool_kernel<true, 1><<<grid, block, 0, hs>>>(xb, yb, s);
     else qmaxpool_kernel<false, 1><<<grid, block, 0, hs>>>(xb, yb, s);
+  }
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_qadaptive_avgpool2d(const void* x, void* y, int64_t B, int64_t H, int64_t W, int64_t C,
+                                       int64_t OH, int64_t OW, int32_t zero_point, int q_signed,
+                                       tmq_stream_t stream) {
+  if (B < 0 || H <= 0 || W <= 0 || C < 0 || OH < 0 || OW < 0) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!zp_ok(zero_point, q_signed)) return TMQ_ERR_INVALID_ARGUMENT;
+  // int32 window sums: 255 * window must stay below 2**31
+  if (H * W > (int64_t{1} << 23)) return TMQ_ERR_UNSUPPORTED;
+  const int64_t n = B * OH * OW * C;
+  if (n == 0) return TMQ_OK;
+  if (x == nullptr || y == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  PoolShape s{B, H, W, C, OH, OW, 0, 0, 0, 0, 0, 0, 0, 0};
+  const bool vec = C % 4 == 0 && aligned(x, 4) && aligned(y, 4);
+  int64_t g = ceil_div(vec ? n / 4 : n, kEwThreads);
+  g = g > (1 << 20) ? (1 << 20) : g;
+  const dim3 grid(static_cast<unsigned>(g)), block(kEwThreads);
+  hipStream_t hs = as_stream(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  if (vec) {
+    if (q_signed) qadaptive_avgpool_kernel<true, 4><<<grid, block, 0, hs>>>(xb, yb, s, zero_point);
+    else qadaptive_avgpool_kernel<false, 4><<<grid, block, 0, hs>>>(xb, yb, s, zero_point);
+  } else {
+    if (q_signed) qadaptive_avgpool_kernel<true, 1><<<grid, block, 0, hs>>>(xb, yb, s, zero_point);
+    else qadaptive_avgpool_kernel<false, 1><<<grid, block, 0, hs>>>(xb, yb, s, zero_point);
   }
   return launch_status();
 }
