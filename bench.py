@@ -289,6 +289,38 @@ def main():
                 "algorithmic_bytes_per_launch": nbytes}
         del pws
 
+        # ------------------------------------------- dynamically quantized linear
+        # quantized::linear_dynamic at config 3's shape: fp32 in, min/max + qparams +
+        # quantize + int8 product + fp32 out, five launches, no host round trip
+        log("[bench] linear_dynamic at config 3's shape (fp32 in, fp32 out)")
+        xds = [torch.randn(M, K, device=dev) for _ in range(2)]
+        dcount = [0]
+
+        def dyn():
+            dcount[0] += 1
+            return torch.ops.quantized.linear_dynamic(xds[dcount[0] % 2], packs[dcount[0] % NSETS], False)
+
+        for _ in range(30):
+            dyn()
+        torch.cuda.synchronize()
+        a_, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a_.record()
+        for _ in range(50):
+            dyn()
+        b_.record()
+        torch.cuda.synchronize()
+        dms = a_.elapsed_time(b_) / 50
+        dbytes = 2 * 4 * M * K + 2 * M * K + N * K + 4 * M * N + 12 * N
+        log(f"[bench] linear_dynamic: {dms*1e3:.1f} us per call, {ops / (dms * 1e-3) / 1e12:.0f} TOP/s")
+        secondary["linear_dynamic_c3_shape"] = {
+            "avg_call_us": round(dms * 1e3, 1), "value": round(ops / (dms * 1e-3) / 1e12, 1), "unit": "TOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(ops / (dms * 1e-3) / 1e12, 1), "peak": PEAK_INT8_TOPS,
+                         "unit": "TOP/s", "frac": round(ops / (dms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4),
+                         "traffic": None},
+            "method": "50 calls back to back between two events, 2 inputs x 4 weights rotated",
+            "algorithmic_bytes_per_call": dbytes, "ops_per_call": ops}
+        del xds
+
         # -------------------------------------------------------------- C5
         log("[bench] config 5: conv2d NHWC [32,56,56,64] x [64,3,3,64]")
         xc = torch.relu(torch.randn(32, 64, 56, 56, device=dev)).contiguous(memory_format=torch.channels_last)

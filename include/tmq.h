@@ -190,6 +190,20 @@ int tmq_linear(const tmq_linear_desc* desc, tmq_stream_t stream);
 int tmq_linear_acc32(const tmq_linear_desc* desc, int32_t* acc, int64_t ldacc,
                      tmq_stream_t stream);
 
+/* Float output of the same product, the second half of a dynamically quantized
+ * linear (PackedLinearWeight::apply_dynamic, which the reference declares and
+ * leaves unimplemented, torch_musa/csrc/aten/quantized/mudnn/Linear.h:35-46;
+ * arithmetic of PyTorch's CPU op, fbgemm ReQuantizeForFloat):
+ *   y[m][n] = fma(float(acc[m][n] - x_zp * colsum[n]), fl(x_scale * w_scale[n]), bias[n])
+ * clamped below at 0 when desc->relu.  Uses M, N, K, x, ldx, x_signed, w_*,
+ * relu, bias of `desc`; y is fp32 [M, ldy].  x_qparams_dev != NULL: the
+ * activation scale and zero point are read from device memory when the kernel
+ * runs (as written by tmq_choose_qparams_dev), desc->x_scale / x_zero_point are
+ * ignored, and min/max -> qparams -> quantize -> linear runs without the host
+ * seeing the parameters. */
+int tmq_linear_f32(const tmq_linear_desc* desc, const tmq_qparams* x_qparams_dev, float* y,
+                   int64_t ldy, tmq_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * quantized::conv2d weights.
  * Replaces PackedConvWeightMudnn<2>::prepack

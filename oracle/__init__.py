@@ -211,6 +211,34 @@ def linear(xq, x_scale, x_zp, wq, w_scales, bias, out_scale, out_zp,
     return y
 
 
+def linear_f32(xq, x_scale, x_zp, wq, w_scales, bias, relu=False, nthreads=1):
+    """Float output of quantized activations times a quantized weight (zero point 0)."""
+    xq = _as_bytes(xq)
+    wq = np.ascontiguousarray(wq, dtype=np.int8)
+    m, k = xq.shape
+    n = wq.shape[0]
+    w_scales = np.ascontiguousarray(np.atleast_1d(w_scales), dtype=np.float64)
+    assert w_scales.size in (1, n)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    y = np.empty((m, n), dtype=np.float32)
+    lib().orc_linear_f32(_p(xq), C.c_int(xq.dtype == np.int8), _p(wq), C.c_int64(m), C.c_int64(n),
+                         C.c_int64(k), C.c_int64(x_zp), C.c_double(x_scale), _p(w_scales),
+                         C.c_int64(w_scales.size), _p(b) if b is not None else None, C.c_int(relu),
+                         _p(y), C.c_int(nthreads))
+    return y
+
+
+def linear_dynamic(x, wq, w_scales, bias, relu=False, reduce_range=False):
+    """quantized::linear_dynamic: per-tensor dynamic quint8 quantization of the
+    float activations, integer product, float output."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    mn, mx = minmax(x)
+    scale, zp = choose_qparams(mn, mx, False, reduce_range)
+    xq = quantize_per_tensor(x.reshape(-1, x.shape[-1]), scale, zp, False)
+    y = linear_f32(xq, scale, zp, wq, w_scales, bias, relu)
+    return y.reshape(x.shape[:-1] + (y.shape[-1],))
+
+
 def conv_out_hw(h, w, kh, kw, stride, padding, dilation):
     oh = (h + 2 * padding[0] - dilation[0] * (kh - 1) - 1) // stride[0] + 1
     ow = (w + 2 * padding[1] - dilation[1] * (kw - 1) - 1) // stride[1] + 1

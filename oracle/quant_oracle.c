@@ -345,6 +345,37 @@ ORC_API void orc_linear(const uint8_t* x, int x_signed, const int8_t* w, int64_t
   free(colsum);
 }
 
+/* Float output stage of a dynamically quantized linear (PyTorch's CPU
+ * quantized::linear_dynamic, fbgemm ReQuantizeForFloat; the reference declares
+ * apply_dynamic and leaves it unimplemented, mudnn/Linear.h:35-46):
+ *   y[m][n] = fma((float)(acc - x_zp * colsum[n]), fl(x_scale_f * w_scale_f[n]), bias[n])
+ * one fused multiply-add per value (what the vectorised CPU kernel executes:
+ * separate multiply and add differ from it in the last bit on about a third of
+ * the values), then max(y, 0) for the relu variant. */
+ORC_API void orc_linear_f32(const uint8_t* x, int x_signed, const int8_t* w, int64_t M,
+                            int64_t N, int64_t K, int64_t x_zp, double x_scale,
+                            const double* w_scales, int64_t n_scales, const float* bias,
+                            int relu, float* y, int nthreads) {
+  int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)M * (size_t)N);
+  int32_t* colsum = (int32_t*)malloc(sizeof(int32_t) * (size_t)N);
+  orc_linear_acc32(x, x_signed, w, M, N, K, acc, nthreads);
+  orc_weight_colsum(w, N, K, colsum);
+  const float xs = (float)x_scale;
+  for (int64_t n = 0; n < N; ++n) {
+    const float ws = (float)w_scales[n_scales == 1 ? 0 : n];
+    volatile float mult = xs * ws;
+    const float b = bias ? bias[n] : 0.f;
+    for (int64_t m = 0; m < M; ++m) {
+      const int32_t raw = acc[m * N + n] - (int32_t)x_zp * colsum[n];
+      float v = fmaf((float)raw, mult, b);
+      if (relu && !(v > 0.f)) v = 0.f;
+      y[m * N + n] = v;
+    }
+  }
+  free(acc);
+  free(colsum);
+}
+
 /* ------------------------------------------------------------------------- */
 /* quantized::conv2d accumulators, NHWC activations x OHWI weights:
  *   acc[b][oh][ow][oc] = sum_{kh,kw,ic} (X[b][ih][iw][g*ICg+ic] - x_zp) * W[oc][kh][kw][ic]

@@ -389,3 +389,32 @@ def qavgpool_cases():
         out.append(dict(name=name, x=rng.integers(lo, hi, shape).astype(np.int8 if signed else np.uint8),
                         out_hw=ohw, zp=zp, signed=signed))
     return out
+
+
+def linear_dynamic_cases():
+    """Float activations for quantized::linear_dynamic: dict(name, x, wq, w_scales,
+    bias, relu, reduce_range). Weight zero points are 0."""
+    spec = [
+        # name, x shape, N, per_channel, bias, relu, reduce_range
+        ("pc_bias_8x64_48", (8, 64), 48, True, True, False, False),
+        ("pt_bias_33x100_70", (33, 100), 70, False, True, False, False),
+        ("pc_relu_16x256_33", (16, 256), 33, True, True, True, False),
+        ("pt_relu_rr_16x256_33", (16, 256), 33, False, True, True, True),
+        ("pc_nobias_rr_5x37_9", (5, 37), 9, True, False, False, True),
+        ("batched_3x7x128_130", (3, 7, 128), 130, True, True, False, True),
+        ("one_row_1x512_256", (1, 512), 256, True, True, False, False),
+        ("tall_300x192_72", (300, 192), 72, True, True, False, False),
+    ]
+    out = []
+    for i, (name, xshape, n, pc, has_bias, relu, rr) in enumerate(spec):
+        rng = np.random.default_rng(1700 + i)
+        k = xshape[-1]
+        x = (rng.standard_normal(xshape) * 1.7 + 0.3).astype(np.float32)
+        wq = rng.integers(-127, 128, (n, k), dtype=np.int8)
+        if pc:
+            w_scales = (0.0005 + 0.001 * rng.random(n)).astype(np.float32).astype(np.float64)
+        else:
+            w_scales = np.array([float(np.float32(0.00093))])
+        bias = rng.standard_normal(n).astype(np.float32) if has_bias else None
+        out.append(dict(name=name, x=x, wq=wq, w_scales=w_scales, bias=bias, relu=relu, reduce_range=rr))
+    return out

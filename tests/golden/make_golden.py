@@ -113,6 +113,18 @@ def main():
         g[k + "/out_scale"] = np.float64(c["out_scale"])
         g[k + "/y"] = y.int_repr().numpy()
 
+    # ---- quantized::linear_dynamic (float in, float out) ------------------------
+    for c in cases.linear_dynamic_cases():
+        w = make_w(c["wq"], c["w_scales"], c["wq"].shape[0])
+        b = None if c["bias"] is None else torch.from_numpy(c["bias"])
+        packed = torch.ops.quantized.linear_prepack(w, b)
+        op = torch.ops.quantized.linear_relu_dynamic if c["relu"] else torch.ops.quantized.linear_dynamic
+        y = op(torch.from_numpy(c["x"]), packed, c["reduce_range"])
+        k = "lindyn/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/wq_crc"] = np.uint32(cases.crc(c["wq"]))
+        g[k + "/y"] = y.numpy()
+
     # ---- C1 ---------------------------------------------------------------
     c1 = cases.c1_case()
     x = torch.from_numpy(c1["x"])

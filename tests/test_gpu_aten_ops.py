@@ -460,3 +460,61 @@ def test_adaptive_avg_pool2d_op(golden, c):
                                       golden["qavgpool/" + c["name"] + "/y"])
     m = torch.nn.AdaptiveAvgPool2d(c["out_hw"])
     np.testing.assert_array_equal(m(xq).int_repr().cpu().numpy(), y.int_repr().cpu().numpy())
+
+
+def _wq_from_case(c):
+    n = c["wq"].shape[0]
+    w = torch.from_numpy(c["wq"])
+    if len(c["w_scales"]) == 1:
+        return torch._make_per_tensor_quantized_tensor(w, float(c["w_scales"][0]), 0)
+    return torch._make_per_channel_quantized_tensor(w, torch.from_numpy(c["w_scales"]),
+                                                    torch.zeros(n, dtype=torch.int64), 0)
+
+
+@pytest.mark.parametrize("c", cases.linear_dynamic_cases(), ids=lambda c: c["name"])
+def test_linear_dynamic_op(golden, c):
+    # float in, float out; live CPU op and golden vector, bit for bit
+    say("aten linear_dynamic", c["name"])
+    wq = _wq_from_case(c)
+    b = None if c["bias"] is None else torch.from_numpy(c["bias"])
+    name = "linear_relu_dynamic" if c["relu"] else "linear_dynamic"
+    op = getattr(torch.ops.quantized, name)
+    x = torch.from_numpy(c["x"])
+    ref = op(x, torch.ops.quantized.linear_prepack(wq, b), c["reduce_range"])
+    packed = torch.ops.quantized.linear_prepack(wq.cuda(), None if b is None else b.cuda())
+    y = op(x.cuda(), packed, c["reduce_range"])
+    assert y.is_cuda and y.dtype == torch.float32 and y.shape == ref.shape
+    assert torch.equal(y.cpu(), ref)
+    np.testing.assert_array_equal(y.cpu().numpy(), golden["lindyn/" + c["name"] + "/y"])
+
+
+def test_dynamic_linear_module():
+    # torch.ao.nn.quantized.dynamic.Linear with GPU packed parameters (set_weight_bias, as
+    # the reference's tests populate quantized modules, test_quantized_linear.py:58-60)
+    say("nnqd.Linear")
+    import torch.ao.nn.quantized.dynamic as nnqd
+    torch.manual_seed(5)
+    w = torch.randn(96, 160) * 0.05
+    b = torch.randn(96)
+    wq = torch.quantize_per_tensor(w, float(w.abs().max() / 127), 0, torch.qint8)
+    x = torch.randn(4, 9, 160)
+    m_cpu = nnqd.Linear(160, 96)
+    m_cpu.set_weight_bias(wq, b)
+    m_gpu = nnqd.Linear(160, 96)
+    m_gpu.set_weight_bias(wq.cuda(), b.cuda())
+    y = m_gpu(x.cuda())
+    assert y.is_cuda and torch.equal(y.cpu(), m_cpu(x))
+    wq2, b2 = m_gpu._packed_params._packed_params.unpack()
+    assert torch.equal(wq2.int_repr().cpu(), wq.int_repr()) and torch.equal(b2.cpu(), b)
+
+
+def test_linear_dynamic_errors():
+    say("aten linear_dynamic errors")
+    w = torch.quantize_per_tensor(torch.randn(8, 16), 0.1, 0, torch.qint8).cuda()
+    packed = torch.ops.quantized.linear_prepack(w, None)
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.linear_dynamic(torch.randn(3, 15).cuda(), packed, False)     # feature count
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.linear_dynamic(torch.randn(3, 16).cuda().half(), packed, False)  # dtype
+    y = torch.ops.quantized.linear_dynamic(torch.zeros(0, 16).cuda(), packed, False)
+    assert y.shape == (0, 8)

@@ -208,3 +208,57 @@ def test_c3_full_size(cabi):
     # the GEMM is linear in x: acc(x) + acc(255 - x) = 255 * colsum
     acc2 = cabi.linear_acc32(255 - xq, pw)
     assert torch.equal(acc + acc2, 255 * pw.colsum[None, :].expand(M, N))
+
+
+# ---- float output (the second half of a dynamically quantized linear) --------------
+# Float results are compared bit for bit: the kernel's epilogue is the oracle's
+# single fused multiply-add, and the dynamic quantization in front of it is
+# bit-exact by the quantizer tests.
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9])
+@pytest.mark.parametrize("shape,relu,bias,pc,x_signed", [((60, 264, 448), False, True, True, False),
+                                                         ((257, 33, 144), True, True, False, False),
+                                                         ((16, 1040, 1168), False, False, True, True)])
+def test_linear_f32_configs(cabi, cfg, shape, relu, bias, pc, x_signed):
+    say("linear_f32 cfg", cfg, shape, relu, bias, pc, x_signed)
+    c = _tile_case(*shape, seed=300 + cfg, x_signed=x_signed, relu=relu, bias=bias, per_channel=pc)
+    if cfg == 8 and shape[0] > 64:
+        pytest.skip("the weight-streaming kernel takes at most 64 rows")
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    cabi.force_linear_config(cfg)
+    try:
+        y = host(cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, relu=relu))
+    finally:
+        cabi.force_linear_config(-1)
+    want = oracle.linear_f32(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], relu=relu)
+    np.testing.assert_array_equal(y, want)
+
+
+@pytest.mark.parametrize("c", cases.linear_dynamic_cases(), ids=lambda c: c["name"])
+def test_linear_dynamic_cases(cabi, golden, c):
+    say("linear_dynamic", c["name"])
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    y = host(cabi.linear_dynamic(dev(c["x"]), pw, ws, b, relu=c["relu"], reduce_range=c["reduce_range"]))
+    np.testing.assert_array_equal(y, golden["lindyn/" + c["name"] + "/y"])
+    np.testing.assert_array_equal(y, oracle.linear_dynamic(c["x"], c["wq"], c["w_scales"], c["bias"], c["relu"],
+                                                           c["reduce_range"]))
+
+
+def test_linear_dynamic_prefill_sized(cabi):
+    # [2048, 1024] x [4096, 1024]^T through the large-tile kernel, against the oracle
+    say("linear_dynamic prefill")
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2048, 1024)).astype(np.float32)
+    wq = rng.integers(-127, 128, (4096, 1024), dtype=np.int8)
+    wsc = (0.0005 + 0.001 * rng.random(4096)).astype(np.float32).astype(np.float64)
+    bias = rng.standard_normal(4096).astype(np.float32)
+    pw = cabi.PackedLinear(dev(wq))
+    y = host(cabi.linear_dynamic(dev(x), pw, dev(wsc.astype(np.float32)), dev(bias)))
+    mn, mx = oracle.minmax(x)
+    scale, zp = oracle.choose_qparams(mn, mx, False, False)
+    xq = oracle.quantize_per_tensor(x, scale, zp, False, nthreads=8)
+    want = oracle.linear_f32(xq, scale, zp, wq, wsc, bias, nthreads=8)
+    np.testing.assert_array_equal(y, want)

@@ -173,3 +173,14 @@ def test_qadaptive_avgpool2d(golden, c):
     assert int(golden[k + "/x_crc"]) == cases.crc(c["x"])
     y = oracle.qadaptive_avgpool2d(c["x"], c["out_hw"], c["zp"])
     np.testing.assert_array_equal(y, golden[k + "/y"])
+
+
+@pytest.mark.parametrize("c", cases.linear_dynamic_cases(), ids=lambda c: c["name"])
+def test_linear_dynamic(golden, c):
+    # float results, compared bit for bit: the oracle's single fused multiply-add
+    # per value is what the CPU op executes
+    k = "lindyn/" + c["name"]
+    assert int(golden[k + "/x_crc"]) == cases.crc(c["x"]) and int(golden[k + "/wq_crc"]) == cases.crc(c["wq"])
+    y = oracle.linear_dynamic(c["x"], c["wq"], c["w_scales"], c["bias"], c["relu"], c["reduce_range"])
+    assert y.dtype == np.float32 and y.shape == golden[k + "/y"].shape
+    np.testing.assert_array_equal(y, golden[k + "/y"])

@@ -321,3 +321,42 @@ def test_qadaptive_avgpool_identity_constant_and_exact_means():
     # window bounds: 10 rows -> 3 outputs use rows [0,4) [3,7) [6,10)
     ramp = np.arange(10, dtype=np.uint8).reshape(1, 10, 1, 1) * 10
     np.testing.assert_array_equal(oracle.qadaptive_avgpool2d(ramp, (3, 1), 0).ravel(), [15, 45, 75])
+
+
+def test_linear_f32_exact_cases():
+    rng = np.random.default_rng(31)
+    xq = rng.integers(0, 256, (6, 40), dtype=np.uint8)
+    wq = rng.integers(-127, 128, (11, 40), dtype=np.int8)
+    acc = (xq.astype(np.int64) - 99) @ wq.astype(np.int64).T
+    # power-of-two scales, no bias: the result is the integer product, scaled exactly
+    y = oracle.linear_f32(xq, 0.5, 99, wq, np.full(11, 0.25), None)
+    np.testing.assert_array_equal(y, (acc * 0.125).astype(np.float32))
+    # bias and relu: still exact while everything stays representable
+    b = (np.arange(11, dtype=np.float32) - 5) * 4096
+    y = oracle.linear_f32(xq, 0.5, 99, wq, [0.25], b, relu=True)
+    np.testing.assert_array_equal(y, np.maximum(acc * 0.125 + b[None, :].astype(np.float64), 0).astype(np.float32))
+    # one rounding, not two: over many accumulators the fused form and
+    # multiply-then-add differ somewhere, and the oracle is the fused one
+    x1 = rng.integers(0, 256, (200, 64), dtype=np.uint8)
+    w1 = rng.integers(-127, 128, (1, 64), dtype=np.int8)
+    acc1 = (x1.astype(np.int64) @ w1.astype(np.int64).T).astype(np.float32)
+    m = np.float32(np.float32(0.1) * np.float32(0.3))
+    b1 = np.float32(0.7431)
+    want = (acc1.astype(np.float64) * np.float64(m) + np.float64(b1)).astype(np.float32)
+    two_step = ((acc1 * m).astype(np.float32) + b1).astype(np.float32)
+    y = oracle.linear_f32(x1, 0.1, 0, w1, [0.3], np.array([b1], np.float32))
+    np.testing.assert_array_equal(y, want)
+    assert (want != two_step).any()   # the data does tell the two apart
+
+
+def test_linear_dynamic_matches_float_linear_within_quantization_error():
+    rng = np.random.default_rng(32)
+    x = rng.standard_normal((20, 64)).astype(np.float32)
+    wq = rng.integers(-127, 128, (12, 64), dtype=np.int8)
+    ws = np.full(12, 0.01)
+    y = oracle.linear_dynamic(x, wq, ws, None)
+    ref = x.astype(np.float64) @ (wq.astype(np.float64) * 0.01).T
+    step = (x.max() - min(x.min(), 0)) / 255
+    # each activation is off by at most half a step
+    bound = 0.5 * step * np.abs(wq.astype(np.float64) * 0.01).sum(axis=1)
+    assert np.all(np.abs(y - ref) <= bound[None, :] * 1.001 + 1e-4)

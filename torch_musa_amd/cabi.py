@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32", "tmq_linear_f32",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d",
@@ -118,6 +118,7 @@ def lib() -> C.CDLL:
         l.tmq_linear_unpack.argtypes = [v, C.c_int64, C.c_int64, v, C.c_int64, v]
         l.tmq_linear.argtypes = [C.POINTER(LinearDesc), v]
         l.tmq_linear_acc32.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, v]
+        l.tmq_linear_f32.argtypes = [C.POINTER(LinearDesc), v, v, C.c_int64, v]
         l.tmq_conv2d_prepack.argtypes = [v, C.POINTER(Conv2dGeom), v, v, v]
         l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         l.tmq_conv2d.argtypes = [C.POINTER(Conv2dDesc), v]
@@ -319,6 +320,27 @@ def linear_acc32(x, pw: PackedLinear):
     check(lib().tmq_linear_acc32(C.byref(d), acc.data_ptr(), acc.stride(0), stream_ptr()),
           "tmq_linear_acc32")
     return acc
+
+
+def linear_f32(x, pw: PackedLinear, x_scale, x_zp, w_scales, bias, relu=False, qparams_dev=None):
+    """fp32 [M,N] = dequantized product; qparams_dev (16 device bytes from
+    choose_qparams_dev) replaces x_scale / x_zp when given."""
+    assert x.dim() == 2 and x.stride(1) == 1
+    y = torch.empty((x.shape[0], pw.N), dtype=torch.float32, device=x.device)
+    d = _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, 1.0, 0, False, relu, None)
+    check(lib().tmq_linear_f32(C.byref(d), qparams_dev.data_ptr() if qparams_dev is not None else None,
+                               y.data_ptr(), y.stride(0), stream_ptr()), "tmq_linear_f32")
+    return y
+
+
+def linear_dynamic(x, pw: PackedLinear, w_scales, bias, relu=False, reduce_range=False):
+    """min/max -> qparams -> quantize -> product, all on the device, no host round trip."""
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    x2 = x.reshape(-1, x.shape[-1])
+    qp = choose_qparams_dev(minmax(x2), False, reduce_range)
+    xq = quantize_per_tensor_dev(x2, qp, False)
+    y = linear_f32(xq, pw, 1.0, 0, w_scales, bias, relu, qparams_dev=qp)
+    return y.reshape(tuple(x.shape[:-1]) + (pw.N,))
 
 
 def quantize_per_channel_float_qparams(x, scales, zps, axis, signed):

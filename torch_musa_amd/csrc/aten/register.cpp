@@ -299,12 +299,14 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
   at::Tensor apply_relu(at::Tensor input, double output_scale, int64_t output_zero_point) override {
     return apply_impl(input, output_scale, output_zero_point, true);
   }
-  // as in the reference (mudnn/Linear.h:35-46)
-  at::Tensor apply_dynamic(at::Tensor, bool) override {
-    TORCH_CHECK(false, "apply_dynamic is not implemented for this packed parameter type");
+  // The reference declares these and throws (mudnn/Linear.h:35-46).  Here:
+  // min/max -> qparams -> quint8 activations -> int8 product -> fp32 output,
+  // five launches on the current stream, the parameters never visit the host.
+  at::Tensor apply_dynamic(at::Tensor input, bool reduce_range) override {
+    return apply_dynamic_impl(input, reduce_range, false);
   }
-  at::Tensor apply_dynamic_relu(at::Tensor, bool) override {
-    TORCH_CHECK(false, "apply_dynamic_relu is not implemented for this packed parameter type");
+  at::Tensor apply_dynamic_relu(at::Tensor input, bool reduce_range) override {
+    return apply_dynamic_impl(input, reduce_range, true);
   }
 
   // The packed buffer holds every weight byte, so the original tensor is
@@ -342,6 +344,52 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
   }
 
  private:
+  at::Tensor apply_dynamic_impl(const at::Tensor& input, bool reduce_range, bool relu) {
+    TORCH_CHECK(input.scalar_type() == at::kFloat, "quantized::linear_dynamic: expected a float input");
+    TORCH_CHECK(input.dim() >= 1, "quantized::linear_dynamic: input needs at least one dimension");
+    TORCH_CHECK(input.size(-1) == K_, "quantized::linear_dynamic: input has ", input.size(-1),
+                " features, the packed weight expects ", K_);
+    TORCH_CHECK(input.device() == packed_.device(),
+                "quantized::linear_dynamic: input and weight on different devices");
+    const c10::OptionalDeviceGuard guard(at::device_of(input));
+    const at::Tensor x = input.contiguous();
+    const int64_t M = K_ == 0 ? 0 : x.numel() / K_;
+    std::vector<int64_t> out_shape = x.sizes().vec();
+    out_shape.back() = N_;
+    at::Tensor y = at::empty(out_shape, x.options());
+    if (y.numel() == 0) return y;
+    TORCH_CHECK(x.numel() > 0, "quantized::linear_dynamic: empty input features");
+    const auto stream = current_stream(x);
+    const auto bytes = x.options().dtype(at::kByte);
+    at::Tensor ws = at::empty({static_cast<int64_t>(tmq_minmax_workspace_bytes(x.numel()))}, bytes);
+    at::Tensor mm = at::empty({2}, x.options());
+    at::Tensor qp = at::empty({static_cast<int64_t>(sizeof(tmq_qparams))}, bytes);
+    at::Tensor xq = at::empty({x.numel()}, bytes);
+    check_status(tmq_minmax(cptr<float>(x), x.numel(), mptr<float>(mm), ws.data_ptr(),
+                            static_cast<size_t>(ws.numel()), stream),
+                 "tmq_minmax");
+    auto* qpd = static_cast<tmq_qparams*>(qp.data_ptr());
+    check_status(tmq_choose_qparams_dev(cptr<float>(mm), 0, reduce_range, qpd, stream), "tmq_choose_qparams_dev");
+    check_status(tmq_quantize_per_tensor_dev(cptr<float>(x), xq.data_ptr(), x.numel(), qpd, 0, stream),
+                 "tmq_quantize_per_tensor_dev");
+    tmq_linear_desc d{};
+    d.M = M;
+    d.N = N_;
+    d.K = K_;
+    d.x = xq.data_ptr();
+    d.ldx = K_;
+    d.x_signed = 0;
+    d.x_scale = 1.f;  // unused: read from qp on the device
+    d.w_packed = packed_.const_data_ptr();
+    d.w_colsum = cptr<int32_t>(colsum_);
+    d.w_scales = cptr<float>(wp_.scales_f32);
+    d.w_per_channel = wp_.per_channel;
+    d.relu = relu;
+    d.bias = bias_.has_value() ? cptr<float>(*bias_) : nullptr;
+    check_status(tmq_linear_f32(&d, qpd, mptr<float>(y), N_, stream), "tmq_linear_f32");
+    return y;
+  }
+
   at::Tensor apply_impl(const at::Tensor& act, double output_scale, int64_t output_zero_point, bool relu) {
     TORCH_CHECK(act.qscheme() == c10::kPerTensorSymmetric || act.qscheme() == c10::kPerTensorAffine,
                 "quantized::linear expects a per-tensor quantized activation");
@@ -389,6 +437,15 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
   std::optional<at::Tensor> bias_;
   int64_t N_, K_;
 };
+
+at::Tensor qlinear_dynamic_run(at::Tensor x, const c10::intrusive_ptr<LinearPackedParamsBase>& w,
+                               bool reduce_range) {
+  return w->apply_dynamic(std::move(x), reduce_range);
+}
+at::Tensor qlinear_relu_dynamic_run(at::Tensor x, const c10::intrusive_ptr<LinearPackedParamsBase>& w,
+                                    bool reduce_range) {
+  return w->apply_dynamic_relu(std::move(x), reduce_range);
+}
 
 at::Tensor qlinear_run(at::Tensor act, const c10::intrusive_ptr<LinearPackedParamsBase>& w, double s, int64_t z) {
   return w->apply(std::move(act), s, z);
@@ -782,6 +839,12 @@ TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d.new"), TORCH_FN(qconv2d_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_relu.new"), TORCH_FN(qconv2d_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_prepack"), TORCH_FN(qconv2d_prepack_run));
+}
+
+// float activations arrive under the plain CUDA key
+TORCH_LIBRARY_IMPL(quantized, CUDA, m) {
+  m.impl(TORCH_SELECTIVE_NAME("quantized::linear_dynamic"), TORCH_FN(qlinear_dynamic_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::linear_relu_dynamic"), TORCH_FN(qlinear_relu_dynamic_run));
 }
 
 // Replacing PyTorch's own GPU kernel of aten::quantize_per_tensor_dynamic is the

@@ -37,7 +37,11 @@ namespace tmq {
 constexpr int kBK = 64;       // k-bytes per LDS stage
 constexpr int kChunks = 4;    // 16-byte k-chunks per stage
 
-enum EpilogueMode { kOutU8 = 0, kOutS8 = 1, kOutAcc32 = 2 };
+// kOutF32: y = fma(float(raw), x_scale * w_scale[n], bias[n]), optionally
+// clamped below at 0 -- the float output of a dynamically quantized linear
+// (fbgemm's ReQuantizeForFloat as PyTorch's CPU op runs it, one fused
+// multiply-add per value).
+enum EpilogueMode { kOutU8 = 0, kOutS8 = 1, kOutAcc32 = 2, kOutF32 = 3 };
 
 // Where a tile's activation rows come from.
 struct XLinear {
@@ -86,7 +90,39 @@ struct GemmArgs {
   int64_t ldy;
   int32_t n_off;         // conv groups: channel offset of this group in y/params
   PostOps post;          // all zero for quantized::linear
+  // Activation scale and zero point read from device memory at run time (the
+  // tail of a min/max -> qparams -> quantize chain with no host round trip);
+  // null: x_scale and acc_coef above hold.  acc_base is acc_coef + zero point.
+  const tmq_qparams* x_qp_dev = nullptr;
+  int32_t acc_base = 0;
 };
+
+struct XQuant {
+  float scale;
+  int32_t coef;  // multiplies colsum[n] into the accumulator start
+};
+__device__ __forceinline__ XQuant x_quant(const GemmArgs& a) {
+  if (a.x_qp_dev != nullptr)
+    return XQuant{static_cast<float>(a.x_qp_dev->scale), a.acc_base - a.x_qp_dev->zero_point};
+  return XQuant{a.x_scale, a.acc_coef};
+}
+
+// Four float results of one output row (kOutF32), channels n .. n+3.
+__device__ __forceinline__ void store_f32x4(const GemmArgs& a, int64_t m, int64_t n, const int (&raw)[4],
+                                            v4f mult, v4f bias) {
+  float* dst = static_cast<float*>(a.y) + m * a.ldy + a.n_off + n;
+  v4f v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    v[j] = __builtin_fmaxf(__builtin_fmaf(static_cast<float>(raw[j]), mult[j], bias[j]), a.lo_f);
+  if (n + 3 < a.N && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+    *reinterpret_cast<v4f*>(dst) = v;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n + j < a.N) dst[j] = v[j];
+  }
+}
 
 __device__ __forceinline__ v4i ld16(const void* p) { return *reinterpret_cast<const v4i*>(p); }
 // Streaming load: data that this CU reads exactly once (packed weight tiles)
@@ -323,7 +359,9 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int kWStage = kChunks * BN * 16, kXStage = BM * kBK;
   constexpr int kOutPitch = BN + 16;  // bytes; keeps rows 16-byte aligned and off one bank
   constexpr int kMainBytes = kWBufs * kWStage + kXBufs * kXStage;
-  constexpr int kOutBytes = (MODE == kOutAcc32) ? 0 : BM * kOutPitch;
+  constexpr int kF32Pitch = BN * 4 + 16;  // float rows of the tile, same idea
+  constexpr int kOutBytes =
+      (MODE == kOutAcc32) ? 0 : (MODE == kOutF32 ? WM * 32 * kF32Pitch : BM * kOutPitch);
   constexpr int kTileBytes = kMainBytes > kOutBytes ? kMainBytes : kOutBytes;
   __shared__ __attribute__((aligned(16))) uint8_t smem[kTileBytes];
   __shared__ __attribute__((aligned(16))) int s_acc0[BN];
@@ -365,15 +403,19 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   // the first operand copies are on their way.
   v16i acc[TN][TM];
   auto init_tile = [&]() {
+    const XQuant xq = x_quant(a);
     for (int i = t; i < BN; i += NT) {
       const int64_t n = n0 + i;
       int acc0 = 0;
       float mult = 0.f, bdiv = 0.f;
       if (n < a.N) {
         const int64_t np = n + a.n_off;
-        acc0 = a.acc_coef * a.colsum[np];
-        if (MODE != kOutAcc32) {
-          const float atw = a.x_scale * a.w_scales[np * a.w_scale_stride];
+        acc0 = xq.coef * a.colsum[np];
+        if (MODE == kOutF32) {
+          mult = xq.scale * a.w_scales[np * a.w_scale_stride];
+          bdiv = a.bias != nullptr ? a.bias[np] : 0.f;
+        } else if (MODE != kOutAcc32) {
+          const float atw = xq.scale * a.w_scales[np * a.w_scale_stride];
           mult = atw / a.out_scale;
           bdiv = a.bias != nullptr ? a.bias[np] / atw : 0.f;
         }
@@ -679,6 +721,48 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
             if (n + j < a.N) dst[j] = acc[tn][tm][4 * g + j];
         }
       }
+  } else if constexpr (MODE == kOutF32) {
+    // Float results, one 32-row MFMA tile of every wave at a time: the waves
+    // write their rows into LDS, then all threads copy whole rows out, 16 B per
+    // lane on consecutive addresses (a lane's own four floats of 32 different
+    // rows would make 32 partial lines per store instruction).
+    float* const yf = static_cast<float*>(a.y) + a.n_off;
+    const bool vec_ok = ((a.ldy & 3) == 0) && ((reinterpret_cast<uintptr_t>(yf) & 15) == 0);
+    constexpr int kRowChunks = BN / 4;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      __syncthreads();  // the operand stages, or the previous pass, are read out
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int nl = wn0 + tn * 32 + 8 * g + 4 * half;
+          const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[nl]);
+          const v4f bias = *reinterpret_cast<const v4f*>(&s_bdiv[nl]);
+          v4f v;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            v[j] = __builtin_fmaxf(
+                __builtin_fmaf(static_cast<float>(acc[tn][tm][4 * g + j]), mult[j], bias[j]), a.lo_f);
+          *reinterpret_cast<v4f*>(&smem[((wave % WM) * 32 + li) * kF32Pitch + nl * 4]) = v;
+        }
+      __syncthreads();
+#pragma unroll 4
+      for (int id = t; id < WM * 32 * kRowChunks; id += NT) {
+        const int lr = id / kRowChunks, cc = id % kRowChunks;
+        const int64_t m = m0 + (lr / 32) * WTM + tm * 32 + (lr % 32), n = n0 + cc * 4;
+        if (m >= a.M || n >= a.N) continue;
+        const v4f v = *reinterpret_cast<const v4f*>(&smem[lr * kF32Pitch + cc * 16]);
+        float* dst = yf + m * a.ldy + n;
+        if (vec_ok && n + 4 <= a.N) {
+          *reinterpret_cast<v4f*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (n + j < a.N) dst[j] = v[j];
+        }
+      }
+    }
   } else {
     // Requantise in registers, transpose through LDS, then write whole rows:
     // 16 bytes per lane, consecutive lanes on consecutive addresses.

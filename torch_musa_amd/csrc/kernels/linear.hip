@@ -161,11 +161,15 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
   v4f bdiv = {0.f, 0.f, 0.f, 0.f}, mult = {0.f, 0.f, 0.f, 0.f};
   int acc0[4] = {0, 0, 0, 0};
   if (t < 64) {
+    const XQuant xq = x_quant(a);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      acc0[j] = a.acc_coef * c_cs[j];
-      if (MODE != kOutAcc32) {
-        const float atw = a.x_scale * c_ws[j];
+      acc0[j] = xq.coef * c_cs[j];
+      if (MODE == kOutF32) {
+        mult[j] = xq.scale * c_ws[j];
+        bdiv[j] = c_b[j];
+      } else if (MODE != kOutAcc32) {
+        const float atw = xq.scale * c_ws[j];
         mult[j] = atw / a.out_scale;
         bdiv[j] = a.bias != nullptr ? c_b[j] / atw : 0.f;
       }
@@ -193,6 +197,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           if (n + j < a.N) dst[j] = raw[j];
+      } else if (MODE == kOutF32) {
+        store_f32x4(a, m, n, raw, mult, bdiv);
       } else {
         const uint32_t packed = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
         uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
@@ -230,13 +236,17 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
     }
   }
   v4f bdiv, mult;
+  const XQuant xq = x_quant(a);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int64_t np = n + j < a.N ? n + j : 0;
     // plain accumulation used the true activation value, so only -x_zp*colsum is left
-    raw[j] += a.acc_coef * a.colsum[np];
-    if (MODE != kOutAcc32) {
-      const float atw = a.x_scale * a.w_scales[np * a.w_scale_stride];
+    raw[j] += xq.coef * a.colsum[np];
+    if (MODE == kOutF32) {
+      mult[j] = xq.scale * a.w_scales[np * a.w_scale_stride];
+      bdiv[j] = a.bias != nullptr ? a.bias[np] : 0.f;
+    } else if (MODE != kOutAcc32) {
+      const float atw = xq.scale * a.w_scales[np * a.w_scale_stride];
       mult[j] = atw / a.out_scale;
       bdiv[j] = a.bias != nullptr ? a.bias[np] / atw : 0.f;
     }
@@ -245,6 +255,8 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
     int32_t* dst = static_cast<int32_t*>(a.y) + m * a.ldy + n;
     for (int j = 0; j < 4; ++j)
       if (n + j < a.N) dst[j] = raw[j];
+  } else if (MODE == kOutF32) {
+    store_f32x4(a, m, n, raw, mult, bdiv);
   } else {
     const uint32_t packed = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
     uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
@@ -272,7 +284,10 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   if (!vec_ok || forced == 9) {
     // plain kernel accumulates true activation values: undo the +128 share
     GemmArgs b = a;
-    if (!x_signed) b.acc_coef -= 128;
+    if (!x_signed) {
+      b.acc_coef -= 128;
+      b.acc_base -= 128;
+    }
     const int64_t work = a.M * ceil_div(a.N, 4);
     const int64_t blocks = ceil_div(work, 256);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
@@ -431,6 +446,30 @@ TMQ_EXPORT int tmq_linear_acc32(const tmq_linear_desc* d, int32_t* acc, int64_t 
   a.y = acc;
   a.ldy = ldacc;
   return dispatch_linear<kOutAcc32>(a, xs, d->x_signed, vec_ok, as_stream(stream));
+}
+
+TMQ_EXPORT int tmq_linear_f32(const tmq_linear_desc* d, const tmq_qparams* x_qparams_dev, float* y,
+                              int64_t ldy, tmq_stream_t stream) {
+  GemmArgs a{};
+  XLinear xs{};
+  bool vec_ok = false;
+  const int rc = fill_args(d, &a, &xs, &vec_ok);
+  if (rc != TMQ_OK || d->M == 0 || d->N == 0) return rc;
+  if (y == nullptr || d->w_scales == nullptr || ldy < d->N) return TMQ_ERR_INVALID_ARGUMENT;
+  if (x_qparams_dev == nullptr && !(d->x_scale > 0.f)) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!aligned(y, 4)) return TMQ_ERR_ALIGNMENT;
+  a.w_scales = d->w_scales;
+  a.w_scale_stride = d->w_per_channel ? 1 : 0;
+  a.bias = d->bias;
+  a.acc_base = d->x_signed ? 0 : 128;
+  a.acc_coef = a.acc_base - d->x_zero_point;
+  a.x_scale = d->x_scale;
+  a.x_qp_dev = x_qparams_dev;
+  a.out_scale = 1.f;
+  a.lo_f = d->relu ? 0.f : -__builtin_inff();
+  a.y = y;
+  a.ldy = ldy;
+  return dispatch_linear<kOutF32>(a, xs, d->x_signed, vec_ok, as_stream(stream));
 }
 
 // Benchmark hook (not part of the public header): force a kernel
