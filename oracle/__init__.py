@@ -386,3 +386,44 @@ def qcat(qs, scales, zps, axis, out_scale, out_zp):
     parts = [quantize_per_tensor(dequantize_per_tensor(q, s, z), out_scale, out_zp, signed)
              for q, s, z in zip(qs, scales, zps)]
     return np.concatenate(parts, axis=axis)
+
+
+# ---------------------------------------------------------------------------
+# Plain-tensor int8 ops (quantized::linear_per_tensor, quantized::conv,
+# quantized::conv_binary).  The reference implements them as dequantize ->
+# fp32 matmul / conv -> (+ accum) -> relu -> round(r / out_scale + zp) -> clamp
+# (mudnn/Qlinear.cpp:36-69, mudnn/Qconv.cpp:45-86,137-181).  Restated here with
+# the product in exact integers and everything after it in float64, i.e. that
+# formula without its fp32 summation error; int8 kernels are held to 1 LSB of
+# it, float outputs to a relative 1e-5.
+# ---------------------------------------------------------------------------
+def _plain_finish(r, out_scale, out_zp, out_dtype, relu):
+    if relu:
+        r = np.maximum(r, 0.0)
+    if out_dtype == "float32":
+        return r.astype(np.float32)
+    lo, hi = (-128, 127) if out_dtype == "int8" else (0, 255)
+    return np.clip(np.rint(r / out_scale + out_zp), lo, hi).astype(np.int8 if out_dtype == "int8" else np.uint8)
+
+
+def plain_linear(x, x_scale, x_zp, w_kn, w_scale, bias, out_scale, out_zp, out_dtype, post="none"):
+    acc = (np.asarray(x, dtype=np.int64) - x_zp) @ np.asarray(w_kn, dtype=np.int64)
+    r = acc.astype(np.float64) * (np.float64(np.float32(x_scale)) * np.asarray(w_scale, dtype=np.float64))[None, :]
+    if bias is not None:
+        r = r + np.asarray(bias, dtype=np.float64)[None, :]
+    assert post in ("none", "relu")
+    return _plain_finish(r, out_scale, out_zp, out_dtype, post == "relu")
+
+
+def plain_conv(x_nchw, x_scale, x_zp, w_oihw, w_scale, bias, stride, pad, groups, out_scale, out_zp, out_dtype,
+               relu=False, accum=None, accum_scale=1.0, accum_zp=0):
+    x = np.ascontiguousarray(np.transpose(np.asarray(x_nchw), (0, 2, 3, 1)))
+    w = np.ascontiguousarray(np.transpose(np.asarray(w_oihw, dtype=np.int8), (0, 2, 3, 1)))
+    acc = conv2d_acc32(x, w, (stride, stride), (pad, pad), (1, 1), groups, x_zp)      # [B,OH,OW,OC], exact
+    r = acc.astype(np.float64) * (np.float64(np.float32(x_scale)) * np.asarray(w_scale, dtype=np.float64))
+    if bias is not None:
+        r = r + np.asarray(bias, dtype=np.float64)
+    r = np.transpose(r, (0, 3, 1, 2))
+    if accum is not None:
+        r = r + (np.asarray(accum, dtype=np.float64) - accum_zp) * np.float64(np.float32(accum_scale))
+    return _plain_finish(r, out_scale, out_zp, out_dtype, relu)

@@ -418,3 +418,91 @@ def linear_dynamic_cases():
         bias = rng.standard_normal(n).astype(np.float32) if has_bias else None
         out.append(dict(name=name, x=x, wq=wq, w_scales=w_scales, bias=bias, relu=relu, reduce_range=rr))
     return out
+
+
+def plain_linear_cases():
+    """quantized::linear_per_tensor: plain uint8 / int8 activations [M,K], int8 weight
+    [K,N] (the layout the schema takes), parameters beside them.  The first three
+    are the reference's (test_quantized_ops.py:745-795: small non-negative
+    integers, unit activation and output scale), where every arithmetic order
+    gives the same integers."""
+    out = []
+    for i, (s1, s2) in enumerate([((1, 10), (10, 5)), ((2, 3), (3, 4)), ((10, 7), (7, 10))]):
+        rng = np.random.default_rng(1800 + i)
+        for dt in ("uint8", "float32"):
+            out.append(dict(name=f"ref{i}_{dt}", x=rng.integers(0, 10, s1).astype(np.int8),
+                            w=rng.integers(0, 10, s2).astype(np.int8), x_scale=1.0, x_zp=0,
+                            w_scale=rng.integers(1, 10, s2[1]).astype(np.float32), bias=np.ones(s2[1], np.float32),
+                            out_scale=1.0, out_zp=0, out_dtype=dt, post="none"))
+    spec = [
+        # name, M, K, N, act dtype, x_zp, out dtype, post, bias
+        ("u8_relu_33x96_70", 33, 96, 70, np.uint8, 121, "uint8", "relu", True),
+        ("s8_s8_17x64_40", 17, 64, 40, np.int8, -5, "int8", "none", True),
+        ("u8_f32_5x37_9", 5, 37, 9, np.uint8, 17, "float32", "none", False),
+        ("u8_f32_relu_64x256_130", 64, 256, 130, np.uint8, 128, "float32", "relu", True),
+        ("u8_tall_300x192_72", 300, 192, 72, np.uint8, 100, "uint8", "none", True),
+    ]
+    for i, (name, m, k, n, adt, zp, odt, post, has_bias) in enumerate(spec):
+        rng = np.random.default_rng(1850 + i)
+        lo, hi = (-128, 128) if adt == np.int8 else (0, 256)
+        x_scale = float(np.float32(0.02))
+        w_scale = (0.001 + 0.002 * rng.random(n)).astype(np.float32)
+        sigma = np.sqrt(k) * 74.0 * 74.0 * x_scale * float(w_scale.mean())
+        out_int = odt != "float32"
+        out.append(dict(name=name, x=rng.integers(lo, hi, (m, k)).astype(adt),
+                        w=rng.integers(-127, 128, (k, n)).astype(np.int8), x_scale=x_scale, x_zp=zp,
+                        w_scale=w_scale, bias=(rng.standard_normal(n) * sigma).astype(np.float32) if has_bias else None,
+                        out_scale=float(np.float32(3 * sigma / 128)) if out_int else 1.0,
+                        out_zp=(-3 if odt == "int8" else 128) if out_int else 0, out_dtype=odt, post=post))
+    return out
+
+
+def plain_conv_cases():
+    """quantized::conv / quantized::conv_binary: plain NCHW uint8 activations, OIHW int8
+    weights.  The first three shapes are the reference's (test_quantized_ops.py:798-951)."""
+    out = []
+    spec = [
+        # name, x shape, w shape, stride, pad, groups, small ints?, out dtype, relu, accum ("none" | "uint8" | "float32")
+        ("ref0_f32", (1, 1, 5, 5), (1, 1, 3, 3), 1, 0, 1, True, "float32", False, "none"),
+        ("ref1_f32_relu", (1, 3, 10, 10), (4, 3, 2, 2), 1, 0, 1, True, "float32", True, "none"),
+        ("ref2_f32", (10, 5, 6, 6), (8, 5, 2, 2), 1, 0, 1, True, "float32", False, "none"),
+        ("ref2_sum_f32", (10, 5, 6, 6), (8, 5, 2, 2), 1, 0, 1, True, "float32", False, "float32"),
+        ("u8_relu_2x32x12x12_k3", (2, 32, 12, 12), (48, 32, 3, 3), 1, 1, 1, False, "uint8", True, "none"),
+        ("u8_s2_groups2", (2, 32, 13, 13), (64, 16, 3, 3), 2, 1, 2, False, "uint8", False, "none"),
+        ("f32_1x1_64", (3, 64, 7, 7), (32, 64, 1, 1), 1, 0, 1, False, "float32", True, "none"),
+        ("u8_sum_relu", (2, 16, 8, 8), (32, 16, 3, 3), 1, 1, 1, False, "uint8", True, "uint8"),
+        ("u8_sum", (2, 16, 8, 8), (32, 16, 3, 3), 1, 1, 1, False, "uint8", False, "uint8"),
+        ("f32_sum_relu", (2, 16, 8, 8), (32, 16, 3, 3), 1, 1, 1, False, "float32", True, "float32"),
+    ]
+    for i, (name, xs, wshape, st, pd, groups, small, odt, relu, accum) in enumerate(spec):
+        rng = np.random.default_rng(1900 + i)
+        oc = wshape[0]
+        kh, kw = wshape[2], wshape[3]
+        oh = (xs[2] + 2 * pd - kh) // st + 1
+        ow = (xs[3] + 2 * pd - kw) // st + 1
+        if small:
+            x = rng.integers(0, 10, xs).astype(np.uint8)
+            w = rng.integers(0, 10, wshape).astype(np.int8)
+            x_scale, x_zp = 1.0, 0
+            w_scale = (np.abs(rng.standard_normal(oc)) + 0.1).astype(np.float32)
+            bias = None
+            out_scale, out_zp = 1.0, 0
+        else:
+            x = rng.integers(0, 256, xs).astype(np.uint8)
+            w = rng.integers(-127, 128, wshape).astype(np.int8)
+            x_scale, x_zp = float(np.float32(0.03)), 120
+            w_scale = (0.002 + 0.01 * rng.random(oc)).astype(np.float32)
+            bias = rng.standard_normal(oc).astype(np.float32)
+            k = wshape[1] * kh * kw
+            sigma = np.sqrt(k) * 74.0 * 74.0 * x_scale * float(w_scale.mean())
+            out_scale, out_zp = (float(np.float32(3 * sigma / 128)), 10 if relu else 128) if odt == "uint8" else (1.0, 0)
+        c = dict(name=name, x=x, w=w, x_scale=x_scale, x_zp=x_zp, w_scale=w_scale, bias=bias, stride=st, pad=pd,
+                 groups=groups, out_scale=out_scale, out_zp=out_zp, out_dtype=odt, relu=relu, accum=None,
+                 accum_scale=1.0, accum_zp=0)
+        if accum == "uint8":
+            c["accum"] = rng.integers(0, 256, (xs[0], oc, oh, ow)).astype(np.uint8)
+            c["accum_scale"], c["accum_zp"] = float(np.float32(out_scale * 0.7)), 100
+        elif accum == "float32":
+            c["accum"] = (rng.standard_normal((xs[0], oc, oh, ow)) * (1.0 if small else 3.0)).astype(np.float32)
+        out.append(c)
+    return out

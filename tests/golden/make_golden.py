@@ -125,6 +125,44 @@ def main():
         g[k + "/wq_crc"] = np.uint32(cases.crc(c["wq"]))
         g[k + "/y"] = y.numpy()
 
+    # ---- plain-tensor int8 ops: goldens from PyTorch's oneDNN CPU ops, the reference
+    # the reference's own tests compare with (test_quantized_ops.py:745-951) -------
+    TD = {"uint8": torch.uint8, "int8": torch.int8, "float32": torch.float32}
+    for c in cases.plain_linear_cases():
+        n = c["w"].shape[1]
+        b = None if c["bias"] is None else torch.from_numpy(c["bias"])
+        y = torch.ops.onednn.qlinear_pointwise.default(
+            torch.from_numpy(c["x"]), c["x_scale"], c["x_zp"], torch.from_numpy(c["w"]).to_mkldnn(),
+            torch.from_numpy(c["w_scale"]), torch.zeros(n, dtype=torch.int), b, c["out_scale"], c["out_zp"],
+            TD[c["out_dtype"]], c["post"], [], "")
+        k = "plainlin/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/w_crc"] = np.uint32(cases.crc(c["w"]))
+        g[k + "/y"] = y.numpy()
+    for c in cases.plain_conv_cases():
+        oc = c["w"].shape[0]
+        ws = torch.from_numpy(c["w_scale"])
+        wz = torch.zeros(oc, dtype=torch.int)
+        b = None if c["bias"] is None else torch.from_numpy(c["bias"])
+        st, pd = [c["stride"]] * 2, [c["pad"]] * 2
+        x = torch.from_numpy(c["x"]).contiguous(memory_format=torch.channels_last)
+        pw = torch.ops.onednn.qconv_prepack(torch.from_numpy(c["w"]), ws, c["x_scale"], c["x_zp"], st, pd, [1, 1],
+                                            c["groups"], None)
+        if c["accum"] is None:
+            y = torch.ops.onednn.qconv2d_pointwise.default(
+                x, c["x_scale"], c["x_zp"], pw, ws, wz, b, st, pd, [1, 1], c["groups"], c["out_scale"], c["out_zp"],
+                TD[c["out_dtype"]], "relu" if c["relu"] else "none", [], "")
+        else:
+            acc = torch.from_numpy(c["accum"].copy()).contiguous(memory_format=torch.channels_last)  # overwritten
+            y = torch.ops.onednn.qconv2d_pointwise.binary(
+                x, c["x_scale"], c["x_zp"], pw, ws, wz, acc, b, st, pd, [1, 1], c["groups"], c["out_scale"],
+                c["out_zp"], TD[c["out_dtype"]], c["accum_scale"], c["accum_zp"], "sum", 1.0,
+                "relu" if c["relu"] else "none", [], "")
+        k = "plainconv/" + c["name"]
+        g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+        g[k + "/w_crc"] = np.uint32(cases.crc(c["w"]))
+        g[k + "/y"] = y.contiguous().numpy()   # NCHW order
+
     # ---- C1 ---------------------------------------------------------------
     c1 = cases.c1_case()
     x = torch.from_numpy(c1["x"])

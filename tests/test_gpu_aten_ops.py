@@ -12,6 +12,7 @@ import torch.ao.nn.intrinsic.quantized as nniq
 import torch.ao.nn.quantized as nnq
 
 import cases
+import oracle
 from gpu_util import say
 
 pytestmark = pytest.mark.gpu
@@ -518,3 +519,81 @@ def test_linear_dynamic_errors():
         torch.ops.quantized.linear_dynamic(torch.randn(3, 16).cuda().half(), packed, False)  # dtype
     y = torch.ops.quantized.linear_dynamic(torch.zeros(0, 16).cuda(), packed, False)
     assert y.shape == (0, 8)
+
+
+# ---- plain-tensor int8 ops (the reference's PT2E lowering targets) ----------------------
+_TD = {"uint8": torch.uint8, "int8": torch.int8, "float32": torch.float32}
+
+
+def _close_to(y, want, out_dtype, what, exact=False):
+    assert y.shape == want.shape and y.dtype == want.dtype, what
+    if exact:
+        np.testing.assert_array_equal(y, want, err_msg=what)
+    elif out_dtype == "float32":
+        np.testing.assert_allclose(y, want, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(want).max())), err_msg=what)
+    else:
+        d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+        assert d.max() <= 1, f"{what}: max diff {d.max()}"
+        assert np.count_nonzero(d) <= 0.002 * d.size + 1, f"{what}: {np.count_nonzero(d)} of {d.size} differ"
+
+
+@pytest.mark.parametrize("c", cases.plain_linear_cases(), ids=lambda c: c["name"])
+def test_linear_per_tensor_op(golden, c):
+    say("aten linear_per_tensor", c["name"])
+    n = c["w"].shape[1]
+    b = None if c["bias"] is None else torch.from_numpy(c["bias"]).cuda()
+    y = torch.ops.quantized.linear_per_tensor(
+        torch.from_numpy(c["x"]).cuda(), c["x_scale"], c["x_zp"], torch.from_numpy(c["w"]).cuda(),
+        torch.from_numpy(c["w_scale"]).cuda(), torch.zeros(n, dtype=torch.int).cuda(), b, c["out_scale"], c["out_zp"],
+        _TD[c["out_dtype"]], c["post"], [], "")
+    assert y.is_cuda and y.dtype == _TD[c["out_dtype"]]
+    y = y.cpu().numpy()
+    exact = c["name"].startswith("ref")
+    _close_to(y, golden["plainlin/" + c["name"] + "/y"], c["out_dtype"], "vs oneDNN CPU op", exact)
+    want = oracle.plain_linear(c["x"], c["x_scale"], c["x_zp"], c["w"], c["w_scale"], c["bias"], c["out_scale"],
+                               c["out_zp"], c["out_dtype"], c["post"])
+    _close_to(y, want, c["out_dtype"], "vs closed form", exact)
+
+
+@pytest.mark.parametrize("c", cases.plain_conv_cases(), ids=lambda c: c["name"])
+def test_plain_conv_ops(golden, c):
+    say("aten conv / conv_binary", c["name"])
+    oc = c["w"].shape[0]
+    b = None if c["bias"] is None else torch.from_numpy(c["bias"]).cuda()
+    args = [torch.from_numpy(c["x"]).cuda(), c["x_scale"], c["x_zp"], torch.from_numpy(c["w"]).cuda(),
+            torch.from_numpy(c["w_scale"]).cuda(), torch.zeros(oc, dtype=torch.int).cuda()]
+    geom = [[c["stride"]] * 2, [c["pad"]] * 2, [1, 1], c["groups"], c["out_scale"], c["out_zp"], _TD[c["out_dtype"]]]
+    if c["accum"] is None:
+        y = torch.ops.quantized.conv(*args, b, *geom, "relu" if c["relu"] else "none", [], None)
+    else:
+        acc = torch.from_numpy(c["accum"]).cuda()
+        y = torch.ops.quantized.conv_binary(*args, acc, b, *geom, c["accum_scale"], c["accum_zp"], "sum", 1.0,
+                                            "relu" if c["relu"] else "none", [], None)
+        assert torch.equal(acc.cpu(), torch.from_numpy(c["accum"]))   # the input is left alone
+    assert y.is_cuda and y.dtype == _TD[c["out_dtype"]]
+    y = y.contiguous().cpu().numpy()
+    _close_to(y, golden["plainconv/" + c["name"] + "/y"], c["out_dtype"], "vs oneDNN CPU op")
+    want = oracle.plain_conv(c["x"], c["x_scale"], c["x_zp"], c["w"], c["w_scale"], c["bias"], c["stride"], c["pad"],
+                             c["groups"], c["out_scale"], c["out_zp"], c["out_dtype"], c["relu"], c["accum"],
+                             c["accum_scale"], c["accum_zp"])
+    _close_to(y, want, c["out_dtype"], "vs closed form")
+
+
+def test_plain_ops_errors():
+    say("aten plain ops errors")
+    x = torch.randint(0, 255, (4, 16), dtype=torch.uint8).cuda()
+    w = torch.randint(-127, 127, (16, 8), dtype=torch.int8).cuda()
+    ws, wz = torch.full((8,), 0.01).cuda(), torch.zeros(8, dtype=torch.int).cuda()
+    call = lambda *a: torch.ops.quantized.linear_per_tensor(*a)
+    with pytest.raises(RuntimeError):
+        call(x[None], 0.1, 0, w, ws, wz, None, 1.0, 0, torch.uint8, "none", [], "")       # 3-D input
+    with pytest.raises(RuntimeError):
+        call(x, 0.1, 0, w, ws, wz + 1, None, 1.0, 0, torch.uint8, "none", [], "")         # weight zero point
+    with pytest.raises(RuntimeError):
+        call(x, 0.1, 0, w, ws, wz, None, 1.0, 0, torch.uint8, "hardswish", [], "")        # post op
+    with pytest.raises(RuntimeError):
+        call(x, 0.1, 0, w[:8], ws, wz, None, 1.0, 0, torch.uint8, "none", [], "")         # K mismatch
+    # tanh goes through the float result, like the reference's fallback
+    y = call(x, 0.02, 128, w, ws, wz, None, 1 / 128, 128, torch.uint8, "tanh", [], "").cpu()
+    r = torch.tanh(((x.cpu().float() - 128) * 0.02) @ (w.cpu().float() * 0.01))
+    assert (y.int() - torch.clamp(torch.round(r * 128 + 128), 0, 255).int()).abs().max() <= 1

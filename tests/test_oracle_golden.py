@@ -184,3 +184,35 @@ def test_linear_dynamic(golden, c):
     y = oracle.linear_dynamic(c["x"], c["wq"], c["w_scales"], c["bias"], c["relu"], c["reduce_range"])
     assert y.dtype == np.float32 and y.shape == golden[k + "/y"].shape
     np.testing.assert_array_equal(y, golden[k + "/y"])
+
+
+def _close_to(y, want, out_dtype, what):
+    assert y.shape == want.shape and y.dtype == want.dtype, what
+    if out_dtype == "float32":
+        np.testing.assert_allclose(y, want, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(want).max())), err_msg=what)
+    else:
+        d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+        assert d.max() <= 1, f"{what}: max diff {d.max()}"
+        assert np.count_nonzero(d) <= 0.002 * d.size + 1, f"{what}: {np.count_nonzero(d)} of {d.size} differ"
+
+
+@pytest.mark.parametrize("c", cases.plain_linear_cases(), ids=lambda c: c["name"])
+def test_plain_linear(golden, c):
+    # golden = PyTorch's oneDNN CPU op, which the reference's tests compare with
+    k = "plainlin/" + c["name"]
+    assert int(golden[k + "/x_crc"]) == cases.crc(c["x"]) and int(golden[k + "/w_crc"]) == cases.crc(c["w"])
+    y = oracle.plain_linear(c["x"], c["x_scale"], c["x_zp"], c["w"], c["w_scale"], c["bias"], c["out_scale"],
+                            c["out_zp"], c["out_dtype"], c["post"])
+    _close_to(y, golden[k + "/y"], c["out_dtype"], c["name"])
+    if c["name"].startswith("ref"):   # small integers, unit scales: exact in any order
+        np.testing.assert_array_equal(y, golden[k + "/y"])
+
+
+@pytest.mark.parametrize("c", cases.plain_conv_cases(), ids=lambda c: c["name"])
+def test_plain_conv(golden, c):
+    k = "plainconv/" + c["name"]
+    assert int(golden[k + "/x_crc"]) == cases.crc(c["x"]) and int(golden[k + "/w_crc"]) == cases.crc(c["w"])
+    y = oracle.plain_conv(c["x"], c["x_scale"], c["x_zp"], c["w"], c["w_scale"], c["bias"], c["stride"], c["pad"],
+                          c["groups"], c["out_scale"], c["out_zp"], c["out_dtype"], c["relu"], c["accum"],
+                          c["accum_scale"], c["accum_zp"])
+    _close_to(y, golden[k + "/y"], c["out_dtype"], c["name"])

@@ -809,6 +809,253 @@ at::Tensor qadaptive_avgpool2d_run(const at::Tensor& input, c10::SymIntArrayRef 
   return input.dim() == 3 ? y.squeeze(0) : y;
 }
 
+// ---------------------------------------------------------------------------
+// quantized::linear_per_tensor, quantized::conv, quantized::conv_binary: the
+// lowering targets of the reference's PT2E path (torch_musa/core/lowering.py:7-60),
+// defined by its patch of ATen's quantized/library.cpp (lines 20-22) and
+// implemented there as dequantize -> fp32 matmul / conv -> requantize fallbacks
+// ("todo W8A8 kernel", mudnn/Qlinear.cpp:36-69, mudnn/Qconv.cpp:45-86,137-181).
+// Activations and weights are plain uint8 / int8 tensors with their parameters
+// passed beside them.  Here the products run on the int8 kernels; the weight
+// is re-tiled on every call because the schema carries no packed object.
+// ---------------------------------------------------------------------------
+struct PlainOut {
+  bool is_int = false, is_signed = false;
+  c10::ScalarType dtype = c10::kFloat;
+};
+PlainOut plain_out(std::optional<c10::ScalarType> output_dtype, c10::ScalarType act_dtype, const char* what) {
+  PlainOut o;
+  o.dtype = output_dtype.value_or(act_dtype);
+  if (o.dtype == c10::kByte || o.dtype == c10::kChar) {
+    o.is_int = true;
+    o.is_signed = o.dtype == c10::kChar;
+  } else {
+    TORCH_CHECK(o.dtype == c10::kFloat || o.dtype == c10::kBFloat16 || o.dtype == c10::kHalf, what,
+                ": output dtype must be uint8, int8 or a floating type, got ", toString(o.dtype));
+  }
+  return o;
+}
+bool plain_signed(const at::Tensor& t, const char* what) {
+  TORCH_CHECK(t.scalar_type() == c10::kByte || t.scalar_type() == c10::kChar, what,
+              ": expected a uint8 or int8 tensor, got ", toString(t.scalar_type()));
+  return t.scalar_type() == c10::kChar;
+}
+// per-output-channel weight scales as fp32 on the weight's device; zero points must be 0
+at::Tensor plain_weight_scales(const at::Tensor& w_scale, const at::Tensor& w_zero_point, int64_t channels,
+                               const at::Tensor& like, const char* what) {
+  TORCH_CHECK(w_scale.numel() == channels || w_scale.numel() == 1, what, ": expected ", channels,
+              " weight scales (or one), got ", w_scale.numel());
+  TORCH_CHECK(!w_zero_point.defined() || w_zero_point.numel() == 0 || !w_zero_point.ne(0).any().item<bool>(), what,
+              ": the int8 kernels take symmetric weights (zero point 0)");
+  return w_scale.to(like.device(), at::kFloat).contiguous().reshape({-1});
+}
+// requantize a float result the way the reference's fallback does (round half to even)
+at::Tensor plain_requant(const at::Tensor& r, double scale, int64_t zp, const PlainOut& o) {
+  if (!o.is_int) return r.to(o.dtype);
+  return at::clamp(at::round(r / scale + zp), o.is_signed ? -128 : 0, o.is_signed ? 127 : 255).to(o.dtype);
+}
+
+at::Tensor qlinear_per_tensor_run(at::Tensor act, double act_scale, int64_t act_zero_point, at::Tensor weight,
+                                  at::Tensor weight_scales, at::Tensor weight_zero_points,
+                                  std::optional<at::Tensor> bias, double output_scale, int64_t output_zero_point,
+                                  std::optional<c10::ScalarType> output_dtype, c10::string_view post_op_name,
+                                  torch::List<std::optional<at::Scalar>> /*post_op_args*/,
+                                  c10::string_view /*post_op_algorithm*/) {
+  const char* what = "quantized::linear_per_tensor";
+  TORCH_CHECK(act.dim() == 2, "qlinear: input dim should be 2, but got", act.dim());
+  TORCH_CHECK(weight.dim() == 2 && weight.scalar_type() == c10::kChar, what, ": weight must be a 2-D int8 tensor");
+  const bool x_signed = plain_signed(act, what);
+  const std::string post(post_op_name.data(), post_op_name.size());
+  TORCH_CHECK(post == "none" || post == "relu" || post == "tanh" || post == "gelu", what,
+              ": unsupported post op ", post);
+  const c10::OptionalDeviceGuard guard(at::device_of(act));
+  const int64_t M = act.size(0), K = act.size(1), N = weight.size(1);
+  TORCH_CHECK(weight.size(0) == K, what, ": weight is [", weight.size(0), ", ", N, "], the input has ", K, " features");
+  TORCH_CHECK(act_scale > 0 && output_scale > 0, what, ": scales must be positive");
+  const PlainOut o = plain_out(output_dtype, act.scalar_type(), what);
+  const at::Tensor ws = plain_weight_scales(weight_scales, weight_zero_points, N, act, what);
+  std::optional<at::Tensor> b;
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->numel() == N, what, ": bias must have ", N, " elements");
+    b = bias->to(act.device(), at::kFloat).contiguous();
+  }
+  const bool float_path = !o.is_int || post == "tanh" || post == "gelu";
+  at::Tensor y = float_path ? at::empty({M, N}, act.options().dtype(at::kFloat))
+                            : at::empty({M, N}, act.options().dtype(o.dtype));
+  if (y.numel() == 0) return float_path ? plain_requant(y, output_scale, output_zero_point, o) : y;
+  const auto stream = current_stream(act);
+  const at::Tensor x = act.contiguous();
+  const at::Tensor w_nk = weight.t().contiguous();  // [N, K], the layout the prepack reads
+  at::Tensor packed = at::empty({std::max<int64_t>(tmq_linear_packed_bytes(N, K), 16)}, act.options().dtype(at::kByte));
+  at::Tensor colsum = at::empty({N}, act.options().dtype(at::kInt));
+  check_status(tmq_linear_prepack(cptr<int8_t>(w_nk), N, K, K, packed.data_ptr(), mptr<int32_t>(colsum), stream),
+               "tmq_linear_prepack");
+  tmq_linear_desc d{};
+  d.M = M;
+  d.N = N;
+  d.K = K;
+  d.x = x.data_ptr();
+  d.ldx = K;
+  d.x_signed = x_signed;
+  d.x_zero_point = static_cast<int32_t>(act_zero_point);
+  d.x_scale = static_cast<float>(act_scale);
+  d.w_packed = packed.const_data_ptr();
+  d.w_colsum = cptr<int32_t>(colsum);
+  d.w_scales = cptr<float>(ws);
+  d.w_per_channel = ws.numel() > 1;
+  d.relu = post == "relu";
+  d.bias = b.has_value() ? cptr<float>(*b) : nullptr;
+  if (float_path) {
+    check_status(tmq_linear_f32(&d, nullptr, mptr<float>(y), N, stream), "tmq_linear_f32");
+    if (post == "tanh") y = at::tanh(y);
+    if (post == "gelu") y = at::gelu(y);
+    return plain_requant(y, output_scale, output_zero_point, o);
+  }
+  d.out_scale = static_cast<float>(output_scale);
+  d.out_zero_point = static_cast<int32_t>(output_zero_point);
+  d.out_signed = o.is_signed;
+  d.y = y.data_ptr();
+  d.ldy = N;
+  check_status(tmq_linear(&d, stream), "tmq_linear");
+  return y;
+}
+
+// Shared body of quantized::conv and quantized::conv_binary.
+at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero_point, const at::Tensor& weight,
+                       const at::Tensor& weight_scales, const at::Tensor& weight_zero_points,
+                       const std::optional<at::Tensor>& accum, double accum_scale, int64_t accum_zero_point,
+                       double alpha, const std::optional<at::Tensor>& bias, const torch::List<int64_t>& stride,
+                       const torch::List<int64_t>& padding, const torch::List<int64_t>& dilation, int64_t groups,
+                       double output_scale, int64_t output_zero_point, std::optional<c10::ScalarType> output_dtype,
+                       bool relu, const char* what) {
+  TORCH_CHECK(act.dim() == 4 && weight.dim() == 4, what, ": expected 4-D input and weight");
+  TORCH_CHECK(weight.scalar_type() == c10::kChar, what, ": weight must be int8");
+  TORCH_CHECK(stride.size() == 2 && padding.size() == 2 && dilation.size() == 2, what,
+              ": stride, padding and dilation need two elements each");
+  const bool x_signed = plain_signed(act, what);
+  TORCH_CHECK(act_scale > 0 && output_scale > 0, what, ": scales must be positive");
+  const c10::OptionalDeviceGuard guard(at::device_of(act));
+  const PlainOut o = plain_out(output_dtype, act.scalar_type(), what);
+  tmq_conv2d_desc d{};
+  tmq_conv2d_geom& g = d.geom;
+  g.B = act.size(0);
+  g.IC = act.size(1);
+  g.H = act.size(2);
+  g.W = act.size(3);
+  g.OC = weight.size(0);
+  g.KH = weight.size(2);
+  g.KW = weight.size(3);
+  g.stride_h = stride[0];
+  g.stride_w = stride[1];
+  g.pad_h = padding[0];
+  g.pad_w = padding[1];
+  g.dil_h = dilation[0];
+  g.dil_w = dilation[1];
+  g.groups = groups;
+  TORCH_CHECK(groups > 0 && g.OC % groups == 0 && g.IC == weight.size(1) * groups, what, ": input has ", g.IC,
+              " channels, weight expects ", weight.size(1) * groups, " in ", groups, " groups");
+  const at::Tensor ws = plain_weight_scales(weight_scales, weight_zero_points, g.OC, act, what);
+  std::optional<at::Tensor> b;
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->numel() == g.OC, what, ": bias must have ", g.OC, " elements");
+    b = bias->to(act.device(), at::kFloat).contiguous();
+  }
+  int64_t OH = (g.H + 2 * g.pad_h - g.dil_h * (g.KH - 1) - 1) / g.stride_h + 1;
+  int64_t OW = (g.W + 2 * g.pad_w - g.dil_w * (g.KW - 1) - 1) / g.stride_w + 1;
+  TORCH_CHECK(OH > 0 && OW > 0, what, ": the kernel does not fit the padded input");
+  const auto stream = current_stream(act);
+  const at::Tensor x = act.contiguous(c10::MemoryFormat::ChannelsLast);
+  const at::Tensor w_ohwi = weight.permute({0, 2, 3, 1}).contiguous();
+  at::Tensor packed = at::empty({std::max<int64_t>(tmq_conv2d_packed_bytes(&g), 16)}, act.options().dtype(at::kByte));
+  at::Tensor colsum = at::empty({g.OC}, act.options().dtype(at::kInt));
+  if (g.B > 0)
+    check_status(tmq_conv2d_prepack(cptr<int8_t>(w_ohwi), &g, packed.data_ptr(), mptr<int32_t>(colsum), stream),
+                 "tmq_conv2d_prepack");
+  d.x = x.data_ptr();
+  d.x_signed = x_signed;
+  d.x_zero_point = static_cast<int32_t>(act_zero_point);
+  d.x_scale = static_cast<float>(act_scale);
+  d.w_per_channel = ws.numel() > 1;
+  d.w_packed = packed.const_data_ptr();
+  d.w_colsum = cptr<int32_t>(colsum);
+  d.w_scales = cptr<float>(ws);
+  d.bias = b.has_value() ? cptr<float>(*b) : nullptr;
+  const std::vector<int64_t> out_shape{g.B, g.OC, OH, OW};
+  if (accum.has_value())
+    TORCH_CHECK(accum->sizes() == c10::IntArrayRef(out_shape) && accum->device() == act.device(), what,
+                ": accum must have the output's shape ", c10::IntArrayRef(out_shape), " and device");
+  if (!o.is_int) {
+    // float output: exact int32 accumulators from the MFMA kernel, scaled here
+    TORCH_CHECK(!accum.has_value() || accum_scale == 1.0, "fp32 or bf16 output, accum_scale must be 1.0.");
+    at::Tensor acc = at::empty({g.B, OH, OW, g.OC}, act.options().dtype(at::kInt));
+    if (acc.numel() > 0) check_status(tmq_conv2d_acc32(&d, mptr<int32_t>(acc), stream), "tmq_conv2d_acc32");
+    at::Tensor r = acc.to(at::kFloat) * (ws * static_cast<float>(act_scale));
+    if (b.has_value()) r = r + *b;
+    r = r.permute({0, 3, 1, 2});  // NCHW-shaped, channels-last in memory
+    if (accum.has_value()) r = r + (accum->to(at::kFloat) - accum_zero_point) * (accum_scale * alpha);
+    if (relu) r = at::relu(r);
+    return r.to(o.dtype);
+  }
+  at::Tensor y = at::empty(out_shape, act.options().dtype(o.dtype), c10::MemoryFormat::ChannelsLast);
+  if (y.numel() == 0) return y;
+  d.out_scale = static_cast<float>(output_scale);
+  d.out_zero_point = static_cast<int32_t>(output_zero_point);
+  d.out_signed = o.is_signed;
+  d.relu = relu;
+  d.y = y.data_ptr();
+  if (!accum.has_value()) {
+    check_status(tmq_conv2d(&d, stream), "tmq_conv2d");
+    return y;
+  }
+  const bool a_signed = plain_signed(*accum, what);
+  const at::Tensor a_nhwc = accum->contiguous(c10::MemoryFormat::ChannelsLast);
+  tmq_conv2d_post post{};
+  post.accum = a_nhwc.data_ptr();
+  post.accum_signed = a_signed;
+  post.accum_zero_point = static_cast<int32_t>(accum_zero_point);
+  post.accum_scale = static_cast<float>(accum_scale * alpha);
+  post.activation = relu ? 1 : 0;
+  check_status(tmq_conv2d_fused(&d, &post, stream), "tmq_conv2d_fused");
+  return y;
+}
+
+at::Tensor qconv_pointwise_run(at::Tensor act, double act_scale, int64_t act_zero_point, at::Tensor weight,
+                               at::Tensor weight_scales, at::Tensor weight_zero_points,
+                               std::optional<at::Tensor> bias, torch::List<int64_t> stride,
+                               torch::List<int64_t> padding, torch::List<int64_t> dilation, int64_t groups,
+                               double output_scale, int64_t output_zero_point,
+                               std::optional<c10::ScalarType> output_dtype, c10::string_view attr,
+                               torch::List<std::optional<at::Scalar>> /*scalars*/,
+                               std::optional<c10::string_view> /*algorithm*/) {
+  const std::string a(attr.data(), attr.size());
+  // the reference also lets hardtanh / hardswish / swish through its check and then
+  // ignores them (mudnn/Qconv.cpp:38-44,63-65); they are refused here instead
+  TORCH_CHECK(a == "none" || a == "relu", "quantized::conv: unsupported post operation ", a);
+  return qconv_plain(act, act_scale, act_zero_point, weight, weight_scales, weight_zero_points, std::nullopt, 1.0, 0,
+                     1.0, bias, stride, padding, dilation, groups, output_scale, output_zero_point, output_dtype,
+                     a == "relu", "quantized::conv");
+}
+
+at::Tensor qconv_binary_run(at::Tensor act, double act_scale, int64_t act_zero_point, at::Tensor weight,
+                            at::Tensor weight_scales, at::Tensor weight_zero_points, at::Tensor accum,
+                            std::optional<at::Tensor> bias, torch::List<int64_t> stride,
+                            torch::List<int64_t> padding, torch::List<int64_t> dilation, int64_t groups,
+                            double output_scale, int64_t output_zero_point,
+                            std::optional<c10::ScalarType> output_dtype, double accum_scale,
+                            int64_t accum_zero_point, c10::string_view binary_attr, std::optional<at::Scalar> alpha,
+                            std::optional<c10::string_view> unary_attr,
+                            torch::List<std::optional<at::Scalar>> /*unary_scalars*/,
+                            std::optional<c10::string_view> /*unary_algorithm*/) {
+  const std::string bin(binary_attr.data(), binary_attr.size());
+  const std::string un = unary_attr.has_value() ? std::string(unary_attr->data(), unary_attr->size()) : "none";
+  TORCH_CHECK(act.dim() == 4 && bin == "sum" && (un == "none" || un == "relu"),
+              "post_op sum or post_op sum_relu is supported for quantized pointwise conv2d. Got binary_post_op: ",
+              bin, " unary_post_op: ", un, ".");
+  return qconv_plain(act, act_scale, act_zero_point, weight, weight_scales, weight_zero_points, accum, accum_scale,
+                     accum_zero_point, alpha.has_value() ? alpha->to<double>() : 1.0, bias, stride, padding, dilation,
+                     groups, output_scale, output_zero_point, output_dtype, un == "relu", "quantized::conv_binary");
+}
+
 }  // namespace
 
 // The two SiLU schemas are not part of upstream PyTorch; the reference adds them
@@ -823,6 +1070,21 @@ TORCH_LIBRARY_FRAGMENT(quantized, m) {
       "quantized::conv2d_add_silu(Tensor qx, Tensor qaccum, "
       "__torch__.torch.classes.quantized.Conv2dPackedParamsBase packed_weight, float output_scale, "
       "int output_zero_point) -> Tensor"));
+  // torch_patches/aten_src_ATen_native_quantized_library.cpp.patch:20-22
+  m.def(TORCH_SELECTIVE_SCHEMA(
+      "quantized::linear_per_tensor(Tensor qx, float x_scale, int x_zero_point, Tensor qw, Tensor w_scale, "
+      "Tensor w_zero_point,  Tensor? bias, float output_scale, int output_zero_point, ScalarType? output_dtype, "
+      "str post_op_name, Scalar?[] post_op_args, str post_op_algorithm) -> Tensor"));
+  m.def(TORCH_SELECTIVE_SCHEMA(
+      "quantized::conv(Tensor qx, float x_scale, int x_zero_point, Tensor qw, Tensor w_scale, Tensor w_zero_point, "
+      "Tensor? bias, int[] stride, int[] padding, int[] dilation, int groups, float output_scale, "
+      "int output_zero_point, ScalarType? output_dtype, str attr, Scalar?[] scalars, str? algorithm) -> Tensor"));
+  m.def(TORCH_SELECTIVE_SCHEMA(
+      "quantized::conv_binary(Tensor qx, float x_scale, int x_zero_point, Tensor qw, Tensor w_scale, "
+      "Tensor w_zero_point, Tensor qaccum, Tensor? bias, int[] stride, int[] padding, int[] dilation, int groups, "
+      "float output_scale, int output_zero_point, ScalarType? output_dtype, float accum_scale, "
+      "int accum_zero_point, str binary_attr, Scalar? alpha, str? unary_attr, Scalar?[] unary_scalars, "
+      "str? unary_algorithm) -> Tensor"));
 }
 
 TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
@@ -845,6 +1107,10 @@ TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
 TORCH_LIBRARY_IMPL(quantized, CUDA, m) {
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear_dynamic"), TORCH_FN(qlinear_dynamic_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear_relu_dynamic"), TORCH_FN(qlinear_relu_dynamic_run));
+  // plain uint8 / int8 tensors with their parameters beside them
+  m.impl(TORCH_SELECTIVE_NAME("quantized::linear_per_tensor"), TORCH_FN(qlinear_per_tensor_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv"), TORCH_FN(qconv_pointwise_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv_binary"), TORCH_FN(qconv_binary_run));
 }
 
 // Replacing PyTorch's own GPU kernel of aten::quantize_per_tensor_dynamic is the
