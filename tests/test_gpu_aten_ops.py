@@ -597,3 +597,49 @@ def test_plain_ops_errors():
     y = call(x, 0.02, 128, w, ws, wz, None, 1 / 128, 128, torch.uint8, "tanh", [], "").cpu()
     r = torch.tanh(((x.cpu().float() - 128) * 0.02) @ (w.cpu().float() * 0.01))
     assert (y.int() - torch.clamp(torch.round(r * 128 + 128), 0, 255).int()).abs().max() <= 1
+
+
+def test_quantized_modules_to_device():
+    # a populated CPU model (conv -> relu -> pool -> flatten -> linear, dynamic linear beside
+    # it) moved to the GPU with its packed parameters; same bytes out as on the CPU
+    say("quantized_modules_to")
+    import torch.ao.nn.quantized.dynamic as nnqd
+    import torch_musa_amd
+    torch.manual_seed(11)
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = nniq.ConvReLU2d(16, 32, 3, padding=1)
+            self.pool = torch.nn.AdaptiveAvgPool2d((2, 2))
+            self.fc = nnq.Linear(128, 24)
+            self.dyn = nnqd.Linear(24, 10)
+
+        def forward(self, xq):
+            y = self.fc(torch.flatten(self.pool(self.conv(xq)), 1))
+            return y, self.dyn(y.dequantize())
+
+    net = Net()
+    wc = torch.randn(32, 16, 3, 3) * 0.1
+    net.conv.set_weight_bias(torch.quantize_per_channel(wc, wc.abs().amax(dim=(1, 2, 3)).double() / 127,
+                                                        torch.zeros(32, dtype=torch.int64), 0, torch.qint8),
+                             torch.randn(32))
+    net.conv.scale, net.conv.zero_point = 0.05, 0
+    wl = torch.randn(24, 128) * 0.1
+    net.fc.set_weight_bias(torch.quantize_per_tensor(wl, float(wl.abs().max() / 127), 0, torch.qint8), torch.randn(24))
+    net.fc.scale, net.fc.zero_point = 0.1, 128
+    wd = torch.randn(10, 24) * 0.2
+    net.dyn.set_weight_bias(torch.quantize_per_tensor(wd, float(wd.abs().max() / 127), 0, torch.qint8), torch.randn(10))
+    xq = torch.quantize_per_tensor(torch.randn(3, 16, 8, 8), 0.03, 128, torch.quint8)
+    q_cpu, f_cpu = net(xq)
+    torch_musa_amd.quantized_modules_to(net, "cuda")
+    q_gpu, f_gpu = net(xq.cuda())
+    assert q_gpu.is_cuda and f_gpu.is_cuda
+    d = (q_gpu.int_repr().cpu().int() - q_cpu.int_repr().int()).abs().max().item()
+    assert d <= 1, f"quantized head differs by {d}"
+    if d == 0:
+        assert torch.equal(f_gpu.cpu(), f_cpu)
+    # and back
+    torch_musa_amd.quantized_modules_to(net, "cpu")
+    q2, f2 = net(xq)
+    assert torch.equal(q2.int_repr(), q_cpu.int_repr()) and torch.equal(f2, f_cpu)

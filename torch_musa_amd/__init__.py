@@ -27,7 +27,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_KERNELS = os.path.join(_PKG, "libtmq.so")
 LIB_ATEN = os.path.join(_PKG, "libtmq_aten.so")
 
-__all__ = ["LIB_KERNELS", "LIB_ATEN", "is_loaded", "load", "quantized_device"]
+__all__ = ["LIB_KERNELS", "LIB_ATEN", "is_loaded", "load", "quantized_device", "quantized_modules_to"]
 
 _loaded = False
 
@@ -59,6 +59,42 @@ def quantized_device() -> torch.device:
     if not torch.cuda.is_available():
         raise RuntimeError("no MI355X visible: the tmq operators have no CPU path")
     return torch.device("cuda", torch.cuda.current_device())
+
+
+def _qtensor_to(t, device):
+    """A dense copy of a (possibly per-channel, possibly strided) quantized tensor on ``device``."""
+    if t is None or not t.is_quantized:
+        return None if t is None else t.to(device)
+    codes = t.int_repr().contiguous().to(device)
+    if t.qscheme() in (torch.per_tensor_affine, torch.per_tensor_symmetric):
+        return torch._make_per_tensor_quantized_tensor(codes, t.q_scale(), t.q_zero_point())
+    return torch._make_per_channel_quantized_tensor(codes, t.q_per_channel_scales().to(device),
+                                                    t.q_per_channel_zero_points().to(device),
+                                                    t.q_per_channel_axis())
+
+
+def quantized_modules_to(module: torch.nn.Module, device) -> torch.nn.Module:
+    """Move a populated quantized model to ``device``, packed parameters included.
+
+    ``nn.Module.to`` moves parameters and buffers but not the packed-parameter
+    objects that ``torch.ao.nn.quantized`` (and ``.dynamic``, ``.intrinsic``)
+    modules hold, and unpickling such an object re-creates it with the CPU
+    engine.  The reference leaves this to the caller, who re-populates each
+    module with ``set_weight_bias`` on device tensors
+    (tests/unittest/quantized/test_quantized_linear.py:58-60,87-89); this does
+    the same for every submodule that has the ``_weight_bias`` /
+    ``set_weight_bias`` pair, in place, and returns ``module``.
+    """
+    device = torch.device(device)
+    repack = []
+    for m in module.modules():
+        if callable(getattr(m, "_weight_bias", None)) and callable(getattr(m, "set_weight_bias", None)):
+            w, b = m._weight_bias()
+            repack.append((m, w, b))
+    module.to(device)
+    for m, w, b in repack:
+        m.set_weight_bias(_qtensor_to(w, device), _qtensor_to(b, device))
+    return module
 
 
 load()
