@@ -287,6 +287,40 @@ def main():
                              "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
                 "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
                 "algorithmic_bytes_per_launch": nbytes}
+
+        # ----------------------------- dynamically quantized linear, decode-sized
+        # fp32 [M, 4096] -> fp32 [M, 4096]: one launch for range + parameters + codes,
+        # one for the product; 40 cold weights replayed in one HIP graph as above
+        for Md in (1, 16):
+            xdf = torch.randn(Md, Kd, device=dev)
+
+            def run_dyn():
+                for p in pws:
+                    cabi.linear_dynamic(xdf, p, wsd, bd)
+
+            run_dyn()
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                run_dyn()
+                side.synchronize()
+                with torch.cuda.graph(graph, stream=side):
+                    run_dyn()
+            torch.cuda.synchronize()
+            for _ in range(3):
+                graph.replay()
+            ts = events_ms(graph.replay, 10)
+            per = sum(ts) / len(ts) / sets
+            nbytes = Nd * Kd + 2 * 4 * Md * Kd + 2 * Md * Kd + 4 * Md * Nd + 12 * Nd
+            gbs = nbytes / (per * 1e-3) / 1e9
+            log(f"[bench] dynamic decode M={Md}: {per*1e3:.2f} us per call (2 launches) in a replayed graph")
+            secondary[f"linear_dynamic_decode_m{Md}"] = {
+                "avg_call_us": round(per * 1e3, 3), "value": round(gbs, 1), "unit": "GB/s",
+                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
+                "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
+                "algorithmic_bytes_per_call": nbytes}
         del pws
 
         # ------------------------------------------- dynamically quantized linear

@@ -98,6 +98,14 @@ int tmq_choose_qparams_dev(const float* minmax, int q_signed, int reduce_range,
 int tmq_quantize_per_tensor_dev(const float* x, void* q, int64_t n,
                                 const tmq_qparams* qparams, int q_signed,
                                 tmq_stream_t stream);
+/* The whole dynamic quantization on the device: min/max over x, the parameters
+ * into *qparams (device memory), the codes into q.  Small inputs (at most
+ * 65536 elements) take one launch, larger ones three; `workspace` as for
+ * tmq_minmax (unused, and may be NULL, for the small case).  Same results as
+ * tmq_minmax + tmq_choose_qparams_dev + tmq_quantize_per_tensor_dev. */
+int tmq_quantize_per_tensor_dynamic_dev(const float* x, void* q, int64_t n, int q_signed,
+                                        int reduce_range, tmq_qparams* qparams, void* workspace,
+                                        size_t workspace_bytes, tmq_stream_t stream);
 /* Host-side ChooseQuantizationParams, same arithmetic (pure CPU, no GPU call). */
 int tmq_choose_qparams_host(float min, float max, int q_signed, int reduce_range,
                             double* scale, int32_t* zero_point);

@@ -275,3 +275,20 @@ def test_qadaptive_avgpool_resnet_head_sized(cabi):
     x = np.random.default_rng(5).integers(0, 256, (64, 7, 7, 2048)).astype(np.uint8)
     y = host(cabi.qadaptive_avgpool2d(dev(x), (1, 1), 128))
     np.testing.assert_array_equal(y, oracle.qadaptive_avgpool2d(x, (1, 1), 128))
+
+
+@pytest.mark.parametrize("n,offset", [(1, 0), (7, 0), (4096, 0), (4099, 1), (65536, 0), (65537, 0), (65541, 3),
+                                      (1 << 20, 0), ((1 << 20) + 3, 1)])
+@pytest.mark.parametrize("signed,reduce_range", [(False, False), (False, True), (True, False)])
+def test_quantize_dynamic_on_device(cabi, n, offset, signed, reduce_range):
+    # one call: range, parameters (left in device memory) and codes; small inputs take
+    # the single-block kernel, larger ones the three-launch chain -- same results
+    say("dynamic dev", n, offset, signed, reduce_range)
+    rng = np.random.default_rng(n + offset)
+    x = (rng.standard_normal(n + offset) * 2.5 + 0.4).astype(np.float32)
+    xd = dev(x)[offset:]
+    q, qp = cabi.quantize_per_tensor_dynamic_dev(xd.contiguous() if offset == 0 else xd, signed, reduce_range)
+    mn, mx = oracle.minmax(x[offset:])
+    scale, zp = oracle.choose_qparams(mn, mx, signed, reduce_range)
+    assert cabi.read_qparams(qp) == (scale, zp)
+    np.testing.assert_array_equal(host(q), oracle.quantize_per_tensor(x[offset:], scale, zp, signed))

@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32", "tmq_linear_f32",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32", "tmq_linear_f32", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d",
@@ -119,6 +119,7 @@ def lib() -> C.CDLL:
         l.tmq_linear.argtypes = [C.POINTER(LinearDesc), v]
         l.tmq_linear_acc32.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, v]
         l.tmq_linear_f32.argtypes = [C.POINTER(LinearDesc), v, v, C.c_int64, v]
+        l.tmq_quantize_per_tensor_dynamic_dev.argtypes = [v, v, C.c_int64, C.c_int, C.c_int, v, v, C.c_size_t, v]
         l.tmq_conv2d_prepack.argtypes = [v, C.POINTER(Conv2dGeom), v, v, v]
         l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         l.tmq_conv2d.argtypes = [C.POINTER(Conv2dDesc), v]
@@ -215,6 +216,18 @@ def quantize_per_tensor_dev(x: torch.Tensor, qp: torch.Tensor, signed: bool) -> 
                                             int(signed), stream_ptr()),
           "tmq_quantize_per_tensor_dev")
     return q
+
+
+def quantize_per_tensor_dynamic_dev(x: torch.Tensor, signed: bool, reduce_range: bool):
+    """-> (codes, 16 device bytes of qparams); one launch for small inputs, three otherwise."""
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    q = torch.empty(x.shape, dtype=torch.int8 if signed else torch.uint8, device=x.device)
+    qp = torch.empty(16, dtype=torch.uint8, device=x.device)
+    ws = minmax_workspace(x.device)
+    check(lib().tmq_quantize_per_tensor_dynamic_dev(x.data_ptr(), q.data_ptr(), x.numel(), int(signed),
+                                                    int(reduce_range), qp.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                    stream_ptr()), "tmq_quantize_per_tensor_dynamic_dev")
+    return q, qp
 
 
 def choose_qparams_host(mn: float, mx: float, signed: bool, reduce_range: bool):
@@ -337,8 +350,7 @@ def linear_dynamic(x, pw: PackedLinear, w_scales, bias, relu=False, reduce_range
     """min/max -> qparams -> quantize -> product, all on the device, no host round trip."""
     assert x.dtype == torch.float32 and x.is_contiguous()
     x2 = x.reshape(-1, x.shape[-1])
-    qp = choose_qparams_dev(minmax(x2), False, reduce_range)
-    xq = quantize_per_tensor_dev(x2, qp, False)
+    xq, qp = quantize_per_tensor_dynamic_dev(x2, False, reduce_range)
     y = linear_f32(xq, pw, 1.0, 0, w_scales, bias, relu, qparams_dev=qp)
     return y.reshape(tuple(x.shape[:-1]) + (pw.N,))
 

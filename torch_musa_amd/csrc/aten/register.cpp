@@ -300,8 +300,9 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     return apply_impl(input, output_scale, output_zero_point, true);
   }
   // The reference declares these and throws (mudnn/Linear.h:35-46).  Here:
-  // min/max -> qparams -> quint8 activations -> int8 product -> fp32 output,
-  // five launches on the current stream, the parameters never visit the host.
+  // min/max -> qparams -> quint8 activations -> int8 product -> fp32 output on
+  // the current stream (two launches for decode-sized inputs, four otherwise),
+  // the parameters never visit the host.
   at::Tensor apply_dynamic(at::Tensor input, bool reduce_range) override {
     return apply_dynamic_impl(input, reduce_range, false);
   }
@@ -362,16 +363,12 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     const auto stream = current_stream(x);
     const auto bytes = x.options().dtype(at::kByte);
     at::Tensor ws = at::empty({static_cast<int64_t>(tmq_minmax_workspace_bytes(x.numel()))}, bytes);
-    at::Tensor mm = at::empty({2}, x.options());
     at::Tensor qp = at::empty({static_cast<int64_t>(sizeof(tmq_qparams))}, bytes);
     at::Tensor xq = at::empty({x.numel()}, bytes);
-    check_status(tmq_minmax(cptr<float>(x), x.numel(), mptr<float>(mm), ws.data_ptr(),
-                            static_cast<size_t>(ws.numel()), stream),
-                 "tmq_minmax");
     auto* qpd = static_cast<tmq_qparams*>(qp.data_ptr());
-    check_status(tmq_choose_qparams_dev(cptr<float>(mm), 0, reduce_range, qpd, stream), "tmq_choose_qparams_dev");
-    check_status(tmq_quantize_per_tensor_dev(cptr<float>(x), xq.data_ptr(), x.numel(), qpd, 0, stream),
-                 "tmq_quantize_per_tensor_dev");
+    check_status(tmq_quantize_per_tensor_dynamic_dev(cptr<float>(x), xq.data_ptr(), x.numel(), 0, reduce_range, qpd,
+                                                     ws.data_ptr(), static_cast<size_t>(ws.numel()), stream),
+                 "tmq_quantize_per_tensor_dynamic_dev");
     tmq_linear_desc d{};
     d.M = M;
     d.N = N_;

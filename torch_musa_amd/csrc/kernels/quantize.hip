@@ -307,6 +307,104 @@ __global__ void choose_qparams_kernel(const float* __restrict__ minmax, int qmin
   }
 }
 
+// Last stage of the min/max reduction and ChooseQuantizationParams in one block.
+__global__ __launch_bounds__(kThreads) void minmax_final_choose_kernel(
+    const float* __restrict__ partials, int count, int qmin, int qmax, int reduce_range,
+    float* __restrict__ minmax_out, tmq_qparams* __restrict__ out) {
+  __shared__ float s_mm[2];
+  float mn = std::numeric_limits<float>::infinity();
+  float mx = -std::numeric_limits<float>::infinity();
+  for (int i = threadIdx.x; i < count; i += kThreads) {
+    mn = fminf(mn, partials[2 * i]);
+    mx = fmaxf(mx, partials[2 * i + 1]);
+  }
+  block_minmax_store(mn, mx, s_mm);
+  if (threadIdx.x == 0) {
+    double s;
+    int32_t z;
+    choose_qparams(s_mm[0], s_mm[1], qmin, qmax, reduce_range != 0, &s, &z);
+    out->scale = s;
+    out->zero_point = z;
+    out->reserved = 0;
+    if (minmax_out != nullptr) {
+      minmax_out[0] = s_mm[0];
+      minmax_out[1] = s_mm[1];
+    }
+  }
+}
+
+// Dynamic quantization of a small tensor in one launch: one block finds the
+// range, chooses the parameters and converts.  A decode-sized activation
+// ([1..16, 4096] floats) is a few tens of KB: three dependent launches would
+// cost several times what the work does.
+constexpr int kDynSmallThreads = 1024;
+constexpr int64_t kDynSmallMax = 65536;  // elements
+template <bool SIGNED>
+__global__ __launch_bounds__(kDynSmallThreads) void dynamic_quantize_small_kernel(
+    const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, int qmin, int qmax,
+    int reduce_range, bool vec, tmq_qparams* __restrict__ out) {
+  __shared__ float s_mn[kDynSmallThreads / kWave], s_mx[kDynSmallThreads / kWave];
+  __shared__ float s_inv, s_zp;
+  const int t = threadIdx.x;
+  const int64_t n4 = vec ? n / 4 : 0;
+  const v4f* x4 = reinterpret_cast<const v4f*>(x);
+  // the whole input fits the block's registers (kDynSmallMax / 4 / threads = 16
+  // groups of four per thread): memory is read once, all loads in flight together
+  constexpr int kHeld = static_cast<int>(kDynSmallMax / 4 / kDynSmallThreads);
+  v4f held[kHeld];
+#pragma unroll
+  for (int u = 0; u < kHeld; ++u) {
+    const int64_t i = t + static_cast<int64_t>(u) * kDynSmallThreads;
+    if (i < n4) held[u] = x4[i];
+  }
+  float mn = std::numeric_limits<float>::infinity();
+  float mx = -std::numeric_limits<float>::infinity();
+#pragma unroll
+  for (int u = 0; u < kHeld; ++u) {
+    const int64_t i = t + static_cast<int64_t>(u) * kDynSmallThreads;
+    if (i < n4) {
+      const v4f v = held[u];
+      mn = fminf(fminf(mn, v.x), fminf(v.y, fminf(v.z, v.w)));
+      mx = fmaxf(fmaxf(mx, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
+    }
+  }
+  for (int64_t i = 4 * n4 + t; i < n; i += kDynSmallThreads) {
+    mn = fminf(mn, x[i]);
+    mx = fmaxf(mx, x[i]);
+  }
+  wave_minmax(mn, mx);
+  if (t % kWave == 0) {
+    s_mn[t / kWave] = mn;
+    s_mx[t / kWave] = mx;
+  }
+  __syncthreads();
+  if (t == 0) {
+#pragma unroll
+    for (int w = 1; w < kDynSmallThreads / kWave; ++w) {
+      mn = fminf(mn, s_mn[w]);
+      mx = fmaxf(mx, s_mx[w]);
+    }
+    double s;
+    int32_t z;
+    choose_qparams(mn, mx, qmin, qmax, reduce_range != 0, &s, &z);
+    out->scale = s;
+    out->zero_point = z;
+    out->reserved = 0;
+    s_inv = 1.0f / static_cast<float>(s);  // IEEE division, as in resolve()
+    s_zp = static_cast<float>(z);
+  }
+  __syncthreads();
+  const float inv = s_inv, zp_f = s_zp;
+  uint32_t* q4 = reinterpret_cast<uint32_t*>(q);
+#pragma unroll
+  for (int u = 0; u < kHeld; ++u) {
+    const int64_t i = t + static_cast<int64_t>(u) * kDynSmallThreads;
+    if (i < n4) q4[i] = quantize_four<SIGNED>(held[u], inv, zp_f);
+  }
+  for (int64_t i = 4 * n4 + t; i < n; i += kDynSmallThreads)
+    q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(x[i], inv, zp_f));
+}
+
 // ---------------------------------------------------------------------------
 // Per-channel kernels over [outer, C, inner].  VEC = 4 when inner % 4 == 0 and
 // the pointers are 16-byte aligned (a group of 4 never straddles a channel).
@@ -552,6 +650,45 @@ TMQ_EXPORT int tmq_choose_qparams_dev(const float* minmax, int q_signed, int red
   choose_qparams_kernel<<<dim3(1), dim3(kWave), 0, as_stream(stream)>>>(
       minmax, q_signed ? -128 : 0, q_signed ? 127 : 255, reduce_range, qparams);
   return launch_status();
+}
+
+TMQ_EXPORT int tmq_quantize_per_tensor_dynamic_dev(const float* x, void* q, int64_t n, int q_signed,
+                                                   int reduce_range, tmq_qparams* qparams, void* workspace,
+                                                   size_t workspace_bytes, tmq_stream_t stream) {
+  if (n < 0 || qparams == nullptr || (n > 0 && (x == nullptr || q == nullptr))) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!aligned(x, 4)) return TMQ_ERR_ALIGNMENT;
+  hipStream_t s = as_stream(stream);
+  const int qmin = q_signed ? -128 : 0, qmax = q_signed ? 127 : 255;
+  if (n <= kDynSmallMax) {
+    const bool vec = aligned(x, 16) && aligned(q, 4);
+    uint8_t* qb = static_cast<uint8_t*>(q);
+    if (q_signed)
+      dynamic_quantize_small_kernel<true><<<dim3(1), dim3(kDynSmallThreads), 0, s>>>(x, qb, n, qmin, qmax,
+                                                                                      reduce_range, vec, qparams);
+    else
+      dynamic_quantize_small_kernel<false><<<dim3(1), dim3(kDynSmallThreads), 0, s>>>(x, qb, n, qmin, qmax,
+                                                                                       reduce_range, vec, qparams);
+    return launch_status();
+  }
+  if (workspace == nullptr || workspace_bytes < tmq_minmax_workspace_bytes(n) || !aligned(workspace, 4))
+    return TMQ_ERR_WORKSPACE;
+  float* partials = static_cast<float*>(workspace);
+  const uintptr_t mis = reinterpret_cast<uintptr_t>(x) & 15u;
+  int64_t head = mis == 0 ? 0 : static_cast<int64_t>((16 - mis) / 4);
+  if (head > n) head = n;
+  const int64_t n4 = (n - head) / 4;
+  const unsigned g = grid_for(n4, kThreads * kUnroll, kMinMaxMaxBlocks);
+  minmax_partial_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(reinterpret_cast<const v4f*>(x + head), n4, x, head,
+                                                           n, partials);
+  if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  minmax_final_choose_kernel<<<dim3(1), dim3(kThreads), 0, s>>>(partials, static_cast<int>(g), qmin, qmax,
+                                                                reduce_range, nullptr, qparams);
+  if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  QParamsArg qp;
+  qp.inv = 0.f;
+  qp.zp_f = 0.f;
+  qp.dev = qparams;
+  return quantize_launch(x, q, n, qp, q_signed, s);
 }
 
 TMQ_EXPORT int tmq_choose_qparams_host(float min, float max, int q_signed, int reduce_range,
