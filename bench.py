@@ -42,7 +42,7 @@ PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
 # 1 048 576 KiB actually read (factor 2.0), WRITE_SIZE reads 1 048 576 (factor 1.0).
 # Summaries: profiles/hbm_traffic_pmc.md.
 MEASURED_TRAFFIC = {
-    "linear_c3": int((161_200 * 2.0 + 44_030) * 1024),      # 375 MB: operands re-fetched 5.3x by the 8 L2s
+    "linear_c3": int((161_100 * 2.0 + 44_030) * 1024),      # 375 MB: operands re-fetched 5.3x by the 8 L2s
     "quantize_c2": int((524_300 * 2.0 + 262_100) * 1024),   # 1.342 GB = algorithmic
     "dequantize_c2": int((131_100 * 2.0 + 1_049_000) * 1024),
     "minmax_c2": int((524_300 * 2.0 + 64) * 1024),
