@@ -262,3 +262,52 @@ def test_linear_dynamic_prefill_sized(cabi):
     xq = oracle.quantize_per_tensor(x, scale, zp, False, nthreads=8)
     want = oracle.linear_f32(xq, scale, zp, wq, wsc, bias, nthreads=8)
     np.testing.assert_array_equal(y, want)
+
+
+def _random_shapes(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        m = int(rng.choice([1, 3, 17, 64, 65, 130, 255, 256, 257, 300, 513, 700]))
+        n = int(rng.choice([1, 5, 16, 31, 48, 100, 255, 256, 257, 300, 520, 777]))
+        k = int(rng.choice([16, 48, 64, 128, 144, 192, 208, 256, 320, 448, 1040]))
+        out.append((m, n, k))
+    return out
+
+
+@pytest.mark.parametrize("cfg", [-1, 6, 7])
+def test_random_shapes_against_oracle(cabi, cfg):
+    # ragged everything: rows, channels and k tails in all combinations, for the automatic
+    # choice and for the two direct-copy tiles (which fall back below three k stages)
+    for i, (m, n, k) in enumerate(_random_shapes(1234 + cfg, 24)):
+        say("random shape", cfg, m, n, k)
+        c = _tile_case(m, n, k, seed=7000 + 31 * i + cfg, x_signed=bool(i & 1), relu=bool(i & 2), bias=bool(i & 4),
+                       per_channel=not (i & 8))
+        y, acc, _ = _run(cabi, c, cfg)
+        np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]), err_msg=f"{(m, n, k)}")
+        want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                             c["out_scale"], c["out_zp"], relu=c["relu"])
+        _check(y, want, f"cfg {cfg} shape {(m, n, k)}")
+
+
+def test_row_pitch_and_output_pitch(cabi):
+    # activations and outputs that are column slices of wider buffers (ldx > K, ldy > N)
+    say("pitches")
+    c = _tile_case(300, 264, 320, seed=77)
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    xbig = torch.zeros((300, 320 + 64), dtype=torch.uint8, device="cuda")
+    xbig[:, 16:336] = dev(c["xq"])
+    ybig = torch.full((300, 264 + 40), 7, dtype=torch.uint8, device="cuda")
+    for cfg in (-1, 6, 7, 3):
+        cabi.force_linear_config(cfg)
+        try:
+            cabi.linear(xbig[:, 16:336], pw, c["x_scale"], c["x_zp"], dev(c["w_scales"].astype(np.float32)),
+                        dev(c["bias"]), c["out_scale"], c["out_zp"], out=ybig[:, 8:272])
+        finally:
+            cabi.force_linear_config(-1)
+        want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                             c["out_scale"], c["out_zp"])
+        got = host(ybig)
+        _check(got[:, 8:272], want, f"cfg {cfg}")
+        assert (got[:, :8] == 7).all() and (got[:, 272:] == 7).all()   # nothing written outside the slice
+        ybig.fill_(7)
