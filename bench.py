@@ -202,13 +202,18 @@ def main():
         # ---------------------------------------------- matrix-pipe ceiling probe
         log("[bench] int8 MFMA ceiling probe (register-only loop, 256 workgroups)")
         probe = {}
-        for mode, name in ((0, "zero_operands"), (1, "uniform_random_int8"), (2, "gaussian_int8")):
+        for mode, name in ((0, "zero_operands"), (1, "uniform_random_int8"), (2, "gaussian_int8"),
+                           (3, "gaussian_int8_fresh_from_lds")):
             tops_p, ghz_p = cabi.probe_mfma_i8(mode)
             probe[name] = {"tops": round(tops_p, 1), "shader_ghz": round(ghz_p, 3)}
             log(f"[bench]   {name}: {tops_p:.0f} TOP/s at {ghz_p:.2f} GHz")
         secondary["mfma_i8_ceiling_probe"] = probe
         roofline["power_limited_ceiling_tops"] = probe["gaussian_int8"]["tops"]
         roofline["frac_of_power_limited_ceiling"] = round(achieved / probe["gaussian_int8"]["tops"], 4)
+        # the same with operands that change every instruction, as a GEMM's do
+        roofline["fresh_operand_ceiling_tops"] = probe["gaussian_int8_fresh_from_lds"]["tops"]
+        roofline["frac_of_fresh_operand_ceiling"] = round(
+            achieved / probe["gaussian_int8_fresh_from_lds"]["tops"], 4)
 
         # -------------------------------------------------------------- C2
         n = 2 ** 28

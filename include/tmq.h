@@ -343,7 +343,9 @@ int tmq_qadaptive_avgpool2d(const void* x, void* y, int64_t B, int64_t H, int64_
  * Measurement probe (no counterpart in the reference; used by bench.py only).
  * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four
  * waves and reports the sustained rate in TOP/s and the shader clock in GHz.
- * data_mode 0: zero operands, 1: uniform random bytes, 2: Gaussian int8.
+ * data_mode 0: zero operands, 1: uniform random bytes, 2: Gaussian int8 (all
+ * held in registers), 3: Gaussian int8 operands read afresh from LDS for every
+ * instruction, eight waves per workgroup (the GEMM's loop without its copies).
  * Unlike every other entry point this one synchronises (default stream) and
  * creates two HIP events; `scratch` is >= 2 KiB of device memory.
  * ------------------------------------------------------------------------- */

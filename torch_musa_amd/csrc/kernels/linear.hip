@@ -323,7 +323,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     else
       cfg = 2;
   }
-  if (cfg == 6 && !dma_ok) cfg = 3;
+  if ((cfg == 6 || cfg == 10) && !dma_ok) cfg = 3;
   if (cfg == 7 && !dma_ok) cfg = 1;
   switch (cfg) {
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
@@ -334,6 +334,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 5: return launch_gemm<256, 128, 2, 2, MODE>(a, xs, s);
     case 6: return launch_gemm<256, 256, 2, 4, MODE, 3, true>(a, xs, s);
     case 7: return launch_gemm<128, 128, 2, 2, MODE, 3, true>(a, xs, s);
+    case 10: return launch_gemm<256, 256, 2, 2, MODE, 3, true>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }

@@ -28,7 +28,8 @@ __device__ __forceinline__ unsigned gaussian_bytes(unsigned seed) {
   return out;
 }
 
-// data_mode 0: zeros, 1: uniform random bytes, 2: Gaussian int8 (sigma ~37)
+// data_mode 0: zeros, 1: uniform random bytes, 2: Gaussian int8 (sigma ~37),
+// all three held in registers for the whole run
 __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int data_mode, int* sink,
                                                          long long* stamps) {
   v16i acc[8];
@@ -70,6 +71,58 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int data_mod
   }
 }
 
+// data_mode 3: the operands of every MFMA are fresh Gaussian bytes read from
+// LDS (12 ds_read_b128 per 16 MFMAs and one barrier per 16, the ratios of the
+// GEMM's main loop; eight waves per block, two per SIMD), nothing else: no
+// global traffic, no address arithmetic.  What this sustains is the ceiling for
+// a GEMM whose matrix pipe never waits, on operands that change every
+// instruction the way real data does.
+__global__ __launch_bounds__(512) void mfma_probe_lds_kernel(int iters, int* sink, long long* stamps) {
+  __shared__ __attribute__((aligned(16))) unsigned char smem[65536];
+  const int t = threadIdx.x;
+  for (int i = t; i < 65536 / 4; i += 512)
+    reinterpret_cast<unsigned*>(smem)[i] = gaussian_bytes(mix(i * 2654435761u + blockIdx.x * 977u));
+  __syncthreads();
+  v16i acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+  v4i f0[6], f1[6];
+  const int rd = (t & 63) * 16 + (t >> 6) * 4096;  // consecutive 16-byte slots per wave
+#pragma unroll
+  for (int i = 0; i < 6; ++i) f0[i] = *reinterpret_cast<const v4i*>(&smem[(rd + i * 1024) & 0xffff]);
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+    const int base = rd + it * 208;  // a different 16-byte-aligned window every iteration
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i < 6) f1[i] = *reinterpret_cast<const v4i*>(&smem[(base + i * 1024 + 8192) & 0xffff]);
+      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f0[i & 1], f0[2 + (i >> 1)], acc[i], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i < 6) f0[i] = *reinterpret_cast<const v4i*>(&smem[(base + i * 1024 + 24576) & 0xffff]);
+      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f1[i & 1], f1[2 + (i >> 1)], acc[i], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[i][r];
+  if (s == 0x7fffffff) sink[threadIdx.x & 255] = s;
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    stamps[0] = c1 - c0;
+    stamps[1] = w1 - w0;
+  }
+}
+
 }  // namespace
 }  // namespace tmq
 
@@ -81,16 +134,21 @@ using namespace tmq;
 // least 2 KiB owned by the caller.
 TMQ_EXPORT int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, double* tops,
                                  double* shader_ghz) {
-  if (data_mode < 0 || data_mode > 2 || blocks <= 0 || iters <= 0 || scratch == nullptr ||
+  if (data_mode < 0 || data_mode > 3 || blocks <= 0 || iters <= 0 || scratch == nullptr ||
       tops == nullptr || shader_ghz == nullptr)
     return TMQ_ERR_INVALID_ARGUMENT;
   int* sink = static_cast<int*>(scratch);
   long long* stamps = reinterpret_cast<long long*>(static_cast<char*>(scratch) + 1024);
   hipEvent_t e0, e1;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return TMQ_ERR_LAUNCH;
-  mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
+  // mode 3: eight waves per block and 16 MFMAs per wave and iteration: half the
+  // iterations give the same number of operations per block as the other modes
+  const int it3 = iters / 4 > 0 ? iters / 4 : 1;
+  if (data_mode == 3) mfma_probe_lds_kernel<<<dim3(blocks), dim3(512), 0, nullptr>>>(it3, sink, stamps);
+  else mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
   hipEventRecord(e0, nullptr);
-  mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
+  if (data_mode == 3) mfma_probe_lds_kernel<<<dim3(blocks), dim3(512), 0, nullptr>>>(it3, sink, stamps);
+  else mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
   hipEventRecord(e1, nullptr);
   int rc = hipEventSynchronize(e1) == hipSuccess ? TMQ_OK : TMQ_ERR_LAUNCH;
   float ms = 0.f;
@@ -101,7 +159,8 @@ TMQ_EXPORT int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scr
   hipEventDestroy(e0);
   hipEventDestroy(e1);
   if (rc != TMQ_OK) return rc;
-  const double ops = 2.0 * 32 * 32 * 32 * 8 * static_cast<double>(iters) * 4 * blocks;
+  const double ops = data_mode == 3 ? 2.0 * 32 * 32 * 32 * 16 * static_cast<double>(it3) * 8 * blocks
+                                    : 2.0 * 32 * 32 * 32 * 8 * static_cast<double>(iters) * 4 * blocks;
   *tops = ops / (ms * 1e-3) / 1e12;
   *shader_ghz = static_cast<double>(host[0]) / (static_cast<double>(host[1]) / 100e6) / 1e9;
   return TMQ_OK;
