@@ -18,6 +18,7 @@ namespace {
 
 constexpr int kEwThreads = 256;
 constexpr int kEwUnroll = 2;  // 16-byte accesses in flight per thread and operand
+constexpr int kReluUnroll = 4;  // one operand only: twice as many per thread
 
 struct AddParams {
   float a_scale, a_premul, b_scale, b_premul, inv_out, out_zp_f;
@@ -128,14 +129,23 @@ __global__ __launch_bounds__(kEwThreads) void qrelu_vec_kernel(const v4i* __rest
                                                                v4i* __restrict__ y16, int64_t n16,
                                                                const uint8_t* __restrict__ x,
                                                                uint8_t* __restrict__ y, int64_t n, int zp) {
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kEwThreads * kEwUnroll) + threadIdx.x;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kEwThreads * kReluUnroll) + threadIdx.x;
+  auto relu16 = [&](v4i v) {
+    return v4i{static_cast<int>(relu_four<SIGNED>(v.x, zp)), static_cast<int>(relu_four<SIGNED>(v.y, zp)),
+               static_cast<int>(relu_four<SIGNED>(v.z, zp)), static_cast<int>(relu_four<SIGNED>(v.w, zp))};
+  };
+  v4i v[kReluUnroll];
+  if (base - threadIdx.x + kEwThreads * kReluUnroll <= n16) {
+    // whole block inside the array: all loads first (read once: non-temporal), then all stores
 #pragma unroll
-  for (int u = 0; u < kEwUnroll; ++u) {
-    const int64_t i = base + u * kEwThreads;
-    if (i < n16) {
-      const v4i v = x16[i];
-      y16[i] = v4i{static_cast<int>(relu_four<SIGNED>(v.x, zp)), static_cast<int>(relu_four<SIGNED>(v.y, zp)),
-                   static_cast<int>(relu_four<SIGNED>(v.z, zp)), static_cast<int>(relu_four<SIGNED>(v.w, zp))};
+    for (int u = 0; u < kReluUnroll; ++u) v[u] = __builtin_nontemporal_load(&x16[base + u * kEwThreads]);
+#pragma unroll
+    for (int u = 0; u < kReluUnroll; ++u) y16[base + u * kEwThreads] = relu16(v[u]);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kReluUnroll; ++u) {
+      const int64_t i = base + u * kEwThreads;
+      if (i < n16) y16[i] = relu16(x16[i]);
     }
   }
   if (blockIdx.x == 0) {
@@ -381,7 +391,7 @@ TMQ_EXPORT int tmq_qrelu(const void* x, void* y, int64_t n, int32_t zero_point, 
   uint8_t* yb = static_cast<uint8_t*>(y);
   if (aligned(x, 16) && aligned(y, 16)) {
     const int64_t n16 = n / 16;
-    const int64_t blocks = n16 == 0 ? 1 : ceil_div(n16, kEwThreads * kEwUnroll);
+    const int64_t blocks = n16 == 0 ? 1 : ceil_div(n16, kEwThreads * kReluUnroll);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
     const dim3 grid(static_cast<unsigned>(blocks)), block(kEwThreads);
     if (q_signed)
