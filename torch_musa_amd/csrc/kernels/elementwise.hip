@@ -279,6 +279,45 @@ __global__ __launch_bounds__(kEwThreads) void qmaxpool_kernel(const uint8_t* __r
   }
 }
 
+// The common 3x3 window (any stride and padding, dilation 1), 16 channels per
+// thread: all nine loads are issued before the first maximum is taken (taps
+// outside the image load a clamped address and are then replaced by the lowest
+// code), where the general kernel's tap loop waits for each load in turn.
+template <bool SIGNED>
+__global__ __launch_bounds__(kEwThreads) void qmaxpool_k3_kernel(const uint8_t* __restrict__ x,
+                                                                 uint8_t* __restrict__ y, PoolShape s) {
+  const int64_t cv = s.C / 16;
+  const int64_t total = s.B * s.OH * s.OW * cv;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kEwThreads;
+  const int lowest = static_cast<int>(SIGNED ? 0x80808080u : 0u);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kEwThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t c = (i % cv) * 16;
+    int64_t t = i / cv;
+    const int64_t ow = t % s.OW;
+    t /= s.OW;
+    const int64_t oh = t % s.OH, b = t / s.OH;
+    const int64_t ih0 = oh * s.sh - s.ph, iw0 = ow * s.sw - s.pw;
+    const uint8_t* img = x + b * s.H * s.W * s.C + c;
+    v4i v[9];
+    bool ok[9];
+#pragma unroll
+    for (int k = 0; k < 9; ++k) {
+      const int64_t ih = ih0 + k / 3, iw = iw0 + k % 3;
+      ok[k] = ih >= 0 && ih < s.H && iw >= 0 && iw < s.W;
+      const int64_t ihc = ih < 0 ? 0 : (ih >= s.H ? s.H - 1 : ih), iwc = iw < 0 ? 0 : (iw >= s.W ? s.W - 1 : iw);
+      v[k] = *reinterpret_cast<const v4i*>(img + (ihc * s.W + iwc) * s.C);
+    }
+    v4i m = {lowest, lowest, lowest, lowest};
+#pragma unroll
+    for (int k = 0; k < 9; ++k) {
+      const v4i u = ok[k] ? v[k] : v4i{lowest, lowest, lowest, lowest};
+      m = v4i{static_cast<int>(max_codes4<SIGNED>(m.x, u.x)), static_cast<int>(max_codes4<SIGNED>(m.y, u.y)),
+              static_cast<int>(max_codes4<SIGNED>(m.z, u.z)), static_cast<int>(max_codes4<SIGNED>(m.w, u.w))};
+    }
+    *reinterpret_cast<v4i*>(y + ((b * s.OH + oh) * s.OW + ow) * s.C + c) = m;
+  }
+}
+
 // Adaptive average pooling: output pixel (oh, ow) averages the input window
 // rows floor(oh*H/OH) .. ceil((oh+1)*H/OH)-1 (likewise columns).  VEC = 4: a
 // thread owns four consecutive channels (one 32-bit word per input pixel).
@@ -469,7 +508,10 @@ TMQ_EXPORT int tmq_qmaxpool2d(const void* x, void* y, int64_t B, int64_t H, int6
   hipStream_t hs = as_stream(stream);
   const uint8_t* xb = static_cast<const uint8_t*>(x);
   uint8_t* yb = static_cast<uint8_t*>(y);
-  if (vec) {
+  if (vec && kh == 3 && kw == 3 && dil_h == 1 && dil_w == 1) {
+    if (q_signed) qmaxpool_k3_kernel<true><<<grid, block, 0, hs>>>(xb, yb, s);
+    else qmaxpool_k3_kernel<false><<<grid, block, 0, hs>>>(xb, yb, s);
+  } else if (vec) {
     if (q_signed) qmaxpool_kernel<true, 16><<<grid, block, 0, hs>>>(xb, yb, s);
     else qmaxpool_kernel<false, 16><<<grid, block, 0, hs>>>(xb, yb, s);
   } else {
