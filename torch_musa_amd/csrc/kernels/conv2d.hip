@@ -241,17 +241,39 @@ bool plan_tiles(const ConvShape& s, bool forced, TilePlan* best) {
   return best_cost >= 0;
 }
 
-template <int MODE>
-int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs& a, hipStream_t stream) {
+template <int MODE, int KIND, bool VEC>
+int launch_conv_tiles_variant(const ConvShape& s, const TilePlan& p, const ConvTileArgs& a, hipStream_t stream) {
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&conv_tile_kernel<MODE>),
+      reinterpret_cast<const void*>(&conv_tile_kernel<MODE, KIND, VEC>),
       hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit() - 3 * kCtBN * 4);
   if (attr != hipSuccess) return TMQ_ERR_LAUNCH;
   const int64_t bx = s.B * a.tiles_h * a.tiles_w, by = static_cast<int64_t>(a.n_tiles) * s.groups;
   if (bx > 0x7fffffff || by > 65535) return TMQ_ERR_UNSUPPORTED;
-  conv_tile_kernel<MODE><<<dim3(static_cast<unsigned>(bx), static_cast<unsigned>(by)),
-                           dim3(kCtThreads), p.lds_total, stream>>>(a);
+  conv_tile_kernel<MODE, KIND, VEC><<<dim3(static_cast<unsigned>(bx), static_cast<unsigned>(by)),
+                                      dim3(kCtThreads), p.lds_total, stream>>>(a);
   return launch_status();
+}
+
+// Which epilogue the launch needs (see conv_tile_kernel) is known on the host.
+template <int MODE>
+int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs& a, hipStream_t stream) {
+  const bool aligned16 = (reinterpret_cast<uintptr_t>(a.y) & 15) == 0;
+  if constexpr (MODE == kOutAcc32) {
+    const bool vec = (a.OC & 3) == 0 && (a.OCg & 3) == 0 && aligned16;
+    return vec ? launch_conv_tiles_variant<MODE, 1, true>(s, p, a, stream)
+               : launch_conv_tiles_variant<MODE, 1, false>(s, p, a, stream);
+  } else {
+    const bool vec = (a.OC & 15) == 0 && (a.OCg & 15) == 0 && aligned16;
+    const int kind = a.post.any() ? 0 : ((MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f) ? 2 : 1);
+    switch (kind * 2 + (vec ? 1 : 0)) {
+      case 0: return launch_conv_tiles_variant<MODE, 0, false>(s, p, a, stream);
+      case 1: return launch_conv_tiles_variant<MODE, 0, true>(s, p, a, stream);
+      case 2: return launch_conv_tiles_variant<MODE, 1, false>(s, p, a, stream);
+      case 3: return launch_conv_tiles_variant<MODE, 1, true>(s, p, a, stream);
+      case 4: return launch_conv_tiles_variant<MODE, 2, false>(s, p, a, stream);
+      default: return launch_conv_tiles_variant<MODE, 2, true>(s, p, a, stream);
+    }
+  }
 }
 
 template <int MODE>

@@ -80,7 +80,13 @@ __device__ __forceinline__ void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int MODE>
+// KIND selects the requantisation compiled in: 0 residual / SiLU, 1 plain with
+// clamp, 2 plain for unsigned output without ReLU (the saturating pack
+// conversion is the clamp).  VEC: output rows take aligned 16-byte (int32 mode:
+// 4-channel) stores.  One variant per launch keeps the straight-line code that
+// every wave runs exactly once small: the kernel with all variants inside was
+// five times longer and spent a quarter of its time fetching instructions.
+template <int MODE, int KIND, bool VEC>
 __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ __attribute__((aligned(16))) int s_acc0[kCtBN];
@@ -126,8 +132,8 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
   //   halo:    slot s of a pass is thread s; a pass covers `rpp` whole halo rows
   //            of `ri` slots (pitch/16 per pixel, the padding slot left alone)
   // Out-of-image positions get the activation zero point from a plain LDS
-  // store; afterwards every thread flips the sign bit (x ^ 0x80) of the slots
-  // it loaded itself.
+  // store.  The sign-bit flip of unsigned activations (x ^ 0x80) is applied to
+  // the fragments in the k loop.
   {
     const int nbv_all = (a.OCg + 15) / 16 - nt * 4;
     const int nbv = nbv_all < 4 ? nbv_all : 4;  // 16-row weight blocks that exist
@@ -154,7 +160,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
     uint32_t xoff = (static_cast<uint32_t>(ih0 + lr) * static_cast<uint32_t>(a.W) +
                      static_cast<uint32_t>(iw0 + hc)) * static_cast<uint32_t>(a.IC) +
                     static_cast<uint32_t>(hb) * 16u;
-    const int padx = static_cast<int>(a.pad_word ^ a.x_xor);
+    const int padx = static_cast<int>(a.pad_word);
     int wave_dst = a.lds_x + wave * (kWave * 16);  // first slot of this wave in the current pass
     int hr = lr;
     for (int i = 0; i < a.cx; ++i) {
@@ -183,29 +189,6 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       s_tab[c] = off;
     }
     __builtin_amdgcn_s_waitcnt(0);  // the direct loads have landed in LDS
-    if (a.x_xor != 0) {
-      const int xm = static_cast<int>(a.x_xor);
-      int slot = a.lds_x + t * 16;
-      hr = lr;
-      for (int i = 0; i < a.cx; i += 4) {
-        v4i v[4];
-        bool mine[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int r = hr + k * a.rpp;
-          mine[k] = i + k < a.cx && active && r < a.HH && col_ok &&
-                    static_cast<unsigned>(ih0 + r) < static_cast<unsigned>(a.H);
-          if (mine[k]) v[k] = *reinterpret_cast<const v4i*>(lds + slot + k * a.xdstep);
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (mine[k])
-            *reinterpret_cast<v4i*>(lds + slot + k * a.xdstep) =
-                v4i{v[k].x ^ xm, v[k].y ^ xm, v[k].z ^ xm, v[k].w ^ xm};
-        hr += 4 * a.rpp;
-        slot += 4 * a.xdstep;
-      }
-    }
   }
   if (t < kCtBN) {
     int acc0 = 0;
@@ -244,11 +227,9 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
   const uint8_t* const sW = lds;
   const uint8_t* const sX = lds + a.lds_x;
   const int img_pix = static_cast<int>(b) * a.OH * a.OW;  // the host keeps pixel counts below 2**31
-  const bool vec_ok = MODE == kOutAcc32
-                          ? ((a.OC & 3) == 0 && (a.OCg & 3) == 0 &&
-                             (reinterpret_cast<uintptr_t>(a.y) & 15) == 0)
-                          : ((a.OC & 15) == 0 && (a.OCg & 15) == 0 &&
-                             (reinterpret_cast<uintptr_t>(a.y) & 15) == 0);
+  constexpr bool vec_ok = VEC;  // the host checked channel counts and the output's alignment
+  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
+                     static_cast<int>(a.x_xor)};
 
   auto run = [&](auto tm_tag, int mt0) {
     constexpr int TM = decltype(tm_tag)::value;
@@ -284,7 +265,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
     // The residual bytes this lane will add (4 consecutive channels per word)
     // are requested now; they arrive while the k loop runs.
     uint32_t accw[TM][8];
-    if (a.post.accum != nullptr) {
+    if (KIND == 0 && a.post.accum != nullptr) {
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
@@ -316,11 +297,14 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       for (int tm = 0; tm < TM; ++tm) xf[tm] = ld16(sX + xb[tm] + cur);
     };
     auto mul_step = [&](const v4i(&wf)[2], const v4i(&xf)[TM]) {
+      v4i xs[TM];
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) xs[tm] = xf[tm] ^ xmask;
 #pragma unroll
       for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
-          acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[tn], xf[tm], acc[tn][tm], 0, 0, 0);
+          acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[tn], xs[tm], acc[tn][tm], 0, 0, 0);
     };
     // KS is even.  The fragments of a step are requested before the MFMAs of
     // the step before it are issued; the fences keep that order.
@@ -362,10 +346,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       uint8_t* y = static_cast<uint8_t*>(a.y);
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
-        // kind 0: residual / SiLU; 1: plain; 2: plain, unsigned output without
-        // ReLU, where the saturating pack conversion is the clamp
-        auto requant_rows = [&](auto kind_tag) {
-          constexpr int KIND = decltype(kind_tag)::value;
+        {
 #pragma unroll
           for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
@@ -383,13 +364,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
                 q4 = requant4<MODE, KIND == 1>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
               *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) = q4;
             }
-        };
-        if (a.post.any())
-          requant_rows(std::integral_constant<int, 0>{});
-        else if (MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f)
-          requant_rows(std::integral_constant<int, 2>{});
-        else
-          requant_rows(std::integral_constant<int, 1>{});
+        }
         wave_sync_lds();
         // whole pixels leave as 16 bytes per lane: 4 lanes per pixel, 16 pixels per pass
 #pragma unroll
