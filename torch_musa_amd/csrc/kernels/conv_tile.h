@@ -141,14 +141,16 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
         a.w_packed + g * a.group_bytes + static_cast<int64_t>(nt) * 4 * a.w_kchunks * 256;
     const uint8_t* const img =
         a.x + static_cast<int64_t>(b) * (static_cast<int64_t>(a.H) * a.W * a.IC) + g * a.ICg;
-    typedef const __attribute__((address_space(1))) void* gptr_t;
-    typedef __attribute__((address_space(3))) void* lptr_t;
+    // copies as "uniform base + 32-bit lane offset" (lds_dma16): the host keeps a
+    // 64-channel weight slice and one image below 4 GB
+    const uint32_t lds0 = lds_address(lds);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
 
     const int nbl = (lane >> 4) & 3, nbc = nbl < nbv ? nbl : nbv - 1;
-    const uint8_t* wp = wsrc + (static_cast<int64_t>(nbc) * a.w_kchunks + wave) * 256 + (lane & 15) * 16;
-    for (int kc = wave; kc < 2 * a.KS; kc += kCtWaves) {
-      __builtin_amdgcn_global_load_lds((gptr_t)(wp), (lptr_t)(lds + kc * (kCtBN * 16)), 16, 0, 0);
-      wp += kCtWaves * 256;
+    uint32_t woff = static_cast<uint32_t>((static_cast<int64_t>(nbc) * a.w_kchunks + wave_u) * 256 + (lane & 15) * 16);
+    for (int kc = wave_u; kc < 2 * a.KS; kc += kCtWaves) {
+      lds_dma16(wsrc, woff, lds0 + kc * (kCtBN * 16));
+      woff += kCtWaves * 256;
     }
 
     const int pslots = a.pitch >> 4;  // slots per pixel
@@ -161,13 +163,13 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
                      static_cast<uint32_t>(iw0 + hc)) * static_cast<uint32_t>(a.IC) +
                     static_cast<uint32_t>(hb) * 16u;
     const int padx = static_cast<int>(a.pad_word);
-    int wave_dst = a.lds_x + wave * (kWave * 16);  // first slot of this wave in the current pass
+    int wave_dst = a.lds_x + wave_u * (kWave * 16);  // first slot of this wave in the current pass
     int hr = lr;
     for (int i = 0; i < a.cx; ++i) {
       const bool live = active && hr < a.HH;
       const bool inside = live && col_ok && static_cast<unsigned>(ih0 + hr) < static_cast<unsigned>(a.H);
       if (inside)
-        __builtin_amdgcn_global_load_lds((gptr_t)(img + xoff), (lptr_t)(lds + wave_dst), 16, 0, 0);
+        lds_dma16(img, xoff, lds0 + wave_dst);
       else if (live)
         *reinterpret_cast<v4i*>(lds + wave_dst + lane * 16) = v4i{padx, padx, padx, padx};
       hr += a.rpp;

@@ -131,6 +131,25 @@ __device__ __forceinline__ v4i ld16_stream(const void* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
 }
 
+// One direct global->LDS copy: every active lane moves the 16 bytes at
+// base + off (uniform 64-bit base, per-lane 32-bit offset) to LDS byte
+// lds_dst + 16 * lane (wave-uniform destination, passed in M0).
+// Issued through inline assembly on purpose: for the compiler's own builtin
+// every later LDS access may alias the copy, and it drains all outstanding
+// loads (vmcnt(0)) before it, which serialises a pipeline of copies.  The
+// caller waits (s_waitcnt vmcnt) before the data is read.
+__device__ __forceinline__ void lds_dma16(const uint8_t* base, uint32_t off, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(off), "s"(base), "s"(lds_dst)
+               : "memory", "m0");
+}
+// LDS byte address of a pointer into shared memory, as a wave-uniform value.
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)p)));
+}
+
 template <class XSRC>
 struct XLoader;
 
@@ -468,14 +487,12 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
     //                dead buffer
     // Activation fragments get their sign-bit flip one MFMA ahead of their
     // first use, so that the flip never sits between a barrier and an MFMA.
-    typedef __attribute__((address_space(3))) void* lptr_t;
     // Every copy is "uniform 64-bit base + per-lane 32-bit offset" on the global
     // side and a wave-uniform LDS address in M0 on the other: per stage only the
     // scalar bases move, no vector instruction is spent on addresses.  The host
     // keeps 256 rows of either operand within 32 bits of the tile's base.
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const uint32_t lds0 =
-        __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)smem)));
+    const uint32_t lds0 = lds_address(smem);
     // weight copy i of wave w: k-chunk w & 3, 64-row group (w >> 2) + i * NWAVES / 4
     static_assert(NWAVES % 4 == 0, "weight copies: one k-chunk per wave");
     const uint8_t* const wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
@@ -505,16 +522,7 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
       xdma_off_last[i] = static_cast<uint32_t>(r * xsrc.ldx + (kc < ktail ? kc : ktail));
     }
     const uint32_t xdma_lds = lds0 + kWBufs * kWStage + wave_u * 1024;
-    // Issued through inline assembly on purpose: for the builtin the compiler
-    // assumes that every later LDS read may alias the copy and drains all
-    // outstanding loads before it, which serialises the pipeline.  The waits
-    // that these copies need are the explicit ones below.
-    auto dma = [&](const uint8_t* base, uint32_t off, uint32_t lds_dst) {
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                   :
-                   : "v"(off), "s"(base), "s"(lds_dst)
-                   : "memory", "m0");
-    };
+    auto dma = [&](const uint8_t* base, uint32_t off, uint32_t lds_dst) { lds_dma16(base, off, lds_dst); };
     // i-th copy of stage kt into buffer b
     auto dma_one = [&](int kt, int b, int i) {
       if (i < NDW) {
