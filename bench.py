@@ -251,6 +251,7 @@ def main():
         q2 = torch.quantize_per_tensor(xf * 0.5, scale, zp, torch.quint8)
         hbm("quantized_add_2p28", lambda: torch.ops.quantized.add(q, q2, scale * 1.5, zp), 3 * n, None)
         hbm("quantized_relu_2p28", lambda: torch.relu(q), 2 * n, None)
+        hbm("quantized_gelu_2p28", lambda: torch.nn.functional.gelu(q), 2 * n, None)
         del xf, q, q2
 
         # -------------------------------------------------------------- C4

@@ -339,6 +339,16 @@ int tmq_qadaptive_avgpool2d(const void* x, void* y, int64_t B, int64_t H, int64_
                             int64_t OH, int64_t OW, int32_t zero_point, int q_signed,
                             tmq_stream_t stream);
 
+/* gelu / sigmoid of a per-tensor quantized tensor (replaces ActQuantizedGeLU and
+ * ActQuantized<SIGMOID>, torch_musa/csrc/aten/quantized/musa/Activation.mu:95-164,
+ * 218-219): y = f((q - in_zp) * in_scale), q' = clamp(rne(y / out_scale) + out_zp),
+ * evaluated once per input code in double precision and applied as a table.
+ * kind 0: gelu (erf), 1: gelu (tanh approximation), 2: sigmoid.  PyTorch's CPU ops
+ * give gelu the input's parameters and sigmoid scale 1/256 with zero point 0
+ * (quint8) or -128 (qint8); the caller passes them. */
+int tmq_qunary(const void* x, void* y, int64_t n, int kind, float in_scale, int32_t in_zero_point,
+               float out_scale, int32_t out_zero_point, int q_signed, tmq_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * Measurement probe (no counterpart in the reference; used by bench.py only).
  * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four

@@ -379,6 +379,31 @@ def qadaptive_avgpool2d(x_nhwc, out_hw, zero_point):
     return y
 
 
+def qunary(q, kind, in_scale, in_zp, out_scale, out_zp):
+    """gelu / gelu_tanh / sigmoid of per-tensor quantized codes, the way PyTorch's CPU
+    ops define them (dequantize, activation, quantize), evaluated in float64:
+    y = f((q - in_zp) * fl(in_scale)); q' = clamp(rne(y / fl(out_scale)) + out_zp)."""
+    from math import erf, tanh, exp, sqrt, pi
+    q = _as_bytes(q)
+    signed = q.dtype == np.int8
+    lo, hi = (-128, 127) if signed else (0, 255)
+    s_in, s_out = float(np.float32(in_scale)), float(np.float32(out_scale))
+    table = {}
+    for code in range(lo, hi + 1):
+        r = (code - in_zp) * s_in
+        if kind == "gelu":
+            f = 0.5 * r * (1.0 + erf(r / sqrt(2.0)))
+        elif kind == "gelu_tanh":
+            f = 0.5 * r * (1.0 + tanh(sqrt(2.0 / pi) * (r + 0.044715 * r ** 3)))
+        elif kind == "sigmoid":
+            f = 1.0 / (1.0 + exp(-r))
+        else:
+            raise ValueError(kind)
+        table[code] = int(min(max(np.rint(f / s_out) + out_zp, lo), hi))
+    lut = np.array([table[c] for c in range(lo, hi + 1)], dtype=q.dtype)
+    return lut[q.astype(np.int64) - lo]
+
+
 def qcat(qs, scales, zps, axis, out_scale, out_zp):
     """quantized::cat: every input dequantized and requantized to the output's
     parameters (the composition PyTorch's CPU op performs), then concatenated."""

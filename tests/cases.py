@@ -506,3 +506,20 @@ def plain_conv_cases():
             c["accum"] = (rng.standard_normal((xs[0], oc, oh, ow)) * (1.0 if small else 3.0)).astype(np.float32)
         out.append(c)
     return out
+
+
+def qunary_cases():
+    spec = [
+        # name, shape, scale, zero point, signed
+        ("u8_zp128_4x3000", (4, 3000), 0.0679, 128, False),
+        ("s8_zp0_2x16x9x9", (2, 16, 9, 9), 0.0431, 0, True),
+        ("u8_zp37_777", (777,), 0.0213, 37, False),
+        ("s8_zpm20_33x65", (33, 65), 0.11, -20, True),
+    ]
+    out = []
+    for i, (name, shape, scale, zp, signed) in enumerate(spec):
+        rng = np.random.default_rng(2000 + i)
+        lo, hi = (-128, 128) if signed else (0, 256)
+        out.append(dict(name=name, x=rng.integers(lo, hi, shape).astype(np.int8 if signed else np.uint8),
+                        scale=float(np.float32(scale)), zp=zp, signed=signed))
+    return out

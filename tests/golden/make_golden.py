@@ -259,6 +259,18 @@ def main():
         g[k + "/x_crc"] = np.uint32(cases.crc(c["x"]))
         g[k + "/y"] = y.int_repr().permute(0, 2, 3, 1).contiguous().numpy()
 
+    # ---- gelu / sigmoid of quantized tensors ------------------------------------
+    for c in cases.qunary_cases():
+        xq = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["x"]), c["scale"], c["zp"])
+        for kind, fn in (("gelu", lambda t: torch.nn.functional.gelu(t)),
+                         ("gelu_tanh", lambda t: torch.nn.functional.gelu(t, approximate="tanh")),
+                         ("sigmoid", torch.sigmoid)):
+            y = fn(xq)
+            k = "qunary/" + c["name"] + "/" + kind
+            g[k + "/y"] = y.int_repr().numpy()
+            g[k + "/qparams"] = np.array([y.q_scale(), y.q_zero_point()], dtype=np.float64)
+        g["qunary/" + c["name"] + "/x_crc"] = np.uint32(cases.crc(c["x"]))
+
     # ---- quantized::conv2d -------------------------------------------------
     for c in cases.conv_cases():
         x_nchw = torch.from_numpy(c["xq"]).permute(0, 3, 1, 2)  # channels-last view

@@ -643,3 +643,18 @@ def test_quantized_modules_to_device():
     torch_musa_amd.quantized_modules_to(net, "cpu")
     q2, f2 = net(xq)
     assert torch.equal(q2.int_repr(), q_cpu.int_repr()) and torch.equal(f2, f_cpu)
+
+
+@pytest.mark.parametrize("c", cases.qunary_cases(), ids=lambda c: c["name"])
+def test_gelu_sigmoid_ops(golden, c):
+    say("aten gelu / sigmoid", c["name"])
+    xq = torch._make_per_tensor_quantized_tensor(torch.from_numpy(c["x"]).cuda(), c["scale"], c["zp"])
+    for kind, fn in (("gelu", lambda t: torch.nn.functional.gelu(t)),
+                     ("gelu_tanh", lambda t: torch.nn.functional.gelu(t, approximate="tanh")),
+                     ("sigmoid", torch.sigmoid)):
+        y = fn(xq)
+        out_scale, out_zp = golden["qunary/" + c["name"] + "/" + kind + "/qparams"]
+        assert y.is_cuda and y.is_quantized and y.q_scale() == out_scale and y.q_zero_point() == out_zp
+        d = (y.int_repr().cpu().numpy().astype(np.int32)
+             - golden["qunary/" + c["name"] + "/" + kind + "/y"].astype(np.int32))
+        assert np.abs(d).max() <= 1 and np.count_nonzero(d) <= 0.001 * d.size + 1

@@ -292,3 +292,25 @@ def test_quantize_dynamic_on_device(cabi, n, offset, signed, reduce_range):
     scale, zp = oracle.choose_qparams(mn, mx, signed, reduce_range)
     assert cabi.read_qparams(qp) == (scale, zp)
     np.testing.assert_array_equal(host(q), oracle.quantize_per_tensor(x[offset:], scale, zp, signed))
+
+
+@pytest.mark.parametrize("kind", ["gelu", "gelu_tanh", "sigmoid"])
+@pytest.mark.parametrize("c", cases.qunary_cases(), ids=lambda c: c["name"])
+def test_qunary(cabi, golden, c, kind):
+    say("qunary", kind, c["name"])
+    out_scale, out_zp = golden["qunary/" + c["name"] + "/" + kind + "/qparams"]
+    y = host(cabi.qunary(dev(c["x"]), kind, c["scale"], c["zp"], float(out_scale), int(out_zp)))
+    # the table is computed in double precision on the device: equal to the float64 oracle
+    np.testing.assert_array_equal(y, oracle.qunary(c["x"], kind, c["scale"], c["zp"], out_scale, int(out_zp)))
+    d = np.abs(y.astype(np.int32) - golden["qunary/" + c["name"] + "/" + kind + "/y"].astype(np.int32))
+    assert d.max() <= 1 and np.count_nonzero(d) <= 0.001 * d.size + 1
+
+
+def test_qunary_unaligned_and_large(cabi):
+    say("qunary unaligned / large")
+    x = np.random.default_rng(9).integers(0, 256, (1 << 22) + 5).astype(np.uint8)
+    xd = dev(x)
+    y = host(cabi.qunary(xd[3:], "gelu", 0.05, 120, 0.05, 120))     # misaligned view
+    np.testing.assert_array_equal(y, oracle.qunary(x[3:], "gelu", 0.05, 120, 0.05, 120))
+    y = host(cabi.qunary(xd, "sigmoid", 0.05, 120, 1 / 256, 0))
+    np.testing.assert_array_equal(y, oracle.qunary(x, "sigmoid", 0.05, 120, 1 / 256, 0))

@@ -216,3 +216,21 @@ def test_plain_conv(golden, c):
                           c["groups"], c["out_scale"], c["out_zp"], c["out_dtype"], c["relu"], c["accum"],
                           c["accum_scale"], c["accum_zp"])
     _close_to(y, golden[k + "/y"], c["out_dtype"], c["name"])
+
+
+@pytest.mark.parametrize("kind", ["gelu", "gelu_tanh", "sigmoid"])
+@pytest.mark.parametrize("c", cases.qunary_cases(), ids=lambda c: c["name"])
+def test_qunary(golden, c, kind):
+    # golden = PyTorch's CPU op (float32 vector math); the oracle evaluates the same
+    # definition in float64: equal except, at most, where a value sits on a rounding boundary
+    k = "qunary/" + c["name"]
+    assert int(golden[k + "/x_crc"]) == cases.crc(c["x"])
+    out_scale, out_zp = golden[k + "/" + kind + "/qparams"]
+    if kind == "sigmoid":
+        assert out_scale == 1.0 / 256 and out_zp == (-128 if c["signed"] else 0)
+    else:
+        assert out_scale == c["scale"] and out_zp == c["zp"]
+    y = oracle.qunary(c["x"], kind, c["scale"], c["zp"], out_scale, int(out_zp))
+    want = golden[k + "/" + kind + "/y"]
+    d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+    assert d.max() <= 1 and np.count_nonzero(d) <= 0.001 * d.size + 1

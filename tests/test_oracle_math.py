@@ -360,3 +360,20 @@ def test_linear_dynamic_matches_float_linear_within_quantization_error():
     # each activation is off by at most half a step
     bound = 0.5 * step * np.abs(wq.astype(np.float64) * 0.01).sum(axis=1)
     assert np.all(np.abs(y - ref) <= bound[None, :] * 1.001 + 1e-4)
+
+
+def test_qunary_known_values():
+    codes = np.arange(256, dtype=np.uint8)
+    # sigmoid: the zero point maps to 0.5 = code 128; far negative -> 0, far positive saturates at 255
+    y = oracle.qunary(codes, "sigmoid", 0.1, 128, 1 / 256, 0)
+    assert y[128] == 128 and y[0] == 0 and y[255] == 255 and np.all(np.diff(y.astype(int)) >= 0)
+    # sigmoid(-x) = 1 - sigmoid(x): codes mirror around the zero point (up to the rounding of .5)
+    assert np.all(np.abs((y[128 + np.arange(1, 100)].astype(int) + y[128 - np.arange(1, 100)].astype(int)) - 256) <= 1)
+    # gelu: 0 at the zero point, identity for large positive, 0 for large negative values
+    g = oracle.qunary(codes, "gelu", 0.1, 100, 0.1, 100)
+    assert g[100] == 100 and g[255] == 255 and g[0] == 100 and g[160] == 160
+    # minimum of gelu is about -0.17 at x = -0.75: one or two steps below the zero point at this scale
+    assert g.min() == 98
+    # the tanh approximation stays within one step of the erf form
+    t = oracle.qunary(codes, "gelu_tanh", 0.1, 100, 0.1, 100)
+    assert np.abs(t.astype(int) - g.astype(int)).max() <= 1

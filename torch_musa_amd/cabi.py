@@ -27,7 +27,7 @@ DECLARED_SYMBOLS = [
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32", "tmq_linear_f32", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
-    "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d",
+    "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
     "tmq_probe_mfma_i8",
 ]
 
@@ -132,6 +132,7 @@ def lib() -> C.CDLL:
                                     C.c_float, C.c_int32, C.c_int, v]
         l.tmq_qmaxpool2d.argtypes = [v, v] + [C.c_int64] * 4 + [C.c_int32] * 8 + [C.c_int64] * 2 + [C.c_int, v]
         l.tmq_qadaptive_avgpool2d.argtypes = [v, v] + [C.c_int64] * 6 + [C.c_int32, C.c_int, v]
+        l.tmq_qunary.argtypes = [v, v, C.c_int64, C.c_int, C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_int, v]
         l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, v, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]
         _lib = l
@@ -502,6 +503,16 @@ def qrelu(q, zp, out=None):
     y = out if out is not None else torch.empty_like(q)
     check(lib().tmq_qrelu(q.data_ptr(), y.data_ptr(), q.numel(), zp, int(q.dtype == torch.int8),
                           stream_ptr()), "tmq_qrelu")
+    return y
+
+
+QUNARY_KINDS = {"gelu": 0, "gelu_tanh": 1, "sigmoid": 2}
+
+
+def qunary(q, kind, in_scale, in_zp, out_scale, out_zp):
+    y = torch.empty_like(q)
+    check(lib().tmq_qunary(q.data_ptr(), y.data_ptr(), q.numel(), QUNARY_KINDS[kind], in_scale, in_zp, out_scale,
+                           out_zp, int(q.dtype == torch.int8), stream_ptr()), "tmq_qunary")
     return y
 
 

@@ -695,6 +695,35 @@ at::Tensor qrelu_run(const at::Tensor& self) {
   return y;
 }
 
+// aten::gelu and aten::sigmoid of per-tensor quantized tensors (reference:
+// ActQuantizedGeLU / ActQuantized<SIGMOID>, musa/Activation.mu:95-164,218-219).
+// Output parameters as PyTorch's CPU ops choose them: gelu keeps the input's,
+// sigmoid uses scale 1/256 with zero point 0 (quint8) or -128 (qint8).
+at::Tensor qunary_impl(const at::Tensor& self, int kind, double out_scale, int64_t out_zp, const char* what) {
+  TORCH_CHECK(self.qscheme() == c10::kPerTensorAffine || self.qscheme() == c10::kPerTensorSymmetric, what,
+              ": only per-tensor quantized tensors are supported, got ", toString(self.qscheme()));
+  const bool sgn = is_signed_qtype(self.scalar_type(), what);
+  const c10::OptionalDeviceGuard guard(at::device_of(self));
+  const auto fmt = self.suggest_memory_format();
+  const at::Tensor x = self.contiguous(fmt);
+  at::Tensor y = at::_empty_affine_quantized(self.sizes(), self.options(), out_scale, out_zp, fmt);
+  if (y.numel() == 0) return y;
+  check_status(tmq_qunary(x.data_ptr(), y.data_ptr(), y.numel(), kind, static_cast<float>(self.q_scale()),
+                          static_cast<int32_t>(self.q_zero_point()), static_cast<float>(out_scale),
+                          static_cast<int32_t>(out_zp), sgn, current_stream(x)),
+               "tmq_qunary");
+  return y;
+}
+at::Tensor qgelu_run(const at::Tensor& self, c10::string_view approximate) {
+  const std::string a(approximate.data(), approximate.size());
+  TORCH_CHECK(a == "none" || a == "tanh", "gelu: approximate must be 'none' or 'tanh', got ", a);
+  return qunary_impl(self, a == "tanh" ? 1 : 0, self.q_scale(), self.q_zero_point(), "gelu");
+}
+at::Tensor qsigmoid_run(const at::Tensor& self) {
+  const bool sgn = self.scalar_type() == c10::kQInt8;
+  return qunary_impl(self, 2, 1.0 / 256.0, sgn ? -128 : 0, "sigmoid");
+}
+
 // ---------------------------------------------------------------------------
 // quantized::cat (TensorShape.cpp:383-426 of the reference) and
 // aten::quantized_max_pool2d (Pool.cpp:178-247)
@@ -1134,6 +1163,8 @@ TORCH_LIBRARY_IMPL(aten, QuantizedCUDA, m) {
   m.impl("relu", TORCH_FN(qrelu_run));
   m.impl("quantized_max_pool2d", TORCH_FN(qmaxpool2d_run));
   m.impl("_adaptive_avg_pool2d", TORCH_FN(qadaptive_avgpool2d_run));
+  m.impl("gelu", TORCH_FN(qgelu_run));
+  m.impl("sigmoid", TORCH_FN(qsigmoid_run));
 }
 
 namespace {

@@ -374,6 +374,58 @@ __global__ __launch_bounds__(kEwThreads) void qadaptive_avgpool_kernel(const uin
   }
 }
 
+// Unary activations of a per-tensor quantized tensor through a 256-entry table:
+// the input has 256 codes, so every block first computes f for each of them
+// (one per thread, in double precision: y = f((c - zp_in) * s_in),
+// q = clamp(rne(y / s_out) + zp_out)) into LDS and then maps the bytes, 16 per
+// lane per access.  kind 0: gelu (erf), 1: gelu (tanh approximation), 2: sigmoid.
+struct UnaryParams {
+  double in_scale, out_scale;
+  int in_zp, out_zp;
+  int kind;
+};
+constexpr int kLutBlocksMax = 4096;
+template <bool SIGNED>
+__global__ __launch_bounds__(kEwThreads) void qunary_lut_kernel(const v4i* __restrict__ x16,
+                                                                v4i* __restrict__ y16, int64_t n16,
+                                                                const uint8_t* __restrict__ x,
+                                                                uint8_t* __restrict__ y, int64_t n,
+                                                                UnaryParams p) {
+  __shared__ uint8_t lut[256];
+  static_assert(kEwThreads == 256, "one table entry per thread");
+  {
+    const int code = SIGNED ? static_cast<int>(static_cast<int8_t>(threadIdx.x)) : static_cast<int>(threadIdx.x);
+    const double r = static_cast<double>(code - p.in_zp) * p.in_scale;
+    double f;
+    if (p.kind == 0) {
+      f = 0.5 * r * (1.0 + erf(r * 0.70710678118654752440));
+    } else if (p.kind == 1) {
+      f = 0.5 * r * (1.0 + tanh(0.79788456080286535588 * (r + 0.044715 * r * r * r)));
+    } else {
+      f = 1.0 / (1.0 + exp(-r));
+    }
+    double q = rint(f / p.out_scale) + static_cast<double>(p.out_zp);
+    const double lo = SIGNED ? -128.0 : 0.0, hi = SIGNED ? 127.0 : 255.0;
+    q = q < lo ? lo : (q > hi ? hi : q);
+    lut[threadIdx.x] = static_cast<uint8_t>(static_cast<int>(q));
+  }
+  __syncthreads();
+  auto map4 = [&](uint32_t w) {
+    return static_cast<uint32_t>(lut[w & 0xffu]) | (static_cast<uint32_t>(lut[(w >> 8) & 0xffu]) << 8) |
+           (static_cast<uint32_t>(lut[(w >> 16) & 0xffu]) << 16) | (static_cast<uint32_t>(lut[w >> 24]) << 24);
+  };
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kEwThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kEwThreads + threadIdx.x; i < n16; i += stride) {
+    const v4i v = __builtin_nontemporal_load(&x16[i]);
+    y16[i] = v4i{static_cast<int>(map4(static_cast<uint32_t>(v.x))), static_cast<int>(map4(static_cast<uint32_t>(v.y))),
+                 static_cast<int>(map4(static_cast<uint32_t>(v.z))), static_cast<int>(map4(static_cast<uint32_t>(v.w)))};
+  }
+  // bytes outside the 16-byte groups (unaligned buffers: all of them)
+  const int64_t done = x16 == nullptr ? 0 : 16 * n16;
+  for (int64_t i = done + static_cast<int64_t>(blockIdx.x) * kEwThreads + threadIdx.x; i < n; i += stride)
+    y[i] = lut[x[i]];
+}
+
 bool zp_ok(int32_t zp, int q_signed) { return q_signed ? (zp >= -128 && zp <= 127) : (zp >= 0 && zp <= 255); }
 
 template <bool SIGNED, bool RELU>
@@ -546,5 +598,32 @@ TMQ_EXPORT int tmq_qadaptive_avgpool2d(const void* x, void* y, int64_t B, int64_
     if (q_signed) qadaptive_avgpool_kernel<true, 1><<<grid, block, 0, hs>>>(xb, yb, s, zero_point);
     else qadaptive_avgpool_kernel<false, 1><<<grid, block, 0, hs>>>(xb, yb, s, zero_point);
   }
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_qunary(const void* x, void* y, int64_t n, int kind, float in_scale, int32_t in_zero_point,
+                          float out_scale, int32_t out_zero_point, int q_signed, tmq_stream_t stream) {
+  if (n < 0 || (n > 0 && (x == nullptr || y == nullptr))) return TMQ_ERR_INVALID_ARGUMENT;
+  if (kind < 0 || kind > 2 || !(in_scale > 0.f) || !(out_scale > 0.f)) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!zp_ok(in_zero_point, q_signed) || !zp_ok(out_zero_point, q_signed)) return TMQ_ERR_INVALID_ARGUMENT;
+  if (n == 0) return TMQ_OK;
+  UnaryParams p;
+  p.in_scale = static_cast<double>(in_scale);
+  p.out_scale = static_cast<double>(out_scale);
+  p.in_zp = in_zero_point;
+  p.out_zp = out_zero_point;
+  p.kind = kind;
+  const bool vec = aligned(x, 16) && aligned(y, 16);
+  const int64_t n16 = vec ? n / 16 : 0;
+  int64_t g = ceil_div(vec ? (n16 > 0 ? n16 : 1) : n, static_cast<int64_t>(kEwThreads) * 4);
+  g = g < 1 ? 1 : (g > kLutBlocksMax ? kLutBlocksMax : g);
+  const dim3 grid(static_cast<unsigned>(g)), block(kEwThreads);
+  hipStream_t s = as_stream(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  const v4i* x16 = vec ? static_cast<const v4i*>(x) : nullptr;
+  v4i* y16 = vec ? static_cast<v4i*>(y) : nullptr;
+  if (q_signed) qunary_lut_kernel<true><<<grid, block, 0, s>>>(x16, y16, n16, xb, yb, n, p);
+  else qunary_lut_kernel<false><<<grid, block, 0, s>>>(x16, y16, n16, xb, yb, n, p);
   return launch_status();
 }
