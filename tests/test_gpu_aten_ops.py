@@ -658,3 +658,22 @@ def test_gelu_sigmoid_ops(golden, c):
         d = (y.int_repr().cpu().numpy().astype(np.int32)
              - golden["qunary/" + c["name"] + "/" + kind + "/y"].astype(np.int32))
         assert np.abs(d).max() <= 1 and np.count_nonzero(d) <= 0.001 * d.size + 1
+
+
+@pytest.mark.parametrize("dtype,zp", [(torch.quint8, 128), (torch.qint8, -3)])
+def test_aten_cat_and_upsample_nearest(dtype, zp):
+    # the reference's test_concat and test_upsample_nearest2d (test_quantized_ops.py:394-462):
+    # torch.cat and nearest-neighbour interpolation of quantized tensors against the CPU ops
+    say("aten cat / upsample_nearest2d", dtype)
+    torch.manual_seed(3)
+    a = torch.quantize_per_tensor(torch.randn(2, 6, 5, 7), 0.05, zp, dtype)
+    b = torch.quantize_per_tensor(torch.randn(2, 3, 5, 7), 0.05, zp, dtype)
+    for dim in (1, 0, -1):
+        x2 = a if dim != 1 else b
+        assert_q_equal(torch.cat([a.cuda(), x2.cuda()], dim), torch.cat([a, x2], dim))
+    for kw in (dict(scale_factor=2), dict(size=(7, 9)), dict(scale_factor=(1.5, 2.5))):
+        for t in (a, a.contiguous(memory_format=torch.channels_last)):
+            got = torch.nn.functional.interpolate(t.cuda(), mode="nearest", **kw)
+            assert_q_equal(got, torch.nn.functional.interpolate(t, mode="nearest", **kw))
+    m = torch.nn.Upsample(scale_factor=2, mode="nearest")
+    assert_q_equal(m(b.cuda()), m(b))

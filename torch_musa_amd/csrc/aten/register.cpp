@@ -770,6 +770,33 @@ at::Tensor qcat_run(const c10::List<at::Tensor>& qxs, int64_t dim, std::optional
   return y;
 }
 
+// aten::cat of quantized tensors (reference: TensorShape.cpp:383-426, the same
+// function as quantized::cat): the result takes the first input's parameters.
+at::Tensor qcat_aten_run(const at::ITensorListRef& tensors, int64_t dim) {
+  c10::List<at::Tensor> list;
+  for (const at::Tensor& t : tensors) list.push_back(t);
+  return qcat_run(list, dim, std::nullopt, std::nullopt);
+}
+
+// aten::upsample_nearest2d of a per-tensor quantized tensor (reference:
+// UpSampleNearest2d.cpp:15-52, a round trip through the integer
+// representation): nearest-neighbour selection moves codes unchanged, so the
+// integer tensor goes through PyTorch-ROCm's own byte kernel and is wrapped
+// again with the input's parameters.
+at::Tensor qupsample_nearest2d_run(const at::Tensor& input, c10::SymIntArrayRef output_size,
+                                   std::optional<double> scales_h, std::optional<double> scales_w) {
+  TORCH_CHECK(input.qscheme() == c10::kPerTensorAffine || input.qscheme() == c10::kPerTensorSymmetric,
+              "upsample_nearest2d: only per-tensor quantized tensors are supported");
+  is_signed_qtype(input.scalar_type(), "upsample_nearest2d");
+  const c10::OptionalDeviceGuard guard(at::device_of(input));
+  const at::Tensor codes = input.int_repr();
+  const bool sgn = codes.scalar_type() == at::kChar;
+  const at::Tensor bytes = sgn ? codes.view(at::kByte) : codes;
+  at::Tensor up = at::upsample_nearest2d_symint(bytes, output_size, scales_h, scales_w);
+  if (sgn) up = up.view(at::kChar);
+  return at::_make_per_tensor_quantized_tensor(up, input.q_scale(), input.q_zero_point());
+}
+
 int64_t pool_out(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d, bool ceil_mode) {
   int64_t out = (n + 2 * p - d * (k - 1) - 1 + (ceil_mode ? s - 1 : 0)) / s + 1;
   if (ceil_mode && (out - 1) * s >= n + p) --out;
@@ -1165,6 +1192,8 @@ TORCH_LIBRARY_IMPL(aten, QuantizedCUDA, m) {
   m.impl("_adaptive_avg_pool2d", TORCH_FN(qadaptive_avgpool2d_run));
   m.impl("gelu", TORCH_FN(qgelu_run));
   m.impl("sigmoid", TORCH_FN(qsigmoid_run));
+  m.impl("cat", TORCH_FN(qcat_aten_run));
+  m.impl("upsample_nearest2d", TORCH_FN(qupsample_nearest2d_run));
 }
 
 namespace {
