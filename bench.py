@@ -254,6 +254,45 @@ def main():
         hbm("quantized_gelu_2p28", lambda: torch.nn.functional.gelu(q), 2 * n, None)
         del xf, q, q2
 
+        # -------------------------------------------------------------- C1
+        # x [128,1024] quint8 x W [1024,1024] per-channel qint8: 268 MOP and 1.2 MB, a
+        # latency measurement (50 launches replayed from one HIP graph)
+        log("[bench] config 1: linear M=128, K=N=1024")
+        x1 = torch.quantize_per_tensor_dynamic(torch.randn(128, 1024, device=dev), torch.quint8, False)
+        w1 = torch.randn(1024, 1024, device=dev) * 0.02
+        w1q = torch.quantize_per_channel(w1, (w1.abs().amax(dim=1) / 127.0).to(torch.float64),
+                                         torch.zeros(1024, dtype=torch.int64, device=dev), 0, torch.qint8)
+        p1 = torch.ops.quantized.linear_prepack(w1q, torch.randn(1024, device=dev))
+
+        def lin1():
+            return torch.ops.quantized.linear(x1, p1, 0.05, 128)
+
+        for _ in range(5):
+            lin1()
+        side = torch.cuda.Stream()
+        g1 = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            lin1()
+            side.synchronize()
+            with torch.cuda.graph(g1, stream=side):
+                for _ in range(50):
+                    lin1()
+        torch.cuda.synchronize()
+        for _ in range(3):
+            g1.replay()
+        ts = events_ms(g1.replay, 10)
+        per1 = sum(ts) / len(ts) / 50
+        ops1 = 2.0 * 128 * 1024 * 1024
+        log(f"[bench] linear C1: {per1*1e3:.2f} us/launch in a replayed graph, {ops1 / (per1 * 1e-3) / 1e12:.1f} TOP/s")
+        secondary["linear_c1"] = {
+            "avg_launch_us": round(per1 * 1e3, 3), "value": round(ops1 / (per1 * 1e-3) / 1e12, 2), "unit": "TOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(ops1 / (per1 * 1e-3) / 1e12, 2), "peak": PEAK_INT8_TOPS,
+                         "unit": "TOP/s", "frac": round(ops1 / (per1 * 1e-3) / 1e12 / PEAK_INT8_TOPS, 5),
+                         "traffic": None},
+            "method": "50 launches replayed in one HIP graph; launch-latency-bound at this size",
+            "ops_per_launch": ops1, "algorithmic_bytes_per_launch": 128 * 1024 + 1024 * 1024 + 128 * 1024 + 12 * 1024}
+        del x1, w1, w1q, p1, g1
+
         # -------------------------------------------------------------- C4
         log("[bench] config 4: decode-shaped linear, K=N=4096, cold weights (40 weight sets, HIP graph)")
         Kd = Nd = 4096
