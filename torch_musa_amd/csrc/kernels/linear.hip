@@ -316,7 +316,11 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
     // the CUs busy, the 128x128 tile (three blocks per CU) down to 64 tiles.
     const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
-    if (nblk(256, 256) >= 160)
+    // (and only when the rows fill at least 55 % of the row tiles: a tile's time
+    // does not shrink with its padding; M = 100 and 150 against N = 49152 sit on
+    // either side)
+    const auto rows_used = [&](int bm) { return a.M * 20 >= ceil_div(a.M, bm) * bm * 11; };
+    if (nblk(256, 256) >= 160 && rows_used(256))
       cfg = 6;  // 8 waves of 128x64, operands copied straight into LDS
     else if (nblk(128, 128) >= 64)
       cfg = 7;
