@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step is one quantized::linear at BASELINE config 3 (x quint8 [4096,4096] from
+A step is one quantized::linear at benchmark configuration 3 (x quint8 [4096,4096] from
 N(0,1), W qint8 per-channel [11008,4096] from N(0,0.02), fp32 bias, quint8
 output), issued through torch.ops.quantized.linear on tensors that are already
 resident in HBM.  The last line of stdout is one JSON object:
@@ -13,11 +13,11 @@ resident in HBM.  The last line of stdout is one JSON object:
   cpu_baseline     the CPU oracle (a scalar C port of the reference CPU
                    numerics, OpenMP over rows) on a bounded sample of the same
                    workload, on this host's cores
-  secondary        the other BASELINE configs: quantize / dequantize / min-max
+  secondary        the other benchmark configurations: quantize / dequantize / min-max
                    over 2**28 fp32 (HBM bound), decode-shaped linear (weight
                    read bound), conv2d NHWC
 
-Everything here is synthetic data of the BASELINE shapes and distributions
+Everything here is synthetic data of the benchmark shapes and distributions
 ("N(0,s)" read as standard deviation s).
 """
 from __future__ import annotations

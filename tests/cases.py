@@ -202,7 +202,7 @@ def linear_cases():
 
 
 def c1_case():
-    """BASELINE config 1: x fp32 [128,1024] ~N(0,1) -> dynamic quint8;
+    """benchmark configuration 1: x fp32 [128,1024] ~N(0,1) -> dynamic quint8;
     W fp32 [1024,1024] ~N(0,0.02) -> per-channel symmetric qint8
     (scale_c = absmax_c / 127); bias fp32 [1024]; out scale 0.05, zp 128."""
     x = randn(41, (128, 1024))

@@ -192,7 +192,7 @@ def test_qlinear_errors():
 
 
 def test_c1_through_the_operators(golden):
-    """BASELINE config 1 with nothing but torch calls on GPU tensors."""
+    """benchmark configuration 1 with nothing but torch calls on GPU tensors."""
     say("aten C1")
     c1 = cases.c1_case()
     xq = torch.quantize_per_tensor_dynamic(torch.from_numpy(c1["x"]).cuda(), torch.quint8, False)

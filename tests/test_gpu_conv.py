@@ -123,7 +123,7 @@ def test_conv_auto_path_shapes(cabi, spec):
 
 
 def test_c5_full_size(cabi):
-    """BASELINE config 5: [32,56,56,64] (x) [64,3,3,64], stride 1, pad 1."""
+    """benchmark configuration 5: [32,56,56,64] (x) [64,3,3,64], stride 1, pad 1."""
     say("C5 full size")
     rng = np.random.default_rng(55)
     xf = np.maximum(rng.standard_normal((32, 56, 56, 64), dtype=np.float32), 0)
@@ -188,7 +188,7 @@ def test_conv_fused(cabi, golden, c, path):
 
 
 def test_conv_fused_c5_sized(cabi):
-    """conv2d_add_relu at BASELINE config 5's size (the residual block of a ResNet stage)."""
+    """conv2d_add_relu at benchmark configuration 5's size (the residual block of a ResNet stage)."""
     say("conv fused C5 size")
     rng = np.random.default_rng(56)
     xq = rng.integers(0, 256, (32, 56, 56, 64), dtype=np.uint8)

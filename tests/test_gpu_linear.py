@@ -102,7 +102,7 @@ def test_dtype_and_epilogue_variants(cabi, x_signed, relu, bias, pc):
 
 @pytest.mark.parametrize("m", [1, 4, 16])
 def test_decode_shapes(cabi, m):
-    """BASELINE config 4: M in {1,4,16}, K = N = 4096."""
+    """benchmark configuration 4: M in {1,4,16}, K = N = 4096."""
     say("decode", m)
     c = _tile_case(m, 4096, 4096, seed=40 + m)
     y, acc, _ = _run(cabi, c)
@@ -152,7 +152,7 @@ def test_empty_batch(cabi):
 
 
 def test_c1_golden(cabi, golden):
-    """BASELINE config 1 end to end on the device: dynamic quantize of x,
+    """benchmark configuration 1 end to end on the device: dynamic quantize of x,
     per-channel quantize of W, prepack, linear."""
     say("C1")
     c1 = cases.c1_case()
@@ -176,7 +176,7 @@ def test_c1_golden(cabi, golden):
 
 
 def test_c3_full_size(cabi):
-    """BASELINE config 3 (M=4096, K=4096, N=11008): oracle parity on sampled
+    """benchmark configuration 3 (M=4096, K=4096, N=11008): oracle parity on sampled
     rows, and the all-ones identity acc[m][n] = colsum[n] on the whole output."""
     M, K, N = 4096, 4096, 11008
     say("C3 full size")

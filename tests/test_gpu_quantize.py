@@ -154,7 +154,7 @@ def test_per_channel_weight_sized(cabi):
 
 
 def test_full_size_properties(cabi):
-    """BASELINE config 2 at full size (2**28 fp32): properties that need no
+    """benchmark configuration 2 at full size (2**28 fp32): properties that need no
     full-size oracle run, plus oracle parity on sampled windows."""
     n = 2 ** 28
     say("C2 full size", n)
