@@ -101,11 +101,19 @@ int tmq_quantize_per_tensor_dev(const float* x, void* q, int64_t n,
 /* The whole dynamic quantization on the device: min/max over x, the parameters
  * into *qparams (device memory), the codes into q.  Small inputs (at most
  * 65536 elements) take one launch, larger ones three; `workspace` as for
- * tmq_minmax (unused, and may be NULL, for the small case).  Same results as
- * tmq_minmax + tmq_choose_qparams_dev + tmq_quantize_per_tensor_dev. */
+ * tmq_minmax (unused, and may be NULL, for the small case).
+ * rounding = TMQ_ROUND_PRODUCT: q = clamp(rne(fl(x * inv)) + zp), the same
+ * results as tmq_minmax + tmq_choose_qparams_dev + tmq_quantize_per_tensor_dev
+ * (aten::quantize_per_tensor_dynamic).
+ * rounding = TMQ_ROUND_FUSED: q = clamp(rne(fl(x * inv + zp))), product and
+ * zero point rounded once: the activation quantization inside PyTorch's CPU
+ * quantized::linear_dynamic (fbgemm PackAWithQuantRowOffset), which differs
+ * from the former for about one value in 10^5. */
+#define TMQ_ROUND_PRODUCT 0
+#define TMQ_ROUND_FUSED 1
 int tmq_quantize_per_tensor_dynamic_dev(const float* x, void* q, int64_t n, int q_signed,
-                                        int reduce_range, tmq_qparams* qparams, void* workspace,
-                                        size_t workspace_bytes, tmq_stream_t stream);
+                                        int reduce_range, int rounding, tmq_qparams* qparams,
+                                        void* workspace, size_t workspace_bytes, tmq_stream_t stream);
 /* Host-side ChooseQuantizationParams, same arithmetic (pure CPU, no GPU call). */
 int tmq_choose_qparams_host(float min, float max, int q_signed, int reduce_range,
                             double* scale, int32_t* zero_point);
@@ -188,9 +196,24 @@ typedef struct tmq_linear_desc {
   int32_t reserved;
   void* y;                 /* [M,N] bytes, row pitch ldy */
   int64_t ldy;
+  /* Optional scratch device memory, owned by the caller like every other
+   * buffer (16-byte aligned; contents undefined before and after the call).
+   * With at least tmq_linear_workspace_bytes(M, N, K) bytes, products whose
+   * tile grid is much smaller than the chip (a few hundred rows) are computed
+   * split along K: partial sums into the workspace, then one pass that adds
+   * and requantises them.  NULL / too small: single-launch kernels, same
+   * results. */
+  void* workspace;
+  int64_t workspace_bytes;
 } tmq_linear_desc;
 
 int tmq_linear(const tmq_linear_desc* desc, tmq_stream_t stream);
+
+/* Bytes of workspace that tmq_linear / tmq_linear_f32 / tmq_linear_acc32 can
+ * use for this problem size; 0 when the single-launch kernels are chosen
+ * anyway.  No counterpart in the reference: muDNN allocates its own scratch
+ * through the InternalMemAlloc callback (torch_musa/csrc/aten/utils/Utils.cpp:79-153). */
+int64_t tmq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* Raw accumulators acc[m][n] = sum_k X[m][k] * W[n][k] as int32 (row pitch
  * ldacc), from the same MFMA main loop, for bit-exactness checks.  Uses

@@ -66,6 +66,17 @@ def quantize_per_tensor(x, scale, zp, is_signed=False, nthreads=1):
     return q
 
 
+def quantize_per_tensor_fused(x, scale, zp, is_signed=False, nthreads=1):
+    """clamp(rne(fma(x, 1/scale, zp))): the activation quantization of the CPU
+    quantized::linear_dynamic."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    q = np.empty(x.shape, dtype=_qdtype(is_signed))
+    lib().orc_quantize_per_tensor_fused(_p(x), C.c_int64(x.size), C.c_double(scale),
+                                        C.c_int64(zp), C.c_int(is_signed), _p(q),
+                                        C.c_int(nthreads))
+    return q
+
+
 def dequantize_per_tensor(q, scale, zp, nthreads=1):
     q = _as_bytes(q)
     r = np.empty(q.shape, dtype=np.float32)
@@ -234,7 +245,7 @@ def linear_dynamic(x, wq, w_scales, bias, relu=False, reduce_range=False):
     x = np.ascontiguousarray(x, dtype=np.float32)
     mn, mx = minmax(x)
     scale, zp = choose_qparams(mn, mx, False, reduce_range)
-    xq = quantize_per_tensor(x.reshape(-1, x.shape[-1]), scale, zp, False)
+    xq = quantize_per_tensor_fused(x.reshape(-1, x.shape[-1]), scale, zp, False)
     y = linear_f32(xq, scale, zp, wq, w_scales, bias, relu)
     return y.reshape(x.shape[:-1] + (y.shape[-1],))
 

@@ -85,6 +85,30 @@ ORC_API void orc_quantize_per_tensor(const float* x, int64_t n, double scale,
     q[i] = (uint8_t)quantize_one(x[i], inv, zp, qmin, qmax);
 }
 
+/* Activation quantization inside PyTorch's CPU quantized::linear_dynamic: the
+ * activations are quantized while fbgemm packs them (PackAWithQuantRowOffset;
+ * its source is not in this image, the form below is pinned by the op's outputs
+ * on inputs chosen where the two forms differ, see tests/golden):
+ *   t = fma(x, inv, zp)   (one fp32 rounding);  clip to [qmin, qmax];  round to
+ *   nearest even
+ * against quantize_one's rne(fl(x * inv)) + zp.  The reference declares
+ * apply_dynamic and leaves it unimplemented (mudnn/Linear.h:35-46). */
+ORC_API void orc_quantize_per_tensor_fused(const float* x, int64_t n, double scale,
+                                           int64_t zp, int is_signed, uint8_t* q,
+                                           int nthreads) {
+  int64_t qmin, qmax;
+  qrange(is_signed, &qmin, &qmax);
+  const float scale_f = (float)scale;
+  const float inv = 1.0f / scale_f;
+  (void)nthreads;
+#pragma omp parallel for num_threads(nthreads > 0 ? nthreads : 1) schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float t = fmaf(x[i], inv, (float)zp);
+    t = t < (float)qmin ? (float)qmin : (t > (float)qmax ? (float)qmax : t);
+    q[i] = (uint8_t)(int32_t)nearbyintf(t);
+  }
+}
+
 /* dequantize per tensor.  fbgemm/QuantUtils.h:155-158:
  *   r = scale_f * (float)(int32(q) - zp)
  * Stands behind reference AffineQuantizer.mu:79-97,145-179. */

@@ -16,6 +16,8 @@ from __future__ import annotations
 
 import zlib
 
+import functools
+
 import numpy as np
 
 
@@ -391,6 +393,27 @@ def qavgpool_cases():
     return out
 
 
+@functools.lru_cache(maxsize=None)
+def _rounding_probe_rows():
+    """[8, 64] float activations with minimum -8 and maximum 9 (scale 17/255,
+    zero point 120) whose other values are picked where rne(fl(x * inv)) + zp
+    and rne(fl(x * inv + zp)) disagree -- about six values in a million do -- so
+    that a dynamic linear that quantizes its activations in the wrong one of the
+    two forms cannot pass."""
+    rng = np.random.default_rng(1799)
+    cand = (rng.standard_normal(6_000_000) * 2.5).astype(np.float32)
+    cand = cand[(cand > -7.9) & (cand < 8.9)]
+    inv = np.float32(1.0) / np.float32(17.0 / 255.0)
+    two_step = np.rint(cand * inv) + np.float32(120)
+    fused = np.rint((cand.astype(np.float64) * np.float64(inv) + 120.0).astype(np.float32))
+    picked = cand[two_step != fused]
+    assert picked.size >= 16, picked.size
+    x = (rng.standard_normal(512) * 2.0).astype(np.float32)
+    x[: picked.size][:400] = picked[:400]
+    x[510], x[511] = np.float32(-8.0), np.float32(9.0)
+    return rng.permutation(x).reshape(8, 64).copy()
+
+
 def linear_dynamic_cases():
     """Float activations for quantized::linear_dynamic: dict(name, x, wq, w_scales,
     bias, relu, reduce_range). Weight zero points are 0."""
@@ -417,6 +440,11 @@ def linear_dynamic_cases():
             w_scales = np.array([float(np.float32(0.00093))])
         bias = rng.standard_normal(n).astype(np.float32) if has_bias else None
         out.append(dict(name=name, x=x, wq=wq, w_scales=w_scales, bias=bias, relu=relu, reduce_range=rr))
+    rng = np.random.default_rng(1798)
+    out.append(dict(name="rounding_forms_8x64_40", x=_rounding_probe_rows(),
+                    wq=rng.integers(-127, 128, (40, 64), dtype=np.int8),
+                    w_scales=(0.0005 + 0.001 * rng.random(40)).astype(np.float32).astype(np.float64),
+                    bias=rng.standard_normal(40).astype(np.float32), relu=False, reduce_range=False))
     return out
 
 

@@ -37,7 +37,7 @@ def test_struct_sizes_match_the_header():
     # natural alignment on x86-64: see include/tmq.h
     import ctypes as C
     assert C.sizeof(cabi.QParams) == 16
-    assert C.sizeof(cabi.LinearDesc) == 128
+    assert C.sizeof(cabi.LinearDesc) == 144
     assert C.sizeof(cabi.Conv2dGeom) == 14 * 8
     assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8
     assert C.sizeof(cabi.Conv2dPost) == 24

@@ -170,6 +170,29 @@ def test_qlinear_matches_cpu_op(per_channel, relu, bias):
     assert (b2 is None) == (b is None) and (b is None or torch.equal(b2.cpu(), b))
 
 
+def test_qlinear_long_k_through_the_operators():
+    """150 rows against K = 8192: the operators hand the C ABI a workspace and the
+    product runs split along K; quantized::linear and quantized::linear_dynamic
+    against the CPU ops, bit for bit."""
+    say("aten qlinear split K")
+    torch.manual_seed(11)
+    x = torch.randn(150, 8192)
+    w = torch.randn(200, 8192) * 0.05
+    b = torch.randn(200)
+    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+    s = (w.abs().amax(dim=1) / 127).to(torch.float64)
+    wq = torch.quantize_per_channel(w, s, torch.zeros(200, dtype=torch.int64), 0, torch.qint8)
+    cpu_packed = torch.ops.quantized.linear_prepack(wq, b)
+    packed = torch.ops.quantized.linear_prepack(wq.cuda(), b.cuda())
+    ref = torch.ops.quantized.linear(xq, cpu_packed, 0.25, 120)
+    got = torch.ops.quantized.linear(xq.cuda(), packed, 0.25, 120)
+    assert 0.2 < ((ref.int_repr() > 0) & (ref.int_repr() < 255)).float().mean()
+    assert_q_equal(got, ref, abs_diff=0)
+    refd = torch.ops.quantized.linear_dynamic(x, cpu_packed, False)
+    gotd = torch.ops.quantized.linear_dynamic(x.cuda(), packed, False)
+    assert torch.equal(gotd.cpu(), refd)
+
+
 def test_qlinear_errors():
     w = torch.quantize_per_tensor(torch.randn(8, 16), 0.1, 3, torch.qint8).cuda()
     with pytest.raises(RuntimeError):

@@ -4,6 +4,7 @@ int32 accumulators: bit-exact against the oracle (exact integer matmul).
 Requantised bytes: the stated bar is 1 LSB; the epilogue restates the oracle's
 operation order, so the tests also report (and require) exact equality against
 the oracle, and stay within 1 LSB of the golden vectors of PyTorch's CPU op."""
+import ctypes as C
 import numpy as np
 import pytest
 import torch
@@ -210,6 +211,66 @@ def test_c3_full_size(cabi):
     assert torch.equal(acc + acc2, 255 * pw.colsum[None, :].expand(M, N))
 
 
+# ---- split K (a few hundred rows, long K: partial sums in a caller-owned workspace) --------
+@pytest.mark.parametrize("shape,x_signed,relu,bias,pc", [
+    ((100, 520, 8208), False, False, True, True),     # 8 splits, K ends inside a stage, ragged M and N
+    ((300, 300, 8192), True, True, False, False),     # qint8 activations, per-tensor weight scale
+    ((130, 4096, 11008), False, True, True, True),    # 64 tiles, 4 splits of 43 stages
+])
+def test_split_k(cabi, shape, x_signed, relu, bias, pc):
+    say("split K", shape, x_signed, relu, bias, pc)
+    M, N, K = shape
+    assert cabi.lib().tmq_linear_workspace_bytes(M, N, K) > 0, "this shape is meant to take the split schedule"
+    c = _tile_case(M, N, K, seed=4242 + M, x_signed=x_signed, relu=relu, bias=bias, per_channel=pc)
+    y, acc, pw = _run(cabi, c, 13)      # 13: split schedule or an error
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "split K")
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    yf = host(cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, relu=relu))
+    np.testing.assert_array_equal(
+        yf, oracle.linear_f32(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], relu=relu,
+                              nthreads=8))
+    # without a workspace the single-launch kernels give the same bytes
+    cabi.use_linear_workspace = False
+    try:
+        y1, acc1, _ = _run(cabi, c)
+        yf1 = host(cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, relu=relu))
+    finally:
+        cabi.use_linear_workspace = True
+    np.testing.assert_array_equal(y1, y)
+    np.testing.assert_array_equal(acc1, acc)
+    np.testing.assert_array_equal(yf1, yf)
+
+
+def test_split_k_workspace_rules(cabi):
+    """No workspace for the weight-streaming rows and for grids that fill the chip; a
+    workspace that is too small is ignored, not overrun."""
+    wsb = cabi.lib().tmq_linear_workspace_bytes
+    assert wsb(16, 4096, 4096) == 0 and wsb(64, 4096, 4096) == 0
+    assert wsb(4096, 11008, 4096) == 0 and wsb(2048, 4096, 4096) == 0
+    assert wsb(128, 4096, 4096) == 0                     # K too short for the cut to pay
+    assert wsb(128, 4096, 11008) == 8 * 128 * 4096 * 4   # 32 tiles of 128 x 128, 8 splits
+    assert wsb(512, 4096, 11008) == 2 * 512 * 4096 * 4   # 128 tiles, 2 splits
+    assert wsb(128, 4098, 8192) == 7 * 128 * 4100 * 4    # 33 tiles, 7 splits; partial rows padded to 16 bytes
+    assert wsb(0, 10, 10) == 0 and wsb(-1, 10, 10) == 0
+    c = _tile_case(100, 520, 8208, seed=5)
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    xq, ws, b = dev(c["xq"]), dev(c["w_scales"].astype(np.float32)), dev(c["bias"])
+    y = torch.empty((100, 520), dtype=torch.uint8, device="cuda")
+    d = cabi._linear_desc(xq, pw, c["x_scale"], c["x_zp"], ws, b, c["out_scale"], c["out_zp"], False, False, y)
+    assert d.workspace_bytes > 1024
+    guard = torch.full((4096,), 0x5A, dtype=torch.uint8, device="cuda")
+    d.workspace, d.workspace_bytes = guard.data_ptr(), 1024    # far too small
+    cabi.check(cabi.lib().tmq_linear(C.byref(d), cabi.stream_ptr()), "tmq_linear")
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"])
+    _check(host(y), want, "small workspace")
+    assert bool((guard == 0x5A).all())
+
+
 # ---- float output (the second half of a dynamically quantized linear) --------------
 # Float results are compared bit for bit: the kernel's epilogue is the oracle's
 # single fused multiply-add, and the dynamic quantization in front of it is
@@ -259,7 +320,7 @@ def test_linear_dynamic_prefill_sized(cabi):
     y = host(cabi.linear_dynamic(dev(x), pw, dev(wsc.astype(np.float32)), dev(bias)))
     mn, mx = oracle.minmax(x)
     scale, zp = oracle.choose_qparams(mn, mx, False, False)
-    xq = oracle.quantize_per_tensor(x, scale, zp, False, nthreads=8)
+    xq = oracle.quantize_per_tensor_fused(x, scale, zp, False, nthreads=8)
     want = oracle.linear_f32(xq, scale, zp, wq, wsc, bias, nthreads=8)
     np.testing.assert_array_equal(y, want)
 

@@ -294,6 +294,25 @@ def test_quantize_dynamic_on_device(cabi, n, offset, signed, reduce_range):
     np.testing.assert_array_equal(host(q), oracle.quantize_per_tensor(x[offset:], scale, zp, signed))
 
 
+@pytest.mark.parametrize("n,offset", [(4099, 1), (65536, 0), ((1 << 22) + 3, 0)])
+@pytest.mark.parametrize("signed", [False, True])
+def test_quantize_dynamic_fused_rounding(cabi, n, offset, signed):
+    # the activation quantization of the CPU quantized::linear_dynamic: x * inv + zp
+    # rounded once; at 4 Mi elements a few dozen codes differ from the two-step form
+    say("dynamic dev fused", n, offset, signed)
+    rng = np.random.default_rng(77 + n)
+    x = (rng.standard_normal(n + offset) * 2.5 + 0.4).astype(np.float32)
+    xd = dev(x)[offset:]
+    q, qp = cabi.quantize_per_tensor_dynamic_dev(xd.contiguous() if offset == 0 else xd, signed, False, fused=True)
+    mn, mx = oracle.minmax(x[offset:])
+    scale, zp = oracle.choose_qparams(mn, mx, signed, False)
+    assert cabi.read_qparams(qp) == (scale, zp)
+    want = oracle.quantize_per_tensor_fused(x[offset:], scale, zp, signed, nthreads=8)
+    np.testing.assert_array_equal(host(q), want)
+    if n > (1 << 22) and not signed:   # (with a zero point near 0 the two forms rarely part)
+        assert np.count_nonzero(want != oracle.quantize_per_tensor(x[offset:], scale, zp, signed, nthreads=8)) > 0
+
+
 @pytest.mark.parametrize("kind", ["gelu", "gelu_tanh", "sigmoid"])
 @pytest.mark.parametrize("c", cases.qunary_cases(), ids=lambda c: c["name"])
 def test_qunary(cabi, golden, c, kind):

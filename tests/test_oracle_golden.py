@@ -186,6 +186,24 @@ def test_linear_dynamic(golden, c):
     np.testing.assert_array_equal(y, golden[k + "/y"])
 
 
+def test_linear_dynamic_pins_the_activation_rounding(golden):
+    """On the case built from values where the two forms disagree, only the fused
+    form (one rounding of x * inv + zp) reproduces the CPU op; the form of
+    quantize_per_tensor does not."""
+    c = [c for c in cases.linear_dynamic_cases() if c["name"].startswith("rounding_forms")][0]
+    want = golden["lindyn/" + c["name"] + "/y"]
+    mn, mx = oracle.minmax(c["x"])
+    scale, zp = oracle.choose_qparams(mn, mx, False, False)
+    assert (scale, zp) == (17.0 / 255.0, 120)
+    fused = oracle.quantize_per_tensor_fused(c["x"], scale, zp)
+    plain = oracle.quantize_per_tensor(c["x"], scale, zp)
+    assert np.count_nonzero(fused != plain) >= 16
+    y_fused = oracle.linear_f32(fused, scale, zp, c["wq"], c["w_scales"], c["bias"])
+    y_plain = oracle.linear_f32(plain, scale, zp, c["wq"], c["w_scales"], c["bias"])
+    np.testing.assert_array_equal(y_fused, want)
+    assert np.count_nonzero(y_plain != want) > 0
+
+
 def _close_to(y, want, out_dtype, what):
     assert y.shape == want.shape and y.dtype == want.dtype, what
     if out_dtype == "float32":

@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_acc32", "tmq_linear_f32", "tmq_quantize_per_tensor_dynamic_dev",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_acc32", "tmq_linear_f32", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
@@ -51,6 +51,7 @@ class LinearDesc(C.Structure):
         ("out_scale", C.c_float), ("out_zero_point", C.c_int32),
         ("out_signed", C.c_int32), ("reserved", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
     ]
 
 
@@ -100,6 +101,8 @@ def lib() -> C.CDLL:
             getattr(l, name).restype = C.c_int64
         l.tmq_linear_packed_kchunks.argtypes = [C.c_int64]
         l.tmq_linear_packed_bytes.argtypes = [C.c_int64, C.c_int64]
+        l.tmq_linear_workspace_bytes.restype = C.c_int64
+        l.tmq_linear_workspace_bytes.argtypes = [C.c_int64, C.c_int64, C.c_int64]
         l.tmq_conv2d_packed_bytes.restype = C.c_int64
         l.tmq_conv2d_packed_bytes.argtypes = [C.POINTER(Conv2dGeom)]
         v = C.c_void_p
@@ -119,7 +122,7 @@ def lib() -> C.CDLL:
         l.tmq_linear.argtypes = [C.POINTER(LinearDesc), v]
         l.tmq_linear_acc32.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, v]
         l.tmq_linear_f32.argtypes = [C.POINTER(LinearDesc), v, v, C.c_int64, v]
-        l.tmq_quantize_per_tensor_dynamic_dev.argtypes = [v, v, C.c_int64, C.c_int, C.c_int, v, v, C.c_size_t, v]
+        l.tmq_quantize_per_tensor_dynamic_dev.argtypes = [v, v, C.c_int64, C.c_int, C.c_int, C.c_int, v, v, C.c_size_t, v]
         l.tmq_conv2d_prepack.argtypes = [v, C.POINTER(Conv2dGeom), v, v, v]
         l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         l.tmq_conv2d.argtypes = [C.POINTER(Conv2dDesc), v]
@@ -219,15 +222,17 @@ def quantize_per_tensor_dev(x: torch.Tensor, qp: torch.Tensor, signed: bool) -> 
     return q
 
 
-def quantize_per_tensor_dynamic_dev(x: torch.Tensor, signed: bool, reduce_range: bool):
-    """-> (codes, 16 device bytes of qparams); one launch for small inputs, three otherwise."""
+def quantize_per_tensor_dynamic_dev(x: torch.Tensor, signed: bool, reduce_range: bool, fused: bool = False):
+    """-> (codes, 16 device bytes of qparams); one launch for small inputs, three otherwise.
+    fused: round x * inv + zp once (the CPU linear_dynamic's activation quantization)
+    instead of rne(x * inv) + zp (quantize_per_tensor)."""
     assert x.dtype == torch.float32 and x.is_contiguous()
     q = torch.empty(x.shape, dtype=torch.int8 if signed else torch.uint8, device=x.device)
     qp = torch.empty(16, dtype=torch.uint8, device=x.device)
     ws = minmax_workspace(x.device)
     check(lib().tmq_quantize_per_tensor_dynamic_dev(x.data_ptr(), q.data_ptr(), x.numel(), int(signed),
-                                                    int(reduce_range), qp.data_ptr(), ws.data_ptr(), ws.numel(),
-                                                    stream_ptr()), "tmq_quantize_per_tensor_dynamic_dev")
+                                                    int(reduce_range), int(fused), qp.data_ptr(), ws.data_ptr(),
+                                                    ws.numel(), stream_ptr()), "tmq_quantize_per_tensor_dynamic_dev")
     return q, qp
 
 
@@ -294,6 +299,13 @@ class PackedLinear:
         return w
 
 
+# False: never hand a workspace to the linear entry points (single-launch kernels only)
+use_linear_workspace = True
+# a preallocated uint8 tensor that every call on its device shares instead (calls
+# on one stream run in order, so one buffer serves them all); None: per call
+linear_workspace = None
+
+
 def _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed, relu, y):
     d = LinearDesc()
     d.M, d.K = x.shape
@@ -312,6 +324,16 @@ def _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_si
     d.out_scale, d.out_zero_point, d.out_signed = out_scale, out_zp, int(out_signed)
     if y is not None:
         d.y, d.ldy = y.data_ptr(), y.stride(0)
+    nbytes = lib().tmq_linear_workspace_bytes(d.M, d.N, d.K) if use_linear_workspace else 0
+    if nbytes > 0:
+        # split-K scratch, from the caching allocator; the descriptor keeps it
+        # alive until the call is queued on the current stream
+        shared = linear_workspace
+        if shared is not None and shared.device == x.device and shared.numel() >= nbytes:
+            d._workspace = shared
+        else:
+            d._workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        d.workspace, d.workspace_bytes = d._workspace.data_ptr(), nbytes
     return d
 
 
@@ -351,7 +373,7 @@ def linear_dynamic(x, pw: PackedLinear, w_scales, bias, relu=False, reduce_range
     """min/max -> qparams -> quantize -> product, all on the device, no host round trip."""
     assert x.dtype == torch.float32 and x.is_contiguous()
     x2 = x.reshape(-1, x.shape[-1])
-    xq, qp = quantize_per_tensor_dynamic_dev(x2, False, reduce_range)
+    xq, qp = quantize_per_tensor_dynamic_dev(x2, False, reduce_range, fused=True)
     y = linear_f32(xq, pw, 1.0, 0, w_scales, bias, relu, qparams_dev=qp)
     return y.reshape(tuple(x.shape[:-1]) + (pw.N,))
 

@@ -48,6 +48,18 @@ void check_status(int status, const char* what) {
   TORCH_CHECK(status == TMQ_OK, what, " failed: ", tmq_status_string(status));
 }
 
+// Scratch memory for the split-K schedule of products with a few hundred rows:
+// allocated through the caching allocator (stream-ordered reuse), attached to
+// the descriptor, kept alive by the returned tensor until the call is queued.
+at::Tensor attach_linear_workspace(tmq_linear_desc& d, const at::TensorOptions& like) {
+  const int64_t bytes = tmq_linear_workspace_bytes(d.M, d.N, d.K);
+  if (bytes <= 0) return at::Tensor();
+  at::Tensor ws = at::empty({bytes}, like.dtype(at::kByte));
+  d.workspace = ws.data_ptr();
+  d.workspace_bytes = bytes;
+  return ws;
+}
+
 bool is_signed_qtype(c10::ScalarType t, const char* what) {
   TORCH_CHECK(t == c10::kQInt8 || t == c10::kQUInt8, what, ": only QInt8 and QUInt8 are supported, got ",
               toString(t));
@@ -366,8 +378,11 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     at::Tensor qp = at::empty({static_cast<int64_t>(sizeof(tmq_qparams))}, bytes);
     at::Tensor xq = at::empty({x.numel()}, bytes);
     auto* qpd = static_cast<tmq_qparams*>(qp.data_ptr());
-    check_status(tmq_quantize_per_tensor_dynamic_dev(cptr<float>(x), xq.data_ptr(), x.numel(), 0, reduce_range, qpd,
-                                                     ws.data_ptr(), static_cast<size_t>(ws.numel()), stream),
+    // the CPU op quantizes the activations while packing them, with product and
+    // zero point rounded once
+    check_status(tmq_quantize_per_tensor_dynamic_dev(cptr<float>(x), xq.data_ptr(), x.numel(), 0, reduce_range,
+                                                     TMQ_ROUND_FUSED, qpd, ws.data_ptr(),
+                                                     static_cast<size_t>(ws.numel()), stream),
                  "tmq_quantize_per_tensor_dynamic_dev");
     tmq_linear_desc d{};
     d.M = M;
@@ -383,6 +398,7 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     d.w_per_channel = wp_.per_channel;
     d.relu = relu;
     d.bias = bias_.has_value() ? cptr<float>(*bias_) : nullptr;
+    const at::Tensor split_ws = attach_linear_workspace(d, bytes);
     check_status(tmq_linear_f32(&d, qpd, mptr<float>(y), N_, stream), "tmq_linear_f32");
     return y;
   }
@@ -425,6 +441,7 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     d.out_signed = x_signed;
     d.y = y.data_ptr();
     d.ldy = N_;
+    const at::Tensor split_ws = attach_linear_workspace(d, x.options());
     check_status(tmq_linear(&d, current_stream(x)), "tmq_linear");
     return y;
   }
@@ -958,6 +975,7 @@ at::Tensor qlinear_per_tensor_run(at::Tensor act, double act_scale, int64_t act_
   d.w_per_channel = ws.numel() > 1;
   d.relu = post == "relu";
   d.bias = b.has_value() ? cptr<float>(*b) : nullptr;
+  const at::Tensor split_ws = attach_linear_workspace(d, act.options());
   if (float_path) {
     check_status(tmq_linear_f32(&d, nullptr, mptr<float>(y), N, stream), "tmq_linear_f32");
     if (post == "tanh") y = at::tanh(y);

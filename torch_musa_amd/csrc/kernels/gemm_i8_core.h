@@ -95,6 +95,12 @@ struct GemmArgs {
   // null: x_scale and acc_coef above hold.  acc_base is acc_coef + zero point.
   const tmq_qparams* x_qp_dev = nullptr;
   int32_t acc_base = 0;
+  // Split K (raw int32 output of plain activation rows only): block row
+  // blockIdx.y multiplies stages [y * split_stages, (y + 1) * split_stages) of
+  // the k loop and writes its partial sums to y + blockIdx.y * split_stride.
+  int32_t splits = 1;
+  int32_t split_stages = 0;
+  int64_t split_stride = 0;
 };
 
 struct XQuant {
@@ -352,6 +358,17 @@ __global__ __launch_bounds__(WM* WN* kWave, (WDMA && WM * WN == 4 && (BM / WM) *
 void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int NT = WM * WN * kWave;
   constexpr bool kHasPost = XSRC::kPostOps;  // residual / activation epilogue compiled in
+  if constexpr (MODE == kOutAcc32 && std::is_same<XSRC, XLinear>::value) {
+    if (a.splits > 1) {  // this block's share of K: move the operands, shorten K
+      const int64_t sp = blockIdx.y;
+      const int64_t k0 = sp * a.split_stages * kBK;
+      const int64_t left = a.K - k0, mine = static_cast<int64_t>(a.split_stages) * kBK;
+      a.K = left < mine ? left : mine;
+      a.w_packed += sp * a.split_stages * (kChunks * 256);
+      xsrc.x += k0;
+      a.y = static_cast<int32_t*>(a.y) + sp * a.split_stride;
+    }
+  }
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int NW = BN * kChunks / NT;  // 16-byte weight chunks per thread per stage
@@ -380,7 +397,7 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int kMainBytes = kWBufs * kWStage + kXBufs * kXStage;
   constexpr int kF32Pitch = BN * 4 + 16;  // float rows of the tile, same idea
   constexpr int kOutBytes =
-      (MODE == kOutAcc32) ? 0 : (MODE == kOutF32 ? WM * 32 * kF32Pitch : BM * kOutPitch);
+      (MODE == kOutAcc32 || MODE == kOutF32) ? WM * 32 * kF32Pitch : BM * kOutPitch;
   constexpr int kTileBytes = kMainBytes > kOutBytes ? kMainBytes : kOutBytes;
   __shared__ __attribute__((aligned(16))) uint8_t smem[kTileBytes];
   __shared__ __attribute__((aligned(16))) int s_acc0[BN];
@@ -712,25 +729,9 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
 
   // ---- epilogue.  A lane holds, per 32x32 MFMA tile, channels
   // n = 8g + 4*half + j (g, j < 4) of activation row m = li.
-  if constexpr (MODE == kOutAcc32) {
-    int32_t* y = static_cast<int32_t*>(a.y);
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int64_t n = n0 + wn0 + tn * 32 + 8 * g + 4 * half;
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
-          const int64_t m = m0 + wm0 + tm * 32 + li;
-          if (m >= a.M) continue;
-          int32_t* dst = y + m * a.ldy + a.n_off + n;
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            if (n + j < a.N) dst[j] = acc[tn][tm][4 * g + j];
-        }
-      }
-  } else if constexpr (MODE == kOutF32) {
-    // Float results, one 32-row MFMA tile of every wave at a time: the waves
+  if constexpr (MODE == kOutF32 || MODE == kOutAcc32) {
+    // Float results (or the raw accumulators, moved as 32-bit patterns through
+    // the same path), one 32-row MFMA tile of every wave at a time: the waves
     // write their rows into LDS, then all threads copy whole rows out, 16 B per
     // lane on consecutive addresses (a lane's own four floats of 32 different
     // rows would make 32 partial lines per store instruction).
@@ -750,8 +751,11 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
           v4f v;
 #pragma unroll
           for (int j = 0; j < 4; ++j)
-            v[j] = __builtin_fmaxf(
-                __builtin_fmaf(static_cast<float>(acc[tn][tm][4 * g + j]), mult[j], bias[j]), a.lo_f);
+            v[j] = MODE == kOutAcc32
+                       ? __int_as_float(acc[tn][tm][4 * g + j])
+                       : __builtin_fmaxf(
+                             __builtin_fmaf(static_cast<float>(acc[tn][tm][4 * g + j]), mult[j], bias[j]),
+                             a.lo_f);
           *reinterpret_cast<v4f*>(&smem[((wave % WM) * 32 + li) * kF32Pitch + nl * 4]) = v;
         }
       __syncthreads();

@@ -6,7 +6,7 @@
 #include "gemm_i8_core.h"
 
 // Layout that non-C++ bindings rely on (natural alignment, x86-64).
-static_assert(sizeof(tmq_linear_desc) == 128, "tmq_linear_desc layout changed");
+static_assert(sizeof(tmq_linear_desc) == 144, "tmq_linear_desc layout changed");
 static_assert(sizeof(tmq_qparams) == 16, "tmq_qparams layout changed");
 
 namespace tmq {
@@ -277,9 +277,154 @@ int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   return launch_status();
 }
 
+// ---- split K for a few hundred rows against a long K.  The tile grid of such a
+// product is far smaller than the chip (M = 128, N = 4096: 32 tiles of
+// 128 x 128) and every block walks all of K alone at the latency of one stage
+// after the other, so K is cut into `splits` runs of whole stages: splits x
+// tiles blocks write raw int32 partial sums [split][M][ldp] into a caller-owned
+// workspace and a second kernel adds them up and requantises.  Writing and
+// re-reading the partial sums costs about 10 us at these sizes, which the
+// shorter k loops repay from K = 8192 on (measured: M = 128, N = 4096,
+// K = 11008: 38.5 -> 25 us; K = 4096: 14.6 -> 20 us, hence no split there).
+struct SplitPlan {
+  int splits = 1;   // 1: single launch
+  int stages = 0;   // k stages (64 bytes of K) per split
+  int64_t ldp = 0;  // row pitch of a partial-sum slice, int32 elements
+};
+
+constexpr int64_t kSplitBlocks = 256;    // blocks wanted: one per CU
+constexpr int64_t kSplitMinKT = 128;     // shortest k loop (stages) worth cutting
+constexpr int64_t kSplitMinStages = 16;  // shortest run of stages per split
+
+SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
+  SplitPlan p;
+  if (M <= kDecodeRowsAuto || K % 16 != 0) return p;
+  const int64_t KT = ceil_div(K, kBK);
+  const int64_t tiles = ceil_div(M, 128) * ceil_div(N, 128);
+  if (KT < kSplitMinKT || tiles > kSplitBlocks / 2) return p;
+  int64_t splits = kSplitBlocks / tiles;
+  if (splits > KT / kSplitMinStages) splits = KT / kSplitMinStages;
+  if (splits < 2) return p;
+  const int64_t stages = ceil_div(KT, splits);
+  splits = ceil_div(KT, stages);
+  // the last split keeps at least three stages (the direct-copy ring's minimum)
+  if (KT - (splits - 1) * stages < 3) --splits;
+  if (splits < 2) return p;
+  p.splits = static_cast<int>(splits);
+  p.stages = static_cast<int>(stages);
+  p.ldp = (N + 3) / 4 * 4;
+  return p;
+}
+
+int64_t split_workspace_bytes(const SplitPlan& p, int64_t M) {
+  return p.splits > 1 ? p.splits * M * p.ldp * static_cast<int64_t>(sizeof(int32_t)) : 0;
+}
+
+// Second kernel of a split-K product: a block owns 256 consecutive channels and
+// `rows` rows.  Its threads first compute the 256 channels' constants, one
+// channel each, into LDS (the two divisions per channel would otherwise be
+// repeated by every row); then a thread adds the `splits` partial sums of four
+// consecutive channels of one row at a time and runs the epilogue of the
+// single-launch kernels (same helper, same operation order).
+template <int MODE>
+__global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs a, const int32_t* parts, int splits,
+                                                            int64_t ldp, int64_t slice, int rows) {
+  __shared__ __attribute__((aligned(16))) int s_add[256];
+  __shared__ __attribute__((aligned(16))) float s_mult[256];
+  __shared__ __attribute__((aligned(16))) float s_bdiv[256];
+  const int t = threadIdx.x;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * 256;
+  {
+    const XQuant xq = x_quant(a);
+    const int64_t nj = n0 + t < a.N ? n0 + t : a.N - 1;
+    float mult = 0.f, bdiv = 0.f;
+    if (MODE != kOutAcc32) {
+      const float atw = xq.scale * a.w_scales[nj * a.w_scale_stride];
+      if (MODE == kOutF32) {
+        mult = atw;
+        bdiv = a.bias != nullptr ? a.bias[nj] : 0.f;
+      } else {
+        mult = atw / a.out_scale;
+        bdiv = a.bias != nullptr ? a.bias[nj] / atw : 0.f;
+      }
+    }
+    s_add[t] = xq.coef * a.colsum[nj];
+    s_mult[t] = mult;
+    s_bdiv[t] = bdiv;
+  }
+  __syncthreads();
+  const int q = t & 63;
+  const int64_t n = n0 + q * 4;
+  if (n >= a.N) return;
+  const v4i add = *reinterpret_cast<const v4i*>(&s_add[q * 4]);
+  const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[q * 4]);
+  const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[q * 4]);
+  const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
+  const int64_t mbeg = static_cast<int64_t>(blockIdx.y) * rows;
+  const int64_t mend = mbeg + rows < a.M ? mbeg + rows : a.M;
+  for (int64_t m = mbeg + (t >> 6); m < mend; m += 4) {
+    const int32_t* src = parts + m * ldp + n;
+    v4i sum = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src));
+    for (int sp = 1; sp < splits; ++sp)
+      sum += __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + sp * slice));
+    sum += add;
+    const int raw[4] = {sum.x, sum.y, sum.z, sum.w};
+    if constexpr (MODE == kOutAcc32) {
+      int32_t* dst = static_cast<int32_t*>(a.y) + m * a.ldy + n;
+      for (int j = 0; j < 4; ++j)
+        if (n + j < a.N) dst[j] = raw[j];
+    } else if constexpr (MODE == kOutF32) {
+      store_f32x4(a, m, n, raw, mult, bdiv);
+    } else {
+      const uint32_t q4 = plain_u8 ? requant4<MODE, false>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f)
+                                   : requant4<MODE, true>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+      uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
+      if (n + 3 < a.N && (reinterpret_cast<uintptr_t>(dst) & 3) == 0) {
+        *reinterpret_cast<uint32_t*>(dst) = q4;
+      } else {
+        for (int j = 0; j < 4; ++j)
+          if (n + j < a.N) dst[j] = static_cast<uint8_t>(q4 >> (8 * j));
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN, int PD = 4, bool WDMA = false>
+int launch_gemm_split(const GemmArgs& a, const XLinear& xs, const SplitPlan& p, hipStream_t s) {
+  const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  gemm_i8_kernel<BM, BN, WM, WN, kOutAcc32, XLinear, PD, WDMA>
+      <<<dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(p.splits)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
+  return launch_status();
+}
+
+template <int MODE>
+int run_split(const GemmArgs& a, const XLinear& xs, const SplitPlan& p, void* workspace, bool dma_ok,
+              hipStream_t s) {
+  GemmArgs part = a;  // first kernel: pure sums of (x ^ flip) * w, no zero-point term
+  part.acc_coef = 0;
+  part.acc_base = 0;
+  part.x_qp_dev = nullptr;
+  part.y = workspace;
+  part.ldy = p.ldp;
+  part.splits = p.splits;
+  part.split_stages = p.stages;
+  part.split_stride = a.M * p.ldp;
+  const int rc = dma_ok ? launch_gemm_split<128, 128, 2, 2, 3, true>(part, xs, p, s)
+                        : launch_gemm_split<128, 128, 2, 2>(part, xs, p, s);
+  if (rc != TMQ_OK) return rc;
+  // rows per block: enough blocks to hide the loads' latency, then longer runs
+  const int rows = a.M <= 256 ? 4 : 16;
+  const int64_t bx = ceil_div(a.N, 256), by = ceil_div(a.M, rows);
+  if (bx > 0x7fffffff || by > 65535) return TMQ_ERR_UNSUPPORTED;  // a split product has a few hundred rows
+  splitk_finish_kernel<MODE><<<dim3(static_cast<unsigned>(bx), static_cast<unsigned>(by)), dim3(256), 0, s>>>(
+      a, static_cast<const int32_t*>(workspace), p.splits, p.ldp, a.M * p.ldp, rows);
+  return launch_status();
+}
+
 template <int MODE>
 int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec_ok,
-                    hipStream_t s) {
+                    hipStream_t s, void* workspace = nullptr, int64_t workspace_bytes = 0) {
   const int forced = g_forced_config.load(std::memory_order_relaxed);
   if (!vec_ok || forced == 9) {
     // plain kernel accumulates true activation values: undo the +128 share
@@ -310,6 +455,13 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   // the direct-copy kernels address 256 rows of either operand with 32-bit offsets
   // and run their three-stage ring at least once around
   const bool dma_ok = xs.ldx <= (int64_t{1} << 23) && a.K <= (int64_t{1} << 23) && a.K > 2 * kBK;
+  if (forced < 0 || forced == 13) {
+    const SplitPlan p = plan_split(a.M, a.N, a.K);
+    if (p.splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(p, a.M) &&
+        aligned(workspace, 16))
+      return run_split<MODE>(a, xs, p, workspace, dma_ok, s);
+    if (forced == 13) return TMQ_ERR_UNSUPPORTED;
+  }
   int cfg = forced;
   if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
@@ -413,6 +565,11 @@ TMQ_EXPORT int tmq_linear_unpack(const void* packed, int64_t N, int64_t K, int8_
   return launch_status();
 }
 
+TMQ_EXPORT int64_t tmq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  return split_workspace_bytes(plan_split(M, N, K), M);
+}
+
 TMQ_EXPORT int tmq_linear(const tmq_linear_desc* d, tmq_stream_t stream) {
   GemmArgs a{};
   XLinear xs{};
@@ -435,8 +592,8 @@ TMQ_EXPORT int tmq_linear(const tmq_linear_desc* d, tmq_stream_t stream) {
   a.y = d->y;
   a.ldy = d->ldy;
   hipStream_t s = as_stream(stream);
-  return d->out_signed ? dispatch_linear<kOutS8>(a, xs, d->x_signed, vec_ok, s)
-                       : dispatch_linear<kOutU8>(a, xs, d->x_signed, vec_ok, s);
+  return d->out_signed ? dispatch_linear<kOutS8>(a, xs, d->x_signed, vec_ok, s, d->workspace, d->workspace_bytes)
+                       : dispatch_linear<kOutU8>(a, xs, d->x_signed, vec_ok, s, d->workspace, d->workspace_bytes);
 }
 
 TMQ_EXPORT int tmq_linear_acc32(const tmq_linear_desc* d, int32_t* acc, int64_t ldacc,
@@ -450,7 +607,8 @@ TMQ_EXPORT int tmq_linear_acc32(const tmq_linear_desc* d, int32_t* acc, int64_t 
   a.acc_coef = d->x_signed ? 0 : 128;  // undo the x ^ 0x80 shift only
   a.y = acc;
   a.ldy = ldacc;
-  return dispatch_linear<kOutAcc32>(a, xs, d->x_signed, vec_ok, as_stream(stream));
+  return dispatch_linear<kOutAcc32>(a, xs, d->x_signed, vec_ok, as_stream(stream), d->workspace,
+                                    d->workspace_bytes);
 }
 
 TMQ_EXPORT int tmq_linear_f32(const tmq_linear_desc* d, const tmq_qparams* x_qparams_dev, float* y,
@@ -474,7 +632,8 @@ TMQ_EXPORT int tmq_linear_f32(const tmq_linear_desc* d, const tmq_qparams* x_qpa
   a.lo_f = d->relu ? 0.f : -__builtin_inff();
   a.y = y;
   a.ldy = ldy;
-  return dispatch_linear<kOutF32>(a, xs, d->x_signed, vec_ok, as_stream(stream));
+  return dispatch_linear<kOutF32>(a, xs, d->x_signed, vec_ok, as_stream(stream), d->workspace,
+                                  d->workspace_bytes);
 }
 
 // Benchmark hook (not part of the public header): force a kernel

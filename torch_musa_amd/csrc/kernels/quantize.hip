@@ -23,25 +23,36 @@ constexpr int kUnroll = 8;    // independent 16-byte loads per thread, min/max p
 // 2**28 elements (6.7 and 7.2 TB/s of algorithmic traffic; 8 per thread: 6.0 / 5.3)
 constexpr int kUnrollQD = 2;
 
-template <bool SIGNED>
+// FUSED = false: q = clamp(rne(fl(x * inv)) + zp), the arithmetic of
+// quantize_per_tensor.  FUSED = true: q = clamp(rne(fl(x * inv + zp))), one
+// rounding of product and zero point together, which is how PyTorch's CPU
+// quantized::linear_dynamic quantizes its activations while it packs them
+// (fbgemm PackAWithQuantRowOffset: fmadd, clip, cvtps); the two differ for
+// about one value in 10^5 whose product lies next to a half.
+template <bool SIGNED, bool FUSED = false>
 __device__ __forceinline__ int quantize_one(float x, float inv, float zp_f) {
   constexpr float lo = SIGNED ? -128.f : 0.f;
   constexpr float hi = SIGNED ? 127.f : 255.f;
-  float t = x * inv;
-  float r = __builtin_rintf(t);  // v_rndne_f32: ties to even
-  // zp_f and every in-range r are small integers, so the sum is exact whenever
-  // it can land inside [lo, hi]; larger magnitudes clamp either way.
-  r = r + zp_f;
+  float r;
+  if constexpr (FUSED) {
+    r = __builtin_rintf(__builtin_fmaf(x, inv, zp_f));
+  } else {
+    float t = x * inv;
+    r = __builtin_rintf(t);  // v_rndne_f32: ties to even
+    // zp_f and every in-range r are small integers, so the sum is exact whenever
+    // it can land inside [lo, hi]; larger magnitudes clamp either way.
+    r = r + zp_f;
+  }
   r = fminf(fmaxf(r, lo), hi);
   return static_cast<int>(r);
 }
 
-template <bool SIGNED>
+template <bool SIGNED, bool FUSED = false>
 __device__ __forceinline__ uint32_t quantize_four(v4f v, float inv, float zp_f) {
-  uint32_t a = static_cast<uint32_t>(quantize_one<SIGNED>(v.x, inv, zp_f)) & 0xffu;
-  uint32_t b = static_cast<uint32_t>(quantize_one<SIGNED>(v.y, inv, zp_f)) & 0xffu;
-  uint32_t c = static_cast<uint32_t>(quantize_one<SIGNED>(v.z, inv, zp_f)) & 0xffu;
-  uint32_t d = static_cast<uint32_t>(quantize_one<SIGNED>(v.w, inv, zp_f)) & 0xffu;
+  uint32_t a = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.x, inv, zp_f)) & 0xffu;
+  uint32_t b = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.y, inv, zp_f)) & 0xffu;
+  uint32_t c = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.z, inv, zp_f)) & 0xffu;
+  uint32_t d = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.w, inv, zp_f)) & 0xffu;
   return a | (b << 8) | (c << 16) | (d << 24);
 }
 
@@ -84,7 +95,7 @@ __device__ __forceinline__ void resolve(const QParamsArg& a, float& inv, float& 
 // The fp32 input is read once and never again: non-temporal loads keep it out of
 // the caches.  The codes are written with ordinary stores, so a consumer that
 // follows on the stream (dequantize, a GEMM) finds them in the last-level cache.
-template <bool SIGNED>
+template <bool SIGNED, bool FUSED = false>
 __global__ __launch_bounds__(kThreads) void quantize_vec_kernel(
     const v4f* __restrict__ x4, uint32_t* __restrict__ q4, int64_t n4,
     const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, QParamsArg qp) {
@@ -96,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void quantize_vec_kernel(
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u) v[u] = __builtin_nontemporal_load(&x4[base + u * kThreads]);
 #pragma unroll
-    for (int u = 0; u < kUnrollQD; ++u) q4[base + u * kThreads] = quantize_four<SIGNED>(v[u], inv, zp_f);
+    for (int u = 0; u < kUnrollQD; ++u) q4[base + u * kThreads] = quantize_four<SIGNED, FUSED>(v[u], inv, zp_f);
   } else {
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u) {
@@ -106,24 +117,24 @@ __global__ __launch_bounds__(kThreads) void quantize_vec_kernel(
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u) {
       const int64_t i = base + u * kThreads;
-      if (i < n4) q4[i] = quantize_four<SIGNED>(v[u], inv, zp_f);
+      if (i < n4) q4[i] = quantize_four<SIGNED, FUSED>(v[u], inv, zp_f);
     }
   }
   if (blockIdx.x == 0) {
     const int64_t i = 4 * n4 + threadIdx.x;
-    if (i < n) q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(x[i], inv, zp_f));
+    if (i < n) q[i] = static_cast<uint8_t>(quantize_one<SIGNED, FUSED>(x[i], inv, zp_f));
   }
 }
 
 // Fallback for pointers that are not 16-byte (x) / 4-byte (q) aligned.
-template <bool SIGNED>
+template <bool SIGNED, bool FUSED = false>
 __global__ __launch_bounds__(kThreads) void quantize_scalar_kernel(
     const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, QParamsArg qp) {
   float inv, zp_f;
   resolve(qp, inv, zp_f);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride)
-    q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(x[i], inv, zp_f));
+    q[i] = static_cast<uint8_t>(quantize_one<SIGNED, FUSED>(x[i], inv, zp_f));
 }
 
 // The codes are read with ordinary loads (they are small and usually still in
@@ -339,7 +350,7 @@ __global__ __launch_bounds__(kThreads) void minmax_final_choose_kernel(
 // cost several times what the work does.
 constexpr int kDynSmallThreads = 1024;
 constexpr int64_t kDynSmallMax = 65536;  // elements
-template <bool SIGNED>
+template <bool SIGNED, bool FUSED>
 __global__ __launch_bounds__(kDynSmallThreads) void dynamic_quantize_small_kernel(
     const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, int qmin, int qmax,
     int reduce_range, bool vec, tmq_qparams* __restrict__ out) {
@@ -399,10 +410,10 @@ __global__ __launch_bounds__(kDynSmallThreads) void dynamic_quantize_small_kerne
 #pragma unroll
   for (int u = 0; u < kHeld; ++u) {
     const int64_t i = t + static_cast<int64_t>(u) * kDynSmallThreads;
-    if (i < n4) q4[i] = quantize_four<SIGNED>(held[u], inv, zp_f);
+    if (i < n4) q4[i] = quantize_four<SIGNED, FUSED>(held[u], inv, zp_f);
   }
   for (int64_t i = 4 * n4 + t; i < n; i += kDynSmallThreads)
-    q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(x[i], inv, zp_f));
+    q[i] = static_cast<uint8_t>(quantize_one<SIGNED, FUSED>(x[i], inv, zp_f));
 }
 
 // ---------------------------------------------------------------------------
@@ -529,28 +540,28 @@ inline unsigned grid_for(int64_t work_items, int64_t per_block, int64_t cap) {
   return static_cast<unsigned>(g);
 }
 
-int quantize_launch(const float* x, void* q, int64_t n, QParamsArg qp, int q_signed,
-                    hipStream_t s) {
-  if (n == 0) return TMQ_OK;
+template <bool SIGNED, bool FUSED>
+int quantize_launch_as(const float* x, void* q, int64_t n, QParamsArg qp, hipStream_t s) {
   uint8_t* qb = static_cast<uint8_t*>(q);
   if (aligned(x, 16) && aligned(q, 4)) {
     const int64_t n4 = n / 4;
     const int64_t blocks = n4 == 0 ? 1 : ceil_div(n4, kThreads * kUnrollQD);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-    auto* x4 = reinterpret_cast<const v4f*>(x);
-    auto* q4 = reinterpret_cast<uint32_t*>(q);
-    if (q_signed)
-      quantize_vec_kernel<true><<<dim3(blocks), dim3(kThreads), 0, s>>>(x4, q4, n4, x, qb, n, qp);
-    else
-      quantize_vec_kernel<false><<<dim3(blocks), dim3(kThreads), 0, s>>>(x4, q4, n4, x, qb, n, qp);
+    quantize_vec_kernel<SIGNED, FUSED><<<dim3(blocks), dim3(kThreads), 0, s>>>(
+        reinterpret_cast<const v4f*>(x), reinterpret_cast<uint32_t*>(q), n4, x, qb, n, qp);
   } else {
     const unsigned g = grid_for(n, kThreads, 65536);
-    if (q_signed)
-      quantize_scalar_kernel<true><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, qp);
-    else
-      quantize_scalar_kernel<false><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, qp);
+    quantize_scalar_kernel<SIGNED, FUSED><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, qp);
   }
   return launch_status();
+}
+
+int quantize_launch(const float* x, void* q, int64_t n, QParamsArg qp, int q_signed, hipStream_t s,
+                    bool fused = false) {
+  if (n == 0) return TMQ_OK;
+  if (fused)
+    return q_signed ? quantize_launch_as<true, true>(x, q, n, qp, s) : quantize_launch_as<false, true>(x, q, n, qp, s);
+  return q_signed ? quantize_launch_as<true, false>(x, q, n, qp, s) : quantize_launch_as<false, false>(x, q, n, qp, s);
 }
 
 bool zp_in_range(int64_t zp, int q_signed) {
@@ -653,21 +664,26 @@ TMQ_EXPORT int tmq_choose_qparams_dev(const float* minmax, int q_signed, int red
 }
 
 TMQ_EXPORT int tmq_quantize_per_tensor_dynamic_dev(const float* x, void* q, int64_t n, int q_signed,
-                                                   int reduce_range, tmq_qparams* qparams, void* workspace,
-                                                   size_t workspace_bytes, tmq_stream_t stream) {
+                                                   int reduce_range, int rounding, tmq_qparams* qparams,
+                                                   void* workspace, size_t workspace_bytes, tmq_stream_t stream) {
   if (n < 0 || qparams == nullptr || (n > 0 && (x == nullptr || q == nullptr))) return TMQ_ERR_INVALID_ARGUMENT;
+  if (rounding != TMQ_ROUND_PRODUCT && rounding != TMQ_ROUND_FUSED) return TMQ_ERR_INVALID_ARGUMENT;
+  const bool fused = rounding == TMQ_ROUND_FUSED;
   if (!aligned(x, 4)) return TMQ_ERR_ALIGNMENT;
   hipStream_t s = as_stream(stream);
   const int qmin = q_signed ? -128 : 0, qmax = q_signed ? 127 : 255;
   if (n <= kDynSmallMax) {
     const bool vec = aligned(x, 16) && aligned(q, 4);
     uint8_t* qb = static_cast<uint8_t*>(q);
-    if (q_signed)
-      dynamic_quantize_small_kernel<true><<<dim3(1), dim3(kDynSmallThreads), 0, s>>>(x, qb, n, qmin, qmax,
-                                                                                      reduce_range, vec, qparams);
+    const dim3 one(1), block(kDynSmallThreads);
+    if (q_signed && fused)
+      dynamic_quantize_small_kernel<true, true><<<one, block, 0, s>>>(x, qb, n, qmin, qmax, reduce_range, vec, qparams);
+    else if (q_signed)
+      dynamic_quantize_small_kernel<true, false><<<one, block, 0, s>>>(x, qb, n, qmin, qmax, reduce_range, vec, qparams);
+    else if (fused)
+      dynamic_quantize_small_kernel<false, true><<<one, block, 0, s>>>(x, qb, n, qmin, qmax, reduce_range, vec, qparams);
     else
-      dynamic_quantize_small_kernel<false><<<dim3(1), dim3(kDynSmallThreads), 0, s>>>(x, qb, n, qmin, qmax,
-                                                                                       reduce_range, vec, qparams);
+      dynamic_quantize_small_kernel<false, false><<<one, block, 0, s>>>(x, qb, n, qmin, qmax, reduce_range, vec, qparams);
     return launch_status();
   }
   if (workspace == nullptr || workspace_bytes < tmq_minmax_workspace_bytes(n) || !aligned(workspace, 4))
@@ -688,7 +704,7 @@ TMQ_EXPORT int tmq_quantize_per_tensor_dynamic_dev(const float* x, void* q, int6
   qp.inv = 0.f;
   qp.zp_f = 0.f;
   qp.dev = qparams;
-  return quantize_launch(x, q, n, qp, q_signed, s);
+  return quantize_launch(x, q, n, qp, q_signed, s, fused);
 }
 
 TMQ_EXPORT int tmq_choose_qparams_host(float min, float max, int q_signed, int reduce_range,
