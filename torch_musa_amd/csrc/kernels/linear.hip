@@ -466,7 +466,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
-    // the CUs busy, the 128x128 tile (three blocks per CU) down to 64 tiles.
+    // the CUs busy, the 128x128 tile (three blocks per CU) down to 128 tiles.
     const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
     // (and only when the rows fill at least 55 % of the row tiles: a tile's time
     // does not shrink with its padding; M = 100 and 150 against N = 49152 sit on
@@ -474,7 +474,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     const auto rows_used = [&](int bm) { return a.M * 20 >= ceil_div(a.M, bm) * bm * 11; };
     if (nblk(256, 256) >= 160 && rows_used(256))
       cfg = 6;  // 8 waves of 128x64, operands copied straight into LDS
-    else if (nblk(128, 128) >= 64)
+    else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
     else
       cfg = 2;
