@@ -108,6 +108,12 @@ def test_conv_mfma_shapes(cabi, spec, x_signed, path):
     (2, 28, 28, 64, 128, 1, 1, 0, 1, 1),     # 1x1
     (1, 40, 40, 16, 64, 7, 2, 3, 1, 1),      # 7x7 stride 2
     (1, 1, 1, 16, 1, 1, 1, 0, 1, 1),         # a single output value
+    (8, 56, 56, 64, 64, 3, 1, 1, 1, 1),      # 56-wide rows: patches a quarter of a row wide, tall
+    (3, 57, 57, 32, 64, 3, 1, 1, 1, 1),      # a width no patch width divides
+    (9, 28, 28, 512, 128, 1, 1, 0, 1, 1),    # 1x1 over many input channels: halo tiles (32 KB slice)
+    (4, 56, 56, 256, 96, 1, 2, 0, 1, 1),     # 1x1 stride 2: kernel smaller than the stride, implicit GEMM
+    (4, 56, 56, 64, 128, 3, 2, 1, 1, 1),     # 3x3 stride 2: halo tiles
+    (2, 38, 19, 16, 64, 2, 2, 0, 1, 1),      # 2x2 stride 2: every pixel used once
 ])
 def test_conv_auto_path_shapes(cabi, spec):
     say("conv auto", spec)

@@ -188,16 +188,27 @@ int lds_limit() {
   return limit;
 }
 
-// Chooses the patch that minimises a simple time estimate: rounds of blocks
-// over the 256 CUs times (fixed cost + MFMA time of the busiest SIMD + copy
-// time).  Returns false when the weight slice or the smallest halo do not fit.
+// Chooses the patch that minimises a time estimate fitted to per-phase cycle
+// stamps and a sweep of patch shapes at [32,56,56,64] x [64,3,3,64].  Per block:
+//   fixed      3000 cycles of set-up, barriers and first-load latency
+//   mfma       the busiest SIMD's row tiles x k-steps x 64 cycles
+//   copy       weight bytes / 16 + 290 cycles per pass of the block over the halo
+//              (a pass moves floor(512 / slots per halo row) whole halo rows, so
+//              narrow halos waste fewer lanes: 28x14 patches take 5 passes where
+//              7x56 patches of the same 392 pixels take 9)
+//   epilogue   8.4 cycles per output pixel
+// Blocks that fit a CU's LDS together overlap: the first costs the whole chain,
+// each further one the larger of its SIMD work (half the fixed cost + mfma +
+// epilogue) and its copies; blocks that do not fit run one after the other.  Returns false when
+// the weight slice or the smallest halo do not fit.
 bool plan_tiles(const ConvShape& s, bool forced, TilePlan* best) {
-  // The halo tiles pay off through the reuse of an input pixel by the taps that
-  // cover it: KH*KW / (stride_h*stride_w) uses per loaded pixel.  1x1 kernels
-  // and strided 3x3 kernels (reuse 1 and 2.25) run faster as an implicit GEMM
-  // (measured over ResNet-50's layer shapes: 1.0-1.5x); 3x3 stride 1 and 7x7
-  // stride 2 (reuse 9 and 12) are 1.3-1.6x faster here.
-  if (!forced && s.KH * s.KW < 3 * s.sh * s.sw) return false;
+  // A block loads every pixel of its halo, so a kernel smaller than its stride
+  // (1x1 stride 2: three of four loaded pixels unused) runs 1.6-3.7x faster as an
+  // implicit GEMM, which gathers only what it multiplies.  Everything else that
+  // fits is faster here, measured over ResNet-50's layer shapes at batch 32:
+  // 3x3 stride 1 and 7x7 stride 2 by 1.8x, 3x3 stride 2 by 1.2-1.7x, 1x1 stride 1
+  // by 1.05-1.8x.
+  if (!forced && s.KH * s.KW < s.sh * s.sw) return false;
   const int64_t icb = s.ICg / 16;
   const int64_t chunks = s.KH * s.KW * icb;
   const int64_t KS = round_up(ceil_div(chunks, 2), 2);  // <= packed k-chunks / 2 (padded to 8)
@@ -206,15 +217,31 @@ bool plan_tiles(const ConvShape& s, bool forced, TilePlan* best) {
   if (w_bytes > 96 * 1024 || icb > 64) return false;
   const int64_t pitch = (icb | 1) * 16;
   const int64_t n_tiles = ceil_div(s.OCg, kCtBN);
-  const int64_t tw_caps[6] = {128, 64, 32, 16, 8, 4};
+  constexpr int64_t kCuLds = 160 * 1024;
+  // patch widths: the whole row or a power of two, and the row cut into 2..8 equal parts
+  int64_t widths[14];
+  int nw = 0;
+  const auto add_width = [&](int64_t w) {
+    if (w < 1) return;
+    for (int i = 0; i < nw; ++i)
+      if (widths[i] == w) return;
+    widths[nw++] = w;
+  };
+  const int forced_cols = g_forced_cols.load(std::memory_order_relaxed);
+  const int forced_rows = g_forced_rows.load(std::memory_order_relaxed);
+  if (forced_cols > 0) {
+    add_width(s.OW < forced_cols ? s.OW : forced_cols);
+  } else {
+    for (int64_t cap : {128, 64, 32, 16, 8, 4}) add_width(s.OW < cap ? s.OW : cap);
+    for (int64_t parts = 2; parts <= 8; ++parts) add_width(ceil_div(s.OW, parts));
+  }
   double best_cost = -1.0;
-  for (int64_t cap : tw_caps) {
-    const int forced_cols = g_forced_cols.load(std::memory_order_relaxed);
-    if (forced_cols > 0 && cap != 128) continue;
-    const int64_t TW = forced_cols > 0 ? (s.OW < forced_cols ? s.OW : forced_cols) : (s.OW < cap ? s.OW : cap);
+  for (int wi = 0; wi < nw; ++wi) {
+    const int64_t TW = widths[wi];
     const int64_t HWd = (TW - 1) * s.sw + (s.KW - 1) * s.dw + 1;
-    if (HWd * (pitch / 16) > kCtThreads) continue;  // one halo row is copied in one pass of the block
-    const int forced_rows = g_forced_rows.load(std::memory_order_relaxed);
+    const int64_t row_slots = HWd * (pitch / 16);
+    if (row_slots > kCtThreads) continue;  // one halo row is copied in one pass of the block
+    const int64_t rows_per_pass = kCtThreads / row_slots;
     for (int64_t TH = 1; TH <= s.OH && TH * TW <= kCtMaxPixels; ++TH) {
       if (forced_rows > 0 && TH != forced_rows) continue;
       const int64_t HH = (TH - 1) * s.sh + (s.KH - 1) * s.dh + 1;
@@ -223,9 +250,18 @@ bool plan_tiles(const ConvShape& s, bool forced, TilePlan* best) {
       if (total > budget) break;
       const int64_t blocks = s.B * ceil_div(s.OH, TH) * ceil_div(s.OW, TW) * n_tiles * s.groups;
       const int64_t MT = ceil_div(TH * TW, 32);
-      const double per_block = 3000.0 + static_cast<double>(ceil_div(MT, 4) * KS * 64) +
-                               static_cast<double>(w_bytes + x_bytes) / 64.0;
-      const double cost = static_cast<double>(ceil_div(blocks, 256)) * per_block;
+      const double mfma = static_cast<double>(ceil_div(MT, 4) * KS * 64);
+      const double copy = static_cast<double>(w_bytes) / 16.0 + 290.0 * static_cast<double>(ceil_div(HH, rows_per_pass));
+      const double epilogue = 8.4 * static_cast<double>(TH * TW);
+      const int64_t per_cu = ceil_div(blocks, 256);
+      int64_t together = kCuLds / (total + 3 * kCtBN * 4);
+      together = together < 1 ? 1 : (together > per_cu ? per_cu : together);
+      // half of the fixed cost is instructions (set-up, address tables), which a
+      // co-resident block cannot hide
+      const double simd = 1500.0 + mfma + epilogue;
+      const double overlapped = simd > copy ? simd : copy;
+      const double group = 3000.0 + mfma + copy + epilogue + static_cast<double>(together - 1) * overlapped;
+      const double cost = static_cast<double>(ceil_div(per_cu, together)) * group;
       if (best_cost < 0 || cost < best_cost) {
         best_cost = cost;
         best->TH = static_cast<int>(TH); best->TW = static_cast<int>(TW);
