@@ -88,6 +88,28 @@ def test_tile_configs(cabi, cfg, shape):
     _check(y, want, f"cfg {cfg}")
 
 
+# wave groups that split the k loop inside a block (stage counts the group count divides)
+@pytest.mark.parametrize("cfg", [14])
+@pytest.mark.parametrize("shape", [(300, 520, 512), (257, 33, 256), (64, 1040, 1024), (130, 260, 1008), (100, 70, 4096), (65, 48, 128)])
+def test_k_split_wave_groups(cabi, cfg, shape):
+    say("k-split groups cfg", cfg, shape)
+    c = _tile_case(*shape, seed=cfg * 7 + shape[0], relu=bool(shape[0] & 1))
+    y, acc, pw = _run(cabi, c, cfg)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, f"cfg {cfg}")
+    cabi.force_linear_config(cfg)
+    try:
+        yf = host(cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], dev(c["w_scales"].astype(np.float32)),
+                                  dev(c["bias"]), relu=c["relu"]))
+    finally:
+        cabi.force_linear_config(-1)
+    np.testing.assert_array_equal(
+        yf, oracle.linear_f32(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], relu=c["relu"],
+                              nthreads=8))
+
+
 @pytest.mark.parametrize("x_signed,relu,bias,pc", [(True, False, True, True), (True, True, False, False),
                                                    (False, True, True, False), (False, False, False, True)])
 def test_dtype_and_epilogue_variants(cabi, x_signed, relu, bias, pc):

@@ -353,10 +353,31 @@ __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv,
 // pipe about a quarter of its time on this chip: the ds_write_b128 traffic of
 // eight waves, mixed with their fragment reads, backs up the LDS queue and the
 // fragment reads behind it.
-template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4, bool WDMA = false>
-__global__ __launch_bounds__(WM* WN* kWave, (WDMA && WM * WN == 4 && (BM / WM) * (BN / WN) <= 128 * 64) ? 2 : 1)
+//
+// KW > 1 (register staging of plain activation rows only): KW groups of WM x WN
+// waves share one output tile and split its k loop into KW equal runs of
+// stages, each group with its own LDS stages and registers; after the loop the
+// groups' accumulators are added through LDS and group 0 runs the epilogue.
+// For grids far smaller than the chip: a lone block per CU spends most of a
+// stage waiting on its own chain LDS store -> barrier -> LDS read -> MFMA, and
+// the other groups' waves fill those gaps.  The host sends only k loops whose
+// stage count KW divides.
+template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4, bool WDMA = false, int KW = 1>
+__global__ __launch_bounds__(WM* WN* KW* kWave, (WDMA && WM * WN == 4 && (BM / WM) * (BN / WN) <= 128 * 64) ? 2 : 1)
 void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
-  constexpr int NT = WM * WN * kWave;
+  constexpr int NT = WM * WN * kWave;   // threads of one group
+  constexpr int NTB = NT * KW;          // threads of the block
+  static_assert(KW >= 1 && (KW == 1 || (!WDMA && std::is_same<XSRC, XLinear>::value)),
+                "k-split groups: register staging of plain rows only");
+  const int kg = KW == 1 ? 0 : static_cast<int>(threadIdx.x) / NT;  // this thread's group
+  if constexpr (KW > 1) {  // this group's share of K: move the operands, shorten K
+    const int64_t per = ceil_div(a.K, kBK) / KW;
+    const int64_t k0 = kg * per * kBK;
+    const int64_t left = a.K - k0;
+    a.K = left < per * kBK ? left : per * kBK;
+    a.w_packed += kg * per * (kChunks * 256);
+    xsrc.x += k0;
+  }
   constexpr bool kHasPost = XSRC::kPostOps;  // residual / activation epilogue compiled in
   if constexpr (MODE == kOutAcc32 && std::is_same<XSRC, XLinear>::value) {
     if (a.splits > 1) {  // this block's share of K: move the operands, shorten K
@@ -398,15 +419,19 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int kF32Pitch = BN * 4 + 16;  // float rows of the tile, same idea
   constexpr int kOutBytes =
       (MODE == kOutAcc32 || MODE == kOutF32) ? WM * 32 * kF32Pitch : BM * kOutPitch;
-  constexpr int kTileBytes = kMainBytes > kOutBytes ? kMainBytes : kOutBytes;
+  constexpr int kSumBytes = (KW - 1) * NT * TN * TM * 64;  // the other groups' accumulators
+  constexpr int kLoopBytes = KW * kMainBytes > kSumBytes ? KW * kMainBytes : kSumBytes;
+  constexpr int kTileBytes = kLoopBytes > kOutBytes ? kLoopBytes : kOutBytes;
   __shared__ __attribute__((aligned(16))) uint8_t smem[kTileBytes];
   __shared__ __attribute__((aligned(16))) int s_acc0[BN];
   __shared__ __attribute__((aligned(16))) float s_mult[BN];
   __shared__ __attribute__((aligned(16))) float s_bdiv[BN];
-  uint8_t* const sW = smem;                      // [kWBufs][kWStage]
-  uint8_t* const sX = smem + kWBufs * kWStage;   // [kXBufs][kXStage]
+  uint8_t* const gmem = smem + kg * kMainBytes;  // this group's stages
+  uint8_t* const sW = gmem;                      // [kWBufs][kWStage]
+  uint8_t* const sX = gmem + kWBufs * kWStage;   // [kXBufs][kXStage]
 
-  const int t = threadIdx.x;
+  const int tb = threadIdx.x;
+  const int t = KW == 1 ? tb : tb - kg * NT;
   const int lane = t % kWave, wave = t / kWave;
   const int li = lane & 31, half = lane >> 5;
   const int wm0 = (wave % WM) * WTM;
@@ -469,6 +494,14 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
         init[r] = s_acc0[wn0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3)];
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = init;
+    }
+    if (KW > 1 && kg > 0) {  // the start value is added once, by group 0
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[tn][tm][r] = 0;
     }
   };
 
@@ -649,9 +682,9 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   // k-th LDS store of a stage
   auto store_one = [&](int set, int buf, int k) {
     if (k < NW)
-      *reinterpret_cast<v4i*>(&smem[buf * kWStage + wdst[k]]) = wreg[set][k];
+      *reinterpret_cast<v4i*>(&gmem[buf * kWStage + wdst[k]]) = wreg[set][k];
     else
-      *reinterpret_cast<v4i*>(&smem[buf * kXStage + xdst[k - NW]]) = xreg[set][k - NW] ^ xmask;
+      *reinterpret_cast<v4i*>(&gmem[buf * kXStage + xdst[k - NW]]) = xreg[set][k - NW] ^ xmask;
   };
 
   // ---- software pipeline.
@@ -727,8 +760,45 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
     if (kt0 + j < KT) stage(kt0 + j, (j + 1) % NSET, (j + 2) % NSET);
   }
 
+  if constexpr (KW > 1) {
+    // add the groups' partial sums: groups 1 .. KW-1 park theirs in LDS (16 B per
+    // lane, consecutive lanes on consecutive addresses), group 0 adds them up
+    __syncthreads();  // every group is done with its stages
+    v4i* const park = reinterpret_cast<v4i*>(smem);
+    if (kg > 0) {
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const v4i v = {acc[tn][tm][4 * g], acc[tn][tm][4 * g + 1], acc[tn][tm][4 * g + 2],
+                           acc[tn][tm][4 * g + 3]};
+            park[(((kg - 1) * TN * TM + tn * TM + tm) * 4 + g) * NT + t] = v;
+          }
+    }
+    __syncthreads();
+    if (kg == 0) {
+#pragma unroll
+      for (int og = 0; og < KW - 1; ++og)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const v4i v = park[((og * TN * TM + tn * TM + tm) * 4 + g) * NT + t];
+              acc[tn][tm][4 * g] += v.x;
+              acc[tn][tm][4 * g + 1] += v.y;
+              acc[tn][tm][4 * g + 2] += v.z;
+              acc[tn][tm][4 * g + 3] += v.w;
+            }
+    }
+  }
+
   // ---- epilogue.  A lane holds, per 32x32 MFMA tile, channels
   // n = 8g + 4*half + j (g, j < 4) of activation row m = li.
+  // (KW > 1: only group 0 holds sums; all threads of the block copy rows out.)
   if constexpr (MODE == kOutF32 || MODE == kOutAcc32) {
     // Float results (or the raw accumulators, moved as 32-bit patterns through
     // the same path), one 32-row MFMA tile of every wave at a time: the waves
@@ -741,6 +811,7 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
       __syncthreads();  // the operand stages, or the previous pass, are read out
+      if (KW == 1 || kg == 0) {
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -758,9 +829,10 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
                              a.lo_f);
           *reinterpret_cast<v4f*>(&smem[((wave % WM) * 32 + li) * kF32Pitch + nl * 4]) = v;
         }
+      }
       __syncthreads();
 #pragma unroll 4
-      for (int id = t; id < WM * 32 * kRowChunks; id += NT) {
+      for (int id = tb; id < WM * 32 * kRowChunks; id += NTB) {
         const int lr = id / kRowChunks, cc = id % kRowChunks;
         const int64_t m = m0 + (lr / 32) * WTM + tm * 32 + (lr % 32), n = n0 + cc * 4;
         if (m >= a.M || n >= a.N) continue;
@@ -809,16 +881,19 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
       }
     };
     // unsigned output without ReLU: the saturating conversion is the clamp
-    if (MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f)
+    if (KW > 1 && kg > 0) {
+      // nothing to requantise in this group
+    } else if (MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f) {
       requant_tile(std::false_type{});
-    else
+    } else {
       requant_tile(std::true_type{});
+    }
     __syncthreads();
     uint8_t* y = static_cast<uint8_t*>(a.y) + a.n_off;
     const bool vec_ok = ((a.ldy & 15) == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
     constexpr int kRowChunks = BN / 16;
 #pragma unroll 4
-    for (int id = t; id < BM * kRowChunks; id += NT) {
+    for (int id = tb; id < BM * kRowChunks; id += NTB) {
       const int row = id / kRowChunks, cc = id % kRowChunks;
       const int64_t m = m0 + row, n = n0 + cc * 16;
       if (m >= a.M || n >= a.N) continue;

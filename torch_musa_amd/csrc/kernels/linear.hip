@@ -268,12 +268,13 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
 // Kernel selection override for benchmarking: -1 = automatic.
 std::atomic<int> g_forced_config{-1};
 
-template <int BM, int BN, int WM, int WN, int MODE, int PD = 4, bool WDMA = false>
+template <int BM, int BN, int WM, int WN, int MODE, int PD = 4, bool WDMA = false, int KW = 1>
 int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
   if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear, PD, WDMA>
-      <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
+  if (KW > 1 && ceil_div(a.K, kBK) % KW != 0) return TMQ_ERR_UNSUPPORTED;  // equal runs of stages only
+  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear, PD, WDMA, KW>
+      <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * KW * kWave), 0, s>>>(a, xs);
   return launch_status();
 }
 
@@ -476,6 +477,9 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
       cfg = 6;  // 8 waves of 128x64, operands copied straight into LDS
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
+    else if (nblk(64, 64) <= 256 && ceil_div(a.K, kBK) >= 32 && ceil_div(a.K, kBK) % 2 == 0)
+      cfg = 14;  // at most one block per CU and a long k loop: two wave groups halve it (14.7 -> 11.7 us
+                 // at M = 128, K = N = 4096; four groups run into the L2's bandwidth: 12.3 us)
     else
       cfg = 2;
   }
@@ -491,6 +495,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 6: return launch_gemm<256, 256, 2, 4, MODE, 3, true>(a, xs, s);
     case 7: return launch_gemm<128, 128, 2, 2, MODE, 3, true>(a, xs, s);
     case 10: return launch_gemm<256, 256, 2, 2, MODE, 3, true>(a, xs, s);
+    case 14: return launch_gemm<64, 64, 2, 2, MODE, 4, false, 2>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
