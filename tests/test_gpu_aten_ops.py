@@ -700,3 +700,60 @@ def test_aten_cat_and_upsample_nearest(dtype, zp):
             assert_q_equal(got, torch.nn.functional.interpolate(t, mode="nearest", **kw))
     m = torch.nn.Upsample(scale_factor=2, mode="nearest")
     assert_q_equal(m(b.cuda()), m(b))
+
+
+def test_ops_replay_from_a_hip_graph():
+    """The operators inside a captured HIP graph (allocations from the graph's pool, no
+    host round trip in the captured region): quantized::linear on a split-K shape and on a
+    large-tile shape, quantized::linear_dynamic, quantized::conv2d_relu and quantized::add.
+    Every replay, with new input contents and eager work in between, equals the eager
+    result."""
+    say("graph replay")
+    torch.manual_seed(21)
+    dev = "cuda"
+    w1 = torch.randn(192, 8192) * 0.05
+    wq1 = torch.quantize_per_tensor(w1, float(w1.abs().max() / 127), 0, torch.qint8).cuda()
+    p1 = torch.ops.quantized.linear_prepack(wq1, torch.randn(192).cuda())
+    w2 = torch.randn(64, 32, 3, 3) * 0.05
+    s2 = (w2.abs().amax(dim=(1, 2, 3)) / 127).double()
+    wq2 = torch.quantize_per_channel(w2, s2, torch.zeros(64, dtype=torch.int64), 0, torch.qint8).cuda()
+    p2 = torch.ops.quantized.conv2d_prepack(wq2, torch.randn(64).cuda(), [1, 1], [1, 1], [1, 1], 1)
+    xf = torch.randn(130, 8192, device=dev)                         # float activations (dynamic linear)
+    xq = torch.quantize_per_tensor(torch.randn(130, 8192, device=dev), 0.04, 120, torch.quint8)
+    xc = torch.quantize_per_tensor(torch.randn(2, 32, 20, 20, device=dev).relu(), 0.03, 0, torch.quint8).contiguous(
+        memory_format=torch.channels_last)
+
+    def work():
+        y1 = torch.ops.quantized.linear(xq, p1, 0.3, 128)
+        y2 = torch.ops.quantized.linear_dynamic(xf, p1, False)
+        y3 = torch.ops.quantized.conv2d_relu(xc, p2, 0.05, 0)
+        y4 = torch.ops.quantized.add(y3, y3, 0.1, 0)
+        return y1, y2, y3, y4
+
+    work()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        work()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            outs = work()
+    torch.cuda.synchronize()
+    for it in range(3):
+        # new contents in the captured input buffers
+        xf.copy_(torch.randn(130, 8192, device=dev) * (1.0 + it))
+        xq_new = torch.quantize_per_tensor(torch.randn(130, 8192, device=dev) * (1.0 + 0.3 * it), 0.04, 120, torch.quint8)
+        xq.copy_(xq_new)
+        xc.copy_(torch.quantize_per_tensor(torch.randn(2, 32, 20, 20, device=dev).relu() * (1.0 + it), 0.03, 0,
+                                           torch.quint8).contiguous(memory_format=torch.channels_last))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = work()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, eager):
+            if got.is_quantized:
+                assert torch.equal(got.int_repr(), want.int_repr()), f"replay {it}"
+            else:
+                assert torch.equal(got, want), f"replay {it}"
