@@ -473,8 +473,20 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     // does not shrink with its padding; M = 100 and 150 against N = 49152 sit on
     // either side)
     const auto rows_used = [&](int bm) { return a.M * 20 >= ceil_div(a.M, bm) * bm * 11; };
+    // One block of either large tile runs per CU, so a launch costs whole rounds
+    // of 256 tiles.  The 128x256 tile (128 activation rows, 256 channels; 8 waves
+    // of 64x64) does half the work of a 256x256 tile in 0.535 of its time (C3:
+    // 181.5 against 170 us) and wins where it rounds better: M = 2048, N = 11008:
+    // 95.4 against 103.3 us; M = 2048, N = 4096: 35.9 against 41.5 us (and 41.3 us
+    // for 128x128 tiles).  Its mirror image, 256 rows x 128 channels, is 17 %
+    // slower than 256x256 at C3: activation rows arrive as 64-byte pieces of
+    // far-apart rows, weight rows as 256-byte pieces of the packed layout.
+    const double rounds256 = static_cast<double>(ceil_div(nblk(256, 256), 256));
+    const double rounds128x256 = 0.535 * static_cast<double>(ceil_div(nblk(128, 256), 256));
     if (nblk(256, 256) >= 160 && rows_used(256))
-      cfg = 6;  // 8 waves of 128x64, operands copied straight into LDS
+      cfg = rounds128x256 < rounds256 ? 17 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
+    else if (nblk(128, 256) >= 160 && rows_used(128))
+      cfg = 17;
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
     else if (nblk(64, 64) <= 256 && ceil_div(a.K, kBK) >= 32 && ceil_div(a.K, kBK) % 2 == 0)
@@ -483,7 +495,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     else
       cfg = 2;
   }
-  if ((cfg == 6 || cfg == 10) && !dma_ok) cfg = 3;
+  if ((cfg == 6 || cfg == 10 || cfg == 17) && !dma_ok) cfg = 3;
   if (cfg == 7 && !dma_ok) cfg = 1;
   switch (cfg) {
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
@@ -496,6 +508,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 7: return launch_gemm<128, 128, 2, 2, MODE, 3, true>(a, xs, s);
     case 10: return launch_gemm<256, 256, 2, 2, MODE, 3, true>(a, xs, s);
     case 14: return launch_gemm<64, 64, 2, 2, MODE, 4, false, 2>(a, xs, s);
+    case 17: return launch_gemm<128, 256, 2, 4, MODE, 3, true>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
