@@ -57,6 +57,19 @@ def test_packed_size_arithmetic():
     assert cabi.conv_out_hw(g2) == (16, 16)
 
 
+def test_split_k_workspace_arithmetic():
+    # host-only: which problem sizes ask for a split-K workspace, and how much
+    wsb = cabi.lib().tmq_linear_workspace_bytes
+    assert wsb(16, 4096, 11008) == 0 and wsb(64, 4096, 11008) == 0     # weight-streaming rows
+    assert wsb(128, 4096, 4096) == 0                                   # K too short to repay the partial sums
+    assert wsb(4096, 11008, 4096) == 0 and wsb(2048, 4096, 16384) == 0  # grids that fill the chip
+    assert wsb(128, 4096, 11008) == 8 * 128 * 4096 * 4                 # 32 tiles of 128 x 128 -> 8 splits
+    assert wsb(512, 4096, 11008) == 2 * 512 * 4096 * 4                 # 128 tiles -> 2 splits
+    assert wsb(100, 30, 8192) == 8 * 100 * 32 * 4                      # rows of partial sums padded to 16 bytes
+    assert wsb(128, 4096, 8200) == 0                                   # K not a multiple of 16: plain kernel
+    assert wsb(0, 8, 8192) == 0 and wsb(-3, 8, 8192) == 0
+
+
 def test_host_choose_qparams_matches_oracle(golden):
     for mn, mx in cases.dynamic_qparams_cases():
         for rr in (False, True):
