@@ -76,8 +76,9 @@ def _tile_case(m, n, k, seed, x_signed=False, relu=False, bias=True, per_channel
 
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 10, 17])
-@pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192)])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19])
+@pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),
+                                   (270, 300, 400), (40, 70, 784)])
 def test_tile_configs(cabi, cfg, shape):
     say("tile cfg", cfg, shape)
     c = _tile_case(*shape, seed=cfg * 10 + shape[0])
@@ -297,7 +298,7 @@ def test_split_k_workspace_rules(cabi):
 # Float results are compared bit for bit: the kernel's epilogue is the oracle's
 # single fused multiply-add, and the dynamic quantization in front of it is
 # bit-exact by the quantizer tests.
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 10, 17])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19])
 @pytest.mark.parametrize("shape,relu,bias,pc,x_signed", [((60, 264, 448), False, True, True, False),
                                                          ((257, 33, 144), True, True, False, False),
                                                          ((16, 1040, 1168), False, False, True, True)])
@@ -358,7 +359,7 @@ def _random_shapes(seed, count):
     return out
 
 
-@pytest.mark.parametrize("cfg", [-1, 6, 7, 17])
+@pytest.mark.parametrize("cfg", [-1, 6, 7, 17, 19])
 def test_random_shapes_against_oracle(cabi, cfg):
     # ragged everything: rows, channels and k tails in all combinations, for the automatic
     # choice and for the two direct-copy tiles (which fall back below three k stages)

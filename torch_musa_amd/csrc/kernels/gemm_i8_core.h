@@ -362,7 +362,8 @@ __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv,
 // stage waiting on its own chain LDS store -> barrier -> LDS read -> MFMA, and
 // the other groups' waves fill those gaps.  The host sends only k loops whose
 // stage count KW divides.
-template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4, bool WDMA = false, int KW = 1>
+template <int BM, int BN, int WM, int WN, int MODE, class XSRC, int PD = 4, bool WDMA = false, int KW = 1,
+          bool XWIDE = false>
 __global__ __launch_bounds__(WM* WN* KW* kWave, (WDMA && WM * WN == 4 && (BM / WM) * (BN / WN) <= 128 * 64) ? 2 : 1)
 void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int NT = WM * WN * kWave;   // threads of one group
@@ -410,10 +411,13 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
                 "direct copies do not divide among the waves");
   static_assert(!WDMA || (TN + TM <= TN * TM && ND <= TN * TM), "one LDS read and one copy per MFMA at most");
   constexpr int kWBufs = WDMA ? kDmaBufs : 2, kXBufs = WDMA ? kDmaBufs : 2;
+  static_assert(!XWIDE || (WDMA && PD == 3 && KW == 1 && (BM / 8) % (2 * NWAVES) == 0),
+                "wide activation copies: three-stage direct-copy ring only");
 
   // LDS: two stages of {weights, activations}; the same bytes are reused after
   // the main loop to transpose the output tile into row-major order.
-  constexpr int kWStage = kChunks * BN * 16, kXStage = BM * kBK;
+  // (XWIDE: an activation buffer holds two stages, 128 k-bytes of every row)
+  constexpr int kWStage = kChunks * BN * 16, kXStage = XWIDE ? BM * 2 * kBK : BM * kBK;
   constexpr int kOutPitch = BN + 16;  // bytes; keeps rows 16-byte aligned and off one bank
   constexpr int kMainBytes = kWBufs * kWStage + kXBufs * kXStage;
   constexpr int kF32Pitch = BN * 4 + 16;  // float rows of the tile, same idea
@@ -526,7 +530,149 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
                                                                acc[q / TM][q % TM], 0, 0, 0);
   };
 
-  if constexpr (WDMA) {
+  if constexpr (WDMA && XWIDE) {
+    // ---- direct-copy pipeline with activation copies two stages wide.  As the
+    // pipeline below, except that an activation copy moves 8 rows x 128 bytes
+    // (whole 128-byte lines of the row-major activations; the narrow copies
+    // take 16 rows x 64 bytes and touch every line twice, in two successive
+    // stages), into a ring of three buffers of two stages each:
+    //   pair u = stages 2u and 2u+1, buffer u % 3, row pitch 128 bytes, 16-byte
+    //   slot XOR-ed with (row >> 1) & 7 (16 consecutive rows then cover all
+    //   sixteen 16-byte slots of the 256-byte bank window once)
+    // Stage t's second half issues the weight copies of stage t+3 and one half
+    // of the activation copies of pair (t+4)/2: the first half when t is even,
+    // the second when t is odd (the pair then starts at stage t+3).  Everything
+    // a stage reads was issued at least two stages earlier, so the wait of the
+    // narrow pipeline holds unchanged: all but the copies of the last stage.
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t lds0 = lds_address(smem);
+    static_assert(NWAVES % 4 == 0, "weight copies: one k-chunk per wave");
+    constexpr int NDXH = (BM / 8) / NWAVES / 2;  // activation copies per wave per stage (half a pair)
+    static_assert(NDXH == NDX, "as many copies per stage as the narrow pipeline");
+    const uint8_t* const wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
+    const int64_t nb_last = NB - 1 - n0 / 16;  // rows past N: clamped, never stored
+    uint32_t wdma_off[NDW];
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) {
+      const int rg = (wave_u >> 2) + i * (NWAVES / 4);
+      int64_t rb = rg * 4 + (lane >> 4);
+      rb = rb < nb_last ? rb : nb_last;
+      wdma_off[i] = static_cast<uint32_t>((rb * a.w_kchunks + (wave_u & 3)) * 256 + (lane & 15) * 16);
+    }
+    const uint32_t wdma_lds = lds0 + ((wave_u & 3) * BN + (wave_u >> 2) * 64) * 16;
+    // activation copy i (of 2 NDX per pair) of wave w: rows 8 (w + i NWAVES) .. + 7,
+    // eight lanes per row; the lane of slot sl fetches the k-chunk the swizzle puts there
+    const uint8_t* const xtile = xsrc.x + m0 * xsrc.ldx;
+    const int64_t m_last = a.M - 1 - m0;
+    const int pair_last = (KT - 1) >> 1;
+    const int ktail = static_cast<int>(a.K) - 16 - pair_last * 2 * kBK;  // last chunk inside K of the last pair
+    uint32_t xdma_off[2 * NDX], xdma_off_last[2 * NDX];
+#pragma unroll
+    for (int i = 0; i < 2 * NDX; ++i) {
+      const int row = (wave_u + i * NWAVES) * 8 + (lane >> 3);
+      const int64_t r = row < m_last ? row : m_last;
+      const int kc = ((lane & 7) ^ ((row >> 1) & 7)) * 16;
+      xdma_off[i] = static_cast<uint32_t>(r * xsrc.ldx + kc);
+      // chunks past K: any valid bytes will do, the packed weight is zero there
+      xdma_off_last[i] = static_cast<uint32_t>(r * xsrc.ldx + (kc < ktail ? kc : ktail));
+    }
+    const uint32_t xdma_lds = lds0 + kWBufs * kWStage + wave_u * 1024;
+    // weight copies of stage kt into weight buffer wb
+    auto dma_w = [&](int kt, int wb, int i) {
+      lds_dma16(wtile + static_cast<int64_t>(kt) * (kChunks * 256), wdma_off[i],
+                wdma_lds + wb * kWStage + i * (NWAVES / 4) * 64 * 16);
+    };
+    // copy i (0 .. 2 NDX - 1) of activation pair u into activation buffer xb
+    auto dma_x = [&](int u, int xb, int i) {
+      const int uc = u < pair_last ? u : pair_last;
+      lds_dma16(xtile + static_cast<int64_t>(uc) * (2 * kBK), uc == pair_last ? xdma_off_last[i] : xdma_off[i],
+                xdma_lds + xb * kXStage + i * NWAVES * 1024);
+    };
+    auto wait_loads = [&](auto left_tag) {  // s_waitcnt vmcnt(left) only
+      constexpr int kLeft = decltype(left_tag)::value;
+      static_assert(kLeft < 64, "load counter range");
+      __builtin_amdgcn_s_waitcnt((kLeft & 15) | ((kLeft >> 4) << 14) | (7 << 4) | (15 << 8));
+    };
+    auto flip = [&](v4i& f) { f ^= xmask; };
+    const int xswz8 = (li >> 1) & 7;
+    // j-th fragment read of k-step s of a stage in weight buffer wb, activation
+    // buffer xb, half p of its pair
+    auto read_w = [&](int wb, int xb, int p, int s, int j, v4i(&wf)[TN], v4i(&xf)[TM]) {
+      const int c = 2 * s + half;
+      if (j < TN)
+        wf[j] = ld16(&sW[wb * kWStage + (c * BN + wn0 + j * 32 + li) * 16]);
+      else
+        xf[j - TN] = ld16(&sX[xb * kXStage + (wm0 + (j - TN) * 32 + li) * (2 * kBK) + (((4 * p + c) ^ xswz8) << 4)]);
+    };
+    // ph = kt % 6 as a compile-time constant
+    auto stage = [&](int kt, int ph) {
+      const int wb = ph % 3, xb = (ph >> 1) % 3, p = ph & 1;
+      const int phn = (ph + 1) % 6;
+      const int wbn = phn % 3, xbn = (phn >> 1) % 3, pn = phn & 1;
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        if (q < NF) read_w(wb, xb, p, 1, q, wf1, xf1);
+        mfma(q, wf0, xf0);
+        if (q + 1 < TM) flip(xf0[q + 1]);
+        if (q == Q - 1) flip(xf1[0]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // only the copies issued by the stage before this one may still be outstanding
+      wait_loads(std::integral_constant<int, ND>{});
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      const int kload = clampk(kt + 3);
+      const int uload = (kt + 4) >> 1;                 // pair whose copies this stage issues ...
+      const int xbl = ((ph + 4) % 6 >> 1) % 3;         // ... into this buffer,
+      const int ihalf = ((ph + 4) & 1) * NDX;          // this half of them
+      constexpr int kFirstDma = (TM - 1 < Q - 1 - ND) ? TM - 1 : (Q - 1 - ND > 0 ? Q - 1 - ND : 0);
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        if (q < NF) read_w(wbn, xbn, pn, 0, q, wf0, xf0);
+        if (q >= kFirstDma && q - kFirstDma < ND) {
+          const int i = q - kFirstDma;
+          if (i < NDW) dma_w(kload, wb, i);
+          else dma_x(uload, xbl, ihalf + i - NDW);
+        }
+        mfma(q, wf1, xf1);
+        if (q + 1 < TM) flip(xf1[q + 1]);
+        if (q == Q - 1) flip(xf0[0]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // prologue: pair 0 and weights 0 first (they alone are waited for), then
+    // weights 1, the first half of pair 1, and last what stage "-1" would have
+    // issued: weights 2 and the second half of pair 1
+#pragma unroll
+    for (int i = 0; i < 2 * NDX; ++i) dma_x(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) dma_w(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) dma_w(clampk(1), 1, i);
+#pragma unroll
+    for (int i = 0; i < NDX; ++i) dma_x(1, 1, i);
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) dma_w(clampk(2), 2, i);
+#pragma unroll
+    for (int i = 0; i < NDX; ++i) dma_x(1, 1, NDX + i);
+    init_tile();
+    wait_loads(std::integral_constant<int, 2 * NDW + 2 * NDX>{});
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NF; ++j) read_w(0, 0, 0, 0, j, wf0, xf0);
+    flip(xf0[0]);
+    // the host sends only K of at least six stages here
+    int kt0 = 0;
+    do {
+#pragma unroll
+      for (int j = 0; j < 6; ++j) stage(kt0 + j, j);
+      kt0 += 6;
+    } while (kt0 + 6 <= KT);
+#pragma unroll
+    for (int j = 0; j < 5; ++j)
+      if (kt0 + j < KT) stage(kt0 + j, j);
+    wait_loads(std::integral_constant<int, 0>{});
+  } else if constexpr (WDMA) {
     // ---- direct-copy pipeline.  Stage s lives in buffer s % kDmaBufs.  The
     // schedule of stage t, one LDS or copy operation per MFMA:
     //   first half   MFMAs of k-step 0 + LDS reads of the k-step 1 fragments

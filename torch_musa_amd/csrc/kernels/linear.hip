@@ -268,12 +268,12 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
 // Kernel selection override for benchmarking: -1 = automatic.
 std::atomic<int> g_forced_config{-1};
 
-template <int BM, int BN, int WM, int WN, int MODE, int PD = 4, bool WDMA = false, int KW = 1>
+template <int BM, int BN, int WM, int WN, int MODE, int PD = 4, bool WDMA = false, int KW = 1, bool XWIDE = false>
 int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
   if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
   if (KW > 1 && ceil_div(a.K, kBK) % KW != 0) return TMQ_ERR_UNSUPPORTED;  // equal runs of stages only
-  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear, PD, WDMA, KW>
+  gemm_i8_kernel<BM, BN, WM, WN, MODE, XLinear, PD, WDMA, KW, XWIDE>
       <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * KW * kWave), 0, s>>>(a, xs);
   return launch_status();
 }
@@ -308,8 +308,8 @@ SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
   if (splits < 2) return p;
   const int64_t stages = ceil_div(KT, splits);
   splits = ceil_div(KT, stages);
-  // the last split keeps at least three stages (the direct-copy ring's minimum)
-  if (KT - (splits - 1) * stages < 3) --splits;
+  // the last split keeps at least six stages (one turn of the direct-copy ring)
+  if (KT - (splits - 1) * stages < 6) --splits;
   if (splits < 2) return p;
   p.splits = static_cast<int>(splits);
   p.stages = static_cast<int>(stages);
@@ -390,11 +390,11 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs a, const in
   }
 }
 
-template <int BM, int BN, int WM, int WN, int PD = 4, bool WDMA = false>
+template <int BM, int BN, int WM, int WN, int PD = 4, bool WDMA = false, bool XWIDE = false>
 int launch_gemm_split(const GemmArgs& a, const XLinear& xs, const SplitPlan& p, hipStream_t s) {
   const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
   if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-  gemm_i8_kernel<BM, BN, WM, WN, kOutAcc32, XLinear, PD, WDMA>
+  gemm_i8_kernel<BM, BN, WM, WN, kOutAcc32, XLinear, PD, WDMA, 1, XWIDE>
       <<<dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(p.splits)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
   return launch_status();
 }
@@ -411,7 +411,7 @@ int run_split(const GemmArgs& a, const XLinear& xs, const SplitPlan& p, void* wo
   part.splits = p.splits;
   part.split_stages = p.stages;
   part.split_stride = a.M * p.ldp;
-  const int rc = dma_ok ? launch_gemm_split<128, 128, 2, 2, 3, true>(part, xs, p, s)
+  const int rc = dma_ok ? launch_gemm_split<128, 128, 2, 2, 3, true, true>(part, xs, p, s)
                         : launch_gemm_split<128, 128, 2, 2>(part, xs, p, s);
   if (rc != TMQ_OK) return rc;
   // rows per block: enough blocks to hide the loads' latency, then longer runs
@@ -475,18 +475,21 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     const auto rows_used = [&](int bm) { return a.M * 20 >= ceil_div(a.M, bm) * bm * 11; };
     // One block of either large tile runs per CU, so a launch costs whole rounds
     // of 256 tiles.  The 128x256 tile (128 activation rows, 256 channels; 8 waves
-    // of 64x64) does half the work of a 256x256 tile in 0.535 of its time (C3:
-    // 181.5 against 170 us) and wins where it rounds better: M = 2048, N = 11008:
+    // of 64x64) does half the work of a 256x256 tile in 0.56 of its time (C3:
+    // 178.8 against 159.4 us) and wins where it rounds better: M = 2048, N = 11008:
     // 95.4 against 103.3 us; M = 2048, N = 4096: 35.9 against 41.5 us (and 41.3 us
     // for 128x128 tiles).  Its mirror image, 256 rows x 128 channels, is 17 %
     // slower than 256x256 at C3: activation rows arrive as 64-byte pieces of
     // far-apart rows, weight rows as 256-byte pieces of the packed layout.
     const double rounds256 = static_cast<double>(ceil_div(nblk(256, 256), 256));
-    const double rounds128x256 = 0.535 * static_cast<double>(ceil_div(nblk(128, 256), 256));
+    const double rounds128x256 = 0.56 * static_cast<double>(ceil_div(nblk(128, 256), 256));
+    // (its activation copies two stages wide pay within one round of tiles only: M = 512, N = 11008:
+    // 36.3 -> 32.7 us, but M = 1024, N = 11008: 53.0 -> 57.7 us)
+    const int cfg128x256 = nblk(128, 256) <= 256 ? 19 : 17;
     if (nblk(256, 256) >= 160 && rows_used(256))
-      cfg = rounds128x256 < rounds256 ? 17 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
+      cfg = rounds128x256 < rounds256 ? cfg128x256 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
     else if (nblk(128, 256) >= 160 && rows_used(128))
-      cfg = 17;
+      cfg = cfg128x256;
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
     else if (nblk(64, 64) <= 256 && ceil_div(a.K, kBK) >= 32 && ceil_div(a.K, kBK) % 2 == 0)
@@ -495,8 +498,12 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     else
       cfg = 2;
   }
-  if ((cfg == 6 || cfg == 10 || cfg == 17) && !dma_ok) cfg = 3;
-  if (cfg == 7 && !dma_ok) cfg = 1;
+  // the wide activation copies walk K in runs of six stages
+  const bool wide_ok = dma_ok && a.K > 5 * kBK;
+  if (cfg == 19 && !wide_ok) cfg = 17;
+  if (cfg == 6 && !wide_ok) cfg = 3;
+  if (cfg == 17 && !dma_ok) cfg = 3;
+  if (cfg == 7 && !wide_ok) cfg = 1;
   switch (cfg) {
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
     case 1: return launch_gemm<128, 128, 2, 2, MODE>(a, xs, s);
@@ -504,11 +511,11 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 3: return launch_gemm<256, 256, 2, 4, MODE, 3>(a, xs, s);
     case 4: return launch_gemm<128, 256, 2, 2, MODE>(a, xs, s);
     case 5: return launch_gemm<256, 128, 2, 2, MODE>(a, xs, s);
-    case 6: return launch_gemm<256, 256, 2, 4, MODE, 3, true>(a, xs, s);
-    case 7: return launch_gemm<128, 128, 2, 2, MODE, 3, true>(a, xs, s);
-    case 10: return launch_gemm<256, 256, 2, 2, MODE, 3, true>(a, xs, s);
+    case 6: return launch_gemm<256, 256, 2, 4, MODE, 3, true, 1, true>(a, xs, s);
+    case 7: return launch_gemm<128, 128, 2, 2, MODE, 3, true, 1, true>(a, xs, s);
     case 14: return launch_gemm<64, 64, 2, 2, MODE, 4, false, 2>(a, xs, s);
     case 17: return launch_gemm<128, 256, 2, 4, MODE, 3, true>(a, xs, s);
+    case 19: return launch_gemm<128, 256, 2, 4, MODE, 3, true, 1, true>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
