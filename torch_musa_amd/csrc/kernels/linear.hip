@@ -467,7 +467,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
-    // the CUs busy, the 128x128 tile (three blocks per CU) down to 128 tiles.
+    // the CUs busy, the 128x128 tile (two blocks per CU) down to 128 tiles.
     const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
     // (and only when the rows fill at least 55 % of the row tiles: a tile's time
     // does not shrink with its padding; M = 100 and 150 against N = 49152 sit on
