@@ -377,15 +377,15 @@ def test_random_shapes_against_oracle(cabi, cfg):
 def test_row_pitch_and_output_pitch(cabi):
     # activations and outputs that are column slices of wider buffers (ldx > K, ldy > N)
     say("pitches")
-    c = _tile_case(300, 264, 320, seed=77)
+    c = _tile_case(300, 264, 448, seed=77)   # seven k stages: the direct-copy kernels take it
     pw = cabi.PackedLinear(dev(c["wq"]))
-    xbig = torch.zeros((300, 320 + 64), dtype=torch.uint8, device="cuda")
-    xbig[:, 16:336] = dev(c["xq"])
+    xbig = torch.zeros((300, 448 + 64), dtype=torch.uint8, device="cuda")
+    xbig[:, 16:464] = dev(c["xq"])
     ybig = torch.full((300, 264 + 40), 7, dtype=torch.uint8, device="cuda")
-    for cfg in (-1, 6, 7, 3):
+    for cfg in (-1, 6, 7, 3, 17, 19):
         cabi.force_linear_config(cfg)
         try:
-            cabi.linear(xbig[:, 16:336], pw, c["x_scale"], c["x_zp"], dev(c["w_scales"].astype(np.float32)),
+            cabi.linear(xbig[:, 16:464], pw, c["x_scale"], c["x_zp"], dev(c["w_scales"].astype(np.float32)),
                         dev(c["bias"]), c["out_scale"], c["out_zp"], out=ybig[:, 8:272])
         finally:
             cabi.force_linear_config(-1)
