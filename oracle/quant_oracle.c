@@ -306,19 +306,32 @@ ORC_API void orc_weight_colsum(const int8_t* w, int64_t N, int64_t K, int32_t* c
 /* One requantisation, fbgemm/OutputProcessing-inl.h:87-127 (scalar branch):
  *   raw   = acc - x_zp * colsum[n]                              (:90-92)
  *   raw_f = (float)raw (+ bias[n] / act_times_w_scale[n])       (:107-118)
+ *           per-channel weight scales: the quotient is rounded, then added;
+ *           one scale for the whole weight (per-tensor): the vector code of
+ *           the CPU op multiplies by the reciprocal and fuses the addition,
+ *           raw_f = fma(bias[n], fl(1 / act_times_w_scale), (float)raw);
+ *           the two agree except on a few values in a million (pinned by the
+ *           op's outputs on cases built where they differ, tests/golden)
  *   ab    = raw_f * C_multiplier[n]                             (:120)
  *   out   = clamp(lrintf(ab) + out_zp, relu ? out_zp : qmin, qmax)  (:121-125)
  * with act_times_w_scale[n] = x_scale_f * w_scale_f[n] and
  * C_multiplier[n] = act_times_w_scale[n] / out_scale_f, all fp32 (qlinear.cpp /
  * qconv.cpp set-up code). `raw` is passed in already corrected by the caller. */
+static inline float add_bias(float raw_f, float bias, float atw, int per_tensor) {
+  if (per_tensor) {
+    volatile float rcp = 1.0f / atw;
+    return fmaf(bias, rcp, raw_f);
+  }
+  volatile float b = bias / atw;
+  volatile float sum = raw_f + b;
+  return sum;
+}
+
 static inline int32_t requant_one(int32_t raw, int has_bias, float bias, float atw,
-                                  float mult, int64_t out_zp, int64_t lo,
+                                  int per_tensor, float mult, int64_t out_zp, int64_t lo,
                                   int64_t hi) {
   volatile float raw_f = (float)raw;
-  if (has_bias) {
-    volatile float b = bias / atw;
-    raw_f = raw_f + b;
-  }
+  if (has_bias) raw_f = add_bias(raw_f, bias, atw, per_tensor);
   volatile float ab = raw_f * mult;
   float r = nearbyintf(ab);
   if (!(r > -2147483648.0f)) return (int32_t)lo;
@@ -347,7 +360,7 @@ ORC_API void orc_requantize(const int32_t* acc, int64_t M, int64_t N,
     for (int64_t m = 0; m < M; ++m) {
       int32_t raw = acc[m * N + n] - (int32_t)x_zp * colsum[n];
       y[m * N + n] = (uint8_t)requant_one(raw, bias != NULL, bias ? bias[n] : 0.f,
-                                          atw, mult, out_zp, lo, qmax);
+                                          atw, n_scales == 1, mult, out_zp, lo, qmax);
     }
   }
 }
@@ -507,10 +520,7 @@ ORC_API void orc_conv2d_fused(const uint8_t* x, int x_signed, const int8_t* w, i
     volatile float mult = atw / os;
     for (int64_t m = 0; m < rows; ++m) {
       volatile float raw_f = (float)acc[m * OC + n];
-      if (bias != NULL) {
-        volatile float b = bias[n] / atw;
-        raw_f = raw_f + b;
-      }
+      if (bias != NULL) raw_f = add_bias(raw_f, bias[n], atw, n_scales == 1);
       volatile float t = raw_f * mult;
       if (accum != NULL) {
         const int32_t qa = accum_signed ? (int32_t)(int8_t)accum[m * OC + n]

@@ -113,6 +113,40 @@ def main():
         g[k + "/out_scale"] = np.float64(c["out_scale"])
         g[k + "/y"] = y.int_repr().numpy()
 
+    # ---- per-tensor weight + bias: rows picked where the two ways of adding the bias
+    # disagree after requantisation (a few outputs in a million), with the CPU op's
+    # answer.  v = float(raw) + fl(bias / atw) is what the op computes for per-channel
+    # weights, v = fma(bias, fl(1 / atw), float(raw)) for per-tensor ones.  The inputs
+    # are stored with the outputs: finding them takes a search over 64 Mi candidates.
+    f32 = np.float32
+    rng = np.random.default_rng(2718)
+    n_, k_, zp_, x_zp_ = 1024, 16, 128, 121
+    xq_all = rng.integers(0, 256, (65536, k_), dtype=np.uint8)
+    wq_ = rng.integers(-127, 128, (n_, k_), dtype=np.int8)
+    bias_ = (rng.standard_normal(n_) * 30).astype(f32)
+    x_scale_, w_scale_, out_scale_ = f32(0.031), f32(0.0027), f32(0.6)
+    raw_ = (xq_all.astype(np.float64) - x_zp_) @ wq_.astype(np.float64).T      # exact in double
+    atw_ = f32(x_scale_ * w_scale_)
+    mult_ = f32(atw_ / out_scale_)
+    v_div = raw_.astype(f32) + (bias_ / atw_).astype(f32)[None, :]
+    v_fma = (bias_.astype(np.float64)[None, :] * np.float64(f32(f32(1) / atw_)) + raw_).astype(f32)
+    q_div = np.rint((v_div * mult_).astype(f32))
+    q_fma = np.rint((v_fma * mult_).astype(f32))
+    inside = (q_fma + zp_ > 0) & (q_fma + zp_ < 255)
+    rows_ = np.unique(np.nonzero((q_div != q_fma) & inside)[0])[:16]
+    assert rows_.size >= 6, rows_.size
+    xq_ = np.ascontiguousarray(xq_all[rows_])
+    wt_ = torch._make_per_tensor_quantized_tensor(torch.from_numpy(wq_), float(w_scale_), 0)
+    xt_ = torch._make_per_tensor_quantized_tensor(torch.from_numpy(xq_), float(x_scale_), x_zp_)
+    y_ = torch.ops.quantized.linear(xt_, torch.ops.quantized.linear_prepack(wt_, torch.from_numpy(bias_)),
+                                    float(out_scale_), zp_)
+    g["ptbias/xq"], g["ptbias/wq"], g["ptbias/bias"] = xq_, wq_, bias_
+    g["ptbias/params"] = np.array([float(x_scale_), x_zp_, float(w_scale_), float(out_scale_), zp_], dtype=np.float64)
+    g["ptbias/y"] = y_.int_repr().numpy()
+    want_div = np.clip(q_div[rows_] + zp_, 0, 255).astype(np.uint8)
+    meta["ptbias_outputs_where_the_division_form_is_wrong"] = int((want_div != g["ptbias/y"]).sum())
+    assert meta["ptbias_outputs_where_the_division_form_is_wrong"] >= 6
+
     # ---- quantized::linear_dynamic (float in, float out) ------------------------
     for c in cases.linear_dynamic_cases():
         w = make_w(c["wq"], c["w_scales"], c["wq"].shape[0])

@@ -75,6 +75,19 @@ def _tile_case(m, n, k, seed, x_signed=False, relu=False, bias=True, per_channel
                 relu=relu)
 
 
+@pytest.mark.parametrize("cfg", [-1, 2, 9])
+def test_per_tensor_weight_bias_form(cabi, golden, cfg):
+    # rows picked where the two ways of adding the bias requantise differently: the
+    # kernels take fma(bias, 1 / atw, raw) for a per-tensor weight, as the CPU op does
+    say("per-tensor bias form", cfg)
+    x_scale, x_zp, w_scale, out_scale, out_zp = golden["ptbias/params"]
+    c = dict(xq=golden["ptbias/xq"], wq=golden["ptbias/wq"], bias=golden["ptbias/bias"], x_scale=float(x_scale),
+             x_zp=int(x_zp), w_scales=np.array([float(w_scale)]), out_scale=float(out_scale), out_zp=int(out_zp),
+             relu=False)
+    y, _, _ = _run(cabi, c, cfg)
+    np.testing.assert_array_equal(y, golden["ptbias/y"])
+
+
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
 @pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19])
 @pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),

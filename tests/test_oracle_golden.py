@@ -186,6 +186,20 @@ def test_linear_dynamic(golden, c):
     np.testing.assert_array_equal(y, golden[k + "/y"])
 
 
+def test_per_tensor_weight_bias_form(golden):
+    """Rows picked where float(raw) + fl(bias / atw) and fma(bias, fl(1 / atw), float(raw))
+    requantise differently: the CPU op takes the second for a per-tensor weight (the
+    oracle follows), the first for per-channel scales."""
+    xq, wq, bias = golden["ptbias/xq"], golden["ptbias/wq"], golden["ptbias/bias"]
+    x_scale, x_zp, w_scale, out_scale, out_zp = golden["ptbias/params"]
+    want = golden["ptbias/y"]
+    y = oracle.linear(xq, x_scale, int(x_zp), wq, np.array([w_scale]), bias, out_scale, int(out_zp))
+    np.testing.assert_array_equal(y, want)
+    # the same weight declared per channel (equal scales) takes the division form: it differs here
+    y_pc = oracle.linear(xq, x_scale, int(x_zp), wq, np.full(wq.shape[0], w_scale), bias, out_scale, int(out_zp))
+    assert np.count_nonzero(y_pc != want) >= 6
+
+
 def test_linear_dynamic_pins_the_activation_rounding(golden):
     """On the case built from values where the two forms disagree, only the fused
     form (one rounding of x * inv + zp) reproduces the CPU op; the form of

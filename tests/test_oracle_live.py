@@ -84,6 +84,34 @@ def test_linear_and_linear_dynamic_512x4096():
                                                        reduce_range=rr).view(np.uint32), f"linear_dynamic rr={rr}")
 
 
+def test_per_tensor_weight_with_bias_2mi():
+    # 2.8 Mi outputs: a handful of them requantise differently under the per-channel form
+    torch.manual_seed(10)
+    M, K, N = 700, 448, 4096
+    x, w, b = torch.randn(M, K) * 2, torch.randn(N, K) * 0.05, torch.randn(N) * 3
+    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+    wq = torch.quantize_per_tensor(w, float(w.abs().max() / 127), 0, torch.qint8)
+    out_scale = float((x @ w.t()).std()) / 40
+    y = torch.ops.quantized.linear(xq, torch.ops.quantized.linear_prepack(wq, b), out_scale, 100).int_repr().numpy()
+    args = (xq.int_repr().numpy(), xq.q_scale(), xq.q_zero_point(), wq.int_repr().numpy())
+    _same(y, oracle.linear(*args, np.array([wq.q_scale()]), b.numpy(), out_scale, 100, nthreads=8), "per-tensor + bias")
+    as_pc = oracle.linear(*args, np.full(N, wq.q_scale()), b.numpy(), out_scale, 100, nthreads=8)
+    assert np.count_nonzero(as_pc != y) > 0
+
+
+def test_conv2d_per_tensor_weight_with_bias():
+    torch.manual_seed(202)
+    x, w, b = torch.relu(torch.randn(16, 64, 28, 28)), torch.randn(96, 64, 3, 3) * 0.05, torch.randn(96) * 3
+    xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False).contiguous(memory_format=torch.channels_last)
+    wq = torch.quantize_per_tensor(w, float(w.abs().max() / 127), 0, torch.qint8)
+    packed = torch.ops.quantized.conv2d_prepack(wq, b, [1, 1], [1, 1], [1, 1], 1)
+    y = torch.ops.quantized.conv2d(xq, packed, 0.05, 100)
+    want = oracle.conv2d(_nhwc(xq), xq.q_scale(), xq.q_zero_point(),
+                         wq.int_repr().permute(0, 2, 3, 1).contiguous().numpy(), np.array([wq.q_scale()]), b.numpy(),
+                         (1, 1), (1, 1), (1, 1), 1, 0.05, 100, nthreads=8)
+    _same(_nhwc(y), want, "conv2d per-tensor + bias")
+
+
 @pytest.mark.parametrize("geom", [(8, 64, 28, 64, 3, 1, 1, 1), (4, 32, 32, 64, 3, 2, 1, 4), (2, 3, 96, 32, 7, 2, 3, 1)])
 def test_conv2d(geom):
     B, C, H, OC, k, s, p, g = geom

@@ -137,7 +137,8 @@ __global__ __launch_bounds__(256) void conv_plain_kernel(ConvShape s, PlainArgs 
     const float atw = a.x_scale * a.w_scales[oc * a.w_scale_stride];
     const float mult = atw / a.out_scale;
     float v = static_cast<float>(acc);
-    if (a.bias != nullptr) v = v + a.bias[oc] / atw;
+    if (a.bias != nullptr)
+      v = __builtin_fmaf(bias_term(a.w_scale_stride == 0, a.bias[oc], atw), bias_mul(a.w_scale_stride == 0, atw), v);
     float ab = v * mult;
     if (a.post.accum != nullptr) {
       const uint8_t b8 = a.post.accum[id];

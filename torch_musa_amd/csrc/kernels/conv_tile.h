@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       if (MODE != kOutAcc32) {
         const float atw = a.x_scale * c_wscale;
         mult = atw / a.out_scale;
-        bdiv = a.bias != nullptr ? c_bias / atw : 0.f;
+        bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, c_bias, atw) : 0.f;
       }
     }
     s_acc0[t] = acc0;
@@ -232,6 +232,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
   constexpr bool vec_ok = VEC;  // the host checked channel counts and the output's alignment
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor)};
+  const float bmul = MODE == kOutAcc32 ? 1.0f : bias_mul(a.w_scale_stride == 0, a.x_scale * a.w_scales[0]);
 
   auto run = [&](auto tm_tag, int mt0) {
     constexpr int TM = decltype(tm_tag)::value;
@@ -361,9 +362,9 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
               for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * gq + j];
               uint32_t q4;
               if constexpr (KIND == 0)
-                q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw[tm][tn * 4 + gq], a.zp_f, a.lo_f, a.hi_f);
+                q4 = requant4_post<MODE>(raw, bdiv, bmul, mult, a.post, accw[tm][tn * 4 + gq], a.zp_f, a.lo_f, a.hi_f);
               else
-                q4 = requant4<MODE, KIND == 1>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+                q4 = requant4<MODE, KIND == 1>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
               *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) = q4;
             }
         }

@@ -269,17 +269,30 @@ struct KCursor<XConv> {
 // Slot swizzle of the activation stage: see the file header.
 __device__ __forceinline__ int x_swizzle(int row) { return (row >> 2) & 3; }
 
+// The bias enters the requantisation as v = fma(bterm, bmul, float(raw)), which
+// covers both forms of PyTorch's CPU ops (fbgemm's output stage):
+//   per-channel weight scales   v = float(raw) + fl(bias / atw)      bterm = fl(bias / atw), bmul = 1
+//   one scale for the weight    v = fma(bias, fl(1 / atw), float(raw))   bterm = bias, bmul = fl(1 / atw)
+// (atw = fl(x_scale * w_scale); a product with 1 is exact, so the first line is
+// a plain addition.)  The two differ on a few outputs in a million.
+__host__ __device__ __forceinline__ float bias_term(bool per_tensor, float bias, float atw) {
+  return per_tensor ? bias : bias / atw;
+}
+__host__ __device__ __forceinline__ float bias_mul(bool per_tensor, float atw) {
+  return per_tensor ? 1.0f / atw : 1.0f;
+}
+
 // One requantised byte group: four consecutive channels of one output row.
 // CLAMP = false (unsigned output, bounds 0 and 255 only): the packing
 // conversion v_cvt_pk_u8_f32 already saturates to [0, 255], no separate clamp.
 template <int MODE, bool CLAMP = true>
-__device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, v4f mult, float zp_f,
+__device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, float bmul, v4f mult, float zp_f,
                                              float lo_f, float hi_f) {
   uint32_t packed = 0;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     float v = static_cast<float>(raw[j]);  // int -> fp32, round to nearest even
-    v = v + bdiv[j];
+    v = __builtin_fmaf(bdiv[j], bmul, v);
     const float ab = v * mult[j];
     float r = __builtin_rintf(ab) + zp_f;
     if constexpr (CLAMP || MODE != kOutU8) r = __builtin_amdgcn_fmed3f(r, lo_f, hi_f);
@@ -306,14 +319,14 @@ __device__ __forceinline__ uint32_t load_accum4(const PostOps& p, int64_t off, i
 
 // requant4 with the post operations (see PostOps) before the rounding.
 template <int MODE>
-__device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv, v4f mult,
+__device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv, float bmul, v4f mult,
                                                   const PostOps& p, uint32_t accw, float zp_f,
                                                   float lo_f, float hi_f) {
   uint32_t packed = 0;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     float v = static_cast<float>(raw[j]);
-    v = v + bdiv[j];
+    v = __builtin_fmaf(bdiv[j], bmul, v);
     float t = v * mult[j];
     if (p.accum != nullptr) {
       const uint32_t b = (accw >> (8 * j)) & 0xffu;
@@ -482,7 +495,7 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
         } else if (MODE != kOutAcc32) {
           const float atw = xq.scale * a.w_scales[np * a.w_scale_stride];
           mult = atw / a.out_scale;
-          bdiv = a.bias != nullptr ? a.bias[np] / atw : 0.f;
+          bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, a.bias[np], atw) : 0.f;
         }
       }
       s_acc0[i] = acc0;
@@ -997,6 +1010,7 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
     // Requantise in registers, transpose through LDS, then write whole rows:
     // 16 bytes per lane, consecutive lanes on consecutive addresses.
     __syncthreads();  // every wave is done with the operand stages
+    const float bmul = bias_mul(a.w_scale_stride == 0, x_quant(a).scale * a.w_scales[0]);
     auto requant_tile = [&](auto clamp_tag) {
       constexpr bool CL = decltype(clamp_tag)::value;
 #pragma unroll
@@ -1018,9 +1032,9 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
             const int nvalid = (m < a.M && left > 0) ? (left < 4 ? static_cast<int>(left) : 4) : 0;
             const uint32_t accw =
                 (a.post.accum != nullptr && nvalid > 0) ? load_accum4(a.post, m * a.ldy + a.n_off + n, nvalid) : 0u;
-            q4 = requant4_post<MODE>(raw, bdiv, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
+            q4 = requant4_post<MODE>(raw, bdiv, bmul, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
           } else {
-            q4 = requant4<MODE, CL>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+            q4 = requant4<MODE, CL>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
           }
           *reinterpret_cast<uint32_t*>(&smem[(wm0 + tm * 32 + li) * kOutPitch + nl]) = q4;
         }

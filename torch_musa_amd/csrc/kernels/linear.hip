@@ -159,6 +159,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
     for (int r = 0; r < 4; ++r) s_part[wave][mg][(4 * lc + r) * 16 + lr] = acc[mg][r];
   // requantisation constants, before the barrier: off the block's critical path
   v4f bdiv = {0.f, 0.f, 0.f, 0.f}, mult = {0.f, 0.f, 0.f, 0.f};
+  float bmul = 1.f;
   int acc0[4] = {0, 0, 0, 0};
   if (t < 64) {
     const XQuant xq = x_quant(a);
@@ -171,7 +172,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
       } else if (MODE != kOutAcc32) {
         const float atw = xq.scale * c_ws[j];
         mult[j] = atw / a.out_scale;
-        bdiv[j] = a.bias != nullptr ? c_b[j] / atw : 0.f;
+        bdiv[j] = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, c_b[j], atw) : 0.f;
+        bmul = bias_mul(a.w_scale_stride == 0, atw);  // (per tensor: the same for every j)
       }
     }
   }
@@ -200,7 +202,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
       } else if (MODE == kOutF32) {
         store_f32x4(a, m, n, raw, mult, bdiv);
       } else {
-        const uint32_t packed = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+        const uint32_t packed = requant4<MODE>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
         uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
         if (n + 3 < a.N && (a.ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 3) == 0) {
           *reinterpret_cast<uint32_t*>(dst) = packed;
@@ -236,6 +238,7 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
     }
   }
   v4f bdiv, mult;
+  float bmul = 1.f;
   const XQuant xq = x_quant(a);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -248,7 +251,8 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
     } else if (MODE != kOutAcc32) {
       const float atw = xq.scale * a.w_scales[np * a.w_scale_stride];
       mult[j] = atw / a.out_scale;
-      bdiv[j] = a.bias != nullptr ? a.bias[np] / atw : 0.f;
+      bdiv[j] = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, a.bias[np], atw) : 0.f;
+      bmul = bias_mul(a.w_scale_stride == 0, atw);
     }
   }
   if (MODE == kOutAcc32) {
@@ -258,7 +262,7 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
   } else if (MODE == kOutF32) {
     store_f32x4(a, m, n, raw, mult, bdiv);
   } else {
-    const uint32_t packed = requant4<MODE>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+    const uint32_t packed = requant4<MODE>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
     uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
     for (int j = 0; j < 4; ++j)
       if (n + j < a.N) dst[j] = static_cast<uint8_t>(packed >> (8 * j));
@@ -346,7 +350,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs a, const in
         bdiv = a.bias != nullptr ? a.bias[nj] : 0.f;
       } else {
         mult = atw / a.out_scale;
-        bdiv = a.bias != nullptr ? a.bias[nj] / atw : 0.f;
+        bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, a.bias[nj], atw) : 0.f;
       }
     }
     s_add[t] = xq.coef * a.colsum[nj];
@@ -361,6 +365,8 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs a, const in
   const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[q * 4]);
   const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[q * 4]);
   const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
+  const float bmul = (MODE == kOutU8 || MODE == kOutS8)
+                         ? bias_mul(a.w_scale_stride == 0, x_quant(a).scale * a.w_scales[0]) : 1.0f;
   const int64_t mbeg = static_cast<int64_t>(blockIdx.y) * rows;
   const int64_t mend = mbeg + rows < a.M ? mbeg + rows : a.M;
   for (int64_t m = mbeg + (t >> 6); m < mend; m += 4) {
@@ -377,8 +383,8 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs a, const in
     } else if constexpr (MODE == kOutF32) {
       store_f32x4(a, m, n, raw, mult, bdiv);
     } else {
-      const uint32_t q4 = plain_u8 ? requant4<MODE, false>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f)
-                                   : requant4<MODE, true>(raw, bdiv, mult, a.zp_f, a.lo_f, a.hi_f);
+      const uint32_t q4 = plain_u8 ? requant4<MODE, false>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f)
+                                   : requant4<MODE, true>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
       uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
       if (n + 3 < a.N && (reinterpret_cast<uintptr_t>(dst) & 3) == 0) {
         *reinterpret_cast<uint32_t*>(dst) = q4;
