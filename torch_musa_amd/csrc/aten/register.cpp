@@ -734,7 +734,9 @@ at::Tensor qunary_impl(const at::Tensor& self, int kind, double out_scale, int64
 at::Tensor qgelu_run(const at::Tensor& self, c10::string_view approximate) {
   const std::string a(approximate.data(), approximate.size());
   TORCH_CHECK(a == "none" || a == "tanh", "gelu: approximate must be 'none' or 'tanh', got ", a);
-  return qunary_impl(self, a == "tanh" ? 1 : 0, self.q_scale(), self.q_zero_point(), "gelu");
+  // the CPU kernel carries the scale as a float and gives it to the output that way
+  return qunary_impl(self, a == "tanh" ? 1 : 0, static_cast<double>(static_cast<float>(self.q_scale())),
+                     self.q_zero_point(), "gelu");
 }
 at::Tensor qsigmoid_run(const at::Tensor& self) {
   const bool sgn = self.scalar_type() == c10::kQInt8;
