@@ -265,20 +265,39 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = init;
     }
 
-    // The residual bytes this lane will add (4 consecutive channels per word)
-    // are requested now; they arrive while the k loop runs.
+    // The residual bytes of the row tile are requested now and arrive while the
+    // k loop runs.  Aligned case: whole pixels, 16 bytes per lane in the order of
+    // the output stores (4 lanes per pixel, 16 pixels per pass: 16 cache lines per
+    // instruction instead of the 32 that per-lane words of 32 pixels touch, 2
+    // instructions instead of 8), turned into this lane's words (4 consecutive
+    // channels each) through the staging rows before the requantisation.
+    // Otherwise: the words themselves, byte by byte.
     uint32_t accw[TM][8];
+    v4i accv[TM][2];
+    const bool res_rows = KIND == 0 && VEC && a.post.accum != nullptr && n0 + kCtBN <= a.OCg &&
+                          ((reinterpret_cast<uintptr_t>(a.post.accum) | static_cast<uintptr_t>(a.OC)) & 15) == 0;
     if (KIND == 0 && a.post.accum != nullptr) {
+      if (res_rows) {
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
+        for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int nl = (u >> 2) * 32 + 8 * (u & 3) + 4 * half;
-          const int left = a.OCg - (n0 + nl);
-          const int nvalid = (opix[tm] >= 0 && left > 0) ? (left < 4 ? left : 4) : 0;
-          accw[tm][u] = nvalid > 0 ? load_accum4(a.post, static_cast<int64_t>(opix[tm]) * a.OC + ch0 + nl, nvalid)
-                                   : 0u;
-        }
+          for (int pass = 0; pass < 2; ++pass) {
+            const int op = __shfl(opix[tm], pass * 16 + (lane >> 2), kWave);
+            accv[tm][pass] = op >= 0 ? ld16(a.post.accum + static_cast<int64_t>(op) * a.OC + ch0 + (lane & 3) * 16)
+                                     : v4i{0, 0, 0, 0};
+          }
+      } else {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int nl = (u >> 2) * 32 + 8 * (u & 3) + 4 * half;
+            const int left = a.OCg - (n0 + nl);
+            const int nvalid = (opix[tm] >= 0 && left > 0) ? (left < 4 ? left : 4) : 0;
+            accw[tm][u] = nvalid > 0 ? load_accum4(a.post, static_cast<int64_t>(opix[tm]) * a.OC + ch0 + nl, nvalid)
+                                     : 0u;
+          }
+      }
     }
 
     // Fragments of successive k-steps; the two halves of the wave take the two
@@ -349,6 +368,16 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       uint8_t* y = static_cast<uint8_t*>(a.y);
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
+        if (KIND == 0 && res_rows) {  // residual pixels -> this lane's words, through the staging rows
+#pragma unroll
+          for (int pass = 0; pass < 2; ++pass)
+            *reinterpret_cast<v4i*>(sT + (pass * 16 + (lane >> 2)) * kCtTPitch + (lane & 3) * 16) = accv[tm][pass];
+          wave_sync_lds();
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            accw[tm][u] = *reinterpret_cast<const uint32_t*>(sT + li * kCtTPitch + (u >> 2) * 32 + 8 * (u & 3) + 4 * half);
+          wave_sync_lds();  // the words are read before the results overwrite the rows
+        }
         {
 #pragma unroll
           for (int tn = 0; tn < 2; ++tn)
