@@ -408,3 +408,26 @@ def test_row_pitch_and_output_pitch(cabi):
         _check(got[:, 8:272], want, f"cfg {cfg}")
         assert (got[:, :8] == 7).all() and (got[:, 272:] == 7).all()   # nothing written outside the slice
         ybig.fill_(7)
+
+
+def test_row_pitch_beyond_the_direct_copy_range(cabi):
+    # activation rows 8 MiB + 64 B apart: past the 32-bit lane offsets of the direct-copy
+    # kernels, the register-staged kernels take over; same bytes
+    say("huge pitch")
+    c = _tile_case(300, 264, 448, seed=78)
+    pitch = (1 << 23) + 64
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    xbig = torch.zeros(300 * pitch, dtype=torch.uint8, device="cuda")
+    xv = xbig.as_strided((300, 448), (pitch, 1))
+    xv.copy_(dev(c["xq"]))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"])
+    for cfg in (-1, 6, 7, 17):
+        cabi.force_linear_config(cfg)
+        try:
+            y = cabi.linear(xv, pw, c["x_scale"], c["x_zp"], dev(c["w_scales"].astype(np.float32)), dev(c["bias"]),
+                            c["out_scale"], c["out_zp"])
+        finally:
+            cabi.force_linear_config(-1)
+        _check(host(y), want, f"cfg {cfg}")
+    del xbig
