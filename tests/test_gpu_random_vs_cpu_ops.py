@@ -67,7 +67,7 @@ def test_linear_ops(seed):
     assert done >= 25
 
 
-@pytest.mark.parametrize("seed", [1, 2])
+@pytest.mark.parametrize("seed", [1, 2, 3])
 def test_conv_and_glue_ops(seed):
     rng = np.random.default_rng(100 + seed)
     done = 0
@@ -78,10 +78,11 @@ def test_conv_and_glue_ops(seed):
         IC, OC = g * int(rng.choice([16, 32, 64, 128])), g * int(rng.choice([8, 16, 64, 96]))
         k, s = int(rng.choice([1, 3, 3, 5])), int(rng.choice([1, 1, 2]))
         p = int(rng.choice([0, k // 2]))
+        d = int(rng.choice([1, 1, 1, 2]))
         pc, relu, bias = (bool(rng.integers(2)) for _ in range(3))
-        if H + 2 * p < k or W + 2 * p < k:
+        if H + 2 * p < d * (k - 1) + 1 or W + 2 * p < d * (k - 1) + 1:
             continue
-        say("random conv", seed, it, (B, H, W, IC, OC, k, s, p, g), pc, relu, bias)
+        say("random conv", seed, it, (B, H, W, IC, OC, k, s, p, d, g), pc, relu, bias)
         torch.manual_seed(5000 * seed + it)
         x, w = torch.relu(torch.randn(B, IC, H, W)) * 1.5, torch.randn(OC, IC // g, k, k) * 0.05
         b = torch.randn(OC) * 2 if bias else None
@@ -91,14 +92,14 @@ def test_conv_and_glue_ops(seed):
             wq = torch.quantize_per_channel(w, sc, torch.zeros(OC, dtype=torch.int64), 0, torch.qint8)
         else:
             wq = torch.quantize_per_tensor(w, float(w.abs().max() / 127), 0, torch.qint8)
-        geom = ([s, s], [p, p], [1, 1], g)
+        geom = ([s, s], [p, p], [d, d], g)
         cpu_packed = torch.ops.quantized.conv2d_prepack(wq, b, *geom)
         gpu_packed = torch.ops.quantized.conv2d_prepack(wq.cuda(), None if b is None else b.cuda(), *geom)
-        out_scale = max(float(torch.nn.functional.conv2d(x, w, b, s, p, 1, g).std()) / 40, 1e-3)
+        out_scale = max(float(torch.nn.functional.conv2d(x, w, b, s, p, d, g).std()) / 40, 1e-3)
         op = torch.ops.quantized.conv2d_relu if relu else torch.ops.quantized.conv2d
         zp = 0 if relu else 110
         ref, got = op(xq, cpu_packed, out_scale, zp), op(xq.cuda(), gpu_packed, out_scale, zp)
-        what = f"conv {(B, H, W, IC, OC, k, s, p, g)} pc={pc} relu={relu} bias={bias}"
+        what = f"conv {(B, H, W, IC, OC, k, s, p, d, g)} pc={pc} relu={relu} bias={bias}"
         _same_q(got, ref, what)
         ref2 = torch.ops.quantized.add(ref, ref, out_scale * 1.7, 100)
         got2 = torch.ops.quantized.add(got, got, out_scale * 1.7, 100)
