@@ -334,8 +334,10 @@ def main():
                 "algorithmic_bytes_per_launch": nbytes}
 
         # ----------------------------- dynamically quantized linear, decode-sized
-        # fp32 [M, 4096] -> fp32 [M, 4096]: one launch for range + parameters + codes,
-        # one for the product; 40 cold weights replayed in one HIP graph as above
+        # fp32 [M, 4096] -> fp32 [M, 4096]: up to 16384 input values one launch (every block
+        # of the weight-streaming kernel quantizes the input itself), else one launch for
+        # range + parameters + codes and one for the product; 40 cold weights replayed in
+        # one HIP graph as above
         for Md in (1, 16):
             xdf = torch.randn(Md, Kd, device=dev)
 
@@ -359,7 +361,9 @@ def main():
             per = sum(ts) / len(ts) / sets
             nbytes = Nd * Kd + 2 * 4 * Md * Kd + 2 * Md * Kd + 4 * Md * Nd + 12 * Nd
             gbs = nbytes / (per * 1e-3) / 1e9
-            log(f"[bench] dynamic decode M={Md}: {per*1e3:.2f} us per call (2 launches) in a replayed graph")
+            nl = 1 if Md * Kd <= 16384 else 2
+            log(f"[bench] dynamic decode M={Md}: {per*1e3:.2f} us per call ({nl} launch{'es' if nl > 1 else ''}) "
+                "in a replayed graph")
             secondary[f"linear_dynamic_decode_m{Md}"] = {
                 "avg_call_us": round(per * 1e3, 3), "value": round(gbs, 1), "unit": "GB/s",
                 "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

@@ -235,6 +235,16 @@ int tmq_linear_acc32(const tmq_linear_desc* desc, int32_t* acc, int64_t ldacc,
 int tmq_linear_f32(const tmq_linear_desc* desc, const tmq_qparams* x_qparams_dev, float* y,
                    int64_t ldy, tmq_stream_t stream);
 
+/* The whole dynamically quantized linear for a handful of rows in one launch:
+ * fp32 x [M, ldx] -> fp32 y [M, ldy] with M <= 16, M * K <= 16384, K a multiple
+ * of 16, x 16-byte aligned, ldx a multiple of 4 (TMQ_ERR_UNSUPPORTED otherwise:
+ * use tmq_quantize_per_tensor_dynamic_dev + tmq_linear_f32, which give the same
+ * results).  Every block of the weight-streaming kernel derives the activation
+ * range, parameters and codes itself while its weights are on their way.  Uses
+ * M, N, K, w_*, relu, bias of `desc`.  Same reference note as tmq_linear_f32. */
+int tmq_linear_dynamic_small(const tmq_linear_desc* desc, const float* x, int64_t ldx, int reduce_range,
+                             float* y, int64_t ldy, tmq_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * quantized::conv2d weights.
  * Replaces PackedConvWeightMudnn<2>::prepack

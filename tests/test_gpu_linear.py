@@ -344,6 +344,35 @@ def test_linear_dynamic_cases(cabi, golden, c):
                                                            c["reduce_range"]))
 
 
+@pytest.mark.parametrize("shape,relu,bias,pc,rr", [((1, 4096, 4096), False, True, True, False),
+                                                   ((4, 4096, 1000), True, True, False, False),
+                                                   ((16, 1024, 300), False, False, True, True),
+                                                   ((3, 48, 17), False, True, True, False),
+                                                   ((1, 16384, 64), True, True, True, False),
+                                                   ((5, 1040, 130), False, True, False, True)])
+def test_linear_dynamic_one_launch(cabi, shape, relu, bias, pc, rr):
+    # a handful of rows: range, parameters, codes and product inside the weight-streaming
+    # kernel; bit for bit the oracle and the two-launch path
+    say("linear_dynamic one launch", shape, relu, bias, pc, rr)
+    M, K, N = shape
+    rng = np.random.default_rng(M * 7 + K)
+    x = (rng.standard_normal((M, K)) * 1.7 + 0.3).astype(np.float32)
+    wq = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    wsc = ((0.0005 + 0.001 * rng.random(N)) if pc else np.array([0.00093])).astype(np.float32).astype(np.float64)
+    b = rng.standard_normal(N).astype(np.float32) if bias else None
+    pw = cabi.PackedLinear(dev(wq))
+    args = (dev(x), pw, dev(wsc.astype(np.float32)), None if b is None else dev(b))
+    assert cabi.fused_small_dynamic
+    y = host(cabi.linear_dynamic(*args, relu=relu, reduce_range=rr))
+    np.testing.assert_array_equal(y, oracle.linear_dynamic(x, wq, wsc, b, relu=relu, reduce_range=rr))
+    cabi.fused_small_dynamic = False
+    try:
+        y2 = host(cabi.linear_dynamic(*args, relu=relu, reduce_range=rr))
+    finally:
+        cabi.fused_small_dynamic = True
+    np.testing.assert_array_equal(y2, y)
+
+
 def test_linear_dynamic_prefill_sized(cabi):
     # [2048, 1024] x [4096, 1024]^T through the large-tile kernel, against the oracle
     say("linear_dynamic prefill")

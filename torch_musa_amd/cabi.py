@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_acc32", "tmq_linear_f32", "tmq_quantize_per_tensor_dynamic_dev",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
@@ -122,6 +122,7 @@ def lib() -> C.CDLL:
         l.tmq_linear.argtypes = [C.POINTER(LinearDesc), v]
         l.tmq_linear_acc32.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, v]
         l.tmq_linear_f32.argtypes = [C.POINTER(LinearDesc), v, v, C.c_int64, v]
+        l.tmq_linear_dynamic_small.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, C.c_int, v, C.c_int64, v]
         l.tmq_quantize_per_tensor_dynamic_dev.argtypes = [v, v, C.c_int64, C.c_int, C.c_int, C.c_int, v, v, C.c_size_t, v]
         l.tmq_conv2d_prepack.argtypes = [v, C.POINTER(Conv2dGeom), v, v, v]
         l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
@@ -301,6 +302,8 @@ class PackedLinear:
 
 # False: never hand a workspace to the linear entry points (single-launch kernels only)
 use_linear_workspace = True
+# False: linear_dynamic always takes the two-launch path (quantize, then multiply)
+fused_small_dynamic = True
 # a preallocated uint8 tensor that every call on its device shares instead (calls
 # on one stream run in order, so one buffer serves them all); None: per call
 linear_workspace = None
@@ -373,6 +376,18 @@ def linear_dynamic(x, pw: PackedLinear, w_scales, bias, relu=False, reduce_range
     """min/max -> qparams -> quantize -> product, all on the device, no host round trip."""
     assert x.dtype == torch.float32 and x.is_contiguous()
     x2 = x.reshape(-1, x.shape[-1])
+    m, k = x2.shape
+    if fused_small_dynamic and 0 < m <= 16 and m * k <= 16384 and k % 16 == 0 and x2.data_ptr() % 16 == 0:
+        # a handful of rows: range, parameters, codes and product in one launch
+        y = torch.empty((m, pw.N), dtype=torch.float32, device=x.device)
+        assert k == pw.K and w_scales.dtype == torch.float32
+        d = LinearDesc()
+        d.M, d.K, d.N = m, k, pw.N
+        d.w_packed, d.w_colsum, d.w_scales = pw.packed.data_ptr(), pw.colsum.data_ptr(), w_scales.data_ptr()
+        d.w_per_channel, d.relu, d.bias = int(w_scales.numel() > 1), int(relu), _ptr(bias)
+        check(lib().tmq_linear_dynamic_small(C.byref(d), x2.data_ptr(), x2.stride(0), int(reduce_range),
+                                             y.data_ptr(), y.stride(0), stream_ptr()), "tmq_linear_dynamic_small")
+        return y.reshape(tuple(x.shape[:-1]) + (pw.N,))
     xq, qp = quantize_per_tensor_dynamic_dev(x2, False, reduce_range, fused=True)
     y = linear_f32(xq, pw, 1.0, 0, w_scales, bias, relu, qparams_dev=qp)
     return y.reshape(tuple(x.shape[:-1]) + (pw.N,))

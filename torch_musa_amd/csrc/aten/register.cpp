@@ -374,6 +374,22 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     TORCH_CHECK(x.numel() > 0, "quantized::linear_dynamic: empty input features");
     const auto stream = current_stream(x);
     const auto bytes = x.options().dtype(at::kByte);
+    if (M <= 16 && M * K_ <= 16384 && K_ % 16 == 0 && reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0) {
+      // a handful of rows: range, parameters, codes and product in one launch
+      tmq_linear_desc d{};
+      d.M = M;
+      d.N = N_;
+      d.K = K_;
+      d.w_packed = packed_.const_data_ptr();
+      d.w_colsum = cptr<int32_t>(colsum_);
+      d.w_scales = cptr<float>(wp_.scales_f32);
+      d.w_per_channel = wp_.per_channel;
+      d.relu = relu;
+      d.bias = bias_.has_value() ? cptr<float>(*bias_) : nullptr;
+      check_status(tmq_linear_dynamic_small(&d, cptr<float>(x), K_, reduce_range, mptr<float>(y), N_, stream),
+                   "tmq_linear_dynamic_small");
+      return y;
+    }
     at::Tensor ws = at::empty({static_cast<int64_t>(tmq_minmax_workspace_bytes(x.numel()))}, bytes);
     at::Tensor qp = at::empty({static_cast<int64_t>(sizeof(tmq_qparams))}, bytes);
     at::Tensor xq = at::empty({x.numel()}, bytes);

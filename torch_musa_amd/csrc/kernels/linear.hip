@@ -4,6 +4,7 @@
 #include <atomic>
 
 #include "gemm_i8_core.h"
+#include "qparams.h"
 
 // Layout that non-C++ bindings rely on (natural alignment, x86-64).
 static_assert(sizeof(tmq_linear_desc) == 144, "tmq_linear_desc layout changed");
@@ -213,6 +214,180 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(Gemm
         }
       }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Dynamically quantized linear for a handful of rows (M <= 16, M * K <= 16384),
+// float in, float out, one launch.  The weight-streaming kernel above with the
+// activation quantization inside: every block requests its weights, then reads
+// the whole float input (at most 64 KB, from L2), reduces min / max, derives the
+// parameters (ChooseQuantizationParams, one thread), quantizes the values it
+// holds into LDS -- product and zero point rounded once, as PyTorch's CPU
+// quantized::linear_dynamic does while packing -- and multiplies from there.
+// Every block repeats the same few microseconds of work on the input, under the
+// latency of its own weight stream, instead of waiting for a launch that does
+// it once.  Same arithmetic, same results as the two launches.
+// ---------------------------------------------------------------------------
+constexpr int64_t kDynSmallMaxValues = 16384;
+// kHeld: float4 groups of the input per thread, M * K / 4 <= kHeld * 512 (a template
+// parameter: the loads are unconditional so that the load counter stays exact).
+template <int kHeld>
+__global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_dynamic_kernel(
+    GemmArgs a, const float* __restrict__ x, int64_t ldxf, int reduce_range) {
+  constexpr int kWaves = kDecodeWaves;
+  constexpr int kBatch = 8;
+  static_assert(kHeld * 4 * kWaves * kWave <= kDynSmallMaxValues, "held values");
+  extern __shared__ __attribute__((aligned(16))) uint8_t sx[];  // [M][K + 16] activation codes
+  __shared__ int s_part[kWaves][16 * 16];
+  __shared__ float s_mn[kWaves], s_mx[kWaves];
+  __shared__ float s_scale, s_inv, s_zp;
+  const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
+  const int lr = lane & 15, lc = lane >> 4;
+  const int64_t nb = blockIdx.x;
+  const int64_t KB = ceil_div(a.K, 64);
+  const int pitch = static_cast<int>(a.K) + 16;  // rows 16 bytes apart in the banks
+  const uint8_t* wp = a.w_packed + nb * a.w_kchunks * 256 + lc * 256 + lr * 16;
+  // per-channel constants of the 64 finishing threads, requested first
+  const int fm = t >> 2, fg = t & 3;
+  int c_cs[4] = {0, 0, 0, 0};
+  float c_ws[4] = {1.f, 1.f, 1.f, 1.f}, c_b[4] = {0.f, 0.f, 0.f, 0.f};
+  if (t < 64) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t n = nb * 16 + 4 * fg + j;
+      const int64_t np = n < a.N ? n : 0;
+      c_cs[j] = a.colsum[np];
+      c_ws[j] = a.w_scales[np * a.w_scale_stride];
+      if (a.bias != nullptr) c_b[j] = a.bias[np];
+    }
+  }
+  // ---- the input: requested first (loads return in order: behind the weight
+  // stream it would arrive only after it), held in registers between the range
+  // pass and the quantization
+  const int k4 = static_cast<int>(a.K / 4);
+  const int total4 = static_cast<int>(a.M) * k4;
+  v4f held[kHeld];
+#pragma unroll
+  for (int u = 0; u < kHeld; ++u) {
+    const int e = t + u * (kWaves * kWave);
+    const int ec = e < total4 ? e : 0;  // unconditional loads keep the load counter exact
+    const int row = ec / k4, c4 = ec - row * k4;
+    held[u] = *reinterpret_cast<const v4f*>(x + row * ldxf + c4 * 4);
+  }
+  // then the first batch of weights: on its way while the input is processed
+  v4i wf[kBatch];
+#pragma unroll
+  for (int u = 0; u < kBatch; ++u) {
+    const int64_t kb = wave + u * kWaves;
+    const int64_t kbc = kb < KB ? kb : KB - 1;
+    wf[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + kbc * 1024));
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+#pragma unroll
+  for (int u = 0; u < kHeld; ++u) {
+    const int e = t + u * (kWaves * kWave);
+    if (e < total4) {
+      const v4f v = held[u];
+      mn = fminf(fminf(mn, v.x), fminf(v.y, fminf(v.z, v.w)));
+      mx = fmaxf(fmaxf(mx, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
+    }
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, off, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+  }
+  if (lane == 0) {
+    s_mn[wave] = mn;
+    s_mx[wave] = mx;
+  }
+  __syncthreads();
+  if (t == 0) {
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      mn = fminf(mn, s_mn[w]);
+      mx = fmaxf(mx, s_mx[w]);
+    }
+    double sc;
+    int32_t zp;
+    choose_qparams(mn, mx, 0, 255, reduce_range != 0, &sc, &zp);
+    const float scf = static_cast<float>(sc);
+    s_scale = scf;
+    s_inv = 1.0f / scf;  // IEEE division, as the separate quantize kernels
+    s_zp = static_cast<float>(zp);
+  }
+  __syncthreads();
+  const float inv = s_inv, zp_f = s_zp;
+#pragma unroll
+  for (int u = 0; u < kHeld; ++u) {
+    const int e = t + u * (kWaves * kWave);
+    if (e < total4) {
+      const int row = e / k4, c4 = e - row * k4;
+      const v4f v = held[u];
+      uint32_t q = 0;
+      const float f[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float r = __builtin_rintf(__builtin_fmaf(f[j], inv, zp_f));
+        r = fminf(fmaxf(r, 0.f), 255.f);
+        q |= static_cast<uint32_t>(static_cast<int>(r)) << (8 * j);
+      }
+      *reinterpret_cast<uint32_t*>(sx + row * pitch + c4 * 4) = q;
+    }
+  }
+  __syncthreads();
+  // ---- the product, activation operands from LDS (rows past M are zero)
+  const v4i xmask = {static_cast<int>(0x80808080u), static_cast<int>(0x80808080u), static_cast<int>(0x80808080u),
+                     static_cast<int>(0x80808080u)};
+  const bool xrow = lr < a.M;
+  const uint8_t* xp = sx + (xrow ? lr : 0) * pitch + lc * 16;
+  v4i acc = {0, 0, 0, 0};
+  for (int64_t kb0 = wave; kb0 < KB; kb0 += kWaves * kBatch) {
+    if (kb0 != wave) {
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int64_t kb = kb0 + u * kWaves;
+        wf[u] = kb < KB ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + kb * 1024)) : v4i{0, 0, 0, 0};
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t kb = kb0 + u * kWaves;
+      const bool xok = kb < KB && xrow && (kb * 64 + lc * 16 < a.K);
+      // (weights of a block past K were loaded from a clamped address: the zero
+      // activation operand removes them from the sum, x ^ 0x80 alone would not)
+      const v4i xf = xok ? ld16(xp + kb * 64) ^ xmask : v4i{0, 0, 0, 0};
+      const v4i wv = kb < KB ? wf[u] : v4i{0, 0, 0, 0};
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv, xf, acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) s_part[wave][(4 * lc + r) * 16 + lr] = acc[r];
+  v4f mult = {0.f, 0.f, 0.f, 0.f}, bias = {0.f, 0.f, 0.f, 0.f};
+  int acc0[4] = {0, 0, 0, 0};
+  if (t < 64) {
+    const int coef = 128 - static_cast<int>(zp_f);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc0[j] = coef * c_cs[j];
+      mult[j] = s_scale * c_ws[j];
+      bias[j] = c_b[j];
+    }
+  }
+  __syncthreads();
+  if (t < 64 && fm < a.M) {
+    int raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = 4 * fg + j;
+      int s = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) s += s_part[w][i * 16 + fm];
+      raw[j] = s + acc0[j];
+    }
+    store_f32x4(a, fm, nb * 16 + 4 * fg, raw, mult, bias);
   }
 }
 
@@ -665,6 +840,46 @@ TMQ_EXPORT int tmq_linear_f32(const tmq_linear_desc* d, const tmq_qparams* x_qpa
   a.ldy = ldy;
   return dispatch_linear<kOutF32>(a, xs, d->x_signed, vec_ok, as_stream(stream), d->workspace,
                                   d->workspace_bytes);
+}
+
+TMQ_EXPORT int tmq_linear_dynamic_small(const tmq_linear_desc* d, const float* x, int64_t ldx, int reduce_range,
+                                        float* y, int64_t ldy, tmq_stream_t stream) {
+  if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  if (d->M < 0 || d->N < 0 || d->K < 0) return TMQ_ERR_INVALID_ARGUMENT;
+  if (d->M == 0 || d->N == 0) return TMQ_OK;
+  if (d->M > 16 || d->K < 16 || d->K % 16 != 0 || d->M * d->K > kDynSmallMaxValues) return TMQ_ERR_UNSUPPORTED;
+  if (x == nullptr || y == nullptr || d->w_packed == nullptr || d->w_colsum == nullptr || d->w_scales == nullptr)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  if (ldx < d->K || ldy < d->N) return TMQ_ERR_INVALID_ARGUMENT;
+  if (!aligned(x, 16) || ldx % 4 != 0 || !aligned(d->w_packed, 16) || !aligned(y, 4)) return TMQ_ERR_UNSUPPORTED;
+  const int64_t blocks = ceil_div(d->N, 16);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  GemmArgs a{};
+  a.M = d->M;
+  a.N = d->N;
+  a.K = d->K;
+  a.w_packed = static_cast<const uint8_t*>(d->w_packed);
+  a.w_kchunks = packed_kchunks(d->K);
+  a.colsum = d->w_colsum;
+  a.w_scales = d->w_scales;
+  a.w_scale_stride = d->w_per_channel ? 1 : 0;
+  a.bias = d->bias;
+  a.lo_f = d->relu ? 0.f : -__builtin_inff();
+  a.y = y;
+  a.ldy = ldy;
+  const size_t lds = static_cast<size_t>(d->M) * static_cast<size_t>(d->K + 16);
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kDecodeWaves * kWave);
+  hipStream_t s = as_stream(stream);
+  const int64_t groups = ceil_div(d->M * d->K / 4, kDecodeWaves * kWave);  // float4 per thread
+  if (groups <= 1)
+    linear_decode_dynamic_kernel<1><<<grid, block, lds, s>>>(a, x, ldx, reduce_range);
+  else if (groups <= 2)
+    linear_decode_dynamic_kernel<2><<<grid, block, lds, s>>>(a, x, ldx, reduce_range);
+  else if (groups <= 4)
+    linear_decode_dynamic_kernel<4><<<grid, block, lds, s>>>(a, x, ldx, reduce_range);
+  else
+    linear_decode_dynamic_kernel<8><<<grid, block, lds, s>>>(a, x, ldx, reduce_range);
+  return launch_status();
 }
 
 // Benchmark hook (not part of the public header): force a kernel
