@@ -723,12 +723,15 @@ def test_ops_replay_from_a_hip_graph():
     xc = torch.quantize_per_tensor(torch.randn(2, 32, 20, 20, device=dev).relu(), 0.03, 0, torch.quint8).contiguous(
         memory_format=torch.channels_last)
 
+    x1 = torch.randn(2, 8192, device=dev)                           # two rows: the one-launch dynamic linear
+
     def work():
         y1 = torch.ops.quantized.linear(xq, p1, 0.3, 128)
         y2 = torch.ops.quantized.linear_dynamic(xf, p1, False)
+        y5 = torch.ops.quantized.linear_dynamic(x1, p1, False)
         y3 = torch.ops.quantized.conv2d_relu(xc, p2, 0.05, 0)
         y4 = torch.ops.quantized.add(y3, y3, 0.1, 0)
-        return y1, y2, y3, y4
+        return y1, y2, y3, y4, y5
 
     work()
     torch.cuda.synchronize()
@@ -743,6 +746,7 @@ def test_ops_replay_from_a_hip_graph():
     for it in range(3):
         # new contents in the captured input buffers
         xf.copy_(torch.randn(130, 8192, device=dev) * (1.0 + it))
+        x1.copy_(torch.randn(2, 8192, device=dev) * (2.0 + it))
         xq_new = torch.quantize_per_tensor(torch.randn(130, 8192, device=dev) * (1.0 + 0.3 * it), 0.04, 120, torch.quint8)
         xq.copy_(xq_new)
         xc.copy_(torch.quantize_per_tensor(torch.randn(2, 32, 20, 20, device=dev).relu() * (1.0 + it), 0.03, 0,
