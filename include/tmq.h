@@ -3,10 +3,12 @@
  *
  * This is the whole device boundary of the library: raw device pointers, sizes,
  * scalars and a HIP stream go in, a status code comes out.  No operator entry point
- * allocates, frees, synchronises the device or touches global mutable state, so
- * all of them are asynchronous on `stream`, re-entrant, and callable from
- * several host threads on different streams.  Every buffer (inputs, outputs,
- * packed weights, workspaces) is owned by the caller.
+ * allocates, frees, synchronises the device or touches global mutable state
+ * (the library caches per-device constants -- the LDS limit, a kernel attribute
+ * -- the first time a device is used, nothing else), so all of them are
+ * asynchronous on `stream`, re-entrant, and callable from several host threads
+ * on different streams.  Every buffer (inputs, outputs, packed weights,
+ * workspaces) is owned by the caller.
  *
  * Each entry point names the interface of the reference (MooreThreads
  * torch_musa, paths relative to its tree) that it replaces.
@@ -193,7 +195,11 @@ typedef struct tmq_linear_desc {
   float out_scale;
   int32_t out_zero_point;
   int32_t out_signed;      /* 0: quint8 output, 1: qint8 */
-  int32_t reserved;
+  /* 0: the library chooses the kernel (what every caller wants).  k + 1 pins
+   * kernel configuration k of the dispatch table in kernels/linear.hip, so
+   * that tests can put every kernel in front of the oracle at any shape; a
+   * configuration that cannot run the problem gives TMQ_ERR_UNSUPPORTED. */
+  int32_t kernel;
   void* y;                 /* [M,N] bytes, row pitch ldy */
   int64_t ldy;
   /* Optional scratch device memory, owned by the caller like every other
@@ -214,6 +220,10 @@ int tmq_linear(const tmq_linear_desc* desc, tmq_stream_t stream);
  * anyway.  No counterpart in the reference: muDNN allocates its own scratch
  * through the InternalMemAlloc callback (torch_musa/csrc/aten/utils/Utils.cpp:79-153). */
 int64_t tmq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+/* The split behind that figure: *splits runs of *stages k-stages (64 bytes of K
+ * each), the last run taking everything that is left; *splits == 1: no split.
+ * Pure host arithmetic, no GPU call. */
+int tmq_linear_split_plan(int64_t M, int64_t N, int64_t K, int32_t* splits, int32_t* stages);
 
 /* Raw accumulators acc[m][n] = sum_k X[m][k] * W[n][k] as int32 (row pitch
  * ldacc), from the same MFMA main loop, for bit-exactness checks.  Uses
@@ -291,6 +301,13 @@ typedef struct tmq_conv2d_desc {
   int32_t out_signed;
   int32_t relu;
   void* y;
+  /* 0: the library chooses.  Otherwise, for tests of every kernel family at any
+   * shape: 1 halo tiles, 2 implicit GEMM, 3 direct (TMQ_ERR_UNSUPPORTED when the
+   * family cannot run the problem).  tile_rows / tile_cols > 0 pin the halo
+   * kernel's patch height / bound its patch width. */
+  int32_t kernel;
+  int32_t tile_rows, tile_cols;
+  int32_t reserved;
 } tmq_conv2d_desc;
 
 int tmq_conv2d(const tmq_conv2d_desc* desc, tmq_stream_t stream);

@@ -39,7 +39,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(cabi.QParams) == 16
     assert C.sizeof(cabi.LinearDesc) == 144
     assert C.sizeof(cabi.Conv2dGeom) == 14 * 8
-    assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8
+    assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8 + 16
     assert C.sizeof(cabi.Conv2dPost) == 24
 
 
@@ -68,6 +68,36 @@ def test_split_k_workspace_arithmetic():
     assert wsb(100, 30, 8192) == 8 * 100 * 32 * 4                      # rows of partial sums padded to 16 bytes
     assert wsb(128, 4096, 8200) == 0                                   # K not a multiple of 16: plain kernel
     assert wsb(0, 8, 8192) == 0 and wsb(-3, 8, 8192) == 0
+
+
+def test_split_k_plan_covers_k():
+    # The plan is `splits` runs of `stages` k-stages with the last run taking
+    # whatever is left: every run must start inside K, the last one must hold at
+    # least six stages (one turn of the direct-copy ring), and the workspace
+    # figure must follow from the plan.  Shapes include those where a short tail
+    # is merged into the split before it (K = 16640, 13328).
+    wsb = cabi.lib().tmq_linear_workspace_bytes
+    merged = 0
+    shapes = [(128, 1024, 16640), (128, 128, 13328), (100, 520, 8208), (130, 4096, 11008)]
+    rng = np.random.default_rng(7)
+    for _ in range(4000):
+        shapes.append((int(rng.integers(65, 1100)), int(rng.integers(16, 5000)),
+                       16 * int(rng.integers(8192 // 16, 40000 // 16))))
+    for m, n, k in shapes:
+        splits, stages = cabi.linear_split_plan(m, n, k)
+        kt = -(-k // 64)
+        if splits == 1:
+            assert wsb(m, n, k) == 0
+            continue
+        assert splits >= 2 and stages >= 16
+        assert (splits - 1) * stages < kt, (m, n, k, splits, stages)
+        last = kt - (splits - 1) * stages
+        assert last >= 6, (m, n, k, splits, stages)
+        merged += last > stages
+        assert wsb(m, n, k) == splits * m * (-(-n // 4) * 4) * 4
+    assert merged > 0, "no shape exercised the merged tail"
+    assert cabi.linear_split_plan(128, 1024, 16640) == (15, 17)    # 260 stages: 14 x 17 + 22
+    assert cabi.linear_split_plan(128, 128, 13328) == (12, 17)     # 209 stages: 11 x 17 + 22
 
 
 def test_host_choose_qparams_matches_oracle(golden):

@@ -761,3 +761,120 @@ def test_ops_replay_from_a_hip_graph():
                 assert torch.equal(got.int_repr(), want.int_repr()), f"replay {it}"
             else:
                 assert torch.equal(got, want), f"replay {it}"
+
+
+# ---- interface leftovers ------------------------------------------------------------------
+def test_quantize_per_tensor_with_tensor_qparams():
+    # aten::quantize_per_tensor.tensor_qparams (musa_functions.yaml:3527-3531): scale and
+    # zero point arrive as one-element tensors
+    say("aten qpt tensor_qparams")
+    torch.manual_seed(41)
+    x = torch.randn(5, 33, 7)
+    for dtype, zp in ((torch.quint8, 121), (torch.qint8, -4)):
+        scale = torch.tensor(float(x.abs().max()) / 120)
+        zpt = torch.tensor(zp, dtype=torch.int64)
+        want = torch.quantize_per_tensor(x, scale, zpt, dtype)
+        got = torch.quantize_per_tensor(x.cuda(), scale.cuda(), zpt.cuda(), dtype)
+        assert_q_equal(got, want)
+        got_host_params = torch.quantize_per_tensor(x.cuda(), scale, zpt, dtype)
+        assert_q_equal(got_host_params, want)
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("groups,stride,padding,dilation", [(1, 1, 1, 1), (2, 2, 3, 2)])
+def test_qconv1d_matches_cpu_op(relu, groups, stride, padding, dilation):
+    # quantized::conv1d_prepack (mudnn/ConvPrepack.cpp:159-221) and quantized::conv1d{,_relu}
+    say("conv1d", relu, groups, stride, padding, dilation)
+    torch.manual_seed(41)
+    x = torch.randn(3, 32, 50)
+    w = torch.randn(48, 32 // groups, 5) * 0.1
+    b = torch.randn(48)
+    xq = torch.quantize_per_tensor(x, float(x.abs().max()) / 127, 128, torch.quint8)
+    wq = torch.quantize_per_channel(w, w.abs().amax(dim=(1, 2)).double() / 127,
+                                    torch.zeros(48, dtype=torch.int64), 0, torch.qint8)
+    op = torch.ops.quantized.conv1d_relu if relu else torch.ops.quantized.conv1d
+    pc = torch.ops.quantized.conv1d_prepack(wq, b, [stride], [padding], [dilation], groups)
+    want = op(xq, pc, 0.08, 100)
+    pg = torch.ops.quantized.conv1d_prepack(wq.cuda(), b.cuda(), [stride], [padding], [dilation], groups)
+    got = op(xq.cuda(), pg, 0.08, 100)
+    assert got.dim() == 3
+    assert_q_equal(got, want, abs_diff=LSB_TOL)
+    wu, bu = torch.ops.quantized.conv1d_unpack(pg)
+    assert wu.is_cuda and wu.dim() == 3 and torch.equal(wu.int_repr().cpu(), wq.int_repr())
+    assert torch.equal(bu.cpu(), b)
+
+
+def test_qconv2d_prepack_wide_input():
+    # 1x1 weights with 2048 input channels (ResNet-50 layer4): the packed size must not
+    # depend on an image size
+    say("conv prepack 2048 -> 512")
+    torch.manual_seed(2)
+    x = torch.randn(2, 2048, 7, 7)
+    w = torch.randn(512, 2048, 1, 1) * 0.02
+    xq = torch.quantize_per_tensor(x, float(x.abs().max()) / 255, 128, torch.quint8)
+    wq = torch.quantize_per_tensor(w, float(w.abs().max()) / 127, 0, torch.qint8)
+    pc = torch.ops.quantized.conv2d_prepack(wq, None, [1, 1], [0, 0], [1, 1], 1)
+    pg = torch.ops.quantized.conv2d_prepack(wq.cuda(), None, [1, 1], [0, 0], [1, 1], 1)
+    want = torch.ops.quantized.conv2d(xq, pc, 0.05, 128)
+    got = torch.ops.quantized.conv2d(xq.cuda(), pg, 0.05, 128)
+    assert_q_equal(got, want, abs_diff=LSB_TOL)
+
+
+def test_qlinear_without_input_features():
+    # K == 0: the product is empty and every row is the requantised bias
+    say("linear K = 0")
+    b = torch.tensor([0.0, 1.0, -2.0, 300.0])
+    wq = torch.quantize_per_tensor(torch.zeros(4, 0), 0.1, 0, torch.qint8)
+    xq = torch.quantize_per_tensor(torch.zeros(3, 0), 0.1, 128, torch.quint8)
+    pg = torch.ops.quantized.linear_prepack(wq.cuda(), b.cuda())
+    y = torch.ops.quantized.linear(xq.cuda(), pg, 0.5, 10)
+    want = torch.quantize_per_tensor(b, 0.5, 10, torch.quint8).int_repr()
+    assert y.shape == (3, 4) and torch.equal(y.int_repr().cpu(), want.expand(3, 4))
+    yd = torch.ops.quantized.linear_dynamic(torch.zeros(3, 0).cuda(), pg)
+    assert torch.equal(yd.cpu(), b.expand(3, 4))
+    yr = torch.ops.quantized.linear_relu_dynamic(torch.zeros(3, 0).cuda(), pg)
+    assert torch.equal(yr.cpu(), b.clamp_min(0).expand(3, 4))
+
+
+def test_saved_modules_with_gpu_packed_params(tmp_path):
+    """torch.save / torch.load / deepcopy of modules whose packed parameters live on the GPU
+    (the limitation the reference notes at test_quantized_linear.py:56-60,87-89): the
+    pickled state is the unpacked weight, and loading re-packs it where the weight lands."""
+    import copy
+    import torch_musa_amd
+    say("save / load of packed modules")
+    torch.manual_seed(9)
+    lin = nnq.Linear(64, 32)
+    w = torch.randn(32, 64) * 0.1
+    lin.set_weight_bias(torch.quantize_per_channel(w, w.abs().amax(dim=1).double() / 127,
+                                                   torch.zeros(32, dtype=torch.int64), 0, torch.qint8),
+                        torch.randn(32))
+    lin.scale, lin.zero_point = 0.1, 128
+    conv = nniq.ConvReLU2d(16, 8, 3, padding=1)
+    wc = torch.randn(8, 16, 3, 3) * 0.1
+    conv.set_weight_bias(torch.quantize_per_tensor(wc, float(wc.abs().max()) / 127, 0, torch.qint8), torch.randn(8))
+    conv.scale, conv.zero_point = 0.05, 0
+    net = torch.nn.ModuleDict({"lin": lin, "conv": conv})
+    xl = torch.quantize_per_tensor(torch.randn(5, 64), 0.03, 128, torch.quint8)
+    xc = torch.quantize_per_tensor(torch.randn(2, 16, 9, 9), 0.03, 128, torch.quint8)
+    want_l, want_c = net["lin"](xl).int_repr(), net["conv"](xc).int_repr()
+
+    def check(m, what):
+        assert m["lin"]._packed_params._packed_params.unpack()[0].is_cuda, what
+        assert torch.equal(m["lin"](xl.cuda()).int_repr().cpu(), want_l), what
+        assert torch.equal(m["conv"](xc.cuda()).int_repr().cpu(), want_c), what
+
+    torch_musa_amd.quantized_modules_to(net, "cuda")
+    check(net, "moved")
+    check(copy.deepcopy(net), "deepcopy")
+    path = str(tmp_path / "net.pt")
+    torch.save(net, path)                      # a file this test wrote
+    check(torch.load(path, weights_only=False), "loaded onto the GPU")
+    on_cpu = torch.load(path, weights_only=False, map_location="cpu")
+    assert torch.equal(on_cpu["lin"](xl).int_repr(), want_l)
+    check(torch_musa_amd.quantized_modules_to(on_cpu, "cuda"), "loaded on the CPU, then moved")
+    # the state dict alone, into a fresh CPU model, then moved
+    fresh = torch.nn.ModuleDict({"lin": nnq.Linear(64, 32), "conv": nniq.ConvReLU2d(16, 8, 3, padding=1)})
+    torch.save(net.state_dict(), path)
+    fresh.load_state_dict(torch.load(path, map_location="cpu", weights_only=False))
+    check(torch_musa_amd.quantized_modules_to(fresh, "cuda"), "state dict")

@@ -252,6 +252,8 @@ def test_c3_full_size(cabi):
     ((100, 520, 8208), False, False, True, True),     # 8 splits, K ends inside a stage, ragged M and N
     ((300, 300, 8192), True, True, False, False),     # qint8 activations, per-tensor weight scale
     ((130, 4096, 11008), False, True, True, True),    # 64 tiles, 4 splits of 43 stages
+    ((128, 1024, 16640), False, False, True, True),   # 260 stages as 14 x 17 + 22: the tail joins the last split
+    ((128, 128, 13328), True, False, True, False),    # 209 stages as 11 x 17 + 22, K ends inside a stage
 ])
 def test_split_k(cabi, shape, x_signed, relu, bias, pc):
     say("split K", shape, x_signed, relu, bias, pc)

@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
@@ -49,7 +49,7 @@ class LinearDesc(C.Structure):
         ("w_per_channel", C.c_int32), ("relu", C.c_int32),
         ("bias", C.c_void_p),
         ("out_scale", C.c_float), ("out_zero_point", C.c_int32),
-        ("out_signed", C.c_int32), ("reserved", C.c_int32),
+        ("out_signed", C.c_int32), ("kernel", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
     ]
@@ -72,6 +72,7 @@ class Conv2dDesc(C.Structure):
         ("out_scale", C.c_float), ("out_zero_point", C.c_int32),
         ("out_signed", C.c_int32), ("relu", C.c_int32),
         ("y", C.c_void_p),
+        ("kernel", C.c_int32), ("tile_rows", C.c_int32), ("tile_cols", C.c_int32), ("reserved", C.c_int32),
     ]
 
 
@@ -103,6 +104,8 @@ def lib() -> C.CDLL:
         l.tmq_linear_packed_bytes.argtypes = [C.c_int64, C.c_int64]
         l.tmq_linear_workspace_bytes.restype = C.c_int64
         l.tmq_linear_workspace_bytes.argtypes = [C.c_int64, C.c_int64, C.c_int64]
+        l.tmq_linear_split_plan.argtypes = [C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_int32),
+                                            C.POINTER(C.c_int32)]
         l.tmq_conv2d_packed_bytes.restype = C.c_int64
         l.tmq_conv2d_packed_bytes.argtypes = [C.POINTER(Conv2dGeom)]
         v = C.c_void_p
@@ -325,6 +328,7 @@ def _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_si
     d.relu = int(relu)
     d.bias = _ptr(bias)
     d.out_scale, d.out_zero_point, d.out_signed = out_scale, out_zp, int(out_signed)
+    d.kernel = _linear_config + 1
     if y is not None:
         d.y, d.ldy = y.data_ptr(), y.stride(0)
     nbytes = lib().tmq_linear_workspace_bytes(d.M, d.N, d.K) if use_linear_workspace else 0
@@ -417,15 +421,37 @@ def dequantize_per_channel_float_qparams(q, scales, zps, axis):
     return r
 
 
+# Kernel pins of this binding (tests and benchmarks): they travel in the
+# descriptors' `kernel` fields, call by call; the library keeps no such state.
+_linear_config = -1
+_conv_path = -1
+_conv_tile = (0, 0)
+
+
 def force_linear_config(cfg: int) -> None:
-    """Benchmark hook: pin the GEMM tile configuration (-1 = automatic)."""
-    lib().tmq_debug_force_linear_config(C.c_int(cfg))
+    """Pin the GEMM tile configuration of later calls through this binding (-1 = automatic)."""
+    global _linear_config
+    _linear_config = int(cfg)
 
 
 def force_conv_path(path: int) -> None:
-    """Test and benchmark hook: pin the conv2d kernel family
+    """Pin the conv2d kernel family of later calls through this binding
     (-1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct)."""
-    lib().tmq_debug_force_conv_path(C.c_int(path))
+    global _conv_path
+    _conv_path = int(path)
+
+
+def force_conv_tile(rows: int, cols: int) -> None:
+    """Pin the halo kernel's patch height / bound its patch width (0 = automatic)."""
+    global _conv_tile
+    _conv_tile = (int(rows), int(cols))
+
+
+def linear_split_plan(m: int, n: int, k: int):
+    """-> (splits, stages per split) of the split-K schedule for this shape."""
+    sp, st = C.c_int32(), C.c_int32()
+    check(lib().tmq_linear_split_plan(m, n, k, C.byref(sp), C.byref(st)), "tmq_linear_split_plan")
+    return sp.value, st.value
 
 
 # ---------------------------------------------------------------------------
@@ -474,6 +500,8 @@ def _conv_desc(x, pw, g, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_s
     d.bias = _ptr(bias)
     d.out_scale, d.out_zero_point, d.out_signed, d.relu = out_scale, out_zp, int(out_signed), int(relu)
     d.y = _ptr(y)
+    d.kernel = _conv_path if _conv_path > 0 else 0
+    d.tile_rows, d.tile_cols = _conv_tile
     return d
 
 

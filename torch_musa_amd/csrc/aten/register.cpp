@@ -366,12 +366,15 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
                 "quantized::linear_dynamic: input and weight on different devices");
     const c10::OptionalDeviceGuard guard(at::device_of(input));
     const at::Tensor x = input.contiguous();
-    const int64_t M = K_ == 0 ? 0 : x.numel() / K_;
     std::vector<int64_t> out_shape = x.sizes().vec();
     out_shape.back() = N_;
     at::Tensor y = at::empty(out_shape, x.options());
     if (y.numel() == 0) return y;
-    TORCH_CHECK(x.numel() > 0, "quantized::linear_dynamic: empty input features");
+    const int64_t M = y.numel() / N_;
+    if (K_ == 0) {  // no input features: the product is empty, the bias remains (as the CPU op)
+      if (bias_.has_value()) y.copy_(bias_->expand_as(y)); else y.zero_();
+      return relu ? y.clamp_min_(0) : y;
+    }
     const auto stream = current_stream(x);
     const auto bytes = x.options().dtype(at::kByte);
     if (M <= 16 && M * K_ <= 16384 && K_ % 16 == 0 && reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0) {
@@ -430,13 +433,15 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     TORCH_CHECK(output_scale > 0, "quantized::linear: output scale must be positive");
     const c10::OptionalDeviceGuard guard(at::device_of(act));
     const at::Tensor x = act.contiguous();
-    const int64_t M = K_ == 0 ? 0 : x.numel() / K_;
     std::vector<int64_t> out_shape = x.sizes().vec();
     out_shape.back() = N_;
     // output dtype follows the activation dtype: quint8 as PyTorch's CPU op,
     // qint8 as the reference (mudnn/Linear.cpp:99-103)
     at::Tensor y = at::_empty_affine_quantized(out_shape, x.options(), output_scale, output_zero_point);
     if (y.numel() == 0) return y;
+    // rows from the output: with K == 0 the input has no elements, and the
+    // library then writes the requantised bias into every row
+    const int64_t M = y.numel() / N_;
     tmq_linear_desc d{};
     d.M = M;
     d.N = N_;
@@ -540,11 +545,15 @@ struct PackedConvWeightTmq final : public ConvPackedParamsBase<2> {
     const at::Tensor w8 = weight.int_repr().permute({0, 2, 3, 1}).contiguous();
     tmq_conv2d_geom g{};
     g.B = 1;
-    g.H = g.W = 1 << 10;  // weights do not depend on the image; any valid size works here
     g.IC = weight.size(1) * groups;
     g.OC = OC;
     g.KH = weight.size(2);
     g.KW = weight.size(3);
+    // weights do not depend on the image: the smallest one the kernel window
+    // fits (the library bounds H * W * IC, which a large stand-in would hit for
+    // wide layers)
+    g.H = g.KH;
+    g.W = g.KW;
     g.stride_h = g.stride_w = 1;
     g.pad_h = g.pad_w = 0;
     g.dil_h = g.dil_w = 1;
@@ -682,6 +691,40 @@ c10::intrusive_ptr<ConvPackedParamsBase<2>> qconv2d_prepack_run(at::Tensor weigh
                                                                 torch::List<int64_t> dilation, int64_t groups) {
   return PackedConvWeightTmq::prepack(std::move(weight), std::move(bias), std::move(stride),
                                       std::move(padding), std::move(dilation), groups);
+}
+
+// quantized::conv1d_prepack (mudnn/ConvPrepack.cpp:159-216): a 1-D convolution
+// is the 2-D one over a height of 1 -- weight [OC, IC/g, L] -> [OC, IC/g, 1, L],
+// stride / padding / dilation [v] -> [1 or 0, v] -- and shares its packed type.
+torch::List<int64_t> conv1d_arg(const torch::List<int64_t>& arg, int64_t base, const char* what) {
+  TORCH_CHECK(!arg.empty(), "quantized::conv1d_prepack: ", what, " must have elements");
+  return torch::List<int64_t>({base, arg.size() == 1 ? arg.get(0) : arg.get(1)});
+}
+c10::intrusive_ptr<ConvPackedParamsBase<2>> qconv1d_prepack_run(at::Tensor weight, std::optional<at::Tensor> bias,
+                                                                torch::List<int64_t> stride,
+                                                                torch::List<int64_t> padding,
+                                                                torch::List<int64_t> dilation, int64_t groups) {
+  TORCH_CHECK(weight.dim() == 3 || weight.dim() == 4, "quantized::conv1d_prepack: weights are expected to have 3 dimensions");
+  if (weight.dim() == 3) weight = weight.unsqueeze(-2);
+  return PackedConvWeightTmq::prepack(std::move(weight), std::move(bias), conv1d_arg(stride, 1, "stride"),
+                                      conv1d_arg(padding, 0, "padding"), conv1d_arg(dilation, 1, "dilation"),
+                                      groups);
+}
+// quantized::conv1d / conv1d_relu as PyTorch's CPU ops run them: [N, C, L] ->
+// [N, C, 1, L], the 2-D convolution, and back.
+at::Tensor qconv1d_impl(const at::Tensor& act, const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w, double s,
+                        int64_t z, bool relu) {
+  TORCH_CHECK(act.dim() == 3, "quantized::conv1d expects a 3-D (N, C, L) input");
+  const at::Tensor x = act.unsqueeze(2);
+  const at::Tensor y = relu ? w->apply_relu(x, s, z) : w->apply(x, s, z);
+  return y.squeeze(2);
+}
+at::Tensor qconv1d_run(at::Tensor act, const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w, double s, int64_t z) {
+  return qconv1d_impl(act, w, s, z, false);
+}
+at::Tensor qconv1d_relu_run(at::Tensor act, const c10::intrusive_ptr<ConvPackedParamsBase<2>>& w, double s,
+                            int64_t z) {
+  return qconv1d_impl(act, w, s, z, true);
 }
 
 // ---------------------------------------------------------------------------
@@ -1190,6 +1233,9 @@ TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d.new"), TORCH_FN(qconv2d_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_relu.new"), TORCH_FN(qconv2d_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_prepack"), TORCH_FN(qconv2d_prepack_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv1d_prepack"), TORCH_FN(qconv1d_prepack_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv1d"), TORCH_FN(qconv1d_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::conv1d_relu"), TORCH_FN(qconv1d_relu_run));
 }
 
 // float activations arrive under the plain CUDA key

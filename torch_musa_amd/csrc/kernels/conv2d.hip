@@ -13,7 +13,7 @@
 #include "gemm_i8_core.h"
 
 static_assert(sizeof(tmq_conv2d_geom) == 112, "tmq_conv2d_geom layout changed");
-static_assert(sizeof(tmq_conv2d_desc) == 192, "tmq_conv2d_desc layout changed");
+static_assert(sizeof(tmq_conv2d_desc) == 208, "tmq_conv2d_desc layout changed");
 static_assert(sizeof(tmq_conv2d_post) == 24, "tmq_conv2d_post layout changed");
 
 namespace tmq {
@@ -168,25 +168,31 @@ int launch_conv_gemm(const GemmArgs& a, const XConv& xs, hipStream_t s) {
   return launch_status();
 }
 
-std::atomic<int> g_forced_path{-1};
-std::atomic<int> g_forced_rows{0};   // > 0: patch height of the halo-tiled kernel
-std::atomic<int> g_forced_cols{0};   // > 0: upper bound of its patch width  // -1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct
-
 // Patch shape and LDS layout of the halo-tiled kernel for one problem.
 struct TilePlan {
   int TH, TW, HH, HW, pitch, KS;
   int lds_x, lds_t, lds_tab, lds_total;
 };
 
+constexpr int kMaxDevices = 64;
+
+int current_device() {
+  int dev = 0;
+  return hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices ? dev : -1;
+}
+
+// LDS bytes a block may use on the current device (cached per device; two
+// threads that race on the first call store the same value).
 int lds_limit() {
-  static const int limit = [] {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
-      return 0;
-    return v;
-  }();
-  return limit;
+  static std::atomic<int> cache[kMaxDevices];
+  const int dev = current_device();
+  if (dev < 0) return 0;
+  int v = cache[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return 0;
+    cache[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
 }
 
 // Chooses the patch that minimises a time estimate fitted to per-phase cycle
@@ -202,7 +208,7 @@ int lds_limit() {
 // each further one the larger of its SIMD work (half the fixed cost + mfma +
 // epilogue) and its copies; blocks that do not fit run one after the other.  Returns false when
 // the weight slice or the smallest halo do not fit.
-bool plan_tiles(const ConvShape& s, bool forced, TilePlan* best) {
+bool plan_tiles(const ConvShape& s, bool forced, int forced_rows, int forced_cols, TilePlan* best) {
   // A block loads every pixel of its halo, so a kernel smaller than its stride
   // (1x1 stride 2: three of four loaded pixels unused) runs 1.6-3.7x faster as an
   // implicit GEMM, which gathers only what it multiplies.  Everything else that
@@ -228,8 +234,6 @@ bool plan_tiles(const ConvShape& s, bool forced, TilePlan* best) {
       if (widths[i] == w) return;
     widths[nw++] = w;
   };
-  const int forced_cols = g_forced_cols.load(std::memory_order_relaxed);
-  const int forced_rows = g_forced_rows.load(std::memory_order_relaxed);
   if (forced_cols > 0) {
     add_width(s.OW < forced_cols ? s.OW : forced_cols);
   } else {
@@ -280,10 +284,16 @@ bool plan_tiles(const ConvShape& s, bool forced, TilePlan* best) {
 
 template <int MODE, int KIND, bool VEC>
 int launch_conv_tiles_variant(const ConvShape& s, const TilePlan& p, const ConvTileArgs& a, hipStream_t stream) {
-  static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&conv_tile_kernel<MODE, KIND, VEC>),
-      hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit() - 3 * kCtBN * 4);
-  if (attr != hipSuccess) return TMQ_ERR_LAUNCH;
+  // the kernel's LDS allowance is a per-device attribute: set once per device
+  static std::atomic<uint64_t> done{0};
+  const int dev = current_device();
+  if (dev < 0) return TMQ_ERR_LAUNCH;
+  if ((done.load(std::memory_order_acquire) >> dev & 1) == 0) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_tile_kernel<MODE, KIND, VEC>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit() - 3 * kCtBN * 4) != hipSuccess)
+      return TMQ_ERR_LAUNCH;
+    done.fetch_or(uint64_t{1} << dev, std::memory_order_release);
+  }
   const int64_t bx = s.B * a.tiles_h * a.tiles_w, by = static_cast<int64_t>(a.n_tiles) * s.groups;
   if (bx > 0x7fffffff || by > 65535) return TMQ_ERR_UNSUPPORTED;
   conv_tile_kernel<MODE, KIND, VEC><<<dim3(static_cast<unsigned>(bx), static_cast<unsigned>(by)),
@@ -354,7 +364,7 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   const float lo_f = static_cast<float>(relu ? d->out_zero_point : qmin);
   const float hi_f = static_cast<float>(qmax);
 
-  const int forced = g_forced_path.load(std::memory_order_relaxed);
+  const int forced = d->kernel > 0 ? d->kernel : -1;
   const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
   if ((forced == 1 || forced == 2) && !mfma_ok) return TMQ_ERR_UNSUPPORTED;
   if (!mfma_ok || forced == 3) {
@@ -379,7 +389,7 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   }
 
   TilePlan plan;
-  const bool tiles_ok = forced != 2 && plan_tiles(s, forced == 1, &plan);
+  const bool tiles_ok = forced != 2 && plan_tiles(s, forced == 1, d->tile_rows, d->tile_cols, &plan);
   if (forced == 1 && !tiles_ok) return TMQ_ERR_UNSUPPORTED;
   if (tiles_ok) {
     ConvTileArgs t{};
@@ -519,16 +529,6 @@ TMQ_EXPORT int tmq_conv2d_fused(const tmq_conv2d_desc* d, const tmq_conv2d_post*
   if (d == nullptr || post == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
   return d->out_signed ? run_conv<kOutS8>(d, post, d->y, as_stream(stream))
                        : run_conv<kOutU8>(d, post, d->y, as_stream(stream));
-}
-
-// Test and benchmark hook (not part of the public header): force a kernel
-// family.  -1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct.
-TMQ_EXPORT void tmq_debug_force_conv_path(int path) {
-  g_forced_path.store(path, std::memory_order_relaxed);
-}
-TMQ_EXPORT void tmq_debug_force_conv_tile(int rows, int cols) {
-  g_forced_rows.store(rows, std::memory_order_relaxed);
-  g_forced_cols.store(cols, std::memory_order_relaxed);
 }
 
 TMQ_EXPORT int tmq_conv2d_acc32(const tmq_conv2d_desc* d, int32_t* acc, tmq_stream_t stream) {

@@ -97,7 +97,8 @@ struct GemmArgs {
   int32_t acc_base = 0;
   // Split K (raw int32 output of plain activation rows only): block row
   // blockIdx.y multiplies stages [y * split_stages, (y + 1) * split_stages) of
-  // the k loop and writes its partial sums to y + blockIdx.y * split_stride.
+  // the k loop -- the last one everything from y * split_stages on -- and
+  // writes its partial sums to y + blockIdx.y * split_stride.
   int32_t splits = 1;
   int32_t split_stages = 0;
   int64_t split_stride = 0;
@@ -397,8 +398,10 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
     if (a.splits > 1) {  // this block's share of K: move the operands, shorten K
       const int64_t sp = blockIdx.y;
       const int64_t k0 = sp * a.split_stages * kBK;
+      // the last split takes everything that is left (the host may have merged a
+      // short tail into it)
       const int64_t left = a.K - k0, mine = static_cast<int64_t>(a.split_stages) * kBK;
-      a.K = left < mine ? left : mine;
+      a.K = (sp == a.splits - 1 || left < mine) ? left : mine;
       a.w_packed += sp * a.split_stages * (kChunks * 256);
       xsrc.x += k0;
       a.y = static_cast<int32_t*>(a.y) + sp * a.split_stride;

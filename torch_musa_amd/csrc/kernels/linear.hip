@@ -1,8 +1,6 @@
 // quantized::linear for gfx950: weight re-tiling, the MFMA GEMM dispatch, a
 // weight-streaming kernel for decode-sized batches, and a plain kernel for
 // shapes the vector paths do not take (K not a multiple of 16, unaligned rows).
-#include <atomic>
-
 #include "gemm_i8_core.h"
 #include "qparams.h"
 
@@ -444,9 +442,6 @@ __global__ __launch_bounds__(256) void linear_plain_kernel(GemmArgs a, XLinear x
   }
 }
 
-// Kernel selection override for benchmarking: -1 = automatic.
-std::atomic<int> g_forced_config{-1};
-
 template <int BM, int BN, int WM, int WN, int MODE, int PD = 4, bool WDMA = false, int KW = 1, bool XWIDE = false>
 int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
@@ -487,7 +482,9 @@ SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
   if (splits < 2) return p;
   const int64_t stages = ceil_div(KT, splits);
   splits = ceil_div(KT, stages);
-  // the last split keeps at least six stages (one turn of the direct-copy ring)
+  // a last run of fewer than six stages (one turn of the direct-copy ring) is
+  // merged into the split before it: the kernel's last split multiplies
+  // everything from (splits - 1) * stages to the end of K
   if (KT - (splits - 1) * stages < 6) --splits;
   if (splits < 2) return p;
   p.splits = static_cast<int>(splits);
@@ -604,10 +601,10 @@ int run_split(const GemmArgs& a, const XLinear& xs, const SplitPlan& p, void* wo
   return launch_status();
 }
 
+// forced: tmq_linear_desc::kernel - 1 (-1 = automatic choice).
 template <int MODE>
-int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec_ok,
+int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec_ok, int forced,
                     hipStream_t s, void* workspace = nullptr, int64_t workspace_bytes = 0) {
-  const int forced = g_forced_config.load(std::memory_order_relaxed);
   if (!vec_ok || forced == 9) {
     // plain kernel accumulates true activation values: undo the +128 share
     GemmArgs b = a;
@@ -776,7 +773,19 @@ TMQ_EXPORT int64_t tmq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return split_workspace_bytes(plan_split(M, N, K), M);
 }
 
-TMQ_EXPORT int tmq_linear(const tmq_linear_desc* d, tmq_stream_t stream) {
+TMQ_EXPORT int tmq_linear_split_plan(int64_t M, int64_t N, int64_t K, int32_t* splits, int32_t* stages) {
+  if (M < 0 || N < 0 || K < 0 || splits == nullptr || stages == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  const SplitPlan p = (M > 0 && N > 0 && K > 0) ? plan_split(M, N, K) : SplitPlan{};
+  *splits = p.splits;
+  *stages = p.stages;
+  return TMQ_OK;
+}
+
+namespace tmq {
+namespace {
+
+// quantized::linear with the split-K scratch passed beside the descriptor.
+int linear_u8s8(const tmq_linear_desc* d, void* workspace, int64_t workspace_bytes, tmq_stream_t stream) {
   GemmArgs a{};
   XLinear xs{};
   bool vec_ok = false;
@@ -798,8 +807,17 @@ TMQ_EXPORT int tmq_linear(const tmq_linear_desc* d, tmq_stream_t stream) {
   a.y = d->y;
   a.ldy = d->ldy;
   hipStream_t s = as_stream(stream);
-  return d->out_signed ? dispatch_linear<kOutS8>(a, xs, d->x_signed, vec_ok, s, d->workspace, d->workspace_bytes)
-                       : dispatch_linear<kOutU8>(a, xs, d->x_signed, vec_ok, s, d->workspace, d->workspace_bytes);
+  return d->out_signed
+             ? dispatch_linear<kOutS8>(a, xs, d->x_signed, vec_ok, d->kernel - 1, s, workspace, workspace_bytes)
+             : dispatch_linear<kOutU8>(a, xs, d->x_signed, vec_ok, d->kernel - 1, s, workspace, workspace_bytes);
+}
+
+}  // namespace
+}  // namespace tmq
+
+TMQ_EXPORT int tmq_linear(const tmq_linear_desc* d, tmq_stream_t stream) {
+  if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  return linear_u8s8(d, d->workspace, d->workspace_bytes, stream);
 }
 
 TMQ_EXPORT int tmq_linear_acc32(const tmq_linear_desc* d, int32_t* acc, int64_t ldacc,
@@ -813,7 +831,7 @@ TMQ_EXPORT int tmq_linear_acc32(const tmq_linear_desc* d, int32_t* acc, int64_t 
   a.acc_coef = d->x_signed ? 0 : 128;  // undo the x ^ 0x80 shift only
   a.y = acc;
   a.ldy = ldacc;
-  return dispatch_linear<kOutAcc32>(a, xs, d->x_signed, vec_ok, as_stream(stream), d->workspace,
+  return dispatch_linear<kOutAcc32>(a, xs, d->x_signed, vec_ok, d->kernel - 1, as_stream(stream), d->workspace,
                                     d->workspace_bytes);
 }
 
@@ -838,7 +856,7 @@ TMQ_EXPORT int tmq_linear_f32(const tmq_linear_desc* d, const tmq_qparams* x_qpa
   a.lo_f = d->relu ? 0.f : -__builtin_inff();
   a.y = y;
   a.ldy = ldy;
-  return dispatch_linear<kOutF32>(a, xs, d->x_signed, vec_ok, as_stream(stream), d->workspace,
+  return dispatch_linear<kOutF32>(a, xs, d->x_signed, vec_ok, d->kernel - 1, as_stream(stream), d->workspace,
                                   d->workspace_bytes);
 }
 
@@ -880,10 +898,4 @@ TMQ_EXPORT int tmq_linear_dynamic_small(const tmq_linear_desc* d, const float* x
   else
     linear_decode_dynamic_kernel<8><<<grid, block, lds, s>>>(a, x, ldx, reduce_range);
   return launch_status();
-}
-
-// Benchmark hook (not part of the public header): force a kernel
-// configuration, -1 restores automatic selection.
-TMQ_EXPORT void tmq_debug_force_linear_config(int cfg) {
-  g_forced_config.store(cfg, std::memory_order_relaxed);
 }
