@@ -225,6 +225,25 @@ int64_t tmq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * Pure host arithmetic, no GPU call. */
 int tmq_linear_split_plan(int64_t M, int64_t N, int64_t K, int32_t* splits, int32_t* stages);
 
+/* tmq_linear for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments and the same bytes as
+ * tmq_linear called with a workspace of tmq_linear_workspace_bytes(M, N, K);
+ * desc->workspace / workspace_bytes are ignored: the split-K partial sums go to
+ * a fixed array of TMQ_LINEAR_STATIC_WORKSPACE_BYTES in the library's own device
+ * memory (one per GPU the library has run on, held until the process ends).
+ * The call allocates and frees nothing.  A problem whose split needs more than
+ * the array holds returns TMQ_ERR_WORKSPACE (the present split plan never asks
+ * for more than 256 tiles of 128 x 128 int32 sums = the array's size).  Calls
+ * on one GPU share that GPU's array: calls that may run at the same time
+ * (different streams, different host threads) race on it and must be ordered
+ * by the caller; calls queued on one stream are safe.  The partial sums are
+ * written before they are read, so nothing has to be cleared between calls.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress):
+ * make one call per device before capturing a graph. */
+#define TMQ_LINEAR_STATIC_WORKSPACE_BYTES (16 * 1024 * 1024)
+int tmq_linear_static_workspace(const tmq_linear_desc* desc, tmq_stream_t stream);
+
 /* Raw accumulators acc[m][n] = sum_k X[m][k] * W[n][k] as int32 (row pitch
  * ldacc), from the same MFMA main loop, for bit-exactness checks.  Uses
  * M, N, K, x, ldx, x_signed, w_packed, w_colsum of `desc`. */

@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_static_workspace", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
@@ -123,6 +123,7 @@ def lib() -> C.CDLL:
         l.tmq_linear_prepack.argtypes = [v, C.c_int64, C.c_int64, C.c_int64, v, v, v]
         l.tmq_linear_unpack.argtypes = [v, C.c_int64, C.c_int64, v, C.c_int64, v]
         l.tmq_linear.argtypes = [C.POINTER(LinearDesc), v]
+        l.tmq_linear_static_workspace.argtypes = [C.POINTER(LinearDesc), v]
         l.tmq_linear_acc32.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, v]
         l.tmq_linear_f32.argtypes = [C.POINTER(LinearDesc), v, v, C.c_int64, v]
         l.tmq_linear_dynamic_small.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, C.c_int, v, C.c_int64, v]
@@ -354,6 +355,25 @@ def linear(x, pw: PackedLinear, x_scale, x_zp, w_scales, bias, out_scale, out_zp
         (x.shape[0], pw.N), dtype=torch.int8 if out_signed else torch.uint8, device=x.device)
     d = _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed, relu, y)
     check(lib().tmq_linear(C.byref(d), stream_ptr()), "tmq_linear")
+    return y
+
+
+def linear_static_workspace(x, pw: PackedLinear, x_scale, x_zp, w_scales, bias, out_scale, out_zp,
+                            out_signed=None, relu=False, out=None):
+    """tmq_linear_static_workspace: as linear(), the split-K scratch inside the library.
+    `out` given: the call allocates nothing at all."""
+    assert x.dim() == 2 and x.stride(1) == 1
+    if out_signed is None:
+        out_signed = x.dtype == torch.int8
+    y = out if out is not None else torch.empty(
+        (x.shape[0], pw.N), dtype=torch.int8 if out_signed else torch.uint8, device=x.device)
+    global use_linear_workspace
+    keep, use_linear_workspace = use_linear_workspace, False   # no workspace tensor in the descriptor
+    try:
+        d = _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_signed, relu, y)
+    finally:
+        use_linear_workspace = keep
+    check(lib().tmq_linear_static_workspace(C.byref(d), stream_ptr()), "tmq_linear_static_workspace")
     return y
 
 

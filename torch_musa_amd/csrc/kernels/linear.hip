@@ -1,6 +1,8 @@
 // quantized::linear for gfx950: weight re-tiling, the MFMA GEMM dispatch, a
 // weight-streaming kernel for decode-sized batches, and a plain kernel for
 // shapes the vector paths do not take (K not a multiple of 16, unaligned rows).
+#include <atomic>
+
 #include "gemm_i8_core.h"
 #include "qparams.h"
 
@@ -818,6 +820,53 @@ int linear_u8s8(const tmq_linear_desc* d, void* workspace, int64_t workspace_byt
 TMQ_EXPORT int tmq_linear(const tmq_linear_desc* d, tmq_stream_t stream) {
   if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
   return linear_u8s8(d, d->workspace, d->workspace_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------
+// quantized::linear for callers that cannot allocate: the split-K partial sums
+// go to a fixed array in the library's own device memory.
+// ---------------------------------------------------------------------------
+namespace tmq {
+namespace {
+
+// Every split plan fits: splits x tiles <= 256 blocks of 128 x 128 int32 sums.
+constexpr int64_t kStaticWorkspaceBytes = int64_t{16} << 20;
+static_assert(kStaticWorkspaceBytes == TMQ_LINEAR_STATIC_WORKSPACE_BYTES, "header and library disagree");
+static __device__ __align__(256) uint8_t scratch[kStaticWorkspaceBytes];
+
+constexpr int kMaxDevices = 64;
+// Device address of `scratch` on every device used so far.  The array's name
+// is a host-side handle in host code; each device holds its own copy of the
+// array at its own address, which hipGetSymbolAddress reports for the current
+// device.  Two threads that race on a device's first call store the same value.
+std::atomic<void*> g_scratch_addr[kMaxDevices];
+
+int static_workspace(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TMQ_ERR_LAUNCH;
+  void* p = g_scratch_addr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return TMQ_ERR_LAUNCH;
+    g_scratch_addr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return TMQ_OK;
+}
+
+}  // namespace
+}  // namespace tmq
+
+TMQ_EXPORT int tmq_linear_static_workspace(const tmq_linear_desc* d, tmq_stream_t stream) {
+  if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  if (d->M < 0 || d->N < 0 || d->K < 0) return TMQ_ERR_INVALID_ARGUMENT;
+  const int64_t need = (d->M > 0 && d->N > 0 && d->K > 0) ? split_workspace_bytes(plan_split(d->M, d->N, d->K), d->M) : 0;
+  if (need > kStaticWorkspaceBytes) return TMQ_ERR_WORKSPACE;  // the caller's own workspace and tmq_linear then
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = static_workspace(&ws);
+    if (rc != TMQ_OK) return rc;
+  }
+  return linear_u8s8(d, ws, need, stream);
 }
 
 TMQ_EXPORT int tmq_linear_acc32(const tmq_linear_desc* d, int32_t* acc, int64_t ldacc,
