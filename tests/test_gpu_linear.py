@@ -89,7 +89,7 @@ def test_per_tensor_weight_bias_form(cabi, golden, cfg):
 
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20])
 @pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),
                                    (270, 300, 400), (40, 70, 784)])
 def test_tile_configs(cabi, cfg, shape):
@@ -100,6 +100,30 @@ def test_tile_configs(cabi, cfg, shape):
     want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
                          c["out_scale"], c["out_zp"], relu=c["relu"])
     _check(y, want, f"cfg {cfg}")
+
+
+# the persistent kernel over more tiles than the chip has CUs: every block walks two tiles
+# (ragged last row and column tiles, K that ends inside a stage and inside a pair of stages)
+@pytest.mark.parametrize("shape,x_signed,relu,pc", [((4389, 4120, 448), False, False, True),
+                                                     ((4100, 4352, 400), True, True, False),
+                                                     ((8200, 2100, 656), False, True, True)])
+def test_persistent_rounds(cabi, shape, x_signed, relu, pc):
+    say("persistent rounds", shape, x_signed, relu, pc)
+    M, N, K = shape
+    assert -(-M // 256) * -(-N // 256) > 256
+    c = _tile_case(M, N, K, seed=77 + K, x_signed=x_signed, relu=relu, per_channel=pc)
+    pw = cabi.PackedLinear(dev(c["wq"]))
+    ws, b = dev(c["w_scales"].astype(np.float32)), dev(c["bias"])
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=relu, nthreads=8)
+    for cfg in (20, -1, 6):   # pinned, the automatic choice (the same kernel), and one tile per block
+        cabi.force_linear_config(cfg)
+        try:
+            y = host(cabi.linear(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, c["out_scale"], c["out_zp"],
+                                 out_signed=x_signed, relu=relu))
+        finally:
+            cabi.force_linear_config(-1)
+        _check(y, want, f"cfg {cfg}")
 
 
 # wave groups that split the k loop inside a block (stage counts the group count divides)

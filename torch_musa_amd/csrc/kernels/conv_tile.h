@@ -72,14 +72,6 @@ __device__ __forceinline__ uint32_t small_div(uint32_t n, uint32_t d, float rcp)
   return q;
 }
 
-__device__ __forceinline__ void wave_sync_lds() {
-  // orders this wave's LDS writes before its later LDS reads of other lanes'
-  // data (the LDS executes one wave's instructions in order)
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 // KIND selects the requantisation compiled in: 0 residual / SiLU, 1 plain with
 // clamp, 2 plain for unsigned output without ReLU (the saturating pack
 // conversion is the clamp).  VEC: output rows take aligned 16-byte (int32 mode:

@@ -157,6 +157,14 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)p)));
 }
 
+__device__ __forceinline__ void wave_sync_lds() {
+  // orders this wave's LDS writes before its later LDS reads of other lanes'
+  // data (the LDS executes one wave's instructions in order)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <class XSRC>
 struct XLoader;
 

@@ -4,6 +4,7 @@
 #include <atomic>
 
 #include "gemm_i8_core.h"
+#include "gemm_i8_persistent.h"
 #include "qparams.h"
 
 // Layout that non-C++ bindings rely on (natural alignment, x86-64).
@@ -454,6 +455,40 @@ int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   return launch_status();
 }
 
+constexpr int kMaxDevices = 64;
+
+// Compute units of the current device (cached per device; two threads that race
+// on a device's first call store the same value).
+int cu_count() {
+  static std::atomic<int> cache[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int v = cache[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cache[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
+// One block per CU walks the 256 x 256 tiles (byte outputs, direct copies two
+// stages wide: the caller checked their address and K ranges).
+template <int MODE>
+int launch_gemm_persistent(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  if constexpr (MODE == kOutU8 || MODE == kOutS8) {
+    const int64_t tiles = ceil_div(a.M, 256) * ceil_div(a.N, 256);
+    const int cus = cu_count();
+    if (cus < 8 || tiles > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    // several rounds: a multiple of 8 blocks, so that the tile sequence deals
+    // every XCD its own run of tiles
+    const int64_t grid = tiles <= cus ? tiles : cus / 8 * 8;
+    gemm_i8_persistent_kernel<MODE><<<dim3(static_cast<unsigned>(grid)), dim3(kPersistThreads), 0, s>>>(a, xs);
+    return launch_status();
+  } else {
+    return TMQ_ERR_UNSUPPORTED;
+  }
+}
+
 // ---- split K for a few hundred rows against a long K.  The tile grid of such a
 // product is far smaller than the chip (M = 128, N = 4096: 32 tiles of
 // 128 x 128) and every block walks all of K alone at the latency of one stage
@@ -681,6 +716,13 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   // the wide activation copies walk K in runs of six stages
   const bool wide_ok = dma_ok && a.K > 5 * kBK;
   if (cfg == 19 && !wide_ok) cfg = 17;
+  // more than one round of 256 x 256 tiles with byte outputs: the persistent
+  // kernel hides each tile's pipeline fill behind the tile before it
+  if (forced < 0 && cfg == 6 && wide_ok && (MODE == kOutU8 || MODE == kOutS8) &&
+      ceil_div(a.M, 256) * ceil_div(a.N, 256) > 256)
+    cfg = 20;
+  if (cfg == 20 && MODE != kOutU8 && MODE != kOutS8) cfg = 6;  // float and raw outputs: one tile per block
+  if (cfg == 20 && !wide_ok) cfg = 3;
   if (cfg == 6 && !wide_ok) cfg = 3;
   if (cfg == 17 && !dma_ok) cfg = 3;
   if (cfg == 7 && !wide_ok) cfg = 1;
@@ -696,6 +738,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 14: return launch_gemm<64, 64, 2, 2, MODE, 4, false, 2>(a, xs, s);
     case 17: return launch_gemm<128, 256, 2, 4, MODE, 3, true>(a, xs, s);
     case 19: return launch_gemm<128, 256, 2, 4, MODE, 3, true, 1, true>(a, xs, s);
+    case 20: return launch_gemm_persistent<MODE>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
@@ -834,7 +877,6 @@ constexpr int64_t kStaticWorkspaceBytes = int64_t{16} << 20;
 static_assert(kStaticWorkspaceBytes == TMQ_LINEAR_STATIC_WORKSPACE_BYTES, "header and library disagree");
 static __device__ __align__(256) uint8_t scratch[kStaticWorkspaceBytes];
 
-constexpr int kMaxDevices = 64;
 // Device address of `scratch` on every device used so far.  The array's name
 // is a host-side handle in host code; each device holds its own copy of the
 // array at its own address, which hipGetSymbolAddress reports for the current
