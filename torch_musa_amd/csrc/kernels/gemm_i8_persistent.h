@@ -66,9 +66,12 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t lds0 = lds_address(smem);
 
-  const int64_t tiles_m = ceil_div(a.M, BM), tiles_n = ceil_div(a.N, BN);
-  const int64_t nblocks = tiles_m * tiles_n;
-  const int64_t NB = ceil_div(a.N, 16);
+  // (the host keeps the tile count below 2**31 and every per-lane operand offset
+  // below 2**32: 32-bit index arithmetic throughout, 64-bit divisions would cost
+  // a block two microseconds per tile)
+  const uint32_t tiles_m = static_cast<uint32_t>(ceil_div(a.M, BM)), tiles_n = static_cast<uint32_t>(ceil_div(a.N, BN));
+  const uint32_t nblocks = tiles_m * tiles_n;
+  const int NB = static_cast<int>(ceil_div(a.N, 16));
   const int KT = static_cast<int>(ceil_div(a.K, kBK));
   const int pair_last = (KT - 1) >> 1;
   const int ktail = static_cast<int>(a.K) - 16 - pair_last * 2 * kBK;  // last chunk inside K of the last pair
@@ -77,17 +80,18 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   // ---- tile sequence: virtual block v = round * gridDim.x + blockIdx.x takes
   // the tile the one-tile-per-block kernel gives block v (every XCD owns one
   // contiguous run of the sequence, ordered in patches four channel tiles wide)
-  auto tile_origin = [&](int64_t v, int64_t* m0, int64_t* n0) {
-    const int64_t q = nblocks / 8, rem = nblocks % 8;
-    const int64_t xcd = v % 8, within = v / 8;
-    const int64_t tile = xcd * q + (xcd < rem ? xcd : rem) + within;
-    constexpr int64_t kGroupN = 4;
-    const int64_t group = tile / (tiles_m * kGroupN);
-    const int64_t gfirst = group * kGroupN;
-    const int64_t gwidth = tiles_n - gfirst < kGroupN ? tiles_n - gfirst : kGroupN;
-    const int64_t in_group = tile - group * (tiles_m * kGroupN);
-    *m0 = (in_group / gwidth) * BM;
-    *n0 = (gfirst + in_group % gwidth) * BN;
+  auto tile_origin = [&](uint32_t v, int* m0, int* n0) {
+    const uint32_t q = nblocks / 8, rem = nblocks % 8;
+    const uint32_t xcd = v % 8, within = v / 8;
+    const uint32_t tile = xcd * q + (xcd < rem ? xcd : rem) + within;
+    constexpr uint32_t kGroupN = 4;
+    const uint32_t group = tile / (tiles_m * kGroupN);
+    const uint32_t gfirst = group * kGroupN;
+    const uint32_t gwidth = tiles_n - gfirst < kGroupN ? tiles_n - gfirst : kGroupN;
+    const uint32_t in_group = tile - group * (tiles_m * kGroupN);
+    const uint32_t row = in_group / gwidth;
+    *m0 = static_cast<int>(row * BM);
+    *n0 = static_cast<int>((gfirst + in_group - row * gwidth) * BN);
   };
   // (a permutation of the tiles as long as the grid is a multiple of 8 or holds
   // every tile in one round, which the host guarantees)
@@ -98,26 +102,27 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   uint32_t wdma_off[NDW], xdma_off[2 * NDX], xdma_off_last[2 * NDX];
   const uint32_t wdma_lds = lds0 + ((wave_u & 3) * BN + (wave_u >> 2) * 64) * 16;
   const uint32_t xdma_lds = lds0 + 3 * kWStage + wave_u * 1024;
-  auto tile_setup = [&](int64_t m0, int64_t n0) {
-    wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
-    const int64_t nb_last = NB - 1 - n0 / 16;  // rows past N: clamped, never stored
+  const uint32_t kch = static_cast<uint32_t>(a.w_kchunks), ldx = static_cast<uint32_t>(xsrc.ldx);
+  auto tile_setup = [&](int m0, int n0) {
+    wtile = a.w_packed + static_cast<int64_t>(n0 / 16) * a.w_kchunks * 256;
+    const int nb_last = NB - 1 - n0 / 16;  // rows past N: clamped, never stored
 #pragma unroll
     for (int i = 0; i < NDW; ++i) {
       const int rg = (wave_u >> 2) + i * (NWAVES / 4);
-      int64_t rb = rg * 4 + (lane >> 4);
+      int rb = rg * 4 + (lane >> 4);
       rb = rb < nb_last ? rb : nb_last;
-      wdma_off[i] = static_cast<uint32_t>((rb * a.w_kchunks + (wave_u & 3)) * 256 + (lane & 15) * 16);
+      wdma_off[i] = (static_cast<uint32_t>(rb) * kch + static_cast<uint32_t>(wave_u & 3)) * 256u + (lane & 15) * 16;
     }
-    xtile = xsrc.x + m0 * xsrc.ldx;
-    const int64_t m_last = a.M - 1 - m0;
+    xtile = xsrc.x + static_cast<int64_t>(m0) * xsrc.ldx;
+    const int m_last = static_cast<int>(a.M) - 1 - m0;
 #pragma unroll
     for (int i = 0; i < 2 * NDX; ++i) {
       const int row = (wave_u + i * NWAVES) * 8 + (lane >> 3);
-      const int64_t r = row < m_last ? row : m_last;
+      const uint32_t r = static_cast<uint32_t>(row < m_last ? row : m_last);
       const int kc = ((lane & 7) ^ ((row >> 1) & 7)) * 16;
-      xdma_off[i] = static_cast<uint32_t>(r * xsrc.ldx + kc);
+      xdma_off[i] = r * ldx + kc;
       // chunks past K: any valid bytes will do, the packed weight is zero there
-      xdma_off_last[i] = static_cast<uint32_t>(r * xsrc.ldx + (kc < ktail ? kc : ktail));
+      xdma_off_last[i] = r * ldx + (kc < ktail ? kc : ktail);
     }
   };
   auto dma_w = [&](int kt, int wb, int i) {
@@ -161,7 +166,7 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
     float wscale, bias;
     bool ok;
   };
-  auto load_consts = [&](int64_t n0) {
+  auto load_consts = [&](int n0) {
     Consts c{0, 1.f, 0.f, false};
     const int64_t n = n0 + t;
     if (t < BN && n < a.N) {
@@ -250,7 +255,7 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   const bool vec_ok = ((a.ldy & 15) == 0) && ((reinterpret_cast<uintptr_t>(a.y) & 15) == 0);
   const float bmul = bias_mul(a.w_scale_stride == 0, xq.scale * a.w_scales[0]);
   const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
-  auto epilogue = [&](int64_t m0, int64_t n0, int par, auto clamp_tag) {
+  auto epilogue = [&](int m0, int n0, int par, auto clamp_tag) {
     constexpr bool CL = decltype(clamp_tag)::value;
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
@@ -268,6 +273,11 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
               requant4<MODE, CL>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
         }
       wave_sync_lds();
+      // The next tile's first copies, requested before this epilogue, are waited
+      // for here: after a quarter of the arithmetic and before the first store,
+      // so that neither their latency nor the stores' sits at the top of the next
+      // tile (a wait there would also wait for the last stores to be acknowledged).
+      if (tm == 0) wait_loads(std::integral_constant<int, 0>{});
 #pragma unroll
       for (int pass = 0; pass < 2; ++pass) {
         const int p = pass * 16 + (lane >> 2), cq = lane & 3;
@@ -290,9 +300,9 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   };
 
   // ---- the block's tiles
-  int64_t v = blockIdx.x;
+  uint32_t v = blockIdx.x;
   if (v >= nblocks) return;
-  int64_t m0, n0;
+  int m0, n0;
   tile_origin(v, &m0, &n0);
   tile_setup(m0, n0);
   {
@@ -300,13 +310,12 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
     issue_prologue();
     store_consts(c, 0);
   }
+  wait_loads(std::integral_constant<int, 0>{});
   int par = 0;
   while (true) {
-    // everything this wave has in flight (the prologue copies, the stores of the
-    // previous epilogue) has landed; the barrier makes the stage-0 operands and
-    // the constants of every wave visible and ends the previous epilogue's use
-    // of the staging rows
-    wait_loads(std::integral_constant<int, 0>{});
+    // this wave's first copies have landed (waited for above or inside the
+    // previous epilogue); the barrier makes every wave's copies and the
+    // constants visible and ends the previous epilogue's use of the staging rows
     __syncthreads();
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
@@ -334,7 +343,7 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
     wait_loads(std::integral_constant<int, 0>{});
     __syncthreads();
 
-    const int64_t em0 = m0, en0 = n0;
+    const int em0 = m0, en0 = n0;
     v += gridDim.x;
     const bool more = v < nblocks;
     Consts next{0, 1.f, 0.f, false};
