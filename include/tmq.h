@@ -418,19 +418,6 @@ int tmq_qadaptive_avgpool2d(const void* x, void* y, int64_t B, int64_t H, int64_
 int tmq_qunary(const void* x, void* y, int64_t n, int kind, float in_scale, int32_t in_zero_point,
                float out_scale, int32_t out_zero_point, int q_signed, tmq_stream_t stream);
 
-/* ---------------------------------------------------------------------------
- * Measurement probe (no counterpart in the reference; used by bench.py only).
- * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four
- * waves and reports the sustained rate in TOP/s and the shader clock in GHz.
- * data_mode 0: zero operands, 1: uniform random bytes, 2: Gaussian int8 (all
- * held in registers), 3: Gaussian int8 operands read afresh from LDS for every
- * instruction, eight waves per workgroup (the GEMM's loop without its copies).
- * Unlike every other entry point this one synchronises (default stream) and
- * creates two HIP events; `scratch` is >= 2 KiB of device memory.
- * ------------------------------------------------------------------------- */
-int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, double* tops,
-                      double* shader_ghz);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,30 @@
+/*
+ * tmq_bench -- measurement helpers for bench.py (libtmq_bench.so).  Not part of
+ * the operator boundary in tmq.h and not linked into libtmq.so: nothing here
+ * has a counterpart in the reference, and unlike the operators these calls
+ * synchronise the device.
+ */
+#ifndef TMQ_BENCH_H_
+#define TMQ_BENCH_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---------------------------------------------------------------------------
+ * Measurement probe.
+ * Runs v_mfma_i32_32x32x32_i8 from registers on `blocks` workgroups of four
+ * waves and reports the sustained rate in TOP/s and the shader clock in GHz.
+ * data_mode 0: zero operands, 1: uniform random bytes, 2: Gaussian int8 (all
+ * held in registers), 3: Gaussian int8 operands read afresh from LDS for every
+ * instruction, eight waves per workgroup (the GEMM's loop without its copies).
+ * The call synchronises (default stream) and creates two HIP events; status
+ * codes are tmq.h's; `scratch` is >= 2 KiB of device memory.
+ * ------------------------------------------------------------------------- */
+int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, double* tops,
+                      double* shader_ghz);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TMQ_BENCH_H_ */

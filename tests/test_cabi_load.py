@@ -33,6 +33,19 @@ def test_library_exports_every_declared_symbol():
     assert lib.tmq_status_string(3) != lib.tmq_status_string(4)
 
 
+def test_measurement_probe_lives_in_its_own_library():
+    # include/tmq_bench.h is bench.py's, not the operator boundary: its symbols are
+    # exported by libtmq_bench.so and absent from libtmq.so
+    text = open(os.path.join(ROOT, "include", "tmq_bench.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(tmq_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["tmq_probe_mfma_i8"]
+    for name in names:
+        assert hasattr(cabi.bench_lib(), name)
+        assert not hasattr(cabi.lib(), name)
+        assert name not in cabi.DECLARED_SYMBOLS
+
+
 def test_struct_sizes_match_the_header():
     # natural alignment on x86-64: see include/tmq.h
     import ctypes as C

@@ -1,6 +1,7 @@
 """Builds the native libraries in-tree with hipcc (cross-compiles without a GPU).
 
   libtmq.so       torch-free HIP kernel library behind include/tmq.h
+  libtmq_bench.so measurement probe behind include/tmq_bench.h (bench.py only)
   libtmq_aten.so  ATen registrations (TORCH_LIBRARY_IMPL + dispatch stubs)
                   that call libtmq.so
 
@@ -23,10 +24,12 @@ CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(PKG, "build")
 LIB_KERNELS = os.path.join(PKG, "libtmq.so")
 LIB_ATEN = os.path.join(PKG, "libtmq_aten.so")
+LIB_BENCH = os.path.join(PKG, "libtmq_bench.so")
 ARCH = "gfx950"
 
 KERNEL_SOURCES = ["kernels/quantize.hip", "kernels/linear.hip", "kernels/conv2d.hip",
-                  "kernels/elementwise.hip", "kernels/probe.hip"]
+                  "kernels/elementwise.hip"]
+BENCH_SOURCES = ["bench/mfma_probe.hip"]
 ATEN_SOURCES = ["aten/register.cpp"]
 
 # -ffp-contract=off: the requantisation epilogue and the quantizer must round
@@ -59,11 +62,19 @@ def _hipcc():
 
 
 def build_kernels(verbose=False):
+    return _build_hip_library(KERNEL_SOURCES, LIB_KERNELS, verbose)
+
+
+def build_bench(verbose=False):
+    return _build_hip_library(BENCH_SOURCES, LIB_BENCH, verbose)
+
+
+def _build_hip_library(sources, lib_path, verbose):
     os.makedirs(OBJ, exist_ok=True)
     hipcc = _hipcc()
     inc = ["-I", os.path.join(ROOT, "include"), "-I", os.path.join(CSRC, "kernels")]
     jobs = []
-    for src in KERNEL_SOURCES:
+    for src in sources:
         path = os.path.join(CSRC, src)
         if not os.path.exists(path):
             continue
@@ -71,9 +82,9 @@ def build_kernels(verbose=False):
         jobs.append((obj, [hipcc] + DEVICE_FLAGS + inc + ["-c", path, "-o", obj]))
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
         list(ex.map(lambda j: _run(j[1], verbose), jobs))
-    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", LIB_KERNELS]
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", lib_path]
          + [j[0] for j in jobs], verbose)
-    return LIB_KERNELS
+    return lib_path
 
 
 def build_aten(verbose=False):
@@ -104,7 +115,7 @@ def build_aten(verbose=False):
 
 
 def build_all(verbose=False, kernels_only=False):
-    out = [build_kernels(verbose)]
+    out = [build_kernels(verbose), build_bench(verbose)]
     if not kernels_only and all(os.path.exists(os.path.join(CSRC, s)) for s in ATEN_SOURCES):
         out.append(build_aten(verbose))
     return out

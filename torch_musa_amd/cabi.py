@@ -28,7 +28,6 @@ DECLARED_SYMBOLS = [
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
-    "tmq_probe_mfma_i8",
 ]
 
 
@@ -141,8 +140,6 @@ def lib() -> C.CDLL:
         l.tmq_qmaxpool2d.argtypes = [v, v] + [C.c_int64] * 4 + [C.c_int32] * 8 + [C.c_int64] * 2 + [C.c_int, v]
         l.tmq_qadaptive_avgpool2d.argtypes = [v, v] + [C.c_int64] * 6 + [C.c_int32, C.c_int, v]
         l.tmq_qunary.argtypes = [v, v, C.c_int64, C.c_int, C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_int, v]
-        l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, v, C.POINTER(C.c_double),
-                                        C.POINTER(C.c_double)]
         _lib = l
     return _lib
 
@@ -645,13 +642,29 @@ def qadaptive_avgpool2d(x_nhwc, out_hw, zero_point):
 
 
 # ---------------------------------------------------------------------------
-# measurement probe
+# measurement probe (include/tmq_bench.h, libtmq_bench.so: not part of libtmq.so)
 # ---------------------------------------------------------------------------
+BENCH_LIB_PATH = os.path.join(_PKG, "libtmq_bench.so")
+_bench_lib = None
+
+
+def bench_lib() -> C.CDLL:
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise TmqError(f"{BENCH_LIB_PATH} is missing: build it with `python torch_musa_amd/build.py`")
+        l = C.CDLL(BENCH_LIB_PATH)
+        l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double),
+                                        C.POINTER(C.c_double)]
+        _bench_lib = l
+    return _bench_lib
+
+
 def probe_mfma_i8(data_mode: int, blocks: int = 256, iters: int = 20000):
     """-> (TOP/s, shader GHz) of a register-only int8 MFMA loop; synchronises."""
     scratch = torch.zeros(2048, dtype=torch.uint8, device="cuda")
     tops, ghz = C.c_double(), C.c_double()
     torch.cuda.synchronize()
-    check(lib().tmq_probe_mfma_i8(data_mode, blocks, iters, scratch.data_ptr(), C.byref(tops),
-                                  C.byref(ghz)), "tmq_probe_mfma_i8")
+    check(bench_lib().tmq_probe_mfma_i8(data_mode, blocks, iters, scratch.data_ptr(), C.byref(tops),
+                                        C.byref(ghz)), "tmq_probe_mfma_i8")
     return float(tops.value), float(ghz.value)

@@ -4,7 +4,10 @@
 // throughput, depends on how much the operands toggle.  bench.py reports the
 // probe next to the GEMM figure so that the GEMM can be read against the
 // ceiling the silicon actually reaches, not only against the nominal peak.
+// Built into libtmq_bench.so, a measurement library of its own: the operator
+// library libtmq.so carries no probe.
 #include "common.h"
+#include "tmq_bench.h"
 
 namespace tmq {
 namespace {
