@@ -10,9 +10,9 @@ resident in HBM.  The last line of stdout is one JSON object:
   value / unit     whole-job int8 throughput of those K steps (TOP/s)
   roofline         the GEMM kernel against the dense int8 MFMA peak, its average
                    launch duration measured with HIP events on the launch stream
-  cpu_baseline     the CPU oracle (a scalar C port of the reference CPU
-                   numerics, OpenMP over rows) on a bounded sample of the same
-                   workload, on this host's cores
+  cpu_baseline     PyTorch's quantized CPU op (fbgemm) on this host's cores at
+                   the same configuration, with a one-thread figure, the CPU
+                   model, the scalar C oracle port and the other configurations
   secondary        the other benchmark configurations: quantize / dequantize / min-max
                    over 2**28 fp32 (HBM bound), decode-shaped linear (weight
                    read bound), conv2d NHWC
@@ -60,8 +60,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--skip-secondary", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy"],
-                    help="run just this kernel --steps times (for rocprofv3 --pmc runs); 'copy' is a plain "
+    ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
+                                       "dequantize_pc", "decode", "conv", "conv_add_relu"],
+                    help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
+                         "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
                          "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -102,8 +104,14 @@ def main():
         elif args.only == "quantize":
             fn = lambda: torch.quantize_per_tensor(xf, 0.39, 128, torch.quint8)
         elif args.only == "dequantize":
-            q = torch.quantize_per_tensor(xf, 0.39, 128, torch.quint8)
-            fn = lambda: q.dequantize()
+            # two code tensors in turn: one alone (256 MiB) is the size of the last-level cache
+            qs_ = [torch.quantize_per_tensor(xf, 0.39, 128, torch.quint8),
+                   torch.quantize_per_tensor(xf * 0.5, 0.39, 128, torch.quint8)]
+            cnt_ = [0]
+
+            def fn():
+                cnt_[0] += 1
+                return qs_[cnt_[0] % 2].dequantize()
         else:
             ws_, mm_ = cabi.minmax_workspace(dev), torch.empty(2, device=dev)
             fn = lambda: cabi.minmax(xf, mm_, ws_)
@@ -111,6 +119,64 @@ def main():
             fn()
         torch.cuda.synchronize()
         print(json.dumps({"only": args.only, "launches": args.steps, "elements": n}))
+        return
+
+    def per_channel_sets(nsets):
+        """[11008, 4096] fp32 weights (config 3's weight shape) with per-row scales."""
+        out = []
+        for _ in range(nsets):
+            w_ = torch.randn(11008, 4096, device=dev) * 0.02
+            sc_ = (w_.abs().amax(dim=1) / 127.0).to(torch.float64)
+            out.append((w_, sc_, torch.zeros(11008, dtype=torch.int64, device=dev)))
+        return out
+
+    if args.only in ("quantize_pc", "dequantize_pc"):
+        sets_ = per_channel_sets(3)
+        qs_ = [torch.quantize_per_channel(w_, sc_, zp_, 0, torch.qint8) for w_, sc_, zp_ in sets_]
+        for i in range(args.steps):
+            if args.only == "quantize_pc":
+                w_, sc_, zp_ = sets_[i % 3]
+                torch.quantize_per_channel(w_, sc_, zp_, 0, torch.qint8)
+            else:
+                qs_[i % 3].dequantize()
+        torch.cuda.synchronize()
+        print(json.dumps({"only": args.only, "launches": args.steps, "shape": [11008, 4096], "axis": 0}))
+        return
+
+    if args.only == "decode":
+        # config 4 at M = 1: 40 packed weights in turn (cold), plain launches
+        pws = [cabi.PackedLinear(torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev))
+               for _ in range(40)]
+        wsd = torch.rand(4096, device=dev) * 0.002 + 0.001
+        bd = torch.randn(4096, device=dev)
+        xd = torch.randint(0, 256, (1, 4096), dtype=torch.uint8, device=dev)
+        yd = torch.empty((1, 4096), dtype=torch.uint8, device=dev)
+        for i in range(args.steps):
+            cabi.linear(xd, pws[i % 40], 0.02, 128, wsd, bd, 0.05, 128, out=yd)
+        torch.cuda.synchronize()
+        print(json.dumps({"only": "decode", "launches": args.steps, "M": 1, "K": 4096, "N": 4096}))
+        return
+
+    if args.only in ("conv", "conv_add_relu"):
+        # config 5: 24 inputs in turn (309 MB, more than the last-level cache)
+        csets = 24
+        xcqs = [torch._make_per_tensor_quantized_tensor(
+            torch.randint(0, 120, (32, 56, 56, 64), dtype=torch.uint8, device=dev).permute(0, 3, 1, 2), 0.03, 0)
+            for _ in range(csets)]
+        accs = [torch._make_per_tensor_quantized_tensor(
+            torch.randint(0, 256, (32, 56, 56, 64), dtype=torch.uint8, device=dev).permute(0, 3, 1, 2), 0.03, 128)
+            for _ in range(csets)] if args.only == "conv_add_relu" else None
+        wc = torch.randn(64, 64, 3, 3, device=dev) * 0.05
+        wcs = (wc.abs().amax(dim=(1, 2, 3)) / 127.0).to(torch.float64)
+        wcq = torch.quantize_per_channel(wc, wcs, torch.zeros(64, dtype=torch.int64, device=dev), 0, torch.qint8)
+        pc = torch.ops.quantized.conv2d_prepack(wcq, torch.randn(64, device=dev), [1, 1], [1, 1], [1, 1], 1)
+        for i in range(args.steps):
+            if accs is None:
+                torch.ops.quantized.conv2d(xcqs[i % csets], pc, 0.05, 0)
+            else:
+                torch.ops.quantized.conv2d_add_relu(xcqs[i % csets], accs[i % csets], pc, 0.05, 0)
+        torch.cuda.synchronize()
+        print(json.dumps({"only": args.only, "launches": args.steps, "x": [32, 56, 56, 64], "w": [64, 3, 3, 64]}))
         return
 
     # ------------------------------------------------------------------ C3
@@ -243,7 +309,16 @@ def main():
 
         hbm("quantize_per_tensor_c2", lambda: torch.quantize_per_tensor(xf, scale, zp, torch.quint8), 5 * n,
             "quantize_c2")
-        hbm("dequantize_c2", lambda: q.dequantize(), 5 * n, "dequantize_c2")
+        # two code tensors in turn: one alone (256 MiB) is the size of the last-level cache
+        q_alt = torch.quantize_per_tensor(xf * 0.5, scale, zp, torch.quint8)
+        dq_count = [0]
+
+        def dequantize_rotating():
+            dq_count[0] += 1
+            return (q if dq_count[0] % 2 else q_alt).dequantize()
+
+        hbm("dequantize_c2", dequantize_rotating, 5 * n, "dequantize_c2")
+        del q_alt
         hbm("minmax_c2", lambda: cabi.minmax(xf, mm_out, ws), 4 * n, "minmax_c2")
         hbm("quantize_per_tensor_dynamic_c2", lambda: torch.quantize_per_tensor_dynamic(xf, torch.quint8, False),
             9 * n, None)
@@ -253,6 +328,49 @@ def main():
         hbm("quantized_relu_2p28", lambda: torch.relu(q), 2 * n, None)
         hbm("quantized_gelu_2p28", lambda: torch.nn.functional.gelu(q), 2 * n, None)
         del xf, q, q2
+
+        # per-channel quantize / dequantize at config 3's weight shape, axis 0: 45 M elements,
+        # three tensors in turn (3 x 225 MB of input and output, more than the last-level cache)
+        log("[bench] per-channel quantize / dequantize, fp32 [11008, 4096], axis 0")
+        pcs = per_channel_sets(3)
+        pc_count = [0]
+        pc_out = [torch.empty((11008, 4096), dtype=torch.int8, device=dev) for _ in range(3)]
+        lib = cabi.lib()
+
+        def quantize_pc_kernel():
+            # the kernel through the C ABI (the operator adds a host-side check of the zero
+            # points' range in front of it, as the reference does: timed below)
+            pc_count[0] += 1
+            i = pc_count[0] % 3
+            w_, sc_, zp_ = pcs[i]
+            cabi.check(lib.tmq_quantize_per_channel(w_.data_ptr(), pc_out[i].data_ptr(), 1, 11008, 4096,
+                                                    sc_.data_ptr(), zp_.data_ptr(), 1, cabi.stream_ptr()),
+                       "tmq_quantize_per_channel")
+
+        npc = 11008 * 4096
+        hbm("quantize_per_channel_11008x4096", quantize_pc_kernel, 5 * npc + 16 * 11008, None)
+
+        def quantize_pc_op():
+            pc_count[0] += 1
+            w_, sc_, zp_ = pcs[pc_count[0] % 3]
+            return torch.quantize_per_channel(w_, sc_, zp_, 0, torch.qint8)
+
+        for _ in range(3):
+            quantize_pc_op()
+        ts = events_ms(quantize_pc_op, 20)
+        secondary["quantize_per_channel_11008x4096"]["operator_call_us"] = round(sum(ts) / len(ts) * 1e3, 1)
+        pc_r = [torch.empty((11008, 4096), dtype=torch.float32, device=dev) for _ in range(3)]
+
+        def dequantize_pc_kernel():
+            pc_count[0] += 1
+            i = pc_count[0] % 3
+            _, sc_, zp_ = pcs[i]
+            cabi.check(lib.tmq_dequantize_per_channel(pc_out[i].data_ptr(), pc_r[i].data_ptr(), 1, 11008, 4096,
+                                                      sc_.data_ptr(), zp_.data_ptr(), 1, cabi.stream_ptr()),
+                       "tmq_dequantize_per_channel")
+
+        hbm("dequantize_per_channel_11008x4096", dequantize_pc_kernel, 5 * npc + 16 * 11008, None)
+        del pcs, pc_out, pc_r
 
         # -------------------------------------------------------------- C1
         # x [128,1024] quint8 x W [1024,1024] per-channel qint8: 268 MOP and 1.2 MB, a
@@ -584,43 +702,120 @@ def main():
         del pxs
 
     # ------------------------------------------------------------ CPU baseline
+    # The reference CPU path = PyTorch's own quantized CPU ops (fbgemm engine), timed on
+    # this host's cores on bounded samples of the same workloads; the scalar C port of the
+    # same arithmetic (the parity oracle) is reported next to it as `oracle_port`.
     cpu_baseline = None
     if not args.skip_cpu:
         import oracle
 
         cores = min(os.cpu_count() or 1, 16)
-        rows = M if cores >= 8 else 512  # ~4 s of CPU work on 16 cores
-        xs = xq.int_repr()[:rows].cpu().numpy()
-        ws_h = wq.int_repr().cpu().numpy()
-        wsc = w_scales.cpu().numpy()
-        b_h = bias.cpu().numpy()
-        log(f"[bench] CPU baseline: oracle linear on {rows} of {M} rows, {cores} threads")
+        cpu_model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as f:
+                for line in f:
+                    if line.startswith("model name"):
+                        cpu_model = line.split(":", 1)[1].strip()
+                        break
+        except OSError:
+            pass
+        torch.backends.quantized.engine = "fbgemm"
+
+        def cpu_time(fn, min_s=0.5, max_reps=50):
+            fn()
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                fn()
+                reps += 1
+                dt = time.perf_counter() - t0
+                if dt >= min_s or reps >= max_reps:
+                    return dt / reps
+
+        xs_all = xq.int_repr().cpu()
+        wq_cpu, bias_cpu = wq.cpu(), bias.cpu()
+        p_cpu = torch.ops.quantized.linear_prepack(wq_cpu, bias_cpu)
+
+        def cpu_linear_tops(rows, threads):
+            torch.set_num_threads(threads)
+            xs_q = torch._make_per_tensor_quantized_tensor(xs_all[:rows].contiguous(), xq.q_scale(),
+                                                           xq.q_zero_point())
+            dt_ = cpu_time(lambda: torch.ops.quantized.linear(xs_q, p_cpu, out_scale, out_zp), min_s=2.0)
+            return 2.0 * rows * N * K / dt_ / 1e12, dt_
+
+        log(f"[bench] CPU baseline on {cpu_model}, {cores} threads: torch.ops.quantized.linear (fbgemm), config 3")
+        all_tops, all_dt = cpu_linear_tops(M, cores)
+        one_rows = 256
+        one_tops, one_dt = cpu_linear_tops(one_rows, 1)
+        log(f"[bench]   {cores} threads: {all_tops:.3f} TOP/s ({all_dt*1e3:.0f} ms per call); "
+            f"1 thread: {one_tops:.4f} TOP/s on {one_rows} rows")
+        cpu_baseline = {"value": round(all_tops, 4), "unit": "TOP/s", "cores": cores, "kind": "reference",
+                        "what": "torch.ops.quantized.linear on CPU tensors, engine fbgemm (the CPU ops the "
+                                "north star names as the reference; the reference's own device code cannot be "
+                                "built without the MUSA SDK)",
+                        "cpu_model": cpu_model,
+                        "sample": f"config 3 at full size (all {M} rows), {all_dt*1e3:.0f} ms per call, repeated "
+                                  "for about 2 s",
+                        "one_thread": {"value": round(one_tops, 5), "unit": "TOP/s", "cores": 1,
+                                       "sample": f"first {one_rows} of {M} rows, {one_dt*1e3:.0f} ms per call"}}
+
+        # the oracle (scalar C, OpenMP over rows) on a bounded sample, and the GPU against it
+        rows = 512
+        xs = xs_all[:rows].numpy()
         t0 = time.perf_counter()
-        y_ref = oracle.linear(xs, xq.q_scale(), xq.q_zero_point(), ws_h, wsc, b_h, out_scale, out_zp,
-                              nthreads=cores)
+        y_ref = oracle.linear(xs, xq.q_scale(), xq.q_zero_point(), wq.int_repr().cpu().numpy(), w_scales.cpu().numpy(),
+                              bias_cpu.numpy(), out_scale, out_zp, nthreads=cores)
         dt = time.perf_counter() - t0
-        cpu_tops = 2.0 * rows * N * K / dt / 1e12
         got = torch.ops.quantized.linear(xq, packed, out_scale, out_zp).int_repr()[:rows].cpu().numpy()
         max_diff = int(np.abs(got.astype(np.int32) - y_ref.astype(np.int32)).max())
-        log(f"[bench] CPU oracle: {dt:.2f} s, {cpu_tops*1e3:.2f} GOP/s; GPU vs oracle max diff {max_diff} LSB")
-        cpu_baseline = {"value": round(cpu_tops, 5), "unit": "TOP/s", "cores": cores, "kind": "port",
-                        "sample": f"first {rows} of {M} rows of config 3 (all {N} x {K} weights), "
-                                  f"{dt:.1f} s of CPU work", "gpu_vs_oracle_max_lsb": max_diff}
-        # PyTorch's own CPU op (fbgemm) on the same sample, for reference
-        try:
-            torch.backends.quantized.engine = "fbgemm"
-            torch.set_num_threads(cores)
-            xs_q = torch._make_per_tensor_quantized_tensor(torch.from_numpy(xs), xq.q_scale(), xq.q_zero_point())
-            p_cpu = torch.ops.quantized.linear_prepack(wq.cpu(), bias.cpu())
-            torch.ops.quantized.linear(xs_q, p_cpu, out_scale, out_zp)
-            t0 = time.perf_counter()
-            for _ in range(3):
-                torch.ops.quantized.linear(xs_q, p_cpu, out_scale, out_zp)
-            dt2 = (time.perf_counter() - t0) / 3
-            cpu_baseline["torch_cpu_fbgemm"] = {"value": round(2.0 * rows * N * K / dt2 / 1e12, 4),
-                                                "unit": "TOP/s", "threads": cores}
-        except Exception as e:  # the CPU op is extra information only
-            cpu_baseline["torch_cpu_fbgemm"] = {"error": str(e)[:200]}
+        y_cpu = torch.ops.quantized.linear(
+            torch._make_per_tensor_quantized_tensor(xs_all[:rows].contiguous(), xq.q_scale(), xq.q_zero_point()),
+            p_cpu, out_scale, out_zp).int_repr().numpy()
+        max_diff_cpu_op = int(np.abs(got.astype(np.int32) - y_cpu.astype(np.int32)).max())
+        log(f"[bench]   oracle port: {2.0 * rows * N * K / dt / 1e12 * 1e3:.1f} GOP/s; GPU vs oracle max diff "
+            f"{max_diff} LSB, GPU vs the CPU op {max_diff_cpu_op} LSB on {rows} rows")
+        cpu_baseline["oracle_port"] = {"value": round(2.0 * rows * N * K / dt / 1e12, 5), "unit": "TOP/s",
+                                       "cores": cores, "kind": "port",
+                                       "sample": f"first {rows} of {M} rows, {dt:.1f} s of CPU work"}
+        cpu_baseline["gpu_vs_oracle_max_lsb"] = max_diff
+        cpu_baseline["gpu_vs_cpu_op_max_lsb"] = max_diff_cpu_op
+        del xs_all, p_cpu, wq_cpu
+
+        # the other configurations on the CPU ops, all threads
+        torch.set_num_threads(cores)
+        others = {}
+        nc2 = 2 ** 26
+        xc2 = torch.randn(nc2) * 3.0
+        dtq = cpu_time(lambda: torch.quantize_per_tensor(xc2, 0.39, 128, torch.quint8))
+        qc2 = torch.quantize_per_tensor(xc2, 0.39, 128, torch.quint8)
+        dtd = cpu_time(lambda: qc2.dequantize())
+        dtm = cpu_time(lambda: torch.aminmax(xc2))
+        others["config2"] = {"sample": "2**26 of the 2**28 fp32 elements", "unit": "GB/s",
+                             "quantize_per_tensor": round(5 * nc2 / dtq / 1e9, 1),
+                             "dequantize": round(5 * nc2 / dtd / 1e9, 1),
+                             "aminmax": round(4 * nc2 / dtm / 1e9, 1)}
+        del xc2, qc2
+        wd = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8)
+        wdq = torch._make_per_channel_quantized_tensor(wd, torch.rand(4096, dtype=torch.float64) * 0.002 + 0.001,
+                                                       torch.zeros(4096, dtype=torch.int64), 0)
+        pd_cpu = torch.ops.quantized.linear_prepack(wdq, torch.randn(4096))
+        dec = {}
+        for Md in (1, 4, 16):
+            xd_ = torch._make_per_tensor_quantized_tensor(torch.randint(0, 256, (Md, 4096), dtype=torch.uint8),
+                                                          0.02, 128)
+            dt_ = cpu_time(lambda: torch.ops.quantized.linear(xd_, pd_cpu, 0.05, 128), min_s=0.3, max_reps=2000)
+            dec[f"m{Md}_us_per_call"] = round(dt_ * 1e6, 1)
+        others["config4"] = dict(dec, sample="K = N = 4096, one weight (cache-warm on the CPU)")
+        xc_ = torch._make_per_tensor_quantized_tensor(
+            torch.randint(0, 120, (32, 56, 56, 64), dtype=torch.uint8).permute(0, 3, 1, 2), 0.03, 0)
+        wc_ = torch._make_per_channel_quantized_tensor(
+            torch.randint(-127, 128, (64, 3, 3, 64), dtype=torch.int8).permute(0, 3, 1, 2),
+            torch.rand(64, dtype=torch.float64) * 0.002 + 0.001, torch.zeros(64, dtype=torch.int64), 0)
+        pc_cpu = torch.ops.quantized.conv2d_prepack(wc_, torch.randn(64), [1, 1], [1, 1], [1, 1], 1)
+        dtc = cpu_time(lambda: torch.ops.quantized.conv2d(xc_, pc_cpu, 0.05, 0))
+        others["config5"] = {"sample": "full size, [32,56,56,64] x [64,3,3,64]", "us_per_call": round(dtc * 1e6, 1),
+                             "value": round(2.0 * 32 * 56 * 56 * 64 * 576 / dtc / 1e12, 4), "unit": "TOP/s"}
+        log(f"[bench]   config 2 {others['config2']}; config 4 {dec}; config 5 {others['config5']['us_per_call']} us")
+        cpu_baseline["other_configs"] = others
 
     out = {
         "metric": "int8 quantized::linear TOPS (% MFMA peak) + quantize GB/s (% HBM), 1 GPU",

@@ -153,6 +153,40 @@ def test_per_channel_weight_sized(cabi):
     np.testing.assert_array_equal(host(q), oracle.quantize_per_channel(w, s, z, 0, True))
 
 
+@pytest.mark.parametrize("shape,axis", [
+    ((3, 5, 64), 1),        # shortest rows of the row kernel, channel index wraps inside a block
+    ((2, 3, 1024), 1),      # one run per row, 8 rows per block, 6 rows in all
+    ((7, 4096), 0),         # four accesses per row, two rows per block, odd row count
+    ((3, 2, 9000), 1),      # two segments per row, ragged end
+    ((5, 301), 0),          # rows that are not a multiple of 4: scalar accesses
+    ((2, 2, 1500, 2), 1),   # inner = 3000 from two trailing axes
+    ((1, 70000), 0),        # nine segments of 8192
+], ids=str)
+def test_per_channel_row_kernel_shapes(cabi, shape, axis):
+    """Rows of 64 elements and more take the kernel that derives the channel from
+    the block index: every decomposition (runs per row, rows per block, segments,
+    ragged ends, scalar accesses), both parameter kinds, both directions."""
+    say("qpc rows", shape, axis)
+    rng = np.random.default_rng(sum(shape) + axis)
+    C = shape[axis]
+    x = cases.randn(500 + sum(shape), shape)
+    for signed in (False, True):
+        s = rng.uniform(0.005, 0.05, C).astype(np.float64)
+        z = rng.integers(-128 if signed else 0, 128 if signed else 256, C).astype(np.int64)
+        q = cabi.quantize_per_channel(dev(x), dev(s), dev(z), axis, signed)
+        want = oracle.quantize_per_channel(x, s, z, axis, signed)
+        np.testing.assert_array_equal(host(q), want)
+        r = cabi.dequantize_per_channel(q, dev(s), dev(z), axis)
+        np.testing.assert_array_equal(host(r), oracle.dequantize_per_channel(want, s, z, axis))
+        sf = s.astype(np.float32)
+        zf = (z + rng.uniform(-0.4, 0.4, C)).astype(np.float32)
+        q = cabi.quantize_per_channel_float_qparams(dev(x), dev(sf), dev(zf), axis, signed)
+        want = oracle.quantize_per_channel_float(x, sf, zf, axis, signed)
+        np.testing.assert_array_equal(host(q), want)
+        r = cabi.dequantize_per_channel_float_qparams(q, dev(sf), dev(zf), axis)
+        np.testing.assert_array_equal(host(r), oracle.dequantize_per_channel_float(want, sf, zf, axis))
+
+
 def test_full_size_properties(cabi):
     """benchmark configuration 2 at full size (2**28 fp32): properties that need no
     full-size oracle run, plus oracle parity on sampled windows."""

@@ -11,6 +11,7 @@
 // the zero point, clamp.  Compiled with -ffp-contract=off.
 #include <cmath>
 #include <limits>
+#include <type_traits>
 
 #include "common.h"
 #include "qparams.h"
@@ -142,27 +143,33 @@ __global__ __launch_bounds__(kThreads) void quantize_scalar_kernel(
 // the last-level cache from the kernel that produced them); the fp32 output is
 // four times larger and streams out with non-temporal stores so that it does
 // not evict them.
+// Blocks of two waves: the kernel is bound by the write stream (four of every
+// five bytes; a plain 1 GiB fill reaches 4.5-5 TB/s on this part), and of the
+// block sizes 64 ... 1024 two waves with two accesses per thread sustained the
+// most over 2**28 elements (204.8 us against 210-240 us for the others).
+constexpr int kDqThreads = 128;
+
 template <bool SIGNED>
-__global__ __launch_bounds__(kThreads) void dequantize_vec_kernel(
+__global__ __launch_bounds__(kDqThreads) void dequantize_vec_kernel(
     const uint32_t* __restrict__ q4, v4f* __restrict__ r4, int64_t n4,
     const uint8_t* __restrict__ q, float* __restrict__ r, int64_t n, float scale, int zp) {
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnrollQD) + threadIdx.x;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kDqThreads * kUnrollQD) + threadIdx.x;
   uint32_t w[kUnrollQD];
-  if (base - threadIdx.x + kThreads * kUnrollQD <= n4) {
+  if (base - threadIdx.x + kDqThreads * kUnrollQD <= n4) {
 #pragma unroll
-    for (int u = 0; u < kUnrollQD; ++u) w[u] = q4[base + u * kThreads];
+    for (int u = 0; u < kUnrollQD; ++u) w[u] = q4[base + u * kDqThreads];
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u)
-      __builtin_nontemporal_store(dequantize_four<SIGNED>(w[u], zp, scale), &r4[base + u * kThreads]);
+      __builtin_nontemporal_store(dequantize_four<SIGNED>(w[u], zp, scale), &r4[base + u * kDqThreads]);
   } else {
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u) {
-      const int64_t i = base + u * kThreads;
+      const int64_t i = base + u * kDqThreads;
       if (i < n4) w[u] = q4[i];
     }
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u) {
-      const int64_t i = base + u * kThreads;
+      const int64_t i = base + u * kDqThreads;
       if (i < n4) r4[i] = dequantize_four<SIGNED>(w[u], zp, scale);
     }
   }
@@ -373,8 +380,11 @@ __global__ __launch_bounds__(kDynSmallThreads) void dynamic_quantize_small_kerne
 }
 
 // ---------------------------------------------------------------------------
-// Per-channel kernels over [outer, C, inner].  VEC = 4 when inner % 4 == 0 and
-// the pointers are 16-byte aligned (a group of 4 never straddles a channel).
+// Per-channel kernels over [outer, C, inner], element-indexed: the channel of
+// an element comes from its flat index.  They serve short rows (inner < 64,
+// e.g. a channel axis that is the last dimension); longer rows take
+// pc_rows_kernel below.  VEC = 4 when inner % 4 == 0 and the pointers are
+// 16-byte aligned (a group of 4 never straddles a channel).
 // ---------------------------------------------------------------------------
 template <bool SIGNED, int VEC>
 __global__ __launch_bounds__(kThreads) void quantize_pc_kernel(
@@ -489,6 +499,191 @@ __global__ __launch_bounds__(kThreads) void dequantize_pcf_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Per-channel kernels for inner >= kPcRowsMinInner: the channel is a property of
+// the block, not of the element.  The tensor is `rows` = outer * C rows of
+// `inner` elements; a block takes RB = A >> lg_us consecutive rows (A accesses per thread) x one
+// segment of US = 1 << lg_us runs of 256 lanes x VEC elements, i.e. eight
+// accesses per thread whatever the row length (a row of 4096 floats is four
+// 16-byte accesses per thread, so a quantizing block takes two rows).  Row and channel come
+// from blockIdx with one division per block; the parameters of a row are
+// wave-uniform (scalar loads); the element loop has no division at all.
+// Loads are batched ahead of the stores and carry the same cache hints as the
+// per-tensor kernels.
+// ---------------------------------------------------------------------------
+constexpr int kPcRowsMinInner = 64;
+
+template <bool SIGNED>
+struct PcQuantize {
+  // fp32 -> codes, double scales, int64 zero points
+  static constexpr int kAccesses = 8;
+  const float* x;
+  uint8_t* q;
+  const double* scales;
+  const int64_t* zps;
+  struct P { float inv, zp; };
+  using In4 = v4f;
+  using In1 = float;
+  __device__ __forceinline__ P params(int64_t c) const {
+    return {1.0f / static_cast<float>(scales[c]), static_cast<float>(zps[c])};
+  }
+  __device__ __forceinline__ In4 load4(int64_t i) const {
+    return __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + i));
+  }
+  __device__ __forceinline__ In1 load1(int64_t i) const { return x[i]; }
+  __device__ __forceinline__ void store4(int64_t i, In4 v, P p) const {
+    *reinterpret_cast<uint32_t*>(q + i) = quantize_four<SIGNED>(v, p.inv, p.zp);
+  }
+  __device__ __forceinline__ void store1(int64_t i, In1 v, P p) const {
+    q[i] = static_cast<uint8_t>(quantize_one<SIGNED>(v, p.inv, p.zp));
+  }
+};
+
+template <bool SIGNED>
+struct PcDequantize {
+  // codes -> fp32, double scales, int64 zero points
+  static constexpr int kAccesses = 4;
+  const uint8_t* q;
+  float* r;
+  const double* scales;
+  const int64_t* zps;
+  struct P { double scale; float zp; };
+  using In4 = uint32_t;
+  using In1 = uint32_t;
+  __device__ __forceinline__ P params(int64_t c) const { return {scales[c], static_cast<float>(zps[c])}; }
+  __device__ __forceinline__ In4 load4(int64_t i) const { return *reinterpret_cast<const uint32_t*>(q + i); }
+  __device__ __forceinline__ In1 load1(int64_t i) const { return q[i]; }
+  __device__ __forceinline__ void store4(int64_t i, In4 w, P p) const {
+    v4f o;
+    o.x = dequantize_pc_one<SIGNED>(w & 0xffu, p.zp, p.scale);
+    o.y = dequantize_pc_one<SIGNED>((w >> 8) & 0xffu, p.zp, p.scale);
+    o.z = dequantize_pc_one<SIGNED>((w >> 16) & 0xffu, p.zp, p.scale);
+    o.w = dequantize_pc_one<SIGNED>(w >> 24, p.zp, p.scale);
+    __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(r + i));
+  }
+  __device__ __forceinline__ void store1(int64_t i, In1 b, P p) const {
+    r[i] = dequantize_pc_one<SIGNED>(b, p.zp, p.scale);
+  }
+};
+
+template <bool SIGNED>
+struct PcfQuantize {
+  // fp32 -> codes, float scales and float zero points
+  static constexpr int kAccesses = 8;
+  const float* x;
+  uint8_t* q;
+  const float* scales;
+  const float* zps;
+  struct P { float inv, zp; };
+  using In4 = v4f;
+  using In1 = float;
+  __device__ __forceinline__ P params(int64_t c) const {
+    const float sc = scales[c];
+    return {sc == 0.f ? 1.0f : 1.0f / sc, zps[c]};
+  }
+  __device__ __forceinline__ In4 load4(int64_t i) const {
+    return __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + i));
+  }
+  __device__ __forceinline__ In1 load1(int64_t i) const { return x[i]; }
+  __device__ __forceinline__ void store4(int64_t i, In4 v, P p) const {
+    *reinterpret_cast<uint32_t*>(q + i) =
+        quantize_fq_one<SIGNED>(v.x, p.inv, p.zp) | (quantize_fq_one<SIGNED>(v.y, p.inv, p.zp) << 8) |
+        (quantize_fq_one<SIGNED>(v.z, p.inv, p.zp) << 16) | (quantize_fq_one<SIGNED>(v.w, p.inv, p.zp) << 24);
+  }
+  __device__ __forceinline__ void store1(int64_t i, In1 v, P p) const {
+    q[i] = static_cast<uint8_t>(quantize_fq_one<SIGNED>(v, p.inv, p.zp));
+  }
+};
+
+template <bool SIGNED>
+struct PcfDequantize {
+  // codes -> fp32, float scales and float zero points
+  static constexpr int kAccesses = 4;
+  const uint8_t* q;
+  float* r;
+  const float* scales;
+  const float* zps;
+  struct P { float scale, zp; };
+  using In4 = uint32_t;
+  using In1 = uint32_t;
+  __device__ __forceinline__ P params(int64_t c) const { return {scales[c], zps[c]}; }
+  __device__ __forceinline__ In4 load4(int64_t i) const { return *reinterpret_cast<const uint32_t*>(q + i); }
+  __device__ __forceinline__ In1 load1(int64_t i) const { return q[i]; }
+  __device__ __forceinline__ void store4(int64_t i, In4 w, P p) const {
+    v4f o;
+    o.x = dequantize_fq_one<SIGNED>(w & 0xffu, p.zp, p.scale);
+    o.y = dequantize_fq_one<SIGNED>((w >> 8) & 0xffu, p.zp, p.scale);
+    o.z = dequantize_fq_one<SIGNED>((w >> 16) & 0xffu, p.zp, p.scale);
+    o.w = dequantize_fq_one<SIGNED>(w >> 24, p.zp, p.scale);
+    __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(r + i));
+  }
+  __device__ __forceinline__ void store1(int64_t i, In1 b, P p) const {
+    r[i] = dequantize_fq_one<SIGNED>(b, p.zp, p.scale);
+  }
+};
+
+// Accesses per thread (Op::kAccesses), all in flight before the first store: eight
+// for the quantizers, four for the dequantizers (at fp32 [11008, 4096], axis 0:
+// quantize 42.5 / 40.5 / 38.4 / 40.4 us with 2 / 4 / 8 / 16, dequantize 33.8 / 33.4 /
+// 36.0 / 38.7 us).
+template <class Op, int VEC>
+__global__ __launch_bounds__(kThreads) void pc_rows_kernel(Op op, int64_t rows, int64_t C, int64_t inner,
+                                                           int lg_us, uint32_t segs) {
+  using In = std::conditional_t<VEC == 4, typename Op::In4, typename Op::In1>;
+  constexpr int kPcAccesses = Op::kAccesses;
+  const uint32_t rg = blockIdx.x / segs, seg = blockIdx.x - rg * segs;
+  const int us_mask = (1 << lg_us) - 1;
+  const int64_t row0 = static_cast<int64_t>(rg) * (kPcAccesses >> lg_us);
+  const int64_t c0 = row0 % C;  // once per block, wave-uniform
+  const int64_t col0 = (static_cast<int64_t>(seg) << lg_us) * (kThreads * VEC) + threadIdx.x * VEC;
+  In held[kPcAccesses];
+  bool live[kPcAccesses];
+#pragma unroll
+  for (int u = 0; u < kPcAccesses; ++u) {
+    const int64_t row = row0 + (u >> lg_us);
+    const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kThreads * VEC);
+    live[u] = row < rows && col < inner;
+    if (live[u]) {
+      if constexpr (VEC == 4) held[u] = op.load4(row * inner + col);
+      else held[u] = op.load1(row * inner + col);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kPcAccesses; ++u) {
+    const int64_t row = row0 + (u >> lg_us);
+    if (row >= rows) break;  // uniform
+    int64_t c = c0 + (u >> lg_us);
+    while (c >= C) c -= C;   // at most A - 1 rows past c0: uniform, a few scalar steps
+    const typename Op::P p = op.params(c);
+    const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kThreads * VEC);
+    if (live[u]) {
+      if constexpr (VEC == 4) op.store4(row * inner + col, held[u], p);
+      else op.store1(row * inner + col, held[u], p);
+    }
+  }
+}
+
+// Launches pc_rows_kernel if the shape suits it; returns false if the caller
+// should use the element-indexed kernels (short rows, or a grid beyond 2**31).
+template <class Op>
+bool launch_pc_rows(const Op& op, int64_t outer, int64_t C, int64_t inner, bool vec, hipStream_t s) {
+  if (inner < kPcRowsMinInner) return false;
+  constexpr int kPcAccesses = Op::kAccesses;
+  const int64_t per_run = kThreads * (vec ? 4 : 1);
+  int lg_us = 0;
+  while ((2 << lg_us) <= kPcAccesses && (per_run << lg_us) < inner) ++lg_us;
+  const int64_t rows = outer * C;
+  const int64_t segs = ceil_div(inner, per_run << lg_us);
+  const int64_t row_groups = ceil_div(rows, kPcAccesses >> lg_us);
+  if (segs > 0x7fffffff || row_groups > 0x7fffffff / segs) return false;
+  const dim3 grid(static_cast<unsigned>(row_groups * segs));
+  if (vec)
+    pc_rows_kernel<Op, 4><<<grid, dim3(kThreads), 0, s>>>(op, rows, C, inner, lg_us, static_cast<uint32_t>(segs));
+  else
+    pc_rows_kernel<Op, 1><<<grid, dim3(kThreads), 0, s>>>(op, rows, C, inner, lg_us, static_cast<uint32_t>(segs));
+  return true;
+}
+
 inline unsigned grid_for(int64_t work_items, int64_t per_block, int64_t cap) {
   int64_t g = ceil_div(work_items, per_block);
   if (g < 1) g = 1;
@@ -563,14 +758,14 @@ TMQ_EXPORT int tmq_dequantize_per_tensor(const void* q, float* r, int64_t n, dou
   const uint8_t* qb = static_cast<const uint8_t*>(q);
   if (aligned(r, 16) && aligned(q, 4)) {
     const int64_t n4 = n / 4;
-    const int64_t blocks = n4 == 0 ? 1 : ceil_div(n4, kThreads * kUnrollQD);
+    const int64_t blocks = n4 == 0 ? 1 : ceil_div(n4, kDqThreads * kUnrollQD);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
     auto* q4 = reinterpret_cast<const uint32_t*>(q);
     auto* r4 = reinterpret_cast<v4f*>(r);
     if (q_signed)
-      dequantize_vec_kernel<true><<<dim3(blocks), dim3(kThreads), 0, s>>>(q4, r4, n4, qb, r, n, scale_f, zp);
+      dequantize_vec_kernel<true><<<dim3(blocks), dim3(kDqThreads), 0, s>>>(q4, r4, n4, qb, r, n, scale_f, zp);
     else
-      dequantize_vec_kernel<false><<<dim3(blocks), dim3(kThreads), 0, s>>>(q4, r4, n4, qb, r, n, scale_f, zp);
+      dequantize_vec_kernel<false><<<dim3(blocks), dim3(kDqThreads), 0, s>>>(q4, r4, n4, qb, r, n, scale_f, zp);
   } else {
     const unsigned g = grid_for(n, kThreads, 65536);
     if (q_signed)
@@ -692,6 +887,9 @@ TMQ_EXPORT int tmq_quantize_per_channel(const float* x, void* q, int64_t outer, 
   hipStream_t s = as_stream(stream);
   uint8_t* qb = static_cast<uint8_t*>(q);
   const bool vec = inner % 4 == 0 && aligned(x, 16) && aligned(q, 4);
+  if (q_signed ? launch_pc_rows(PcQuantize<true>{x, qb, scales, zero_points}, outer, channels, inner, vec, s)
+               : launch_pc_rows(PcQuantize<false>{x, qb, scales, zero_points}, outer, channels, inner, vec, s))
+    return launch_status();
   const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
   if (vec) {
     if (q_signed)
@@ -718,6 +916,9 @@ TMQ_EXPORT int tmq_dequantize_per_channel(const void* q, float* r, int64_t outer
   hipStream_t s = as_stream(stream);
   const uint8_t* qb = static_cast<const uint8_t*>(q);
   const bool vec = inner % 4 == 0 && aligned(r, 16) && aligned(q, 4);
+  if (q_signed ? launch_pc_rows(PcDequantize<true>{qb, r, scales, zero_points}, outer, channels, inner, vec, s)
+               : launch_pc_rows(PcDequantize<false>{qb, r, scales, zero_points}, outer, channels, inner, vec, s))
+    return launch_status();
   const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
   if (vec) {
     if (q_signed)
@@ -745,6 +946,9 @@ TMQ_EXPORT int tmq_quantize_per_channel_float_qparams(const float* x, void* q, i
   hipStream_t s = as_stream(stream);
   uint8_t* qb = static_cast<uint8_t*>(q);
   const bool vec = inner % 4 == 0 && aligned(x, 16) && aligned(q, 4);
+  if (q_signed ? launch_pc_rows(PcfQuantize<true>{x, qb, scales, zero_points}, outer, channels, inner, vec, s)
+               : launch_pc_rows(PcfQuantize<false>{x, qb, scales, zero_points}, outer, channels, inner, vec, s))
+    return launch_status();
   const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
   if (vec) {
     if (q_signed)
@@ -772,6 +976,9 @@ TMQ_EXPORT int tmq_dequantize_per_channel_float_qparams(const void* q, float* r,
   hipStream_t s = as_stream(stream);
   const uint8_t* qb = static_cast<const uint8_t*>(q);
   const bool vec = inner % 4 == 0 && aligned(r, 16) && aligned(q, 4);
+  if (q_signed ? launch_pc_rows(PcfDequantize<true>{qb, r, scales, zero_points}, outer, channels, inner, vec, s)
+               : launch_pc_rows(PcfDequantize<false>{qb, r, scales, zero_points}, outer, channels, inner, vec, s))
+    return launch_status();
   const unsigned g = grid_for(n, kThreads * (vec ? 4 : 1), 1 << 20);
   if (vec) {
     if (q_signed)
