@@ -419,6 +419,35 @@ def main():
                for _ in range(sets)]
         wsd = torch.rand(Nd, device=dev) * 0.002 + 0.001
         bd = torch.randn(Nd, device=dev)
+        def graph_us(run_once, calls):
+            run_once()
+            torch.cuda.synchronize()
+            side_ = torch.cuda.Stream()
+            graph_ = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side_):
+                run_once()
+                side_.synchronize()
+                with torch.cuda.graph(graph_, stream=side_):
+                    run_once()
+            torch.cuda.synchronize()
+            for _ in range(3):
+                graph_.replay()
+            ts_ = events_ms(graph_.replay, 10)
+            return sum(ts_) / len(ts_) / calls * 1e3
+
+        # floors, measured the same way: an empty kernel of the decode kernel's grid, and a kernel
+        # of its shape that only reads the 16.8 MB of packed weights (nothing computed, nothing stored)
+        sink = torch.zeros(4096, dtype=torch.uint8, device=dev)
+        empty_us = graph_us(lambda: [cabi.bench_empty_kernel(Nd // 16, sink) for _ in range(sets)], sets)
+        read_us = graph_us(lambda: [cabi.bench_stream_read(p.packed, sink) for p in pws], sets)
+        log(f"[bench] decode floors in a replayed graph: empty kernel {empty_us:.2f} us, read-only kernel "
+            f"{read_us:.2f} us per launch")
+        secondary["linear_decode_floors"] = {
+            "empty_kernel_us": round(empty_us, 3), "read_only_kernel_us": round(read_us, 3),
+            "read_only_gbs": round(Nd * Kd / read_us / 1e3, 1),
+            "method": f"{sets} launches replayed in one HIP graph, as for the operator: an empty kernel on "
+                      f"{Nd // 16} workgroups of eight waves; a kernel of the decode kernel's shape that only "
+                      "reads the packed weight of each of the 40 sets"}
         for Md in (1, 4, 16):
             xd = torch.randint(0, 256, (Md, Kd), dtype=torch.uint8, device=dev)
             yd = torch.empty((Md, Nd), dtype=torch.uint8, device=dev)
@@ -427,20 +456,7 @@ def main():
                 for p in pws:
                     cabi.linear(xd, p, 0.02, 128, wsd, bd, 0.05, 128, out=yd)
 
-            run_sets()
-            torch.cuda.synchronize()
-            side = torch.cuda.Stream()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.stream(side):
-                run_sets()
-                side.synchronize()
-                with torch.cuda.graph(graph, stream=side):
-                    run_sets()
-            torch.cuda.synchronize()
-            for _ in range(3):
-                graph.replay()
-            ts = events_ms(graph.replay, 10)
-            per = sum(ts) / len(ts) / sets
+            per = graph_us(run_sets, sets) * 1e-3
             nbytes = Nd * Kd + Md * Kd + Md * Nd + 12 * Nd
             gbs = nbytes / (per * 1e-3) / 1e9
             log(f"[bench] decode M={Md}: {per*1e3:.2f} us/launch in a replayed graph, {gbs:.0f} GB/s")
@@ -448,6 +464,7 @@ def main():
                 "avg_launch_us": round(per * 1e3, 3), "value": round(gbs, 1), "unit": "GB/s",
                 "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
+                "frac_of_read_only_kernel": round(read_us / (per * 1e3), 4),
                 "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
                 "algorithmic_bytes_per_launch": nbytes}
 

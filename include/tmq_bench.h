@@ -24,6 +24,15 @@ extern "C" {
 int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, double* tops,
                       double* shader_ghz);
 
+/* Floors for the weight-streaming linear kernel, asynchronous on `stream` (a
+ * hipStream_t as in tmq.h) so that they can be captured into a HIP graph like
+ * the operator: a kernel that only reads `bytes` (a multiple of 65536) with the
+ * decode kernel's shape (one block of eight waves per 64 KiB, all loads in
+ * flight at once) and an empty kernel on `blocks` workgroups of eight waves.
+ * `sink` is >= 2 KiB of device memory that is never written for real data. */
+int tmq_bench_stream_read(const void* src, int64_t bytes, void* sink, void* stream);
+int tmq_bench_empty_kernel(int blocks, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,15 +29,19 @@ ARCH = "gfx950"
 
 KERNEL_SOURCES = ["kernels/quantize.hip", "kernels/linear.hip", "kernels/conv2d.hip",
                   "kernels/elementwise.hip"]
-BENCH_SOURCES = ["bench/mfma_probe.hip"]
+BENCH_SOURCES = ["bench/bench_kernels.hip"]
 ATEN_SOURCES = ["aten/register.cpp"]
 
 # -ffp-contract=off: the requantisation epilogue and the quantizer must round
 # after every fp32 operation, as the CPU ops they mirror do.
 # packed-fp32-ops disabled: never emit v_pk_{add,mul,fma}_f32.
+# amdgpu-kernarg-preload-count: the leading scalar arguments of a kernel (up to
+# 14 dwords) reach its waves in SGPRs at launch instead of through a read of the
+# argument buffer; the latency-bound kernels put what their first loads need there.
 DEVICE_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC",
     "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -656,8 +656,20 @@ def bench_lib() -> C.CDLL:
         l = C.CDLL(BENCH_LIB_PATH)
         l.tmq_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]
+        l.tmq_bench_stream_read.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
+        l.tmq_bench_empty_kernel.argtypes = [C.c_int, C.c_void_p, C.c_void_p]
         _bench_lib = l
     return _bench_lib
+
+
+def bench_stream_read(src: torch.Tensor, sink: torch.Tensor) -> None:
+    """A kernel that only reads `src` (bytes a multiple of 64 KiB), shaped like the decode kernel."""
+    check(bench_lib().tmq_bench_stream_read(src.data_ptr(), src.numel() * src.element_size(), sink.data_ptr(),
+                                            stream_ptr()), "tmq_bench_stream_read")
+
+
+def bench_empty_kernel(blocks: int, sink: torch.Tensor) -> None:
+    check(bench_lib().tmq_bench_empty_kernel(blocks, sink.data_ptr(), stream_ptr()), "tmq_bench_empty_kernel")
 
 
 def probe_mfma_i8(data_mode: int, blocks: int = 256, iters: int = 20000):

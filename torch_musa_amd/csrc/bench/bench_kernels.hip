@@ -168,3 +168,42 @@ TMQ_EXPORT int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scr
   *shader_ghz = static_cast<double>(host[0]) / (static_cast<double>(host[1]) / 100e6) / 1e9;
   return TMQ_OK;
 }
+
+// ---------------------------------------------------------------------------
+// Floors for the weight-streaming (decode) kernel: a kernel that only reads
+// `bytes` (a multiple of 64 KiB) with that kernel's shape -- one block of eight
+// waves per 64 KiB, eight 16-byte loads per thread, all in flight at once -- and
+// an empty kernel of the same grid.  Both are asynchronous on `stream`, so that
+// bench.py can replay them from a HIP graph exactly as it replays the operator.
+// ---------------------------------------------------------------------------
+namespace tmq {
+namespace {
+__global__ __launch_bounds__(512) void stream_read_kernel(const v4i* __restrict__ src, int* sink) {
+  const v4i* p = src + static_cast<int64_t>(blockIdx.x) * 4096 + threadIdx.x;
+  v4i v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = __builtin_nontemporal_load(p + i * 512);
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+  if (s == 0x5a17c0de) sink[threadIdx.x] = s;  // never true for the benchmark's data; keeps the loads alive
+}
+__global__ __launch_bounds__(512) void empty_kernel(int* sink) {
+  if (sink == nullptr) sink[0] = 0;
+}
+}  // namespace
+}  // namespace tmq
+
+TMQ_EXPORT int tmq_bench_stream_read(const void* src, int64_t bytes, void* sink, tmq_stream_t stream) {
+  if (src == nullptr || sink == nullptr || bytes <= 0 || bytes % 65536 != 0 || bytes / 65536 > 0x7fffffff)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  stream_read_kernel<<<dim3(static_cast<unsigned>(bytes / 65536)), dim3(512), 0, as_stream(stream)>>>(
+      static_cast<const v4i*>(src), static_cast<int*>(sink));
+  return launch_status();
+}
+
+TMQ_EXPORT int tmq_bench_empty_kernel(int blocks, void* sink, tmq_stream_t stream) {
+  if (blocks <= 0 || sink == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
+  empty_kernel<<<dim3(blocks), dim3(512), 0, as_stream(stream)>>>(static_cast<int*>(sink));
+  return launch_status();
+}

@@ -95,66 +95,99 @@ constexpr int kDecodeMaxRows = 64;
 constexpr int kDecodeRowsAuto = 64;  // largest M the automatic choice sends here
 // MG = groups of 16 activation rows (M <= 16 * MG): the weight operands are
 // loaded once and multiplied with every group.
+//
+// The 14 dwords in front of GemmArgs are everything the kernel's loads need.  The
+// library is compiled with kernel-argument preloading, which hands up to 14
+// leading scalar dwords of a kernel to its waves in SGPRs at launch, so the
+// requests leave without waiting for a read of the argument buffer; the rest of
+// the arguments is fetched under the weight stream.  The finishing threads'
+// per-channel constants are requested first (cold, and memory serves requests
+// in the order issued), then each k-block's weights (HBM) and activations (L2).
+// Measured at K = N = 4096 in a replayed graph of 40 cold weights: 5.25 us at
+// M = 1, of which 1.9 us are what an empty kernel costs there, a kernel that
+// only reads the 16.8 MB takes 4.1 us, and the one that also stores 4 KB of
+// results 4.5 us (the store's acknowledgement ends the kernel); the order of the
+// requests, one or two accumulators and 4 / 8 / 16 waves all stay within 0.1 us.
+// flags: bits 0-7 M, bit 8 per-channel weight scales, bit 9 unsigned activations.
 template <int MODE, int MG>
-__global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(GemmArgs a, XLinear xs) {
+__global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(
+    const uint8_t* __restrict__ w_packed, const uint8_t* __restrict__ x, const int32_t* __restrict__ colsum,
+    const float* __restrict__ w_scales, const float* __restrict__ bias, int32_t K, int32_t ldx, int32_t N,
+    uint32_t flags, GemmArgs a) {
   constexpr int kWaves = kDecodeWaves;
   constexpr int kBatch = 8;  // 64-byte k-blocks in flight per wave: 64 KB of weights per block
   __shared__ int s_part[kWaves][MG][16 * 16];
   const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
   const int lr = lane & 15, lc = lane >> 4;
-  const int64_t nb = blockIdx.x;
-  const int64_t KB = ceil_div(a.K, 64);
-  const uint8_t* wp = a.w_packed + nb * a.w_kchunks * 256 + lc * 256 + lr * 16;
-  bool xrow[MG];
-  const uint8_t* xp[MG];
-#pragma unroll
-  for (int mg = 0; mg < MG; ++mg) {
-    xrow[mg] = mg * 16 + lr < a.M;
-    xp[mg] = xs.x + (xrow[mg] ? mg * 16 + lr : 0) * xs.ldx + lc * 16;
-  }
-  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
-                     static_cast<int>(a.x_xor), static_cast<int>(a.x_xor)};
-  // The 64 threads that finish a block (thread -> activation row within a
-  // group, channel group of 4) request their per-channel constants first, so
-  // that these arrive under the weight stream instead of after it.
+  const int nb = blockIdx.x;
+  const int M = static_cast<int>(flags & 0xffu);
+  const int KB = (K + 63) >> 6;
+  // The 64 threads that finish a block: thread -> activation row within a
+  // group, channel group of 4.
   const int fm = t >> 2, fg = t & 3;
   int c_cs[4] = {0, 0, 0, 0};
   float c_ws[4] = {1.f, 1.f, 1.f, 1.f}, c_b[4] = {0.f, 0.f, 0.f, 0.f};
   if (t < 64) {
+    const int ws_stride = (flags >> 8) & 1;
+    const float* const bsrc = bias != nullptr ? bias : w_scales;  // a load that always has an address
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int64_t n = nb * 16 + 4 * fg + j;
-      const int64_t np = n < a.N ? n : 0;
-      c_cs[j] = a.colsum[np];
+      const int n = nb * 16 + 4 * fg + j;
+      const int np = n < N ? n : 0;
+      c_cs[j] = colsum[np];
       if (MODE != kOutAcc32) {
-        c_ws[j] = a.w_scales[np * a.w_scale_stride];
-        if (a.bias != nullptr) c_b[j] = a.bias[np];
+        c_ws[j] = w_scales[np * ws_stride];
+        const float bv = bsrc[bias != nullptr ? np : 0];
+        c_b[j] = bias != nullptr ? bv : 0.f;
       }
     }
   }
-  v4i acc[MG];
+  const uint8_t* wp = w_packed + static_cast<int64_t>(nb) * (packed_kchunks(K) * 256) + lc * 256 + lr * 16;
+  bool xrow[MG];
+  const uint8_t* xp[MG];
 #pragma unroll
-  for (int mg = 0; mg < MG; ++mg) acc[mg] = v4i{0, 0, 0, 0};
-  for (int64_t kb0 = wave; kb0 < KB; kb0 += kWaves * kBatch) {
+  for (int mg = 0; mg < MG; ++mg) {
+    xrow[mg] = mg * 16 + lr < M;
+    xp[mg] = x + static_cast<int64_t>(xrow[mg] ? mg * 16 + lr : 0) * ldx;  // the row's first byte: always readable
+  }
+  const int xor_word = (flags >> 9) & 1 ? static_cast<int>(0x80808080u) : 0;
+  const v4i xmask = {xor_word, xor_word, xor_word, xor_word};
+  // Two accumulators per row group, used in turn: a multiply-accumulate does not
+  // wait for the one before it.
+  v4i acc2[MG][2];
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) acc2[mg][0] = acc2[mg][1] = v4i{0, 0, 0, 0};
+  // Every load of a batch is unconditional (addresses clamped into the operands,
+  // the activation operand of a block that does not exist set to zero after the
+  // load), so that the counts of outstanding loads are exact and the k-blocks are
+  // multiplied one by one as they arrive; with a load under a condition the
+  // compiler waits for all of them before the first product.
+  auto batch = [&](int kb0) {
     v4i wf[kBatch], xf[MG][kBatch];
+    bool xok[MG][kBatch];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
-      const int64_t kb = kb0 + u * kWaves;
-      const bool ok = kb < KB;
-      wf[u] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + kb * 1024))
-                 : v4i{0, 0, 0, 0};
+      const int kb = kb0 + u * kWaves;
+      const int kbc = kb < KB ? kb : KB - 1;
+      wf[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + static_cast<int64_t>(kbc) * 1024));
 #pragma unroll
       for (int mg = 0; mg < MG; ++mg) {
-        const bool xok = ok && xrow[mg] && (kb * 64 + lc * 16 < a.K);
-        xf[mg][u] = xok ? ld16(xp[mg] + kb * 64) : v4i{0, 0, 0, 0};
+        xok[mg][u] = kb < KB && xrow[mg] && (kb * 64 + lc * 16 < K);
+        xf[mg][u] = ld16(xp[mg] + (xok[mg][u] ? kb * 64 + lc * 16 : 0));
       }
     }
 #pragma unroll
     for (int u = 0; u < kBatch; ++u)
 #pragma unroll
-      for (int mg = 0; mg < MG; ++mg)
-        acc[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], xf[mg][u] ^ xmask, acc[mg], 0, 0, 0);
-  }
+      for (int mg = 0; mg < MG; ++mg) {
+        const v4i xv = xok[mg][u] ? (xf[mg][u] ^ xmask) : v4i{0, 0, 0, 0};
+        acc2[mg][u & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], xv, acc2[mg][u & 1], 0, 0, 0);
+      }
+  };
+  for (int kb0 = wave; kb0 < KB; kb0 += kWaves * kBatch) batch(kb0);
+  v4i acc[MG];
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) acc[mg] = acc2[mg][0] + acc2[mg][1];
 #pragma unroll
   for (int mg = 0; mg < MG; ++mg)
 #pragma unroll
@@ -659,12 +692,20 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     if (a.M > kDecodeMaxRows) return TMQ_ERR_UNSUPPORTED;
     const int64_t blocks = ceil_div(a.N, 16);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+    // (the kernel takes K, the row pitch and N as 32-bit arguments and derives the
+    // packed pitch from K, as prepack does)
+    if (a.K > 0x7fffff00 || xs.ldx > 0x7fffffff || a.N > 0x7ffffff0 || a.w_kchunks != packed_kchunks(a.K))
+      return TMQ_ERR_UNSUPPORTED;
     const dim3 grid(static_cast<unsigned>(blocks)), block(kDecodeWaves * kWave);
+    const int32_t k32 = static_cast<int32_t>(a.K), ldx32 = static_cast<int32_t>(xs.ldx);
+    const int32_t n32 = static_cast<int32_t>(a.N);
+    const uint32_t flags = static_cast<uint32_t>(a.M) | (a.w_scale_stride != 0 ? 0x100u : 0u) |
+                           (a.x_xor != 0 ? 0x200u : 0u);
     switch ((a.M + 15) / 16) {
-      case 1: linear_decode_kernel<MODE, 1><<<grid, block, 0, s>>>(a, xs); break;
-      case 2: linear_decode_kernel<MODE, 2><<<grid, block, 0, s>>>(a, xs); break;
-      case 3: linear_decode_kernel<MODE, 3><<<grid, block, 0, s>>>(a, xs); break;
-      default: linear_decode_kernel<MODE, 4><<<grid, block, 0, s>>>(a, xs); break;
+      case 1: linear_decode_kernel<MODE, 1><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+      case 2: linear_decode_kernel<MODE, 2><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+      case 3: linear_decode_kernel<MODE, 3><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+      default: linear_decode_kernel<MODE, 4><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
     }
     return launch_status();
   }
