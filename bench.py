@@ -581,6 +581,43 @@ def main():
             "algorithmic_bytes_per_call": dbytes, "ops_per_call": ops}
         del xds
 
+        # --------------------- the plain-tensor op at config 3's shape, steady state
+        # quantized::linear_per_tensor takes the int8 weight as an ordinary [K, N] tensor on
+        # every call; its re-tiled copy is kept per weight tensor, so calls after the first
+        # launch the GEMM only
+        log("[bench] quantized::linear_per_tensor at config 3's shape (plain uint8 / int8 tensors)")
+        w_kn = wq.int_repr().t().contiguous()
+        x_u8 = xq.int_repr()
+        ws32 = w_scales.to(torch.float32)
+        wz32 = torch.zeros(N, dtype=torch.int32, device=dev)
+
+        def lin_plain():
+            return torch.ops.quantized.linear_per_tensor(x_u8, xq.q_scale(), xq.q_zero_point(), w_kn, ws32, wz32, bias,
+                                                         out_scale, out_zp, torch.uint8, "none", [], "")
+
+        ev_a, ev_b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev_a.record()
+        y_first = lin_plain()
+        ev_b.record()
+        torch.cuda.synchronize()
+        first_us = ev_a.elapsed_time(ev_b) * 1e3
+        assert torch.equal(y_first, torch.ops.quantized.linear(xq, packed, out_scale, out_zp).int_repr())
+        for _ in range(20):
+            lin_plain()
+        ts = events_ms(lin_plain, 50)
+        steady_us = sum(ts) / len(ts) * 1e3
+        ts = events_ms(lambda: torch.ops.quantized.linear(xq, packed, out_scale, out_zp), 50)
+        packed_us = sum(ts) / len(ts) * 1e3
+        log(f"[bench] linear_per_tensor: first call {first_us:.0f} us (re-tiles the weight), then {steady_us:.1f} us "
+            f"per call; quantized::linear with the packed weight {packed_us:.1f} us")
+        secondary["linear_per_tensor_c3_shape"] = {
+            "first_call_us": round(first_us, 1), "steady_call_us": round(steady_us, 1),
+            "quantized_linear_same_operands_us": round(packed_us, 1),
+            "value": round(ops / (steady_us * 1e-6) / 1e12, 1), "unit": "TOP/s",
+            "method": "one operand set, 50 calls timed one by one with HIP events after 20 warm-up calls; "
+                      "output bytes equal quantized::linear's"}
+        del w_kn, x_u8
+
         # -------------------------------------------------------------- C5
         log("[bench] config 5: conv2d NHWC [32,56,56,64] x [64,3,3,64]")
         xc = torch.relu(torch.randn(32, 64, 56, 56, device=dev)).contiguous(memory_format=torch.channels_last)

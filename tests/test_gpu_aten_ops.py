@@ -622,6 +622,60 @@ def test_plain_ops_errors():
     assert (y.int() - torch.clamp(torch.round(r * 128 + 128), 0, 255).int()).abs().max() <= 1
 
 
+def test_plain_ops_keep_their_packed_weight():
+    """The plain-tensor ops re-tile a weight once: a second call with the same weight, scale and
+    zero-point tensors hits the cache and gives the same bytes; an in-place change of the weight,
+    other scales, or a new tensor at a recycled address miss and give the new result."""
+    import torch_musa_amd as tm
+    say("aten plain-op weight cache")
+    tm.plain_weight_cache_clear()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(0, 255, (33, 64), dtype=torch.uint8, generator=g).cuda()
+    w = torch.randint(-127, 127, (64, 48), dtype=torch.int8, generator=g).cuda()
+    ws, wz = (torch.rand(48, generator=g) * 0.01 + 0.001).cuda(), torch.zeros(48, dtype=torch.int).cuda()
+    call = lambda w_, ws_: torch.ops.quantized.linear_per_tensor(x, 0.02, 120, w_, ws_, wz, None, 0.3, 100,
+                                                                  torch.uint8, "none", [], "")
+
+    def same(y, w_, ws_, what):
+        want = oracle.plain_linear(x.cpu().numpy(), 0.02, 120, w_.cpu().numpy(), ws_.cpu().numpy(), None, 0.3, 100,
+                                   "uint8", "none")
+        _close_to(y.cpu().numpy(), want, "uint8", what)
+
+    h0, m0, _ = tm.plain_weight_cache_counters()
+    y1 = call(w, ws)
+    y2 = call(w, ws)
+    h1, m1, e1 = tm.plain_weight_cache_counters()
+    assert (h1 - h0, m1 - m0) == (1, 1) and e1 >= 1
+    assert torch.equal(y1, y2)
+    same(y1, w, ws, "first call")
+    w[0, :] = 5                      # in place: the version counter moves, the entry no longer matches
+    y3 = call(w, ws)
+    assert tm.plain_weight_cache_counters()[1] - m1 == 1
+    same(y3, w, ws, "after an in-place change of the weight")
+    assert not torch.equal(y3, y1)
+    ws2 = ws * 2                     # other scales with the same weight
+    same(call(w, ws2), w, ws2, "other scales")
+    # a weight freed and another allocated (very likely at the same address): must not hit
+    for seed in range(3):
+        wn = torch.randint(-127, 127, (64, 48), dtype=torch.int8, generator=g).cuda()
+        same(call(wn, ws), wn, ws, f"fresh weight {seed}")
+        del wn
+    # conv: the same packed weight serves two image sizes
+    wc = torch.randint(-127, 127, (16, 16, 3, 3), dtype=torch.int8, generator=g).cuda()
+    wcs, wcz = torch.full((16,), 0.004).cuda(), torch.zeros(16, dtype=torch.int).cuda()
+    hc0 = tm.plain_weight_cache_counters()[0]
+    for hw in (9, 14, 9):
+        xc = torch.randint(0, 255, (2, 16, hw, hw), dtype=torch.uint8, generator=g).cuda()
+        yc = torch.ops.quantized.conv(xc, 0.03, 3, wc, wcs, wcz, None, [1, 1], [1, 1], [1, 1], 1, 0.5, 10,
+                                      torch.uint8, "none", [], None)
+        want = oracle.plain_conv(xc.cpu().numpy(), 0.03, 3, wc.cpu().numpy(), wcs.cpu().numpy(), None, 1, 1, 1, 0.5, 10,
+                                 "uint8", False, None, 1.0, 0)
+        _close_to(yc.contiguous().cpu().numpy(), want, "uint8", f"conv {hw}x{hw}")
+    assert tm.plain_weight_cache_counters()[0] - hc0 == 2
+    tm.plain_weight_cache_clear()
+    assert tm.plain_weight_cache_counters()[2] == 0
+
+
 def test_quantized_modules_to_device():
     # a populated CPU model (conv -> relu -> pool -> flatten -> linear, dynamic linear beside
     # it) moved to the GPU with its packed parameters; same bytes out as on the CPU

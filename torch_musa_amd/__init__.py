@@ -27,7 +27,8 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_KERNELS = os.path.join(_PKG, "libtmq.so")
 LIB_ATEN = os.path.join(_PKG, "libtmq_aten.so")
 
-__all__ = ["LIB_KERNELS", "LIB_ATEN", "is_loaded", "load", "quantized_device", "quantized_modules_to"]
+__all__ = ["LIB_KERNELS", "LIB_ATEN", "is_loaded", "load", "quantized_device", "quantized_modules_to",
+           "plain_weight_cache_clear", "plain_weight_cache_counters"]
 
 _loaded = False
 
@@ -52,6 +53,31 @@ def load() -> None:
 
 def is_loaded() -> bool:
     return _loaded
+
+
+def _aten_lib():
+    import ctypes
+
+    load()
+    lib = ctypes.CDLL(LIB_ATEN)  # already loaded by torch.ops.load_library: the same handle
+    lib.tmq_aten_plain_weight_cache_counters.argtypes = [ctypes.POINTER(ctypes.c_int64)] * 3
+    return lib
+
+
+def plain_weight_cache_clear() -> None:
+    """Drop the packed weights kept for ``quantized::linear_per_tensor`` / ``conv`` / ``conv_binary``
+    (their schemas pass the int8 weight as a plain tensor on every call; the re-tiled copy is kept
+    per weight tensor, at most 64 of them)."""
+    _aten_lib().tmq_aten_plain_weight_cache_clear()
+
+
+def plain_weight_cache_counters():
+    """-> (hits, misses, entries) of that cache."""
+    import ctypes
+
+    h, m, e = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+    _aten_lib().tmq_aten_plain_weight_cache_counters(ctypes.byref(h), ctypes.byref(m), ctypes.byref(e))
+    return h.value, m.value, e.value
 
 
 def quantized_device() -> torch.device:

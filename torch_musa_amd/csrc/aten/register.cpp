@@ -26,6 +26,9 @@
 #include <torch/library.h>
 
 #include <array>
+#include <cstdlib>
+#include <list>
+#include <mutex>
 #include <tuple>
 #include <vector>
 
@@ -986,6 +989,114 @@ at::Tensor plain_requant(const at::Tensor& r, double scale, int64_t zp, const Pl
   return at::clamp(at::round(r / scale + zp), o.is_signed ? -128 : 0, o.is_signed ? 127 : 255).to(o.dtype);
 }
 
+// ---------------------------------------------------------------------------
+// Packed weights of the plain-tensor ops.  Their schemas carry the int8 weight as
+// an ordinary tensor on every call, so the re-tiled copy, its column sums and the
+// fp32 scales are kept from one call to the next: a small most-recently-used
+// list keyed on the identity of the weight, scale and zero-point tensors
+// (storage, address, version counter, shape, strides) and on the geometry the
+// packing depends on.  An in-place change of any of the three bumps its version
+// counter and misses; a freed storage is recognised by its expired weak
+// reference, so an address that is handed out again cannot hit.  Tensors without
+// a version counter (inference mode) are never cached.  TMQ_PLAIN_WEIGHT_CACHE=0
+// in the environment turns the cache off.
+// ---------------------------------------------------------------------------
+struct TensorIdentity {
+  std::optional<c10::weak_intrusive_ptr<c10::StorageImpl>> storage;
+  const void* data = nullptr;
+  uint32_t version = 0;
+  c10::ScalarType dtype = c10::ScalarType::Undefined;
+  std::vector<int64_t> sizes, strides;
+  bool defined = false;
+
+  static bool cacheable(const at::Tensor& t) { return !t.defined() || !t.is_inference(); }
+  explicit TensorIdentity(const at::Tensor& t) {
+    if (!t.defined()) return;
+    defined = true;
+    storage = t.storage().getWeakStorageImpl();
+    data = t.const_data_ptr();
+    version = t._version();
+    dtype = t.scalar_type();
+    sizes = t.sizes().vec();
+    strides = t.strides().vec();
+  }
+  bool matches(const at::Tensor& t) const {
+    if (!t.defined()) return !defined;
+    if (!defined || storage->expired()) return false;
+    return t.const_data_ptr() == data && t._version() == version && t.scalar_type() == dtype &&
+           t.storage().unsafeGetStorageImpl() == storage->_unsafe_get_target() && t.sizes() == c10::IntArrayRef(sizes) &&
+           t.strides() == c10::IntArrayRef(strides);
+  }
+  bool alive() const { return !defined || !storage->expired(); }
+};
+
+struct PlainWeightEntry {
+  TensorIdentity weight, scales, zero_points;
+  std::array<int64_t, 8> geometry;  // what the packing depends on besides the weight (conv: taps, groups, ...)
+  at::Tensor packed, colsum, scales_f32;
+};
+
+class PlainWeightCache {
+ public:
+  static PlainWeightCache& get() {
+    static PlainWeightCache c;
+    return c;
+  }
+  bool enabled() const { return enabled_; }
+  bool find(const at::Tensor& w, const at::Tensor& sc, const at::Tensor& zp, const std::array<int64_t, 8>& geom,
+            at::Tensor* packed, at::Tensor* colsum, at::Tensor* scales_f32) {
+    std::lock_guard<std::mutex> lock(mu_);
+    for (auto it = entries_.begin(); it != entries_.end(); ++it) {
+      if (it->geometry == geom && it->weight.matches(w) && it->scales.matches(sc) && it->zero_points.matches(zp)) {
+        entries_.splice(entries_.begin(), entries_, it);  // most recently used first
+        *packed = it->packed;
+        *colsum = it->colsum;
+        *scales_f32 = it->scales_f32;
+        ++hits_;
+        return true;
+      }
+    }
+    ++misses_;
+    return false;
+  }
+  void insert(const at::Tensor& w, const at::Tensor& sc, const at::Tensor& zp, const std::array<int64_t, 8>& geom,
+              const at::Tensor& packed, const at::Tensor& colsum, const at::Tensor& scales_f32) {
+    std::lock_guard<std::mutex> lock(mu_);
+    entries_.remove_if([](const PlainWeightEntry& e) {
+      return !(e.weight.alive() && e.scales.alive() && e.zero_points.alive());
+    });
+    entries_.push_front(PlainWeightEntry{TensorIdentity(w), TensorIdentity(sc), TensorIdentity(zp), geom, packed,
+                                         colsum, scales_f32});
+    while (entries_.size() > kMaxEntries) entries_.pop_back();
+  }
+  void clear() {
+    std::lock_guard<std::mutex> lock(mu_);
+    entries_.clear();
+  }
+  void counters(int64_t* hits, int64_t* misses, int64_t* entries) {
+    std::lock_guard<std::mutex> lock(mu_);
+    *hits = hits_;
+    *misses = misses_;
+    *entries = static_cast<int64_t>(entries_.size());
+  }
+
+ private:
+  PlainWeightCache() {
+    const char* e = std::getenv("TMQ_PLAIN_WEIGHT_CACHE");
+    enabled_ = !(e != nullptr && e[0] == '0');
+  }
+  static constexpr size_t kMaxEntries = 64;
+  std::mutex mu_;
+  std::list<PlainWeightEntry> entries_;
+  int64_t hits_ = 0, misses_ = 0;
+  bool enabled_ = true;
+};
+
+bool plain_cacheable(const at::Tensor& w, const at::Tensor& sc, const at::Tensor& zp) {
+  return PlainWeightCache::get().enabled() && TensorIdentity::cacheable(w) && TensorIdentity::cacheable(sc) &&
+         TensorIdentity::cacheable(zp);
+}
+
 at::Tensor qlinear_per_tensor_run(at::Tensor act, double act_scale, int64_t act_zero_point, at::Tensor weight,
                                   at::Tensor weight_scales, at::Tensor weight_zero_points,
                                   std::optional<at::Tensor> bias, double output_scale, int64_t output_zero_point,
@@ -1004,7 +1115,6 @@ at::Tensor qlinear_per_tensor_run(at::Tensor act, double act_scale, int64_t act_
   TORCH_CHECK(weight.size(0) == K, what, ": weight is [", weight.size(0), ", ", N, "], the input has ", K, " features");
   TORCH_CHECK(act_scale > 0 && output_scale > 0, what, ": scales must be positive");
   const PlainOut o = plain_out(output_dtype, act.scalar_type(), what);
-  const at::Tensor ws = plain_weight_scales(weight_scales, weight_zero_points, N, act, what);
   std::optional<at::Tensor> b;
   if (bias.has_value() && bias->defined()) {
     TORCH_CHECK(bias->numel() == N, what, ": bias must have ", N, " elements");
@@ -1013,14 +1123,23 @@ at::Tensor qlinear_per_tensor_run(at::Tensor act, double act_scale, int64_t act_
   const bool float_path = !o.is_int || post == "tanh" || post == "gelu";
   at::Tensor y = float_path ? at::empty({M, N}, act.options().dtype(at::kFloat))
                             : at::empty({M, N}, act.options().dtype(o.dtype));
-  if (y.numel() == 0) return float_path ? plain_requant(y, output_scale, output_zero_point, o) : y;
   const auto stream = current_stream(act);
   const at::Tensor x = act.contiguous();
-  const at::Tensor w_nk = weight.t().contiguous();  // [N, K], the layout the prepack reads
-  at::Tensor packed = at::empty({std::max<int64_t>(tmq_linear_packed_bytes(N, K), 16)}, act.options().dtype(at::kByte));
-  at::Tensor colsum = at::empty({N}, act.options().dtype(at::kInt));
-  check_status(tmq_linear_prepack(cptr<int8_t>(w_nk), N, K, K, packed.data_ptr(), mptr<int32_t>(colsum), stream),
-               "tmq_linear_prepack");
+  if (y.numel() == 0) return float_path ? plain_requant(y, output_scale, output_zero_point, o) : y;
+  // weight side: re-tiled copy, column sums and fp32 scales, made once per weight
+  at::Tensor packed, colsum, ws;
+  const std::array<int64_t, 8> geom{0, N, K, act.device().index(), 0, 0, 0, 0};
+  const bool cacheable = plain_cacheable(weight, weight_scales, weight_zero_points);
+  if (!cacheable || !PlainWeightCache::get().find(weight, weight_scales, weight_zero_points, geom, &packed, &colsum, &ws)) {
+    ws = plain_weight_scales(weight_scales, weight_zero_points, N, act, what);
+    packed = at::empty({std::max<int64_t>(tmq_linear_packed_bytes(N, K), 16)}, act.options().dtype(at::kByte));
+    colsum = at::empty({N}, act.options().dtype(at::kInt));
+    const at::Tensor w_nk = weight.t().contiguous();  // [N, K], the layout the prepack reads
+    check_status(tmq_linear_prepack(cptr<int8_t>(w_nk), N, K, K, packed.data_ptr(), mptr<int32_t>(colsum), stream),
+                 "tmq_linear_prepack");
+    if (cacheable)
+      PlainWeightCache::get().insert(weight, weight_scales, weight_zero_points, geom, packed, colsum, ws);
+  }
   tmq_linear_desc d{};
   d.M = M;
   d.N = N;
@@ -1086,7 +1205,6 @@ at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero
   g.groups = groups;
   TORCH_CHECK(groups > 0 && g.OC % groups == 0 && g.IC == weight.size(1) * groups, what, ": input has ", g.IC,
               " channels, weight expects ", weight.size(1) * groups, " in ", groups, " groups");
-  const at::Tensor ws = plain_weight_scales(weight_scales, weight_zero_points, g.OC, act, what);
   std::optional<at::Tensor> b;
   if (bias.has_value() && bias->defined()) {
     TORCH_CHECK(bias->numel() == g.OC, what, ": bias must have ", g.OC, " elements");
@@ -1097,12 +1215,22 @@ at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero
   TORCH_CHECK(OH > 0 && OW > 0, what, ": the kernel does not fit the padded input");
   const auto stream = current_stream(act);
   const at::Tensor x = act.contiguous(c10::MemoryFormat::ChannelsLast);
-  const at::Tensor w_ohwi = weight.permute({0, 2, 3, 1}).contiguous();
-  at::Tensor packed = at::empty({std::max<int64_t>(tmq_conv2d_packed_bytes(&g), 16)}, act.options().dtype(at::kByte));
-  at::Tensor colsum = at::empty({g.OC}, act.options().dtype(at::kInt));
-  if (g.B > 0)
-    check_status(tmq_conv2d_prepack(cptr<int8_t>(w_ohwi), &g, packed.data_ptr(), mptr<int32_t>(colsum), stream),
-                 "tmq_conv2d_prepack");
+  // weight side: re-tiled copy, column sums and fp32 scales, made once per weight (the
+  // packing depends on the weight's shape and the group count, not on the image)
+  at::Tensor packed, colsum, ws;
+  const std::array<int64_t, 8> geom{1, g.OC, g.IC, g.KH, g.KW, g.groups, act.device().index(), 0};
+  const bool cacheable = g.B > 0 && plain_cacheable(weight, weight_scales, weight_zero_points);
+  if (!cacheable || !PlainWeightCache::get().find(weight, weight_scales, weight_zero_points, geom, &packed, &colsum, &ws)) {
+    ws = plain_weight_scales(weight_scales, weight_zero_points, g.OC, act, what);
+    const at::Tensor w_ohwi = weight.permute({0, 2, 3, 1}).contiguous();
+    packed = at::empty({std::max<int64_t>(tmq_conv2d_packed_bytes(&g), 16)}, act.options().dtype(at::kByte));
+    colsum = at::empty({g.OC}, act.options().dtype(at::kInt));
+    if (g.B > 0)
+      check_status(tmq_conv2d_prepack(cptr<int8_t>(w_ohwi), &g, packed.data_ptr(), mptr<int32_t>(colsum), stream),
+                   "tmq_conv2d_prepack");
+    if (cacheable)
+      PlainWeightCache::get().insert(weight, weight_scales, weight_zero_points, geom, packed, colsum, ws);
+  }
   d.x = x.data_ptr();
   d.x_signed = x_signed;
   d.x_zero_point = static_cast<int32_t>(act_zero_point);
@@ -1283,3 +1411,14 @@ struct MuteOff {
   MuteOff() { c10::WarningUtils::set_warning_handler(g_mute_on.previous); }
 } const g_mute_off;
 }  // namespace
+
+// Controls of the packed-weight cache of the plain-tensor ops (ctypes, for tests
+// and for callers that want the memory back).
+extern "C" __attribute__((visibility("default"))) void tmq_aten_plain_weight_cache_clear() {
+  PlainWeightCache::get().clear();
+}
+extern "C" __attribute__((visibility("default"))) void tmq_aten_plain_weight_cache_counters(int64_t* hits,
+                                                                                             int64_t* misses,
+                                                                                             int64_t* entries) {
+  PlainWeightCache::get().counters(hits, misses, entries);
+}
