@@ -269,7 +269,8 @@ def main():
         log("[bench] int8 MFMA ceiling probe (register-only loop, 256 workgroups)")
         probe = {}
         for mode, name in ((0, "zero_operands"), (1, "uniform_random_int8"), (2, "gaussian_int8"),
-                           (3, "gaussian_int8_fresh_from_lds")):
+                           (3, "gaussian_int8_fresh_from_lds"), (4, "gaussian_int8_one_operand_non_negative"),
+                           (5, "gaussian_int8_16x16x64")):
             tops_p, ghz_p = cabi.probe_mfma_i8(mode)
             probe[name] = {"tops": round(tops_p, 1), "shader_ghz": round(ghz_p, 3)}
             log(f"[bench]   {name}: {tops_p:.0f} TOP/s at {ghz_p:.2f} GHz")

@@ -17,7 +17,10 @@ extern "C" {
  * waves and reports the sustained rate in TOP/s and the shader clock in GHz.
  * data_mode 0: zero operands, 1: uniform random bytes, 2: Gaussian int8 (all
  * held in registers), 3: Gaussian int8 operands read afresh from LDS for every
- * instruction, eight waves per workgroup (the GEMM's loop without its copies).
+ * instruction, eight waves per workgroup (the GEMM's loop without its copies),
+ * 4: as 2 with the sign bits of the second operand cleared (what the part
+ * sustains depends on how much the operands toggle, sign extension included),
+ * 5: as 2 on v_mfma_i32_16x16x64_i8.
  * The call synchronises (default stream) and creates two HIP events; status
  * codes are tmq.h's; `scratch` is >= 2 KiB of device memory.
  * ------------------------------------------------------------------------- */

@@ -32,7 +32,8 @@ __device__ __forceinline__ unsigned gaussian_bytes(unsigned seed) {
 }
 
 // data_mode 0: zeros, 1: uniform random bytes, 2: Gaussian int8 (sigma ~37),
-// all three held in registers for the whole run
+// 4: Gaussian int8 with the second operand's sign bits cleared (non-negative
+// values), all held in registers for the whole run
 __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int data_mode, int* sink,
                                                          long long* stamps) {
   v16i acc[8];
@@ -48,10 +49,11 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int data_mod
     for (int j = 0; j < 4; ++j) {
       unsigned ra = mix(seed + i * 8 + j), rb = mix(seed + 1000 + i * 8 + j);
       if (data_mode == 0) ra = rb = 0;
-      if (data_mode == 2) {
+      if (data_mode == 2 || data_mode == 4) {
         ra = gaussian_bytes(ra);
         rb = gaussian_bytes(rb);
       }
+      if (data_mode == 4) rb &= 0x7f7f7f7fu;
       a[i][j] = static_cast<int>(ra);
       b[i][j] = static_cast<int>(rb);
     }
@@ -71,6 +73,37 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, int data_mod
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     stamps[0] = c1 - c0;  // shader clock cycles
     stamps[1] = w1 - w0;  // 100 MHz ticks
+  }
+}
+
+// data_mode 5: the same register-only loop on v_mfma_i32_16x16x64_i8, Gaussian int8
+__global__ __launch_bounds__(256) void mfma_probe_16x16_kernel(int iters, int* sink, long long* stamps) {
+  v4i acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = v4i{0, 0, 0, 0};
+  v4i a[4], b[4];
+  const unsigned seed = threadIdx.x * 977u + blockIdx.x * 131071u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a[i][j] = static_cast<int>(gaussian_bytes(mix(seed + i * 8 + j)));
+      b[i][j] = static_cast<int>(gaussian_bytes(mix(seed + 1000 + i * 8 + j)));
+    }
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i & 3], b[(i >> 2) & 3], acc[i], 0, 0, 0);
+  }
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += acc[i].x + acc[i].y + acc[i].z + acc[i].w;
+  if (s == 0x7fffffff) sink[threadIdx.x] = s;
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    stamps[0] = c1 - c0;
+    stamps[1] = w1 - w0;
   }
 }
 
@@ -137,7 +170,7 @@ using namespace tmq;
 // least 2 KiB owned by the caller.
 TMQ_EXPORT int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, double* tops,
                                  double* shader_ghz) {
-  if (data_mode < 0 || data_mode > 3 || blocks <= 0 || iters <= 0 || scratch == nullptr ||
+  if (data_mode < 0 || data_mode > 5 || blocks <= 0 || iters <= 0 || scratch == nullptr ||
       tops == nullptr || shader_ghz == nullptr)
     return TMQ_ERR_INVALID_ARGUMENT;
   int* sink = static_cast<int*>(scratch);
@@ -147,11 +180,14 @@ TMQ_EXPORT int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scr
   // mode 3: eight waves per block and 16 MFMAs per wave and iteration: half the
   // iterations give the same number of operations per block as the other modes
   const int it3 = iters / 4 > 0 ? iters / 4 : 1;
-  if (data_mode == 3) mfma_probe_lds_kernel<<<dim3(blocks), dim3(512), 0, nullptr>>>(it3, sink, stamps);
-  else mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
+  auto launch = [&]() {
+    if (data_mode == 3) mfma_probe_lds_kernel<<<dim3(blocks), dim3(512), 0, nullptr>>>(it3, sink, stamps);
+    else if (data_mode == 5) mfma_probe_16x16_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, sink, stamps);
+    else mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
+  };
+  launch();
   hipEventRecord(e0, nullptr);
-  if (data_mode == 3) mfma_probe_lds_kernel<<<dim3(blocks), dim3(512), 0, nullptr>>>(it3, sink, stamps);
-  else mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(iters, data_mode, sink, stamps);
+  launch();
   hipEventRecord(e1, nullptr);
   int rc = hipEventSynchronize(e1) == hipSuccess ? TMQ_OK : TMQ_ERR_LAUNCH;
   float ms = 0.f;
@@ -162,6 +198,7 @@ TMQ_EXPORT int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scr
   hipEventDestroy(e0);
   hipEventDestroy(e1);
   if (rc != TMQ_OK) return rc;
+  // (mode 5: 16 instructions of 16 x 16 x 64 per iteration are the operations of 8 of 32 x 32 x 32)
   const double ops = data_mode == 3 ? 2.0 * 32 * 32 * 32 * 16 * static_cast<double>(it3) * 8 * blocks
                                     : 2.0 * 32 * 32 * 32 * 8 * static_cast<double>(iters) * 4 * blocks;
   *tops = ops / (ms * 1e-3) / 1e12;

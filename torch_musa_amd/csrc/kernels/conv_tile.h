@@ -13,8 +13,10 @@
 //
 // LDS layout (byte offsets from the dynamic LDS base):
 //   weights  [k-chunk][64 rows][16 B]          (the packed order, rows of this tile)
-//   halo     [HH*HW pixels][pitch], pitch = ICg rounded up to an odd number of
-//            16-byte slots: 16 consecutive pixels then fall into distinct bank groups
+//   halo     [HH rows][ri slots of 16 B]: HW pixels of `pitch` bytes (ICg rounded up to an
+//            odd number of slots: 16 consecutive pixels fall into distinct bank groups),
+//            then padding slots chosen so that a row tile that crosses patch rows keeps
+//            that property
 //   staging  8 waves x [32 pixels][80 B] for the row-major output transpose
 //   taps     int32[2*(KS+4)]: halo byte offset of every 16-byte k-chunk
 //
@@ -48,7 +50,7 @@ struct ConvTileArgs {
   int sh, sw, ph, pw, dh, dw;
   int ICg, OCg, n_tiles;     // n_tiles = 64-channel tiles per group
   int TH, TW, HH, HW, pitch;
-  int ri, rpp;               // 16-byte LDS slots per halo row (<= 512), halo rows per pass of the block
+  int ri, rpp;               // 16-byte LDS slots per halo row (<= 512; the last ones may be padding), halo rows per pass of the block
   int cx;                    // passes over the halo
   uint32_t xstep;            // image bytes between a thread's successive halo items
   int xdstep;                // and the LDS bytes between them
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
     const int pslots = a.pitch >> 4;  // slots per pixel
     const int lr = static_cast<int>(small_div(t, a.ri, a.rcp_ri)), it = t - lr * a.ri;
     const int hc = static_cast<int>(small_div(it, pslots, a.rcp_pslots)), hb = it - hc * pslots;
-    const bool active = lr < a.rpp && hb < a.icb;
+    const bool active = lr < a.rpp && hb < a.icb && hc < a.HW;
     const bool col_ok = static_cast<unsigned>(iw0 + hc) < static_cast<unsigned>(a.W);
     // byte offset inside the image; wraps harmlessly where it is not used
     uint32_t xoff = (static_cast<uint32_t>(ih0 + lr) * static_cast<uint32_t>(a.W) +
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       wave_dst += a.xdstep;
     }
     // Halo byte offset of the two 16-byte k-chunks of every k-step: chunk
-    // c = tap * icb + blk lies at ((kh*dil_h)*HW + kw*dil_w) * pitch + blk*16.
+    // c = tap * icb + blk lies at (kh*dil_h) * row bytes + (kw*dil_w) * pitch + blk*16.
     // Chunks past the last tap carry zero weights and read pixel 0; the k loop
     // reads three steps past the end.
     int* const s_tab = reinterpret_cast<int*>(lds + a.lds_tab);
@@ -178,7 +180,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       if (c < a.kchunks) {
         const int tap = static_cast<int>(small_div(c, a.icb, a.rcp_icb)), blk = c - tap * a.icb;
         const int kh = static_cast<int>(small_div(tap, a.KW, a.rcp_kw)), kw = tap - kh * a.KW;
-        off = (kh * a.dh * a.HW + kw * a.dw) * a.pitch + blk * 16;
+        off = kh * a.dh * (a.ri * 16) + kw * a.dw * a.pitch + blk * 16;
       }
       s_tab[c] = off;
     }
@@ -237,7 +239,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       m = in_tile ? m : TP - 1;
       const int r = static_cast<int>(small_div(static_cast<uint32_t>(m), static_cast<uint32_t>(a.TW), a.rcp_tw));
       const int c = m - r * a.TW;
-      xb[tm] = (r * a.sh * a.HW + c * a.sw) * a.pitch;
+      xb[tm] = r * a.sh * (a.ri * 16) + c * a.sw * a.pitch;
       const int oh = oh0 + r, ow = ow0 + c;
       opix[tm] = (in_tile && oh < a.OH && ow < a.OW) ? img_pix + oh * a.OW + ow : -1;
     }
