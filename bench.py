@@ -49,6 +49,11 @@ MEASURED_TRAFFIC = {
 }
 
 
+PROBE_MODES = ((0, "zero_operands"), (1, "uniform_random_int8"), (2, "gaussian_int8"),
+               (3, "gaussian_int8_fresh_from_lds"), (4, "gaussian_int8_one_operand_non_negative"),
+               (5, "gaussian_int8_16x16x64"))
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -61,7 +66,7 @@ def main():
     ap.add_argument("--skip-secondary", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
-                                       "dequantize_pc", "decode", "conv", "conv_add_relu"],
+                                       "dequantize_pc", "decode", "conv", "conv_add_relu", "probe"],
                     help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
                          "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
                          "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
@@ -119,6 +124,16 @@ def main():
             fn()
         torch.cuda.synchronize()
         print(json.dumps({"only": args.only, "launches": args.steps, "elements": n}))
+        return
+
+    if args.only == "probe":
+        # the int8 MFMA ceiling probes alone (for counter runs: matrix-pipe busy cycles and
+        # shader clock of a loop that does nothing but multiply)
+        res = {}
+        for mode, name in PROBE_MODES:
+            tops_p, ghz_p = cabi.probe_mfma_i8(mode)
+            res[name] = {"tops": round(tops_p, 1), "shader_ghz": round(ghz_p, 3)}
+        print(json.dumps({"only": "probe", "modes": res}))
         return
 
     def per_channel_sets(nsets):
@@ -268,9 +283,7 @@ def main():
         # ---------------------------------------------- matrix-pipe ceiling probe
         log("[bench] int8 MFMA ceiling probe (register-only loop, 256 workgroups)")
         probe = {}
-        for mode, name in ((0, "zero_operands"), (1, "uniform_random_int8"), (2, "gaussian_int8"),
-                           (3, "gaussian_int8_fresh_from_lds"), (4, "gaussian_int8_one_operand_non_negative"),
-                           (5, "gaussian_int8_16x16x64")):
+        for mode, name in PROBE_MODES:
             tops_p, ghz_p = cabi.probe_mfma_i8(mode)
             probe[name] = {"tops": round(tops_p, 1), "shader_ghz": round(ghz_p, 3)}
             log(f"[bench]   {name}: {tops_p:.0f} TOP/s at {ghz_p:.2f} GHz")
