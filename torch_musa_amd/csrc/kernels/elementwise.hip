@@ -318,6 +318,43 @@ __global__ __launch_bounds__(kEwThreads) void qmaxpool_k3_kernel(const uint8_t* 
   }
 }
 
+// The same 3x3 window with the output row in the block index: blockIdx.y = oh,
+// blockIdx.z = image, threads over (ow, group of 16 channels), 32-bit arithmetic
+// and one division per thread -- the flat kernel above spends most of its
+// instructions on five 64-bit divisions per output.  The host sends shapes here
+// whose byte offsets inside one image fit 31 bits.
+template <bool SIGNED>
+__global__ __launch_bounds__(kEwThreads) void qmaxpool_k3_rows_kernel(const uint8_t* __restrict__ x,
+                                                                      uint8_t* __restrict__ y, int H, int W, int C,
+                                                                      int OH, int OW, int sh, int sw, int ph, int pw) {
+  const int cv = C >> 4;
+  const int idx = static_cast<int>(blockIdx.x) * kEwThreads + threadIdx.x;
+  if (idx >= OW * cv) return;
+  const int ow = idx / cv, c = (idx - ow * cv) << 4;
+  const int oh = blockIdx.y;
+  const int64_t b = blockIdx.z;
+  const int ih0 = oh * sh - ph, iw0 = ow * sw - pw;
+  const uint8_t* img = x + b * (static_cast<int64_t>(H) * W * C) + c;
+  const int lowest = static_cast<int>(SIGNED ? 0x80808080u : 0u);
+  v4i v[9];
+  bool ok[9];
+#pragma unroll
+  for (int k = 0; k < 9; ++k) {
+    const int ih = ih0 + k / 3, iw = iw0 + k % 3;
+    ok[k] = ih >= 0 && ih < H && iw >= 0 && iw < W;
+    const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih), iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);
+    v[k] = *reinterpret_cast<const v4i*>(img + (ihc * W + iwc) * C);
+  }
+  v4i m = {lowest, lowest, lowest, lowest};
+#pragma unroll
+  for (int k = 0; k < 9; ++k) {
+    const v4i u = ok[k] ? v[k] : v4i{lowest, lowest, lowest, lowest};
+    m = v4i{static_cast<int>(max_codes4<SIGNED>(m.x, u.x)), static_cast<int>(max_codes4<SIGNED>(m.y, u.y)),
+            static_cast<int>(max_codes4<SIGNED>(m.z, u.z)), static_cast<int>(max_codes4<SIGNED>(m.w, u.w))};
+  }
+  *reinterpret_cast<v4i*>(y + ((b * OH + oh) * OW + ow) * static_cast<int64_t>(C) + c) = m;
+}
+
 // Adaptive average pooling: output pixel (oh, ow) averages the input window
 // rows floor(oh*H/OH) .. ceil((oh+1)*H/OH)-1 (likewise columns).  VEC = 4: a
 // thread owns four consecutive channels (one 32-bit word per input pixel).
@@ -560,7 +597,17 @@ TMQ_EXPORT int tmq_qmaxpool2d(const void* x, void* y, int64_t B, int64_t H, int6
   hipStream_t hs = as_stream(stream);
   const uint8_t* xb = static_cast<const uint8_t*>(x);
   uint8_t* yb = static_cast<uint8_t*>(y);
-  if (vec && kh == 3 && kw == 3 && dil_h == 1 && dil_w == 1) {
+  if (vec && kh == 3 && kw == 3 && dil_h == 1 && dil_w == 1 && H * W * C < (int64_t{1} << 31) && OH <= 65535 &&
+      B <= 65535 && OW * (C / 16) < (int64_t{1} << 30)) {
+    const dim3 rgrid(static_cast<unsigned>(ceil_div(OW * (C / 16), kEwThreads)), static_cast<unsigned>(OH),
+                     static_cast<unsigned>(B));
+    const int h = static_cast<int>(H), w = static_cast<int>(W), c = static_cast<int>(C);
+    const int oh = static_cast<int>(OH), ow = static_cast<int>(OW);
+    if (q_signed)
+      qmaxpool_k3_rows_kernel<true><<<rgrid, block, 0, hs>>>(xb, yb, h, w, c, oh, ow, stride_h, stride_w, pad_h, pad_w);
+    else
+      qmaxpool_k3_rows_kernel<false><<<rgrid, block, 0, hs>>>(xb, yb, h, w, c, oh, ow, stride_h, stride_w, pad_h, pad_w);
+  } else if (vec && kh == 3 && kw == 3 && dil_h == 1 && dil_w == 1) {
     if (q_signed) qmaxpool_k3_kernel<true><<<grid, block, 0, hs>>>(xb, yb, s);
     else qmaxpool_k3_kernel<false><<<grid, block, 0, hs>>>(xb, yb, s);
   } else if (vec) {
