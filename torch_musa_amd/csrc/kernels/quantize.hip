@@ -626,8 +626,9 @@ struct PcfDequantize {
 // for the quantizers, four for the dequantizers (at fp32 [11008, 4096], axis 0:
 // quantize 42.5 / 40.5 / 38.4 / 40.4 us with 2 / 4 / 8 / 16, dequantize 33.8 / 33.4 /
 // 36.0 / 38.7 us).
+constexpr int kPcThreads = 256;  // 64 ... 512 threads per block measure within 3 % of each other
 template <class Op, int VEC>
-__global__ __launch_bounds__(kThreads) void pc_rows_kernel(Op op, int64_t rows, int64_t C, int64_t inner,
+__global__ __launch_bounds__(kPcThreads) void pc_rows_kernel(Op op, int64_t rows, int64_t C, int64_t inner,
                                                            int lg_us, uint32_t segs) {
   using In = std::conditional_t<VEC == 4, typename Op::In4, typename Op::In1>;
   constexpr int kPcAccesses = Op::kAccesses;
@@ -635,13 +636,13 @@ __global__ __launch_bounds__(kThreads) void pc_rows_kernel(Op op, int64_t rows, 
   const int us_mask = (1 << lg_us) - 1;
   const int64_t row0 = static_cast<int64_t>(rg) * (kPcAccesses >> lg_us);
   const int64_t c0 = row0 % C;  // once per block, wave-uniform
-  const int64_t col0 = (static_cast<int64_t>(seg) << lg_us) * (kThreads * VEC) + threadIdx.x * VEC;
+  const int64_t col0 = (static_cast<int64_t>(seg) << lg_us) * (kPcThreads * VEC) + threadIdx.x * VEC;
   In held[kPcAccesses];
   bool live[kPcAccesses];
 #pragma unroll
   for (int u = 0; u < kPcAccesses; ++u) {
     const int64_t row = row0 + (u >> lg_us);
-    const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kThreads * VEC);
+    const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kPcThreads * VEC);
     live[u] = row < rows && col < inner;
     if (live[u]) {
       if constexpr (VEC == 4) held[u] = op.load4(row * inner + col);
@@ -655,7 +656,7 @@ __global__ __launch_bounds__(kThreads) void pc_rows_kernel(Op op, int64_t rows, 
     int64_t c = c0 + (u >> lg_us);
     while (c >= C) c -= C;   // at most A - 1 rows past c0: uniform, a few scalar steps
     const typename Op::P p = op.params(c);
-    const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kThreads * VEC);
+    const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kPcThreads * VEC);
     if (live[u]) {
       if constexpr (VEC == 4) op.store4(row * inner + col, held[u], p);
       else op.store1(row * inner + col, held[u], p);
@@ -669,7 +670,7 @@ template <class Op>
 bool launch_pc_rows(const Op& op, int64_t outer, int64_t C, int64_t inner, bool vec, hipStream_t s) {
   if (inner < kPcRowsMinInner) return false;
   constexpr int kPcAccesses = Op::kAccesses;
-  const int64_t per_run = kThreads * (vec ? 4 : 1);
+  const int64_t per_run = kPcThreads * (vec ? 4 : 1);
   int lg_us = 0;
   while ((2 << lg_us) <= kPcAccesses && (per_run << lg_us) < inner) ++lg_us;
   const int64_t rows = outer * C;
@@ -678,9 +679,9 @@ bool launch_pc_rows(const Op& op, int64_t outer, int64_t C, int64_t inner, bool 
   if (segs > 0x7fffffff || row_groups > 0x7fffffff / segs) return false;
   const dim3 grid(static_cast<unsigned>(row_groups * segs));
   if (vec)
-    pc_rows_kernel<Op, 4><<<grid, dim3(kThreads), 0, s>>>(op, rows, C, inner, lg_us, static_cast<uint32_t>(segs));
+    pc_rows_kernel<Op, 4><<<grid, dim3(kPcThreads), 0, s>>>(op, rows, C, inner, lg_us, static_cast<uint32_t>(segs));
   else
-    pc_rows_kernel<Op, 1><<<grid, dim3(kThreads), 0, s>>>(op, rows, C, inner, lg_us, static_cast<uint32_t>(segs));
+    pc_rows_kernel<Op, 1><<<grid, dim3(kPcThreads), 0, s>>>(op, rows, C, inner, lg_us, static_cast<uint32_t>(segs));
   return true;
 }
 
