@@ -37,15 +37,24 @@ PEAK_INT8_TOPS = 5000.0   # dense int8 MFMA, 5.0 POP/s
 PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
-# dispatch, one run each: `rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --only linear --steps 3`).
+# dispatch, one run each: `rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --only linear --steps 6`).
 # Calibration against a plain 1 GiB device copy (`--only copy`): FETCH_SIZE reads 524 300 for
 # 1 048 576 KiB actually read (factor 2.0), WRITE_SIZE reads 1 048 576 (factor 1.0).
 # Summaries: profiles/hbm_traffic_pmc.md.
+def _traffic(fetch_kib, write_kib):
+    return int((fetch_kib * 2.0 + write_kib) * 1024)
+
+
 MEASURED_TRAFFIC = {
-    "linear_c3": int((161_100 * 2.0 + 44_030) * 1024),      # 375 MB: operands re-fetched 5.3x by the 8 L2s
-    "quantize_c2": int((524_300 * 2.0 + 262_100) * 1024),   # 1.342 GB = algorithmic
-    "dequantize_c2": int((131_100 * 2.0 + 1_049_000) * 1024),
-    "minmax_c2": int((524_300 * 2.0 + 64) * 1024),
+    "linear_c3": _traffic(161_134, 44_033),       # 375 MB: operands re-fetched 5.3x by the 8 L2s
+    "quantize_c2": _traffic(524_304, 262_144),    # 1.342 GB = algorithmic
+    "dequantize_c2": _traffic(131_084, 1_048_988),
+    "minmax_c2": _traffic(524_312, 64),
+    "quantize_pc": _traffic(88_805, 44_032),
+    "dequantize_pc": _traffic(23_422, 176_241),
+    "decode_m1": _traffic(8_299, 8),              # 17.0 MB for 16.8 MB algorithmic
+    "conv_c5": _traffic(4_163, 6_272),            # 14.9 MB for 12.9 MB algorithmic (halo overlap)
+    "conv_add_relu_c5": _traffic(7_560, 6_272),
 }
 
 
@@ -272,7 +281,7 @@ def main():
         f"timed region), {achieved:.0f} TOP/s; {iso_ms*1e3:.1f} us/launch when launches are timed one by one")
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                 "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": MEASURED_TRAFFIC["linear_c3"],
-                "kernel": "tmq::gemm_i8_kernel", "ops_per_launch": ops,
+                "kernel": "tmq::gemm_i8_persistent_kernel", "ops_per_launch": ops,
                 "avg_launch_us": round(kern_ms * 1e3, 2),
                 "isolated_launch_us": round(iso_ms * 1e3, 2),
                 "algorithmic_bytes_per_launch": M * K + N * K + M * N + 12 * N,
@@ -362,7 +371,7 @@ def main():
                        "tmq_quantize_per_channel")
 
         npc = 11008 * 4096
-        hbm("quantize_per_channel_11008x4096", quantize_pc_kernel, 5 * npc + 16 * 11008, None)
+        hbm("quantize_per_channel_11008x4096", quantize_pc_kernel, 5 * npc + 16 * 11008, "quantize_pc")
 
         def quantize_pc_op():
             pc_count[0] += 1
@@ -383,7 +392,7 @@ def main():
                                                       sc_.data_ptr(), zp_.data_ptr(), 1, cabi.stream_ptr()),
                        "tmq_dequantize_per_channel")
 
-        hbm("dequantize_per_channel_11008x4096", dequantize_pc_kernel, 5 * npc + 16 * 11008, None)
+        hbm("dequantize_per_channel_11008x4096", dequantize_pc_kernel, 5 * npc + 16 * 11008, "dequantize_pc")
         del pcs, pc_out, pc_r
 
         # -------------------------------------------------------------- C1
@@ -477,7 +486,8 @@ def main():
             secondary[f"linear_decode_m{Md}"] = {
                 "avg_launch_us": round(per * 1e3, 3), "value": round(gbs, 1), "unit": "GB/s",
                 "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
+                             "frac": round(gbs / PEAK_HBM_GBS, 4),
+                             "traffic": MEASURED_TRAFFIC["decode_m1"] if Md == 1 else None},
                 "frac_of_read_only_kernel": round(read_us / (per * 1e3), 4),
                 "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
                 "algorithmic_bytes_per_launch": nbytes}
@@ -684,7 +694,8 @@ def main():
             "value": round(cops / (avg * 1e-3) / 1e12, 1), "unit": "TOP/s",
             "roofline": {"bound": "mfma", "achieved": round(cops / (avg * 1e-3) / 1e12, 1),
                          "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                         "frac": round(cops / (avg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "traffic": None},
+                         "frac": round(cops / (avg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4),
+                         "traffic": MEASURED_TRAFFIC["conv_c5"]},
             "hbm_frac": round(cbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
             "method": f"{reps} launches over {csets} rotating inputs replayed back to back in one HIP graph",
             "algorithmic_bytes_per_launch": cbytes, "ops_per_launch": cops}
@@ -724,7 +735,8 @@ def main():
             "avg_launch_us": round(favg * 1e3, 2), "value": round(cops / (favg * 1e-3) / 1e12, 1), "unit": "TOP/s",
             "roofline": {"bound": "mfma", "achieved": round(cops / (favg * 1e-3) / 1e12, 1),
                          "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                         "frac": round(cops / (favg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "traffic": None},
+                         "frac": round(cops / (favg * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4),
+                         "traffic": MEASURED_TRAFFIC["conv_add_relu_c5"]},
             "hbm_frac": round(fbytes / (favg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
             "method": f"{reps} launches over {csets} rotating inputs and residuals replayed in one HIP graph",
             "algorithmic_bytes_per_launch": fbytes, "ops_per_launch": cops}
