@@ -124,6 +124,16 @@ def test_persistent_rounds(cabi, shape, x_signed, relu, pc):
         finally:
             cabi.force_linear_config(-1)
         _check(y, want, f"cfg {cfg}")
+    # the same tiles with float output (the product inside a dynamically quantized linear)
+    wantf = oracle.linear_f32(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], relu=relu,
+                              nthreads=8)
+    for cfg in (20, -1):
+        cabi.force_linear_config(cfg)
+        try:
+            yf = host(cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, relu=relu))
+        finally:
+            cabi.force_linear_config(-1)
+        np.testing.assert_array_equal(yf, wantf, err_msg=f"float output, cfg {cfg}")
 
 
 # wave groups that split the k loop inside a block (stage counts the group count divides)
@@ -337,7 +347,7 @@ def test_split_k_workspace_rules(cabi):
 # Float results are compared bit for bit: the kernel's epilogue is the oracle's
 # single fused multiply-add, and the dynamic quantization in front of it is
 # bit-exact by the quantizer tests.
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20])
 @pytest.mark.parametrize("shape,relu,bias,pc,x_signed", [((60, 264, 448), False, True, True, False),
                                                          ((257, 33, 144), True, True, False, False),
                                                          ((16, 1040, 1168), False, False, True, True)])

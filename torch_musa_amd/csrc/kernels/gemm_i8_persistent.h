@@ -19,7 +19,8 @@
 //     written while the current tile's are still being read).
 //
 // LDS map (bytes): weights 3 x 16 KB | activation pairs 3 x 32 KB | constants
-// 2 x 3 KB.  Activation pair buffer 2 doubles as 8 x 2560 B of staging.
+// 2 x 3 KB.  Activation pair buffer 2 doubles as 8 x 2560 B of staging (float
+// output: 8 x 4608 B, which runs 4 KB past the ring into bytes appended for it).
 #pragma once
 
 #include <type_traits>
@@ -32,7 +33,7 @@ constexpr int kPersistThreads = 512;
 
 template <int MODE>
 __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(GemmArgs a, XLinear xsrc) {
-  static_assert(MODE == kOutU8 || MODE == kOutS8, "byte outputs only");
+  static_assert(MODE == kOutU8 || MODE == kOutS8 || MODE == kOutF32, "byte or float outputs");
   constexpr int BM = 256, BN = 256, WM = 2, WN = 4;
   constexpr int NWAVES = WM * WN;
   constexpr int NT = NWAVES * kWave;
@@ -50,8 +51,14 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   constexpr int kTBytes = 32 * kTPitch;
   constexpr int kStagingOff = 3 * kWStage + 2 * kXStage;  // activation pair buffer 2
   static_assert(NWAVES * kTBytes <= kXStage, "staging fits the idle pair buffer");
+  // float output: a wave stages one 32 x 32 MFMA tile at a time, rows of 128 + 16 bytes;
+  // eight such areas are 4 KB more than the idle pair buffer, appended to the ring
+  constexpr int kFPitch = 32 * 4 + 16;
+  constexpr int kFBytes = 32 * kFPitch;
+  constexpr int kFExtra = MODE == kOutF32 ? NWAVES * kFBytes - kXStage : 0;
+  static_assert(kFExtra >= 0 && kRing + kFExtra + 2 * 3 * BN * 4 <= 160 * 1024, "LDS budget");
 
-  __shared__ __attribute__((aligned(16))) uint8_t smem[kRing];
+  __shared__ __attribute__((aligned(16))) uint8_t smem[kRing + kFExtra];
   __shared__ __attribute__((aligned(16))) int s_acc0[2][BN];
   __shared__ __attribute__((aligned(16))) float s_mult[2][BN];
   __shared__ __attribute__((aligned(16))) float s_bdiv[2][BN];
@@ -184,8 +191,13 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
       if (c.ok) {
         acc0 = xq.coef * c.colsum;
         const float atw = xq.scale * c.wscale;
-        mult = atw / a.out_scale;
-        bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, c.bias, atw) : 0.f;
+        if (MODE == kOutF32) {
+          mult = atw;
+          bdiv = c.bias;  // 0 without a bias
+        } else {
+          mult = atw / a.out_scale;
+          bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, c.bias, atw) : 0.f;
+        }
       }
       s_acc0[par][t] = acc0;
       s_mult[par][t] = mult;
@@ -253,8 +265,52 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   uint8_t* const sT = smem + kStagingOff + wave * kTBytes;
   uint8_t* const ybase = static_cast<uint8_t*>(a.y);
   const bool vec_ok = ((a.ldy & 15) == 0) && ((reinterpret_cast<uintptr_t>(a.y) & 15) == 0);
-  const float bmul = bias_mul(a.w_scale_stride == 0, xq.scale * a.w_scales[0]);
+  const float bmul = MODE == kOutF32 ? 1.0f : bias_mul(a.w_scale_stride == 0, xq.scale * a.w_scales[0]);
   const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
+  // float output: y = max(fma(float(acc), x_scale * w_scale[n], bias[n]), lo); a 32 x 32
+  // MFMA tile at a time through this wave's staging rows, whole 128-byte row pieces out
+  // (8 lanes per row, 8 rows per store instruction)
+  auto epilogue_f32 = [&](int m0, int n0, int par) {
+    uint8_t* const sF = smem + kStagingOff + wave * kFBytes;
+    float* const yf = static_cast<float*>(a.y);
+    const bool fvec_ok = ((a.ldy & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.y) & 15) == 0);
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int cl = 8 * g + 4 * half;  // channel inside the MFMA tile
+          const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[par][wn0 + tn * 32 + cl]);
+          const v4f bias = *reinterpret_cast<const v4f*>(&s_bdiv[par][wn0 + tn * 32 + cl]);
+          v4f v;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            v[j] = __builtin_fmaxf(__builtin_fmaf(static_cast<float>(acc[tn][tm][4 * g + j]), mult[j], bias[j]),
+                                   a.lo_f);
+          *reinterpret_cast<v4f*>(sF + li * kFPitch + cl * 4) = v;
+        }
+        wave_sync_lds();
+        if (tm == 0 && tn == 0) wait_loads(std::integral_constant<int, 0>{});  // as in the byte epilogue
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+          const int p = pass * 8 + (lane >> 3), cq = lane & 7;
+          const v4f v = *reinterpret_cast<const v4f*>(sF + p * kFPitch + cq * 16);
+          const int64_t m = m0 + wm0 + tm * 32 + p, n = n0 + wn0 + tn * 32 + cq * 4;
+          if (m < a.M && n < a.N) {
+            float* dst = yf + m * a.ldy + n;
+            if (fvec_ok && n + 4 <= a.N) {
+              *reinterpret_cast<v4f*>(dst) = v;
+            } else {
+              for (int j = 0; j < 4; ++j)
+                if (n + j < a.N) dst[j] = v[j];
+            }
+          }
+        }
+        wave_sync_lds();  // the staging rows are rewritten by the next tile
+      }
+    }
+  };
   auto epilogue = [&](int m0, int n0, int par, auto clamp_tag) {
     constexpr bool CL = decltype(clamp_tag)::value;
 #pragma unroll
@@ -353,10 +409,14 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
       next = load_consts(n0);
       issue_prologue();
     }
-    if (plain_u8)
-      epilogue(em0, en0, par, std::false_type{});  // the saturating conversion is the clamp
-    else
-      epilogue(em0, en0, par, std::true_type{});
+    if constexpr (MODE == kOutF32) {
+      epilogue_f32(em0, en0, par);
+    } else {
+      if (plain_u8)
+        epilogue(em0, en0, par, std::false_type{});  // the saturating conversion is the clamp
+      else
+        epilogue(em0, en0, par, std::true_type{});
+    }
     if (!more) break;
     store_consts(next, par ^ 1);
     par ^= 1;

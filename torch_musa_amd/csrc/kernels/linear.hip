@@ -504,11 +504,11 @@ int cu_count() {
   return v;
 }
 
-// One block per CU walks the 256 x 256 tiles (byte outputs, direct copies two
+// One block per CU walks the 256 x 256 tiles (byte or float outputs, direct copies two
 // stages wide: the caller checked their address and K ranges).
 template <int MODE>
 int launch_gemm_persistent(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
-  if constexpr (MODE == kOutU8 || MODE == kOutS8) {
+  if constexpr (MODE == kOutU8 || MODE == kOutS8 || MODE == kOutF32) {
     const int64_t tiles = ceil_div(a.M, 256) * ceil_div(a.N, 256);
     const int cus = cu_count();
     if (cus < 8 || tiles > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
@@ -759,10 +759,9 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   if (cfg == 19 && !wide_ok) cfg = 17;
   // more than one round of 256 x 256 tiles with byte outputs: the persistent
   // kernel hides each tile's pipeline fill behind the tile before it
-  if (forced < 0 && cfg == 6 && wide_ok && (MODE == kOutU8 || MODE == kOutS8) &&
-      ceil_div(a.M, 256) * ceil_div(a.N, 256) > 256)
+  if (forced < 0 && cfg == 6 && wide_ok && MODE != kOutAcc32 && ceil_div(a.M, 256) * ceil_div(a.N, 256) > 256)
     cfg = 20;
-  if (cfg == 20 && MODE != kOutU8 && MODE != kOutS8) cfg = 6;  // float and raw outputs: one tile per block
+  if (cfg == 20 && MODE == kOutAcc32) cfg = 6;  // raw outputs: one tile per block
   if (cfg == 20 && !wide_ok) cfg = 3;
   if (cfg == 6 && !wide_ok) cfg = 3;
   if (cfg == 17 && !dma_ok) cfg = 3;
