@@ -214,6 +214,25 @@ def test_row_strided_and_unaligned_activations(cabi):
     _check(host(y), want, "unaligned rows")
 
 
+def test_decode_row_pitch_and_exact_buffers(cabi):
+    """The weight-streaming kernel with a row pitch larger than K, and with activation
+    buffers that end exactly at the last row's last byte (its clamped loads must stay
+    inside: every load of a missing k-block reads the row's first bytes)."""
+    say("decode strided x")
+    for m, n, k, pitch in ((5, 48, 128, 160), (1, 16, 16, 16), (16, 130, 4096 + 64, 4096 + 64), (3, 33, 80, 96)):
+        c = _tile_case(m, n, k, seed=900 + m + k)
+        pw = cabi.PackedLinear(dev(c["wq"]))
+        ws, b = dev(c["w_scales"].astype(np.float32)), dev(c["bias"])
+        want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                             c["out_scale"], c["out_zp"])
+        flat = np.zeros(m * pitch - (pitch - k), dtype=np.uint8)   # ends with the last row's last byte
+        for r in range(m):
+            flat[r * pitch:r * pitch + k] = c["xq"][r]
+        xb = torch.as_strided(dev(flat), (m, k), (pitch, 1))
+        y = cabi.linear(xb, pw, c["x_scale"], c["x_zp"], ws, b, c["out_scale"], c["out_zp"])
+        _check(host(y), want, f"decode m={m} k={k} pitch={pitch}")
+
+
 def test_empty_batch(cabi):
     c = _tile_case(4, 32, 64, seed=1)
     pw = cabi.PackedLinear(dev(c["wq"]))
