@@ -756,6 +756,125 @@ def test_aten_cat_and_upsample_nearest(dtype, zp):
     assert_q_equal(m(b.cuda()), m(b))
 
 
+@pytest.mark.parametrize("dtype,zp", [(torch.quint8, 128), (torch.qint8, -3)])
+def test_cat_out_and_add_tensor(dtype, zp):
+    # quantized::cat_out / aten::cat.out requantise into the parameters `out` carries
+    # (reference: TensorShape.cpp:331-381); aten::add.Tensor with a quantized operand
+    # gives the float sum (reference: mudnn/BinaryOps.cpp:11-31)
+    say("aten cat_out / add.Tensor", dtype)
+    torch.manual_seed(5)
+    a = torch.quantize_per_tensor(torch.randn(2, 6, 5, 7), 0.05, zp, dtype)
+    b = torch.quantize_per_tensor(torch.randn(2, 3, 5, 7), 0.03, zp + 2, dtype)
+
+    def out_like(shape, device):
+        return torch._empty_affine_quantized(shape, scale=0.07, zero_point=zp + 1, dtype=dtype, device=device)
+
+    for dim, second in ((1, b), (0, a), (-1, a)):
+        shape = list(torch.cat([a, second], dim).shape)
+        want = torch.ops.quantized.cat_out([a, second], dim, out_like(shape, "cpu"))
+        o = out_like(shape, "cuda")
+        got = torch.ops.quantized.cat_out([a.cuda(), second.cuda()], dim, o)
+        assert got.data_ptr() == o.data_ptr()
+        assert_q_equal(got, want)
+        o2 = out_like(shape, "cuda")
+        assert torch.cat([a.cuda(), second.cuda()], dim, out=o2).data_ptr() == o2.data_ptr()
+        assert_q_equal(o2, want)
+    # an `out` that is not contiguous is filled in place as well
+    base = out_like((2, 7, 5, 9), "cuda")
+    view = base.permute(0, 3, 2, 1)[:, :, :, :]          # shape (2, 9, 5, 7), strided
+    want = torch.ops.quantized.cat_out([a, b], 1, out_like((2, 9, 5, 7), "cpu"))
+    torch.ops.quantized.cat_out([a.cuda(), b.cuda()], 1, view)
+    assert_q_equal(view, want)
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.cat_out([a.cuda(), b.cuda()], 1, out_like((2, 8, 5, 7), "cuda"))
+    with pytest.raises(RuntimeError):
+        torch.ops.quantized.cat_out([a.cuda(), b.cuda()], 1,
+                                    torch._empty_affine_quantized((2, 9, 5, 7), scale=0.1, zero_point=0,
+                                                                  dtype=torch.qint8 if dtype == torch.quint8
+                                                                  else torch.quint8, device="cuda"))
+
+    f = torch.randn(2, 6, 5, 7)
+    a2 = torch.quantize_per_tensor(torch.randn(2, 6, 5, 7), 0.02, zp, dtype)
+    for x, y, want in ((a.cuda(), f.cuda(), a.dequantize() + f),
+                       (f.cuda(), a.cuda(), f + a.dequantize()),
+                       (a.cuda(), a2.cuda(), a.dequantize() + a2.dequantize())):
+        got = torch.add(x, y)
+        assert not got.is_quantized and got.dtype == torch.float32
+        assert torch.equal(got.cpu(), want)
+    assert torch.equal((a.cuda() + f.cuda()).cpu(), a.dequantize() + f)
+    with pytest.raises(RuntimeError):
+        torch.add(a.cuda(), f.cuda(), alpha=2)
+
+
+def test_tensor_utilities_on_quantized_gpu_tensors():
+    """The view, fill, select and reduction helpers the reference registers for its
+    quantized device key (musa_functions.yaml: squeeze / unsqueeze / view / unfold /
+    as_strided / fill_ / masked_fill_ / index_select / flip / max.dim / min.dim / clone /
+    int_repr / empty_like / set_ and the q_* accessors) come from PyTorch-ROCm's own
+    QuantizedCUDA kernels here: each must give what the CPU op gives."""
+    say("aten tensor utilities on quantized tensors")
+    torch.manual_seed(0)
+    x = torch.randn(2, 3, 8, 8)
+    q = torch.quantize_per_tensor(x, 0.05, 128, torch.quint8)
+
+    def per_channel(t, d):
+        return torch._make_per_channel_quantized_tensor(
+            t.int_repr(), torch.tensor([0.1, 0.2, 0.3], dtype=torch.float64, device=d),
+            torch.tensor([1, 2, 3], device=d), 1)
+
+    def empty_q(shape, d):
+        return torch._empty_affine_quantized(shape, scale=0.05, zero_point=128, dtype=torch.quint8, device=d)
+
+    utilities = {
+        "make_per_tensor": lambda t, d: torch._make_per_tensor_quantized_tensor(t.int_repr(), 0.1, 3),
+        "make_per_channel": per_channel,
+        "squeeze": lambda t, d: t[:1].squeeze(0),
+        "unsqueeze": lambda t, d: t.unsqueeze(0),
+        "fill_": lambda t, d: t.clone().fill_(0.5),
+        "masked_fill_": lambda t, d: t.clone().masked_fill_(torch.arange(8, device=d) % 2 == 0, 1.0),
+        "index_select": lambda t, d: torch.index_select(t, 1, torch.tensor([2, 0], device=d)),
+        "index_select_out": lambda t, d: torch.index_select(t, 1, torch.tensor([2, 0], device=d),
+                                                            out=empty_q((2, 2, 8, 8), d)),
+        "as_strided": lambda t, d: torch.as_strided(t, (2, 3, 4, 4), (192, 64, 16, 2)),
+        "relu_": lambda t, d: torch.relu_(t.clone()),
+        "unfold": lambda t, d: t.unfold(2, 2, 2),
+        "max.dim": lambda t, d: t.max(dim=1)[0],
+        "min.dim": lambda t, d: t.min(dim=1, keepdim=True)[0],
+        "flip": lambda t, d: t.flip(3),
+        "clone": lambda t, d: t.clone(),
+        "channels_last": lambda t, d: t.contiguous(memory_format=torch.channels_last),
+        "permute": lambda t, d: t.permute(0, 2, 3, 1),
+        "reshape": lambda t, d: t.reshape(6, 64),
+        "view": lambda t, d: t.view(2, 3, 64),
+        "slice": lambda t, d: t[:, 1:, ::2],
+        "flatten": lambda t, d: torch.flatten(t, 1),
+        "transpose": lambda t, d: t.transpose(1, 3),
+        "copy_": lambda t, d: empty_q(t.shape, d).copy_(t),
+        "empty_like": lambda t, d: torch.empty_like(t).copy_(t),
+        "set_": lambda t, d: empty_q((0,), d).set_(t.untyped_storage(), 0, (2, 192), (192, 1)),
+        "int_repr": lambda t, d: t.int_repr(),
+        "dequantize per channel": lambda t, d: per_channel(t, d).dequantize(),
+        "q_per_channel_zero_points": lambda t, d: per_channel(t, d).q_per_channel_zero_points(),
+        "q_per_channel_axis": lambda t, d: per_channel(t, d).q_per_channel_axis(),
+        "qscheme": lambda t, d: t.qscheme(),
+        "to cpu": lambda t, d: t.cpu(),
+    }
+    g = q.cuda()
+    for name, f in utilities.items():
+        want, got = f(q, "cpu"), f(g, "cuda")
+        if isinstance(want, torch.Tensor) and want.is_quantized:
+            assert got.is_quantized, name
+            if name != "to cpu":
+                assert got.is_cuda, name
+            assert got.shape == want.shape and got.qscheme() == want.qscheme(), name
+            assert torch.equal(got.int_repr().cpu(), want.int_repr()), name
+            assert torch.equal(got.dequantize().cpu(), want.dequantize()), name
+        elif isinstance(want, torch.Tensor):
+            assert torch.equal(got.cpu(), want), name
+        else:
+            assert got == want, name
+
+
 def test_ops_replay_from_a_hip_graph():
     """The operators inside a captured HIP graph (allocations from the graph's pool, no
     host round trip in the captured region): quantized::linear on a split-K shape and on a

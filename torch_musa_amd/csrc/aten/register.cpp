@@ -809,46 +809,104 @@ at::Tensor qsigmoid_run(const at::Tensor& self) {
 // quantized::cat (TensorShape.cpp:383-426 of the reference) and
 // aten::quantized_max_pool2d (Pool.cpp:178-247)
 // ---------------------------------------------------------------------------
-at::Tensor qcat_run(const c10::List<at::Tensor>& qxs, int64_t dim, std::optional<double> scale,
-                    std::optional<int64_t> zero_point) {
-  TORCH_CHECK(qxs.size() > 0, "quantized::cat expects at least one tensor");
+// Checks the inputs of a concatenation against the first one and returns the
+// output shape; `dim` comes back normalised.
+std::vector<int64_t> qcat_shape(const c10::List<at::Tensor>& qxs, int64_t& dim, const char* op) {
+  TORCH_CHECK(qxs.size() > 0, op, " expects at least one tensor");
   const at::Tensor qx0 = qxs[0];
   if (dim < 0) dim += qx0.dim();
   TORCH_CHECK(dim >= 0 && dim < qx0.dim(), "Wrong dim: ", dim);
-  TORCH_CHECK(qx0.qscheme() == c10::kPerTensorAffine || qx0.qscheme() == c10::kPerTensorSymmetric,
-              "Quantized cat only supports quantize-per-tensor");
-  const bool sgn = is_signed_qtype(qx0.scalar_type(), "quantized::cat");
-  const double out_scale = scale.has_value() ? *scale : qx0.q_scale();
-  const int64_t out_zp = zero_point.has_value() ? *zero_point : qx0.q_zero_point();
-  TORCH_CHECK(out_scale > 0, "quantized::cat: output scale must be positive");
   std::vector<int64_t> shape = qx0.sizes().vec();
   shape[dim] = 0;
   for (const at::Tensor& qx : qxs) {
     TORCH_CHECK(qx.scalar_type() == qx0.scalar_type() && qx.dim() == qx0.dim() && qx.device() == qx0.device(),
-                "quantized::cat: all inputs need the dtype, rank and device of the first");
+                op, ": all inputs need the dtype, rank and device of the first");
     TORCH_CHECK(qx.qscheme() == c10::kPerTensorAffine || qx.qscheme() == c10::kPerTensorSymmetric,
                 "Quantized cat only supports quantize-per-tensor");
     for (int64_t d = 0; d < qx0.dim(); ++d)
-      TORCH_CHECK(d == dim || qx.size(d) == qx0.size(d), "quantized::cat: sizes differ outside dim ", dim);
+      TORCH_CHECK(d == dim || qx.size(d) == qx0.size(d), op, ": sizes differ outside dim ", dim);
     shape[dim] += qx.size(dim);
   }
-  const c10::OptionalDeviceGuard guard(at::device_of(qx0));
-  at::Tensor y = at::_empty_affine_quantized(shape, qx0.options(), out_scale, out_zp, c10::MemoryFormat::Contiguous);
-  if (y.numel() == 0) return y;
+  return shape;
+}
+
+// Requantises every input to y's parameters and writes it at its offset along
+// `dim`; y is contiguous and has the concatenated shape.
+void qcat_into(const c10::List<at::Tensor>& qxs, int64_t dim, const at::Tensor& y) {
+  if (y.numel() == 0) return;
+  const bool sgn = is_signed_qtype(y.scalar_type(), "quantized::cat");
   int64_t outer = 1, inner = 1;
-  for (int64_t d = 0; d < dim; ++d) outer *= shape[d];
-  for (int64_t d = dim + 1; d < qx0.dim(); ++d) inner *= shape[d];
+  for (int64_t d = 0; d < dim; ++d) outer *= y.size(d);
+  for (int64_t d = dim + 1; d < y.dim(); ++d) inner *= y.size(d);
   int64_t off = 0;
   for (const at::Tensor& qx : qxs) {
     const at::Tensor x = qx.contiguous();
     const int64_t row = x.size(dim) * inner;
-    check_status(tmq_qcat_rows(x.data_ptr(), y.data_ptr(), outer, row, shape[dim] * inner, off,
+    check_status(tmq_qcat_rows(x.data_ptr(), y.data_ptr(), outer, row, y.size(dim) * inner, off,
                                static_cast<float>(x.q_scale()), static_cast<int32_t>(x.q_zero_point()),
-                               static_cast<float>(out_scale), static_cast<int32_t>(out_zp), sgn, current_stream(y)),
+                               static_cast<float>(y.q_scale()), static_cast<int32_t>(y.q_zero_point()), sgn,
+                               current_stream(y)),
                  "tmq_qcat_rows");
     off += row;
   }
+}
+
+at::Tensor qcat_run(const c10::List<at::Tensor>& qxs, int64_t dim, std::optional<double> scale,
+                    std::optional<int64_t> zero_point) {
+  const std::vector<int64_t> shape = qcat_shape(qxs, dim, "quantized::cat");
+  const at::Tensor qx0 = qxs[0];
+  const double out_scale = scale.has_value() ? *scale : qx0.q_scale();
+  const int64_t out_zp = zero_point.has_value() ? *zero_point : qx0.q_zero_point();
+  TORCH_CHECK(out_scale > 0, "quantized::cat: output scale must be positive");
+  const c10::OptionalDeviceGuard guard(at::device_of(qx0));
+  at::Tensor y = at::_empty_affine_quantized(shape, qx0.options(), out_scale, out_zp, c10::MemoryFormat::Contiguous);
+  qcat_into(qxs, dim, y);
   return y;
+}
+
+// quantized::cat_out and aten::cat.out (TensorShape.cpp:331-381 of the
+// reference): the inputs are requantised to the parameters `out` already
+// carries.  The reference accepts a qint8 `out` only; quint8 works here too.
+// `out` must have the concatenated shape; one that is not contiguous is
+// filled through a contiguous temporary.
+at::Tensor& qcat_out_impl(const c10::List<at::Tensor>& qxs, int64_t dim, at::Tensor& out) {
+  TORCH_CHECK(out.is_quantized() &&
+                  (out.qscheme() == c10::kPerTensorAffine || out.qscheme() == c10::kPerTensorSymmetric),
+              "Quantized cat only supports quantize-per-tensor");
+  const std::vector<int64_t> shape = qcat_shape(qxs, dim, "quantized::cat_out");
+  const at::Tensor qx0 = qxs[0];
+  TORCH_CHECK(out.scalar_type() == qx0.scalar_type() && out.device() == qx0.device(),
+              "quantized::cat_out: out needs the dtype and device of the inputs");
+  TORCH_CHECK(out.sizes().vec() == shape, "quantized::cat_out: out has shape ", out.sizes(), ", the inputs give ",
+              c10::IntArrayRef(shape));
+  const c10::OptionalDeviceGuard guard(at::device_of(out));
+  if (out.is_contiguous()) {
+    qcat_into(qxs, dim, out);
+  } else {
+    at::Tensor y = at::_empty_affine_quantized(shape, out.options(), out.q_scale(), out.q_zero_point(),
+                                               c10::MemoryFormat::Contiguous);
+    qcat_into(qxs, dim, y);
+    out.copy_(y);
+  }
+  return out;
+}
+at::Tensor qcat_out_run(const c10::List<at::Tensor>& qxs, int64_t dim, at::Tensor out) {
+  return qcat_out_impl(qxs, dim, out);
+}
+at::Tensor& qcat_aten_out_run(const at::ITensorListRef& tensors, int64_t dim, at::Tensor& out) {
+  c10::List<at::Tensor> list;
+  for (const at::Tensor& t : tensors) list.push_back(t);
+  return qcat_out_impl(list, dim, out);
+}
+
+// aten::add.Tensor with a quantized operand (mudnn/BinaryOps.cpp:11-31 of the
+// reference): quantized graphs add a quantized tensor to a float one (or to
+// another quantized one) and expect a float result; alpha must be 1.
+at::Tensor qadd_tensor_run(const at::Tensor& a, const at::Tensor& b, const at::Scalar& alpha) {
+  TORCH_CHECK(alpha.equal(1), "Quantized add don't support set alpha yet.");
+  const at::Tensor fa = a.is_quantized() ? a.dequantize() : a;
+  const at::Tensor fb = b.is_quantized() ? b.dequantize() : b;
+  return at::add(fa, fb, alpha);
 }
 
 // aten::cat of quantized tensors (reference: TensorShape.cpp:383-426, the same
@@ -1353,6 +1411,7 @@ TORCH_LIBRARY_IMPL(quantized, QuantizedCUDA, m) {
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_silu.new"), TORCH_FN(qconv2d_silu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::conv2d_add_silu"), TORCH_FN(qconv2d_add_silu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::cat"), TORCH_FN(qcat_run));
+  m.impl(TORCH_SELECTIVE_NAME("quantized::cat_out"), TORCH_FN(qcat_out_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::add"), TORCH_FN(qadd_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::add_relu"), TORCH_FN(qadd_relu_run));
   m.impl(TORCH_SELECTIVE_NAME("quantized::linear"), TORCH_FN(qlinear_run));
@@ -1403,6 +1462,8 @@ TORCH_LIBRARY_IMPL(aten, QuantizedCUDA, m) {
   m.impl("gelu", TORCH_FN(qgelu_run));
   m.impl("sigmoid", TORCH_FN(qsigmoid_run));
   m.impl("cat", TORCH_FN(qcat_aten_run));
+  m.impl("cat.out", TORCH_FN(qcat_aten_out_run));
+  m.impl("add.Tensor", TORCH_FN(qadd_tensor_run));
   m.impl("upsample_nearest2d", TORCH_FN(qupsample_nearest2d_run));
 }
 
