@@ -875,6 +875,100 @@ def test_tensor_utilities_on_quantized_gpu_tensors():
             assert got == want, name
 
 
+@pytest.mark.parametrize("dtype", [torch.quint8, torch.qint8])
+@pytest.mark.parametrize("cfg", [
+    dict(in_channels=16, out_channels=32, kernel_size=3, stride=1, padding=1, dilation=1, groups=1, bias=True),
+    dict(in_channels=32, out_channels=64, kernel_size=3, stride=2, padding=1, dilation=1, groups=1, bias=False),
+    dict(in_channels=64, out_channels=64, kernel_size=1, stride=1, padding=0, dilation=1, groups=1, bias=True),
+    dict(in_channels=32, out_channels=32, kernel_size=3, stride=1, padding=2, dilation=2, groups=2, bias=True),
+], ids=lambda c: "{in_channels}to{out_channels}k{kernel_size}s{stride}g{groups}".format(**c))
+def test_silu_conv_modules(cfg, dtype):
+    """nniq.ConvSiLU2d / nniq.ConvAddSiLU2d the way the reference tests them
+    (test_quantized_conv.py:236-375): weights through set_weight_bias, output parameters
+    set on the module, result against quantize(silu(float conv of the dequantized
+    operands [+ dequantized residual])) within 1 LSB."""
+    import torch.ao.nn.intrinsic.quantized as nniq
+    say("nniq SiLU conv modules", cfg, dtype)
+    torch.manual_seed(41)
+    zp = 128 if dtype == torch.quint8 else 0
+    data = torch.randn(2, cfg["in_channels"], 14, 14)
+    module = torch.nn.Conv2d(**cfg)
+    fweight, fbias = module.weight.detach(), None if module.bias is None else module.bias.detach()
+    qweight = torch.quantize_per_tensor(fweight, float(fweight.abs().max() / 2 ** 7), 0, torch.qint8)
+    qdata = torch.quantize_per_tensor(data, float(data.abs().max()) / 2 ** 7, zp, dtype)
+    with torch.no_grad():
+        conv_out = torch.nn.functional.conv2d(qdata.dequantize(), qweight.dequantize(), fbias, cfg["stride"],
+                                              cfg["padding"], cfg["dilation"], cfg["groups"])
+    accum = torch.randn_like(conv_out)
+    qaccum = torch.quantize_per_tensor(accum, float(accum.abs().max()) / 2 ** 7, zp, dtype)
+
+    for cls, extra, want_f in (
+            (nniq.ConvSiLU2d, (), torch.nn.functional.silu(conv_out)),
+            (nniq.ConvAddSiLU2d, (qaccum.cuda(),), torch.nn.functional.silu(conv_out + qaccum.dequantize()))):
+        qmodule = cls(**cfg)
+        qmodule.set_weight_bias(qweight.cuda(), None if fbias is None else fbias.cuda())
+        out_scale = float(want_f.abs().max() / 2 ** 7)
+        qmodule.scale, qmodule.zero_point = out_scale, zp
+        got = qmodule(qdata.cuda(), *extra)
+        want = torch.quantize_per_tensor(want_f, out_scale, zp, dtype)
+        assert got.is_cuda and got.dtype == dtype and got.shape == want.shape
+        assert got.q_scale() == out_scale and got.q_zero_point() == zp
+        d = (got.int_repr().cpu().int() - want.int_repr().int()).abs()
+        assert d.max() <= 1, f"{cls.__name__}: differs by {d.max()}"
+        w_back, b_back = qmodule._weight_bias()
+        assert torch.equal(w_back.int_repr().cpu(), qweight.int_repr())
+        assert (b_back is None) == (fbias is None)
+        with pytest.raises(ValueError):
+            qmodule(qdata.cuda()[0], *extra)
+
+
+def test_silu_conv_eager_workflow_to_gpu():
+    """Float model with the fused containers -> prepare -> calibrate -> convert with the
+    package's mapping (all on the CPU) -> quantized_modules_to("cuda") -> forward; the
+    quantized model stays close to the float one and equals the ops called by hand."""
+    import torch.ao.quantization as tq
+    from torch_musa_amd import ao, quantized_modules_to
+    say("eager quantization workflow with SiLU convolutions")
+    torch.manual_seed(11)
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.quant = tq.QuantStub()
+            self.stem = ao.fused.ConvSiLU2d(torch.nn.Conv2d(3, 16, 3, padding=1), torch.nn.SiLU())
+            self.body = ao.fused.ConvAddSiLU2d(torch.nn.Conv2d(16, 16, 3, padding=1), torch.add, torch.nn.SiLU())
+            self.dequant = tq.DeQuantStub()
+
+        def forward(self, x):
+            h = self.stem(self.quant(x))
+            return self.dequant(self.body(h, h))
+
+    net = Net().eval()
+    x = torch.randn(4, 3, 24, 24)
+    with torch.no_grad():
+        want = net(x)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        net.qconfig = tq.get_default_qconfig("fbgemm")
+        prepared = tq.prepare(net)
+        prepared(x)
+        mapping = dict(tq.get_default_static_quant_module_mappings())
+        mapping.update(ao.STATIC_QUANT_MODULE_MAPPINGS)
+        qnet = tq.convert(prepared, mapping=mapping)
+    assert type(qnet.stem) is ao.quantized.ConvSiLU2d and type(qnet.body) is ao.quantized.ConvAddSiLU2d
+    quantized_modules_to(qnet, "cuda")
+    got = qnet(x.cuda())
+    assert got.is_cuda and not got.is_quantized and got.shape == want.shape
+    err = (got.cpu() - want).abs().max().item()
+    assert err < 0.06 * want.abs().max().item(), err
+    # the same three steps by hand
+    xq = torch.quantize_per_tensor(x.cuda(), float(qnet.quant.scale), int(qnet.quant.zero_point), torch.quint8)
+    h = torch.ops.quantized.conv2d_silu(xq, qnet.stem._packed_params, qnet.stem.scale, qnet.stem.zero_point)
+    y = torch.ops.quantized.conv2d_add_silu(h, h, qnet.body._packed_params, qnet.body.scale, qnet.body.zero_point)
+    assert torch.equal(y.dequantize(), got)
+
+
 def test_ops_replay_from_a_hip_graph():
     """The operators inside a captured HIP graph (allocations from the graph's pool, no
     host round trip in the captured region): quantized::linear on a split-K shape and on a

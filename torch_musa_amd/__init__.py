@@ -48,6 +48,8 @@ def load() -> None:
         # is intended; the dispatcher warns about it once
         warnings.filterwarnings("ignore", message=".*Overriding a previously registered kernel.*")
         torch.ops.load_library(LIB_ATEN)
+    from . import ao  # the fused SiLU convolution modules, under the reference's torch.ao names
+    ao.register()
     _loaded = True
 
 
