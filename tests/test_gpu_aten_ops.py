@@ -969,6 +969,57 @@ def test_silu_conv_eager_workflow_to_gpu():
     assert torch.equal(y.dequantize(), got)
 
 
+def test_silu_conv_qat_on_gpu_then_int8():
+    """Quantization-aware training of the fused SiLU convolution on the GPU (PyTorch-ROCm's
+    fake-quantize kernels), then `from_float` on the device: weights are quantized and packed
+    there, and the int8 module reproduces the QAT module's own fake-quantized forward pass
+    to within one output step."""
+    import copy
+    import warnings
+    import torch.ao.quantization as tq
+    from torch_musa_amd import ao
+    say("QAT ConvBnSiLU2d on the GPU -> quantized ConvSiLU2d")
+    torch.manual_seed(17)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        qconfig = tq.get_default_qat_qconfig("fbgemm")
+        float_mod = ao.fused.ConvBnSiLU2d(torch.nn.Conv2d(8, 16, 3, padding=1), torch.nn.BatchNorm2d(16),
+                                          torch.nn.SiLU()).train()
+        float_mod.qconfig = qconfig
+        tq.propagate_qconfig_(float_mod)
+        qat = ao.qat.ConvBnSiLU2d.from_float(float_mod).cuda()
+        qat.activation_post_process = qconfig.activation().cuda()
+        in_obs = qconfig.activation().cuda()
+    opt = torch.optim.SGD(qat.parameters(), lr=0.01)
+    x = torch.randn(8, 8, 12, 12, device="cuda")
+    for _ in range(4):
+        opt.zero_grad()
+        y = qat.activation_post_process(qat(in_obs(x)))
+        y.square().mean().backward()
+        opt.step()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in qat.parameters())
+    qat.eval()
+    in_obs.disable_observer()
+    qat.apply(tq.disable_observer)
+    with torch.no_grad():
+        want = qat.activation_post_process(qat(in_obs(x)))       # fake-quantized end to end
+    on_cpu = copy.deepcopy(qat).cpu()
+    q = ao.quantized.ConvSiLU2d.from_float(qat)
+    assert type(q) is ao.quantized.ConvSiLU2d
+    w, b = q._weight_bias()
+    assert w.is_cuda and b.is_cuda
+    q_cpu = ao.quantized.ConvSiLU2d.from_float(on_cpu)           # same conversion on the CPU
+    assert (w.int_repr().cpu().int() - q_cpu.weight().int_repr().int()).abs().max() <= 1
+    assert torch.allclose(b.cpu(), q_cpu.bias(), rtol=1e-5, atol=1e-6)
+    assert q.scale == pytest.approx(q_cpu.scale, rel=1e-6) and q.zero_point == q_cpu.zero_point
+    s_in, z_in = in_obs.calculate_qparams()
+    xq = torch.quantize_per_tensor(x, float(s_in), int(z_in), torch.quint8)
+    got = q(xq)
+    assert got.is_cuda and got.q_scale() == q.scale
+    steps = ((got.dequantize() - want).abs().max() / q.scale).item()
+    assert steps <= 1.01, steps
+
+
 def test_ops_replay_from_a_hip_graph():
     """The operators inside a captured HIP graph (allocations from the graph's pool, no
     host round trip in the captured region): quantized::linear on a split-K shape and on a
