@@ -367,6 +367,25 @@ def test_quantized_add_keeps_channels_last_and_checks_shapes():
         torch.ops.quantized.add(qa, qb[:, :4], 0.08, 128)
 
 
+@pytest.mark.parametrize("dtype,zp", [(torch.quint8, 128), (torch.qint8, 0)])
+@pytest.mark.parametrize("shape", [(128, 512), (256, 256), (2, 32, 32, 16)])
+def test_qfunctional(shape, dtype, zp):
+    # the reference's test_qfunctional (test_quantized_binary_ops.py:36-80): nnq.QFunctional's
+    # add / add_relu (and cat) on device tensors against the same calls on the CPU, within 1 LSB
+    say("nnq.QFunctional", shape, dtype)
+    torch.manual_seed(41)
+    a, b = torch.randn(shape), torch.randn(shape)
+    scale = float(a.abs().max() / 2 ** 7)
+    qa, qb = (torch.quantize_per_tensor(t, scale, zp, dtype) for t in (a, b))
+    if len(shape) == 4:
+        qa, qb = qa.permute(0, 3, 1, 2), qb.permute(0, 3, 1, 2)
+    f = nnq.QFunctional()
+    f.scale, f.zero_point = 0.05, zp
+    for call in (f.add, f.add_relu):
+        assert_q_equal(call(qa.cuda(), qb.cuda()), call(qa, qb), abs_diff=1)
+    assert_q_equal(f.cat([qa.cuda(), qb.cuda()], 1), f.cat([qa, qb], 1), abs_diff=1)
+
+
 @pytest.mark.parametrize("c", cases.qcat_cases(), ids=lambda c: c["name"])
 def test_quantized_cat_op(golden, c):
     say("aten qcat", c["name"])
