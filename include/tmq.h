@@ -205,7 +205,8 @@ typedef struct tmq_linear_desc {
   /* Optional scratch device memory, owned by the caller like every other
    * buffer (16-byte aligned; contents undefined before and after the call).
    * With at least tmq_linear_workspace_bytes(M, N, K) bytes, products whose
-   * tile grid is much smaller than the chip (a few hundred rows) are computed
+   * tile grid is much smaller than the chip (some tens to a few hundred rows
+   * against a long K) are computed
    * split along K: partial sums into the workspace, then one pass that adds
    * and requantises them.  NULL / too small: single-launch kernels, same
    * results. */

@@ -73,7 +73,9 @@ def test_packed_size_arithmetic():
 def test_split_k_workspace_arithmetic():
     # host-only: which problem sizes ask for a split-K workspace, and how much
     wsb = cabi.lib().tmq_linear_workspace_bytes
-    assert wsb(16, 4096, 11008) == 0 and wsb(64, 4096, 11008) == 0     # weight-streaming rows
+    assert wsb(16, 4096, 11008) == 0 and wsb(32, 4096, 11008) == 0     # weight-streaming rows
+    assert wsb(64, 4096, 11008) == 8 * 64 * 4096 * 4                   # 33 ... 64 rows against a long K: split
+    assert wsb(64, 4096, 4096) == 0 and wsb(48, 11008, 4096) == 0      # (K too short for it)
     assert wsb(128, 4096, 4096) == 0                                   # K too short to repay the partial sums
     assert wsb(4096, 11008, 4096) == 0 and wsb(2048, 4096, 16384) == 0  # grids that fill the chip
     assert wsb(128, 4096, 11008) == 8 * 128 * 4096 * 4                 # 32 tiles of 128 x 128 -> 8 splits

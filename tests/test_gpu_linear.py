@@ -336,6 +336,34 @@ def test_split_k(cabi, shape, x_signed, relu, bias, pc):
     np.testing.assert_array_equal(yf1, yf)
 
 
+@pytest.mark.parametrize("shape,path", [((24, 4096, 4096), "stream"), ((40, 11008, 4096), "tiles"),
+                                        ((48, 1024, 1024), "tiles"), ((64, 4096, 11008), "split"),
+                                        ((33, 2048, 8192), "stream"), ((17, 520, 80), "tiles")])
+def test_rows_17_to_64_automatic_choice(cabi, shape, path):
+    """Between 17 and 64 rows the library picks the weight-streaming kernel, 64 x 64 tiles
+    or split K from a time estimate; every choice gives the oracle's bytes, and forcing
+    the streaming kernel gives them too.  (Which kernel ran is visible through the
+    workspace the shape asks for: only the split schedule wants one.)"""
+    say("17-64 rows", shape, path)
+    M, N, K = shape
+    assert (cabi.lib().tmq_linear_workspace_bytes(M, N, K) > 0) == (path == "split")
+    c = _tile_case(M, N, K, seed=99 + M, x_signed=M % 2 == 0, relu=M % 3 == 0, bias=True, per_channel=True)
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    want_acc = oracle.linear_acc32(c["xq"], c["wq"], nthreads=8)
+    for cfg in (-1, 8):
+        y, acc, _ = _run(cabi, c, cfg)
+        _check(y, want, f"cfg {cfg}")
+        np.testing.assert_array_equal(acc, want_acc)
+    cabi.use_linear_workspace = False
+    try:
+        y, acc, _ = _run(cabi, c)
+    finally:
+        cabi.use_linear_workspace = True
+    _check(y, want, "no workspace")
+    np.testing.assert_array_equal(acc, want_acc)
+
+
 def test_split_k_workspace_rules(cabi):
     """No workspace for the weight-streaming rows and for grids that fill the chip; a
     workspace that is too small is ignored, not overrun."""

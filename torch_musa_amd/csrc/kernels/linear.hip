@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ 
 // ---------------------------------------------------------------------------
 constexpr int kDecodeWaves = 8;
 constexpr int kDecodeMaxRows = 64;
-constexpr int kDecodeRowsAuto = 64;  // largest M the automatic choice sends here
+constexpr int kDecodeRowsAuto = 16;  // up to here the automatic choice always streams the weights
 // MG = groups of 16 activation rows (M <= 16 * MG): the weight operands are
 // loaded once and multiplied with every group.
 //
@@ -143,12 +143,19 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(
     }
   }
   const uint8_t* wp = w_packed + static_cast<int64_t>(nb) * (packed_kchunks(K) * 256) + lc * 256 + lr * 16;
+  // Activations are loaded with four consecutive lanes on the 64 bytes one row
+  // contributes to a k-block (lane -> row lane / 4, 16-byte piece lane % 4): a
+  // quad of lanes then asks for one cache line instead of four.  The multiply
+  // wants row lane % 16 and piece lane / 16, so every loaded register goes
+  // through one cross-lane permutation (lane l takes from lane 4 (l % 16) + l / 16).
+  const int sr = lane >> 2, sp = lane & 3;
+  const int perm_addr = (4 * lr + lc) * 4;
   bool xrow[MG];
   const uint8_t* xp[MG];
 #pragma unroll
   for (int mg = 0; mg < MG; ++mg) {
-    xrow[mg] = mg * 16 + lr < M;
-    xp[mg] = x + static_cast<int64_t>(xrow[mg] ? mg * 16 + lr : 0) * ldx;  // the row's first byte: always readable
+    xrow[mg] = mg * 16 + sr < M;
+    xp[mg] = x + static_cast<int64_t>(xrow[mg] ? mg * 16 + sr : 0) * ldx;  // the row's first byte: always readable
   }
   const int xor_word = (flags >> 9) & 1 ? static_cast<int>(0x80808080u) : 0;
   const v4i xmask = {xor_word, xor_word, xor_word, xor_word};
@@ -172,15 +179,18 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(
       wf[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + static_cast<int64_t>(kbc) * 1024));
 #pragma unroll
       for (int mg = 0; mg < MG; ++mg) {
-        xok[mg][u] = kb < KB && xrow[mg] && (kb * 64 + lc * 16 < K);
-        xf[mg][u] = ld16(xp[mg] + (xok[mg][u] ? kb * 64 + lc * 16 : 0));
+        xok[mg][u] = kb < KB && xrow[mg] && (kb * 64 + sp * 16 < K);
+        xf[mg][u] = ld16(xp[mg] + (xok[mg][u] ? kb * 64 + sp * 16 : 0));
       }
     }
 #pragma unroll
     for (int u = 0; u < kBatch; ++u)
 #pragma unroll
       for (int mg = 0; mg < MG; ++mg) {
-        const v4i xv = xok[mg][u] ? (xf[mg][u] ^ xmask) : v4i{0, 0, 0, 0};
+        const v4i xs = xok[mg][u] ? (xf[mg][u] ^ xmask) : v4i{0, 0, 0, 0};
+        v4i xv;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) xv[c] = __builtin_amdgcn_ds_bpermute(perm_addr, xs[c]);
         acc2[mg][u & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], xv, acc2[mg][u & 1], 0, 0, 0);
       }
   };
@@ -541,7 +551,49 @@ constexpr int64_t kSplitBlocks = 256;    // blocks wanted: one per CU
 constexpr int64_t kSplitMinKT = 128;     // shortest k loop (stages) worth cutting
 constexpr int64_t kSplitMinStages = 16;  // shortest run of stages per split
 
-SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
+// ---- 17 ... 64 rows: three kernels can run such a product, and which is fastest
+// depends on the shape.  Estimated microseconds per launch, fitted to sweeps with
+// cold weights (more weight sets in rotation than the last-level cache holds):
+//  * the weight-streaming kernel re-reads all M x K activation bytes in every
+//    block of 16 channels, so its time grows with rows x blocks x K, the bytes
+//    the L2s hand out (K = N = 4096: 5.9 / 7.8 / 12.2 us at M = 16 / 32 / 64;
+//    N = 11008, K = 4096: 12.6 / 18.9 / 32.3 us);
+//  * 64 x 64 tiles walk K at the latency of one stage after the other, almost
+//    whatever M is (K = N = 4096 with two wave groups: 12.8 / 14.8 us at
+//    M = 32 / 64; N = 11008: 14.9 / 16.8 us; K = N = 1024: 6.2 us);
+//  * split K moves the weights at about 3.4 TB/s plus 8 us for the partial sums
+//    (N = 4096, K = 11008: 21.7 us at M = 65 against 30.6 us streaming at M = 64).
+enum class SmallRows { kStream, kTiles, kSplit };
+
+bool two_wave_groups_fit(int64_t M, int64_t N, int64_t K) {
+  const int64_t stages = ceil_div(K, kBK);
+  return ceil_div(M, 64) * ceil_div(N, 64) <= 256 && stages >= 32 && stages % 2 == 0;
+}
+
+SplitPlan plan_split_tiles(int64_t M, int64_t N, int64_t K);
+
+SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
+  const double mib = static_cast<double>(N) * static_cast<double>(K) / 1048576.0;
+  const double stages = static_cast<double>(ceil_div(K, kBK));
+  const double rows = static_cast<double>(M);
+  const double l2_mib_per_row = static_cast<double>(ceil_div(N, 16)) * static_cast<double>(K) / 1048576.0;
+  const double stream = 2.4 + 0.11 * mib + 0.4 * mib / 16.0 + rows * std::max(0.10, 0.135 * l2_mib_per_row);
+  const double nblk = static_cast<double>(ceil_div(M, 64) * ceil_div(N, 64));
+  double tiles;
+  if (two_wave_groups_fit(M, N, K))
+    tiles = (4.4 + 0.123 * stages + 0.013 * std::max(0.0, nblk - 64.0)) *
+            (1.0 + 0.35 * (rows / 64.0) * (rows / 64.0) * std::min(1.0, stages / 172.0));
+  else
+    tiles = (3.0 + 0.2 * stages) * (1.0 + nblk / 1024.0);
+  double best = std::min(stream, tiles);
+  if (workspace && plan_split_tiles(M, N, K).splits > 1) {
+    const double split = 8.0 + 0.295 * mib + 0.02 * rows;
+    if (split < best) return SmallRows::kSplit;
+  }
+  return stream <= tiles ? SmallRows::kStream : SmallRows::kTiles;
+}
+
+SplitPlan plan_split_tiles(int64_t M, int64_t N, int64_t K) {
   SplitPlan p;
   if (M <= kDecodeRowsAuto || K % 16 != 0) return p;
   const int64_t KT = ceil_div(K, kBK);
@@ -561,6 +613,14 @@ SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
   p.stages = static_cast<int>(stages);
   p.ldp = (N + 3) / 4 * 4;
   return p;
+}
+
+// The plan the automatic choice follows: none for the rows that stream the
+// weights, and for 17 ... 64 rows only where the estimate above prefers it.
+SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
+  if (M > kDecodeRowsAuto && M <= kDecodeMaxRows && small_rows_path(M, N, K, true) != SmallRows::kSplit)
+    return SplitPlan{};
+  return plan_split_tiles(M, N, K);
 }
 
 int64_t split_workspace_bytes(const SplitPlan& p, int64_t M) {
@@ -688,7 +748,11 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     linear_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(b, xs, x_signed);
     return launch_status();
   }
-  if ((a.M <= kDecodeRowsAuto && forced < 0) || forced == 8) {
+  const bool stream_auto =
+      forced < 0 && (a.M <= kDecodeRowsAuto ||
+                     (a.M <= kDecodeMaxRows &&
+                      small_rows_path(a.M, a.N, a.K, workspace != nullptr && a.K % 16 == 0) == SmallRows::kStream));
+  if (stream_auto || forced == 8) {
     if (a.M > kDecodeMaxRows) return TMQ_ERR_UNSUPPORTED;
     const int64_t blocks = ceil_div(a.N, 16);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
@@ -713,7 +777,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   // and run their three-stage ring at least once around
   const bool dma_ok = xs.ldx <= (int64_t{1} << 23) && a.K <= (int64_t{1} << 23) && a.K > 2 * kBK;
   if (forced < 0 || forced == 13) {
-    const SplitPlan p = plan_split(a.M, a.N, a.K);
+    const SplitPlan p = forced == 13 ? plan_split_tiles(a.M, a.N, a.K) : plan_split(a.M, a.N, a.K);
     if (p.splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(p, a.M) &&
         aligned(workspace, 16))
       return run_split<MODE>(a, xs, p, workspace, dma_ok, s);
