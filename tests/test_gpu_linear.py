@@ -89,17 +89,50 @@ def test_per_tensor_weight_bias_form(cabi, golden, cfg):
 
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21])
 @pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),
                                    (270, 300, 400), (40, 70, 784)])
 def test_tile_configs(cabi, cfg, shape):
     say("tile cfg", cfg, shape)
+    if cfg == 21 and shape[2] > 1024:
+        pytest.skip("the kernel that holds all of K in LDS takes K <= 1024")
     c = _tile_case(*shape, seed=cfg * 10 + shape[0])
     y, acc, _ = _run(cabi, c, cfg)
     np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]))
     want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
                          c["out_scale"], c["out_zp"], relu=c["relu"])
     _check(y, want, f"cfg {cfg}")
+
+
+# all of K in LDS (K <= 1024): every number of 256-byte phases, K that ends inside a phase and on
+# an odd 16-byte chunk, one row, ragged rows and channels, both activation types, every epilogue
+@pytest.mark.parametrize("shape", [(128, 1024, 1024), (1, 16, 16), (64, 64, 32), (65, 70, 48), (100, 130, 1008),
+                                   (33, 200, 272), (257, 129, 528), (1000, 1000, 1024), (90, 33, 784)])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_whole_k_in_lds_kernel(cabi, shape, x_signed):
+    say("K in LDS", shape, x_signed)
+    M, N, K = shape
+    c = _tile_case(M, N, K, seed=2100 + M, x_signed=x_signed, relu=N % 2 == 1, bias=M % 3 != 0,
+                   per_channel=(M + N) % 2 == 0)
+    y, acc, pw = _run(cabi, c, 21)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "K in LDS")
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    cabi.force_linear_config(21)
+    try:
+        yf = host(cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, relu=c["relu"]))
+    finally:
+        cabi.force_linear_config(-1)
+    np.testing.assert_array_equal(
+        yf, oracle.linear_f32(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], relu=c["relu"],
+                              nthreads=8))
+    if M * N <= 64 * 64 * 256:      # the automatic choice for grids no larger than the chip
+        y1, acc1, _ = _run(cabi, c)
+        np.testing.assert_array_equal(y1, y)
+        np.testing.assert_array_equal(acc1, acc)
 
 
 # the persistent kernel over more tiles than the chip has CUs: every block walks two tiles
@@ -394,7 +427,7 @@ def test_split_k_workspace_rules(cabi):
 # Float results are compared bit for bit: the kernel's epilogue is the oracle's
 # single fused multiply-add, and the dynamic quantization in front of it is
 # bit-exact by the quantizer tests.
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20, 21])
 @pytest.mark.parametrize("shape,relu,bias,pc,x_signed", [((60, 264, 448), False, True, True, False),
                                                          ((257, 33, 144), True, True, False, False),
                                                          ((16, 1040, 1168), False, False, True, True)])
@@ -403,6 +436,8 @@ def test_linear_f32_configs(cabi, cfg, shape, relu, bias, pc, x_signed):
     c = _tile_case(*shape, seed=300 + cfg, x_signed=x_signed, relu=relu, bias=bias, per_channel=pc)
     if cfg == 8 and shape[0] > 64:
         pytest.skip("the weight-streaming kernel takes at most 64 rows")
+    if cfg == 21 and shape[2] > 1024:
+        pytest.skip("the kernel that holds all of K in LDS takes K <= 1024")
     pw = cabi.PackedLinear(dev(c["wq"]))
     ws = dev(c["w_scales"].astype(np.float32))
     b = None if c["bias"] is None else dev(c["bias"])

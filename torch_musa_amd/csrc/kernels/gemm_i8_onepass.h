@@ -1,0 +1,244 @@
+// int8 MFMA GEMM for short K (K <= 1024 bytes) on 64 x 64 tiles: both operands
+// of a tile, all of K, are copied into LDS before anything is multiplied.
+//
+// The pipelined kernels of gemm_i8_core.h walk K one 64-byte stage after the
+// other; a block that is alone on its CU spends 0.2 us per stage in the chain
+// copy -> barrier -> LDS read -> MFMA whatever the prefetch depth, so a product
+// like M = 128, K = N = 1024 (32 blocks, 16 stages) takes 6 us of which the
+// multiplying is 0.5.  Here every wave requests its share of the whole tile at
+// once with direct global -> LDS copies (128 KB in flight per block), the block
+// meets at one barrier per 256 bytes of K (four at most) as the copies land in
+// the order issued, and between the barriers the waves multiply from LDS with no
+// further synchronisation.
+//
+// LDS layout
+//   weights      [k-chunk (16 B of K)][64 rows][16 B]: the packed layout as it is
+//   activations  [256-byte block of K][64 rows][256 B], the sixteen 16-byte slots
+//                of a row's 256 bytes XOR-ed with row % 16, so that the 16 rows a
+//                quarter wave reads for one k-chunk fall on 16 different slots
+//                (every bank once)
+// A copy instruction moves 1 KB: one weight k-chunk of the 64 rows, or the 256
+// bytes of 4 activation rows (16 lanes per row: whole cache lines).
+#pragma once
+
+#include "gemm_i8_core.h"
+
+namespace tmq {
+
+constexpr int kOnePassMaxK = 1024;
+
+// As lds_dma16 with 4 bytes per lane: lane l's dword lands at lds_dst + 4 l.
+__device__ __forceinline__ void lds_dma4(const void* base, uint32_t off, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               :
+               : "v"(off), "s"(base), "s"(lds_dst)
+               : "memory", "m0");
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinear xs) {
+  constexpr int BM = 64, BN = 64;
+  constexpr int kPhaseChunks = 16;                 // k-chunks per barrier: 256 bytes of K
+  constexpr int kCopiesPerPhase = 8;               // per wave: 4 weight chunks + 4 activation row groups
+  __shared__ __attribute__((aligned(16))) uint8_t sW[(kOnePassMaxK / 16) * BN * 16];
+  __shared__ __attribute__((aligned(16))) uint8_t sX[(kOnePassMaxK / 256) * BM * 256];
+  __shared__ __attribute__((aligned(16))) int s_raw[3][BN];  // colsum, weight scale, bias as fetched
+  __shared__ __attribute__((aligned(16))) int s_acc0[BN];
+  __shared__ __attribute__((aligned(16))) float s_mult[BN];
+  __shared__ __attribute__((aligned(16))) float s_bdiv[BN];
+
+  const int t = threadIdx.x, lane = t % kWave;
+  const int wave_u = __builtin_amdgcn_readfirstlane(t / kWave);
+  const int li = lane & 31, half = lane >> 5;
+  const int wm0 = (wave_u & 1) * 32, wn0 = (wave_u >> 1) * 32;
+  const int64_t tiles_n = ceil_div(a.N, BN);
+  const int64_t m0 = (static_cast<int64_t>(blockIdx.x) / tiles_n) * BM;
+  const int64_t n0 = (static_cast<int64_t>(blockIdx.x) % tiles_n) * BN;
+  const int KC = static_cast<int>(a.K >> 4);       // k-chunks (K is a multiple of 16)
+  const int S = (KC + 1) >> 1;                     // 32-byte k-steps
+  const int NP = (KC + kPhaseChunks - 1) / kPhaseChunks;
+
+  // ---- requests, oldest first: the tile's per-channel constants (wave 0), then
+  // phase by phase the weight chunks and activation row groups of this wave
+  if (wave_u == 0) {
+    const int64_t n = n0 + lane < a.N ? n0 + lane : a.N - 1;
+    const uint32_t np = static_cast<uint32_t>(n + a.n_off);
+    lds_dma4(a.colsum, np * 4u, lds_address(&s_raw[0][0]));
+    if constexpr (MODE != kOutAcc32) {  // (raw accumulators: the caller passes no scales)
+      lds_dma4(a.w_scales, np * static_cast<uint32_t>(a.w_scale_stride) * 4u, lds_address(&s_raw[1][0]));
+      lds_dma4(a.bias != nullptr ? a.bias : a.w_scales, a.bias != nullptr ? np * 4u : 0u,
+               lds_address(&s_raw[2][0]));
+    }
+  }
+  {
+    const int64_t NB = ceil_div(a.N, 16);
+    const int64_t nb_last = NB - 1 - n0 / 16;      // 16-row blocks past N: clamped, never stored
+    const uint8_t* const wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
+    const int64_t rb = (lane >> 4) < nb_last ? (lane >> 4) : nb_last;
+    const uint32_t woff = static_cast<uint32_t>(rb * a.w_kchunks * 256 + (lane & 15) * 16);
+    const int kc_last = static_cast<int>(a.w_kchunks) - 1;
+    const uint8_t* const xtile = xs.x + m0 * xs.ldx;
+    const int64_t m_last = a.M - 1 - m0;           // rows past M: clamped, never stored
+    const uint32_t ldsW = lds_address(sW), ldsX = lds_address(sX);
+    for (int p = 0; p < NP; ++p) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int kc = p * kPhaseChunks + 4 * wave_u + i;
+        const int kcc = kc < kc_last ? kc : kc_last;   // (chunks past the packed pitch are never read)
+        lds_dma16(wtile + static_cast<int64_t>(kcc) * 256, woff, ldsW + static_cast<uint32_t>(kc) * 1024u);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int g = 4 * wave_u + i;                  // rows 4g .. 4g+3
+        const int r = 4 * g + (lane >> 4);
+        const int64_t rc = r < m_last ? r : m_last;
+        const int cc = p * kPhaseChunks + ((lane & 15) ^ (r & 15));
+        // chunks past K: any bytes of the row will do, the packed weight is zero there
+        const int ccc = cc < KC ? cc : KC - 1;
+        lds_dma16(xtile, static_cast<uint32_t>(rc * xs.ldx + ccc * 16),
+                  ldsX + static_cast<uint32_t>(p * BM + 4 * g) * 256u);
+      }
+    }
+  }
+
+  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
+                     static_cast<int>(a.x_xor)};
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  const int xrow = wm0 + li;
+  const uint8_t* const wrd = sW + (wn0 + li) * 16;
+  const uint8_t* const xrd = sX + xrow * 256;
+
+  for (int p = 0; p < NP; ++p) {
+    // the copies of the phases after this one may still be on their way
+    switch (NP - 1 - p) {
+      case 0: __builtin_amdgcn_s_waitcnt((0 & 15) | ((0 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+      case 1: __builtin_amdgcn_s_waitcnt((8 & 15) | ((8 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+      case 2: __builtin_amdgcn_s_waitcnt((16 & 15) | ((16 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+      default: __builtin_amdgcn_s_waitcnt((24 & 15) | ((24 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+    }
+    static_assert(kCopiesPerPhase == 8, "the wait counts above are multiples of the copies per phase");
+    __syncthreads();
+    if (p == 0 && t < BN) {
+      // the constants landed before the first phase: turn them into the
+      // accumulator's start value and the requantisation factors
+      const XQuant xq = x_quant(a);
+      const bool live = n0 + t < a.N;
+      float mult = 0.f, bdiv = 0.f;
+      if constexpr (MODE != kOutAcc32) {
+        const float ws = __int_as_float(s_raw[1][t]), bs = __int_as_float(s_raw[2][t]);
+        const float atw = xq.scale * ws;
+        if (MODE == kOutF32) {
+          mult = atw;
+          bdiv = a.bias != nullptr ? bs : 0.f;
+        } else {
+          mult = atw / a.out_scale;
+          bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, bs, atw) : 0.f;
+        }
+      }
+      s_acc0[t] = live ? xq.coef * s_raw[0][t] : 0;
+      s_mult[t] = live ? mult : 0.f;
+      s_bdiv[t] = live ? bdiv : 0.f;
+    }
+    const int s0 = p * (kPhaseChunks / 2);
+    const int nsteps = S - s0 < kPhaseChunks / 2 ? S - s0 : kPhaseChunks / 2;
+    // (k-steps past the end of K in the last phase read whatever the buffers
+    // hold and multiply it with a zeroed activation operand: no branches here)
+    v4i wf[kPhaseChunks / 2], xf[kPhaseChunks / 2];
+#pragma unroll
+    for (int j = 0; j < kPhaseChunks / 2; ++j) {
+      const int c = 2 * (s0 + j) + half;
+      wf[j] = ld16(wrd + c * (BN * 16));
+      xf[j] = ld16(xrd + p * (BM * 256) + (((c & 15) ^ (xrow & 15)) << 4));
+    }
+#pragma unroll
+    for (int j = 0; j < kPhaseChunks / 2; ++j) {
+      const int keep = j < nsteps ? -1 : 0;
+      const v4i xv = (xf[j] ^ xmask) & v4i{keep, keep, keep, keep};
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xv, acc, 0, 0, 0);
+    }
+  }
+
+  // ---- epilogue.  A lane holds channels n = 8g + 4 half + j (g, j < 4) of
+  // activation row li of its wave's 32 x 32 part; the tile goes through LDS (over
+  // the weight chunks, which every wave has finished reading at the barrier) so
+  // that whole rows leave with 16 bytes per lane.
+  __syncthreads();
+  if constexpr (MODE == kOutF32 || MODE == kOutAcc32) {
+    constexpr int kPitch = BN * 4 + 16;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int nl = wn0 + 8 * g + 4 * half;
+      const v4i add = *reinterpret_cast<const v4i*>(&s_acc0[nl]);
+      const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[nl]);
+      const v4f bias = *reinterpret_cast<const v4f*>(&s_bdiv[nl]);
+      v4f v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int raw = acc[4 * g + j] + add[j];
+        v[j] = MODE == kOutAcc32
+                   ? __int_as_float(raw)
+                   : __builtin_fmaxf(__builtin_fmaf(static_cast<float>(raw), mult[j], bias[j]), a.lo_f);
+      }
+      *reinterpret_cast<v4f*>(&sW[(wm0 + li) * kPitch + nl * 4]) = v;
+    }
+    __syncthreads();
+    float* const yf = static_cast<float*>(a.y) + a.n_off;
+    const bool vec_ok = ((a.ldy & 3) == 0) && ((reinterpret_cast<uintptr_t>(yf) & 15) == 0);
+    constexpr int kRowChunks = BN / 4;
+#pragma unroll
+    for (int id = t; id < BM * kRowChunks; id += 256) {
+      const int row = id / kRowChunks, cc = id % kRowChunks;
+      const int64_t m = m0 + row, n = n0 + cc * 4;
+      if (m >= a.M || n >= a.N) continue;
+      const v4f v = *reinterpret_cast<const v4f*>(&sW[row * kPitch + cc * 16]);
+      float* dst = yf + m * a.ldy + n;
+      if (vec_ok && n + 4 <= a.N) {
+        *reinterpret_cast<v4f*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < a.N) dst[j] = v[j];
+      }
+    }
+  } else {
+    constexpr int kPitch = BN + 16;
+    const float bmul = bias_mul(a.w_scale_stride == 0, x_quant(a).scale * __int_as_float(s_raw[1][0]));
+    const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int nl = wn0 + 8 * g + 4 * half;
+      const v4i add = *reinterpret_cast<const v4i*>(&s_acc0[nl]);
+      const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[nl]);
+      const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[nl]);
+      int raw[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) raw[j] = acc[4 * g + j] + add[j];
+      // unsigned output without ReLU: the saturating conversion is the clamp
+      const uint32_t q4 = plain_u8 ? requant4<MODE, false>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f)
+                                   : requant4<MODE, true>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+      *reinterpret_cast<uint32_t*>(&sW[(wm0 + li) * kPitch + nl]) = q4;
+    }
+    __syncthreads();
+    uint8_t* const y = static_cast<uint8_t*>(a.y) + a.n_off;
+    const bool vec_ok = ((a.ldy & 15) == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+    constexpr int kRowChunks = BN / 16;
+    const int row = t / kRowChunks, cc = t % kRowChunks;   // 256 threads: one 16-byte piece each
+    const int64_t m = m0 + row, n = n0 + cc * 16;
+    if (m < a.M && n < a.N) {
+      const v4i v = ld16(&sW[row * kPitch + cc * 16]);
+      uint8_t* dst = y + m * a.ldy + n;
+      if (vec_ok && n + 16 <= a.N) {
+        *reinterpret_cast<v4i*>(dst) = v;
+      } else {
+        const uint32_t w[4] = {static_cast<uint32_t>(v.x), static_cast<uint32_t>(v.y), static_cast<uint32_t>(v.z),
+                               static_cast<uint32_t>(v.w)};
+        for (int b = 0; b < 16; ++b)
+          if (n + b < a.N) dst[b] = static_cast<uint8_t>(w[b >> 2] >> (8 * (b & 3)));
+      }
+    }
+  }
+}
+
+}  // namespace tmq

@@ -4,6 +4,7 @@
 #include <atomic>
 
 #include "gemm_i8_core.h"
+#include "gemm_i8_onepass.h"
 #include "gemm_i8_persistent.h"
 #include "qparams.h"
 
@@ -498,6 +499,15 @@ int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   return launch_status();
 }
 
+// 64 x 64 tiles with all of K in LDS (K <= 1024; the caller checked the address ranges).
+template <int MODE>
+int launch_gemm_onepass(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  const int64_t blocks = ceil_div(a.M, 64) * ceil_div(a.N, 64);
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  gemm_i8_onepass_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(a, xs);
+  return launch_status();
+}
+
 constexpr int kMaxDevices = 64;
 
 // Compute units of the current device (cached per device; two threads that race
@@ -560,7 +570,8 @@ constexpr int64_t kSplitMinStages = 16;  // shortest run of stages per split
 //    N = 11008, K = 4096: 12.6 / 18.9 / 32.3 us);
 //  * 64 x 64 tiles walk K at the latency of one stage after the other, almost
 //    whatever M is (K = N = 4096 with two wave groups: 12.8 / 14.8 us at
-//    M = 32 / 64; N = 11008: 14.9 / 16.8 us; K = N = 1024: 6.2 us);
+//    M = 32 / 64; N = 11008: 14.9 / 16.8 us), and K <= 1024 fits LDS whole
+//    (gemm_i8_onepass.h: K = N = 1024: 5.8 us);
 //  * split K moves the weights at about 3.4 TB/s plus 8 us for the partial sums
 //    (N = 4096, K = 11008: 21.7 us at M = 65 against 30.6 us streaming at M = 64).
 enum class SmallRows { kStream, kTiles, kSplit };
@@ -577,10 +588,14 @@ SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
   const double stages = static_cast<double>(ceil_div(K, kBK));
   const double rows = static_cast<double>(M);
   const double l2_mib_per_row = static_cast<double>(ceil_div(N, 16)) * static_cast<double>(K) / 1048576.0;
-  const double stream = 2.4 + 0.11 * mib + 0.4 * mib / 16.0 + rows * std::max(0.10, 0.135 * l2_mib_per_row);
+  const double stream_blocks = static_cast<double>(ceil_div(N, 16));
+  const double stream = 2.4 + 0.11 * mib + 0.4 * mib / 16.0 +
+                        rows * std::max(0.10 * std::max(1.0, stream_blocks / 256.0), 0.135 * l2_mib_per_row);
   const double nblk = static_cast<double>(ceil_div(M, 64) * ceil_div(N, 64));
   double tiles;
-  if (two_wave_groups_fit(M, N, K))
+  if (K <= kOnePassMaxK && nblk <= 256.0)  // all of K in LDS (K = N = 1024: 5.8 us, K = N = 512: 3.9 us)
+    tiles = 2.0 + 3.8 * static_cast<double>(K) / 1024.0 + 0.012 * std::max(0.0, nblk - 64.0);
+  else if (two_wave_groups_fit(M, N, K))
     tiles = (4.4 + 0.123 * stages + 0.013 * std::max(0.0, nblk - 64.0)) *
             (1.0 + 0.35 * (rows / 64.0) * (rows / 64.0) * std::min(1.0, stages / 172.0));
   else
@@ -783,8 +798,15 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
       return run_split<MODE>(a, xs, p, workspace, dma_ok, s);
     if (forced == 13) return TMQ_ERR_UNSUPPORTED;
   }
+  // all of K in LDS: 32-bit offsets over 64 rows of either operand, N * 4 as a 32-bit offset
+  const bool onepass_ok = a.K <= kOnePassMaxK && a.K % 16 == 0 && xs.ldx <= (int64_t{1} << 23) &&
+                          a.N + a.n_off < (int64_t{1} << 29) && a.splits == 1;
   int cfg = forced;
-  if (cfg < 0) {
+  if (cfg < 0 && onepass_ok && ceil_div(a.M, 64) * ceil_div(a.N, 64) <= 256) {
+    // short K on a grid no larger than the chip: one latency instead of one per stage
+    // (M = 128, K = N = 1024: 6.0 -> 4.x us)
+    cfg = 21;
+  } else if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
     // the CUs busy, the 128x128 tile (two blocks per CU) down to 128 tiles.
@@ -843,6 +865,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 17: return launch_gemm<128, 256, 2, 4, MODE, 3, true>(a, xs, s);
     case 19: return launch_gemm<128, 256, 2, 4, MODE, 3, true, 1, true>(a, xs, s);
     case 20: return launch_gemm_persistent<MODE>(a, xs, s);
+    case 21: return onepass_ok ? launch_gemm_onepass<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
