@@ -1,22 +1,29 @@
-// int8 MFMA GEMM for short K (K <= 1024 bytes) on 64 x 64 tiles: both operands
-// of a tile, all of K, are copied into LDS before anything is multiplied.
+// int8 MFMA GEMM on 64 x 64 tiles whose operands reach LDS in phases of 256 bytes
+// of K, four phases (128 KB) requested ahead.  For K <= 1024 that is all of K at
+// once, which is what the kernel is for.
 //
 // The pipelined kernels of gemm_i8_core.h walk K one 64-byte stage after the
 // other; a block that is alone on its CU spends 0.2 us per stage in the chain
 // copy -> barrier -> LDS read -> MFMA whatever the prefetch depth, so a product
 // like M = 128, K = N = 1024 (32 blocks, 16 stages) takes 6 us of which the
-// multiplying is 0.5.  Here every wave requests its share of the whole tile at
-// once with direct global -> LDS copies (128 KB in flight per block), the block
-// meets at one barrier per 256 bytes of K (four at most) as the copies land in
-// the order issued, and between the barriers the waves multiply from LDS with no
-// further synchronisation.
+// multiplying is 0.5.  Here every wave requests its share of four phases of the
+// tile at once with direct global -> LDS copies (128 KB in flight per block), the
+// block meets at one barrier per phase as the copies land in the order issued,
+// and between the barriers the waves multiply from LDS with no further
+// synchronisation; behind the barrier that ends phase p the buffer it used takes
+// phase p + 4.
 //
-// LDS layout
-//   weights      [k-chunk (16 B of K)][64 rows][16 B]: the packed layout as it is
-//   activations  [256-byte block of K][64 rows][256 B], the sixteen 16-byte slots
-//                of a row's 256 bytes XOR-ed with row % 16, so that the 16 rows a
-//                quarter wave reads for one k-chunk fall on 16 different slots
-//                (every bank once)
+// The automatic choice sends K <= 1024 here (grids of at most 256 tiles).  Longer
+// K runs (any K, for tests) but does not pay: with cold weights a phase then
+// waits for memory, 96 KB in flight per CU against about 2 us of latency, and
+// K = N = 4096 at M = 128 takes 15.0 us against 12.5 us for the 64 x 64 tiles
+// with two wave groups.
+//
+// LDS layout (ring buffer b = phase % 4)
+//   weights      [b][k-chunk (16 B of K)][64 rows][16 B]: the packed layout as it is
+//   activations  [b][64 rows][256 B], the sixteen 16-byte slots of a row's 256
+//                bytes XOR-ed with row % 16, so that the 16 rows a quarter wave
+//                reads for one k-chunk fall on 16 different slots (every bank once)
 // A copy instruction moves 1 KB: one weight k-chunk of the 64 rows, or the 256
 // bytes of 4 activation rows (16 lanes per row: whole cache lines).
 #pragma once
@@ -25,7 +32,7 @@
 
 namespace tmq {
 
-constexpr int kOnePassMaxK = 1024;
+constexpr int kOnePassMaxK = 1024;  // longest K the automatic choice sends here: four phases
 
 // As lds_dma16 with 4 bytes per lane: lane l's dword lands at lds_dst + 4 l.
 __device__ __forceinline__ void lds_dma4(const void* base, uint32_t off, uint32_t lds_dst) {
@@ -39,9 +46,10 @@ template <int MODE>
 __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinear xs) {
   constexpr int BM = 64, BN = 64;
   constexpr int kPhaseChunks = 16;                 // k-chunks per barrier: 256 bytes of K
+  constexpr int kRing = 4;                         // phases the LDS buffers hold
   constexpr int kCopiesPerPhase = 8;               // per wave: 4 weight chunks + 4 activation row groups
-  __shared__ __attribute__((aligned(16))) uint8_t sW[(kOnePassMaxK / 16) * BN * 16];
-  __shared__ __attribute__((aligned(16))) uint8_t sX[(kOnePassMaxK / 256) * BM * 256];
+  __shared__ __attribute__((aligned(16))) uint8_t sW[kRing * kPhaseChunks * BN * 16];
+  __shared__ __attribute__((aligned(16))) uint8_t sX[kRing * BM * 256];
   __shared__ __attribute__((aligned(16))) int s_raw[3][BN];  // colsum, weight scale, bias as fetched
   __shared__ __attribute__((aligned(16))) int s_acc0[BN];
   __shared__ __attribute__((aligned(16))) float s_mult[BN];
@@ -56,7 +64,7 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
   const int64_t n0 = (static_cast<int64_t>(blockIdx.x) % tiles_n) * BN;
   const int KC = static_cast<int>(a.K >> 4);       // k-chunks (K is a multiple of 16)
   const int S = (KC + 1) >> 1;                     // 32-byte k-steps
-  const int NP = (KC + kPhaseChunks - 1) / kPhaseChunks;
+  const int NP = (KC + kPhaseChunks - 1) / kPhaseChunks;   // phases of 256 bytes of K
 
   // ---- requests, oldest first: the tile's per-channel constants (wave 0), then
   // phase by phase the weight chunks and activation row groups of this wave
@@ -70,36 +78,56 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
                lds_address(&s_raw[2][0]));
     }
   }
-  {
-    const int64_t NB = ceil_div(a.N, 16);
-    const int64_t nb_last = NB - 1 - n0 / 16;      // 16-row blocks past N: clamped, never stored
-    const uint8_t* const wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
-    const int64_t rb = (lane >> 4) < nb_last ? (lane >> 4) : nb_last;
-    const uint32_t woff = static_cast<uint32_t>(rb * a.w_kchunks * 256 + (lane & 15) * 16);
-    const int kc_last = static_cast<int>(a.w_kchunks) - 1;
-    const uint8_t* const xtile = xs.x + m0 * xs.ldx;
-    const int64_t m_last = a.M - 1 - m0;           // rows past M: clamped, never stored
-    const uint32_t ldsW = lds_address(sW), ldsX = lds_address(sX);
-    for (int p = 0; p < NP; ++p) {
+  const int64_t NB = ceil_div(a.N, 16);
+  const int64_t nb_last = NB - 1 - n0 / 16;        // 16-row blocks past N: clamped, never stored
+  const uint8_t* const wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
+  const int64_t rb = (lane >> 4) < nb_last ? (lane >> 4) : nb_last;
+  const uint32_t woff = static_cast<uint32_t>(rb * a.w_kchunks * 256 + (lane & 15) * 16);
+  const int kc_last = static_cast<int>(a.w_kchunks) - 1;
+  const uint8_t* const xtile = xs.x + m0 * xs.ldx;
+  const int64_t m_last = a.M - 1 - m0;             // rows past M: clamped, never stored
+  const uint32_t ldsW = lds_address(sW), ldsX = lds_address(sX);
+  uint32_t xrow_off[4];                            // this lane's row of the wave's four activation copies
+  int xslot[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int kc = p * kPhaseChunks + 4 * wave_u + i;
-        const int kcc = kc < kc_last ? kc : kc_last;   // (chunks past the packed pitch are never read)
-        lds_dma16(wtile + static_cast<int64_t>(kcc) * 256, woff, ldsW + static_cast<uint32_t>(kc) * 1024u);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int g = 4 * wave_u + i;                  // rows 4g .. 4g+3
-        const int r = 4 * g + (lane >> 4);
-        const int64_t rc = r < m_last ? r : m_last;
-        const int cc = p * kPhaseChunks + ((lane & 15) ^ (r & 15));
-        // chunks past K: any bytes of the row will do, the packed weight is zero there
-        const int ccc = cc < KC ? cc : KC - 1;
-        lds_dma16(xtile, static_cast<uint32_t>(rc * xs.ldx + ccc * 16),
-                  ldsX + static_cast<uint32_t>(p * BM + 4 * g) * 256u);
-      }
-    }
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * (4 * wave_u + i) + (lane >> 4);
+    const int64_t rc = r < m_last ? r : m_last;
+    xrow_off[i] = static_cast<uint32_t>(rc * xs.ldx);
+    xslot[i] = (lane & 15) ^ (r & 15);
   }
+  // the eight copies of this wave for phase p, into ring buffer p % kRing
+  auto issue = [&](int p) {
+    const int b = p & (kRing - 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int kc = p * kPhaseChunks + 4 * wave_u + i;
+      const int kcc = kc < kc_last ? kc : kc_last;   // (chunks past the packed pitch are never multiplied)
+      lds_dma16(wtile + static_cast<int64_t>(kcc) * 256, woff,
+                ldsW + static_cast<uint32_t>(b * kPhaseChunks + 4 * wave_u + i) * 1024u);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int cc = p * kPhaseChunks + xslot[i];
+      // chunks past K: any bytes of the row will do, they meet a zeroed operand or zero weights
+      const int ccc = cc < KC ? cc : KC - 1;
+      lds_dma16(xtile, xrow_off[i] + static_cast<uint32_t>(ccc) * 16u,
+                ldsX + static_cast<uint32_t>(b * BM + 4 * (4 * wave_u + i)) * 256u);
+    }
+  };
+  // waits until at most `phases` phases of this wave's copies (the youngest) are outstanding
+  auto wait_phases = [&](int phases) {
+    static_assert(kCopiesPerPhase == 8, "the wait counts below are multiples of the copies per phase");
+    switch (phases) {
+      case 0: __builtin_amdgcn_s_waitcnt((0 & 15) | ((0 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+      case 1: __builtin_amdgcn_s_waitcnt((8 & 15) | ((8 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+      case 2: __builtin_amdgcn_s_waitcnt((16 & 15) | ((16 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+      default: __builtin_amdgcn_s_waitcnt((24 & 15) | ((24 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
+    }
+  };
+
+  const int first = NP < kRing ? NP : kRing;
+  for (int p = 0; p < first; ++p) issue(p);
 
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor)};
@@ -110,53 +138,56 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
   const uint8_t* const wrd = sW + (wn0 + li) * 16;
   const uint8_t* const xrd = sX + xrow * 256;
 
-  for (int p = 0; p < NP; ++p) {
-    // the copies of the phases after this one may still be on their way
-    switch (NP - 1 - p) {
-      case 0: __builtin_amdgcn_s_waitcnt((0 & 15) | ((0 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
-      case 1: __builtin_amdgcn_s_waitcnt((8 & 15) | ((8 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
-      case 2: __builtin_amdgcn_s_waitcnt((16 & 15) | ((16 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
-      default: __builtin_amdgcn_s_waitcnt((24 & 15) | ((24 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
-    }
-    static_assert(kCopiesPerPhase == 8, "the wait counts above are multiples of the copies per phase");
-    __syncthreads();
-    if (p == 0 && t < BN) {
-      // the constants landed before the first phase: turn them into the
-      // accumulator's start value and the requantisation factors
-      const XQuant xq = x_quant(a);
-      const bool live = n0 + t < a.N;
-      float mult = 0.f, bdiv = 0.f;
-      if constexpr (MODE != kOutAcc32) {
-        const float ws = __int_as_float(s_raw[1][t]), bs = __int_as_float(s_raw[2][t]);
-        const float atw = xq.scale * ws;
-        if (MODE == kOutF32) {
-          mult = atw;
-          bdiv = a.bias != nullptr ? bs : 0.f;
-        } else {
-          mult = atw / a.out_scale;
-          bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, bs, atw) : 0.f;
-        }
+  wait_phases(first - 1);   // phase 0 (and, older than it, the constants) has landed
+  __syncthreads();
+  if (t < BN) {
+    // turn the constants into the accumulator's start value and the requantisation factors
+    const XQuant xq = x_quant(a);
+    const bool live = n0 + t < a.N;
+    float mult = 0.f, bdiv = 0.f;
+    if constexpr (MODE != kOutAcc32) {
+      const float ws = __int_as_float(s_raw[1][t]), bs = __int_as_float(s_raw[2][t]);
+      const float atw = xq.scale * ws;
+      if (MODE == kOutF32) {
+        mult = atw;
+        bdiv = a.bias != nullptr ? bs : 0.f;
+      } else {
+        mult = atw / a.out_scale;
+        bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, bs, atw) : 0.f;
       }
-      s_acc0[t] = live ? xq.coef * s_raw[0][t] : 0;
-      s_mult[t] = live ? mult : 0.f;
-      s_bdiv[t] = live ? bdiv : 0.f;
     }
-    const int s0 = p * (kPhaseChunks / 2);
-    const int nsteps = S - s0 < kPhaseChunks / 2 ? S - s0 : kPhaseChunks / 2;
+    s_acc0[t] = live ? xq.coef * s_raw[0][t] : 0;
+    s_mult[t] = live ? mult : 0.f;
+    s_bdiv[t] = live ? bdiv : 0.f;
+  }
+
+  for (int p = 0; p < NP; ++p) {
+    const int b = p & (kRing - 1);
+    const int left = S - p * (kPhaseChunks / 2);
+    const int nsteps = left < kPhaseChunks / 2 ? left : kPhaseChunks / 2;
     // (k-steps past the end of K in the last phase read whatever the buffers
     // hold and multiply it with a zeroed activation operand: no branches here)
     v4i wf[kPhaseChunks / 2], xf[kPhaseChunks / 2];
 #pragma unroll
     for (int j = 0; j < kPhaseChunks / 2; ++j) {
-      const int c = 2 * (s0 + j) + half;
-      wf[j] = ld16(wrd + c * (BN * 16));
-      xf[j] = ld16(xrd + p * (BM * 256) + (((c & 15) ^ (xrow & 15)) << 4));
+      const int c = 2 * j + half;
+      wf[j] = ld16(wrd + (b * kPhaseChunks + c) * (BN * 16));
+      xf[j] = ld16(xrd + b * (BM * 256) + ((c ^ (xrow & 15)) << 4));
     }
 #pragma unroll
     for (int j = 0; j < kPhaseChunks / 2; ++j) {
       const int keep = j < nsteps ? -1 : 0;
       const v4i xv = (xf[j] ^ xmask) & v4i{keep, keep, keep, keep};
       acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xv, acc, 0, 0, 0);
+    }
+    if (p + 1 < NP) {
+      // Phase p+1 must have landed; what this wave may still have on its way are
+      // the phases after it that were already requested (up to p+3).  Behind the
+      // barrier every wave is done with buffer p % kRing, which takes phase p+kRing.
+      const int youngest = p + kRing - 1 < NP - 1 ? p + kRing - 1 : NP - 1;
+      wait_phases(youngest - (p + 1));
+      __syncthreads();
+      if (p + kRing < NP) issue(p + kRing);
     }
   }
 

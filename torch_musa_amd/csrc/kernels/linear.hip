@@ -799,10 +799,10 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     if (forced == 13) return TMQ_ERR_UNSUPPORTED;
   }
   // all of K in LDS: 32-bit offsets over 64 rows of either operand, N * 4 as a 32-bit offset
-  const bool onepass_ok = a.K <= kOnePassMaxK && a.K % 16 == 0 && xs.ldx <= (int64_t{1} << 23) &&
+  const bool onepass_ok = a.K % 16 == 0 && a.K <= (int64_t{1} << 23) && xs.ldx <= (int64_t{1} << 23) &&
                           a.N + a.n_off < (int64_t{1} << 29) && a.splits == 1;
   int cfg = forced;
-  if (cfg < 0 && onepass_ok && ceil_div(a.M, 64) * ceil_div(a.N, 64) <= 256) {
+  if (cfg < 0 && onepass_ok && a.K <= kOnePassMaxK && ceil_div(a.M, 64) * ceil_div(a.N, 64) <= 256) {
     // short K on a grid no larger than the chip: one latency instead of one per stage
     // (M = 128, K = N = 1024: 6.0 -> 4.x us)
     cfg = 21;
@@ -832,6 +832,15 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
       cfg = rounds128x256 < rounds256 ? cfg128x256 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
     else if (nblk(128, 256) >= 160 && rows_used(128))
       cfg = cfg128x256;
+    else if (a.N >= 2048 && nblk(64, 64) > 256 && nblk(64, 128) <= 256)
+      // a few hundred rows whose 128 x 128 tiles would leave half the chip idle and whose
+      // 64 x 64 tiles need a second round: 64 rows x 128 channels, one round (K = N = 4096,
+      // cold weights: M = 448: 24.6 -> 19.1 us, M = 512: 24.8 -> 19.3 us; K = 2048: 14.7 -> 11.7 us;
+      // N = 8192, M = 192: 25.9 -> 19.9 us; against N = 1024 the 128 x 128 tiles stay ahead:
+      // M = 1536, K = 4096: 17.4 against 20.2 us)
+      cfg = 23;
+    else if (a.N >= 2048 && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
+      cfg = 22;
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
     else if (nblk(64, 64) <= 256 && ceil_div(a.K, kBK) >= 32 && ceil_div(a.K, kBK) % 2 == 0)
@@ -865,6 +874,8 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 17: return launch_gemm<128, 256, 2, 4, MODE, 3, true>(a, xs, s);
     case 19: return launch_gemm<128, 256, 2, 4, MODE, 3, true, 1, true>(a, xs, s);
     case 20: return launch_gemm_persistent<MODE>(a, xs, s);
+    case 22: return launch_gemm<128, 64, 2, 2, MODE>(a, xs, s);
+    case 23: return launch_gemm<64, 128, 2, 2, MODE>(a, xs, s);
     case 21: return onepass_ok ? launch_gemm_onepass<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
     default: return TMQ_ERR_UNSUPPORTED;
   }
