@@ -1039,6 +1039,74 @@ def test_silu_conv_qat_on_gpu_then_int8():
     assert steps <= 1.01, steps
 
 
+def test_fake_quantize_ops_on_gpu_tensors():
+    """The fake-quantize operators quantization-aware training runs on (the reference tests
+    its own device kernels for them, test_quantized_ops.py:465-700) are PyTorch-ROCm's own
+    GPU kernels here; each gives the CPU op's values to 1e-6 (relative for the summed gradients), masks included."""
+    say("fake-quantize ops against the CPU ops")
+    torch.manual_seed(9)
+    aten = torch.ops.aten
+
+    def close(got, want):
+        got = got if isinstance(got, (tuple, list)) else (got,)
+        want = want if isinstance(want, (tuple, list)) else (want,)
+        for g_, w_ in zip(got, want):
+            assert g_.is_cuda and g_.dtype == w_.dtype and g_.shape == w_.shape
+            if w_.dtype == torch.bool:
+                assert torch.equal(g_.cpu(), w_)
+            else:
+                # (summed gradients: the order of the sum differs, so relative to their size)
+                assert (g_.cpu().double() - w_.double()).abs().max().item() <= 1e-6 * max(1.0, w_.abs().max().item())
+
+    for shape, qmin, qmax, axis in (((2, 2), 0, 255, 1), ((2, 3, 16), 0, 255, 1), ((1, 4, 8, 8), 0, 127, 1),
+                                    ((2, 2, 32), 0, 240, 1)):
+        x = torch.randn(shape) * 4
+        scale = torch.rand(shape[axis]) * 0.1 + 0.01
+        zp = torch.randint(0, 10, (shape[axis],)).float()
+        close(aten.fake_quantize_per_channel_affine_cachemask(x.cuda(), scale.cuda(), zp.cuda(), axis, qmin, qmax),
+              aten.fake_quantize_per_channel_affine_cachemask(x, scale, zp, axis, qmin, qmax))
+        outs = []
+        for dev_ in ("cpu", "cuda"):
+            xi, si, zi = (t.clone().to(dev_).requires_grad_(True) for t in (x, scale, zp))
+            y = aten._fake_quantize_learnable_per_channel_affine(xi, si, zi, axis, qmin, qmax, 1.0)
+            y.sum().backward()
+            outs.append((y.detach(), xi.grad, si.grad, zi.grad))
+        close(outs[1], outs[0])
+    for shape, qmin, qmax, scale, zp in (((2, 2), 0, 255, 0.1, 4), ((2, 3, 16), 0, 255, 0.2, 254),
+                                         ((1, 4, 8, 8), 0, 127, 10.0, 1), ((2, 2, 32), 10, 240, 1.0, 100)):
+        x = torch.randn(shape) * 40
+        s_t, z_t = torch.tensor(scale), torch.tensor(zp, dtype=torch.int)
+        close(aten.fake_quantize_per_tensor_affine_cachemask(x.cuda(), scale, zp, qmin, qmax),
+              aten.fake_quantize_per_tensor_affine_cachemask(x, scale, zp, qmin, qmax))
+        on = torch.tensor(1, dtype=torch.long)
+        close(aten._fake_quantize_per_tensor_affine_cachemask_tensor_qparams(x.cuda(), s_t.cuda(), z_t.cuda(),
+                                                                             on.cuda(), qmin, qmax),
+              aten._fake_quantize_per_tensor_affine_cachemask_tensor_qparams(x, s_t, z_t, on, qmin, qmax))
+        outs = []
+        for dev_ in (("cpu", "cuda") if qmin == 0 else ()):   # (the learnable form wants 0 inside the range)
+            xi = x.clone().to(dev_).requires_grad_(True)
+            si = torch.tensor([scale], device=dev_, requires_grad=True)
+            zi = torch.tensor([float(zp)], device=dev_, requires_grad=True)
+            y = aten._fake_quantize_learnable_per_tensor_affine(xi, si, zi, qmin, qmax, 1.0)
+            y.sum().backward()
+            outs.append((y.detach(), xi.grad, si.grad, zi.grad))
+        if outs:
+            close(outs[1], outs[0])
+    # the fused observer + fake-quantize step of torch.ao's FusedMovingAvgObsFakeQuantize
+    x = torch.randn(4, 8, 6, 6)
+    outs = []
+    for dev_ in ("cpu", "cuda"):
+        st = dict(obs=torch.tensor(1, dtype=torch.int, device=dev_), fq=torch.tensor(1, dtype=torch.int, device=dev_),
+                  mn=torch.tensor([float("inf")], device=dev_), mx=torch.tensor([float("-inf")], device=dev_),
+                  sc=torch.ones(1, device=dev_), zp=torch.zeros(1, dtype=torch.int, device=dev_))
+        y = None
+        for k in range(3):
+            y = torch.fused_moving_avg_obs_fake_quant(x.to(dev_) * (k + 1), st["obs"], st["fq"], st["mn"], st["mx"],
+                                                      st["sc"], st["zp"], 0.01, 0, 255, 0, False, False)
+        outs.append((y, st["mn"], st["mx"], st["sc"], st["zp"]))
+    close(outs[1], outs[0])
+
+
 def test_ops_replay_from_a_hip_graph():
     """The operators inside a captured HIP graph (allocations from the graph's pool, no
     host round trip in the captured region): quantized::linear on a split-K shape and on a
