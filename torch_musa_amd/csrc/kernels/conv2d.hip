@@ -327,14 +327,18 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
                : launch_conv_tiles_variant<MODE, 1, false>(s, p, a, stream);
   } else {
     const bool vec = (a.OC & 15) == 0 && (a.OCg & 15) == 0 && aligned16;
-    const int kind = a.post.any() ? 0 : ((MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f) ? 2 : 1);
+    const int kind = a.post.silu ? 3
+                     : a.post.accum != nullptr ? 0
+                     : ((MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f) ? 2 : 1);
     switch (kind * 2 + (vec ? 1 : 0)) {
       case 0: return launch_conv_tiles_variant<MODE, 0, false>(s, p, a, stream);
       case 1: return launch_conv_tiles_variant<MODE, 0, true>(s, p, a, stream);
       case 2: return launch_conv_tiles_variant<MODE, 1, false>(s, p, a, stream);
       case 3: return launch_conv_tiles_variant<MODE, 1, true>(s, p, a, stream);
       case 4: return launch_conv_tiles_variant<MODE, 2, false>(s, p, a, stream);
-      default: return launch_conv_tiles_variant<MODE, 2, true>(s, p, a, stream);
+      case 5: return launch_conv_tiles_variant<MODE, 2, true>(s, p, a, stream);
+      case 6: return launch_conv_tiles_variant<MODE, 3, false>(s, p, a, stream);
+      default: return launch_conv_tiles_variant<MODE, 3, true>(s, p, a, stream);
     }
   }
 }

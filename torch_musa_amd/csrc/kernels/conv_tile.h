@@ -74,14 +74,15 @@ __device__ __forceinline__ uint32_t small_div(uint32_t n, uint32_t d, float rcp)
   return q;
 }
 
-// KIND selects the requantisation compiled in: 0 residual / SiLU, 1 plain with
-// clamp, 2 plain for unsigned output without ReLU (the saturating pack
-// conversion is the clamp).  VEC: output rows take aligned 16-byte (int32 mode:
+// KIND selects the requantisation compiled in: 0 a residual and no SiLU, 3 SiLU
+// (with a residual if there is one), 1 plain with clamp, 2 plain for unsigned
+// output without ReLU (the saturating pack conversion is the clamp).  VEC: output rows take aligned 16-byte (int32 mode:
 // 4-channel) stores.  One variant per launch keeps the straight-line code that
 // every wave runs exactly once small: the kernel with all variants inside was
 // five times longer and spent a quarter of its time fetching instructions.
 template <int MODE, int KIND, bool VEC>
 __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
+  constexpr bool kPost = KIND == 0 || KIND == 3;  // the epilogue with post operations
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ __attribute__((aligned(16))) int s_acc0[kCtBN];
   __shared__ __attribute__((aligned(16))) float s_mult[kCtBN];
@@ -268,9 +269,9 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
     // Otherwise: the words themselves, byte by byte.
     uint32_t accw[TM][8];
     v4i accv[TM][2];
-    const bool res_rows = KIND == 0 && VEC && a.post.accum != nullptr && n0 + kCtBN <= a.OCg &&
+    const bool res_rows = kPost && VEC && a.post.accum != nullptr && n0 + kCtBN <= a.OCg &&
                           ((reinterpret_cast<uintptr_t>(a.post.accum) | static_cast<uintptr_t>(a.OC)) & 15) == 0;
-    if (KIND == 0 && a.post.accum != nullptr) {
+    if (kPost && a.post.accum != nullptr) {
       if (res_rows) {
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
       uint8_t* y = static_cast<uint8_t*>(a.y);
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
-        if (KIND == 0 && res_rows) {  // residual pixels -> this lane's words, through the staging rows
+        if (kPost && res_rows) {  // residual pixels -> this lane's words, through the staging rows
 #pragma unroll
           for (int pass = 0; pass < 2; ++pass)
             *reinterpret_cast<v4i*>(sT + (pass * 16 + (lane >> 2)) * kCtTPitch + (lane & 3) * 16) = accv[tm][pass];
@@ -384,8 +385,9 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
 #pragma unroll
               for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * gq + j];
               uint32_t q4;
-              if constexpr (KIND == 0)
-                q4 = requant4_post<MODE>(raw, bdiv, bmul, mult, a.post, accw[tm][tn * 4 + gq], a.zp_f, a.lo_f, a.hi_f);
+              if constexpr (kPost)
+                q4 = requant4_post<MODE, KIND == 0 ? 1 : 2>(raw, bdiv, bmul, mult, a.post, accw[tm][tn * 4 + gq],
+                                                            a.zp_f, a.lo_f, a.hi_f);
               else
                 q4 = requant4<MODE, KIND == 1>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
               *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) = q4;
@@ -421,7 +423,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
   // residual rows and the stores of the first tile then run under the k loop of
   // the second, and the two waves of a SIMD drift out of phase (C5 with a residual
   // and ReLU: 14.3 -> 13.5 us per launch; without a residual it changes nothing).
-  while (KIND != 0 && count >= 2) {
+  while (!kPost && count >= 2) {
     run(std::integral_constant<int, 2>{}, first);
     first += 2;
     count -= 2;

@@ -326,24 +326,31 @@ __device__ __forceinline__ uint32_t load_accum4(const PostOps& p, int64_t off, i
   return w;
 }
 
-// requant4 with the post operations (see PostOps) before the rounding.
-template <int MODE>
+// requant4 with the post operations (see PostOps) before the rounding.  POST says
+// what the caller knows at compile time: 0 nothing (both operations are looked up
+// in `p`), 1 a residual and no SiLU, 2 SiLU (a residual if `p` has one).
+template <int MODE, int POST = 0>
 __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv, float bmul, v4f mult,
                                                   const PostOps& p, uint32_t accw, float zp_f,
                                                   float lo_f, float hi_f) {
   uint32_t packed = 0;
+  // The residual bytes are taken as unsigned values (one conversion instruction
+  // per byte): a signed byte s equals (s ^ 0x80) - 128, so the word is flipped
+  // once and 128 joins the zero point.  Both terms of the difference are small
+  // integers, exact in fp32, so it equals float(q - zero_point).
+  const uint32_t accu = p.accum_signed ? accw ^ 0x80808080u : accw;
+  const float acc_zp_f = static_cast<float>(p.accum_zp + (p.accum_signed ? 128 : 0));
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     float v = static_cast<float>(raw[j]);
     v = __builtin_fmaf(bdiv[j], bmul, v);
     float t = v * mult[j];
-    if (p.accum != nullptr) {
-      const uint32_t b = (accw >> (8 * j)) & 0xffu;
-      const int qa = p.accum_signed ? static_cast<int>(static_cast<int8_t>(b)) : static_cast<int>(b);
-      const float a = static_cast<float>(qa - p.accum_zp) * p.amult;
+    if (POST == 1 || p.accum != nullptr) {
+      const float qf = static_cast<float>((accu >> (8 * j)) & 0xffu);
+      const float a = (qf - acc_zp_f) * p.amult;
       t = t + a;
     }
-    if (p.silu) {
+    if (POST == 2 || (POST == 0 && p.silu)) {
       const float r = t * p.out_scale;
       const float e = expf(-r);
       const float d = 1.0f + e;
