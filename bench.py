@@ -48,13 +48,13 @@ def _traffic(fetch_kib, write_kib):
 MEASURED_TRAFFIC = {
     "linear_c3": _traffic(161_135, 44_032),       # 375 MB: operands re-fetched 5.3x by the 8 L2s
     "quantize_c2": _traffic(524_304, 262_144),    # 1.342 GB = algorithmic
-    "dequantize_c2": _traffic(131_084, 1_048_913),
-    "minmax_c2": _traffic(524_312, 64),
+    "dequantize_c2": _traffic(131_084, 1_048_986),
+    "minmax_c2": _traffic(524_315, 64),
     "quantize_pc": _traffic(88_805, 44_032),
-    "dequantize_pc": _traffic(23_422, 176_208),
+    "dequantize_pc": _traffic(23_422, 176_218),
     "decode_m1": _traffic(8_300, 8),              # 17.0 MB for 16.8 MB algorithmic
     "conv_c5": _traffic(3_940, 6_272),            # 14.5 MB for 12.9 MB algorithmic (halo overlap)
-    "conv_add_relu_c5": _traffic(7_140, 6_272),
+    "conv_add_relu_c5": _traffic(7_066, 6_272),
 }
 
 
