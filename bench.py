@@ -297,6 +297,66 @@ def main():
             probe[name] = {"tops": round(tops_p, 1), "shader_ghz": round(ghz_p, 3)}
             log(f"[bench]   {name}: {tops_p:.0f} TOP/s at {ghz_p:.2f} GHz")
         secondary["mfma_i8_ceiling_probe"] = probe
+
+        # ---------------------------------------------- where a C3 launch spends its time
+        # The instrumented instantiation of the persistent GEMM (measurement library) writes
+        # wall-clock and cycle stamps per block and tile; with the copies left out (results
+        # wrong) it also says what the operand traffic costs in clock and cycles.
+        log("[bench] time budget of a config 3 launch (instrumented kernel, stamps per block and tile)")
+        pw_b = cabi.PackedLinear(wq.int_repr())
+        ws_b = w_scales.to(torch.float32)
+        x_b = xq.int_repr()
+        y_b = torch.empty((M, N), dtype=torch.uint8, device=dev)
+
+        def budget_once(flags):
+            for _ in range(20):
+                step()
+            st = cabi.bench_linear_stamps(x_b, pw_b, xq.q_scale(), xq.q_zero_point(), ws_b, bias, out_scale, out_zp,
+                                          y_b, flags)
+            torch.cuda.synchronize()
+            return st.cpu().numpy().astype(np.float64)
+
+        def summarise(st):
+            wall, cyc = st[:, 0, :] / 100.0, st[:, 1, :]          # us, cycles
+            tiles_total = ((M + 255) // 256) * ((N + 255) // 256)
+            ntile = np.where(np.arange(256) < tiles_total - 2 * 256, 3, 2)
+            out = {"launch_us": round(float(max(wall[i, 4 * ntile[i]] for i in range(256)) - wall[:, 0].min()), 1),
+                   "first_operands_us": round(float(np.mean(wall[:, 1] - wall[:, 0])), 2)}
+            for t, name in ((0, "round_1"), (1, "round_2"), (2, "round_3")):
+                sel = ntile > t
+                ls, le, lb, ee = (wall[sel, 1 + 4 * t + k] for k in range(4))
+                cl = cyc[sel, 2 + 4 * t] - cyc[sel, 1 + 4 * t]
+                ce = cyc[sel, 4 + 4 * t] - cyc[sel, 3 + 4 * t]
+                out[name] = {"blocks": int(sel.sum()), "loop_us": round(float(np.mean(le - ls)), 2),
+                             "loop_cycles": int(np.mean(cl)),
+                             "shader_ghz_in_loop": round(float(np.mean(cl) / np.mean(le - ls) / 1e3), 3),
+                             "barrier_us": round(float(np.mean(lb - le)), 2),
+                             "epilogue_us": round(float(np.mean(ee - lb)), 2), "epilogue_cycles": int(np.mean(ce))}
+            return out
+
+        for _ in range(300):
+            step()
+        torch.cuda.synchronize()
+        # the four variants in turn, seven times over; per variant the launch with the median full-round loop time
+        names = ("all_copies", "no_activation_copies", "no_weight_copies", "no_copies")
+        runs = {n: [] for n in names}
+        for _ in range(7):
+            for f, n in enumerate(names):
+                runs[n].append(summarise(budget_once(f)))
+        tb = {n: sorted(r, key=lambda o: o["round_1"]["loop_us"])[len(r) // 2] for n, r in runs.items()}
+        tb["full_round_loop_us_all_launches"] = {n: [o["round_1"]["loop_us"] for o in r] for n, r in runs.items()}
+        tb["matrix_pipe_cycles_per_tile"] = (K // 64) * 512
+        tb["method"] = ("single launches of gemm_i8_persistent_kernel<kOutU8, STAMPS, SKIP> after 20 operator steps "
+                        "each, the four variants in turn, seven times; thread 0 of every block stamps the 100 MHz wall "
+                        "clock and the shader cycle counter; the variants without copies multiply stale operands "
+                        "(timing only); reported per variant: the launch with the median full-round loop time")
+        secondary["linear_c3_time_budget"] = tb
+        r1 = tb["all_copies"]["round_1"]
+        log(f"[bench]   full round: loop {r1['loop_us']} us = {r1['loop_cycles']} cycles at {r1['shader_ghz_in_loop']} GHz "
+            f"(matrix pipe alone: {tb['matrix_pipe_cycles_per_tile']}), epilogue {r1['epilogue_cycles']} cycles; last round "
+            f"at {tb['all_copies']['round_3']['shader_ghz_in_loop']} GHz; without copies "
+            f"{tb['no_copies']['round_1']['loop_us']} us at {tb['no_copies']['round_1']['shader_ghz_in_loop']} GHz")
+        del pw_b, x_b, y_b
         roofline["power_limited_ceiling_tops"] = probe["gaussian_int8"]["tops"]
         roofline["frac_of_power_limited_ceiling"] = round(achieved / probe["gaussian_int8"]["tops"], 4)
         # the same with operands that change every instruction, as a GEMM's do

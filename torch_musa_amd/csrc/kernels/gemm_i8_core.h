@@ -102,6 +102,9 @@ struct GemmArgs {
   int32_t splits = 1;
   int32_t split_stages = 0;
   int64_t split_stride = 0;
+  // Instrumented builds of a kernel only (the measurement library): where the
+  // blocks write their time stamps.
+  uint64_t* stamps = nullptr;
 };
 
 struct XQuant {
