@@ -59,9 +59,9 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
   const int wave_u = __builtin_amdgcn_readfirstlane(t / kWave);
   const int li = lane & 31, half = lane >> 5;
   const int wm0 = (wave_u & 1) * 32, wn0 = (wave_u >> 1) * 32;
-  const int64_t tiles_n = ceil_div(a.N, BN);
-  const int64_t m0 = (static_cast<int64_t>(blockIdx.x) / tiles_n) * BM;
-  const int64_t n0 = (static_cast<int64_t>(blockIdx.x) % tiles_n) * BN;
+  // grid (channel tiles, row tiles): no division to find the tile
+  const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * BN;
   const int KC = static_cast<int>(a.K >> 4);       // k-chunks (K is a multiple of 16)
   const int S = (KC + 1) >> 1;                     // 32-byte k-steps
   const int NP = (KC + kPhaseChunks - 1) / kPhaseChunks;   // phases of 256 bytes of K

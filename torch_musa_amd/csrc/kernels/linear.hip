@@ -502,9 +502,10 @@ int launch_gemm(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
 // 64 x 64 tiles with all of K in LDS (K <= 1024; the caller checked the address ranges).
 template <int MODE>
 int launch_gemm_onepass(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
-  const int64_t blocks = ceil_div(a.M, 64) * ceil_div(a.N, 64);
-  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-  gemm_i8_onepass_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(a, xs);
+  const int64_t tiles_m = ceil_div(a.M, 64), tiles_n = ceil_div(a.N, 64);
+  if (tiles_n > 0x7fffffff || tiles_m > 65535) return TMQ_ERR_UNSUPPORTED;
+  gemm_i8_onepass_kernel<MODE>
+      <<<dim3(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m)), dim3(256), 0, s>>>(a, xs);
   return launch_status();
 }
 
