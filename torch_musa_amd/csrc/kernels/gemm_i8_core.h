@@ -479,22 +479,26 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   // its own L2: give every XCD one contiguous run of the tile sequence, and order
   // the sequence so that the ~32 tiles an XCD runs at once form a compact patch
   // (kGroupN channel tiles wide, row tiles next) that shares operand tiles.
-  const int64_t tiles_m = ceil_div(a.M, BM), tiles_n = ceil_div(a.N, BN);
-  const int64_t nblocks = tiles_m * tiles_n;
-  int64_t tile;
+  // (32-bit arithmetic: the host launches fewer than 2**31 blocks, and a 64-bit
+  // division costs a block that is alone on its CU a hundred instructions before
+  // its first load)
+  const uint32_t tiles_m = static_cast<uint32_t>(ceil_div(a.M, BM)), tiles_n = static_cast<uint32_t>(ceil_div(a.N, BN));
+  const uint32_t nblocks = tiles_m * tiles_n;
+  uint32_t tile;
   {
-    const int64_t bid = blockIdx.x;
-    const int64_t q = nblocks / 8, rem = nblocks % 8;
-    const int64_t xcd = bid % 8, within = bid / 8;
+    const uint32_t bid = blockIdx.x;
+    const uint32_t q = nblocks / 8, rem = nblocks % 8;
+    const uint32_t xcd = bid % 8, within = bid / 8;
     tile = xcd * q + (xcd < rem ? xcd : rem) + within;
   }
-  constexpr int64_t kGroupN = 4;
-  const int64_t group = tile / (tiles_m * kGroupN);
-  const int64_t gfirst = group * kGroupN;
-  const int64_t gwidth = tiles_n - gfirst < kGroupN ? tiles_n - gfirst : kGroupN;
-  const int64_t in_group = tile - group * (tiles_m * kGroupN);
-  const int64_t m0 = (in_group / gwidth) * BM;
-  const int64_t n0 = (gfirst + in_group % gwidth) * BN;
+  constexpr uint32_t kGroupN = 4;
+  const uint32_t group = tile / (tiles_m * kGroupN);
+  const uint32_t gfirst = group * kGroupN;
+  const uint32_t gwidth = tiles_n - gfirst < kGroupN ? tiles_n - gfirst : kGroupN;
+  const uint32_t in_group = tile - group * (tiles_m * kGroupN);
+  const uint32_t tile_row = in_group / gwidth;
+  const int64_t m0 = static_cast<int64_t>(tile_row) * BM;
+  const int64_t n0 = static_cast<int64_t>(gfirst + in_group - tile_row * gwidth) * BN;
   const int64_t NB = ceil_div(a.N, 16);
 
   // ---- per-channel constants of this tile's BN output channels, then the

@@ -833,14 +833,14 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
       cfg = rounds128x256 < rounds256 ? cfg128x256 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
     else if (nblk(128, 256) >= 160 && rows_used(128))
       cfg = cfg128x256;
-    else if (a.N >= 2048 && nblk(64, 64) > 256 && nblk(64, 128) <= 256)
+    else if (a.N >= 2048 && (a.N >= 4096 || a.K >= 4096) && nblk(64, 64) > 256 && nblk(64, 128) <= 256)
       // a few hundred rows whose 128 x 128 tiles would leave half the chip idle and whose
       // 64 x 64 tiles need a second round: 64 rows x 128 channels, one round (K = N = 4096,
       // cold weights: M = 448: 24.6 -> 19.1 us, M = 512: 24.8 -> 19.3 us; K = 2048: 14.7 -> 11.7 us;
       // N = 8192, M = 192: 25.9 -> 19.9 us; against N = 1024 the 128 x 128 tiles stay ahead:
-      // M = 1536, K = 4096: 17.4 against 20.2 us)
+      // M = 1536, K = 4096: 17.4 against 20.2 us, and at K = N = 2048, M = 1024: 11.5 against 12.2 us)
       cfg = 23;
-    else if (a.N >= 2048 && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
+    else if (a.N >= 2048 && (a.N >= 4096 || a.K >= 4096) && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
       cfg = 22;
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
