@@ -350,6 +350,17 @@ def main():
                         "each, the four variants in turn, seven times; thread 0 of every block stamps the 100 MHz wall "
                         "clock and the shader cycle counter; the variants without copies multiply stale operands "
                         "(timing only); reported per variant: the launch with the median full-round loop time")
+        # Does the order of the work matter?  Blocks that have slack (two tiles instead of
+        # three) start 40 us late; every second CU of each XCD starts 24 us late, so that the
+        # halves of the chip reach their epilogues at different times.  Same output bytes.
+        late = {"none": 0, "two_tile_blocks_40us_late": 40 << 8, "every_second_cu_24us_late": (24 << 8) | (1 << 4)}
+        late_runs = {n: [] for n in late}
+        for _ in range(5):
+            for n, f in late.items():
+                late_runs[n].append(summarise(budget_once(f))["launch_us"])
+        tb["late_start_launch_us"] = {n: float(np.median(r)) for n, r in late_runs.items()}
+        tb["late_start_method"] = ("the same instrumented kernel with a bounded wait on the wall clock before a block's "
+                                   "first copy; launch = first block start to last epilogue end; median of 5, in turn")
         secondary["linear_c3_time_budget"] = tb
         r1 = tb["all_copies"]["round_1"]
         log(f"[bench]   full round: loop {r1['loop_us']} us = {r1['loop_cycles']} cycles at {r1['shader_ghz_in_loop']} GHz "

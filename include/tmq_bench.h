@@ -50,6 +50,9 @@ int tmq_bench_empty_kernel(int blocks, void* sink, void* stream);
  * loop starts, 2 + 4t: main loop ends, 3 + 4t: behind the barrier after it,
  * 4 + 4t: epilogue ends.  flags & 1 leaves out the activation copies, flags & 2
  * the weight copies (stale operands: the output is wrong, for timing only).
+ * Bits 8..15 of flags: some blocks start that many microseconds late (a schedule
+ * experiment; same output) -- with bit 4 clear the blocks that have one tile
+ * fewer than the others, with bit 4 set every second compute unit of each XCD.
  * Asynchronous on `stream`. */
 int tmq_bench_linear_stamps(const tmq_linear_desc* desc, uint64_t* stamps, int flags, void* stream);
 

@@ -135,6 +135,19 @@ def test_instrumented_persistent_kernel_gives_the_same_bytes(cabi):
     np.testing.assert_array_equal(host(out2), y2)
     s2 = st2.cpu().numpy()                           # 18 x 17 = 306 tiles on 256 blocks: 50 blocks take a second one
     assert (s2[:50, 0, 8] > 0).all() and (s2[50:, 0, 8] == 0).all() and (s2[:, 0, 4] > 0).all()
+    # late starts (bits 8..15 of the flags: microseconds; bit 4: which blocks) change the
+    # timing, not the bytes: the one-tile blocks, then every second CU of an XCD
+    for flags, late_blocks in (((20 << 8), np.arange(256) >= 50), ((20 << 8) | (1 << 4), (np.arange(256) >> 3) % 2 == 1)):
+        out2.zero_()
+        st2.zero_()
+        cabi.check(cabi.bench_lib().tmq_bench_linear_stamps(C.byref(cabi_desc_relu), st2.data_ptr(), flags,
+                                                            cabi.stream_ptr()), "tmq_bench_linear_stamps")
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host(out2), y2)
+        s2 = st2.cpu().numpy()
+        first_copy = (s2[:, 0, 1] - s2[:, 0, 0]) / 100.0          # us from block start to loop start
+        assert (first_copy[late_blocks] >= 20.0).all() and (first_copy[~late_blocks] < 20.0).all()
+    assert cabi.bench_lib().tmq_bench_linear_stamps(C.byref(cabi_desc_relu), st2.data_ptr(), 4, cabi.stream_ptr()) != 0
 
 
 # all of K in LDS (K <= 1024): every number of 256-byte phases, K that ends inside a phase and on

@@ -58,7 +58,10 @@ TMQ_EXPORT int tmq_bench_linear_stamps(const tmq_linear_desc* d, uint64_t* stamp
   const int64_t grid = tiles <= cus ? tiles : cus / 8 * 8;  // as the product launches it
   const dim3 g(static_cast<unsigned>(grid)), b(kPersistThreads);
   hipStream_t s = as_stream(stream);
-  switch (flags) {  // what to leave out is compiled in: the instrumented loop has the product's instructions
+  a.late_ticks = static_cast<uint32_t>((flags >> 8) & 0xff) * 100u;  // microseconds of late start
+  a.late_mode = static_cast<uint32_t>((flags >> 4) & 1);
+  if ((flags & ~0xff13) != 0) return TMQ_ERR_INVALID_ARGUMENT;
+  switch (flags & 3) {  // what to leave out is compiled in: the instrumented loop has the product's instructions
     case 0: gemm_i8_persistent_kernel<kOutU8, true, 0><<<g, b, 0, s>>>(a, xs); break;
     case 1: gemm_i8_persistent_kernel<kOutU8, true, 1><<<g, b, 0, s>>>(a, xs); break;
     case 2: gemm_i8_persistent_kernel<kOutU8, true, 2><<<g, b, 0, s>>>(a, xs); break;

@@ -105,6 +105,10 @@ struct GemmArgs {
   // Instrumented builds of a kernel only (the measurement library): where the
   // blocks write their time stamps.
   uint64_t* stamps = nullptr;
+  // Instrumented builds only: the blocks late_mode selects wait late_ticks of the
+  // 100 MHz wall clock before their first copy.  0: nobody waits.
+  uint32_t late_ticks = 0;
+  uint32_t late_mode = 0;
 };
 
 struct XQuant {

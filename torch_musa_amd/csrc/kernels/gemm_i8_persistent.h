@@ -37,7 +37,8 @@ constexpr int kPersistThreads = 512;
 // counter to a.stamps[block][2][16] at the block's start and, per tile, when its
 // main loop starts, when it ends, behind the barrier after it and when the
 // epilogue ends; SKIP & 1 leaves out the activation copies, SKIP & 2 the weight
-// copies (stale operands: wrong results, for timing only).
+// copies (stale operands: wrong results, for timing only); a.late_ticks delays
+// the start of some blocks (same results, for timing only).
 template <int MODE, bool STAMPS = false, int SKIP = 0>
 __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(GemmArgs a, XLinear xsrc) {
   static_assert(MODE == kOutU8 || MODE == kOutS8 || MODE == kOutF32, "byte or float outputs");
@@ -380,6 +381,18 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   stamp();
   uint32_t v = blockIdx.x;
   if (v >= nblocks) return;
+  if constexpr (STAMPS) {
+    if (a.late_ticks != 0) {
+      // A schedule experiment: some blocks wait before their first copy (a bounded
+      // wait on the wall clock).  Mode 0: the blocks with one tile fewer than the
+      // others, which have that slack; mode 1: every second CU of each XCD, so that
+      // the halves of the chip reach their epilogues at different times.
+      const uint32_t part = nblocks % gridDim.x;
+      const bool waits = a.late_mode == 0 ? (part != 0 && blockIdx.x >= part) : ((blockIdx.x >> 3) & 1) != 0;
+      const uint64_t t0 = wall_clock64();
+      for (int i = 0; waits && i < 400 && wall_clock64() - t0 < a.late_ticks; ++i) __builtin_amdgcn_s_sleep(8);
+    }
+  }
   int m0, n0;
   tile_origin(v, &m0, &n0);
   tile_setup(m0, n0);
