@@ -89,13 +89,13 @@ def test_per_tensor_weight_bias_form(cabi, golden, cfg):
 
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23, 24])
 @pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),
                                    (270, 300, 400), (40, 70, 784)])
 def test_tile_configs(cabi, cfg, shape):
     say("tile cfg", cfg, shape)
-    if cfg == 21 and shape[2] > 1024:
-        pytest.skip("the kernel that holds all of K in LDS takes K <= 1024")
+    if cfg == 24 and shape[2] > 1024:
+        pytest.skip("the 32 x 32 tiles whose waves split K take K <= 1024")
     c = _tile_case(*shape, seed=cfg * 10 + shape[0])
     y, acc, _ = _run(cabi, c, cfg)
     np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]))
@@ -155,19 +155,20 @@ def test_instrumented_persistent_kernel_gives_the_same_bytes(cabi):
 @pytest.mark.parametrize("shape", [(128, 1024, 1024), (1, 16, 16), (64, 64, 32), (65, 70, 48), (100, 130, 1008),
                                    (33, 200, 272), (257, 129, 528), (1000, 1000, 1024), (90, 33, 784)])
 @pytest.mark.parametrize("x_signed", [False, True])
-def test_whole_k_in_lds_kernel(cabi, shape, x_signed):
-    say("K in LDS", shape, x_signed)
+@pytest.mark.parametrize("cfg", [21, 24])    # 64 x 64 tiles; 32 x 32 tiles whose waves split K
+def test_whole_k_in_lds_kernel(cabi, shape, x_signed, cfg):
+    say("K in LDS", shape, x_signed, cfg)
     M, N, K = shape
     c = _tile_case(M, N, K, seed=2100 + M, x_signed=x_signed, relu=N % 2 == 1, bias=M % 3 != 0,
                    per_channel=(M + N) % 2 == 0)
-    y, acc, pw = _run(cabi, c, 21)
+    y, acc, pw = _run(cabi, c, cfg)
     np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
     want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
                          c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
     _check(y, want, "K in LDS")
     ws = dev(c["w_scales"].astype(np.float32))
     b = None if c["bias"] is None else dev(c["bias"])
-    cabi.force_linear_config(21)
+    cabi.force_linear_config(cfg)
     try:
         yf = host(cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, relu=c["relu"]))
     finally:
@@ -473,7 +474,7 @@ def test_split_k_workspace_rules(cabi):
 # Float results are compared bit for bit: the kernel's epilogue is the oracle's
 # single fused multiply-add, and the dynamic quantization in front of it is
 # bit-exact by the quantizer tests.
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20, 21, 22, 23])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20, 21, 22, 23, 24])
 @pytest.mark.parametrize("shape,relu,bias,pc,x_signed", [((60, 264, 448), False, True, True, False),
                                                          ((257, 33, 144), True, True, False, False),
                                                          ((16, 1040, 1168), False, False, True, True)])
@@ -482,8 +483,8 @@ def test_linear_f32_configs(cabi, cfg, shape, relu, bias, pc, x_signed):
     c = _tile_case(*shape, seed=300 + cfg, x_signed=x_signed, relu=relu, bias=bias, per_channel=pc)
     if cfg == 8 and shape[0] > 64:
         pytest.skip("the weight-streaming kernel takes at most 64 rows")
-    if cfg == 21 and shape[2] > 1024:
-        pytest.skip("the kernel that holds all of K in LDS takes K <= 1024")
+    if cfg == 24 and shape[2] > 1024:
+        pytest.skip("the 32 x 32 tiles whose waves split K take K <= 1024")
     pw = cabi.PackedLinear(dev(c["wq"]))
     ws = dev(c["w_scales"].astype(np.float32))
     b = None if c["bias"] is None else dev(c["bias"])

@@ -281,6 +281,26 @@ def test_qmaxpool2d(cabi, golden, c):
     np.testing.assert_array_equal(y, want)
 
 
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("geom", [((3, 17, 19, 32), (2, 2), (1, 1)), ((2, 9, 30, 16), (1, 1), (1, 1)),
+                                  ((1, 12, 12, 48), (2, 1), (0, 1)), ((2, 8, 8, 16), (3, 3), (1, 0)),
+                                  ((1, 3, 3, 16), (1, 1), (1, 1))])
+def test_qmaxpool_3x3_sixteen_channel_kernels(cabi, signed, geom):
+    """The 3 x 3 kernels that take 16 channels per thread compare bytes as 16-bit lanes:
+    extreme codes, runs of equal codes and both code types against the oracle."""
+    shape, stride, padding = geom
+    say("qmaxpool 3x3 x16", shape, stride, padding, signed)
+    rng = np.random.default_rng(hash((shape, stride, padding, signed)) % (1 << 31))
+    lo, hi = (-128, 128) if signed else (0, 256)
+    x = rng.integers(lo, hi, shape).astype(np.int8 if signed else np.uint8)
+    x[rng.random(shape) < 0.2] = lo                       # many taps at the lowest code
+    x[rng.random(shape) < 0.1] = hi - 1
+    x[0, : shape[1] // 2] = np.where(rng.random((shape[1] // 2,) + shape[2:]) < 0.5, -1 if signed else 127, 0 if signed else 128)
+    want = oracle.qmaxpool2d(x, (3, 3), stride, padding)
+    y = host(cabi.qmaxpool2d(dev(x), (3, 3), stride, padding, (1, 1), want.shape[1:3]))
+    np.testing.assert_array_equal(y, want)
+
+
 def test_qmaxpool_resnet_stem_sized(cabi):
     """[32,112,112,64] -> 3x3 / 2, pad 1: the pooling after a ResNet stem."""
     say("qmaxpool stem")

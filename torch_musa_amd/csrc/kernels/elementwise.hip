@@ -241,6 +241,38 @@ __device__ __forceinline__ uint32_t max_codes4(uint32_t a, uint32_t b) {
   return (__builtin_bit_cast(uint32_t, me) | (__builtin_bit_cast(uint32_t, mo) << 8)) ^ bias;
 }
 
+// Running maximum of 16 codes (four words) over many taps at three vector
+// operations per word and tap.  The bytes of a word are compared as the two
+// 16-bit lanes of a packed maximum: the even bytes masked into the lanes' low
+// halves; the odd bytes as they are -- a lane whose high byte is larger wins
+// whatever its low byte holds, and only the high byte of that result is used.
+// Signed codes are compared as code ^ 0x80 (flipped when the result is read).
+template <bool SIGNED>
+struct CodeMax16 {
+  uint32_t even[4] = {0, 0, 0, 0}, odd[4] = {0, 0, 0, 0};
+  // `take` false: the tap is outside the image and does not take part
+  __device__ __forceinline__ void add(const v4i& v, bool take) {
+    const uint32_t w[4] = {static_cast<uint32_t>(v.x), static_cast<uint32_t>(v.y), static_cast<uint32_t>(v.z),
+                           static_cast<uint32_t>(v.w)};
+    const uint32_t lowest = SIGNED ? 0x80808080u : 0u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t u = take ? w[j] : lowest;
+      if (SIGNED) u ^= 0x80808080u;
+      even[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(us2, even[j]),
+                                                                       __builtin_bit_cast(us2, u & 0x00ff00ffu)));
+      odd[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(us2, odd[j]),
+                                                                      __builtin_bit_cast(us2, u)));
+    }
+  }
+  __device__ __forceinline__ v4i result() const {
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = ((odd[j] & 0xff00ff00u) | even[j]) ^ (SIGNED ? 0x80808080u : 0u);
+    return v4i{static_cast<int>(r[0]), static_cast<int>(r[1]), static_cast<int>(r[2]), static_cast<int>(r[3])};
+  }
+};
+
 template <bool SIGNED, int VEC>
 __global__ __launch_bounds__(kEwThreads) void qmaxpool_kernel(const uint8_t* __restrict__ x,
                                                               uint8_t* __restrict__ y, PoolShape s) {
@@ -289,7 +321,6 @@ __global__ __launch_bounds__(kEwThreads) void qmaxpool_k3_kernel(const uint8_t* 
   const int64_t cv = s.C / 16;
   const int64_t total = s.B * s.OH * s.OW * cv;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kEwThreads;
-  const int lowest = static_cast<int>(SIGNED ? 0x80808080u : 0u);
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kEwThreads + threadIdx.x; i < total; i += stride) {
     const int64_t c = (i % cv) * 16;
     int64_t t = i / cv;
@@ -307,14 +338,10 @@ __global__ __launch_bounds__(kEwThreads) void qmaxpool_k3_kernel(const uint8_t* 
       const int64_t ihc = ih < 0 ? 0 : (ih >= s.H ? s.H - 1 : ih), iwc = iw < 0 ? 0 : (iw >= s.W ? s.W - 1 : iw);
       v[k] = *reinterpret_cast<const v4i*>(img + (ihc * s.W + iwc) * s.C);
     }
-    v4i m = {lowest, lowest, lowest, lowest};
+    CodeMax16<SIGNED> m;
 #pragma unroll
-    for (int k = 0; k < 9; ++k) {
-      const v4i u = ok[k] ? v[k] : v4i{lowest, lowest, lowest, lowest};
-      m = v4i{static_cast<int>(max_codes4<SIGNED>(m.x, u.x)), static_cast<int>(max_codes4<SIGNED>(m.y, u.y)),
-              static_cast<int>(max_codes4<SIGNED>(m.z, u.z)), static_cast<int>(max_codes4<SIGNED>(m.w, u.w))};
-    }
-    *reinterpret_cast<v4i*>(y + ((b * s.OH + oh) * s.OW + ow) * s.C + c) = m;
+    for (int k = 0; k < 9; ++k) m.add(v[k], ok[k]);
+    *reinterpret_cast<v4i*>(y + ((b * s.OH + oh) * s.OW + ow) * s.C + c) = m.result();
   }
 }
 
@@ -335,7 +362,6 @@ __global__ __launch_bounds__(kEwThreads) void qmaxpool_k3_rows_kernel(const uint
   const int64_t b = blockIdx.z;
   const int ih0 = oh * sh - ph, iw0 = ow * sw - pw;
   const uint8_t* img = x + b * (static_cast<int64_t>(H) * W * C) + c;
-  const int lowest = static_cast<int>(SIGNED ? 0x80808080u : 0u);
   v4i v[9];
   bool ok[9];
 #pragma unroll
@@ -345,14 +371,10 @@ __global__ __launch_bounds__(kEwThreads) void qmaxpool_k3_rows_kernel(const uint
     const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih), iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);
     v[k] = *reinterpret_cast<const v4i*>(img + (ihc * W + iwc) * C);
   }
-  v4i m = {lowest, lowest, lowest, lowest};
+  CodeMax16<SIGNED> m;
 #pragma unroll
-  for (int k = 0; k < 9; ++k) {
-    const v4i u = ok[k] ? v[k] : v4i{lowest, lowest, lowest, lowest};
-    m = v4i{static_cast<int>(max_codes4<SIGNED>(m.x, u.x)), static_cast<int>(max_codes4<SIGNED>(m.y, u.y)),
-            static_cast<int>(max_codes4<SIGNED>(m.z, u.z)), static_cast<int>(max_codes4<SIGNED>(m.w, u.w))};
-  }
-  *reinterpret_cast<v4i*>(y + ((b * OH + oh) * OW + ow) * static_cast<int64_t>(C) + c) = m;
+  for (int k = 0; k < 9; ++k) m.add(v[k], ok[k]);
+  *reinterpret_cast<v4i*>(y + ((b * OH + oh) * OW + ow) * static_cast<int64_t>(C) + c) = m.result();
 }
 
 // Adaptive average pooling: output pixel (oh, ow) averages the input window

@@ -13,7 +13,8 @@
 // synchronisation; behind the barrier that ends phase p the buffer it used takes
 // phase p + 4.
 //
-// The automatic choice sends K <= 1024 here (grids of at most 256 tiles).  Longer
+// The automatic choice sends K <= 1024 here (grids of at most 256 tiles; up to 512
+// tiles of 32 x 32 go to gemm_i8_ksplit_kernel at the end of this file).  Longer
 // K runs (any K, for tests) but does not pay: with cold weights a phase then
 // waits for memory, 96 KB in flight per CU against about 2 us of latency, and
 // K = N = 4096 at M = 128 takes 15.0 us against 12.5 us for the 64 x 64 tiles
@@ -268,6 +269,173 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
         for (int b = 0; b < 16; ++b)
           if (n + b < a.N) dst[b] = static_cast<uint8_t>(w[b >> 2] >> (8 * (b & 3)));
       }
+    }
+  }
+}
+
+// 32 x 32 tiles for K <= 1024 on grids of at most 256 such tiles: the four waves
+// of a block split K between them.  A 64 x 64 tile of the kernel above pulls
+// 128 KB into one CU's LDS, at 16 - 45 bytes per clock: 1.5 us of M = 128,
+// K = N = 1024 on 32 of the chip's 256 CUs.  Here 128 blocks pull 64 KB each, and
+// every wave copies only the quarter of K it multiplies itself (its own 16 KB of
+// LDS), so it waits for nobody before its MFMAs; the four partial tiles meet in
+// LDS behind the block's one barrier, where 256 threads add them, requantise
+// four channels of one row each and store.
+//
+// LDS of wave w:  weights [k-step][k-chunk of the step][32 rows][16 B] (a copy
+// instruction moves one k-step: two 16-row blocks of two k-chunks of the packed
+// layout), activations [32 rows][256 B] with the slot swizzle of the kernel above.
+template <int MODE>
+__global__ __launch_bounds__(256) void gemm_i8_ksplit_kernel(GemmArgs a, XLinear xs) {
+  constexpr int BM = 32, BN = 32;
+  constexpr int kWaveSteps = 8;                    // 32-byte k-steps a wave can hold: 256 bytes of K
+  constexpr int kRedPitch = BN * 4 + 16;           // a row of a wave's partial tile
+  __shared__ __attribute__((aligned(16))) uint8_t sW[4][kWaveSteps * 1024];
+  __shared__ __attribute__((aligned(16))) uint8_t sX[4][BM * 256];
+  __shared__ __attribute__((aligned(16))) int s_raw[3][kWave];  // colsum, weight scale, bias as fetched
+  static_assert(BM * kRedPitch <= kWaveSteps * 1024, "a wave's partial tile fits over its weights");
+
+  const int t = threadIdx.x, lane = t % kWave;
+  const int wave_u = __builtin_amdgcn_readfirstlane(t / kWave);
+  const int li = lane & 31, half = lane >> 5;
+  const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * BN;
+  const int KC = static_cast<int>(a.K >> 4);       // k-chunks (K is a multiple of 16, at most 1024)
+  const int S = (KC + 1) >> 1;                     // 32-byte k-steps, at most 32
+  const int sp = (S + 3) >> 2;                     // k-steps per wave
+  const int s0 = wave_u * sp;                      // this wave's first k-step
+  const int mine = S - s0 < sp ? (S - s0 < 0 ? 0 : S - s0) : sp;
+
+  // ---- requests: the tile's per-channel constants (wave 0), then this wave's operands
+  if (wave_u == 0) {
+    const int64_t n = n0 + lane < a.N ? n0 + lane : a.N - 1;
+    const uint32_t np = static_cast<uint32_t>(n + a.n_off);
+    lds_dma4(a.colsum, np * 4u, lds_address(&s_raw[0][0]));
+    if constexpr (MODE != kOutAcc32) {  // (raw accumulators: the caller passes no scales)
+      lds_dma4(a.w_scales, np * static_cast<uint32_t>(a.w_scale_stride) * 4u, lds_address(&s_raw[1][0]));
+      lds_dma4(a.bias != nullptr ? a.bias : a.w_scales, a.bias != nullptr ? np * 4u : 0u,
+               lds_address(&s_raw[2][0]));
+    }
+  }
+  {
+    const int64_t NB = ceil_div(a.N, 16);
+    const int64_t nb_last = NB - 1 - n0 / 16;      // a 16-row block past N: clamped, never stored
+    const uint8_t* const wtile = a.w_packed + (n0 / 16) * a.w_kchunks * 256;
+    const int64_t rb = ((lane >> 4) & 1) < nb_last ? ((lane >> 4) & 1) : nb_last;
+    const int kc_last = static_cast<int>(a.w_kchunks) - 1;
+    const uint32_t ldsW = lds_address(&sW[wave_u][0]);
+#pragma unroll
+    for (int j = 0; j < kWaveSteps; ++j) {
+      if (j < sp) {
+        // (k-steps past the end of K fetch the last chunk again and are not multiplied;
+        // an odd last chunk is followed by the zero padding of the packed layout)
+        const int kc = 2 * (s0 + j) + half;
+        const int kcc = kc < kc_last ? kc : kc_last;
+        const uint32_t off = static_cast<uint32_t>((rb * a.w_kchunks + kcc) * 256 + (lane & 15) * 16);
+        lds_dma16(wtile, off, ldsW + static_cast<uint32_t>(j) * 1024u);
+      }
+    }
+    const uint8_t* const xtile = xs.x + m0 * xs.ldx;
+    const int64_t m_last = a.M - 1 - m0;           // rows past M: clamped, never stored
+    const uint32_t ldsX = lds_address(&sX[wave_u][0]);
+#pragma unroll
+    for (int i = 0; i < BM / 4; ++i) {
+      const int r = 4 * i + (lane >> 4);
+      const int64_t rc = r < m_last ? r : m_last;
+      const int slot = (lane & 15) ^ (r & 15);
+      // this wave's 256 bytes of the row; chunks past K: any bytes of the row will do
+      const int cc = 2 * s0 + slot;
+      const int ccc = cc < KC ? cc : KC - 1;
+      if (slot < 2 * sp)
+        lds_dma16(xtile, static_cast<uint32_t>(rc * xs.ldx) + static_cast<uint32_t>(ccc) * 16u,
+                  ldsX + static_cast<uint32_t>(4 * i) * 256u);
+    }
+  }
+
+  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
+                     static_cast<int>(a.x_xor)};
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  // this wave's own copies have landed: nobody else's are needed before the MFMAs
+  __builtin_amdgcn_s_waitcnt((0 & 15) | ((0 >> 4) << 14) | (7 << 4) | (15 << 8));
+  {
+    const uint8_t* const wrd = &sW[wave_u][0] + half * 512 + (li >> 4) * 256 + (li & 15) * 16;
+    const uint8_t* const xrd = &sX[wave_u][0] + li * 256;
+    v4i wf[kWaveSteps], xf[kWaveSteps];
+#pragma unroll
+    for (int j = 0; j < kWaveSteps; ++j) {
+      wf[j] = ld16(wrd + j * 1024);
+      xf[j] = ld16(xrd + (((2 * j + half) ^ (li & 15)) << 4));
+    }
+#pragma unroll
+    for (int j = 0; j < kWaveSteps; ++j) {
+      const int keep = j < mine ? -1 : 0;
+      const v4i xv = (xf[j] ^ xmask) & v4i{keep, keep, keep, keep};
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xv, acc, 0, 0, 0);
+    }
+  }
+  // ---- the partial tile of this wave, over its own weights: a lane holds channels
+  // 8g + 4 half + j (g, j < 4) of activation row li
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const v4i part = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+    *reinterpret_cast<v4i*>(&sW[wave_u][li * kRedPitch + (8 * g + 4 * half) * 4]) = part;
+  }
+  __syncthreads();
+
+  // ---- thread t: row t / 8, channels 4 (t % 8) ... + 3
+  const int row = t >> 3, cl = (t & 7) * 4;
+  const int64_t m = m0 + row, n = n0 + cl;
+  if (m >= a.M || n >= a.N) return;
+  v4i sum = *reinterpret_cast<const v4i*>(&sW[0][row * kRedPitch + cl * 4]);
+#pragma unroll
+  for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const v4i*>(&sW[w][row * kRedPitch + cl * 4]);
+  const XQuant xq = x_quant(a);
+  int raw[4];
+  v4f mult = {0.f, 0.f, 0.f, 0.f}, bdiv = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    raw[j] = sum[j] + xq.coef * s_raw[0][cl + j];
+    if constexpr (MODE != kOutAcc32) {
+      const float ws = __int_as_float(s_raw[1][cl + j]), bs = __int_as_float(s_raw[2][cl + j]);
+      const float atw = xq.scale * ws;
+      if (MODE == kOutF32) {
+        mult[j] = atw;
+        bdiv[j] = a.bias != nullptr ? bs : 0.f;
+      } else {
+        mult[j] = atw / a.out_scale;
+        bdiv[j] = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, bs, atw) : 0.f;
+      }
+    }
+  }
+  if constexpr (MODE == kOutF32 || MODE == kOutAcc32) {
+    float* const dst = static_cast<float*>(a.y) + a.n_off + m * a.ldy + n;
+    v4f v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      v[j] = MODE == kOutAcc32 ? __int_as_float(raw[j])
+                               : __builtin_fmaxf(__builtin_fmaf(static_cast<float>(raw[j]), mult[j], bdiv[j]), a.lo_f);
+    if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0 && n + 4 <= a.N) {
+      *reinterpret_cast<v4f*>(dst) = v;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < a.N) dst[j] = v[j];
+    }
+  } else {
+    const float bmul = bias_mul(a.w_scale_stride == 0, xq.scale * __int_as_float(s_raw[1][0]));
+    const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
+    // unsigned output without ReLU: the saturating conversion is the clamp
+    const uint32_t q4 = plain_u8 ? requant4<MODE, false>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f)
+                                 : requant4<MODE, true>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+    uint8_t* const dst = static_cast<uint8_t*>(a.y) + a.n_off + m * a.ldy + n;
+    if ((reinterpret_cast<uintptr_t>(dst) & 3) == 0 && n + 4 <= a.N) {
+      *reinterpret_cast<uint32_t*>(dst) = q4;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < a.N) dst[j] = static_cast<uint8_t>(q4 >> (8 * j));
     }
   }
 }

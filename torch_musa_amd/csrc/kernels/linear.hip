@@ -509,6 +509,16 @@ int launch_gemm_onepass(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   return launch_status();
 }
 
+// 32 x 32 tiles whose four waves split K (K <= 1024; the caller checked the address ranges).
+template <int MODE>
+int launch_gemm_ksplit(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  const int64_t tiles_m = ceil_div(a.M, 32), tiles_n = ceil_div(a.N, 32);
+  if (tiles_n > 0x7fffffff || tiles_m > 65535 || a.K > kOnePassMaxK) return TMQ_ERR_UNSUPPORTED;
+  gemm_i8_ksplit_kernel<MODE>
+      <<<dim3(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m)), dim3(256), 0, s>>>(a, xs);
+  return launch_status();
+}
+
 constexpr int kMaxDevices = 64;
 
 // Compute units of the current device (cached per device; two threads that race
@@ -572,7 +582,7 @@ constexpr int64_t kSplitMinStages = 16;  // shortest run of stages per split
 //  * 64 x 64 tiles walk K at the latency of one stage after the other, almost
 //    whatever M is (K = N = 4096 with two wave groups: 12.8 / 14.8 us at
 //    M = 32 / 64; N = 11008: 14.9 / 16.8 us), and K <= 1024 fits LDS whole
-//    (gemm_i8_onepass.h: K = N = 1024: 5.8 us);
+//    (gemm_i8_onepass.h: K = N = 1024: 3.8 us on 32 x 32 tiles);
 //  * split K moves the weights at about 3.4 TB/s plus 8 us for the partial sums
 //    (N = 4096, K = 11008: 21.7 us at M = 65 against 30.6 us streaming at M = 64).
 enum class SmallRows { kStream, kTiles, kSplit };
@@ -594,7 +604,10 @@ SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
                         rows * std::max(0.10 * std::max(1.0, stream_blocks / 256.0), 0.135 * l2_mib_per_row);
   const double nblk = static_cast<double>(ceil_div(M, 64) * ceil_div(N, 64));
   double tiles;
-  if (K <= kOnePassMaxK && nblk <= 256.0)  // all of K in LDS (K = N = 1024: 5.8 us, K = N = 512: 3.9 us)
+  if (K <= kOnePassMaxK && K > 256 && ceil_div(M, 32) * ceil_div(N, 32) <= 512)
+    // all of K in LDS, 32 x 32 tiles (K = N = 1024: 3.8 us, K = N = 512: 3.2 us, N = 4096, K = 512: 3.9 us)
+    tiles = 3.0 + 0.6 * mib + (ceil_div(M, 32) * ceil_div(N, 32) > 256 ? 0.5 : 0.0);
+  else if (K <= kOnePassMaxK && nblk <= 256.0)  // 64 x 64 tiles (K = N = 1024: 5.6 us, N = 1024, K = 256: 3.1 us)
     tiles = 2.0 + 3.8 * static_cast<double>(K) / 1024.0 + 0.012 * std::max(0.0, nblk - 64.0);
   else if (two_wave_groups_fit(M, N, K))
     tiles = (4.4 + 0.123 * stages + 0.013 * std::max(0.0, nblk - 64.0)) *
@@ -805,8 +818,10 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
   int cfg = forced;
   if (cfg < 0 && onepass_ok && a.K <= kOnePassMaxK && ceil_div(a.M, 64) * ceil_div(a.N, 64) <= 256) {
     // short K on a grid no larger than the chip: one latency instead of one per stage
-    // (M = 128, K = N = 1024: 6.0 -> 4.x us)
-    cfg = 21;
+    // (M = 128, K = N = 1024: 6.0 -> 5.6 us with cold weights); up to 512 tiles of 32 x 32
+    // whose waves split K spread the copies over more CUs (3.8 us; M = 512: 5.7 -> 4.4 us;
+    // N = 4096, K = 512, M = 128: 4.4 -> 4.3 us; 640 tiles and more, or K <= 256: slower)
+    cfg = a.K > 256 && ceil_div(a.M, 32) * ceil_div(a.N, 32) <= 512 ? 24 : 21;
   } else if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
@@ -878,6 +893,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 22: return launch_gemm<128, 64, 2, 2, MODE>(a, xs, s);
     case 23: return launch_gemm<64, 128, 2, 2, MODE>(a, xs, s);
     case 21: return onepass_ok ? launch_gemm_onepass<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
+    case 24: return onepass_ok ? launch_gemm_ksplit<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
