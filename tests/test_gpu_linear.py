@@ -89,7 +89,7 @@ def test_per_tensor_weight_bias_form(cabi, golden, cfg):
 
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23, 24])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23, 24, 25])
 @pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),
                                    (270, 300, 400), (40, 70, 784)])
 def test_tile_configs(cabi, cfg, shape):
@@ -155,7 +155,8 @@ def test_instrumented_persistent_kernel_gives_the_same_bytes(cabi):
 @pytest.mark.parametrize("shape", [(128, 1024, 1024), (1, 16, 16), (64, 64, 32), (65, 70, 48), (100, 130, 1008),
                                    (33, 200, 272), (257, 129, 528), (1000, 1000, 1024), (90, 33, 784)])
 @pytest.mark.parametrize("x_signed", [False, True])
-@pytest.mark.parametrize("cfg", [21, 24])    # 64 x 64 tiles; 32 x 32 tiles whose waves split K
+# 64 x 64 tiles; 32 x 32 tiles whose waves split K, weights through LDS / through registers
+@pytest.mark.parametrize("cfg", [21, 24, 25])
 def test_whole_k_in_lds_kernel(cabi, shape, x_signed, cfg):
     say("K in LDS", shape, x_signed, cfg)
     M, N, K = shape
@@ -180,6 +181,26 @@ def test_whole_k_in_lds_kernel(cabi, shape, x_signed, cfg):
         y1, acc1, _ = _run(cabi, c)
         np.testing.assert_array_equal(y1, y)
         np.testing.assert_array_equal(acc1, acc)
+
+
+# 32 x 32 tiles whose waves split K with the weights through registers: K up to 4096 (both
+# instantiations: 16 and 32 k-steps per wave), K that leaves waves without work, odd chunks
+@pytest.mark.parametrize("shape", [(64, 160, 4096), (33, 200, 2064), (100, 130, 4080), (17, 70, 3088),
+                                   (128, 64, 2048), (40, 33, 1040), (5, 32, 2304)])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_weights_through_registers_kernel(cabi, shape, x_signed):
+    say("weights through registers", shape, x_signed)
+    M, N, K = shape
+    c = _tile_case(M, N, K, seed=2500 + K, x_signed=x_signed, relu=N % 2 == 1, bias=M % 3 != 0,
+                   per_channel=(M + N) % 2 == 0)
+    y, acc, pw = _run(cabi, c, 25)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "weights through registers")
+    y1, acc1, _ = _run(cabi, c)          # the automatic choice, whichever kernel it is
+    np.testing.assert_array_equal(y1, y)
+    np.testing.assert_array_equal(acc1, acc)
 
 
 # the persistent kernel over more tiles than the chip has CUs: every block walks two tiles
@@ -474,7 +495,7 @@ def test_split_k_workspace_rules(cabi):
 # Float results are compared bit for bit: the kernel's epilogue is the oracle's
 # single fused multiply-add, and the dynamic quantization in front of it is
 # bit-exact by the quantizer tests.
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20, 21, 22, 23, 24])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20, 21, 22, 23, 24, 25])
 @pytest.mark.parametrize("shape,relu,bias,pc,x_signed", [((60, 264, 448), False, True, True, False),
                                                          ((257, 33, 144), True, True, False, False),
                                                          ((16, 1040, 1168), False, False, True, True)])

@@ -273,6 +273,73 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
   }
 }
 
+// The end of a 32 x 32 tile whose four waves each hold a partial sum over their
+// share of K: the partial tiles lie in LDS (wave w's at red + w * red_stride,
+// rows of kSplitRedPitch bytes, written before the barrier the caller has just
+// passed); thread t adds the four for row t / 8, channels 4 (t % 8) ... + 3,
+// requantises and stores.  s_raw: colsum, weight scale and bias of the tile's
+// channels as fetched.
+constexpr int kSplitRedPitch = 32 * 4 + 16;
+template <int MODE>
+__device__ __forceinline__ void ksplit_finish(const GemmArgs& a, const uint8_t* red, int red_stride,
+                                              const int (*s_raw)[kWave], int64_t m0, int64_t n0, int t) {
+  constexpr int kRedPitch = kSplitRedPitch;
+  // ---- thread t: row t / 8, channels 4 (t % 8) ... + 3
+  const int row = t >> 3, cl = (t & 7) * 4;
+  const int64_t m = m0 + row, n = n0 + cl;
+  if (m >= a.M || n >= a.N) return;
+  v4i sum = *reinterpret_cast<const v4i*>(&red[row * kRedPitch + cl * 4]);
+#pragma unroll
+  for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const v4i*>(&red[w * red_stride + row * kRedPitch + cl * 4]);
+  const XQuant xq = x_quant(a);
+  int raw[4];
+  v4f mult = {0.f, 0.f, 0.f, 0.f}, bdiv = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    raw[j] = sum[j] + xq.coef * s_raw[0][cl + j];
+    if constexpr (MODE != kOutAcc32) {
+      const float ws = __int_as_float(s_raw[1][cl + j]), bs = __int_as_float(s_raw[2][cl + j]);
+      const float atw = xq.scale * ws;
+      if (MODE == kOutF32) {
+        mult[j] = atw;
+        bdiv[j] = a.bias != nullptr ? bs : 0.f;
+      } else {
+        mult[j] = atw / a.out_scale;
+        bdiv[j] = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, bs, atw) : 0.f;
+      }
+    }
+  }
+  if constexpr (MODE == kOutF32 || MODE == kOutAcc32) {
+    float* const dst = static_cast<float*>(a.y) + a.n_off + m * a.ldy + n;
+    v4f v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      v[j] = MODE == kOutAcc32 ? __int_as_float(raw[j])
+                               : __builtin_fmaxf(__builtin_fmaf(static_cast<float>(raw[j]), mult[j], bdiv[j]), a.lo_f);
+    if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0 && n + 4 <= a.N) {
+      *reinterpret_cast<v4f*>(dst) = v;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < a.N) dst[j] = v[j];
+    }
+  } else {
+    const float bmul = bias_mul(a.w_scale_stride == 0, xq.scale * __int_as_float(s_raw[1][0]));
+    const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
+    // unsigned output without ReLU: the saturating conversion is the clamp
+    const uint32_t q4 = plain_u8 ? requant4<MODE, false>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f)
+                                 : requant4<MODE, true>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+    uint8_t* const dst = static_cast<uint8_t*>(a.y) + a.n_off + m * a.ldy + n;
+    if ((reinterpret_cast<uintptr_t>(dst) & 3) == 0 && n + 4 <= a.N) {
+      *reinterpret_cast<uint32_t*>(dst) = q4;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < a.N) dst[j] = static_cast<uint8_t>(q4 >> (8 * j));
+    }
+  }
+}
+
 // 32 x 32 tiles for K <= 1024 on grids of at most 256 such tiles: the four waves
 // of a block split K between them.  A 64 x 64 tile of the kernel above pulls
 // 128 KB into one CU's LDS, at 16 - 45 bytes per clock: 1.5 us of M = 128,
@@ -289,7 +356,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void gemm_i8_ksplit_kernel(GemmArgs a, XLinear xs) {
   constexpr int BM = 32, BN = 32;
   constexpr int kWaveSteps = 8;                    // 32-byte k-steps a wave can hold: 256 bytes of K
-  constexpr int kRedPitch = BN * 4 + 16;           // a row of a wave's partial tile
+  constexpr int kRedPitch = kSplitRedPitch;        // a row of a wave's partial tile
   __shared__ __attribute__((aligned(16))) uint8_t sW[4][kWaveSteps * 1024];
   __shared__ __attribute__((aligned(16))) uint8_t sX[4][BM * 256];
   __shared__ __attribute__((aligned(16))) int s_raw[3][kWave];  // colsum, weight scale, bias as fetched
@@ -384,60 +451,127 @@ __global__ __launch_bounds__(256) void gemm_i8_ksplit_kernel(GemmArgs a, XLinear
   }
   __syncthreads();
 
-  // ---- thread t: row t / 8, channels 4 (t % 8) ... + 3
-  const int row = t >> 3, cl = (t & 7) * 4;
-  const int64_t m = m0 + row, n = n0 + cl;
-  if (m >= a.M || n >= a.N) return;
-  v4i sum = *reinterpret_cast<const v4i*>(&sW[0][row * kRedPitch + cl * 4]);
+  ksplit_finish<MODE>(a, &sW[0][0], kWaveSteps * 1024, s_raw, m0, n0, t);
+}
+
+// 32 x 32 tiles for K up to 32 * 4 * STEPS bytes (STEPS = 16: 2048, STEPS = 32: 4096)
+// whose four waves split K, the weights going through registers instead of LDS.
+//
+// What a CU can have on its way bounds what it pulls per microsecond: LDS holds
+// at most 160 KB of copies in flight, which at the latency of cold memory is
+// 16 - 45 bytes per clock, and that is what 64 x 64 tiles of a few dozen rows
+// x several thousand channels run at (K = N = 4096, M = 64: 14.8 us for 17 MB of
+// weights).  Here a wave copies its quarter of the activation rows' K into its own
+// LDS (at K = 4096: 32 rows x 1024 bytes, 128 KB per block, L2 hits) and requests
+// ALL of its weight fragments at once into registers (STEPS loads of 16 bytes per
+// lane, one per MFMA: in the packed layout a fragment is four contiguous 256-byte
+// runs), another 128 KB per block in flight, waits for nobody but its own
+// requests and multiplies as they arrive.  Partial tiles and epilogue as in the
+// kernel above.
+template <int MODE, int STEPS>
+__global__ __launch_bounds__(256) void gemm_i8_wstream_kernel(GemmArgs a, XLinear xs) {
+  constexpr int BM = 32, BN = 32;
+  constexpr int SEGS = STEPS / 8;                  // 256-byte segments of K per wave
+  constexpr int kRedPitch = kSplitRedPitch;
+  static_assert(STEPS == 16 || STEPS == 32, "the wait below encodes STEPS outstanding loads in six bits");
+  __shared__ __attribute__((aligned(16))) uint8_t sX[4][SEGS * BM * 256];
+  __shared__ __attribute__((aligned(16))) int s_raw[3][kWave];  // colsum, weight scale, bias as fetched
+  static_assert(BM * kRedPitch <= SEGS * BM * 256, "a wave's partial tile fits over its activations");
+
+  const int t = threadIdx.x, lane = t % kWave;
+  const int wave_u = __builtin_amdgcn_readfirstlane(t / kWave);
+  const int li = lane & 31, half = lane >> 5;
+  const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * BN;
+  const int KC = static_cast<int>(a.K >> 4);       // k-chunks (K is a multiple of 16)
+  const int S = (KC + 1) >> 1;                     // 32-byte k-steps, at most 4 * STEPS
+  const int sp = (S + 3) >> 2;                     // k-steps per wave, at most STEPS
+  const int s0 = wave_u * sp;                      // this wave's first k-step
+  const int mine = S - s0 < sp ? (S - s0 < 0 ? 0 : S - s0) : sp;
+
+  // ---- requests, oldest first: the tile's per-channel constants (wave 0), this
+  // wave's activations (into LDS), this wave's weights (into registers)
+  if (wave_u == 0) {
+    const int64_t n = n0 + lane < a.N ? n0 + lane : a.N - 1;
+    const uint32_t np = static_cast<uint32_t>(n + a.n_off);
+    lds_dma4(a.colsum, np * 4u, lds_address(&s_raw[0][0]));
+    if constexpr (MODE != kOutAcc32) {  // (raw accumulators: the caller passes no scales)
+      lds_dma4(a.w_scales, np * static_cast<uint32_t>(a.w_scale_stride) * 4u, lds_address(&s_raw[1][0]));
+      lds_dma4(a.bias != nullptr ? a.bias : a.w_scales, a.bias != nullptr ? np * 4u : 0u,
+               lds_address(&s_raw[2][0]));
+    }
+  }
+  {
+    const uint8_t* const xtile = xs.x + m0 * xs.ldx;
+    const int64_t m_last = a.M - 1 - m0;           // rows past M: clamped, never stored
+    const uint32_t ldsX = lds_address(&sX[wave_u][0]);
 #pragma unroll
-  for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const v4i*>(&sW[w][row * kRedPitch + cl * 4]);
-  const XQuant xq = x_quant(a);
-  int raw[4];
-  v4f mult = {0.f, 0.f, 0.f, 0.f}, bdiv = {0.f, 0.f, 0.f, 0.f};
+    for (int seg = 0; seg < SEGS; ++seg) {
+      if (seg * 8 < sp) {                          // (uniform: segments past this wave's share stay unwritten)
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    raw[j] = sum[j] + xq.coef * s_raw[0][cl + j];
-    if constexpr (MODE != kOutAcc32) {
-      const float ws = __int_as_float(s_raw[1][cl + j]), bs = __int_as_float(s_raw[2][cl + j]);
-      const float atw = xq.scale * ws;
-      if (MODE == kOutF32) {
-        mult[j] = atw;
-        bdiv[j] = a.bias != nullptr ? bs : 0.f;
-      } else {
-        mult[j] = atw / a.out_scale;
-        bdiv[j] = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, bs, atw) : 0.f;
+        for (int i = 0; i < BM / 4; ++i) {
+          const int r = 4 * i + (lane >> 4);
+          const int64_t rc = r < m_last ? r : m_last;
+          const int slot = (lane & 15) ^ (r & 15);
+          // chunks past K: any bytes of the row will do, they meet a zeroed operand or zero weights
+          const int cc = 2 * s0 + 16 * seg + slot;
+          const int ccc = cc < KC ? cc : KC - 1;
+          lds_dma16(xtile, static_cast<uint32_t>(rc * xs.ldx) + static_cast<uint32_t>(ccc) * 16u,
+                    ldsX + static_cast<uint32_t>(seg * BM + 4 * i) * 256u);
+        }
       }
     }
   }
-  if constexpr (MODE == kOutF32 || MODE == kOutAcc32) {
-    float* const dst = static_cast<float*>(a.y) + a.n_off + m * a.ldy + n;
-    v4f v;
+  v4i wf[STEPS];
+  {
+    const int64_t NB = ceil_div(a.N, 16);
+    const int64_t nb_last = NB - 1 - n0 / 16;      // a 16-row block past N: clamped, never stored
+    const int64_t rb = ((lane >> 4) & 1) < nb_last ? ((lane >> 4) & 1) : nb_last;
+    const uint8_t* const wlane = a.w_packed + ((n0 / 16 + rb) * a.w_kchunks) * 256 + (lane & 15) * 16;
+    const int kc_last = static_cast<int>(a.w_kchunks) - 1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      v[j] = MODE == kOutAcc32 ? __int_as_float(raw[j])
-                               : __builtin_fmaxf(__builtin_fmaf(static_cast<float>(raw[j]), mult[j], bdiv[j]), a.lo_f);
-    if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0 && n + 4 <= a.N) {
-      *reinterpret_cast<v4f*>(dst) = v;
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n + j < a.N) dst[j] = v[j];
-    }
-  } else {
-    const float bmul = bias_mul(a.w_scale_stride == 0, xq.scale * __int_as_float(s_raw[1][0]));
-    const bool plain_u8 = MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f;
-    // unsigned output without ReLU: the saturating conversion is the clamp
-    const uint32_t q4 = plain_u8 ? requant4<MODE, false>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f)
-                                 : requant4<MODE, true>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
-    uint8_t* const dst = static_cast<uint8_t*>(a.y) + a.n_off + m * a.ldy + n;
-    if ((reinterpret_cast<uintptr_t>(dst) & 3) == 0 && n + 4 <= a.N) {
-      *reinterpret_cast<uint32_t*>(dst) = q4;
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n + j < a.N) dst[j] = static_cast<uint8_t>(q4 >> (8 * j));
+    for (int j = 0; j < STEPS; ++j) {
+      // (k-steps past this wave's share fetch its last one again and are not multiplied;
+      // an odd last chunk is followed by the zero padding of the packed layout)
+      const int step = s0 + (j < sp ? j : sp - 1);
+      const int kc = 2 * step + half;
+      const int kcc = kc < kc_last ? kc : kc_last;
+      wf[j] = *reinterpret_cast<const v4i*>(wlane + static_cast<int64_t>(kcc) * 256);
     }
   }
+
+  const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
+                     static_cast<int>(a.x_xor)};
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  // The copies into LDS are older than the weight loads and requests return in
+  // order: at most STEPS requests outstanding means the activations have landed.
+  // (as an asm statement that clobbers memory: the compiler may neither sink a
+  // weight load below it nor hoist an LDS read above it)
+  if constexpr (STEPS == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+  {
+    const uint8_t* const xrd = &sX[wave_u][0] + li * 256;
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+      if (j / 8 * 8 < sp) {                        // (uniform, per segment)
+        const v4i xf = ld16(xrd + (j / 8) * (BM * 256) + (((2 * (j % 8) + half) ^ (li & 15)) << 4));
+        const int keep = j < mine ? -1 : 0;
+        const v4i xv = (xf ^ xmask) & v4i{keep, keep, keep, keep};
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xv, acc, 0, 0, 0);
+      }
+    }
+  }
+  // ---- the partial tile of this wave, over its own activations: a lane holds
+  // channels 8g + 4 half + j (g, j < 4) of activation row li
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const v4i part = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+    *reinterpret_cast<v4i*>(&sX[wave_u][li * kRedPitch + (8 * g + 4 * half) * 4]) = part;
+  }
+  __syncthreads();
+  ksplit_finish<MODE>(a, &sX[0][0], SEGS * BM * 256, s_raw, m0, n0, t);
 }
 
 }  // namespace tmq

@@ -519,6 +519,20 @@ int launch_gemm_ksplit(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   return launch_status();
 }
 
+// 32 x 32 tiles whose four waves split K, weights through registers (K <= 4096; the caller
+// checked the address ranges).
+template <int MODE>
+int launch_gemm_wstream(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  const int64_t tiles_m = ceil_div(a.M, 32), tiles_n = ceil_div(a.N, 32);
+  if (tiles_n > 0x7fffffff || tiles_m > 65535 || a.K > 4096) return TMQ_ERR_UNSUPPORTED;
+  const dim3 grid(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m));
+  if (a.K <= 2048)
+    gemm_i8_wstream_kernel<MODE, 16><<<grid, dim3(256), 0, s>>>(a, xs);
+  else
+    gemm_i8_wstream_kernel<MODE, 32><<<grid, dim3(256), 0, s>>>(a, xs);
+  return launch_status();
+}
+
 constexpr int kMaxDevices = 64;
 
 // Compute units of the current device (cached per device; two threads that race
@@ -594,7 +608,24 @@ bool two_wave_groups_fit(int64_t M, int64_t N, int64_t K) {
 
 SplitPlan plan_split_tiles(int64_t M, int64_t N, int64_t K);
 
+// Shapes for the 32 x 32 tiles whose waves split K and stream their weights through
+// registers: K beyond what the kernels with all operands in LDS take, one round of
+// blocks (two blocks share a CU while a block's activations, 32 rows x K, are at
+// most 64 KB).  With more blocks than that it loses to the larger tiles (K = 4096:
+// N = 4096, M = 96: 13.7 against 12.8 us; K = 2048, N = 4096, M = 256: 10.7 against 9.7 us).
+bool wstream_fits(int64_t M, int64_t N, int64_t K) {
+  if (K <= kOnePassMaxK || K > 4096) return false;
+  return ceil_div(M, 32) * ceil_div(N, 32) <= (K <= 2048 ? 512 : 256);
+}
+
 SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
+  // Where the 32 x 32 tiles with the weights through registers fit, they are measured
+  // directly against the weight-streaming kernel (us at M = 17 / 32 / 64, tiles | streaming):
+  //   K = 2048, N = 4096:  5.4 / 5.4 / 5.5 | 6.2 / 6.9 / 9.4     K = 1280, N = 2048:  4.6 / 4.6 / 4.7 | 5.6 / 6.1 / 9.7
+  //   K = 4096, N = 4096:  8.2 / 8.3 / 8.6 | 6.8 / 7.8 / 12.2    K = 4096, N = 1024:  6.5 / 6.5 / 6.6 | 6.0 / 7.0 / 11.3
+  //   K = 3072, N = 4096:  7.2 / 7.3 / 7.6 | 6.4 / 7.5 / 11.7    K = 4096, N = 8192: 10.6 / 10.7 / -  | 11.7 / 13.6 / 22.6
+  // streaming keeps the longer K up to about two dozen rows while its blocks fit one round.
+  if (wstream_fits(M, N, K)) return K > 2048 && M <= 24 && N <= 4096 ? SmallRows::kStream : SmallRows::kTiles;
   const double mib = static_cast<double>(N) * static_cast<double>(K) / 1048576.0;
   const double stages = static_cast<double>(ceil_div(K, kBK));
   const double rows = static_cast<double>(M);
@@ -609,6 +640,7 @@ SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
     tiles = 3.0 + 0.6 * mib + (ceil_div(M, 32) * ceil_div(N, 32) > 256 ? 0.5 : 0.0);
   else if (K <= kOnePassMaxK && nblk <= 256.0)  // 64 x 64 tiles (K = N = 1024: 5.6 us, N = 1024, K = 256: 3.1 us)
     tiles = 2.0 + 3.8 * static_cast<double>(K) / 1024.0 + 0.012 * std::max(0.0, nblk - 64.0);
+
   else if (two_wave_groups_fit(M, N, K))
     tiles = (4.4 + 0.123 * stages + 0.013 * std::max(0.0, nblk - 64.0)) *
             (1.0 + 0.35 * (rows / 64.0) * (rows / 64.0) * std::min(1.0, stages / 172.0));
@@ -822,6 +854,12 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     // whose waves split K spread the copies over more CUs (3.8 us; M = 512: 5.7 -> 4.4 us;
     // N = 4096, K = 512, M = 128: 4.4 -> 4.3 us; 640 tiles and more, or K <= 256: slower)
     cfg = a.K > 256 && ceil_div(a.M, 32) * ceil_div(a.N, 32) <= 512 ? 24 : 21;
+  } else if (cfg < 0 && onepass_ok && wstream_fits(a.M, a.N, a.K)) {
+    // K up to 4096 on a grid of 32 x 32 tiles that the chip holds at once: the waves split
+    // K and take their weights through registers (cold weights, K = N = 4096, M = 64:
+    // 12.2 -> 8.6 us; K = 2048, N = 4096: M = 64 9.4 -> 5.5 us, M = 128 9.4 -> 7.0 us;
+    // K = N = 2048: M = 128 7.8 -> 5.0 us, M = 256 8.0 -> 6.3 us)
+    cfg = 25;
   } else if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
@@ -894,6 +932,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 23: return launch_gemm<64, 128, 2, 2, MODE>(a, xs, s);
     case 21: return onepass_ok ? launch_gemm_onepass<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
     case 24: return onepass_ok ? launch_gemm_ksplit<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
+    case 25: return onepass_ok ? launch_gemm_wstream<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
