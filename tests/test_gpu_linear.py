@@ -89,7 +89,7 @@ def test_per_tensor_weight_bias_form(cabi, golden, cfg):
 
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23, 24, 25])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23, 24, 25, 26])
 @pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),
                                    (270, 300, 400), (40, 70, 784)])
 def test_tile_configs(cabi, cfg, shape):
@@ -188,12 +188,13 @@ def test_whole_k_in_lds_kernel(cabi, shape, x_signed, cfg):
 @pytest.mark.parametrize("shape", [(64, 160, 4096), (33, 200, 2064), (100, 130, 4080), (17, 70, 3088),
                                    (128, 64, 2048), (40, 33, 1040), (5, 32, 2304)])
 @pytest.mark.parametrize("x_signed", [False, True])
-def test_weights_through_registers_kernel(cabi, shape, x_signed):
-    say("weights through registers", shape, x_signed)
+@pytest.mark.parametrize("cfg", [25, 26])       # 32 and 64 channels per tile
+def test_weights_through_registers_kernel(cabi, shape, x_signed, cfg):
+    say("weights through registers", shape, x_signed, cfg)
     M, N, K = shape
     c = _tile_case(M, N, K, seed=2500 + K, x_signed=x_signed, relu=N % 2 == 1, bias=M % 3 != 0,
                    per_channel=(M + N) % 2 == 0)
-    y, acc, pw = _run(cabi, c, 25)
+    y, acc, pw = _run(cabi, c, cfg)
     np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
     want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
                          c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
@@ -495,7 +496,7 @@ def test_split_k_workspace_rules(cabi):
 # Float results are compared bit for bit: the kernel's epilogue is the oracle's
 # single fused multiply-add, and the dynamic quantization in front of it is
 # bit-exact by the quantizer tests.
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20, 21, 22, 23, 24, 25])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 6, 7, 8, 9, 17, 19, 20, 21, 22, 23, 24, 25, 26])
 @pytest.mark.parametrize("shape,relu,bias,pc,x_signed", [((60, 264, 448), False, True, True, False),
                                                          ((257, 33, 144), True, True, False, False),
                                                          ((16, 1040, 1168), False, False, True, True)])

@@ -273,24 +273,17 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
   }
 }
 
-// The end of a 32 x 32 tile whose four waves each hold a partial sum over their
-// share of K: the partial tiles lie in LDS (wave w's at red + w * red_stride,
-// rows of kSplitRedPitch bytes, written before the barrier the caller has just
-// passed); thread t adds the four for row t / 8, channels 4 (t % 8) ... + 3,
-// requantises and stores.  s_raw: colsum, weight scale and bias of the tile's
-// channels as fetched.
-constexpr int kSplitRedPitch = 32 * 4 + 16;
-template <int MODE>
-__device__ __forceinline__ void ksplit_finish(const GemmArgs& a, const uint8_t* red, int red_stride,
-                                              const int (*s_raw)[kWave], int64_t m0, int64_t n0, int t) {
-  constexpr int kRedPitch = kSplitRedPitch;
-  // ---- thread t: row t / 8, channels 4 (t % 8) ... + 3
-  const int row = t >> 3, cl = (t & 7) * 4;
+// (one thread's share of ksplit_finish: row idx / (BN / 4), channels 4 (idx % (BN / 4)) ... + 3)
+template <int MODE, int BN, int WAVES>
+__device__ __forceinline__ void ksplit_finish_four(const GemmArgs& a, const uint8_t* red, int red_stride,
+                                                   const int (*s_raw)[kWave], int64_t m0, int64_t n0, int idx) {
+  constexpr int kRedPitch = BN * 4 + 16;
+  const int row = idx / (BN / 4), cl = (idx % (BN / 4)) * 4;
   const int64_t m = m0 + row, n = n0 + cl;
   if (m >= a.M || n >= a.N) return;
   v4i sum = *reinterpret_cast<const v4i*>(&red[row * kRedPitch + cl * 4]);
 #pragma unroll
-  for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const v4i*>(&red[w * red_stride + row * kRedPitch + cl * 4]);
+  for (int w = 1; w < WAVES; ++w) sum += *reinterpret_cast<const v4i*>(&red[w * red_stride + row * kRedPitch + cl * 4]);
   const XQuant xq = x_quant(a);
   int raw[4];
   v4f mult = {0.f, 0.f, 0.f, 0.f}, bdiv = {0.f, 0.f, 0.f, 0.f};
@@ -338,6 +331,22 @@ __device__ __forceinline__ void ksplit_finish(const GemmArgs& a, const uint8_t* 
         if (n + j < a.N) dst[j] = static_cast<uint8_t>(q4 >> (8 * j));
     }
   }
+}
+
+// The end of a tile of 32 rows x BN channels whose WAVES waves each hold a partial
+// sum over their share of K: the partial tiles lie in LDS (wave w's at
+// red + w * red_stride, rows of BN * 4 + 16 bytes, written before the barrier the
+// caller has just passed); a thread adds them for four channels of one row,
+// requantises and stores.  s_raw: colsum, weight scale and bias of the tile's
+// channels as fetched.
+constexpr int kSplitRedPitch = 32 * 4 + 16;
+template <int MODE, int BN = 32, int WAVES = 4>
+__device__ __forceinline__ void ksplit_finish(const GemmArgs& a, const uint8_t* red, int red_stride,
+                                              const int (*s_raw)[kWave], int64_t m0, int64_t n0, int t) {
+  constexpr int kRedPitch = BN * 4 + 16;
+  static_assert(BN <= kWave && (32 * BN / 4) % (WAVES * kWave) == 0, "whole passes over the tile");
+#pragma unroll
+  for (int idx = t; idx < 32 * BN / 4; idx += WAVES * kWave) ksplit_finish_four<MODE, BN, WAVES>(a, red, red_stride, s_raw, m0, n0, idx);
 }
 
 // 32 x 32 tiles for K <= 1024 on grids of at most 256 such tiles: the four waves
@@ -455,7 +464,7 @@ __global__ __launch_bounds__(256) void gemm_i8_ksplit_kernel(GemmArgs a, XLinear
 }
 
 // 32 x 32 tiles for K up to 32 * 4 * STEPS bytes (STEPS = 16: 2048, STEPS = 32: 4096)
-// whose four waves split K, the weights going through registers instead of LDS.
+// whose waves split K, the weights going through registers instead of LDS.
 //
 // What a CU can have on its way bounds what it pulls per microsecond: LDS holds
 // at most 160 KB of copies in flight, which at the latency of cold memory is
@@ -468,13 +477,17 @@ __global__ __launch_bounds__(256) void gemm_i8_ksplit_kernel(GemmArgs a, XLinear
 // runs), another 128 KB per block in flight, waits for nobody but its own
 // requests and multiplies as they arrive.  Partial tiles and epilogue as in the
 // kernel above.
-template <int MODE, int STEPS>
-__global__ __launch_bounds__(256) void gemm_i8_wstream_kernel(GemmArgs a, XLinear xs) {
-  constexpr int BM = 32, BN = 32;
+// CT = 2 gives a wave two channel tiles (a block 32 rows x 64 channels, for grids
+// that 32 x 32 tiles would overfill) and WAVES = 8 splits K eight ways, which keeps
+// the weight fragments of two channel tiles within the register file at K up to
+// 4096 (four waves with two channel tiles each measured 9.4 us where eight take 7.3).
+template <int MODE, int STEPS, int CT = 1, int WAVES = 4>
+__global__ __launch_bounds__(WAVES* kWave) void gemm_i8_wstream_kernel(GemmArgs a, XLinear xs) {
+  constexpr int BM = 32, BN = 32 * CT;
   constexpr int SEGS = STEPS / 8;                  // 256-byte segments of K per wave
-  constexpr int kRedPitch = kSplitRedPitch;
-  static_assert(STEPS == 16 || STEPS == 32, "the wait below encodes STEPS outstanding loads in six bits");
-  __shared__ __attribute__((aligned(16))) uint8_t sX[4][SEGS * BM * 256];
+  constexpr int kRedPitch = BN * 4 + 16;
+  static_assert(CT * STEPS == 16 || CT * STEPS == 32, "the wait below names the number of weight loads");
+  __shared__ __attribute__((aligned(16))) uint8_t sX[WAVES][SEGS * BM * 256];
   __shared__ __attribute__((aligned(16))) int s_raw[3][kWave];  // colsum, weight scale, bias as fetched
   static_assert(BM * kRedPitch <= SEGS * BM * 256, "a wave's partial tile fits over its activations");
 
@@ -484,8 +497,8 @@ __global__ __launch_bounds__(256) void gemm_i8_wstream_kernel(GemmArgs a, XLinea
   const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM;
   const int64_t n0 = static_cast<int64_t>(blockIdx.x) * BN;
   const int KC = static_cast<int>(a.K >> 4);       // k-chunks (K is a multiple of 16)
-  const int S = (KC + 1) >> 1;                     // 32-byte k-steps, at most 4 * STEPS
-  const int sp = (S + 3) >> 2;                     // k-steps per wave, at most STEPS
+  const int S = (KC + 1) >> 1;                     // 32-byte k-steps, at most WAVES * STEPS
+  const int sp = (S + WAVES - 1) / WAVES;          // k-steps per wave, at most STEPS
   const int s0 = wave_u * sp;                      // this wave's first k-step
   const int mine = S - s0 < sp ? (S - s0 < 0 ? 0 : S - s0) : sp;
 
@@ -522,34 +535,40 @@ __global__ __launch_bounds__(256) void gemm_i8_wstream_kernel(GemmArgs a, XLinea
       }
     }
   }
-  v4i wf[STEPS];
+  v4i wf[CT][STEPS];
   {
     const int64_t NB = ceil_div(a.N, 16);
-    const int64_t nb_last = NB - 1 - n0 / 16;      // a 16-row block past N: clamped, never stored
-    const int64_t rb = ((lane >> 4) & 1) < nb_last ? ((lane >> 4) & 1) : nb_last;
-    const uint8_t* const wlane = a.w_packed + ((n0 / 16 + rb) * a.w_kchunks) * 256 + (lane & 15) * 16;
+    const int64_t nb_last = NB - 1 - n0 / 16;      // 16-row blocks past N: clamped, never stored
     const int kc_last = static_cast<int>(a.w_kchunks) - 1;
 #pragma unroll
-    for (int j = 0; j < STEPS; ++j) {
-      // (k-steps past this wave's share fetch its last one again and are not multiplied;
-      // an odd last chunk is followed by the zero padding of the packed layout)
-      const int step = s0 + (j < sp ? j : sp - 1);
-      const int kc = 2 * step + half;
-      const int kcc = kc < kc_last ? kc : kc_last;
-      wf[j] = *reinterpret_cast<const v4i*>(wlane + static_cast<int64_t>(kcc) * 256);
+    for (int ct = 0; ct < CT; ++ct) {
+      const int64_t rb0 = 2 * ct + ((lane >> 4) & 1);
+      const int64_t rb = rb0 < nb_last ? rb0 : nb_last;
+      const uint8_t* const wlane = a.w_packed + ((n0 / 16 + rb) * a.w_kchunks) * 256 + (lane & 15) * 16;
+#pragma unroll
+      for (int j = 0; j < STEPS; ++j) {
+        // (k-steps past this wave's share fetch its last one again and are not multiplied;
+        // an odd last chunk is followed by the zero padding of the packed layout)
+        const int step = s0 + (j < sp ? j : sp - 1);
+        const int kc = 2 * step + half;
+        const int kcc = kc < kc_last ? kc : kc_last;
+        wf[ct][j] = *reinterpret_cast<const v4i*>(wlane + static_cast<int64_t>(kcc) * 256);
+      }
     }
   }
 
   const v4i xmask = {static_cast<int>(a.x_xor), static_cast<int>(a.x_xor), static_cast<int>(a.x_xor),
                      static_cast<int>(a.x_xor)};
-  v16i acc;
+  v16i acc[CT];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[ct][r] = 0;
   // The copies into LDS are older than the weight loads and requests return in
-  // order: at most STEPS requests outstanding means the activations have landed.
-  // (as an asm statement that clobbers memory: the compiler may neither sink a
-  // weight load below it nor hoist an LDS read above it)
-  if constexpr (STEPS == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  // order: at most as many requests outstanding as there are weight loads means the
+  // activations have landed.  (An asm statement that clobbers memory: the compiler
+  // may neither sink a weight load below it nor hoist an LDS read above it.)
+  if constexpr (CT * STEPS == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
   {
     const uint8_t* const xrd = &sX[wave_u][0] + li * 256;
@@ -559,19 +578,24 @@ __global__ __launch_bounds__(256) void gemm_i8_wstream_kernel(GemmArgs a, XLinea
         const v4i xf = ld16(xrd + (j / 8) * (BM * 256) + (((2 * (j % 8) + half) ^ (li & 15)) << 4));
         const int keep = j < mine ? -1 : 0;
         const v4i xv = (xf ^ xmask) & v4i{keep, keep, keep, keep};
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xv, acc, 0, 0, 0);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          acc[ct] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ct][j], xv, acc[ct], 0, 0, 0);
       }
     }
   }
   // ---- the partial tile of this wave, over its own activations: a lane holds
-  // channels 8g + 4 half + j (g, j < 4) of activation row li
+  // channels 32 ct + 8g + 4 half + j (g, j < 4) of activation row li
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const v4i part = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
-    *reinterpret_cast<v4i*>(&sX[wave_u][li * kRedPitch + (8 * g + 4 * half) * 4]) = part;
+  for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const v4i part = {acc[ct][4 * g], acc[ct][4 * g + 1], acc[ct][4 * g + 2], acc[ct][4 * g + 3]};
+      *reinterpret_cast<v4i*>(&sX[wave_u][li * kRedPitch + (32 * ct + 8 * g + 4 * half) * 4]) = part;
+    }
   }
   __syncthreads();
-  ksplit_finish<MODE>(a, &sX[0][0], SEGS * BM * 256, s_raw, m0, n0, t);
+  ksplit_finish<MODE, BN, WAVES>(a, &sX[0][0], SEGS * BM * 256, s_raw, m0, n0, t);
 }
 
 }  // namespace tmq

@@ -519,17 +519,19 @@ int launch_gemm_ksplit(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   return launch_status();
 }
 
-// 32 x 32 tiles whose four waves split K, weights through registers (K <= 4096; the caller
-// checked the address ranges).
+// Tiles of 32 rows whose waves split K, weights through registers (K <= 4096; the caller
+// checked the address ranges).  wide: 64 channels per tile instead of 32.
 template <int MODE>
-int launch_gemm_wstream(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
-  const int64_t tiles_m = ceil_div(a.M, 32), tiles_n = ceil_div(a.N, 32);
+int launch_gemm_wstream(const GemmArgs& a, const XLinear& xs, bool wide, hipStream_t s) {
+  const int64_t tiles_m = ceil_div(a.M, 32), tiles_n = ceil_div(a.N, wide ? 64 : 32);
   if (tiles_n > 0x7fffffff || tiles_m > 65535 || a.K > 4096) return TMQ_ERR_UNSUPPORTED;
   const dim3 grid(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m));
-  if (a.K <= 2048)
+  if (!wide && a.K <= 2048)
     gemm_i8_wstream_kernel<MODE, 16><<<grid, dim3(256), 0, s>>>(a, xs);
-  else
+  else if (!wide)
     gemm_i8_wstream_kernel<MODE, 32><<<grid, dim3(256), 0, s>>>(a, xs);
+  else
+    gemm_i8_wstream_kernel<MODE, 16, 2, 8><<<grid, dim3(512), 0, s>>>(a, xs);
   return launch_status();
 }
 
@@ -608,14 +610,21 @@ bool two_wave_groups_fit(int64_t M, int64_t N, int64_t K) {
 
 SplitPlan plan_split_tiles(int64_t M, int64_t N, int64_t K);
 
-// Shapes for the 32 x 32 tiles whose waves split K and stream their weights through
+// Shapes for the tiles of 32 rows whose waves split K and stream their weights through
 // registers: K beyond what the kernels with all operands in LDS take, one round of
 // blocks (two blocks share a CU while a block's activations, 32 rows x K, are at
 // most 64 KB).  With more blocks than that it loses to the larger tiles (K = 4096:
 // N = 4096, M = 96: 13.7 against 12.8 us; K = 2048, N = 4096, M = 256: 10.7 against 9.7 us).
-bool wstream_fits(int64_t M, int64_t N, int64_t K) {
-  if (K <= kOnePassMaxK || K > 4096) return false;
-  return ceil_div(M, 32) * ceil_div(N, 32) <= (K <= 2048 ? 512 : 256);
+// Returns the channels per tile: 32; 64 (eight waves, K > 2048 only: at K <= 2048 it
+// never beat the 32 x 32 tiles where they fit nor the larger tiles where they do not)
+// when only those fit one round (K = N = 4096: M = 96 12.8 -> 9.9 us, M = 128 14.1 -> 10.0 us;
+// N = 8192, M = 64: 15.7 -> 11.5 us; N = 2048, M = 256: 13.6 -> 9.5 us; where both fit, 32
+// channels are 1.5 us ahead); 0: neither.
+int wstream_tile(int64_t M, int64_t N, int64_t K) {
+  if (K <= kOnePassMaxK || K > 4096) return 0;
+  if (ceil_div(M, 32) * ceil_div(N, 32) <= (K <= 2048 ? 512 : 256)) return 32;
+  if (K > 2048 && ceil_div(M, 32) * ceil_div(N, 64) <= 256) return 64;
+  return 0;
 }
 
 SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
@@ -625,7 +634,7 @@ SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
   //   K = 4096, N = 4096:  8.2 / 8.3 / 8.6 | 6.8 / 7.8 / 12.2    K = 4096, N = 1024:  6.5 / 6.5 / 6.6 | 6.0 / 7.0 / 11.3
   //   K = 3072, N = 4096:  7.2 / 7.3 / 7.6 | 6.4 / 7.5 / 11.7    K = 4096, N = 8192: 10.6 / 10.7 / -  | 11.7 / 13.6 / 22.6
   // streaming keeps the longer K up to about two dozen rows while its blocks fit one round.
-  if (wstream_fits(M, N, K)) return K > 2048 && M <= 24 && N <= 4096 ? SmallRows::kStream : SmallRows::kTiles;
+  if (wstream_tile(M, N, K) != 0) return K > 2048 && M <= 24 && N <= 4096 ? SmallRows::kStream : SmallRows::kTiles;
   const double mib = static_cast<double>(N) * static_cast<double>(K) / 1048576.0;
   const double stages = static_cast<double>(ceil_div(K, kBK));
   const double rows = static_cast<double>(M);
@@ -854,12 +863,12 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     // whose waves split K spread the copies over more CUs (3.8 us; M = 512: 5.7 -> 4.4 us;
     // N = 4096, K = 512, M = 128: 4.4 -> 4.3 us; 640 tiles and more, or K <= 256: slower)
     cfg = a.K > 256 && ceil_div(a.M, 32) * ceil_div(a.N, 32) <= 512 ? 24 : 21;
-  } else if (cfg < 0 && onepass_ok && wstream_fits(a.M, a.N, a.K)) {
+  } else if (cfg < 0 && onepass_ok && wstream_tile(a.M, a.N, a.K) != 0) {
     // K up to 4096 on a grid of 32 x 32 tiles that the chip holds at once: the waves split
     // K and take their weights through registers (cold weights, K = N = 4096, M = 64:
     // 12.2 -> 8.6 us; K = 2048, N = 4096: M = 64 9.4 -> 5.5 us, M = 128 9.4 -> 7.0 us;
     // K = N = 2048: M = 128 7.8 -> 5.0 us, M = 256 8.0 -> 6.3 us)
-    cfg = 25;
+    cfg = wstream_tile(a.M, a.N, a.K) == 32 ? 25 : 26;
   } else if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
@@ -932,7 +941,8 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 23: return launch_gemm<64, 128, 2, 2, MODE>(a, xs, s);
     case 21: return onepass_ok ? launch_gemm_onepass<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
     case 24: return onepass_ok ? launch_gemm_ksplit<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
-    case 25: return onepass_ok ? launch_gemm_wstream<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
+    case 25: return onepass_ok ? launch_gemm_wstream<MODE>(a, xs, false, s) : TMQ_ERR_UNSUPPORTED;
+    case 26: return onepass_ok ? launch_gemm_wstream<MODE>(a, xs, true, s) : TMQ_ERR_UNSUPPORTED;
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
