@@ -38,7 +38,7 @@ def test_linear_ops(seed):
     done = 0
     for it in range(40):
         M = int(rng.choice([1, 3, 17, 24, 32, 48, 64, 65, 100, 128, 200, 256, 300, 384, 448, 512, 700, 1024, 1500, 2048]))
-        K = int(rng.choice([16, 64, 100, 128, 320, 384, 448, 1024, 2048, 4096, 8192, 11008]))
+        K = int(rng.choice([16, 64, 100, 128, 320, 384, 448, 1024, 1536, 2048, 3072, 4096, 8192, 11008]))
         N = int(rng.choice([1, 16, 33, 64, 100, 256, 300, 512, 1000, 2048, 4096]))
         pc, relu, bias = (bool(rng.integers(2)) for _ in range(3))
         xs = float(rng.uniform(0.5, 3))
