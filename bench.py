@@ -563,6 +563,39 @@ def main():
                 "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
                 "algorithmic_bytes_per_launch": nbytes}
 
+        # ----------------------------- the same cold weights against a few dozen rows
+        # (32 x 32 / 32 x 64 tiles whose waves split K and take their weights through registers),
+        # with the vendor's int8 GEMM (torch._int_mm: int32 output, no requantisation) beside it
+        wts_mm = None
+        for Md in (64, 128):
+            xd = torch.randint(0, 256, (Md, Kd), dtype=torch.uint8, device=dev)
+            yd = torch.empty((Md, Nd), dtype=torch.uint8, device=dev)
+
+            def run_sets():
+                for p in pws:
+                    cabi.linear(xd, p, 0.02, 128, wsd, bd, 0.05, 128, out=yd)
+
+            per = graph_us(run_sets, sets)
+            vendor = None
+            try:
+                if wts_mm is None:
+                    wts_mm = [torch.randint(-127, 128, (Nd, Kd), dtype=torch.int8, device=dev).t() for _ in range(sets)]
+                xs8 = torch.randint(-128, 128, (Md, Kd), dtype=torch.int8, device=dev)
+                vendor = graph_us(lambda: [torch._int_mm(xs8, wt) for wt in wts_mm], sets)
+            except Exception as ex:  # the comparison is optional: a torch build without the op
+                log(f"[bench] torch._int_mm not timed: {ex}")
+            nbytes = Nd * Kd + Md * Kd + Md * Nd + 12 * Nd
+            log(f"[bench] M={Md} against config 4's cold weights: {per:.2f} us/launch in a replayed graph"
+                + (f" (torch._int_mm: {vendor:.2f} us)" if vendor else ""))
+            secondary[f"linear_m{Md}_k4096_n4096"] = {
+                "avg_launch_us": round(per, 3), "value": round(2.0 * Md * Kd * Nd / per / 1e6, 1), "unit": "TOP/s",
+                "weights_gbs": round(Nd * Kd / per / 1e3, 1),
+                "torch_int_mm_us": None if vendor is None else round(vendor, 3),
+                "method": f"{sets} distinct packed weights replayed back to back in one HIP graph; the vendor GEMM "
+                          "the same way on as many int8 matrices of the shape",
+                "algorithmic_bytes_per_launch": nbytes}
+        del wts_mm
+
         # ----------------------------- dynamically quantized linear, decode-sized
         # fp32 [M, 4096] -> fp32 [M, 4096]: up to 16384 input values one launch (every block
         # of the weight-streaming kernel quantizes the input itself), else one launch for
