@@ -75,7 +75,7 @@ def main():
     ap.add_argument("--skip-secondary", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
-                                       "dequantize_pc", "decode", "conv", "conv_add_relu", "probe"],
+                                       "dequantize_pc", "decode", "rows64", "c1", "conv", "conv_add_relu", "probe"],
                     help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
                          "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
                          "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
@@ -167,18 +167,20 @@ def main():
         print(json.dumps({"only": args.only, "launches": args.steps, "shape": [11008, 4096], "axis": 0}))
         return
 
-    if args.only == "decode":
-        # config 4 at M = 1: 40 packed weights in turn (cold), plain launches
-        pws = [cabi.PackedLinear(torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev))
+    if args.only in ("decode", "rows64", "c1"):
+        # config 4 at M = 1, or 64 rows against the same weights: 40 packed weights in turn (cold);
+        # config 1 (M = 128, K = N = 1024) likewise; plain launches
+        Mo, Ko = {"decode": (1, 4096), "rows64": (64, 4096), "c1": (128, 1024)}[args.only]
+        pws = [cabi.PackedLinear(torch.randint(-127, 128, (Ko, Ko), dtype=torch.int8, device=dev))
                for _ in range(40)]
-        wsd = torch.rand(4096, device=dev) * 0.002 + 0.001
-        bd = torch.randn(4096, device=dev)
-        xd = torch.randint(0, 256, (1, 4096), dtype=torch.uint8, device=dev)
-        yd = torch.empty((1, 4096), dtype=torch.uint8, device=dev)
+        wsd = torch.rand(Ko, device=dev) * 0.002 + 0.001
+        bd = torch.randn(Ko, device=dev)
+        xd = torch.randint(0, 256, (Mo, Ko), dtype=torch.uint8, device=dev)
+        yd = torch.empty((Mo, Ko), dtype=torch.uint8, device=dev)
         for i in range(args.steps):
             cabi.linear(xd, pws[i % 40], 0.02, 128, wsd, bd, 0.05, 128, out=yd)
         torch.cuda.synchronize()
-        print(json.dumps({"only": "decode", "launches": args.steps, "M": 1, "K": 4096, "N": 4096}))
+        print(json.dumps({"only": args.only, "launches": args.steps, "M": Mo, "K": Ko, "N": Ko}))
         return
 
     if args.only in ("conv", "conv_add_relu"):

@@ -223,8 +223,9 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
                      static_cast<int>(a.x_xor)};
   v4i wf0[TN], xf0[TM], wf1[TN], xf1[TM];
   auto mfma = [&](int q, const v4i(&wf)[TN], const v4i(&xf)[TM]) {
-    acc[q / TM][q % TM] =
-        __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[q / TM], xf[q % TM], acc[q / TM][q % TM], 0, 0, 0);
+    static_assert(TN == 2, "the order below pairs the two channel tiles of a row tile");
+    const int tm = q / 2, tn = (q % 2) ^ (tm & 1);  // consecutive products share one operand
+    acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[tn], xf[tm], acc[tn][tm], 0, 0, 0);
   };
   auto flip = [&](v4i& f) { f ^= xmask; };
   const int xswz8 = (li >> 1) & 7;
