@@ -46,13 +46,15 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    "linear_c3": _traffic(161_135, 44_032),       # 375 MB: operands re-fetched 5.3x by the 8 L2s
+    "linear_c3": _traffic(161_128, 44_033),       # 375 MB: operands re-fetched 5.3x by the 8 L2s
     "quantize_c2": _traffic(524_304, 262_144),    # 1.342 GB = algorithmic
-    "dequantize_c2": _traffic(131_084, 1_048_986),
+    "dequantize_c2": _traffic(131_084, 1_048_940),
     "minmax_c2": _traffic(524_315, 64),
-    "quantize_pc": _traffic(88_805, 44_032),
-    "dequantize_pc": _traffic(23_422, 176_218),
-    "decode_m1": _traffic(8_300, 8),              # 17.0 MB for 16.8 MB algorithmic
+    "quantize_pc": _traffic(88_803, 44_032),
+    "dequantize_pc": _traffic(23_421, 176_233),
+    "decode_m1": _traffic(8_301, 8),              # 17.0 MB for 16.8 MB algorithmic
+    "rows64": _traffic(9_347, 256),               # 19.4 MB for 17.4 MB (two row tiles fetch each weight)
+    "c1": _traffic(1_072, 128),
     "conv_c5": _traffic(3_940, 6_272),            # 14.5 MB for 12.9 MB algorithmic (halo overlap)
     "conv_add_relu_c5": _traffic(7_066, 6_272),
 }
@@ -503,6 +505,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(ops1 / (per1 * 1e-3) / 1e12, 2), "peak": PEAK_INT8_TOPS,
                          "unit": "TOP/s", "frac": round(ops1 / (per1 * 1e-3) / 1e12 / PEAK_INT8_TOPS, 5),
                          "traffic": None},
+            "traffic_with_cold_weights": MEASURED_TRAFFIC["c1"],
             "method": "50 launches replayed in one HIP graph; launch-latency-bound at this size",
             "ops_per_launch": ops1, "algorithmic_bytes_per_launch": 128 * 1024 + 1024 * 1024 + 128 * 1024 + 12 * 1024}
         del x1, w1, w1q, p1, g1
@@ -593,6 +596,7 @@ def main():
                 "avg_launch_us": round(per, 3), "value": round(2.0 * Md * Kd * Nd / per / 1e6, 1), "unit": "TOP/s",
                 "weights_gbs": round(Nd * Kd / per / 1e3, 1),
                 "torch_int_mm_us": None if vendor is None else round(vendor, 3),
+                "traffic": MEASURED_TRAFFIC["rows64"] if Md == 64 else None,
                 "method": f"{sets} distinct packed weights replayed back to back in one HIP graph; the vendor GEMM "
                           "the same way on as many int8 matrices of the shape",
                 "algorithmic_bytes_per_launch": nbytes}
