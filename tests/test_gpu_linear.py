@@ -611,18 +611,19 @@ def test_row_pitch_and_output_pitch(cabi):
     xbig = torch.zeros((300, 448 + 64), dtype=torch.uint8, device="cuda")
     xbig[:, 16:464] = dev(c["xq"])
     ybig = torch.full((300, 264 + 40), 7, dtype=torch.uint8, device="cuda")
-    for cfg in (-1, 6, 7, 3, 17, 19):
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"])
+    # (output slices that start on a 4-byte boundary and off it: word and byte stores)
+    for cfg, y0 in [(f, 8) for f in (-1, 6, 7, 3, 17, 19, 21, 24, 25, 26)] + [(f, 6) for f in (-1, 2, 21, 24, 25, 26)]:
         cabi.force_linear_config(cfg)
         try:
             cabi.linear(xbig[:, 16:464], pw, c["x_scale"], c["x_zp"], dev(c["w_scales"].astype(np.float32)),
-                        dev(c["bias"]), c["out_scale"], c["out_zp"], out=ybig[:, 8:272])
+                        dev(c["bias"]), c["out_scale"], c["out_zp"], out=ybig[:, y0:y0 + 264])
         finally:
             cabi.force_linear_config(-1)
-        want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
-                             c["out_scale"], c["out_zp"])
         got = host(ybig)
-        _check(got[:, 8:272], want, f"cfg {cfg}")
-        assert (got[:, :8] == 7).all() and (got[:, 272:] == 7).all()   # nothing written outside the slice
+        _check(got[:, y0:y0 + 264], want, f"cfg {cfg} at column {y0}")
+        assert (got[:, :y0] == 7).all() and (got[:, y0 + 264:] == 7).all()   # nothing written outside the slice
         ybig.fill_(7)
 
 
