@@ -46,15 +46,15 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    "linear_c3": _traffic(161_128, 44_033),       # 375 MB: operands re-fetched 5.3x by the 8 L2s
+    "linear_c3": _traffic(161_134, 44_033),       # 375 MB: operands re-fetched 5.3x by the 8 L2s
     "quantize_c2": _traffic(524_304, 262_144),    # 1.342 GB = algorithmic
-    "dequantize_c2": _traffic(131_084, 1_048_940),
+    "dequantize_c2": _traffic(131_084, 1_049_003),
     "minmax_c2": _traffic(524_315, 64),
-    "quantize_pc": _traffic(88_803, 44_032),
-    "dequantize_pc": _traffic(23_421, 176_233),
-    "decode_m1": _traffic(8_301, 8),              # 17.0 MB for 16.8 MB algorithmic
+    "quantize_pc": _traffic(89_481, 44_032),
+    "dequantize_pc": _traffic(23_424, 176_252),
+    "decode_m1": _traffic(8_300, 8),              # 17.0 MB for 16.8 MB algorithmic
     "rows64": _traffic(9_347, 256),               # 19.4 MB for 17.4 MB (two row tiles fetch each weight)
-    "c1": _traffic(1_072, 128),
+    "c1": _traffic(1_076, 128),
     "conv_c5": _traffic(3_940, 6_272),            # 14.5 MB for 12.9 MB algorithmic (halo overlap)
     "conv_add_relu_c5": _traffic(7_066, 6_272),
 }
