@@ -343,7 +343,6 @@ constexpr int kSplitRedPitch = 32 * 4 + 16;
 template <int MODE, int BN = 32, int WAVES = 4>
 __device__ __forceinline__ void ksplit_finish(const GemmArgs& a, const uint8_t* red, int red_stride,
                                               const int (*s_raw)[kWave], int64_t m0, int64_t n0, int t) {
-  constexpr int kRedPitch = BN * 4 + 16;
   static_assert(BN <= kWave && (32 * BN / 4) % (WAVES * kWave) == 0, "whole passes over the tile");
 #pragma unroll
   for (int idx = t; idx < 32 * BN / 4; idx += WAVES * kWave) ksplit_finish_four<MODE, BN, WAVES>(a, red, red_stride, s_raw, m0, n0, idx);

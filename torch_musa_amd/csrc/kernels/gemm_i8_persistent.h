@@ -46,7 +46,6 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   uint64_t* const __restrict__ stamps = STAMPS ? a.stamps : nullptr;
   constexpr int BM = 256, BN = 256, WM = 2, WN = 4;
   constexpr int NWAVES = WM * WN;
-  constexpr int NT = NWAVES * kWave;
   constexpr int WTM = BM / WM, WTN = BN / WN;      // 128 rows x 64 channels per wave
   constexpr int TM = WTM / 32, TN = WTN / 32;      // 4 x 2 MFMA tiles
   constexpr int Q = TN * TM, NF = TN + TM;
