@@ -96,13 +96,17 @@ __device__ __forceinline__ void resolve(const QParamsArg& a, float& inv, float& 
 // n - 4*n4 (< 4) trailing elements one by one.
 // The fp32 input is read once and never again: non-temporal loads keep it out of
 // the caches.  The codes are written with ordinary stores, so a consumer that
-// follows on the stream (dequantize, a GEMM) finds them in the last-level cache.
+// follows on the stream (dequantize, a GEMM) finds them in the last-level cache --
+// unless there are more of them than that cache holds (STREAM_OUT, 128 MiB and
+// up): then they leave with non-temporal stores as well (2**28 elements into a
+// different output buffer every launch: 211 -> 205.5 us).
 // Blocks of two waves, as for the dequantizer below: of 128 / 256 / 512 threads with two
 // or four accesses each, two waves x two accesses moved 2**28 elements fastest (213 us
 // against 219-225 us in one run).
 constexpr int kQThreads = 128;
 
-template <bool SIGNED, bool FUSED = false>
+constexpr int64_t kStreamOutCodes = int64_t{1} << 27;
+template <bool SIGNED, bool FUSED = false, bool STREAM_OUT = false>
 __global__ __launch_bounds__(kQThreads) void quantize_vec_kernel(
     const v4f* __restrict__ x4, uint32_t* __restrict__ q4, int64_t n4,
     const float* __restrict__ x, uint8_t* __restrict__ q, int64_t n, QParamsArg qp) {
@@ -114,7 +118,11 @@ __global__ __launch_bounds__(kQThreads) void quantize_vec_kernel(
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u) v[u] = __builtin_nontemporal_load(&x4[base + u * kQThreads]);
 #pragma unroll
-    for (int u = 0; u < kUnrollQD; ++u) q4[base + u * kQThreads] = quantize_four<SIGNED, FUSED>(v[u], inv, zp_f);
+    for (int u = 0; u < kUnrollQD; ++u) {
+      const uint32_t codes = quantize_four<SIGNED, FUSED>(v[u], inv, zp_f);
+      if constexpr (STREAM_OUT) __builtin_nontemporal_store(codes, &q4[base + u * kQThreads]);
+      else q4[base + u * kQThreads] = codes;
+    }
   } else {
 #pragma unroll
     for (int u = 0; u < kUnrollQD; ++u) {
@@ -741,8 +749,12 @@ int quantize_launch_as(const float* x, void* q, int64_t n, QParamsArg qp, hipStr
     const int64_t n4 = n / 4;
     const int64_t blocks = n4 == 0 ? 1 : ceil_div(n4, kQThreads * kUnrollQD);
     if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-    quantize_vec_kernel<SIGNED, FUSED><<<dim3(blocks), dim3(kQThreads), 0, s>>>(
-        reinterpret_cast<const v4f*>(x), reinterpret_cast<uint32_t*>(q), n4, x, qb, n, qp);
+    if (n >= kStreamOutCodes)
+      quantize_vec_kernel<SIGNED, FUSED, true><<<dim3(blocks), dim3(kQThreads), 0, s>>>(
+          reinterpret_cast<const v4f*>(x), reinterpret_cast<uint32_t*>(q), n4, x, qb, n, qp);
+    else
+      quantize_vec_kernel<SIGNED, FUSED><<<dim3(blocks), dim3(kQThreads), 0, s>>>(
+          reinterpret_cast<const v4f*>(x), reinterpret_cast<uint32_t*>(q), n4, x, qb, n, qp);
   } else {
     const unsigned g = grid_for(n, kThreads, 65536);
     quantize_scalar_kernel<SIGNED, FUSED><<<dim3(g), dim3(kThreads), 0, s>>>(x, qb, n, qp);
