@@ -193,8 +193,8 @@ def main():
         return
 
     if args.only in ("conv", "conv_add_relu"):
-        # config 5: 24 inputs in turn (309 MB, more than the last-level cache)
-        csets = 24
+        # config 5: 48 inputs in turn (308 MB, more than the last-level cache)
+        csets = 48
         xcqs = [torch._make_per_tensor_quantized_tensor(
             torch.randint(0, 120, (32, 56, 56, 64), dtype=torch.uint8, device=dev).permute(0, 3, 1, 2), 0.03, 0)
             for _ in range(csets)]
@@ -785,9 +785,9 @@ def main():
         wcs = (wc.abs().amax(dim=(1, 2, 3)) / 127.0).to(torch.float64)
         wcq = torch.quantize_per_channel(wc, wcs, torch.zeros(64, dtype=torch.int64, device=dev), 0, torch.qint8)
         pc = torch.ops.quantized.conv2d_prepack(wcq, torch.randn(64, device=dev), [1, 1], [1, 1], [1, 1], 1)
-        # 24 input tensors (and as many outputs inside the graph): 309 MB, more than
-        # the last-level cache, so a launch does not find its input cached
-        csets = 24
+        # 48 input tensors: 308 MB, more than the last-level cache, so a launch does not
+        # find its input cached
+        csets = 48
         xcqs = [xcq]
         for _ in range(csets - 1):
             xf_ = torch.relu(torch.randn(32, 64, 56, 56, device=dev)).contiguous(memory_format=torch.channels_last)
