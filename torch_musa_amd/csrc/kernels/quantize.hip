@@ -566,7 +566,7 @@ struct PcQuantize {
 template <bool SIGNED>
 struct PcDequantize {
   // codes -> fp32, double scales, int64 zero points
-  static constexpr int kAccesses = 4;
+  static constexpr int kAccesses = 2;
   const uint8_t* q;
   float* r;
   const double* scales;
@@ -622,7 +622,7 @@ struct PcfQuantize {
 template <bool SIGNED>
 struct PcfDequantize {
   // codes -> fp32, float scales and float zero points
-  static constexpr int kAccesses = 4;
+  static constexpr int kAccesses = 2;
   const uint8_t* q;
   float* r;
   const float* scales;
@@ -646,13 +646,14 @@ struct PcfDequantize {
   }
 };
 
-// Accesses per thread (Op::kAccesses), all in flight before the first store: four
-// (at fp32 [11008, 4096], axis 0, with blocks inside the tensor taking the path
-// without a condition per access: quantize 36.7 / 36.7 / 37.4 us with 2 / 4 / 8,
-// against 38.7 us with 8 and a condition per access; dequantize 33.8 / 33.4 /
-// 36.0 / 38.7 us with 2 / 4 / 8 / 16; the per-tensor quantizer on as many
-// elements takes 35.7 us).
-constexpr int kPcThreads = 256;  // 64 ... 512 threads per block measure within 3 % of each other
+// Accesses per thread (Op::kAccesses), all in flight before the first store: four for
+// the quantizers, two for the dequantizers, in blocks of two waves -- the shape the
+// per-tensor kernels settled on as well.  At fp32 [11008, 4096], axis 0, inputs and
+// outputs rotating over more bytes than the last-level cache holds: quantize 39.8 us
+// (per-tensor kernel on as many elements: 38.4 us), dequantize 37.6 us (35.4 us);
+// the dequantizer took 42.2 us with a parameter request per access, each waiting for
+// the one before it, 39.4 us with one per row in blocks of four waves x four accesses.
+constexpr int kPcThreads = 128;
 template <class Op, int VEC>
 __global__ __launch_bounds__(kPcThreads) void pc_rows_kernel(Op op, int64_t rows, int64_t C, int64_t inner,
                                                            int lg_us, uint32_t segs) {
@@ -670,22 +671,43 @@ __global__ __launch_bounds__(kPcThreads) void pc_rows_kernel(Op op, int64_t rows
   const bool whole = row0 + (kPcAccesses >> lg_us) <= rows &&
                      ((static_cast<int64_t>(seg) + 1) << lg_us) * (kPcThreads * VEC) <= inner;
   if (whole) {
+    // with the number of runs per row as a constant, every index below is one: the
+    // parameters of the block's rows are requested together, once per row (not once
+    // per access, each request waiting for the one before it)
+    auto run = [&](auto lg_tag) {
+      constexpr int LG = decltype(lg_tag)::value;
+      if constexpr ((1 << LG) <= kPcAccesses) {
+        constexpr int kRows = kPcAccesses >> LG, kRuns = 1 << LG;
 #pragma unroll
-    for (int u = 0; u < kPcAccesses; ++u) {
-      const int64_t row = row0 + (u >> lg_us);
-      const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kPcThreads * VEC);
-      if constexpr (VEC == 4) held[u] = op.load4(row * inner + col);
-      else held[u] = op.load1(row * inner + col);
-    }
+        for (int r = 0; r < kRows; ++r)
 #pragma unroll
-    for (int u = 0; u < kPcAccesses; ++u) {
-      const int64_t row = row0 + (u >> lg_us);
-      int64_t c = c0 + (u >> lg_us);
-      while (c >= C) c -= C;
-      const typename Op::P p = op.params(c);
-      const int64_t col = col0 + static_cast<int64_t>(u & us_mask) * (kPcThreads * VEC);
-      if constexpr (VEC == 4) op.store4(row * inner + col, held[u], p);
-      else op.store1(row * inner + col, held[u], p);
+          for (int k = 0; k < kRuns; ++k) {
+            const int64_t at = (row0 + r) * inner + col0 + static_cast<int64_t>(k) * (kPcThreads * VEC);
+            if constexpr (VEC == 4) held[r * kRuns + k] = op.load4(at);
+            else held[r * kRuns + k] = op.load1(at);
+          }
+        typename Op::P prm[kRows];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+          int64_t c = c0 + r;
+          while (c >= C) c -= C;   // at most kRows - 1 rows past c0: uniform, a few scalar steps
+          prm[r] = op.params(c);
+        }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+          for (int k = 0; k < kRuns; ++k) {
+            const int64_t at = (row0 + r) * inner + col0 + static_cast<int64_t>(k) * (kPcThreads * VEC);
+            if constexpr (VEC == 4) op.store4(at, held[r * kRuns + k], prm[r]);
+            else op.store1(at, held[r * kRuns + k], prm[r]);
+          }
+      }
+    };
+    switch (lg_us) {
+      case 0: run(std::integral_constant<int, 0>{}); break;
+      case 1: run(std::integral_constant<int, 1>{}); break;
+      case 2: run(std::integral_constant<int, 2>{}); break;
+      default: run(std::integral_constant<int, 3>{}); break;
     }
     return;
   }
