@@ -49,10 +49,10 @@ def _traffic(fetch_kib, write_kib):
 MEASURED_TRAFFIC = {
     "linear_c3": _traffic(161_134, 44_033),       # 375 MB: operands re-fetched 5.3x by the 8 L2s
     "quantize_c2": _traffic(524_304, 262_144),    # 1.342 GB = algorithmic
-    "dequantize_c2": _traffic(131_084, 1_048_847),
+    "dequantize_c2": _traffic(131_084, 1_048_819),
     "minmax_c2": _traffic(524_316, 64),
-    "quantize_pc": _traffic(89_475, 44_032),
-    "dequantize_pc": _traffic(23_433, 176_180),
+    "quantize_pc": _traffic(89_478, 44_032),
+    "dequantize_pc": _traffic(23_423, 176_136),
     "decode_m1": _traffic(8_300, 8),              # 17.0 MB for 16.8 MB algorithmic
     "rows64": _traffic(9_347, 256),               # 19.4 MB for 17.4 MB (two row tiles fetch each weight)
     "c1": _traffic(1_076, 128),
