@@ -204,6 +204,42 @@ def test_weights_through_registers_kernel(cabi, shape, x_signed, cfg):
     np.testing.assert_array_equal(acc1, acc)
 
 
+def test_small_batch_kernels_on_random_shapes(cabi):
+    """The kernels that hold or stream all of K (64 x 64 and 32 x 32 tiles in LDS, 32-row tiles
+    with weights through registers) against the pipelined 64 x 64 tiles on seeded random shapes
+    around their tile and K boundaries: bytes, accumulators and float outputs equal, and the
+    automatic choice with them."""
+    import random
+    rnd = random.Random(7)
+    torch.manual_seed(7)
+    for it in range(48):
+        M = rnd.choice([1, 2, 17, 31, 32, 33, 63, 64, 65, 100, 129, 255, 300]) if it % 3 else rnd.randint(1, 300)
+        N = rnd.choice([1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 257, 600]) if it % 2 else rnd.randint(1, 600)
+        K = 16 * rnd.randint(1, 256)
+        signed, pc, relu, bias = (bool(rnd.getrandbits(1)) for _ in range(4))
+        say("random small-batch shape", it, (M, N, K), signed, pc, relu, bias)
+        xq = (torch.randint(-128, 128, (M, K), device="cuda", dtype=torch.int8) if signed
+              else torch.randint(0, 256, (M, K), device="cuda", dtype=torch.uint8))
+        pw = cabi.PackedLinear(torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8))
+        ws = torch.rand(N if pc else 1, device="cuda") * 0.002 + 0.0005
+        b = torch.randn(N, device="cuda") if bias else None
+        zp = rnd.randint(-20, 20) if signed else rnd.randint(0, 255)
+        ozp = rnd.randint(-128, 127) if signed else rnd.randint(0, 255)
+
+        def run(cfg):
+            cabi.force_linear_config(cfg)
+            try:
+                return (cabi.linear(xq, pw, 0.03, zp, ws, b, 0.7, ozp, relu=relu), cabi.linear_acc32(xq, pw),
+                        cabi.linear_f32(xq, pw, 0.03, zp, ws, b, relu=relu))
+            finally:
+                cabi.force_linear_config(-1)
+
+        want = run(2)
+        for cfg in [c for c in (21, 24, 25, 26, -1) if not (c == 24 and K > 1024)]:
+            for got, ref, what in zip(run(cfg), want, ("bytes", "accumulators", "float output")):
+                assert torch.equal(got, ref), f"cfg {cfg} {what} at {(M, N, K)}"
+
+
 # the persistent kernel over more tiles than the chip has CUs: every block walks two tiles
 # (ragged last row and column tiles, K that ends inside a stage and inside a pair of stages)
 @pytest.mark.parametrize("shape,x_signed,relu,pc", [((4389, 4120, 448), False, False, True),
