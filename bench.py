@@ -249,23 +249,36 @@ def main():
         counter[0] += 1
         return torch.ops.quantized.linear(xqs[i], packs[i], out_scale, out_zp)
 
+    def settle():
+        """The clock governor needs ~40 ms of this load before the launch time settles (206 us
+        for the first launches, 170 us from about the 200th on): 0.2 s of untimed steps."""
+        t_, n_ = time.perf_counter(), 0
+        while time.perf_counter() - t_ < 0.2:
+            for _ in range(20):
+                step()
+            torch.cuda.synchronize()
+            n_ += 20
+        return n_
+
     if args.only == "linear":
+        # the timed region of the full run and nothing else: the same settle phase, then
+        # --steps launches between one pair of events (a kernel trace of this command holds
+        # settle + steps launches of the one kernel; its last --steps rows are the timed ones)
+        settle_steps = settle()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
         for _ in range(args.steps):
             step()
+        ev1.record()
         torch.cuda.synchronize()
-        print(json.dumps({"only": "linear", "launches": args.steps, "M": M, "K": K, "N": N}))
+        us = ev0.elapsed_time(ev1) / args.steps * 1e3
+        print(json.dumps({"only": "linear", "launches": args.steps, "untimed_settle_steps": settle_steps,
+                          "avg_launch_us": round(us, 2), "tops": round(2.0 * M * N * K / us / 1e6, 1),
+                          "frac_of_int8_peak": round(2.0 * M * N * K / us / 1e6 / PEAK_INT8_TOPS, 4),
+                          "M": M, "K": K, "N": N}))
         return
 
-    # The clock governor needs ~40 ms of this load before the launch time
-    # settles (206 us for the first launches, 170 us from about the 200th on):
-    # 0.2 s of untimed steps first, then the W warm-up steps, then the K timed ones.
-    settle_t0 = time.perf_counter()
-    settle_steps = 0
-    while time.perf_counter() - settle_t0 < 0.2:
-        for _ in range(20):
-            step()
-        torch.cuda.synchronize()
-        settle_steps += 20
+    settle_steps = settle()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -309,76 +322,6 @@ def main():
             log(f"[bench]   {name}: {tops_p:.0f} TOP/s at {ghz_p:.2f} GHz")
         secondary["mfma_i8_ceiling_probe"] = probe
 
-        # ---------------------------------------------- where a C3 launch spends its time
-        # The instrumented instantiation of the persistent GEMM (measurement library) writes
-        # wall-clock and cycle stamps per block and tile; with the copies left out (results
-        # wrong) it also says what the operand traffic costs in clock and cycles.
-        log("[bench] time budget of a config 3 launch (instrumented kernel, stamps per block and tile)")
-        pw_b = cabi.PackedLinear(wq.int_repr())
-        ws_b = w_scales.to(torch.float32)
-        x_b = xq.int_repr()
-        y_b = torch.empty((M, N), dtype=torch.uint8, device=dev)
-
-        def budget_once(flags):
-            for _ in range(20):
-                step()
-            st = cabi.bench_linear_stamps(x_b, pw_b, xq.q_scale(), xq.q_zero_point(), ws_b, bias, out_scale, out_zp,
-                                          y_b, flags)
-            torch.cuda.synchronize()
-            return st.cpu().numpy().astype(np.float64)
-
-        def summarise(st):
-            wall, cyc = st[:, 0, :] / 100.0, st[:, 1, :]          # us, cycles
-            tiles_total = ((M + 255) // 256) * ((N + 255) // 256)
-            ntile = np.where(np.arange(256) < tiles_total - 2 * 256, 3, 2)
-            out = {"launch_us": round(float(max(wall[i, 4 * ntile[i]] for i in range(256)) - wall[:, 0].min()), 1),
-                   "first_operands_us": round(float(np.mean(wall[:, 1] - wall[:, 0])), 2)}
-            for t, name in ((0, "round_1"), (1, "round_2"), (2, "round_3")):
-                sel = ntile > t
-                ls, le, lb, ee = (wall[sel, 1 + 4 * t + k] for k in range(4))
-                cl = cyc[sel, 2 + 4 * t] - cyc[sel, 1 + 4 * t]
-                ce = cyc[sel, 4 + 4 * t] - cyc[sel, 3 + 4 * t]
-                out[name] = {"blocks": int(sel.sum()), "loop_us": round(float(np.mean(le - ls)), 2),
-                             "loop_cycles": int(np.mean(cl)),
-                             "shader_ghz_in_loop": round(float(np.mean(cl) / np.mean(le - ls) / 1e3), 3),
-                             "barrier_us": round(float(np.mean(lb - le)), 2),
-                             "epilogue_us": round(float(np.mean(ee - lb)), 2), "epilogue_cycles": int(np.mean(ce))}
-            return out
-
-        for _ in range(300):
-            step()
-        torch.cuda.synchronize()
-        # the four variants in turn, seven times over; per variant the launch with the median full-round loop time
-        names = ("all_copies", "no_activation_copies", "no_weight_copies", "no_copies")
-        runs = {n: [] for n in names}
-        for _ in range(7):
-            for f, n in enumerate(names):
-                runs[n].append(summarise(budget_once(f)))
-        tb = {n: sorted(r, key=lambda o: o["round_1"]["loop_us"])[len(r) // 2] for n, r in runs.items()}
-        tb["full_round_loop_us_all_launches"] = {n: [o["round_1"]["loop_us"] for o in r] for n, r in runs.items()}
-        tb["matrix_pipe_cycles_per_tile"] = (K // 64) * 512
-        tb["method"] = ("single launches of gemm_i8_persistent_kernel<kOutU8, STAMPS, SKIP> after 20 operator steps "
-                        "each, the four variants in turn, seven times; thread 0 of every block stamps the 100 MHz wall "
-                        "clock and the shader cycle counter; the variants without copies multiply stale operands "
-                        "(timing only); reported per variant: the launch with the median full-round loop time")
-        # Does the order of the work matter?  Blocks that have slack (two tiles instead of
-        # three) start 40 us late; every second CU of each XCD starts 24 us late, so that the
-        # halves of the chip reach their epilogues at different times.  Same output bytes.
-        late = {"none": 0, "two_tile_blocks_40us_late": 40 << 8, "every_second_cu_24us_late": (24 << 8) | (1 << 4)}
-        late_runs = {n: [] for n in late}
-        for _ in range(5):
-            for n, f in late.items():
-                late_runs[n].append(summarise(budget_once(f))["launch_us"])
-        tb["late_start_launch_us"] = {n: float(np.median(r)) for n, r in late_runs.items()}
-        tb["late_start_method"] = ("the same instrumented kernel with a bounded wait on the wall clock before a block's "
-                                   "first copy; launch = first block start to last epilogue end; median of 5, in turn")
-        secondary["linear_c3_time_budget"] = tb
-        r1 = tb["all_copies"]["round_1"]
-        log(f"[bench]   full round: loop {r1['loop_us']} us = {r1['loop_cycles']} cycles at {r1['shader_ghz_in_loop']} GHz "
-            f"(matrix pipe alone: {tb['matrix_pipe_cycles_per_tile']}), epilogue {r1['epilogue_cycles']} cycles; last round "
-            f"at {tb['all_copies']['round_3']['shader_ghz_in_loop']} GHz; without copies "
-            f"{tb['no_copies']['round_1']['loop_us']} us at {tb['no_copies']['round_1']['shader_ghz_in_loop']} GHz")
-        del pw_b, x_b, y_b
         roofline["power_limited_ceiling_tops"] = probe["gaussian_int8"]["tops"]
         roofline["frac_of_power_limited_ceiling"] = round(achieved / probe["gaussian_int8"]["tops"], 4)
         # the same with operands that change every instruction, as a GEMM's do

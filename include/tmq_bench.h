@@ -40,22 +40,6 @@ int tmq_probe_mfma_i8(int data_mode, int blocks, int iters, void* scratch, doubl
 int tmq_bench_stream_read(const void* src, int64_t bytes, void* sink, void* stream);
 int tmq_bench_empty_kernel(int blocks, void* sink, void* stream);
 
-/* Where a launch of the persistent int8 GEMM (quantized::linear on more than one
- * round of 256 x 256 tiles) spends its time: launches the kernel's instrumented
- * instantiation on `desc` (tmq.h's descriptor; quint8 output, the shapes the
- * library sends to that kernel) with `stamps` = device memory for
- * blocks x 2 x 16 uint64 (blocks = min(tiles, compute units rounded down to a
- * multiple of 8)): [block][0][i] the 100 MHz wall clock, [block][1][i] the
- * shader cycle counter, i = 0 at the block's start, then per tile 1 + 4t: main
- * loop starts, 2 + 4t: main loop ends, 3 + 4t: behind the barrier after it,
- * 4 + 4t: epilogue ends.  flags & 1 leaves out the activation copies, flags & 2
- * the weight copies (stale operands: the output is wrong, for timing only).
- * Bits 8..15 of flags: some blocks start that many microseconds late (a schedule
- * experiment; same output) -- with bit 4 clear the blocks that have one tile
- * fewer than the others, with bit 4 set every second compute unit of each XCD.
- * Asynchronous on `stream`. */
-int tmq_bench_linear_stamps(const tmq_linear_desc* desc, uint64_t* stamps, int flags, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -39,7 +39,7 @@ def test_measurement_probe_lives_in_its_own_library():
     text = open(os.path.join(ROOT, "include", "tmq_bench.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = sorted(set(re.findall(r"\b(tmq_[a-z0-9_]+)\s*\(", text)))
-    assert names == ["tmq_bench_empty_kernel", "tmq_bench_linear_stamps", "tmq_bench_stream_read", "tmq_probe_mfma_i8"]
+    assert names == ["tmq_bench_empty_kernel", "tmq_bench_stream_read", "tmq_probe_mfma_i8"]
     for name in names:
         assert hasattr(cabi.bench_lib(), name)
         assert not hasattr(cabi.lib(), name)

@@ -29,7 +29,7 @@ ARCH = "gfx950"
 
 KERNEL_SOURCES = ["kernels/quantize.hip", "kernels/linear.hip", "kernels/conv2d.hip",
                   "kernels/elementwise.hip"]
-BENCH_SOURCES = ["bench/bench_kernels.hip", "bench/linear_stamps.hip"]
+BENCH_SOURCES = ["bench/bench_kernels.hip"]
 ATEN_SOURCES = ["aten/register.cpp"]
 
 # -ffp-contract=off: the requantisation epilogue and the quantizer must round

@@ -658,7 +658,6 @@ def bench_lib() -> C.CDLL:
                                         C.POINTER(C.c_double)]
         l.tmq_bench_stream_read.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
         l.tmq_bench_empty_kernel.argtypes = [C.c_int, C.c_void_p, C.c_void_p]
-        l.tmq_bench_linear_stamps.argtypes = [C.POINTER(LinearDesc), C.c_void_p, C.c_int, C.c_void_p]
         _bench_lib = l
     return _bench_lib
 
@@ -671,19 +670,6 @@ def bench_stream_read(src: torch.Tensor, sink: torch.Tensor) -> None:
 
 def bench_empty_kernel(blocks: int, sink: torch.Tensor) -> None:
     check(bench_lib().tmq_bench_empty_kernel(blocks, sink.data_ptr(), stream_ptr()), "tmq_bench_empty_kernel")
-
-
-def bench_linear_stamps(x, pw: "PackedLinear", x_scale, x_zp, w_scales, bias, out_scale, out_zp, out,
-                        flags: int = 0) -> torch.Tensor:
-    """One launch of the instrumented persistent GEMM (quint8 in and out) -> int64 [blocks, 2, 16]
-    on the device: wall clock (10 ns units) and shader cycles at the block's start and per tile at
-    loop start / loop end / behind the barrier / epilogue end.  flags & 1 / & 2 leave out the
-    activation / weight copies (wrong output, timing only)."""
-    d = _linear_desc(x, pw, x_scale, x_zp, w_scales, bias, out_scale, out_zp, False, False, out)
-    stamps = torch.zeros((256, 2, 16), dtype=torch.int64, device=x.device)
-    check(bench_lib().tmq_bench_linear_stamps(C.byref(d), stamps.data_ptr(), flags, stream_ptr()),
-          "tmq_bench_linear_stamps")
-    return stamps
 
 
 def probe_mfma_i8(data_mode: int, blocks: int = 256, iters: int = 20000):

@@ -102,13 +102,6 @@ struct GemmArgs {
   int32_t splits = 1;
   int32_t split_stages = 0;
   int64_t split_stride = 0;
-  // Instrumented builds of a kernel only (the measurement library): where the
-  // blocks write their time stamps.
-  uint64_t* stamps = nullptr;
-  // Instrumented builds only: the blocks late_mode selects wait late_ticks of the
-  // 100 MHz wall clock before their first copy.  0: nobody waits.
-  uint32_t late_ticks = 0;
-  uint32_t late_mode = 0;
 };
 
 struct XQuant {

@@ -31,19 +31,9 @@ namespace tmq {
 
 constexpr int kPersistThreads = 512;
 
-//
-// STAMPS = true is the instrumented instantiation of the measurement library:
-// thread 0 of every block writes the 100 MHz wall clock and the shader cycle
-// counter to a.stamps[block][2][16] at the block's start and, per tile, when its
-// main loop starts, when it ends, behind the barrier after it and when the
-// epilogue ends; SKIP & 1 leaves out the activation copies, SKIP & 2 the weight
-// copies (stale operands: wrong results, for timing only); a.late_ticks delays
-// the start of some blocks (same results, for timing only).
-template <int MODE, bool STAMPS = false, int SKIP = 0>
+template <int MODE>
 __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(GemmArgs a, XLinear xsrc) {
   static_assert(MODE == kOutU8 || MODE == kOutS8 || MODE == kOutF32, "byte or float outputs");
-  // (read once, before anything is stored: the arguments stay in scalar registers)
-  uint64_t* const __restrict__ stamps = STAMPS ? a.stamps : nullptr;
   constexpr int BM = 256, BN = 256, WM = 2, WN = 4;
   constexpr int NWAVES = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;      // 128 rows x 64 channels per wave
@@ -142,13 +132,11 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
     }
   };
   auto dma_w = [&](int kt, int wb, int i) {
-    if constexpr ((SKIP & 2) != 0) return;
     lds_dma16(wtile + static_cast<int64_t>(kt) * (kChunks * 256), wdma_off[i],
               wdma_lds + wb * kWStage + i * (NWAVES / 4) * 64 * 16);
   };
   auto dma_x = [&](int u, int xb, int i) {
     const int uc = u < pair_last ? u : pair_last;
-    if constexpr ((SKIP & 1) != 0) return;
     lds_dma16(xtile + static_cast<int64_t>(uc) * (2 * kBK), uc == pair_last ? xdma_off_last[i] : xdma_off[i],
               xdma_lds + xb * kXStage + i * NWAVES * 1024);
   };
@@ -371,31 +359,8 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
   };
 
   // ---- the block's tiles
-  int stamp_i = 0;
-  auto stamp = [&]() {
-    if constexpr (STAMPS) {
-      if (stamps != nullptr && threadIdx.x == 0 && stamp_i < 16) {
-        stamps[blockIdx.x * 32 + stamp_i] = wall_clock64();
-        stamps[blockIdx.x * 32 + 16 + stamp_i] = clock64();
-      }
-      ++stamp_i;
-    }
-  };
-  stamp();
   uint32_t v = blockIdx.x;
   if (v >= nblocks) return;
-  if constexpr (STAMPS) {
-    if (a.late_ticks != 0) {
-      // A schedule experiment: some blocks wait before their first copy (a bounded
-      // wait on the wall clock).  Mode 0: the blocks with one tile fewer than the
-      // others, which have that slack; mode 1: every second CU of each XCD, so that
-      // the halves of the chip reach their epilogues at different times.
-      const uint32_t part = nblocks % gridDim.x;
-      const bool waits = a.late_mode == 0 ? (part != 0 && blockIdx.x >= part) : ((blockIdx.x >> 3) & 1) != 0;
-      const uint64_t t0 = wall_clock64();
-      for (int i = 0; waits && i < 400 && wall_clock64() - t0 < a.late_ticks; ++i) __builtin_amdgcn_s_sleep(8);
-    }
-  }
   int m0, n0;
   tile_origin(v, &m0, &n0);
   tile_setup(m0, n0);
@@ -411,7 +376,6 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
     // previous epilogue); the barrier makes every wave's copies and the
     // constants visible and ends the previous epilogue's use of the staging rows
     __syncthreads();
-    stamp();
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
       v16i init;
@@ -435,10 +399,8 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
       if (kt0 + j < KT) stage(kt0 + j, j);
     // the last copies (past the end of K, never read) must have landed, and every
     // wave must be done with the ring, before the next tile's copies reuse it
-    stamp();
     wait_loads(std::integral_constant<int, 0>{});
     __syncthreads();
-    stamp();
 
     const int em0 = m0, en0 = n0;
     v += gridDim.x;
@@ -458,7 +420,6 @@ __global__ __launch_bounds__(kPersistThreads, 1) void gemm_i8_persistent_kernel(
       else
         epilogue(em0, en0, par, std::true_type{});
     }
-    stamp();
     if (!more) break;
     store_consts(next, par ^ 1);
     par ^= 1;
