@@ -65,6 +65,96 @@ PROBE_MODES = ((0, "zero_operands"), (1, "uniform_random_int8"), (2, "gaussian_i
                (3, "gaussian_int8_fresh_from_lds"), (4, "gaussian_int8_one_operand_non_negative"),
                (5, "gaussian_int8_16x16x64"))
 
+# Socket power and shader clock while a load runs: a child process, started before this
+# process touches the GPU and never touching the GPU runtime itself, waits on its stdin for
+# "S <seconds>", then reads the amdgpu hwmon files of card 0 every ~2 ms for that long, asks
+# amd-smi for the per-XCD shader clocks once in the middle, and answers with one JSON line.
+# Everything is optional: a box that hides the files gives {"available": false, ...}.
+_SAMPLER = r"""
+import glob, json, subprocess, sys, time
+def rd(p):
+    with open(p) as f:
+        return int(f.read().strip())
+def sample(seconds):
+    out = {"available": False}
+    try:
+        hw = sorted(glob.glob("/sys/class/drm/card[0-9]*/device/hwmon/hwmon*"))
+        hw = [h for h in hw if glob.glob(h + "/power1_input") or glob.glob(h + "/power1_average")]
+        h = hw[0]
+        pfile = (glob.glob(h + "/power1_input") + glob.glob(h + "/power1_average"))[0]
+        try:
+            out["power_cap_w"] = rd(h + "/power1_cap") / 1e6
+        except Exception:
+            out["power_cap_w"] = None
+        watts, clocks, t0, asked = [], [], time.time(), False
+        while time.time() - t0 < seconds:
+            watts.append(rd(pfile) / 1e6)
+            if not asked and time.time() - t0 > seconds * 0.4:
+                asked = True
+                try:
+                    r = subprocess.run(["amd-smi", "metric", "--clock", "--json"], stdout=subprocess.PIPE,
+                                       stderr=subprocess.DEVNULL, text=True, timeout=10)
+                    g = json.loads(r.stdout)
+                    g = g["gpu_data"][0] if isinstance(g, dict) else g[0]
+                    clocks = [v["clk"]["value"] for k, v in g["clock"].items()
+                              if k.startswith("gfx_") and isinstance(v.get("clk"), dict)
+                              and isinstance(v["clk"].get("value"), (int, float))]
+                except Exception as e:
+                    out["clock_error"] = str(e)[:120]
+            time.sleep(0.002)
+        watts.sort()
+        out.update(available=True, samples=len(watts), socket_power_w_avg=round(sum(watts) / len(watts), 1),
+                   socket_power_w_median=watts[len(watts) // 2], socket_power_w_max=watts[-1],
+                   source=pfile, xcd_shader_clocks_mhz=clocks,
+                   shader_clock_mhz_avg=round(sum(clocks) / len(clocks), 1) if clocks else None)
+    except Exception as e:
+        out["error"] = (type(e).__name__ + ": " + str(e))[:200]
+    return out
+for line in sys.stdin:
+    parts = line.split()
+    if not parts or parts[0] != "S":
+        break
+    print(json.dumps(sample(float(parts[1]))), flush=True)
+"""
+_sampler_proc = None
+
+
+def start_power_sampler():
+    """Call before the first GPU call of this process."""
+    global _sampler_proc
+    import subprocess
+    try:
+        _sampler_proc = subprocess.Popen([sys.executable, "-c", _SAMPLER], stdin=subprocess.PIPE,
+                                         stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
+    except OSError:
+        _sampler_proc = None
+
+
+def stop_power_sampler():
+    global _sampler_proc
+    if _sampler_proc is not None:
+        try:
+            _sampler_proc.stdin.close()
+            _sampler_proc.wait(timeout=5)
+        except Exception:  # noqa: BLE001
+            _sampler_proc.kill()
+        _sampler_proc = None
+
+
+def sample_power_while(load, seconds=0.6):
+    """Runs load() again and again for `seconds` while the sampler reads the socket power."""
+    if _sampler_proc is None or _sampler_proc.poll() is not None:
+        return {"available": False, "error": "sampler process not running"}
+    try:
+        _sampler_proc.stdin.write(f"S {seconds}\n")
+        _sampler_proc.stdin.flush()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds + 0.02:
+            load()
+        return json.loads(_sampler_proc.stdout.readline())
+    except Exception as e:  # noqa: BLE001
+        return {"available": False, "error": (type(e).__name__ + ": " + str(e))[:200]}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -87,6 +177,9 @@ def main():
         print("bench.py measures one GPU: the quantized operator path is single-device "
               "(no collectives); run it with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.only is None and not args.skip_secondary:
+        start_power_sampler()
 
     import numpy as np
     import torch
@@ -322,6 +415,75 @@ def main():
             log(f"[bench]   {name}: {tops_p:.0f} TOP/s at {ghz_p:.2f} GHz")
         secondary["mfma_i8_ceiling_probe"] = probe
 
+        # ---------------------------------------------- power under the timed load, and a control
+        # The product kernel (torch.ops.quantized.linear, config 3's shape, same settle phase and
+        # timing as the headline) on operands that barely toggle the multipliers: every
+        # activation byte 128 (the kernel feeds x ^ 0x80 = 0) and weights 0..3.  Same
+        # instruction stream, same bytes moved; what differs is the energy of a multiply.  The
+        # socket power is sampled by a child process while each load runs.
+        log("[bench] socket power under config 3, and the same kernel on low-toggle operands")
+
+        def load20():
+            for _ in range(20):
+                step()
+            torch.cuda.synchronize()
+
+        power_c3 = sample_power_while(load20)
+        lt_x, lt_p = [], []
+        for i in range(NSETS):
+            lt_x.append(torch._make_per_tensor_quantized_tensor(
+                torch.full((M, K), 128, dtype=torch.uint8, device=dev), xq.q_scale(), 128))
+            wlt = torch._make_per_channel_quantized_tensor(
+                torch.randint(0, 4, (N, K), dtype=torch.int8, device=dev), w_scales,
+                torch.zeros(N, dtype=torch.int64, device=dev), 0)
+            lt_p.append(torch.ops.quantized.linear_prepack(wlt, bias))
+            del wlt
+        lt_count = [0]
+
+        def lt_step():
+            i = lt_count[0] % NSETS
+            lt_count[0] += 1
+            return torch.ops.quantized.linear(lt_x[i], lt_p[i], out_scale, out_zp)
+
+        def lt_load20():
+            for _ in range(20):
+                lt_step()
+            torch.cuda.synchronize()
+
+        t_ = time.perf_counter()
+        while time.perf_counter() - t_ < 0.2:
+            lt_load20()
+        ea, eb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ea.record()
+        for _ in range(args.steps):
+            lt_step()
+        eb.record()
+        torch.cuda.synchronize()
+        lt_us = ea.elapsed_time(eb) / args.steps * 1e3
+        power_lt = sample_power_while(lt_load20)
+        # back to the benchmark operands for a second reading of the headline in the same state
+        settle()
+        ea.record()
+        for _ in range(args.steps):
+            step()
+        eb.record()
+        torch.cuda.synchronize()
+        again_us = ea.elapsed_time(eb) / args.steps * 1e3
+        lt_tops = ops / lt_us / 1e6
+        log(f"[bench]   low-toggle operands: {lt_us:.1f} us/launch = {lt_tops:.0f} TOP/s ({lt_tops / PEAK_INT8_TOPS:.3f} of "
+            f"peak), benchmark operands again {again_us:.1f} us; socket power {power_c3.get('socket_power_w_avg')} W "
+            f"(benchmark) / {power_lt.get('socket_power_w_avg')} W (low toggle), cap {power_c3.get('power_cap_w')} W")
+        secondary["linear_c3_low_toggle"] = {
+            "avg_launch_us": round(lt_us, 2), "value": round(lt_tops, 1), "unit": "TOP/s",
+            "frac_of_int8_peak": round(lt_tops / PEAK_INT8_TOPS, 4),
+            "benchmark_operands_same_state_us": round(again_us, 2),
+            "speedup_over_benchmark_operands": round(again_us / lt_us, 4),
+            "power": power_lt,
+            "method": "torch.ops.quantized.linear at config 3's shape, x = 128 everywhere (fed to the matrix "
+                      "pipe as 0), weights uniform in 0..3, 4 operand sets rotated; 0.2 s settle, then --steps "
+                      "launches between one pair of events, as the headline"}
+        roofline["socket_power"] = power_c3
+        del lt_x, lt_p
         roofline["power_limited_ceiling_tops"] = probe["gaussian_int8"]["tops"]
         roofline["frac_of_power_limited_ceiling"] = round(achieved / probe["gaussian_int8"]["tops"], 4)
         # the same with operands that change every instruction, as a GEMM's do
@@ -991,6 +1153,7 @@ def main():
         "roofline": roofline, "cpu_baseline": cpu_baseline, "secondary": secondary,
         "device": torch.cuda.get_device_name(0),
     }
+    stop_power_sampler()
     print(json.dumps(out))
 
 

@@ -226,6 +226,34 @@ int64_t tmq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * Pure host arithmetic, no GPU call. */
 int tmq_linear_split_plan(int64_t M, int64_t N, int64_t K, int32_t* splits, int32_t* stages);
 
+/* Which kernel tmq_linear / tmq_linear_f32 / tmq_linear_acc32 launch for a shape,
+ * and on what grid.  Pure host arithmetic, no GPU call: the choice depends on
+ * the sizes, the row pitch, the output kind and whether a workspace is attached,
+ * never on the data.  No counterpart in the reference (muDNN chooses its kernels
+ * out of sight, torch_musa/csrc/aten/quantized/mudnn/Linear.cpp:48-58); it is
+ * here so that the choice and every kernel's preconditions can be swept on the
+ * host over thousands of shapes. */
+typedef struct tmq_linear_choice {
+  int32_t kernel;        /* value that pins this kernel in tmq_linear_desc::kernel (configuration + 1);
+                            0: no kernel takes the shape (TMQ_ERR_UNSUPPORTED from the call) */
+  int32_t tile_rows;     /* activation rows per workgroup tile (0: plain kernel) */
+  int32_t tile_channels; /* output channels per workgroup tile */
+  int32_t waves;         /* wavefronts per workgroup */
+  int32_t splits;        /* runs of k-stages (1: no split along K) */
+  int32_t split_stages;  /* k-stages per run */
+  int64_t tiles;         /* tiles of the product (x splits for split K) */
+  int64_t blocks;        /* workgroups launched (the persistent kernel: fewer than tiles) */
+  int64_t k_stages;      /* 64-byte stages of K */
+} tmq_linear_choice;
+enum tmq_linear_output_kind { TMQ_LINEAR_OUT_BYTES = 0, TMQ_LINEAR_OUT_F32 = 1, TMQ_LINEAR_OUT_ACC32 = 2 };
+/* flags: bits 0-1 a tmq_linear_output_kind; bit 2: a workspace of
+ * tmq_linear_workspace_bytes(M, N, K) is attached; bit 3: K, the row pitch or
+ * the activation pointer is not a multiple of 16 (the plain kernel's case).
+ * forced_kernel: tmq_linear_desc::kernel (0 = automatic).  compute_units: of
+ * the device the product would run on (the persistent kernel's grid follows it). */
+int tmq_linear_kernel_choice(int64_t M, int64_t N, int64_t K, int64_t ldx, int32_t flags, int32_t forced_kernel,
+                             int32_t compute_units, tmq_linear_choice* out);
+
 /* tmq_linear for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference.  Same arguments and the same bytes as
@@ -241,7 +269,9 @@ int tmq_linear_split_plan(int64_t M, int64_t N, int64_t K, int32_t* splits, int3
  * by the caller; calls queued on one stream are safe.  The partial sums are
  * written before they are read, so nothing has to be cleared between calls.
  * The first call on a device looks the array's address up (hipGetSymbolAddress):
- * make one call per device before capturing a graph. */
+ * make one call per device before capturing a graph.  The current device must
+ * be the device that owns `stream` (each GPU holds its own array at its own
+ * address): a stream of another GPU returns TMQ_ERR_INVALID_ARGUMENT. */
 #define TMQ_LINEAR_STATIC_WORKSPACE_BYTES (16 * 1024 * 1024)
 int tmq_linear_static_workspace(const tmq_linear_desc* desc, tmq_stream_t stream);
 

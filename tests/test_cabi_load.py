@@ -51,6 +51,7 @@ def test_struct_sizes_match_the_header():
     import ctypes as C
     assert C.sizeof(cabi.QParams) == 16
     assert C.sizeof(cabi.LinearDesc) == 144
+    assert C.sizeof(cabi.LinearChoice) == 48
     assert C.sizeof(cabi.Conv2dGeom) == 14 * 8
     assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8 + 16
     assert C.sizeof(cabi.Conv2dPost) == 24
@@ -113,6 +114,140 @@ def test_split_k_plan_covers_k():
     assert merged > 0, "no shape exercised the merged tail"
     assert cabi.linear_split_plan(128, 1024, 16640) == (15, 17)    # 260 stages: 14 x 17 + 22
     assert cabi.linear_split_plan(128, 128, 13328) == (12, 17)     # 209 stages: 11 x 17 + 22
+
+
+# ---- the automatic kernel choice of quantized::linear, swept on the host.  Each kernel's
+# preconditions are restated here from the kernels' own index arithmetic and LDS / register
+# budgets (not from the dispatcher's code): a choice outside them is a wrong result or a fault.
+def _ceil(a, b):
+    return -(-a // b)
+
+
+def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256):
+    what = (m, n, k, ldx, out, workspace, misaligned, forced, c)
+    cfg = c["kernel"] - 1
+    kt = _ceil(k, 64)
+    assert c["k_stages"] == kt, what
+    vec_ok = (not misaligned) and k >= 16 and k % 16 == 0 and ldx % 16 == 0
+    if cfg == 9 - 0 and not vec_ok:
+        assert c["tile_rows"] == 0 and c["blocks"] == _ceil(m * _ceil(n, 4), 256), what
+        return
+    # every other kernel loads 16 aligned bytes per lane
+    assert vec_ok or cfg == 9, what
+    if cfg == 9:
+        return
+    bm, bn = c["tile_rows"], c["tile_channels"]
+    tiles = _ceil(m, bm) * _ceil(n, bn)
+    assert c["tiles"] == tiles * c["splits"] and 0 < c["blocks"] <= c["tiles"] < 2 ** 31, what
+    if cfg != 13:
+        assert c["splits"] == 1, what
+    if cfg == 8:                                    # weight streaming: up to four groups of 16 rows
+        assert m <= 64 and bm == 16 * _ceil(m, 16) and bn == 16 and k <= 0x7fffff00 and ldx < 2 ** 31, what
+    elif cfg == 13:                                 # split K: runs of whole stages into a workspace
+        sp, st = c["splits"], c["split_stages"]
+        assert workspace and (bm, bn) == (128, 128) and sp >= 2 and tiles * sp <= 256, what
+        assert (sp - 1) * st < kt and kt - (sp - 1) * st >= 6 and st >= 6, what
+        assert cabi.lib().tmq_linear_workspace_bytes(m, n, k) == sp * m * _ceil(n, 4) * 4 * 4, what
+    elif cfg in (6, 7, 19, 20):                     # direct copies two stages wide: K walked in runs of six stages,
+        assert kt >= 6 and 256 * ldx <= 2 ** 31 and 15 * 16 * _ceil(k, 128) * 128 < 2 ** 32, what   # 32-bit offsets
+        if cfg == 20:                               # persistent: byte / float outputs, several rounds, whole XCD runs
+            assert out != "acc32" and (bm, bn) == (256, 256), what
+            assert forced != 0 or tiles > cus, what
+            # (the tile sequence is a permutation only on a multiple of 8 blocks or with every tile in one round)
+            assert c["blocks"] == (cus // 8 * 8 if tiles > cus else tiles), what
+        else:
+            assert c["blocks"] == tiles, what
+    elif cfg == 17:                                 # direct copies one stage wide: a ring of three stages
+        assert kt >= 3 and 256 * ldx <= 2 ** 31, what
+    elif cfg == 14:                                 # two wave groups halve the k loop
+        assert kt % 2 == 0 and (bm, bn) == (64, 64), what
+        if forced == 0:
+            assert tiles <= 256 and kt >= 32, what
+    elif cfg == 21:                                 # 64 x 64, four phases of 256 bytes of K in LDS: all of K <= 1024
+        assert (bm, bn) == (64, 64) and 64 * ldx <= 2 ** 29, what      # (longer K runs as a ring, for tests)
+        if forced == 0:
+            assert k <= 1024 and tiles <= 256, what
+    elif cfg == 24:                                 # all of K in LDS, 32 x 32, a quarter of K per wave
+        assert k <= 1024 and (bm, bn) == (32, 32) and 64 * ldx <= 2 ** 29, what
+        if forced == 0:
+            assert tiles <= 512 and k > 256, what
+    elif cfg == 25:                                 # weights through registers: 32 fragments per wave at most
+        assert k <= 4096 and (bm, bn) == (32, 32) and 64 * ldx <= 2 ** 29, what
+        if forced == 0:                             # one round: two blocks per CU while 32 x K <= 64 KB
+            assert k > 1024 and tiles <= (512 if k <= 2048 else 256), what
+    elif cfg == 26:
+        assert k <= 4096 and (bm, bn) == (32, 64) and c["waves"] == 8 and 64 * ldx <= 2 ** 29, what
+        if forced == 0:
+            assert k > 2048 and tiles <= 256, what
+    else:                                           # register-staged tiles take any aligned shape
+        assert cfg in (0, 1, 2, 3, 4, 5, 22, 23), what
+    if forced == 0 and cfg in (22, 23):             # a few hundred rows: one round of oblong tiles
+        assert tiles <= 256, what
+
+
+def _random_linear_shapes(rng, count):
+    for _ in range(count):
+        m = int(2 ** rng.uniform(0, 13.2))
+        n = int(2 ** rng.uniform(0, 15.7))
+        k = 16 * int(2 ** rng.uniform(0, 11.2))
+        if rng.random() < 0.1:
+            k += int(rng.integers(1, 16))           # not a multiple of 16: the plain kernel's
+        if rng.random() < 0.25:                     # the sizes the thresholds were fitted at
+            m = int(rng.choice([1, 16, 17, 24, 25, 32, 64, 65, 96, 128, 200, 256, 448, 512, 1024, 2048, 4096]))
+            n = int(rng.choice([1024, 2048, 4096, 8192, 11008, 12288, 32000]))
+            k = int(rng.choice([256, 272, 512, 1024, 1040, 2048, 2064, 3072, 4096, 4112, 8192, 11008]))
+        ldx = k + (16 * int(rng.integers(0, 9)) if rng.random() < 0.2 else 0)
+        if rng.random() < 0.02:
+            ldx = k + int(rng.integers(1, 16))      # a pitch that breaks the alignment
+        yield m, n, k, ldx
+
+
+def test_automatic_kernel_choice_keeps_every_kernels_preconditions():
+    rng = np.random.default_rng(20)
+    seen = set()
+    for m, n, k, ldx in _random_linear_shapes(rng, 6000):
+        for out in ("bytes", "f32", "acc32"):
+            for workspace in (False, True):
+                c = cabi.linear_kernel_choice(m, n, k, ldx, out, workspace)
+                assert c["kernel"] != 0, (m, n, k, ldx, out, workspace)      # the automatic choice always runs
+                _check_choice(c, m, n, k, ldx, out, workspace, False)
+                seen.add(c["kernel"] - 1)
+    # huge pitches and K: the 32-bit offset limits of the direct-copy kernels
+    for m, n, k, ldx in ((4096, 11008, 4096, 2 ** 23 + 16), (4096, 11008, 2 ** 23 + 64, 2 ** 23 + 64),
+                         (512, 4096, 4096, 2 ** 24), (128, 1024, 1024, 2 ** 23 + 16), (64, 4096, 4096, 2 ** 23 + 16)):
+        for out in ("bytes", "acc32"):
+            c = cabi.linear_kernel_choice(m, n, k, ldx, out)
+            assert c["kernel"] != 0
+            _check_choice(c, m, n, k, ldx, out, False, False)
+            seen.add(c["kernel"] - 1)
+    c = cabi.linear_kernel_choice(300, 500, 4096, misaligned=True)
+    assert c["kernel"] == 10
+    assert seen >= {2, 3, 6, 7, 8, 9, 13, 14, 17, 19, 20, 21, 23, 24, 25, 26}, sorted(seen)
+    # the benchmark configurations
+    assert cabi.linear_kernel_choice(4096, 11008, 4096)["kernel"] - 1 == 20
+    assert cabi.linear_kernel_choice(4096, 11008, 4096)["blocks"] == 256
+    assert cabi.linear_kernel_choice(4096, 11008, 4096, compute_units=252)["blocks"] == 248
+    assert cabi.linear_kernel_choice(128, 1024, 1024)["kernel"] - 1 == 24
+    for m in (1, 4, 16):
+        assert cabi.linear_kernel_choice(m, 4096, 4096)["kernel"] - 1 == 8
+    assert cabi.linear_kernel_choice(0, 4096, 4096) == dict(kernel=0, tile_rows=0, tile_channels=0, waves=0, splits=1,
+                                                           split_stages=0, tiles=0, blocks=0, k_stages=64)
+
+
+def test_forced_kernels_run_inside_their_preconditions_or_not_at_all():
+    rng = np.random.default_rng(21)
+    refused = 0
+    for m, n, k, ldx in _random_linear_shapes(rng, 1500):
+        for cfg in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26):
+            for out in ("bytes", "acc32"):
+                c = cabi.linear_kernel_choice(m, n, k, ldx, out, workspace=True, forced=cfg + 1)
+                if c["kernel"] == 0:
+                    refused += 1
+                    continue
+                _check_choice(c, m, n, k, ldx, out, True, False, forced=cfg + 1)
+    assert refused > 0
+    with pytest.raises(cabi.TmqError):
+        cabi.linear_kernel_choice(8, 8, 64, ldx=32)
 
 
 def test_host_choose_qparams_matches_oracle(golden):

@@ -695,6 +695,102 @@ def test_plain_ops_keep_their_packed_weight():
     assert tm.plain_weight_cache_counters()[2] == 0
 
 
+def test_plain_weight_cache_across_streams_and_graph_capture():
+    """A miss packs on the caller's stream; a hit from another stream must wait for that packing.
+    A capture takes an entry whose packing has finished and records no wait for it."""
+    import torch_musa_amd as tm
+    say("aten plain-op weight cache: streams and capture")
+    tm.plain_weight_cache_clear()
+    g = torch.Generator().manual_seed(11)
+    M, K, N = 64, 4096, 4096            # a packing long enough to be in flight when the hit arrives
+    x = torch.randint(0, 255, (M, K), dtype=torch.uint8, generator=g).cuda()
+    wz = torch.zeros(N, dtype=torch.int).cuda()
+    ws = (torch.rand(N, generator=g) * 0.002 + 0.001).cuda()
+    call = lambda w_: torch.ops.quantized.linear_per_tensor(x, 0.02, 120, w_, ws, wz, None, 0.6, 100, torch.uint8,
+                                                             "none", [], "")
+
+    def want(w_):
+        return oracle.plain_linear(x.cpu().numpy(), 0.02, 120, w_.cpu().numpy(), ws.cpu().numpy(), None, 0.6, 100,
+                                   "uint8", "none")
+
+    side = torch.cuda.Stream()
+    for rep in range(3):
+        w = torch.randint(-127, 127, (K, N), dtype=torch.int8, generator=g).cuda()
+        torch.cuda.synchronize()
+        before = tm.plain_weight_cache_stats()
+        with torch.cuda.stream(side):
+            # a long queue in front of the packing, so that the default stream's hit arrives first
+            filler = torch.empty(1 << 26, device="cuda")
+            for _ in range(4):
+                filler.normal_()
+            y_side = call(w)            # miss: packs on `side`
+        y_main = call(w)                # hit from the default stream, packing possibly still queued
+        torch.cuda.synchronize()
+        after = tm.plain_weight_cache_stats()
+        assert after["misses"] - before["misses"] == 1 and after["hits"] - before["hits"] == 1
+        assert after["cross_stream_hits"] - before["cross_stream_hits"] == 1
+        ref = want(w)
+        _close_to(y_main.cpu().numpy(), ref, "uint8", f"hit on the default stream, round {rep}")
+        _close_to(y_side.cpu().numpy(), ref, "uint8", f"miss on the side stream, round {rep}")
+        assert torch.equal(y_main, y_side)
+        del filler
+    # capture: a weight packed by an eager call beforehand (a miss inside a capture is refused
+    # with an error: the zero-point check alone needs the host)
+    w2 = torch.randint(-127, 127, (K, N), dtype=torch.int8, generator=g).cuda()
+    ref2 = want(w2)
+    y_eager = call(w2)
+    torch.cuda.synchronize()
+    _close_to(y_eager.cpu().numpy(), ref2, "uint8", "eager call before the capture")
+    # a capture that finds a finished entry uses it (no packing kernels in the graph)
+    graph2 = torch.cuda.CUDAGraph()
+    h0 = tm.plain_weight_cache_stats()["hits"]
+    with torch.cuda.stream(side):
+        side.synchronize()
+        with torch.cuda.graph(graph2, stream=side):
+            y_cap2 = call(w2)
+    torch.cuda.synchronize()
+    assert tm.plain_weight_cache_stats()["hits"] == h0 + 1
+    assert tm.plain_weight_cache_stats()["cross_stream_hits"] == after["cross_stream_hits"]   # no wait recorded
+    for _ in range(2):
+        y_cap2.zero_()
+        torch.cuda.synchronize()
+        graph2.replay()
+        torch.cuda.synchronize()
+        _close_to(y_cap2.cpu().numpy(), ref2, "uint8", "graph that hit the cache")
+    tm.plain_weight_cache_clear()
+
+
+def test_plain_weight_cache_holds_more_than_64_weights_and_respects_its_byte_limit():
+    import torch_musa_amd as tm
+    say("aten plain-op weight cache: 65 weights in rotation, byte limit")
+    tm.plain_weight_cache_clear()
+    g = torch.Generator().manual_seed(12)
+    x = torch.randint(0, 255, (8, 64), dtype=torch.uint8, generator=g).cuda()
+    wz, ws = torch.zeros(32, dtype=torch.int).cuda(), torch.full((32,), 0.01).cuda()
+    weights = [torch.randint(-127, 127, (64, 32), dtype=torch.int8, generator=g).cuda() for _ in range(65)]
+    call = lambda w_: torch.ops.quantized.linear_per_tensor(x, 0.02, 120, w_, ws, wz, None, 0.3, 100, torch.uint8,
+                                                             "none", [], "")
+    first = [call(w_) for w_ in weights]
+    s1 = tm.plain_weight_cache_stats()
+    second = [call(w_) for w_ in weights]          # a model's second pass: every layer hits
+    s2 = tm.plain_weight_cache_stats()
+    assert s2["hits"] - s1["hits"] == 65 and s2["misses"] == s1["misses"] and s2["entries"] >= 65
+    assert all(torch.equal(a, b) for a, b in zip(first, second))
+    per_entry = s2["bytes"] // s2["entries"]
+    default_limit = s2["max_bytes"]
+    try:
+        tm.plain_weight_cache_set_max_bytes(10 * per_entry)      # room for ten: the rest leaves, oldest first
+        s3 = tm.plain_weight_cache_stats()
+        assert s3["entries"] == 10 and s3["bytes"] <= 10 * per_entry and s3["evictions"] - s2["evictions"] == 55
+        third = [call(w_) for w_ in weights]       # rotation over more than the limit holds: misses, same bytes
+        s4 = tm.plain_weight_cache_stats()
+        assert s4["entries"] == 10 and s4["misses"] - s3["misses"] == 65
+        assert all(torch.equal(a, b) for a, b in zip(first, third))
+    finally:
+        tm.plain_weight_cache_set_max_bytes(default_limit)
+        tm.plain_weight_cache_clear()
+
+
 def test_quantized_modules_to_device():
     # a populated CPU model (conv -> relu -> pool -> flatten -> linear, dynamic linear beside
     # it) moved to the GPU with its packed parameters; same bytes out as on the CPU

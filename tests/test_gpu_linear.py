@@ -114,9 +114,9 @@ def test_persistent_kernel_one_and_several_tiles_per_block(cabi, shape, kw):
     say("persistent kernel", shape)
     c = _tile_case(*shape, seed=77 + shape[0] % 7, **kw)
     y, acc, _ = _run(cabi, c, 20)
-    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"]))
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
     want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
-                         c["out_scale"], c["out_zp"], relu=c["relu"])
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
     _check(y, want, "cfg 20")
 
 
@@ -375,7 +375,7 @@ def test_c1_golden(cabi, golden):
 
 def test_c3_full_size(cabi):
     """benchmark configuration 3 (M=4096, K=4096, N=11008): oracle parity on sampled
-    rows, and the all-ones identity acc[m][n] = colsum[n] on the whole output."""
+    rows, integer identities on the whole output, and every output byte against the live CPU operator."""
     M, K, N = 4096, 4096, 11008
     say("C3 full size")
     rng = np.random.default_rng(3)
@@ -406,6 +406,18 @@ def test_c3_full_size(cabi):
     # the GEMM is linear in x: acc(x) + acc(255 - x) = 255 * colsum
     acc2 = cabi.linear_acc32(255 - xq, pw)
     assert torch.equal(acc + acc2, 255 * pw.colsum[None, :].expand(M, N))
+    del acc, acc1, acc2, ones
+    # all 45 M requantised bytes against the live CPU operator on the same codes (the way the
+    # reference's harness compares device and CPU results, torch_musa/testing/base_test_tool.py:814-825)
+    torch.backends.quantized.engine = "fbgemm"
+    x_cpu = torch._make_per_tensor_quantized_tensor(xq.cpu(), s, z)
+    w_cpu = torch._make_per_channel_quantized_tensor(wq.cpu(), torch.from_numpy(ws), torch.zeros(N, dtype=torch.int64), 0)
+    p_cpu = torch.ops.quantized.linear_prepack(w_cpu, torch.from_numpy(bias))
+    y_cpu = torch.ops.quantized.linear(x_cpu, p_cpu, out_scale, out_zp).int_repr()
+    y_gpu = y.cpu()
+    differ = int((y_cpu != y_gpu).sum())
+    assert differ == 0, f"{differ} of {M * N} bytes differ from the CPU operator's (max " \
+                        f"{int((y_cpu.int() - y_gpu.int()).abs().max())} LSB)"
 
 
 # ---- split K (a few hundred rows, long K: partial sums in a caller-owned workspace) --------

@@ -33,8 +33,11 @@ def _both(cabi, c, allocations_allowed=True):
     out = torch.empty_like(want)
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    free_before, _ = torch.cuda.mem_get_info()       # the driver's own count: sees a hipMalloc inside the library too
     got = cabi.linear_static_workspace(*args, out_signed=signed, relu=c["relu"], out=out)
+    torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before, "the call allocated through torch"
+    assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
     return host(got), host(want)
 
 

@@ -28,7 +28,8 @@ LIB_KERNELS = os.path.join(_PKG, "libtmq.so")
 LIB_ATEN = os.path.join(_PKG, "libtmq_aten.so")
 
 __all__ = ["LIB_KERNELS", "LIB_ATEN", "is_loaded", "load", "quantized_device", "quantized_modules_to",
-           "plain_weight_cache_clear", "plain_weight_cache_counters"]
+           "plain_weight_cache_clear", "plain_weight_cache_counters", "plain_weight_cache_stats",
+           "plain_weight_cache_set_max_bytes"]
 
 _loaded = False
 
@@ -63,13 +64,15 @@ def _aten_lib():
     load()
     lib = ctypes.CDLL(LIB_ATEN)  # already loaded by torch.ops.load_library: the same handle
     lib.tmq_aten_plain_weight_cache_counters.argtypes = [ctypes.POINTER(ctypes.c_int64)] * 3
+    lib.tmq_aten_plain_weight_cache_stats.argtypes = [ctypes.POINTER(ctypes.c_int64), ctypes.c_int]
+    lib.tmq_aten_plain_weight_cache_set_max_bytes.argtypes = [ctypes.c_int64]
     return lib
 
 
 def plain_weight_cache_clear() -> None:
     """Drop the packed weights kept for ``quantized::linear_per_tensor`` / ``conv`` / ``conv_binary``
     (their schemas pass the int8 weight as a plain tensor on every call; the re-tiled copy is kept
-    per weight tensor, at most 64 of them)."""
+    per weight tensor, least recently used entries leaving once the byte limit is exceeded)."""
     _aten_lib().tmq_aten_plain_weight_cache_clear()
 
 
@@ -80,6 +83,23 @@ def plain_weight_cache_counters():
     h, m, e = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
     _aten_lib().tmq_aten_plain_weight_cache_counters(ctypes.byref(h), ctypes.byref(m), ctypes.byref(e))
     return h.value, m.value, e.value
+
+
+def plain_weight_cache_stats() -> dict:
+    """Counters of that cache: hits, misses, entries, bytes held, byte limit, evictions, and hits
+    from a stream other than the one that packed the entry (those wait for the packing's event)."""
+    import ctypes
+
+    v = (ctypes.c_int64 * 7)()
+    _aten_lib().tmq_aten_plain_weight_cache_stats(v, 7)
+    names = ("hits", "misses", "entries", "bytes", "max_bytes", "evictions", "cross_stream_hits")
+    return dict(zip(names, (int(x) for x in v)))
+
+
+def plain_weight_cache_set_max_bytes(nbytes: int) -> None:
+    """Byte limit of that cache (default 16 GiB, or ``TMQ_PLAIN_WEIGHT_CACHE_MB`` in the environment).
+    A model whose plain-tensor weights exceed it re-packs the evicted ones on every pass."""
+    _aten_lib().tmq_aten_plain_weight_cache_set_max_bytes(int(nbytes))
 
 
 def quantized_device() -> torch.device:

@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_static_workspace", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_kernel_choice", "tmq_linear_static_workspace", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
@@ -52,6 +52,12 @@ class LinearDesc(C.Structure):
         ("y", C.c_void_p), ("ldy", C.c_int64),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
     ]
+
+
+class LinearChoice(C.Structure):
+    _fields_ = [("kernel", C.c_int32), ("tile_rows", C.c_int32), ("tile_channels", C.c_int32), ("waves", C.c_int32),
+                ("splits", C.c_int32), ("split_stages", C.c_int32), ("tiles", C.c_int64), ("blocks", C.c_int64),
+                ("k_stages", C.c_int64)]
 
 
 class Conv2dGeom(C.Structure):
@@ -105,6 +111,8 @@ def lib() -> C.CDLL:
         l.tmq_linear_workspace_bytes.argtypes = [C.c_int64, C.c_int64, C.c_int64]
         l.tmq_linear_split_plan.argtypes = [C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_int32),
                                             C.POINTER(C.c_int32)]
+        l.tmq_linear_kernel_choice.argtypes = [C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32,
+                                               C.c_int32, C.POINTER(LinearChoice)]
         l.tmq_conv2d_packed_bytes.restype = C.c_int64
         l.tmq_conv2d_packed_bytes.argtypes = [C.POINTER(Conv2dGeom)]
         v = C.c_void_p
@@ -469,6 +477,20 @@ def linear_split_plan(m: int, n: int, k: int):
     sp, st = C.c_int32(), C.c_int32()
     check(lib().tmq_linear_split_plan(m, n, k, C.byref(sp), C.byref(st)), "tmq_linear_split_plan")
     return sp.value, st.value
+
+
+LINEAR_OUT_KINDS = {"bytes": 0, "f32": 1, "acc32": 2}
+
+
+def linear_kernel_choice(m: int, n: int, k: int, ldx: int = None, out: str = "bytes", workspace: bool = False,
+                         misaligned: bool = False, forced: int = 0, compute_units: int = 256) -> dict:
+    """Which kernel the library launches for this shape (host arithmetic only): a dict of
+    include/tmq.h's tmq_linear_choice fields; kernel == 0 says that no kernel takes it."""
+    c = LinearChoice()
+    flags = LINEAR_OUT_KINDS[out] | (4 if workspace else 0) | (8 if misaligned else 0)
+    check(lib().tmq_linear_kernel_choice(m, n, k, k if ldx is None else ldx, flags, forced, compute_units,
+                                         C.byref(c)), "tmq_linear_kernel_choice")
+    return {f: getattr(c, f) for f, _ in LinearChoice._fields_}
 
 
 # ---------------------------------------------------------------------------

@@ -22,12 +22,14 @@
 #include <ATen/native/quantized/AffineQuantizer.h>
 #include <ATen/native/quantized/PackedParams.h>
 #include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPCachingAllocator.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
 
 #include <array>
 #include <cstdlib>
 #include <list>
+#include <memory>
 #include <mutex>
 #include <tuple>
 #include <vector>
@@ -1050,7 +1052,7 @@ at::Tensor plain_requant(const at::Tensor& r, double scale, int64_t zp, const Pl
 // ---------------------------------------------------------------------------
 // Packed weights of the plain-tensor ops.  Their schemas carry the int8 weight as
 // an ordinary tensor on every call, so the re-tiled copy, its column sums and the
-// fp32 scales are kept from one call to the next: a small most-recently-used
+// fp32 scales are kept from one call to the next: a most-recently-used
 // list keyed on the identity of the weight, scale and zero-point tensors
 // (storage, address, version counter, shape, strides) and on the geometry the
 // packing depends on.  An in-place change of any of the three bumps its version
@@ -1088,11 +1090,49 @@ struct TensorIdentity {
   bool alive() const { return !defined || !storage->expired(); }
 };
 
+// Streams.  The packing kernels of a miss run on the caller's current stream; the entry
+// keeps an event recorded behind them.  A hit from the same stream is ordered by the
+// stream; a hit from another stream (or another host thread's stream) makes that stream
+// wait for the event and tells the caching allocator that the buffers are in use there.
+// While the current stream is being captured into a graph nothing is inserted (the
+// packing would only be recorded, not run) and only entries whose packing has already
+// finished are handed out (waiting for an event of eager work cannot be recorded); a
+// capture that misses is refused with an error -- the packing's zero-point check needs
+// the host -- so a graph is warmed up with one eager call per weight first.
+struct ReadyEvent {  // one HIP event without timing, destroyed with its last holder
+  hipEvent_t ev = nullptr;
+  ReadyEvent() { TORCH_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess, "hipEventCreate failed"); }
+  ~ReadyEvent() {
+    if (ev != nullptr) (void)hipEventDestroy(ev);
+  }
+  ReadyEvent(const ReadyEvent&) = delete;
+  ReadyEvent& operator=(const ReadyEvent&) = delete;
+  void record(hipStream_t s) { TORCH_CHECK(hipEventRecord(ev, s) == hipSuccess, "hipEventRecord failed"); }
+  void block(hipStream_t s) { TORCH_CHECK(hipStreamWaitEvent(s, ev, 0) == hipSuccess, "hipStreamWaitEvent failed"); }
+  bool query() {
+    const hipError_t e = hipEventQuery(ev);
+    if (e != hipSuccess) (void)hipGetLastError();  // hipErrorNotReady is an answer, not a failure
+    return e == hipSuccess;
+  }
+};
+
 struct PlainWeightEntry {
   TensorIdentity weight, scales, zero_points;
   std::array<int64_t, 8> geometry;  // what the packing depends on besides the weight (conv: taps, groups, ...)
   at::Tensor packed, colsum, scales_f32;
+  std::shared_ptr<ReadyEvent> ready;  // behind the packing kernels on `stream`
+  c10::hip::HIPStream stream;
+  int64_t bytes = 0;
 };
+
+bool stream_is_capturing(const c10::hip::HIPStream& s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s.stream(), &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // unknown: take the safe side
+  }
+  return st != hipStreamCaptureStatusNone;
+}
 
 class PlainWeightCache {
  public:
@@ -1101,11 +1141,20 @@ class PlainWeightCache {
     return c;
   }
   bool enabled() const { return enabled_; }
+  // `on`: the stream the caller is about to launch on.
   bool find(const at::Tensor& w, const at::Tensor& sc, const at::Tensor& zp, const std::array<int64_t, 8>& geom,
-            at::Tensor* packed, at::Tensor* colsum, at::Tensor* scales_f32) {
+            const c10::hip::HIPStream& on, at::Tensor* packed, at::Tensor* colsum, at::Tensor* scales_f32) {
+    const bool capturing = stream_is_capturing(on);
     std::lock_guard<std::mutex> lock(mu_);
     for (auto it = entries_.begin(); it != entries_.end(); ++it) {
       if (it->geometry == geom && it->weight.matches(w) && it->scales.matches(sc) && it->zero_points.matches(zp)) {
+        if (capturing && !it->ready->query()) break;  // packing still in flight: not usable inside a capture
+        if (!capturing && it->stream != on) {
+          it->ready->block(on.stream());
+          for (const at::Tensor* t : {&it->packed, &it->colsum, &it->scales_f32})
+            c10::hip::HIPCachingAllocator::recordStream(t->storage().data_ptr(), on);
+          ++cross_stream_hits_;
+        }
         entries_.splice(entries_.begin(), entries_, it);  // most recently used first
         *packed = it->packed;
         *colsum = it->colsum;
@@ -1117,38 +1166,74 @@ class PlainWeightCache {
     ++misses_;
     return false;
   }
+  // Call after the packing kernels were queued on `on`.
   void insert(const at::Tensor& w, const at::Tensor& sc, const at::Tensor& zp, const std::array<int64_t, 8>& geom,
-              const at::Tensor& packed, const at::Tensor& colsum, const at::Tensor& scales_f32) {
+              const c10::hip::HIPStream& on, const at::Tensor& packed, const at::Tensor& colsum,
+              const at::Tensor& scales_f32) {
+    if (stream_is_capturing(on)) return;
+    auto ready = std::make_shared<ReadyEvent>();
+    ready->record(on.stream());
+    const int64_t bytes = static_cast<int64_t>(packed.nbytes() + colsum.nbytes() + scales_f32.nbytes());
     std::lock_guard<std::mutex> lock(mu_);
-    entries_.remove_if([](const PlainWeightEntry& e) {
-      return !(e.weight.alive() && e.scales.alive() && e.zero_points.alive());
+    entries_.remove_if([this](const PlainWeightEntry& e) {
+      const bool dead = !(e.weight.alive() && e.scales.alive() && e.zero_points.alive());
+      if (dead) bytes_ -= e.bytes;
+      return dead;
     });
+    if (bytes > max_bytes_) return;  // larger than the whole budget: never kept
     entries_.push_front(PlainWeightEntry{TensorIdentity(w), TensorIdentity(sc), TensorIdentity(zp), geom, packed,
-                                         colsum, scales_f32});
-    while (entries_.size() > kMaxEntries) entries_.pop_back();
+                                         colsum, scales_f32, std::move(ready), on, bytes});
+    bytes_ += bytes;
+    while (bytes_ > max_bytes_ || entries_.size() > kMaxEntries) {
+      bytes_ -= entries_.back().bytes;
+      entries_.pop_back();
+      ++evictions_;
+    }
   }
   void clear() {
     std::lock_guard<std::mutex> lock(mu_);
     entries_.clear();
+    bytes_ = 0;
   }
-  void counters(int64_t* hits, int64_t* misses, int64_t* entries) {
+  void set_max_bytes(int64_t b) {
     std::lock_guard<std::mutex> lock(mu_);
-    *hits = hits_;
-    *misses = misses_;
-    *entries = static_cast<int64_t>(entries_.size());
+    max_bytes_ = b < 0 ? 0 : b;
+    while (bytes_ > max_bytes_ && !entries_.empty()) {
+      bytes_ -= entries_.back().bytes;
+      entries_.pop_back();
+      ++evictions_;
+    }
+  }
+  void counters(int64_t* out, int n) {
+    std::lock_guard<std::mutex> lock(mu_);
+    const int64_t v[7] = {hits_, misses_, static_cast<int64_t>(entries_.size()), bytes_, max_bytes_, evictions_,
+                          cross_stream_hits_};
+    for (int i = 0; i < n && i < 7; ++i) out[i] = v[i];
   }
 
  private:
   PlainWeightCache() {
     const char* e = std::getenv("TMQ_PLAIN_WEIGHT_CACHE");
     enabled_ = !(e != nullptr && e[0] == '0');
+    if (const char* mb = std::getenv("TMQ_PLAIN_WEIGHT_CACHE_MB")) {
+      char* end = nullptr;
+      const long long v = std::strtoll(mb, &end, 10);
+      if (end != mb && v >= 0) max_bytes_ = static_cast<int64_t>(v) << 20;
+    }
   }
-  static constexpr size_t kMaxEntries = 64;
+  // Bounded by bytes (packed copies are the size of the weights: a 7 B-parameter model's
+  // linear layers are about 7 GB), with a cap on the entry count that keeps a lookup short.
+  static constexpr size_t kMaxEntries = 4096;
   std::mutex mu_;
   std::list<PlainWeightEntry> entries_;
-  int64_t hits_ = 0, misses_ = 0;
+  int64_t bytes_ = 0, max_bytes_ = int64_t{16} << 30;
+  int64_t hits_ = 0, misses_ = 0, evictions_ = 0, cross_stream_hits_ = 0;
   bool enabled_ = true;
 };
+
+constexpr const char* kPackBeforeCapture =
+    ": this weight has not been packed yet (or its packing is still in flight) and the current stream is being "
+    "captured into a graph; call the operator once on these weight tensors outside the capture first";
 
 bool plain_cacheable(const at::Tensor& w, const at::Tensor& sc, const at::Tensor& zp) {
   return PlainWeightCache::get().enabled() && TensorIdentity::cacheable(w) && TensorIdentity::cacheable(sc) &&
@@ -1188,7 +1273,10 @@ at::Tensor qlinear_per_tensor_run(at::Tensor act, double act_scale, int64_t act_
   at::Tensor packed, colsum, ws;
   const std::array<int64_t, 8> geom{0, N, K, act.device().index(), 0, 0, 0, 0};
   const bool cacheable = plain_cacheable(weight, weight_scales, weight_zero_points);
-  if (!cacheable || !PlainWeightCache::get().find(weight, weight_scales, weight_zero_points, geom, &packed, &colsum, &ws)) {
+  const auto hstream = c10::hip::getCurrentHIPStream(act.device().index());
+  if (!cacheable ||
+      !PlainWeightCache::get().find(weight, weight_scales, weight_zero_points, geom, hstream, &packed, &colsum, &ws)) {
+    TORCH_CHECK(!stream_is_capturing(hstream), what, kPackBeforeCapture);
     ws = plain_weight_scales(weight_scales, weight_zero_points, N, act, what);
     packed = at::empty({std::max<int64_t>(tmq_linear_packed_bytes(N, K), 16)}, act.options().dtype(at::kByte));
     colsum = at::empty({N}, act.options().dtype(at::kInt));
@@ -1196,7 +1284,7 @@ at::Tensor qlinear_per_tensor_run(at::Tensor act, double act_scale, int64_t act_
     check_status(tmq_linear_prepack(cptr<int8_t>(w_nk), N, K, K, packed.data_ptr(), mptr<int32_t>(colsum), stream),
                  "tmq_linear_prepack");
     if (cacheable)
-      PlainWeightCache::get().insert(weight, weight_scales, weight_zero_points, geom, packed, colsum, ws);
+      PlainWeightCache::get().insert(weight, weight_scales, weight_zero_points, geom, hstream, packed, colsum, ws);
   }
   tmq_linear_desc d{};
   d.M = M;
@@ -1278,7 +1366,10 @@ at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero
   at::Tensor packed, colsum, ws;
   const std::array<int64_t, 8> geom{1, g.OC, g.IC, g.KH, g.KW, g.groups, act.device().index(), 0};
   const bool cacheable = g.B > 0 && plain_cacheable(weight, weight_scales, weight_zero_points);
-  if (!cacheable || !PlainWeightCache::get().find(weight, weight_scales, weight_zero_points, geom, &packed, &colsum, &ws)) {
+  const auto hstream = c10::hip::getCurrentHIPStream(act.device().index());
+  if (!cacheable ||
+      !PlainWeightCache::get().find(weight, weight_scales, weight_zero_points, geom, hstream, &packed, &colsum, &ws)) {
+    TORCH_CHECK(!stream_is_capturing(hstream), what, kPackBeforeCapture);
     ws = plain_weight_scales(weight_scales, weight_zero_points, g.OC, act, what);
     const at::Tensor w_ohwi = weight.permute({0, 2, 3, 1}).contiguous();
     packed = at::empty({std::max<int64_t>(tmq_conv2d_packed_bytes(&g), 16)}, act.options().dtype(at::kByte));
@@ -1287,7 +1378,7 @@ at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero
       check_status(tmq_conv2d_prepack(cptr<int8_t>(w_ohwi), &g, packed.data_ptr(), mptr<int32_t>(colsum), stream),
                    "tmq_conv2d_prepack");
     if (cacheable)
-      PlainWeightCache::get().insert(weight, weight_scales, weight_zero_points, geom, packed, colsum, ws);
+      PlainWeightCache::get().insert(weight, weight_scales, weight_zero_points, geom, hstream, packed, colsum, ws);
   }
   d.x = x.data_ptr();
   d.x_signed = x_signed;
@@ -1481,5 +1572,19 @@ extern "C" __attribute__((visibility("default"))) void tmq_aten_plain_weight_cac
 extern "C" __attribute__((visibility("default"))) void tmq_aten_plain_weight_cache_counters(int64_t* hits,
                                                                                              int64_t* misses,
                                                                                              int64_t* entries) {
-  PlainWeightCache::get().counters(hits, misses, entries);
+  int64_t v[3] = {0, 0, 0};
+  PlainWeightCache::get().counters(v, 3);
+  *hits = v[0];
+  *misses = v[1];
+  *entries = v[2];
+}
+// out[0..n): hits, misses, entries, bytes held, byte limit, evictions, hits from a stream
+// other than the one that packed the entry.
+extern "C" __attribute__((visibility("default"))) void tmq_aten_plain_weight_cache_stats(int64_t* out, int n) {
+  PlainWeightCache::get().counters(out, n);
+}
+// The byte limit (default 16 GiB, or TMQ_PLAIN_WEIGHT_CACHE_MB in the environment);
+// entries beyond it leave, least recently used first.
+extern "C" __attribute__((visibility("default"))) void tmq_aten_plain_weight_cache_set_max_bytes(int64_t bytes) {
+  PlainWeightCache::get().set_max_bytes(bytes);
 }

@@ -819,83 +819,92 @@ int run_split(const GemmArgs& a, const XLinear& xs, const SplitPlan& p, void* wo
   return launch_status();
 }
 
+// ---- which kernel runs a product: a host-side function of the shape alone, so that
+// it can be queried (tmq_linear_kernel_choice) and swept without a device.
+struct LinearQuery {
+  int64_t M, N, K, ldx;
+  int64_t n_off = 0;
+  int mode = kOutU8;             // EpilogueMode
+  bool vec_ok = true;            // K, the row pitch and the activation pointer are multiples of 16
+  bool workspace_attached = false;
+  int64_t workspace_bytes = 0;   // usable (16-byte aligned) split-K scratch
+};
+// cfg: tmq_linear_desc::kernel - 1.  0-7, 14, 17, 19, 22, 23: tiles of gemm_i8_kernel; 8: weight
+// streaming; 9: plain kernel; 13: split K (plan in `split`); 20: persistent 256 x 256 tiles;
+// 21 / 24: all of K in LDS (64 x 64 / 32 x 32 tiles); 25 / 26: weights through registers
+// (32 x 32 / 32 x 64 tiles); kNoKernel: the forced kernel does not take this shape.
+constexpr int kNoKernel = -2;
+struct LinearChoice {
+  int cfg = kNoKernel;
+  SplitPlan split;
+};
+
+// Limits of the kernels' own index arithmetic, shared by the choice and the launches.
+// Direct-copy kernels: 256 rows of either operand addressed with 32-bit offsets, and
+// their three-stage ring runs at least once around.
+bool dma_limits_ok(int64_t K, int64_t ldx) { return ldx <= (int64_t{1} << 23) && K <= (int64_t{1} << 23) && K > 2 * kBK; }
+// The copies two stages wide walk K in runs of six stages.
+bool wide_limits_ok(int64_t K, int64_t ldx) { return dma_limits_ok(K, ldx) && K > 5 * kBK; }
+// All of K in LDS / weights through registers: 32-bit offsets over 64 rows of either
+// operand, N * 4 as a 32-bit offset.
+bool onepass_limits_ok(const LinearQuery& q) {
+  return q.K % 16 == 0 && q.K <= (int64_t{1} << 23) && q.ldx <= (int64_t{1} << 23) && q.N + q.n_off < (int64_t{1} << 29);
+}
+// The weight-streaming kernel takes K, the row pitch and N as 32-bit arguments.
+bool stream_limits_ok(const LinearQuery& q) {
+  return q.M <= kDecodeMaxRows && ceil_div(q.N, 16) <= 0x7fffffff && q.K <= 0x7fffff00 && q.ldx <= 0x7fffffff &&
+         q.N <= 0x7ffffff0;
+}
+
 // forced: tmq_linear_desc::kernel - 1 (-1 = automatic choice).
-template <int MODE>
-int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec_ok, int forced,
-                    hipStream_t s, void* workspace = nullptr, int64_t workspace_bytes = 0) {
-  if (!vec_ok || forced == 9) {
-    // plain kernel accumulates true activation values: undo the +128 share
-    GemmArgs b = a;
-    if (!x_signed) {
-      b.acc_coef -= 128;
-      b.acc_base -= 128;
-    }
-    const int64_t work = a.M * ceil_div(a.N, 4);
-    const int64_t blocks = ceil_div(work, 256);
-    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-    linear_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(b, xs, x_signed);
-    return launch_status();
+LinearChoice choose_linear(const LinearQuery& q, int forced) {
+  LinearChoice c;
+  if (!q.vec_ok || forced == 9) {
+    c.cfg = 9;
+    return c;
   }
   const bool stream_auto =
-      forced < 0 && (a.M <= kDecodeRowsAuto ||
-                     (a.M <= kDecodeMaxRows &&
-                      small_rows_path(a.M, a.N, a.K, workspace != nullptr && a.K % 16 == 0) == SmallRows::kStream));
+      forced < 0 && (q.M <= kDecodeRowsAuto ||
+                     (q.M <= kDecodeMaxRows &&
+                      small_rows_path(q.M, q.N, q.K, q.workspace_attached && q.K % 16 == 0) == SmallRows::kStream));
   if (stream_auto || forced == 8) {
-    if (a.M > kDecodeMaxRows) return TMQ_ERR_UNSUPPORTED;
-    const int64_t blocks = ceil_div(a.N, 16);
-    if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-    // (the kernel takes K, the row pitch and N as 32-bit arguments and derives the
-    // packed pitch from K, as prepack does)
-    if (a.K > 0x7fffff00 || xs.ldx > 0x7fffffff || a.N > 0x7ffffff0 || a.w_kchunks != packed_kchunks(a.K))
-      return TMQ_ERR_UNSUPPORTED;
-    const dim3 grid(static_cast<unsigned>(blocks)), block(kDecodeWaves * kWave);
-    const int32_t k32 = static_cast<int32_t>(a.K), ldx32 = static_cast<int32_t>(xs.ldx);
-    const int32_t n32 = static_cast<int32_t>(a.N);
-    const uint32_t flags = static_cast<uint32_t>(a.M) | (a.w_scale_stride != 0 ? 0x100u : 0u) |
-                           (a.x_xor != 0 ? 0x200u : 0u);
-    switch ((a.M + 15) / 16) {
-      case 1: linear_decode_kernel<MODE, 1><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-      case 2: linear_decode_kernel<MODE, 2><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-      case 3: linear_decode_kernel<MODE, 3><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-      default: linear_decode_kernel<MODE, 4><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-    }
-    return launch_status();
+    c.cfg = stream_limits_ok(q) ? 8 : kNoKernel;
+    return c;
   }
-  // the direct-copy kernels address 256 rows of either operand with 32-bit offsets
-  // and run their three-stage ring at least once around
-  const bool dma_ok = xs.ldx <= (int64_t{1} << 23) && a.K <= (int64_t{1} << 23) && a.K > 2 * kBK;
+  const bool dma_ok = dma_limits_ok(q.K, q.ldx);
   if (forced < 0 || forced == 13) {
-    const SplitPlan p = forced == 13 ? plan_split_tiles(a.M, a.N, a.K) : plan_split(a.M, a.N, a.K);
-    if (p.splits > 1 && workspace != nullptr && workspace_bytes >= split_workspace_bytes(p, a.M) &&
-        aligned(workspace, 16))
-      return run_split<MODE>(a, xs, p, workspace, dma_ok, s);
-    if (forced == 13) return TMQ_ERR_UNSUPPORTED;
+    const SplitPlan p = forced == 13 ? plan_split_tiles(q.M, q.N, q.K) : plan_split(q.M, q.N, q.K);
+    if (p.splits > 1 && q.workspace_bytes >= split_workspace_bytes(p, q.M)) {
+      c.cfg = 13;
+      c.split = p;
+      return c;
+    }
+    if (forced == 13) return c;
   }
-  // all of K in LDS: 32-bit offsets over 64 rows of either operand, N * 4 as a 32-bit offset
-  const bool onepass_ok = a.K % 16 == 0 && a.K <= (int64_t{1} << 23) && xs.ldx <= (int64_t{1} << 23) &&
-                          a.N + a.n_off < (int64_t{1} << 29) && a.splits == 1;
+  const bool onepass_ok = onepass_limits_ok(q);
+  const int64_t M = q.M, N = q.N, K = q.K;
   int cfg = forced;
-  if (cfg < 0 && onepass_ok && a.K <= kOnePassMaxK && ceil_div(a.M, 64) * ceil_div(a.N, 64) <= 256) {
+  if (cfg < 0 && onepass_ok && K <= kOnePassMaxK && ceil_div(M, 64) * ceil_div(N, 64) <= 256) {
     // short K on a grid no larger than the chip: one latency instead of one per stage
     // (M = 128, K = N = 1024: 6.0 -> 5.6 us with cold weights); up to 512 tiles of 32 x 32
     // whose waves split K spread the copies over more CUs (3.8 us; M = 512: 5.7 -> 4.4 us;
     // N = 4096, K = 512, M = 128: 4.4 -> 4.3 us; 640 tiles and more, or K <= 256: slower)
-    cfg = a.K > 256 && ceil_div(a.M, 32) * ceil_div(a.N, 32) <= 512 ? 24 : 21;
-  } else if (cfg < 0 && onepass_ok && wstream_tile(a.M, a.N, a.K) != 0) {
+    cfg = K > 256 && ceil_div(M, 32) * ceil_div(N, 32) <= 512 ? 24 : 21;
+  } else if (cfg < 0 && onepass_ok && wstream_tile(M, N, K) != 0) {
     // K up to 4096 on a grid of 32 x 32 tiles that the chip holds at once: the waves split
     // K and take their weights through registers (cold weights, K = N = 4096, M = 64:
     // 12.2 -> 8.6 us; K = 2048, N = 4096: M = 64 9.4 -> 5.5 us, M = 128 9.4 -> 7.0 us;
     // K = N = 2048: M = 128 7.8 -> 5.0 us, M = 256 8.0 -> 6.3 us)
-    cfg = wstream_tile(a.M, a.N, a.K) == 32 ? 25 : 26;
+    cfg = wstream_tile(M, N, K) == 32 ? 25 : 26;
   } else if (cfg < 0) {
     // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
     // 256x256 tile (one block per CU) wins once it keeps about two thirds of
     // the CUs busy, the 128x128 tile (two blocks per CU) down to 128 tiles.
-    const auto nblk = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.N, bn); };
+    const auto nblk = [&](int bm, int bn) { return ceil_div(M, bm) * ceil_div(N, bn); };
     // (and only when the rows fill at least 55 % of the row tiles: a tile's time
     // does not shrink with its padding; M = 100 and 150 against N = 49152 sit on
     // either side)
-    const auto rows_used = [&](int bm) { return a.M * 20 >= ceil_div(a.M, bm) * bm * 11; };
+    const auto rows_used = [&](int bm) { return M * 20 >= ceil_div(M, bm) * bm * 11; };
     // One block of either large tile runs per CU, so a launch costs whole rounds
     // of 256 tiles.  The 128x256 tile (128 activation rows, 256 channels; 8 waves
     // of 64x64) does half the work of a 256x256 tile in 0.56 of its time (C3:
@@ -913,36 +922,102 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
       cfg = rounds128x256 < rounds256 ? cfg128x256 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
     else if (nblk(128, 256) >= 160 && rows_used(128))
       cfg = cfg128x256;
-    else if (a.N >= 2048 && (a.N >= 4096 || a.K >= 4096) && nblk(64, 64) > 256 && nblk(64, 128) <= 256)
+    else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && nblk(64, 128) <= 256)
       // a few hundred rows whose 128 x 128 tiles would leave half the chip idle and whose
       // 64 x 64 tiles need a second round: 64 rows x 128 channels, one round (K = N = 4096,
       // cold weights: M = 448: 24.6 -> 19.1 us, M = 512: 24.8 -> 19.3 us; K = 2048: 14.7 -> 11.7 us;
       // N = 8192, M = 192: 25.9 -> 19.9 us; against N = 1024 the 128 x 128 tiles stay ahead:
       // M = 1536, K = 4096: 17.4 against 20.2 us, and at K = N = 2048, M = 1024: 11.5 against 12.2 us)
       cfg = 23;
-    else if (a.N >= 2048 && (a.N >= 4096 || a.K >= 4096) && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
+    else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
       cfg = 22;
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
-    else if (nblk(64, 64) <= 256 && ceil_div(a.K, kBK) >= 32 && ceil_div(a.K, kBK) % 2 == 0)
+    else if (nblk(64, 64) <= 256 && ceil_div(K, kBK) >= 32 && ceil_div(K, kBK) % 2 == 0)
       cfg = 14;  // at most one block per CU and a long k loop: two wave groups halve it (14.7 -> 11.7 us
                  // at M = 128, K = N = 4096; four groups run into the L2's bandwidth: 12.3 us)
     else
       cfg = 2;
   }
-  // the wide activation copies walk K in runs of six stages
-  const bool wide_ok = dma_ok && a.K > 5 * kBK;
+  const bool wide_ok = wide_limits_ok(K, q.ldx);
   if (cfg == 19 && !wide_ok) cfg = 17;
-  // more than one round of 256 x 256 tiles with byte outputs: the persistent
+  // more than one round of 256 x 256 tiles with byte or float outputs: the persistent
   // kernel hides each tile's pipeline fill behind the tile before it
-  if (forced < 0 && cfg == 6 && wide_ok && MODE != kOutAcc32 && ceil_div(a.M, 256) * ceil_div(a.N, 256) > 256)
+  if (forced < 0 && cfg == 6 && wide_ok && q.mode != kOutAcc32 && ceil_div(M, 256) * ceil_div(N, 256) > 256)
     cfg = 20;
-  if (cfg == 20 && MODE == kOutAcc32) cfg = 6;  // raw outputs: one tile per block
+  if (cfg == 20 && q.mode == kOutAcc32) cfg = 6;  // raw outputs: one tile per block
   if (cfg == 20 && !wide_ok) cfg = 3;
   if (cfg == 6 && !wide_ok) cfg = 3;
   if (cfg == 17 && !dma_ok) cfg = 3;
   if (cfg == 7 && !wide_ok) cfg = 1;
   switch (cfg) {
+    case 0: case 1: case 2: case 3: case 4: case 5: case 6: case 7: case 17: case 19: case 20: case 22: case 23:
+      break;
+    case 14:  // two wave groups: equal runs of stages only
+      if (ceil_div(K, kBK) % 2 != 0) cfg = kNoKernel;
+      break;
+    case 21:
+      if (!onepass_ok) cfg = kNoKernel;
+      break;
+    case 24:
+      if (!onepass_ok || K > kOnePassMaxK) cfg = kNoKernel;
+      break;
+    case 25: case 26:
+      if (!onepass_ok || K > 4096) cfg = kNoKernel;
+      break;
+    default:
+      cfg = kNoKernel;
+  }
+  c.cfg = cfg;
+  return c;
+}
+
+template <int MODE>
+int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec_ok, int forced,
+                    hipStream_t s, void* workspace = nullptr, int64_t workspace_bytes = 0) {
+  LinearQuery q;
+  q.M = a.M;
+  q.N = a.N;
+  q.K = a.K;
+  q.ldx = xs.ldx;
+  q.n_off = a.n_off;
+  q.mode = MODE;
+  q.vec_ok = vec_ok;
+  q.workspace_attached = workspace != nullptr;
+  q.workspace_bytes = workspace != nullptr && aligned(workspace, 16) ? workspace_bytes : 0;
+  if (a.splits != 1) return TMQ_ERR_INVALID_ARGUMENT;  // the split is this function's to plan
+  const LinearChoice c = choose_linear(q, forced);
+  switch (c.cfg) {
+    case 9: {
+      // plain kernel accumulates true activation values: undo the +128 share
+      GemmArgs b = a;
+      if (!x_signed) {
+        b.acc_coef -= 128;
+        b.acc_base -= 128;
+      }
+      const int64_t work = a.M * ceil_div(a.N, 4);
+      const int64_t blocks = ceil_div(work, 256);
+      if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+      linear_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(b, xs, x_signed);
+      return launch_status();
+    }
+    case 8: {
+      // (the kernel derives the packed pitch from K, as prepack does)
+      if (a.w_kchunks != packed_kchunks(a.K)) return TMQ_ERR_UNSUPPORTED;
+      const dim3 grid(static_cast<unsigned>(ceil_div(a.N, 16))), block(kDecodeWaves * kWave);
+      const int32_t k32 = static_cast<int32_t>(a.K), ldx32 = static_cast<int32_t>(xs.ldx);
+      const int32_t n32 = static_cast<int32_t>(a.N);
+      const uint32_t flags = static_cast<uint32_t>(a.M) | (a.w_scale_stride != 0 ? 0x100u : 0u) |
+                             (a.x_xor != 0 ? 0x200u : 0u);
+      switch ((a.M + 15) / 16) {
+        case 1: linear_decode_kernel<MODE, 1><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+        case 2: linear_decode_kernel<MODE, 2><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+        case 3: linear_decode_kernel<MODE, 3><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+        default: linear_decode_kernel<MODE, 4><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+      }
+      return launch_status();
+    }
+    case 13: return run_split<MODE>(a, xs, c.split, workspace, dma_limits_ok(a.K, xs.ldx), s);
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
     case 1: return launch_gemm<128, 128, 2, 2, MODE>(a, xs, s);
     case 2: return launch_gemm<64, 64, 2, 2, MODE>(a, xs, s);
@@ -957,10 +1032,10 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 20: return launch_gemm_persistent<MODE>(a, xs, s);
     case 22: return launch_gemm<128, 64, 2, 2, MODE>(a, xs, s);
     case 23: return launch_gemm<64, 128, 2, 2, MODE>(a, xs, s);
-    case 21: return onepass_ok ? launch_gemm_onepass<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
-    case 24: return onepass_ok ? launch_gemm_ksplit<MODE>(a, xs, s) : TMQ_ERR_UNSUPPORTED;
-    case 25: return onepass_ok ? launch_gemm_wstream<MODE>(a, xs, false, s) : TMQ_ERR_UNSUPPORTED;
-    case 26: return onepass_ok ? launch_gemm_wstream<MODE>(a, xs, true, s) : TMQ_ERR_UNSUPPORTED;
+    case 21: return launch_gemm_onepass<MODE>(a, xs, s);
+    case 24: return launch_gemm_ksplit<MODE>(a, xs, s);
+    case 25: return launch_gemm_wstream<MODE>(a, xs, false, s);
+    case 26: return launch_gemm_wstream<MODE>(a, xs, true, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
@@ -1048,6 +1123,60 @@ TMQ_EXPORT int tmq_linear_split_plan(int64_t M, int64_t N, int64_t K, int32_t* s
   return TMQ_OK;
 }
 
+static_assert(sizeof(tmq_linear_choice) == 48, "tmq_linear_choice layout changed");
+
+TMQ_EXPORT int tmq_linear_kernel_choice(int64_t M, int64_t N, int64_t K, int64_t ldx, int32_t flags,
+                                        int32_t forced_kernel, int32_t compute_units, tmq_linear_choice* out) {
+  if (out == nullptr || M < 0 || N < 0 || K < 0 || ldx < K || (flags & 3) == 3 || compute_units < 0)
+    return TMQ_ERR_INVALID_ARGUMENT;
+  *out = tmq_linear_choice{};
+  out->splits = 1;
+  out->k_stages = ceil_div(K, kBK);
+  if (M == 0 || N == 0) return TMQ_OK;  // nothing is launched
+  LinearQuery q;
+  q.M = M;
+  q.N = N;
+  q.K = K;
+  q.ldx = ldx;
+  q.mode = (flags & 3) == TMQ_LINEAR_OUT_F32 ? kOutF32 : (flags & 3) == TMQ_LINEAR_OUT_ACC32 ? kOutAcc32 : kOutU8;
+  q.vec_ok = (flags & 8) == 0 && K >= 16 && K % 16 == 0 && ldx % 16 == 0;
+  q.workspace_attached = (flags & 4) != 0;
+  q.workspace_bytes = q.workspace_attached && K > 0 ? split_workspace_bytes(plan_split(M, N, K), M) : 0;
+  const LinearChoice c = choose_linear(q, forced_kernel - 1);
+  if (c.cfg == kNoKernel) return TMQ_OK;
+  int bm = 0, bn = 0, waves = 4;
+  switch (c.cfg) {
+    case 0: bm = 256, bn = 256; break;
+    case 3: case 6: case 20: bm = 256, bn = 256, waves = 8; break;
+    case 1: case 7: case 13: bm = 128, bn = 128; break;
+    case 2: case 21: bm = 64, bn = 64; break;
+    case 14: bm = 64, bn = 64, waves = 8; break;
+    case 4: bm = 128, bn = 256; break;
+    case 17: case 19: bm = 128, bn = 256, waves = 8; break;
+    case 5: bm = 256, bn = 128; break;
+    case 22: bm = 128, bn = 64; break;
+    case 23: bm = 64, bn = 128; break;
+    case 24: case 25: bm = 32, bn = 32; break;
+    case 26: bm = 32, bn = 64, waves = 8; break;
+    case 8: bm = 16 * static_cast<int>(ceil_div(M, 16)), bn = 16, waves = kDecodeWaves; break;
+    default: break;  // 9: one thread per four outputs
+  }
+  out->kernel = c.cfg + 1;
+  out->tile_rows = bm;
+  out->tile_channels = bn;
+  out->waves = waves;
+  out->splits = c.split.splits;
+  out->split_stages = c.split.stages;
+  if (c.cfg == 9) {
+    out->tiles = out->blocks = ceil_div(M * ceil_div(N, 4), 256);
+  } else {
+    out->tiles = ceil_div(M, bm) * ceil_div(N, bn) * c.split.splits;
+    out->blocks = out->tiles;
+    if (c.cfg == 20 && out->tiles > compute_units) out->blocks = compute_units / 8 * 8;
+  }
+  return TMQ_OK;
+}
+
 namespace tmq {
 namespace {
 
@@ -1105,9 +1234,19 @@ static __device__ __align__(256) uint8_t scratch[kStaticWorkspaceBytes];
 // device.  Two threads that race on a device's first call store the same value.
 std::atomic<void*> g_scratch_addr[kMaxDevices];
 
-int static_workspace(void** out) {
+// The array of the device that owns `s` -- which must be the current device: the
+// symbol's address can only be asked for on the current device.
+int static_workspace(hipStream_t s, void** out) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TMQ_ERR_LAUNCH;
+  if (s != nullptr) {
+    int sdev = -1;
+    if (hipStreamGetDevice(s, &sdev) != hipSuccess) {
+      (void)hipGetLastError();
+      return TMQ_ERR_INVALID_ARGUMENT;
+    }
+    if (sdev != dev) return TMQ_ERR_INVALID_ARGUMENT;  // another GPU's stream: that GPU has its own array
+  }
   void* p = g_scratch_addr[dev].load(std::memory_order_acquire);
   if (p == nullptr) {
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return TMQ_ERR_LAUNCH;
@@ -1127,7 +1266,7 @@ TMQ_EXPORT int tmq_linear_static_workspace(const tmq_linear_desc* d, tmq_stream_
   if (need > kStaticWorkspaceBytes) return TMQ_ERR_WORKSPACE;  // the caller's own workspace and tmq_linear then
   void* ws = nullptr;
   if (need > 0) {
-    const int rc = static_workspace(&ws);
+    const int rc = static_workspace(as_stream(stream), &ws);
     if (rc != TMQ_OK) return rc;
   }
   return linear_u8s8(d, ws, need, stream);
