@@ -332,23 +332,25 @@ def test_qadaptive_avgpool_resnet_head_sized(cabi):
 
 
 @pytest.mark.parametrize("n,offset", [(1, 0), (7, 0), (4096, 0), (4099, 1), (65536, 0), (65537, 0), (65541, 3),
-                                      (1 << 20, 0), ((1 << 20) + 3, 1)])
+                                      (1 << 20, 0), ((1 << 20) + 3, 1), ((1 << 23) + 1029, 0), ((1 << 25) + 4, 0)])
 @pytest.mark.parametrize("signed,reduce_range", [(False, False), (False, True), (True, False)])
 def test_quantize_dynamic_on_device(cabi, n, offset, signed, reduce_range):
-    # one call: range, parameters (left in device memory) and codes; small inputs take
-    # the single-block kernel, larger ones the three-launch chain -- same results
+    # one call: range, parameters (left in device memory) and codes; small inputs take the
+    # single-block kernel, aligned ones of up to 2**25 elements two launches (the quantizer's
+    # blocks finish the reduction; 2**23 + 1029 walks its grid-stride loop more than once and
+    # ends inside a chunk), larger or unaligned ones the three-launch chain -- same results
     say("dynamic dev", n, offset, signed, reduce_range)
     rng = np.random.default_rng(n + offset)
     x = (rng.standard_normal(n + offset) * 2.5 + 0.4).astype(np.float32)
     xd = dev(x)[offset:]
     q, qp = cabi.quantize_per_tensor_dynamic_dev(xd.contiguous() if offset == 0 else xd, signed, reduce_range)
-    mn, mx = oracle.minmax(x[offset:])
+    mn, mx = oracle.minmax(x[offset:], nthreads=8)
     scale, zp = oracle.choose_qparams(mn, mx, signed, reduce_range)
     assert cabi.read_qparams(qp) == (scale, zp)
-    np.testing.assert_array_equal(host(q), oracle.quantize_per_tensor(x[offset:], scale, zp, signed))
+    np.testing.assert_array_equal(host(q), oracle.quantize_per_tensor(x[offset:], scale, zp, signed, nthreads=8))
 
 
-@pytest.mark.parametrize("n,offset", [(4099, 1), (65536, 0), ((1 << 22) + 3, 0)])
+@pytest.mark.parametrize("n,offset", [(4099, 1), (65536, 0), ((1 << 22) + 3, 0), ((1 << 23) + 1029, 0)])
 @pytest.mark.parametrize("signed", [False, True])
 def test_quantize_dynamic_fused_rounding(cabi, n, offset, signed):
     # the activation quantization of the CPU quantized::linear_dynamic: x * inv + zp

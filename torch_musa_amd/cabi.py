@@ -233,7 +233,7 @@ def quantize_per_tensor_dev(x: torch.Tensor, qp: torch.Tensor, signed: bool) -> 
 
 
 def quantize_per_tensor_dynamic_dev(x: torch.Tensor, signed: bool, reduce_range: bool, fused: bool = False):
-    """-> (codes, 16 device bytes of qparams); one launch for small inputs, three otherwise.
+    """-> (codes, 16 device bytes of qparams); one launch for small inputs, two or three otherwise.
     fused: round x * inv + zp once (the CPU linear_dynamic's activation quantization)
     instead of rne(x * inv) + zp (quantize_per_tensor)."""
     assert x.dtype == torch.float32 and x.is_contiguous()

@@ -117,11 +117,19 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(
     uint32_t flags, GemmArgs a) {
   constexpr int kWaves = kDecodeWaves;
   constexpr int kBatch = 8;  // 64-byte k-blocks in flight per wave: 64 KB of weights per block
-  __shared__ int s_part[kWaves][MG][16 * 16];
+  // The eight waves' partial sums meet in one [4 registers][64 lanes] array per row group:
+  // every wave adds its accumulators with LDS atomics as it finishes (a wave instruction covers
+  // 64 consecutive words: no bank conflicts, and the early waves' additions are off the block's
+  // critical path), and the 64 finishing threads read four words each instead of 32.
+  __shared__ int s_sum[MG][4][kWave];
   const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
   const int lr = lane & 15, lc = lane >> 4;
   const int nb = blockIdx.x;
   const int M = static_cast<int>(flags & 0xffu);
+  for (int i = t; i < MG * 4 * kWave; i += kWaves * kWave) (&s_sum[0][0][0])[i] = 0;
+  // (before any global request is made: the barrier's wait for outstanding memory
+  // operations is then a wait for this one LDS store)
+  __syncthreads();
   const int KB = (K + 63) >> 6;
   // The 64 threads that finish a block: thread -> activation row within a
   // group, channel group of 4.
@@ -220,7 +228,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(
 #pragma unroll
   for (int mg = 0; mg < MG; ++mg)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) s_part[wave][mg][(4 * lc + r) * 16 + lr] = acc[mg][r];
+    for (int r = 0; r < 4; ++r)
+      __hip_atomic_fetch_add(&s_sum[mg][r][lane], acc[mg][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   // requantisation constants, before the barrier: off the block's critical path
   v4f bdiv = {0.f, 0.f, 0.f, 0.f}, mult = {0.f, 0.f, 0.f, 0.f};
   float bmul = 1.f;
@@ -250,13 +259,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_kernel(
       if (m >= a.M) continue;
       int raw[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        int s = 0;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) s += s_part[w][mg][i * 16 + fm];
-        raw[j] = s + acc0[j];
-      }
+      for (int j = 0; j < 4; ++j)  // channel 4 g + j of row fm: register j of lane 16 g + fm
+        raw[j] = s_sum[mg][j][16 * g + fm] + acc0[j];
       const int64_t n = nb * 16 + 4 * g;
       if (MODE == kOutAcc32) {
         int32_t* dst = static_cast<int32_t*>(a.y) + m * a.ldy + n;
@@ -302,7 +306,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_dynamic_ker
   constexpr int kBatch = 8;
   static_assert(kHeld * 4 * kWaves * kWave <= kDynSmallMaxValues, "held values");
   extern __shared__ __attribute__((aligned(16))) uint8_t sx[];  // [M][K + 16] activation codes
-  __shared__ int s_part[kWaves][16 * 16];
+  __shared__ int s_sum[4][kWave];  // the waves' partial sums, added with LDS atomics (see linear_decode_kernel)
   __shared__ float s_mn[kWaves], s_mx[kWaves];
   __shared__ float s_scale, s_inv, s_zp;
   const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
@@ -366,6 +370,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_dynamic_ker
     s_mn[wave] = mn;
     s_mx[wave] = mx;
   }
+  if (t < 4 * kWave) (&s_sum[0][0])[t] = 0;  // (two barriers before the first addition)
   __syncthreads();
   if (t == 0) {
 #pragma unroll
@@ -427,7 +432,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_dynamic_ker
     }
   }
 #pragma unroll
-  for (int r = 0; r < 4; ++r) s_part[wave][(4 * lc + r) * 16 + lr] = acc[r];
+  for (int r = 0; r < 4; ++r)
+    __hip_atomic_fetch_add(&s_sum[r][lane], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   v4f mult = {0.f, 0.f, 0.f, 0.f}, bias = {0.f, 0.f, 0.f, 0.f};
   int acc0[4] = {0, 0, 0, 0};
   if (t < 64) {
@@ -443,13 +449,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void linear_decode_dynamic_ker
   if (t < 64 && fm < a.M) {
     int raw[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int i = 4 * fg + j;
-      int s = 0;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) s += s_part[w][i * 16 + fm];
-      raw[j] = s + acc0[j];
-    }
+    for (int j = 0; j < 4; ++j) raw[j] = s_sum[j][16 * fg + fm] + acc0[j];
     store_f32x4(a, fm, nb * 16 + 4 * fg, raw, mult, bias);
   }
 }

@@ -235,9 +235,13 @@ __device__ __forceinline__ void block_minmax_store(float mn, float mx, float* ou
   }
 }
 
+// KEEP: ordinary loads instead of non-temporal ones, for an input that a second pass on
+// the stream reads again while the last-level cache still holds it.
+template <bool KEEP = false>
 __global__ __launch_bounds__(kThreads) void minmax_partial_kernel(
     const v4f* __restrict__ x4, int64_t n4, const float* __restrict__ x, int64_t head,
     int64_t n, float* __restrict__ partials) {
+  auto ld = [](const v4f* p) { return KEEP ? *p : __builtin_nontemporal_load(p); };
   float mn = std::numeric_limits<float>::infinity();
   float mx = -std::numeric_limits<float>::infinity();
   const int64_t step = static_cast<int64_t>(gridDim.x) * (kThreads * kUnroll);
@@ -247,7 +251,7 @@ __global__ __launch_bounds__(kThreads) void minmax_partial_kernel(
     if (base - threadIdx.x + kThreads * kUnroll <= n4) {
       // a whole chunk: unconditional loads, all in flight before the first comparison
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) v[u] = __builtin_nontemporal_load(&x4[base + u * kThreads]);
+      for (int u = 0; u < kUnroll; ++u) v[u] = ld(&x4[base + u * kThreads]);
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         mn = fminf(fminf(mn, v[u].x), fminf(v[u].y, fminf(v[u].z, v[u].w)));
@@ -258,7 +262,7 @@ __global__ __launch_bounds__(kThreads) void minmax_partial_kernel(
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t i = base + u * kThreads;
-      if (i < n4) v[u] = __builtin_nontemporal_load(&x4[i]);
+      if (i < n4) v[u] = ld(&x4[i]);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -328,6 +332,81 @@ __global__ __launch_bounds__(kThreads) void minmax_final_choose_kernel(
       minmax_out[0] = s_mm[0];
       minmax_out[1] = s_mm[1];
     }
+  }
+}
+
+// Second launch of a dynamic quantization: every block first finishes the range
+// reduction for itself -- the partial {min, max} pairs of the pass before it (at most
+// kDynPartials of them, 4 KB from the L2s), ChooseQuantizationParams in one thread --
+// while the loads of its first elements are already in flight, then quantizes its
+// share of the input in a grid-stride loop with the next chunk requested before the
+// current one is converted.  Block 0 also publishes the parameters.  This replaces a
+// one-block launch between the two passes (5 us of a 32 us chain at 2**24 elements:
+// launch, 16 KB through one block, the double-precision divisions) by a few hundred
+// cycles under each block's first loads.  Same arithmetic in the same order as the
+// three launches: min and max do not depend on the order of the reduction.
+constexpr int kDynPartials = 512;
+constexpr int kDynQBlocks = 2048;
+constexpr int64_t kDynKeepMax = int64_t{1} << 25;  // 128 MiB of fp32: half the last-level cache
+template <bool SIGNED, bool FUSED>
+__global__ __launch_bounds__(kThreads) void quantize_after_minmax_kernel(
+    const v4f* __restrict__ x4, uint32_t* __restrict__ q4, int64_t n4, const float* __restrict__ x,
+    uint8_t* __restrict__ q, int64_t n, const float* __restrict__ partials, int count, int qmin, int qmax,
+    int reduce_range, tmq_qparams* __restrict__ out) {
+  __shared__ float s_mm[2];
+  __shared__ float s_inv, s_zp;
+  constexpr int U = kUnrollQD;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * (kThreads * U);
+  int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * U) + threadIdx.x;
+  // (loads are unconditional -- indices clamped into the input -- so that they can be
+  // counted: a load under a condition would be waited for before anything else is requested)
+  auto request = [&](int64_t b, v4f(&v)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = b + u * kThreads;
+      v[u] = x4[i < n4 ? i : (n4 > 0 ? n4 - 1 : 0)];
+    }
+  };
+  v4f cur[U], nxt[U];
+  if (n4 > 0) request(base, cur);
+  float mn = std::numeric_limits<float>::infinity();
+  float mx = -std::numeric_limits<float>::infinity();
+  for (int i = threadIdx.x; i < count; i += kThreads) {
+    const float2 p = *reinterpret_cast<const float2*>(partials + 2 * i);
+    mn = fminf(mn, p.x);
+    mx = fmaxf(mx, p.y);
+  }
+  block_minmax_store(mn, mx, s_mm);  // (ends with thread 0 holding the block's result)
+  if (threadIdx.x == 0) {
+    double sc;
+    int32_t z;
+    choose_qparams(s_mm[0], s_mm[1], qmin, qmax, reduce_range != 0, &sc, &z);
+    s_inv = 1.0f / static_cast<float>(sc);  // IEEE division, as resolve()
+    s_zp = static_cast<float>(z);
+    if (blockIdx.x == 0) {
+      out->scale = sc;
+      out->zero_point = z;
+      out->reserved = 0;
+    }
+  }
+  __syncthreads();
+  const float inv = s_inv, zp_f = s_zp;
+  for (; base - threadIdx.x < n4; base += step) {
+    const bool more = base - threadIdx.x + step < n4;
+    if (more) request(base + step, nxt);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < n4) q4[i] = quantize_four<SIGNED, FUSED>(cur[u], inv, zp_f);
+    }
+    if (more) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) cur[u] = nxt[u];
+    }
+  }
+  if (blockIdx.x == 0) {
+    const int64_t i = 4 * n4 + threadIdx.x;
+    if (i < n) q[i] = static_cast<uint8_t>(quantize_one<SIGNED, FUSED>(x[i], inv, zp_f));
   }
 }
 
@@ -876,7 +955,7 @@ TMQ_EXPORT int tmq_minmax(const float* x, int64_t n, float* minmax, void* worksp
   }
   const int64_t n4 = (n - head) / 4;
   const unsigned g = grid_for(n4, kThreads * kUnroll, kMinMaxMaxBlocks);
-  minmax_partial_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(
+  minmax_partial_kernel<false><<<dim3(g), dim3(kThreads), 0, s>>>(
       reinterpret_cast<const v4f*>(x + head), n4, x, head, n, partials);
   if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
   minmax_final_kernel<<<dim3(1), dim3(kThreads), 0, s>>>(partials, static_cast<int>(g), minmax);
@@ -917,12 +996,38 @@ TMQ_EXPORT int tmq_quantize_per_tensor_dynamic_dev(const float* x, void* q, int6
   if (workspace == nullptr || workspace_bytes < tmq_minmax_workspace_bytes(n) || !aligned(workspace, 4))
     return TMQ_ERR_WORKSPACE;
   float* partials = static_cast<float*>(workspace);
+  if (n <= kDynKeepMax && aligned(x, 16) && aligned(q, 4) && aligned(workspace, 8)) {
+    // Inputs that fit the last-level cache with room to spare (where the launches, not the
+    // bytes, are what counts): two launches -- partial ranges, read with ordinary loads so
+    // that the second pass finds the input cached, then the quantizer whose blocks finish
+    // the reduction themselves.
+    const int64_t n4 = n / 4;
+    const unsigned g = grid_for(n4, kThreads * kUnroll, kDynPartials);
+    const v4f* x4 = reinterpret_cast<const v4f*>(x);
+    minmax_partial_kernel<true><<<dim3(g), dim3(kThreads), 0, s>>>(x4, n4, x, 0, n, partials);
+    if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+    const dim3 grid(grid_for(n4, kThreads * kUnrollQD, kDynQBlocks)), block(kThreads);
+    uint32_t* q4 = static_cast<uint32_t*>(q);
+    uint8_t* qb = static_cast<uint8_t*>(q);
+    const int cnt = static_cast<int>(g);
+    if (q_signed && fused)
+      quantize_after_minmax_kernel<true, true><<<grid, block, 0, s>>>(x4, q4, n4, x, qb, n, partials, cnt, qmin, qmax, reduce_range, qparams);
+    else if (q_signed)
+      quantize_after_minmax_kernel<true, false><<<grid, block, 0, s>>>(x4, q4, n4, x, qb, n, partials, cnt, qmin, qmax, reduce_range, qparams);
+    else if (fused)
+      quantize_after_minmax_kernel<false, true><<<grid, block, 0, s>>>(x4, q4, n4, x, qb, n, partials, cnt, qmin, qmax, reduce_range, qparams);
+    else
+      quantize_after_minmax_kernel<false, false><<<grid, block, 0, s>>>(x4, q4, n4, x, qb, n, partials, cnt, qmin, qmax, reduce_range, qparams);
+    return launch_status();
+  }
+  // larger inputs (streamed past the caches) and unaligned buffers: range, parameters and
+  // codes in three launches
   const uintptr_t mis = reinterpret_cast<uintptr_t>(x) & 15u;
   int64_t head = mis == 0 ? 0 : static_cast<int64_t>((16 - mis) / 4);
   if (head > n) head = n;
   const int64_t n4 = (n - head) / 4;
   const unsigned g = grid_for(n4, kThreads * kUnroll, kMinMaxMaxBlocks);
-  minmax_partial_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(reinterpret_cast<const v4f*>(x + head), n4, x, head,
+  minmax_partial_kernel<false><<<dim3(g), dim3(kThreads), 0, s>>>(reinterpret_cast<const v4f*>(x + head), n4, x, head,
                                                            n, partials);
   if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
   minmax_final_choose_kernel<<<dim3(1), dim3(kThreads), 0, s>>>(partials, static_cast<int>(g), qmin, qmax,
