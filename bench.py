@@ -168,7 +168,7 @@ def main():
     ap.add_argument("--skip-secondary", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
-                                       "dequantize_pc", "decode", "rows64", "c1", "conv", "conv_add_relu", "probe"],
+                                       "dequantize_pc", "decode", "rows64", "c1", "conv", "conv_add_relu", "probe", "choice"],
                     help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
                          "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
                          "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
@@ -241,6 +241,71 @@ def main():
             tops_p, ghz_p = cabi.probe_mfma_i8(mode)
             res[name] = {"tops": round(tops_p, 1), "shader_ghz": round(ghz_p, 3)}
         print(json.dumps({"only": "probe", "modes": res}))
+        return
+
+    if args.only == "choice":
+        # The automatic kernel choice of quantized::linear against every kernel that can run the
+        # shape, at shapes on either side of the dispatcher's thresholds: cold weights (as many
+        # weight sets in rotation as exceed the 256 MB last-level cache, at most 40) replayed
+        # in one HIP graph per candidate.  A ratio well above 1 says a threshold has gone stale.
+        shapes = [(17, 4096, 4096), (24, 4096, 4096), (32, 4096, 4096), (64, 4096, 4096), (96, 4096, 4096),
+                  (128, 4096, 4096), (256, 4096, 4096), (448, 4096, 4096), (512, 4096, 4096), (1024, 4096, 4096),
+                  (2048, 4096, 4096), (64, 11008, 4096), (256, 11008, 4096), (2048, 11008, 4096),
+                  (64, 4096, 11008), (256, 4096, 11008), (128, 1024, 1024), (512, 1024, 1024), (640, 1024, 1024),
+                  (128, 2048, 2048), (256, 4096, 2048), (4096, 4096, 4096)]
+        candidates = (2, 3, 6, 7, 8, 13, 14, 17, 19, 20, 21, 23, 24, 25, 26)
+        rows = []
+        for (Ms, Ns, Ks) in shapes:
+            sets = max(2, min(40, (600 << 20) // (Ns * Ks)))
+            pws = [cabi.PackedLinear(torch.randint(-127, 128, (Ns, Ks), dtype=torch.int8, device=dev))
+                   for _ in range(sets)]
+            wsd, bd = torch.rand(Ns, device=dev) * 0.002 + 0.001, torch.randn(Ns, device=dev)
+            xd = torch.randint(0, 256, (Ms, Ks), dtype=torch.uint8, device=dev)
+            yd = torch.empty((Ms, Ns), dtype=torch.uint8, device=dev)
+            wbytes = cabi.lib().tmq_linear_workspace_bytes(Ms, Ns, Ks)
+            cabi.linear_workspace = torch.empty(max(wbytes, 16), dtype=torch.uint8, device=dev)
+
+            def timed(cfg):
+                cabi.force_linear_config(cfg)
+                try:
+                    def run_sets():
+                        for p_ in pws:
+                            cabi.linear(xd, p_, 0.02, 128, wsd, bd, 0.05, 128, out=yd)
+                    run_sets()
+                    torch.cuda.synchronize()
+                    side_, graph_ = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+                    with torch.cuda.stream(side_):
+                        side_.synchronize()
+                        with torch.cuda.graph(graph_, stream=side_):
+                            run_sets()
+                    torch.cuda.synchronize()
+                    graph_.replay()
+                    ts_ = sorted(events_ms(graph_.replay, 5))
+                    return ts_[len(ts_) // 2] / sets * 1e3
+                finally:
+                    cabi.force_linear_config(-1)
+
+            auto = cabi.linear_kernel_choice(Ms, Ns, Ks, workspace=wbytes > 0)
+            t_auto = timed(-1)
+            others = {}
+            for cfg in candidates:
+                c_ = cabi.linear_kernel_choice(Ms, Ns, Ks, workspace=wbytes > 0, forced=cfg + 1)
+                if c_["kernel"] - 1 != cfg or cfg == auto["kernel"] - 1:
+                    continue          # refused, or replaced by another kernel
+                if c_["blocks"] > 8192 or (cfg in (2, 14, 21, 24, 25, 26) and Ms * Ns > 1 << 22):
+                    continue          # small tiles on a large product: not a candidate
+                others[cfg] = round(timed(cfg), 2)
+            best = min(others, key=others.get) if others else None
+            rows.append({"M": Ms, "N": Ns, "K": Ks, "auto_kernel": auto["kernel"] - 1, "auto_us": round(t_auto, 2),
+                         "best_other_kernel": best, "best_other_us": others.get(best),
+                         "auto_over_best": round(t_auto / min([t_auto] + list(others.values())), 3),
+                         "others_us": others})
+            log(f"[bench] choice M={Ms} N={Ns} K={Ks}: auto cfg {auto['kernel'] - 1} {t_auto:.2f} us; "
+                f"best other cfg {best} {others.get(best)} us")
+            cabi.linear_workspace = None
+            del pws
+        print(json.dumps({"only": "choice", "worst_auto_over_best": max(r["auto_over_best"] for r in rows),
+                          "rows": rows}))
         return
 
     def per_channel_sets(nsets):
