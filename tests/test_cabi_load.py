@@ -152,7 +152,6 @@ def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256
         assert kt >= 6 and 256 * ldx <= 2 ** 31 and 15 * 16 * _ceil(k, 128) * 128 < 2 ** 32, what   # 32-bit offsets
         if cfg == 20:                               # persistent: byte / float outputs, several rounds, whole XCD runs
             assert out != "acc32" and (bm, bn) == (256, 256), what
-            assert forced != 0 or tiles > cus, what
             # (the tile sequence is a permutation only on a multiple of 8 blocks or with every tile in one round)
             assert c["blocks"] == (cus // 8 * 8 if tiles > cus else tiles), what
         else:
@@ -179,6 +178,10 @@ def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256
         assert k <= 4096 and (bm, bn) == (32, 64) and c["waves"] == 8 and 64 * ldx <= 2 ** 29, what
         if forced == 0:
             assert k > 2048 and tiles <= 256, what
+    elif cfg == 27:                                 # 64 x 64, an eighth of K per wave: 16 k-steps of weights in registers
+        assert k <= 4096 and (bm, bn) == (64, 64) and c["waves"] == 8 and 64 * ldx <= 2 ** 29, what
+        if forced == 0:                             # one round, and a K long enough to fill the waves' shares
+            assert k >= 3072 and tiles <= 256, what
     else:                                           # register-staged tiles take any aligned shape
         assert cfg in (0, 1, 2, 3, 4, 5, 22, 23), what
     if forced == 0 and cfg in (22, 23):             # a few hundred rows: one round of oblong tiles
@@ -222,7 +225,7 @@ def test_automatic_kernel_choice_keeps_every_kernels_preconditions():
             seen.add(c["kernel"] - 1)
     c = cabi.linear_kernel_choice(300, 500, 4096, misaligned=True)
     assert c["kernel"] == 10
-    assert seen >= {2, 3, 6, 7, 8, 9, 13, 14, 17, 19, 20, 21, 23, 24, 25, 26}, sorted(seen)
+    assert seen >= {2, 3, 7, 8, 9, 13, 14, 17, 19, 20, 21, 23, 24, 25, 26, 27}, sorted(seen)
     # the benchmark configurations
     assert cabi.linear_kernel_choice(4096, 11008, 4096)["kernel"] - 1 == 20
     assert cabi.linear_kernel_choice(4096, 11008, 4096)["blocks"] == 256
@@ -238,7 +241,7 @@ def test_forced_kernels_run_inside_their_preconditions_or_not_at_all():
     rng = np.random.default_rng(21)
     refused = 0
     for m, n, k, ldx in _random_linear_shapes(rng, 1500):
-        for cfg in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26):
+        for cfg in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26, 27):
             for out in ("bytes", "acc32"):
                 c = cabi.linear_kernel_choice(m, n, k, ldx, out, workspace=True, forced=cfg + 1)
                 if c["kernel"] == 0:

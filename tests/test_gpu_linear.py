@@ -89,7 +89,7 @@ def test_per_tensor_weight_bias_form(cabi, golden, cfg):
 
 
 # every tile configuration of the MFMA kernel, with ragged M / N / K-stage tails
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23, 24, 25, 26])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 9, 17, 19, 20, 21, 22, 23, 24, 25, 26, 27])
 @pytest.mark.parametrize("shape", [(300, 520, 448), (257, 33, 64), (64, 1040, 1168), (130, 260, 144), (256, 256, 192),
                                    (270, 300, 400), (40, 70, 784)])
 def test_tile_configs(cabi, cfg, shape):
@@ -156,9 +156,9 @@ def test_whole_k_in_lds_kernel(cabi, shape, x_signed, cfg):
 # 32 x 32 tiles whose waves split K with the weights through registers: K up to 4096 (both
 # instantiations: 16 and 32 k-steps per wave), K that leaves waves without work, odd chunks
 @pytest.mark.parametrize("shape", [(64, 160, 4096), (33, 200, 2064), (100, 130, 4080), (17, 70, 3088),
-                                   (128, 64, 2048), (40, 33, 1040), (5, 32, 2304)])
+                                   (128, 64, 2048), (40, 33, 1040), (5, 32, 2304), (200, 300, 3600), (256, 192, 16)])
 @pytest.mark.parametrize("x_signed", [False, True])
-@pytest.mark.parametrize("cfg", [25, 26])       # 32 and 64 channels per tile
+@pytest.mark.parametrize("cfg", [25, 26, 27])   # 32 x 32, 32 x 64, and 64 x 64 tiles with an activation ring
 def test_weights_through_registers_kernel(cabi, shape, x_signed, cfg):
     say("weights through registers", shape, x_signed, cfg)
     M, N, K = shape
@@ -205,7 +205,7 @@ def test_small_batch_kernels_on_random_shapes(cabi):
                 cabi.force_linear_config(-1)
 
         want = run(2)
-        for cfg in [c for c in (21, 24, 25, 26, -1) if not (c == 24 and K > 1024)]:
+        for cfg in [c for c in (21, 24, 25, 26, 27, -1) if not (c == 24 and K > 1024)]:
             for got, ref, what in zip(run(cfg), want, ("bytes", "accumulators", "float output")):
                 assert torch.equal(got, ref), f"cfg {cfg} {what} at {(M, N, K)}"
 

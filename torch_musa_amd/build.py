@@ -46,6 +46,35 @@ DEVICE_FLAGS = [
 ]
 
 
+# Kernels whose loads are asm statements with hand-counted waits: a fragment that the
+# compiler moved to scratch memory would be copied before its load has landed, so the
+# build fails if any of them uses scratch (the compiler reports each kernel's resources).
+NO_SCRATCH_KERNELS = ("gemm_i8_wring_kernel",)
+RESOURCE_REMARKS = ["-Rpass-analysis=kernel-resource-usage"]
+
+
+def _needs_register_check(obj):
+    return os.path.basename(obj) == "linear.hip.o"
+
+
+def _check_no_scratch(remarks, kernels):
+    name, seen = None, set()
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split()[0]
+        elif "ScratchSize [bytes/lane]:" in line and name is not None:
+            for k in kernels:
+                if k in name:
+                    seen.add(k)
+                    size = int(line.split("ScratchSize [bytes/lane]:", 1)[1].split()[0])
+                    if size != 0:
+                        raise RuntimeError(f"{name} uses {size} bytes of scratch per lane: its asm loads "
+                                           "must stay in registers")
+    missing = set(kernels) - seen
+    if missing:
+        raise RuntimeError(f"no resource report for {sorted(missing)}: the register check did not run")
+
+
 def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -56,6 +85,7 @@ def _run(cmd, verbose):
         raise RuntimeError(f"command failed ({p.returncode}): {' '.join(cmd)}\n{out}")
     if verbose and out.strip():
         print(out, flush=True)
+    return out
 
 
 def _hipcc():
@@ -85,7 +115,11 @@ def _build_hip_library(sources, lib_path, verbose):
         obj = os.path.join(OBJ, os.path.basename(src) + ".o")
         jobs.append((obj, [hipcc] + DEVICE_FLAGS + inc + ["-c", path, "-o", obj]))
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
-        list(ex.map(lambda j: _run(j[1], verbose), jobs))
+        outs = list(ex.map(lambda j: _run(j[1] + (RESOURCE_REMARKS if _needs_register_check(j[0]) else []),
+                                          verbose and not _needs_register_check(j[0])), jobs))
+    for (obj, _), out in zip(jobs, outs):
+        if _needs_register_check(obj):
+            _check_no_scratch(out, NO_SCRATCH_KERNELS)
     _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", lib_path]
          + [j[0] for j in jobs], verbose)
     return lib_path

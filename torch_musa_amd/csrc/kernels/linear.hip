@@ -6,6 +6,7 @@
 #include "gemm_i8_core.h"
 #include "gemm_i8_onepass.h"
 #include "gemm_i8_persistent.h"
+#include "gemm_i8_wring.h"
 #include "qparams.h"
 
 // Layout that non-C++ bindings rely on (natural alignment, x86-64).
@@ -553,6 +554,17 @@ int launch_gemm_wstream(const GemmArgs& a, const XLinear& xs, bool wide, hipStre
   return launch_status();
 }
 
+// 64 x 64 tiles whose eight waves split K, weights through registers, activations through
+// a ring per wave (K <= 4096; the caller checked the address ranges).
+template <int MODE>
+int launch_gemm_wring(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  const int64_t tiles_m = ceil_div(a.M, 64), tiles_n = ceil_div(a.N, 64);
+  if (tiles_n > 0x7fffffff || tiles_m > 65535 || a.K > kWringMaxK || a.K % 16 != 0) return TMQ_ERR_UNSUPPORTED;
+  gemm_i8_wring_kernel<MODE><<<dim3(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m)),
+                               dim3(kWringThreads), 0, s>>>(a, xs);
+  return launch_status();
+}
+
 constexpr int kMaxDevices = 64;
 
 // Compute units of the current device (cached per device; two threads that race
@@ -652,7 +664,12 @@ SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
   //   K = 4096, N = 4096:  8.2 / 8.3 / 8.6 | 6.8 / 7.8 / 12.2    K = 4096, N = 1024:  6.5 / 6.5 / 6.6 | 6.0 / 7.0 / 11.3
   //   K = 3072, N = 4096:  7.2 / 7.3 / 7.6 | 6.4 / 7.5 / 11.7    K = 4096, N = 8192: 10.6 / 10.7 / -  | 11.7 / 13.6 / 22.6
   // streaming keeps the longer K up to about two dozen rows while its blocks fit one round.
-  if (wstream_tile(M, N, K) != 0) return K > 2048 && M <= 24 && N <= 4096 ? SmallRows::kStream : SmallRows::kTiles;
+  // (K = N = 4096, M = 32: 7.6 against 8.5 us, so the longest K streams up to 32 rows there;
+  // at K = 3072, or against N = 1024, the tiles are ahead from 25 rows on)
+  if (wstream_tile(M, N, K) != 0) {
+    const int64_t stream_rows = K > 3072 && N >= 2048 ? 32 : 24;
+    return K > 2048 && M <= stream_rows && N <= 4096 ? SmallRows::kStream : SmallRows::kTiles;
+  }
   const double mib = static_cast<double>(N) * static_cast<double>(K) / 1048576.0;
   const double stages = static_cast<double>(ceil_div(K, kBK));
   const double rows = static_cast<double>(M);
@@ -832,7 +849,8 @@ struct LinearQuery {
 // cfg: tmq_linear_desc::kernel - 1.  0-7, 14, 17, 19, 22, 23: tiles of gemm_i8_kernel; 8: weight
 // streaming; 9: plain kernel; 13: split K (plan in `split`); 20: persistent 256 x 256 tiles;
 // 21 / 24: all of K in LDS (64 x 64 / 32 x 32 tiles); 25 / 26: weights through registers
-// (32 x 32 / 32 x 64 tiles); kNoKernel: the forced kernel does not take this shape.
+// (32 x 32 / 32 x 64 tiles); 27: the same with 64 x 64 tiles and the activations in a ring
+// per wave; kNoKernel: the forced kernel does not take this shape.
 constexpr int kNoKernel = -2;
 struct LinearChoice {
   int cfg = kNoKernel;
@@ -933,6 +951,14 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
       cfg = 22;
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
       cfg = 7;
+    else if (onepass_ok && K >= 3072 && K <= kWringMaxK && nblk(64, 64) <= 256 && N * K <= (int64_t{1} << 24))
+      // one round of 64 x 64 tiles against a long K: eight waves split K, weights through
+      // registers, activations through a ring per wave, no barrier before the partial tiles
+      // meet (cold weights, K = N = 4096: M = 130 12.1 -> 11.8 us, M = 192 14.0 -> 12.8 us,
+      // M = 256 14.3 -> 13.6 us; N = 2048: M = 512 14.0 -> 13.0 us; K = 3072: M = 192
+      // 13.0 -> 12.1 us; behind the two wave groups at K = 2560 (12.3 against 11.7 us) and
+      // against 32 MB of weights, N = 8192: 15.3 against 14.6 us)
+      cfg = 27;
     else if (nblk(64, 64) <= 256 && ceil_div(K, kBK) >= 32 && ceil_div(K, kBK) % 2 == 0)
       cfg = 14;  // at most one block per CU and a long k loop: two wave groups halve it (14.7 -> 11.7 us
                  // at M = 128, K = N = 4096; four groups run into the L2's bandwidth: 12.3 us)
@@ -941,10 +967,11 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
   }
   const bool wide_ok = wide_limits_ok(K, q.ldx);
   if (cfg == 19 && !wide_ok) cfg = 17;
-  // more than one round of 256 x 256 tiles with byte or float outputs: the persistent
-  // kernel hides each tile's pipeline fill behind the tile before it
-  if (forced < 0 && cfg == 6 && wide_ok && q.mode != kOutAcc32 && ceil_div(M, 256) * ceil_div(N, 256) > 256)
-    cfg = 20;
+  // 256 x 256 tiles with byte or float outputs: the persistent kernel, which hides each
+  // tile's pipeline fill behind the tile before it and whose epilogue needs no block
+  // barrier (also ahead on a single round: M = N = K = 4096, 256 tiles: 61.9 -> 59.7 us;
+  // 2560 x 4096: 46.4 -> 45.8 us; never behind in a sweep of one to three rounds)
+  if (forced < 0 && cfg == 6 && wide_ok && q.mode != kOutAcc32) cfg = 20;
   if (cfg == 20 && q.mode == kOutAcc32) cfg = 6;  // raw outputs: one tile per block
   if (cfg == 20 && !wide_ok) cfg = 3;
   if (cfg == 6 && !wide_ok) cfg = 3;
@@ -964,6 +991,9 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
       break;
     case 25: case 26:
       if (!onepass_ok || K > 4096) cfg = kNoKernel;
+      break;
+    case 27:
+      if (!onepass_ok || K > kWringMaxK) cfg = kNoKernel;
       break;
     default:
       cfg = kNoKernel;
@@ -1036,6 +1066,7 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
     case 24: return launch_gemm_ksplit<MODE>(a, xs, s);
     case 25: return launch_gemm_wstream<MODE>(a, xs, false, s);
     case 26: return launch_gemm_wstream<MODE>(a, xs, true, s);
+    case 27: return launch_gemm_wring<MODE>(a, xs, s);
     default: return TMQ_ERR_UNSUPPORTED;
   }
 }
@@ -1158,6 +1189,7 @@ TMQ_EXPORT int tmq_linear_kernel_choice(int64_t M, int64_t N, int64_t K, int64_t
     case 23: bm = 64, bn = 128; break;
     case 24: case 25: bm = 32, bn = 32; break;
     case 26: bm = 32, bn = 64, waves = 8; break;
+    case 27: bm = 64, bn = 64, waves = 8; break;
     case 8: bm = 16 * static_cast<int>(ceil_div(M, 16)), bn = 16, waves = kDecodeWaves; break;
     default: break;  // 9: one thread per four outputs
   }
