@@ -167,8 +167,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--skip-secondary", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--no-power", action="store_true",
+                    help="do not start the child process that samples the socket power (for runs under a profiler, "
+                         "whose library has initialised the GPU before this program starts)")
     ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
-                                       "dequantize_pc", "decode", "rows64", "c1", "conv", "conv_add_relu", "probe", "choice"],
+                                       "dequantize_pc", "decode", "rows64", "rows256", "c1", "conv", "conv_add_relu", "probe", "choice"],
                     help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
                          "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
                          "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
@@ -178,7 +181,7 @@ def main():
               "(no collectives); run it with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
-    if args.only is None and not args.skip_secondary:
+    if args.only is None and not args.skip_secondary and not args.no_power:
         start_power_sampler()
 
     import numpy as np
@@ -334,10 +337,10 @@ def main():
         print(json.dumps({"only": args.only, "launches": args.steps, "shape": [11008, 4096], "axis": 0}))
         return
 
-    if args.only in ("decode", "rows64", "c1"):
-        # config 4 at M = 1, or 64 rows against the same weights: 40 packed weights in turn (cold);
-        # config 1 (M = 128, K = N = 1024) likewise; plain launches
-        Mo, Ko = {"decode": (1, 4096), "rows64": (64, 4096), "c1": (128, 1024)}[args.only]
+    if args.only in ("decode", "rows64", "rows256", "c1"):
+        # config 4 at M = 1, or 64 / 256 rows against the same weights: 40 packed weights in turn
+        # (cold); config 1 (M = 128, K = N = 1024) likewise; plain launches
+        Mo, Ko = {"decode": (1, 4096), "rows64": (64, 4096), "rows256": (256, 4096), "c1": (128, 1024)}[args.only]
         pws = [cabi.PackedLinear(torch.randint(-127, 128, (Ko, Ko), dtype=torch.int8, device=dev))
                for _ in range(40)]
         wsd = torch.rand(Ko, device=dev) * 0.002 + 0.001
@@ -763,11 +766,12 @@ def main():
                 "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
                 "algorithmic_bytes_per_launch": nbytes}
 
-        # ----------------------------- the same cold weights against a few dozen rows
-        # (32 x 32 / 32 x 64 tiles whose waves split K and take their weights through registers),
-        # with the vendor's int8 GEMM (torch._int_mm: int32 output, no requantisation) beside it
+        # ----------------------------- the same cold weights against a few dozen to a few hundred rows
+        # (32 x 32 / 32 x 64 / 64 x 64 tiles whose waves split K and take their weights through
+        # registers; 64 x 128 pipelined tiles at 512 rows), with the vendor's int8 GEMM
+        # (torch._int_mm: int32 output, no requantisation) beside it
         wts_mm = None
-        for Md in (64, 128):
+        for Md in (64, 128, 256, 512):
             xd = torch.randint(0, 256, (Md, Kd), dtype=torch.uint8, device=dev)
             yd = torch.empty((Md, Nd), dtype=torch.uint8, device=dev)
 
@@ -843,44 +847,48 @@ def main():
         log("[bench] linear M=256, K=11008, N=4096: split K against the single-launch kernel (8 weight sets, HIP graph)")
         Ms, Ks, Ns = 256, 11008, 4096
         pws = [cabi.PackedLinear(torch.randint(-127, 128, (Ns, Ks), dtype=torch.int8, device=dev)) for _ in range(8)]
-        xs_ = torch.randint(0, 256, (Ms, Ks), dtype=torch.uint8, device=dev)
-        ys_ = torch.empty((Ms, Ns), dtype=torch.uint8, device=dev)
         cabi.linear_workspace = torch.empty(cabi.lib().tmq_linear_workspace_bytes(Ms, Ns, Ks), dtype=torch.uint8,
                                             device=dev)
-        split_us = {}
-        for use in (False, True):
-            cabi.use_linear_workspace = use
+        wts_mm = None
+        for Ms in (256, 64):
+            xs_ = torch.randint(0, 256, (Ms, Ks), dtype=torch.uint8, device=dev)
+            ys_ = torch.empty((Ms, Ns), dtype=torch.uint8, device=dev)
+            split_us = {}
+            for use in (False, True):
+                cabi.use_linear_workspace = use
 
-            def run_split_sets():
-                for p in pws:
-                    cabi.linear(xs_, p, 0.02, 128, wsd, bd, 0.05, 128, out=ys_)
+                def run_split_sets():
+                    for p in pws:
+                        cabi.linear(xs_, p, 0.02, 128, wsd, bd, 0.05, 128, out=ys_)
 
-            side = torch.cuda.Stream()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.stream(side):
-                run_split_sets()
-                side.synchronize()
-                with torch.cuda.graph(graph, stream=side):
-                    run_split_sets()
-            torch.cuda.synchronize()
-            for _ in range(3):
-                graph.replay()
-            ts = events_ms(graph.replay, 10)
-            split_us[use] = sum(ts) / len(ts) / len(pws) * 1e3
-        cabi.use_linear_workspace = True
+                split_us[use] = graph_us(run_split_sets, len(pws))
+            cabi.use_linear_workspace = True
+            vendor = None
+            try:
+                if wts_mm is None:
+                    wts_mm = [torch.randint(-127, 128, (Ns, Ks), dtype=torch.int8, device=dev).t() for _ in range(8)]
+                xs8 = torch.randint(-128, 128, (Ms, Ks), dtype=torch.int8, device=dev)
+                vendor = graph_us(lambda: [torch._int_mm(xs8, wt) for wt in wts_mm], len(wts_mm))
+            except Exception as ex:  # the comparison is optional
+                log(f"[bench] torch._int_mm not timed: {ex}")
+            ops_s = 2.0 * Ms * Ns * Ks
+            plan = cabi.linear_split_plan(Ms, Ns, Ks)
+            log(f"[bench] M={Ms}, K=11008, N=4096: {split_us[True]:.1f} us per call (split K, 2 launches), single "
+                f"launch {split_us[False]:.1f} us" + (f", torch._int_mm {vendor:.1f} us" if vendor else ""))
+            key = "linear_split_k_m256_k11008_n4096" if Ms == 256 else f"linear_m{Ms}_k11008_n4096"
+            secondary[key] = {
+                "avg_call_us": round(split_us[True], 2), "single_launch_us": round(split_us[False], 2),
+                "torch_int_mm_us": None if vendor is None else round(vendor, 2),
+                "value": round(ops_s / (split_us[True] * 1e-6) / 1e12, 1), "unit": "TOP/s",
+                "method": f"8 distinct packed weights replayed back to back in one HIP graph; {plan[0]} splits of "
+                          f"{plan[1]} stages, int32 partial sums in a shared workspace; the vendor GEMM the same way "
+                          "(int32 output, no requantisation)"}
         cabi.linear_workspace = None
-        ops_s = 2.0 * Ms * Ns * Ks
-        log(f"[bench] split K: {split_us[True]:.1f} us per call (2 launches), single launch {split_us[False]:.1f} us")
-        secondary["linear_split_k_m256_k11008_n4096"] = {
-            "avg_call_us": round(split_us[True], 2), "single_launch_us": round(split_us[False], 2),
-            "value": round(ops_s / (split_us[True] * 1e-6) / 1e12, 1), "unit": "TOP/s",
-            "method": "8 distinct packed weights replayed back to back in one HIP graph; 4 splits of 43 stages, "
-                      "16.8 MB of int32 partial sums in a shared workspace"}
-        del pws, xs_, ys_
+        del pws, xs_, ys_, wts_mm
 
         # ------------------------------------------- dynamically quantized linear
         # quantized::linear_dynamic at config 3's shape: fp32 in, min/max + qparams +
-        # quantize + int8 product + fp32 out, five launches, no host round trip
+        # quantize + int8 product + fp32 out: three launches (range, codes, product), no host round trip
         log("[bench] linear_dynamic at config 3's shape (fp32 in, fp32 out)")
         xds = [torch.randn(M, K, device=dev) for _ in range(2)]
         dcount = [0]

@@ -102,7 +102,7 @@ int tmq_quantize_per_tensor_dev(const float* x, void* q, int64_t n,
                                 tmq_stream_t stream);
 /* The whole dynamic quantization on the device: min/max over x, the parameters
  * into *qparams (device memory), the codes into q.  Small inputs (at most
- * 65536 elements) take one launch, inputs of up to 2**25 elements two (the
+ * 32768 elements) take one launch, inputs of up to 2**25 elements two (the
  * quantizer's workgroups finish the range reduction themselves), larger or
  * unaligned ones three; `workspace` as for tmq_minmax (unused, and may be NULL,
  * for the small case).

@@ -331,7 +331,7 @@ def test_qadaptive_avgpool_resnet_head_sized(cabi):
     np.testing.assert_array_equal(y, oracle.qadaptive_avgpool2d(x, (1, 1), 128))
 
 
-@pytest.mark.parametrize("n,offset", [(1, 0), (7, 0), (4096, 0), (4099, 1), (65536, 0), (65537, 0), (65541, 3),
+@pytest.mark.parametrize("n,offset", [(1, 0), (7, 0), (4096, 0), (4099, 1), (32768, 0), (32769, 0), (32772, 0), (65541, 3),
                                       (1 << 20, 0), ((1 << 20) + 3, 1), ((1 << 23) + 1029, 0), ((1 << 25) + 4, 0)])
 @pytest.mark.parametrize("signed,reduce_range", [(False, False), (False, True), (True, False)])
 def test_quantize_dynamic_on_device(cabi, n, offset, signed, reduce_range):
@@ -350,7 +350,7 @@ def test_quantize_dynamic_on_device(cabi, n, offset, signed, reduce_range):
     np.testing.assert_array_equal(host(q), oracle.quantize_per_tensor(x[offset:], scale, zp, signed, nthreads=8))
 
 
-@pytest.mark.parametrize("n,offset", [(4099, 1), (65536, 0), ((1 << 22) + 3, 0), ((1 << 23) + 1029, 0)])
+@pytest.mark.parametrize("n,offset", [(4099, 1), (32768, 0), (32772, 0), ((1 << 22) + 3, 0), ((1 << 23) + 1029, 0)])
 @pytest.mark.parametrize("signed", [False, True])
 def test_quantize_dynamic_fused_rounding(cabi, n, offset, signed):
     # the activation quantization of the CPU quantized::linear_dynamic: x * inv + zp
