@@ -925,14 +925,16 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
     const auto rows_used = [&](int bm) { return M * 20 >= ceil_div(M, bm) * bm * 11; };
     // One block of either large tile runs per CU, so a launch costs whole rounds
     // of 256 tiles.  The 128x256 tile (128 activation rows, 256 channels; 8 waves
-    // of 64x64) does half the work of a 256x256 tile in 0.56 of its time (C3:
+    // of 64x64) does half the work of a 256x256 tile in 0.56-0.58 of its time (C3:
     // 178.8 against 159.4 us) and wins where it rounds better: M = 2048, N = 11008:
     // 95.4 against 103.3 us; M = 2048, N = 4096: 35.9 against 41.5 us (and 41.3 us
     // for 128x128 tiles).  Its mirror image, 256 rows x 128 channels, is 17 %
     // slower than 256x256 at C3: activation rows arrive as 64-byte pieces of
     // far-apart rows, weight rows as 256-byte pieces of the packed layout.
     const double rounds256 = static_cast<double>(ceil_div(nblk(256, 256), 256));
-    const double rounds128x256 = 0.56 * static_cast<double>(ceil_div(nblk(128, 256), 256));
+    // (0.58 since the persistent schedule: M = 5120, N = 11008, four rounds against seven: 207
+    // against 217 us; M = 1536: 93.3 against 86.1 us, two rounds against three)
+    const double rounds128x256 = 0.58 * static_cast<double>(ceil_div(nblk(128, 256), 256));
     // (its activation copies two stages wide pay within one round of tiles only: M = 512, N = 11008:
     // 36.3 -> 32.7 us, but M = 1024, N = 11008: 53.0 -> 57.7 us)
     const int cfg128x256 = nblk(128, 256) <= 256 ? 19 : 17;
