@@ -32,7 +32,20 @@ def _same_q(got, ref, what):
     assert n == 0, f"{what}: {n} of {ref.numel()} codes differ"
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3])
+def _close_q(got, ref, inp, what):
+    """As _same_q, for the two activations of a quantized tensor `inp` that the CPU evaluates in
+    float32 vector arithmetic and the GPU once per input code in double precision: the output of
+    an input code whose exact value lies next to a rounding boundary may differ by 1 -- for every
+    element that holds that code, so the bound is on input codes, not on elements."""
+    assert got.is_cuda and got.shape == ref.shape and got.dtype == ref.dtype, what
+    assert got.q_scale() == ref.q_scale() and got.q_zero_point() == ref.q_zero_point(), what
+    d = (got.int_repr().cpu().int() - ref.int_repr().int()).abs()
+    assert int(d.max()) <= 1, f"{what}: a code differs by {int(d.max())}"
+    codes = torch.unique(inp.int_repr().cpu()[d != 0])
+    assert codes.numel() <= 4, f"{what}: the outputs of {codes.numel()} input codes differ"
+
+
+@pytest.mark.parametrize("seed", list(range(1, 13)))
 def test_linear_ops(seed):
     rng = np.random.default_rng(seed)
     done = 0
@@ -67,7 +80,7 @@ def test_linear_ops(seed):
     assert done >= 25
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3])
+@pytest.mark.parametrize("seed", list(range(1, 13)))
 def test_conv_and_glue_ops(seed):
     rng = np.random.default_rng(100 + seed)
     done = 0
@@ -109,8 +122,8 @@ def test_conv_and_glue_ops(seed):
                     what + " max_pool2d")
         _same_q(torch.nn.functional.adaptive_avg_pool2d(got, (1, 1)),
                 torch.nn.functional.adaptive_avg_pool2d(ref, (1, 1)), what + " adaptive_avg_pool2d")
-        _same_q(torch.nn.functional.gelu(got), torch.nn.functional.gelu(ref), what + " gelu")
-        _same_q(torch.sigmoid(got), torch.sigmoid(ref), what + " sigmoid")
+        _close_q(torch.nn.functional.gelu(got), torch.nn.functional.gelu(ref), ref, what + " gelu")
+        _close_q(torch.sigmoid(got), torch.sigmoid(ref), ref, what + " sigmoid")
         _same_q(torch.ops.quantized.cat([got, got2], 1, out_scale * 1.5, 90),
                 torch.ops.quantized.cat([ref, ref2], 1, out_scale * 1.5, 90), what + " cat")
         done += 1
