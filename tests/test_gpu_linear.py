@@ -174,6 +174,27 @@ def test_weights_through_registers_kernel(cabi, shape, x_signed, cfg):
     np.testing.assert_array_equal(acc1, acc)
 
 
+# K beyond 4096 on one round of 64 x 64 tiles whose last row tile is nearly full: the automatic
+# choice is the kernel that walks K through LDS as a ring of 256-byte phases (K that ends inside
+# a phase and on an odd 16-byte chunk, ragged channels, both activation types)
+@pytest.mark.parametrize("shape, x_signed", [((64, 4500, 8208), False), ((128, 1000, 5136), True),
+                                             ((48, 4200, 4112), False), ((113, 130, 4112), True)])
+def test_long_k_as_a_ring_of_phases(cabi, shape, x_signed):
+    say("ring of phases", shape, x_signed)
+    M, N, K = shape
+    assert cabi.linear_kernel_choice(M, N, K)["kernel"] - 1 == 21
+    c = _tile_case(M, N, K, seed=3300 + M, x_signed=x_signed, relu=N % 2 == 1, bias=M % 3 != 0,
+                   per_channel=(M + N) % 2 == 0)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "ring of phases")
+    y2, acc2, _ = _run(cabi, c, 2)
+    np.testing.assert_array_equal(y2, y)
+    np.testing.assert_array_equal(acc2, acc)
+
+
 def test_small_batch_kernels_on_random_shapes(cabi):
     """The kernels that hold or stream all of K (64 x 64 and 32 x 32 tiles in LDS, 32-row tiles
     with weights through registers) against the pipelined 64 x 64 tiles on seeded random shapes

@@ -618,19 +618,23 @@ constexpr int64_t kSplitBlocks = 256;    // blocks wanted: one per CU
 constexpr int64_t kSplitMinKT = 128;     // shortest k loop (stages) worth cutting
 constexpr int64_t kSplitMinStages = 16;  // shortest run of stages per split
 
-// ---- 17 ... 64 rows: three kernels can run such a product, and which is fastest
+// ---- 17 ... 64 rows: several kernels can run such a product, and which is fastest
 // depends on the shape.  Estimated microseconds per launch, fitted to sweeps with
 // cold weights (more weight sets in rotation than the last-level cache holds):
-//  * the weight-streaming kernel re-reads all M x K activation bytes in every
-//    block of 16 channels, so its time grows with rows x blocks x K, the bytes
-//    the L2s hand out (K = N = 4096: 5.9 / 7.8 / 12.2 us at M = 16 / 32 / 64;
-//    N = 11008, K = 4096: 12.6 / 18.9 / 32.3 us);
+//  * the weight-streaming kernel: a block of 16 channels streams its K x 16 weight
+//    bytes once and re-reads the activations of every group of 16 rows, so one round
+//    of blocks (N <= 4096) costs a base that grows with the weight bytes plus a share
+//    per row group that grows with K (K = N = 4096: 6.4 / 7.5 / 11.3 us at M = 17 / 32 / 64;
+//    N = 4096, K = 8192: 10.2 / 12.2 / 18.8 us), and further rounds cost about three
+//    quarters of the first (N = K = 8192, two rounds: 19.2 / 20.9 / 34.8 us; N = 11008,
+//    K = 4096, three rounds: 15.1 / 16.3 / 28.1 us);
 //  * 64 x 64 tiles walk K at the latency of one stage after the other, almost
-//    whatever M is (K = N = 4096 with two wave groups: 12.8 / 14.8 us at
-//    M = 32 / 64; N = 11008: 14.9 / 16.8 us), and K <= 1024 fits LDS whole
-//    (gemm_i8_onepass.h: K = N = 1024: 3.8 us on 32 x 32 tiles);
-//  * split K moves the weights at about 3.4 TB/s plus 8 us for the partial sums
-//    (N = 4096, K = 11008: 21.7 us at M = 65 against 30.6 us streaming at M = 64).
+//    whatever M is (K = N = 4096 with two wave groups: 12.6 / 14.3 us at
+//    M = 32 / 64; N = 11008: 14.6 / 16.9 us), and K <= 1024 fits LDS whole
+//    (gemm_i8_onepass.h: K = 1024 on 32 x 32 tiles: 3.8 / 4.1 / 4.9 us at N = 1024 / 4096 / 8192);
+//  * split K moves the weights at about 4.5 TB/s plus 10 us for the partial sums
+//    (N = 4096, K = 11008: 21.7 us at M = 64 against 27.0 us streaming; K = 8192, M = 48:
+//    18.0 against 15.5 us streaming).
 enum class SmallRows { kStream, kTiles, kSplit };
 
 bool two_wave_groups_fit(int64_t M, int64_t N, int64_t K) {
@@ -657,42 +661,53 @@ int wstream_tile(int64_t M, int64_t N, int64_t K) {
   return 0;
 }
 
+// One round of 64 x 64 tiles against K > 4096 whose last row tile is at least three
+// quarters full, up to 128 rows: the kernel that copies K through LDS in phases takes the
+// same time whatever the rows (N = K = 5120: 17.1 ... 17.9 us from 40 to 128 rows; N = K = 8192:
+// 26.5 us at 64 rows), while two wave groups slow down as the tiles fill (20.9 us and 29.3 us
+// at 64 rows; N = 4096, K = 11008, M = 64: 32.2 against 37.3 us).  With a tile half empty, or
+// from 192 rows on, the wave groups are ahead (N = 4096, K = 14336, M = 256: 42.4 against 45.6 us).
+bool phased_ring_preferred(int64_t M, int64_t N, int64_t K) {
+  return K > 4096 && K % 16 == 0 && ceil_div(M, 64) * ceil_div(N, 64) <= 256 && M <= 128 && (M - 1) % 64 >= 47;
+}
+
 SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
   // Where the 32 x 32 tiles with the weights through registers fit, they are measured
-  // directly against the weight-streaming kernel (us at M = 17 / 32 / 64, tiles | streaming):
-  //   K = 2048, N = 4096:  5.4 / 5.4 / 5.5 | 6.2 / 6.9 / 9.4     K = 1280, N = 2048:  4.6 / 4.6 / 4.7 | 5.6 / 6.1 / 9.7
-  //   K = 4096, N = 4096:  8.2 / 8.3 / 8.6 | 6.8 / 7.8 / 12.2    K = 4096, N = 1024:  6.5 / 6.5 / 6.6 | 6.0 / 7.0 / 11.3
-  //   K = 3072, N = 4096:  7.2 / 7.3 / 7.6 | 6.4 / 7.5 / 11.7    K = 4096, N = 8192: 10.6 / 10.7 / -  | 11.7 / 13.6 / 22.6
-  // streaming keeps the longer K up to about two dozen rows while its blocks fit one round.
-  // (K = N = 4096, M = 32: 7.6 against 8.5 us, so the longest K streams up to 32 rows there;
-  // at K = 3072, or against N = 1024, the tiles are ahead from 25 rows on)
-  if (wstream_tile(M, N, K) != 0) {
-    const int64_t stream_rows = K > 3072 && N >= 2048 ? 32 : 24;
-    return K > 2048 && M <= stream_rows && N <= 4096 ? SmallRows::kStream : SmallRows::kTiles;
-  }
+  // directly against the weight-streaming kernel (us at M = 17 / 32 / 40 / 64, tiles | streaming):
+  //   K = 2048, N = 4096:  5.2 / 5.4 / 5.5 / 5.5 | 5.7 / 5.9 / 7.2 / 9.3    K = 4096, N = 1024:  6.7 / 6.7 / 6.7 / 6.7 | 5.3 / 5.5 / 6.9 / 8.6
+  //   K = 4096, N = 4096:  8.4 / 8.5 / 8.6 / 8.7 | 6.4 / 7.5 / 8.6 / 11.3   K = 3072, N = 3072:  7.2 / 7.2 / 7.2 / 7.4 | 5.5 / 6.1 / 7.2 / 10.0
+  //   K = 3072, N = 4096:  7.4 / 7.4 / 7.5 / 7.7 | 5.9 / 6.5 / 7.7 / 10.9   K = 4096, N = 8192: 10.8 / 10.9 / -   / -   | 11.1 / 12.2 / 14.5 / 20.6
+  // streaming keeps K > 2048 up to 32 rows (two row groups) while its blocks fit one round.
+  if (wstream_tile(M, N, K) != 0)
+    return K > 2048 && M <= 32 && N <= 4096 ? SmallRows::kStream : SmallRows::kTiles;
   const double mib = static_cast<double>(N) * static_cast<double>(K) / 1048576.0;
   const double stages = static_cast<double>(ceil_div(K, kBK));
   const double rows = static_cast<double>(M);
-  const double l2_mib_per_row = static_cast<double>(ceil_div(N, 16)) * static_cast<double>(K) / 1048576.0;
-  const double stream_blocks = static_cast<double>(ceil_div(N, 16));
-  const double stream = 2.4 + 0.11 * mib + 0.4 * mib / 16.0 +
-                        rows * std::max(0.10 * std::max(1.0, stream_blocks / 256.0), 0.135 * l2_mib_per_row);
+  const double kk = static_cast<double>(K) / 1024.0;
+  const double stream_rounds = static_cast<double>(ceil_div(ceil_div(N, 16), 256));
+  const double round_mib = static_cast<double>(std::min<int64_t>(N, 4096)) * static_cast<double>(K) / 1048576.0;
+  const double one_round = 1.9 + 0.09 * round_mib + static_cast<double>(ceil_div(M, 16)) * std::max(1.6, 0.42 * kk);
+  const double stream = stream_rounds <= 1.0 ? one_round : one_round * (0.3 + 0.75 * stream_rounds);
   const double nblk = static_cast<double>(ceil_div(M, 64) * ceil_div(N, 64));
   double tiles;
   if (K <= kOnePassMaxK && K > 256 && ceil_div(M, 32) * ceil_div(N, 32) <= 512)
-    // all of K in LDS, 32 x 32 tiles (K = N = 1024: 3.8 us, K = N = 512: 3.2 us, N = 4096, K = 512: 3.9 us)
-    tiles = 3.0 + 0.6 * mib + (ceil_div(M, 32) * ceil_div(N, 32) > 256 ? 0.5 : 0.0);
+    // all of K in LDS, 32 x 32 tiles (K = 1024: 3.8 / 3.8 / 4.1 / 4.9 us at N = 1024 / 2048 / 4096 / 8192;
+    // more than 256 tiles, N = 8192, M = 40: 5.4 us)
+    tiles = 3.6 + 0.13 * mib + (ceil_div(M, 32) * ceil_div(N, 32) > 256 ? 0.5 : 0.0);
   else if (K <= kOnePassMaxK && nblk <= 256.0)  // 64 x 64 tiles (K = N = 1024: 5.6 us, N = 1024, K = 256: 3.1 us)
-    tiles = 2.0 + 3.8 * static_cast<double>(K) / 1024.0 + 0.012 * std::max(0.0, nblk - 64.0);
-
+    tiles = 2.0 + 3.8 * kk + 0.012 * std::max(0.0, nblk - 64.0);
+  else if (phased_ring_preferred(M, N, K))
+    // (N = 4096: 25.3 / 32.2 / 40.9 us at K = 8192 / 11008 / 14336; N = K = 5120: 17.4 us; N = K = 8192: 26.5 us)
+    tiles = 3.3 + 2.65 * kk + 0.2 * std::max(0.0, static_cast<double>(N) - 4096.0) / 1024.0;
   else if (two_wave_groups_fit(M, N, K))
     tiles = (4.4 + 0.123 * stages + 0.013 * std::max(0.0, nblk - 64.0)) *
             (1.0 + 0.35 * (rows / 64.0) * (rows / 64.0) * std::min(1.0, stages / 172.0));
   else
     tiles = (3.0 + 0.2 * stages) * (1.0 + nblk / 1024.0);
-  double best = std::min(stream, tiles);
+  const double best = std::min(stream, tiles);
   if (workspace && plan_split_tiles(M, N, K).splits > 1) {
-    const double split = 8.0 + 0.295 * mib + 0.02 * rows;
+    // (N = 4096: 18.0 / 21.3 / 23.5 us at K = 8192 / 11008 / 14336, 48 rows)
+    const double split = 10.0 + 0.23 * mib + 0.025 * rows;
     if (split < best) return SmallRows::kSplit;
   }
   return stream <= tiles ? SmallRows::kStream : SmallRows::kTiles;
@@ -915,40 +930,49 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
     // K = N = 2048: M = 128 7.8 -> 5.0 us, M = 256 8.0 -> 6.3 us)
     cfg = wstream_tile(M, N, K) == 32 ? 25 : 26;
   } else if (cfg < 0) {
-    // Thresholds from timing sweeps over M, N, K on the chip (256 CUs): the
-    // 256x256 tile (one block per CU) wins once it keeps about two thirds of
-    // the CUs busy, the 128x128 tile (two blocks per CU) down to 128 tiles.
+    // Thresholds from timing sweeps over M, N, K on the chip (256 CUs, cold weights): the
+    // 256x256 tile (one block per CU) wins from 129 tiles on, the 128x256 tile while
+    // it fits one round, the 128x128 tile (two blocks per CU) down to 128 tiles.
     const auto nblk = [&](int bm, int bn) { return ceil_div(M, bm) * ceil_div(N, bn); };
     // (and only when the rows fill at least 55 % of the row tiles: a tile's time
     // does not shrink with its padding; M = 100 and 150 against N = 49152 sit on
     // either side)
     const auto rows_used = [&](int bm) { return M * 20 >= ceil_div(M, bm) * bm * 11; };
-    // One block of either large tile runs per CU, so a launch costs whole rounds
-    // of 256 tiles.  The 128x256 tile (128 activation rows, 256 channels; 8 waves
-    // of 64x64) does half the work of a 256x256 tile in 0.56-0.58 of its time (C3:
-    // 178.8 against 159.4 us) and wins where it rounds better: M = 2048, N = 11008:
-    // 95.4 against 103.3 us; M = 2048, N = 4096: 35.9 against 41.5 us (and 41.3 us
-    // for 128x128 tiles).  Its mirror image, 256 rows x 128 channels, is 17 %
-    // slower than 256x256 at C3: activation rows arrive as 64-byte pieces of
-    // far-apart rows, weight rows as 256-byte pieces of the packed layout.
-    const double rounds256 = static_cast<double>(ceil_div(nblk(256, 256), 256));
-    // (0.58 since the persistent schedule: M = 5120, N = 11008, four rounds against seven: 207
-    // against 217 us; M = 1536: 93.3 against 86.1 us, two rounds against three)
-    const double rounds128x256 = 0.58 * static_cast<double>(ceil_div(nblk(128, 256), 256));
-    // (its activation copies two stages wide pay within one round of tiles only: M = 512, N = 11008:
-    // 36.3 -> 32.7 us, but M = 1024, N = 11008: 53.0 -> 57.7 us)
-    const int cfg128x256 = nblk(128, 256) <= 256 ? 19 : 17;
-    if (nblk(256, 256) >= 160 && rows_used(256))
-      cfg = rounds128x256 < rounds256 ? cfg128x256 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
-    else if (nblk(128, 256) >= 160 && rows_used(128))
-      cfg = cfg128x256;
+    // One block of either large tile runs per CU.  The 128x256 tile (128 activation rows,
+    // 256 channels; 8 waves of 64x64) keeps a single round to itself (M = 2048, N = 4096,
+    // 256 tiles: 34.4 us against 40.1 us for 128 tiles of 256x256); once it needs a second
+    // round the 256x256 tiles take over (M = 768, N = 11008, 129 tiles: 43.4 against 49.4 us;
+    // M = 3072, K = N = 3072, 144 tiles: 34.3 against 39.1 us), except just past a full round
+    // of them, where the second round of 256x256 tiles is nearly empty and three rounds of
+    // 128x256 are shorter (258 tiles, M = 1536, N = 11008: 84.9 against 91.8 us; 344 tiles:
+    // 90.6 against 91.6 us; at 375 ... 384 tiles the two are within 4 % of each other, either
+    // way round from box to box; 430 tiles: 102.4 against 115.8 us; at 516 tiles, just past
+    // two rounds, the two are level: 146.8 against 146.3 us).  Its
+    // mirror image, 256 rows x 128 channels, is 17 % slower than 256x256 at C3: activation
+    // rows arrive as 64-byte pieces of far-apart rows, weight rows as 256-byte pieces of
+    // the packed layout.
+    const int64_t t256 = nblk(256, 256), t128x256 = nblk(128, 256);
+    // (the 128x256 tile's activation copies two stages wide pay within one round of tiles only:
+    // M = 512, N = 11008: 36.3 -> 32.7 us, but M = 1024, N = 11008: 53.0 -> 57.7 us)
+    const int cfg128x256 = t128x256 <= 256 ? 19 : 17;
+    // equal tile counts: the 64 x 128 tile; more row tiles than its mirror image has fewer
+    // blocks and idle CUs (M = 192: N = 6144, K = 3072: 17.1 against 15.3 us with 128 x 64;
+    // N = 4096, K = 11008: 46.8 against 43.4 us)
+    const int cfg_half = nblk(128, 64) <= 256 && nblk(128, 64) > nblk(64, 128) ? 22 : 23;
+    if (t128x256 > 256 && rows_used(256))
+      cfg = t256 > 256 && t256 <= 400 ? 17 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
+    else if (t128x256 >= 160 && rows_used(128))
+      // (barely more than half a round of them, against a long K: 128x128 tiles, at most 320,
+      // all resident at once: M = 640, N = K = 8192: 53.9 against 59.7 us; N = 8192, K = 4096:
+      // 30.2 against 31.6 us; at K = 2048 the 128x256 tiles stay ahead)
+      cfg = K >= 4096 && nblk(128, 128) <= 320 ? 7 : cfg128x256;
     else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && nblk(64, 128) <= 256)
       // a few hundred rows whose 128 x 128 tiles would leave half the chip idle and whose
       // 64 x 64 tiles need a second round: 64 rows x 128 channels, one round (K = N = 4096,
       // cold weights: M = 448: 24.6 -> 19.1 us, M = 512: 24.8 -> 19.3 us; K = 2048: 14.7 -> 11.7 us;
       // N = 8192, M = 192: 25.9 -> 19.9 us; against N = 1024 the 128 x 128 tiles stay ahead:
       // M = 1536, K = 4096: 17.4 against 20.2 us, and at K = N = 2048, M = 1024: 11.5 against 12.2 us)
-      cfg = 23;
+      cfg = cfg_half;
     else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
       cfg = 22;
     else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
@@ -961,6 +985,8 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
       // 13.0 -> 12.1 us; behind the two wave groups at K = 2560 (12.3 against 11.7 us) and
       // against 32 MB of weights, N = 8192: 15.3 against 14.6 us)
       cfg = 27;
+    else if (onepass_ok && phased_ring_preferred(M, N, K))
+      cfg = 21;
     else if (nblk(64, 64) <= 256 && ceil_div(K, kBK) >= 32 && ceil_div(K, kBK) % 2 == 0)
       cfg = 14;  // at most one block per CU and a long k loop: two wave groups halve it (14.7 -> 11.7 us
                  // at M = 128, K = N = 4096; four groups run into the L2's bandwidth: 12.3 us)
