@@ -182,6 +182,14 @@ def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256
         assert k <= 4096 and (bm, bn) == (64, 64) and c["waves"] == 8 and 64 * ldx <= 2 ** 29, what
         if forced == 0:                             # one round, and a K long enough to fill the waves' shares
             assert k >= 3072 and tiles <= 256, what
+    elif cfg == 28:                                 # activations resident in LDS: 16 MG x K bytes, K padded to 16 k-blocks,
+        mg = _ceil(m, 16)                           # in 128 KB; the constants of at most 64 channel groups per block
+        assert m <= 64 and (bm, bn) == (16 * mg, 16) and c["waves"] == 16, what
+        assert 16 * mg * _ceil(k, 1024) * 1024 <= 128 * 1024 and _ceil(n, 16) <= 64 * cus, what
+        assert c["blocks"] == min(tiles, cus), what
+        if forced == 0:                             # rows that share the streamed weights, or a short K
+            assert k >= 1024 and ((m <= 16 and (k <= 2048 or m >= 12)) or n >= 98304), what
+        return
     else:                                           # register-staged tiles take any aligned shape
         assert cfg in (0, 1, 2, 3, 4, 5, 22, 23), what
     if forced == 0 and cfg in (22, 23):             # a few hundred rows: one round of oblong tiles
@@ -225,7 +233,7 @@ def test_automatic_kernel_choice_keeps_every_kernels_preconditions():
             seen.add(c["kernel"] - 1)
     c = cabi.linear_kernel_choice(300, 500, 4096, misaligned=True)
     assert c["kernel"] == 10
-    assert seen >= {2, 3, 7, 8, 9, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26, 27}, sorted(seen)
+    assert seen >= {2, 3, 7, 8, 9, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28}, sorted(seen)
     # the benchmark configurations
     assert cabi.linear_kernel_choice(4096, 11008, 4096)["kernel"] - 1 == 20
     assert cabi.linear_kernel_choice(4096, 11008, 4096)["blocks"] == 256
@@ -241,7 +249,7 @@ def test_forced_kernels_run_inside_their_preconditions_or_not_at_all():
     rng = np.random.default_rng(21)
     refused = 0
     for m, n, k, ldx in _random_linear_shapes(rng, 1500):
-        for cfg in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26, 27):
+        for cfg in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28):
             for out in ("bytes", "acc32"):
                 c = cabi.linear_kernel_choice(m, n, k, ldx, out, workspace=True, forced=cfg + 1)
                 if c["kernel"] == 0:

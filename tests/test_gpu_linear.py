@@ -195,6 +195,39 @@ def test_long_k_as_a_ring_of_phases(cabi, shape, x_signed):
     np.testing.assert_array_equal(acc2, acc)
 
 
+# up to 64 rows with the activations resident in LDS, one block per CU walking its channel groups:
+# one group and several per block (ragged last round), K that ends inside a k-block / inside the
+# padding to 16 k-blocks, every number of row groups, a single row, both activation types
+@pytest.mark.parametrize("shape, x_signed", [((16, 4113, 1024), False), ((1, 100, 1040), True), ((13, 12300, 1024), False),
+                                             ((32, 1000, 2048), True), ((64, 300, 1040), False), ((9, 5000, 8192), True),
+                                             ((40, 530, 2048), False), ((12, 8200, 4112), True)])
+def test_activations_resident_in_lds(cabi, shape, x_signed):
+    say("resident activations", shape, x_signed)
+    M, N, K = shape
+    assert cabi.linear_kernel_choice(M, N, K, forced=29)["kernel"] == 29
+    c = _tile_case(M, N, K, seed=2800 + M, x_signed=x_signed, relu=N % 2 == 1, bias=M % 3 != 0,
+                   per_channel=(M + N) % 2 == 0)
+    y, acc, pw = _run(cabi, c, 28)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "resident activations")
+    # the float output against the streaming kernel's, and the automatic choice, whichever kernel it is
+    ws = dev(c["w_scales"].astype(np.float32))
+    b = None if c["bias"] is None else dev(c["bias"])
+    f = {}
+    for cfg in (28, 8):
+        cabi.force_linear_config(cfg)
+        try:
+            f[cfg] = cabi.linear_f32(dev(c["xq"]), pw, c["x_scale"], c["x_zp"], ws, b, relu=c["relu"])
+        finally:
+            cabi.force_linear_config(-1)
+    assert torch.equal(f[28], f[8])
+    y1, acc1, _ = _run(cabi, c)
+    np.testing.assert_array_equal(y1, y)
+    np.testing.assert_array_equal(acc1, acc)
+
+
 def test_small_batch_kernels_on_random_shapes(cabi):
     """The kernels that hold or stream all of K (64 x 64 and 32 x 32 tiles in LDS, 32-row tiles
     with weights through registers) against the pipelined 64 x 64 tiles on seeded random shapes
@@ -226,7 +259,8 @@ def test_small_batch_kernels_on_random_shapes(cabi):
                 cabi.force_linear_config(-1)
 
         want = run(2)
-        for cfg in [c for c in (21, 24, 25, 26, 27, -1) if not (c == 24 and K > 1024)]:
+        fits28 = cabi.linear_kernel_choice(M, N, K, forced=29)["kernel"] == 29
+        for cfg in [c for c in (21, 24, 25, 26, 27, 28, -1) if not (c == 24 and K > 1024) and not (c == 28 and not fits28)]:
             for got, ref, what in zip(run(cfg), want, ("bytes", "accumulators", "float output")):
                 assert torch.equal(got, ref), f"cfg {cfg} {what} at {(M, N, K)}"
 

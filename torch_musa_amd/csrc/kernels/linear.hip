@@ -7,6 +7,7 @@
 #include "gemm_i8_onepass.h"
 #include "gemm_i8_persistent.h"
 #include "gemm_i8_wring.h"
+#include "linear_resident.h"
 #include "qparams.h"
 
 // Layout that non-C++ bindings rely on (natural alignment, x86-64).
@@ -599,6 +600,49 @@ int launch_gemm_persistent(const GemmArgs& a, const XLinear& xs, hipStream_t s) 
   }
 }
 
+// Weight streaming for up to 64 rows: one block per 16 channels.
+template <int MODE>
+int launch_linear_decode(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  // (the kernel derives the packed pitch from K, as prepack does)
+  if (a.w_kchunks != packed_kchunks(a.K)) return TMQ_ERR_UNSUPPORTED;
+  const dim3 grid(static_cast<unsigned>(ceil_div(a.N, 16))), block(kDecodeWaves * kWave);
+  const int32_t k32 = static_cast<int32_t>(a.K), ldx32 = static_cast<int32_t>(xs.ldx);
+  const int32_t n32 = static_cast<int32_t>(a.N);
+  const uint32_t flags = static_cast<uint32_t>(a.M) | (a.w_scale_stride != 0 ? 0x100u : 0u) |
+                         (a.x_xor != 0 ? 0x200u : 0u);
+  switch ((a.M + 15) / 16) {
+    case 1: linear_decode_kernel<MODE, 1><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+    case 2: linear_decode_kernel<MODE, 2><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+    case 3: linear_decode_kernel<MODE, 3><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+    default: linear_decode_kernel<MODE, 4><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
+  }
+  return launch_status();
+}
+
+// Up to 64 rows whose activations (16 MG x K bytes, MG = groups of 16 rows) fit the
+// kernel's LDS area: one block per CU streams the channel groups it owns.
+bool resident_limits_ok(int64_t M, int64_t N, int64_t K, int64_t ldx, int cus) {
+  if (M < 1 || M > 64 || K < 64 || K % 16 != 0 || cus < 1) return false;
+  const int64_t mg = ceil_div(M, 16), groups = ceil_div(N, 16);
+  return 16 * mg * ceil_div(K, 64 * kResidentWaves) * (64 * kResidentWaves) <= kResidentXBytes && groups <= static_cast<int64_t>(kResidentMaxGroups) * cus &&
+         N <= 0x7ffffff0 && ldx <= (int64_t{1} << 40);
+}
+
+template <int MODE>
+int launch_linear_resident(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
+  const int cus = cu_count();
+  if (!resident_limits_ok(a.M, a.N, a.K, xs.ldx, cus)) return TMQ_ERR_UNSUPPORTED;
+  const int64_t groups = ceil_div(a.N, 16);
+  const dim3 grid(static_cast<unsigned>(groups < cus ? groups : cus)), block(kResidentThreads);
+  switch ((a.M + 15) / 16) {
+    case 1: linear_resident_kernel<MODE, 1><<<grid, block, 0, s>>>(a, xs); break;
+    case 2: linear_resident_kernel<MODE, 2><<<grid, block, 0, s>>>(a, xs); break;
+    case 3: linear_resident_kernel<MODE, 3><<<grid, block, 0, s>>>(a, xs); break;
+    default: linear_resident_kernel<MODE, 4><<<grid, block, 0, s>>>(a, xs); break;
+  }
+  return launch_status();
+}
+
 // ---- split K for a few hundred rows against a long K.  The tile grid of such a
 // product is far smaller than the chip (M = 128, N = 4096: 32 tiles of
 // 128 x 128) and every block walks all of K alone at the latency of one stage
@@ -865,7 +909,8 @@ struct LinearQuery {
 // streaming; 9: plain kernel; 13: split K (plan in `split`); 20: persistent 256 x 256 tiles;
 // 21 / 24: all of K in LDS (64 x 64 / 32 x 32 tiles); 25 / 26: weights through registers
 // (32 x 32 / 32 x 64 tiles); 27: the same with 64 x 64 tiles and the activations in a ring
-// per wave; kNoKernel: the forced kernel does not take this shape.
+// per wave; 28: activations resident in LDS, one block per CU streams its channel groups;
+// kNoKernel: the forced kernel does not take this shape.
 constexpr int kNoKernel = -2;
 struct LinearChoice {
   int cfg = kNoKernel;
@@ -889,11 +934,32 @@ bool stream_limits_ok(const LinearQuery& q) {
          q.N <= 0x7ffffff0;
 }
 
+// Where the kernel that keeps the activations in LDS is ahead of a block per 16 channels
+// (cold weights, us, resident | streaming; neither depends on N beyond what is shown):
+//   K <= 2048, from N = 4096 on, any M <= 16:  N = 4096, K = 1024: 3.9 | 4.2 ... 4.5;  N = 8192, K = 1024:
+//     4.8 ... 5.0 | 5.8 ... 6.3;  N = 4096, K = 2048: 4.5 | 4.7 ... 5.0;  N = 65536, K = 2048: 24.5 | 35 ... 42
+//   longer K, 12 rows and more (the streaming blocks re-read the rows from the L2s), from N = 5120 on:
+//     K = 4096, M = 16: N = 5120 7.7 | 8.6, N = 11008 10.6 | 12.3, N = 32000 25.4 | 32.2, N = 128256 97 | 122;
+//     M = 12: N = 49152 38.2 | 39.6, N = 65536 50.3 | 54.4;  N = K = 8192, M = 16: 14.7 | 16.1
+//   (M <= 8 at K = 4096: level up to N = 32000, then the independent blocks stream faster: N = 128256,
+//   M = 1: 91 | 85; N = 4096 at K >= 4096: level or behind, 6.1 | 5.9 at M = 16)
+//   17 ... 32 rows against the largest N only (N = 128256, K = 4096: 104 against 111 us for 128 x 128 tiles;
+//   N = 32000: 27 against 25.4 us for 64 x 128 tiles).
+bool resident_preferred(const LinearQuery& q) {
+  if (!q.vec_ok || q.K < 1024 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
+  if (q.M <= 16) return q.K <= 2048 ? q.N >= 4096 : (q.M >= 12 && q.N >= 5120);
+  return q.M <= 32 && q.N >= 98304;
+}
+
 // forced: tmq_linear_desc::kernel - 1 (-1 = automatic choice).
 LinearChoice choose_linear(const LinearQuery& q, int forced) {
   LinearChoice c;
   if (!q.vec_ok || forced == 9) {
     c.cfg = 9;
+    return c;
+  }
+  if (forced < 0 && resident_preferred(q)) {
+    c.cfg = 28;
     return c;
   }
   const bool stream_auto =
@@ -1023,6 +1089,9 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
     case 27:
       if (!onepass_ok || K > kWringMaxK) cfg = kNoKernel;
       break;
+    case 28:
+      if (!resident_limits_ok(M, N, K, q.ldx, 256)) cfg = kNoKernel;
+      break;
     default:
       cfg = kNoKernel;
   }
@@ -1059,21 +1128,11 @@ int dispatch_linear(const GemmArgs& a, const XLinear& xs, int x_signed, bool vec
       linear_plain_kernel<MODE><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(b, xs, x_signed);
       return launch_status();
     }
-    case 8: {
-      // (the kernel derives the packed pitch from K, as prepack does)
-      if (a.w_kchunks != packed_kchunks(a.K)) return TMQ_ERR_UNSUPPORTED;
-      const dim3 grid(static_cast<unsigned>(ceil_div(a.N, 16))), block(kDecodeWaves * kWave);
-      const int32_t k32 = static_cast<int32_t>(a.K), ldx32 = static_cast<int32_t>(xs.ldx);
-      const int32_t n32 = static_cast<int32_t>(a.N);
-      const uint32_t flags = static_cast<uint32_t>(a.M) | (a.w_scale_stride != 0 ? 0x100u : 0u) |
-                             (a.x_xor != 0 ? 0x200u : 0u);
-      switch ((a.M + 15) / 16) {
-        case 1: linear_decode_kernel<MODE, 1><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-        case 2: linear_decode_kernel<MODE, 2><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-        case 3: linear_decode_kernel<MODE, 3><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-        default: linear_decode_kernel<MODE, 4><<<grid, block, 0, s>>>(a.w_packed, xs.x, a.colsum, a.w_scales, a.bias, k32, ldx32, n32, flags, a); break;
-      }
-      return launch_status();
+    case 8: return launch_linear_decode<MODE>(a, xs, s);
+    case 28: {
+      const int rc = launch_linear_resident<MODE>(a, xs, s);
+      // (a device with too few CUs for this many channel groups: the automatic choice streams instead)
+      return rc == TMQ_ERR_UNSUPPORTED && forced < 0 && stream_limits_ok(q) ? launch_linear_decode<MODE>(a, xs, s) : rc;
     }
     case 13: return run_split<MODE>(a, xs, c.split, workspace, dma_limits_ok(a.K, xs.ldx), s);
     case 0: return launch_gemm<256, 256, 2, 2, MODE>(a, xs, s);
@@ -1219,6 +1278,7 @@ TMQ_EXPORT int tmq_linear_kernel_choice(int64_t M, int64_t N, int64_t K, int64_t
     case 26: bm = 32, bn = 64, waves = 8; break;
     case 27: bm = 64, bn = 64, waves = 8; break;
     case 8: bm = 16 * static_cast<int>(ceil_div(M, 16)), bn = 16, waves = kDecodeWaves; break;
+    case 28: bm = 16 * static_cast<int>(ceil_div(M, 16)), bn = 16, waves = kResidentWaves; break;
     default: break;  // 9: one thread per four outputs
   }
   out->kernel = c.cfg + 1;
@@ -1233,6 +1293,7 @@ TMQ_EXPORT int tmq_linear_kernel_choice(int64_t M, int64_t N, int64_t K, int64_t
     out->tiles = ceil_div(M, bm) * ceil_div(N, bn) * c.split.splits;
     out->blocks = out->tiles;
     if (c.cfg == 20 && out->tiles > compute_units) out->blocks = compute_units / 8 * 8;
+    if (c.cfg == 28 && out->tiles > compute_units) out->blocks = compute_units;
   }
   return TMQ_OK;
 }

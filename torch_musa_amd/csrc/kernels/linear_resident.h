@@ -1,0 +1,248 @@
+// quantized::linear for up to 64 activation rows against many output channels (gfx950):
+// one block per CU keeps the activations in LDS and streams the weights of one group
+// of 16 channels after the other through its sixteen waves.
+//
+// The weight-streaming kernel of linear.hip gives every group of 16 channels a block of
+// its own, and every block fetches all M x K activation bytes again from the L2s: at
+// M = 16 those are as many bytes as the block's weights, and with more blocks than the
+// chip holds at once each one starts its weight stream from nothing.  Here
+//   * the block stages the activations once, already in MFMA operand order
+//     ([k-block][16-byte piece][row][16 B], zeros past K: a wave's B operand of v_mfma_i32_16x16x64_i8
+//     is four contiguous runs of 256 bytes) and with the sign flip of unsigned
+//     activations applied, and the requantisation constants of every channel it owns
+//     (accumulator start, multiplier, bias term) next to them;
+//   * block b owns the channel groups b, b + G, b + 2 G, ...; the sixteen waves split
+//     the 64-byte k-blocks of a group (wave w takes k-blocks w, w + 16, ...) and a wave's
+//     loads run kDepth k-blocks ahead of its multiplications, across group boundaries,
+//     so the stream never drains;
+//   * the waves' partial sums of a group meet in LDS (atomic adds into one of two slots,
+//     used in turn), one barrier per group, then one wave -- a different one each
+//     group -- requantises and stores while the others go on multiplying.  The barrier
+//     carries no memory fence: only the LDS counter is waited for, the weight loads in
+//     flight stay in flight.
+// D[i][j] of v_mfma_i32_16x16x64_i8: lane l, register r -> i = 4 (l / 16) + r (channel),
+// j = l % 16 (activation row).
+#pragma once
+
+#include "gemm_i8_core.h"
+
+namespace tmq {
+
+constexpr int kResidentWaves = 16;
+constexpr int kResidentThreads = kResidentWaves * kWave;
+constexpr int kResidentDepth = 8;                 // k-blocks in flight per wave: 128 KB per block (12 and 16: no faster)
+constexpr int kResidentMaxGroups = 64;            // channel groups a block can own (their constants sit in LDS)
+constexpr int kResidentXBytes = 128 * 1024;       // 16 MG x K activation bytes
+
+// LDS barrier of the block without a fence: every wave's LDS operations so far are
+// complete before it arrives, global loads stay outstanding.
+__device__ __forceinline__ void resident_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <int MODE, int MG>
+__global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmArgs a, XLinear xs) {
+  constexpr int D = kResidentDepth;
+  __shared__ __attribute__((aligned(16))) uint8_t s_x[kResidentXBytes];
+  __shared__ __attribute__((aligned(16))) int s_sum[2][MG][4][kWave];
+  __shared__ __attribute__((aligned(16))) int s_acc0[kResidentMaxGroups * 16];
+  __shared__ __attribute__((aligned(16))) float s_mult[kResidentMaxGroups * 16];
+  __shared__ __attribute__((aligned(16))) float s_bdiv[kResidentMaxGroups * 16];
+  __shared__ float s_bmul;
+
+  const int t = threadIdx.x, lane = t % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(t / kWave);
+  const int lr = lane & 15, lc = lane >> 4;
+  const int K = static_cast<int>(a.K), M = static_cast<int>(a.M), N = static_cast<int>(a.N);
+  const int KB = (K + 63) >> 6;                    // 64-byte k-blocks
+  const int KC = K >> 4;                           // 16-byte chunks (K is a multiple of 16)
+  const int NG = (N + 15) >> 4;                    // channel groups
+  const int G = static_cast<int>(gridDim.x), b = static_cast<int>(blockIdx.x);
+  const int ngb = (NG - b + G - 1) / G;            // groups of this block (G <= NG: at least one)
+  const int U = (KB + kResidentWaves - 1) / kResidentWaves;  // k-blocks of a group per wave
+  const int KBP = U * kResidentWaves;              // k-blocks in LDS: those past K hold zeros
+  const int Q = ngb * U;                           // this wave's stream of (group, k-block) units
+  const int64_t slab = a.w_kchunks * 256;          // packed bytes of one channel group
+
+  // ---- requests, oldest first: the activations (L2) ...
+  // piece (mg, kb) = 16 rows x 64 bytes: lane -> row lane / 4, 16-byte chunk lane % 4
+  // (four lanes ask for one cache line); pieces are dealt round-robin to the waves
+  constexpr int kXPieces = kResidentXBytes / 1024 / kResidentWaves;  // per wave, at most
+  v4i xr[kXPieces];
+  const int sr = lane >> 2, sp = lane & 3;
+#pragma unroll
+  for (int j = 0; j < kXPieces; ++j) {
+    const int p = wave + kResidentWaves * j;
+    if (p < MG * KBP) {
+      const int kb = p / MG, mg = p - kb * MG;
+      const int row = mg * 16 + sr, c = kb * 4 + sp;
+      const bool ok = row < M && c < KC;
+      xr[j] = ld16(xs.x + (ok ? static_cast<int64_t>(row) * xs.ldx + c * 16 : 0));
+    }
+  }
+  // ... the constants of this block's channels (cold): thread -> group slot t / 16, channel t % 16
+  const int cslot = t >> 4, cch = t & 15;
+  int c_cs = 0;
+  float c_ws = 1.f, c_b = 0.f;
+  {
+    const int n = (b + cslot * G) * 16 + cch;
+    const int np = cslot < ngb && n < N ? n : 0;
+    c_cs = a.colsum[np];
+    if constexpr (MODE != kOutAcc32) {  // (raw accumulators: the caller passes no scales)
+      c_ws = a.w_scales[np * a.w_scale_stride];
+      const float* const bsrc = a.bias != nullptr ? a.bias : a.w_scales;  // a load that always has an address
+      const float bv = bsrc[a.bias != nullptr ? np : 0];
+      c_b = a.bias != nullptr ? bv : 0.f;
+    }
+  }
+  // ... and the first kDepth k-blocks of the weight stream (memory).  The load cursor
+  // (group li, k-block slot lu) runs kDepth units ahead of the multiply cursor.
+  const uint8_t* const wlane = a.w_packed + lane * 16;
+  int li = 0, lu = 0;
+  auto next_weights = [&]() {
+    const int kb = wave + kResidentWaves * lu;
+    const int kbc = kb < KB ? kb : KB - 1;         // (slots past K: any k-block, it meets zeros)
+    const v4i w = __builtin_nontemporal_load(
+        reinterpret_cast<const v4i*>(wlane + static_cast<int64_t>(b + li * G) * slab + static_cast<int64_t>(kbc) * 1024));
+    if (++lu == U) {
+      lu = 0;
+      ++li;
+    }
+    return w;
+  };
+  v4i wf[D];
+#pragma unroll
+  for (int j = 0; j < D; ++j)
+    if (j < Q) wf[j] = next_weights();
+
+  // ---- activations into LDS: piece (mg, kb), chunk c of row r -> ((4 kb + c) * 16 MG + 16 mg + r) * 16
+  for (int i = t; i < 2 * MG * 4 * kWave; i += kResidentThreads) (&s_sum[0][0][0][0])[i] = 0;
+  {
+    const int xor_word = static_cast<int>(a.x_xor);
+    const v4i xmask = {xor_word, xor_word, xor_word, xor_word};
+#pragma unroll
+    for (int j = 0; j < kXPieces; ++j) {
+      const int p = wave + kResidentWaves * j;
+      if (p < MG * KBP) {
+        const int kb = p / MG, mg = p - kb * MG;
+        const bool ok = mg * 16 + sr < M && kb * 4 + sp < KC;
+        const v4i v = ok ? (xr[j] ^ xmask) : v4i{0, 0, 0, 0};
+        *reinterpret_cast<v4i*>(&s_x[(((kb * 4 + sp) * MG + mg) * 16 + sr) * 16]) = v;
+      }
+    }
+  }
+  // ---- the channels' constants, ready for the epilogue
+  {
+    const XQuant xq = x_quant(a);
+    float mult = 0.f, bdiv = 0.f, bmul = 1.f;
+    if constexpr (MODE == kOutF32) {
+      mult = xq.scale * c_ws;
+      bdiv = c_b;
+    } else if constexpr (MODE != kOutAcc32) {
+      const float atw = xq.scale * c_ws;
+      mult = atw / a.out_scale;
+      bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, c_b, atw) : 0.f;
+      bmul = bias_mul(a.w_scale_stride == 0, atw);  // (per tensor: the same for every channel)
+    }
+    if (cslot < kResidentMaxGroups) {
+      s_acc0[t] = xq.coef * c_cs;
+      s_mult[t] = mult;
+      s_bdiv[t] = bdiv;
+    }
+    if (t == 0) s_bmul = bmul;
+  }
+  resident_barrier();
+
+  // ---- the stream
+  v4i acc2[MG][2];  // two accumulators per row group, used in turn
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) acc2[mg][0] = acc2[mg][1] = v4i{0, 0, 0, 0};
+  const uint8_t* const xop = &s_x[(lc * MG * 16 + lr) * 16];   // + kb * MG * 1024 + mg * 256
+  const int fm = lane >> 2, fg = lane & 3;         // finishing wave: lane -> row within a group, four channels
+
+  auto finish_group = [&](int gi) {
+    const int par = gi & 1;
+#pragma unroll
+    for (int mg = 0; mg < MG; ++mg) {
+      const v4i acc = acc2[mg][0] + acc2[mg][1];
+      acc2[mg][0] = acc2[mg][1] = v4i{0, 0, 0, 0};
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        __hip_atomic_fetch_add(&s_sum[par][mg][r][lane], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    resident_barrier();
+    // One wave finishes the group and clears the slot.  The slot is next added to after
+    // the following group's barrier, which this wave reaches only after its clears.
+    if (wave != (gi & (kResidentWaves - 1))) return;
+    const int64_t n = static_cast<int64_t>(b + gi * G) * 16 + 4 * fg;
+    const v4i add = *reinterpret_cast<const v4i*>(&s_acc0[gi * 16 + 4 * fg]);
+    const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[gi * 16 + 4 * fg]);
+    const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[gi * 16 + 4 * fg]);
+    const float bmul = s_bmul;
+#pragma unroll
+    for (int mg = 0; mg < MG; ++mg) {
+      int raw[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {  // channel 4 fg + j of row fm: register j of lane 16 fg + fm
+        raw[j] = s_sum[par][mg][j][16 * fg + fm] + add[j];
+        s_sum[par][mg][j][16 * fg + fm] = 0;
+      }
+      const int64_t m = mg * 16 + fm;
+      if (m >= a.M || n >= a.N) continue;
+      if constexpr (MODE == kOutAcc32) {
+        int32_t* dst = static_cast<int32_t*>(a.y) + m * a.ldy + n;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < a.N) dst[j] = raw[j];
+      } else if constexpr (MODE == kOutF32) {
+        store_f32x4(a, m, n, raw, mult, bdiv);
+      } else {
+        const uint32_t packed = requant4<MODE>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+        uint8_t* dst = static_cast<uint8_t*>(a.y) + m * a.ldy + n;
+        if (n + 3 < a.N && (a.ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 3) == 0) {
+          *reinterpret_cast<uint32_t*>(dst) = packed;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (n + j < a.N) dst[j] = static_cast<uint8_t>(packed >> (8 * j));
+        }
+      }
+    }
+  };
+
+  int ci = 0, cu = 0;  // multiply cursor: group, k-block slot
+  // unit j of a run of kDepth: multiply with wf[j], refill it with the unit kDepth further on
+  auto unit = [&](int j, bool refill) {
+    const int kb = wave + kResidentWaves * cu;
+#pragma unroll
+    for (int mg = 0; mg < MG; ++mg) {
+      const v4i xv = ld16(xop + kb * (MG * 1024) + mg * 256);
+      acc2[mg][j & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[j], xv, acc2[mg][j & 1], 0, 0, 0);
+    }
+    if (refill) wf[j] = next_weights();
+    if (++cu == U) {
+      cu = 0;
+      finish_group(ci);
+      ++ci;
+    }
+  };
+  // Runs whose every unit has a successor kDepth further on issue their loads without a
+  // condition, so that the count of loads in flight the waits are derived from is exact;
+  // the last two runs decide per unit.
+  int q0 = 0;
+  for (; q0 + 2 * D <= Q; q0 += D) {
+#pragma unroll
+    for (int j = 0; j < D; ++j) unit(j, true);
+  }
+  for (; q0 < Q; q0 += D) {
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+      if (q0 + j >= Q) break;
+      unit(j, q0 + j + D < Q);
+    }
+  }
+}
+
+}  // namespace tmq
