@@ -255,8 +255,11 @@ def main():
                   (128, 4096, 4096), (256, 4096, 4096), (448, 4096, 4096), (512, 4096, 4096), (1024, 4096, 4096),
                   (2048, 4096, 4096), (64, 11008, 4096), (256, 11008, 4096), (2048, 11008, 4096),
                   (64, 4096, 11008), (256, 4096, 11008), (128, 1024, 1024), (512, 1024, 1024), (640, 1024, 1024),
-                  (128, 2048, 2048), (256, 4096, 2048), (4096, 4096, 4096)]
-        candidates = (2, 3, 6, 7, 8, 13, 14, 17, 19, 20, 21, 23, 24, 25, 26)
+                  (128, 2048, 2048), (256, 4096, 2048), (4096, 4096, 4096),
+                  (8, 11008, 4096), (16, 11008, 4096), (16, 32000, 4096), (16, 4096, 4096), (4, 8192, 1024),
+                  (32, 8192, 8192), (64, 5120, 5120), (768, 11008, 4096), (1536, 11008, 4096), (192, 6144, 3072),
+                  (640, 8192, 8192)]
+        candidates = (2, 3, 6, 7, 8, 13, 14, 17, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28)
         rows = []
         for (Ms, Ns, Ks) in shapes:
             sets = max(2, min(40, (600 << 20) // (Ns * Ks)))
@@ -295,7 +298,7 @@ def main():
                 c_ = cabi.linear_kernel_choice(Ms, Ns, Ks, workspace=wbytes > 0, forced=cfg + 1)
                 if c_["kernel"] - 1 != cfg or cfg == auto["kernel"] - 1:
                     continue          # refused, or replaced by another kernel
-                if c_["blocks"] > 8192 or (cfg in (2, 14, 21, 24, 25, 26) and Ms * Ns > 1 << 22):
+                if c_["blocks"] > 8192 or (cfg in (2, 14, 21, 24, 25, 26, 27) and Ms * Ns > 1 << 22):
                     continue          # small tiles on a large product: not a candidate
                 others[cfg] = round(timed(cfg), 2)
             best = min(others, key=others.get) if others else None
@@ -765,6 +768,47 @@ def main():
                 "frac_of_read_only_kernel": round(read_us / (per * 1e3), 4),
                 "method": f"{sets} distinct packed weights replayed back to back in one HIP graph",
                 "algorithmic_bytes_per_launch": nbytes}
+
+        # ----------------------------- decode rows against an output projection: K = 4096, N = 32000
+        # (131 MB of weights per launch, nine sets in rotation; from 12 rows on the kernel that keeps
+        # the rows in LDS, below it a block per 16 channels), torch._int_mm beside it
+        Np = 32000
+        sets_p = 9
+        pwp = [cabi.PackedLinear(torch.randint(-127, 128, (Np, Kd), dtype=torch.int8, device=dev))
+               for _ in range(sets_p)]
+        wsp = torch.rand(Np, device=dev) * 0.002 + 0.001
+        bp = torch.randn(Np, device=dev)
+        wts_p = None
+        for Md in (1, 16):
+            xd = torch.randint(0, 256, (Md, Kd), dtype=torch.uint8, device=dev)
+            yd = torch.empty((Md, Np), dtype=torch.uint8, device=dev)
+
+            def run_proj():
+                for p in pwp:
+                    cabi.linear(xd, p, 0.02, 128, wsp, bp, 0.05, 128, out=yd)
+
+            per = graph_us(run_proj, sets_p)
+            vendor = None
+            try:
+                if wts_p is None:
+                    wts_p = [torch.randint(-127, 128, (Np, Kd), dtype=torch.int8, device=dev).t() for _ in range(sets_p)]
+                xs8 = torch.randint(-128, 128, (max(Md, 32), Kd), dtype=torch.int8, device=dev)  # (the op wants > 16 rows)
+                vendor = graph_us(lambda: [torch._int_mm(xs8, wt) for wt in wts_p], sets_p)
+            except Exception as ex:
+                log(f"[bench] torch._int_mm not timed: {ex}")
+            nbytes = Np * Kd + Md * Kd + Md * Np + 12 * Np
+            gbs = nbytes / per / 1e3
+            kern = cabi.linear_kernel_choice(Md, Np, Kd)["kernel"] - 1
+            log(f"[bench] decode M={Md} against N={Np}: {per:.2f} us/launch (kernel {kern}), {gbs:.0f} GB/s"
+                + (f" (torch._int_mm on {max(Md, 32)} rows: {vendor:.2f} us)" if vendor else ""))
+            secondary[f"linear_decode_m{Md}_n{Np}"] = {
+                "avg_launch_us": round(per, 3), "value": round(gbs, 1), "unit": "GB/s", "kernel": kern,
+                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
+                "torch_int_mm_us": None if vendor is None else round(vendor, 3),
+                "method": f"{sets_p} distinct packed weights replayed back to back in one HIP graph",
+                "algorithmic_bytes_per_launch": nbytes}
+        del pwp, wts_p
 
         # ----------------------------- the same cold weights against a few dozen to a few hundred rows
         # (32 x 32 / 32 x 64 / 64 x 64 tiles whose waves split K and take their weights through

@@ -184,11 +184,15 @@ def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256
             assert k >= 3072 and tiles <= 256, what
     elif cfg == 28:                                 # activations resident in LDS: 16 MG x K bytes, K padded to 16 k-blocks,
         mg = _ceil(m, 16)                           # in 128 KB; the constants of at most 64 channel groups per block
-        assert m <= 64 and (bm, bn) == (16 * mg, 16) and c["waves"] == 16, what
-        assert 16 * mg * _ceil(k, 1024) * 1024 <= 128 * 1024 and _ceil(n, 16) <= 64 * cus, what
-        assert c["blocks"] == min(tiles, cus), what
+        assert m <= 64 and (bm, bn) == (16 * mg, 16) and c["waves"] in (8, 16), what
+        if c["waves"] == 16:                        # one block per CU
+            assert 16 * mg * _ceil(k, 1024) * 1024 <= 128 * 1024 and _ceil(n, 16) <= 64 * cus, what
+            assert c["blocks"] == min(tiles, cus), what
+        else:                                       # two blocks of eight waves per CU: half the LDS area, 32 groups each
+            assert mg == 1 and 16 * _ceil(k, 512) * 512 <= 64 * 1024 and 2 * cus <= _ceil(n, 16) <= 64 * cus, what
+            assert c["blocks"] == min(tiles, 2 * cus), what
         if forced == 0:                             # rows that share the streamed weights, or a short K
-            assert k >= 1024 and ((m <= 16 and (k <= 2048 or m >= 12)) or n >= 98304), what
+            assert k >= 1024 and ((m <= 16 and (k <= 2048 or m >= 12 or (m >= 5 and n >= 16384))) or n >= 98304), what
         return
     else:                                           # register-staged tiles take any aligned shape
         assert cfg in (0, 1, 2, 3, 4, 5, 22, 23), what

@@ -197,10 +197,12 @@ def test_long_k_as_a_ring_of_phases(cabi, shape, x_signed):
 
 # up to 64 rows with the activations resident in LDS, one block per CU walking its channel groups:
 # one group and several per block (ragged last round), K that ends inside a k-block / inside the
-# padding to 16 k-blocks, every number of row groups, a single row, both activation types
+# padding to 16 k-blocks, every number of row groups, a single row, both activation types; the last
+# two (and the third) as two blocks of eight waves per CU
 @pytest.mark.parametrize("shape, x_signed", [((16, 4113, 1024), False), ((1, 100, 1040), True), ((13, 12300, 1024), False),
                                              ((32, 1000, 2048), True), ((64, 300, 1040), False), ((9, 5000, 8192), True),
-                                             ((40, 530, 2048), False), ((12, 8200, 4112), True)])
+                                             ((40, 530, 2048), False), ((12, 8200, 4112), True),
+                                             ((7, 16400, 4096), True), ((16, 8200, 2048), False)])
 def test_activations_resident_in_lds(cabi, shape, x_signed):
     say("resident activations", shape, x_signed)
     M, N, K = shape

@@ -628,11 +628,27 @@ bool resident_limits_ok(int64_t M, int64_t N, int64_t K, int64_t ldx, int cus) {
          N <= 0x7ffffff0 && ldx <= (int64_t{1} << 40);
 }
 
+// Two blocks of eight waves per CU where the rows fit half the LDS area (one group of rows,
+// K <= 4096) and a block still owns at most 32 channel groups: the two blocks' bursts of
+// requests interleave (M = 8, K = 4096, N = 32000: 25.2 -> 24.0 us; N = 16384, K = 1024: 6.7 -> 6.0 us;
+// N = 8192, K = 2048: 6.2 -> 5.8 us).  Not below two groups per block at K > 2048: the rows are then
+// staged twice per CU for nothing (N = 5120, K = 4096, M = 16: 7.7 -> 8.8 us; N = 11008: 10.6 -> 11.0 us).
+bool resident_pair(int64_t M, int64_t N, int64_t K, int cus) {
+  const int64_t groups = ceil_div(N, 16);
+  return M <= 16 && 16 * ceil_div(K, 64 * 8) * (64 * 8) <= kResidentXBytes / 2 && groups <= int64_t{32} * 2 * cus &&
+         groups >= (K <= 2048 ? 2 : 4) * static_cast<int64_t>(cus);
+}
+
 template <int MODE>
 int launch_linear_resident(const GemmArgs& a, const XLinear& xs, hipStream_t s) {
   const int cus = cu_count();
   if (!resident_limits_ok(a.M, a.N, a.K, xs.ldx, cus)) return TMQ_ERR_UNSUPPORTED;
   const int64_t groups = ceil_div(a.N, 16);
+  if (resident_pair(a.M, a.N, a.K, cus)) {
+    const dim3 grid(static_cast<unsigned>(groups < 2 * cus ? groups : 2 * cus)), block(8 * kWave);
+    linear_resident_kernel<MODE, 1, 8><<<grid, block, 0, s>>>(a, xs);
+    return launch_status();
+  }
   const dim3 grid(static_cast<unsigned>(groups < cus ? groups : cus)), block(kResidentThreads);
   switch ((a.M + 15) / 16) {
     case 1: linear_resident_kernel<MODE, 1><<<grid, block, 0, s>>>(a, xs); break;
@@ -941,13 +957,14 @@ bool stream_limits_ok(const LinearQuery& q) {
 //   longer K, 12 rows and more (the streaming blocks re-read the rows from the L2s), from N = 5120 on:
 //     K = 4096, M = 16: N = 5120 7.7 | 8.6, N = 11008 10.6 | 12.3, N = 32000 25.4 | 32.2, N = 128256 97 | 122;
 //     M = 12: N = 49152 38.2 | 39.6, N = 65536 50.3 | 54.4;  N = K = 8192, M = 16: 14.7 | 16.1
-//   (M <= 8 at K = 4096: level up to N = 32000, then the independent blocks stream faster: N = 128256,
-//   M = 1: 91 | 85; N = 4096 at K >= 4096: level or behind, 6.1 | 5.9 at M = 16)
+//   5 ... 11 rows at K = 4096 from N = 16384 on, as two blocks per CU: M = 8: N = 32000 24.0 | 25.6, N = 128256 91.7 | 95.7
+//   (fewer rows: level up to N = 32000, then the independent blocks stream faster: N = 128256, M = 1: 89 | 85;
+//   N = 4096 at K >= 4096: level or behind, 6.1 | 5.9 at M = 16)
 //   17 ... 32 rows against the largest N only (N = 128256, K = 4096: 104 against 111 us for 128 x 128 tiles;
 //   N = 32000: 27 against 25.4 us for 64 x 128 tiles).
 bool resident_preferred(const LinearQuery& q) {
   if (!q.vec_ok || q.K < 1024 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
-  if (q.M <= 16) return q.K <= 2048 ? q.N >= 4096 : (q.M >= 12 && q.N >= 5120);
+  if (q.M <= 16) return q.K <= 2048 ? q.N >= 4096 : ((q.M >= 12 && q.N >= 5120) || (q.M >= 5 && q.N >= 16384));
   return q.M <= 32 && q.N >= 98304;
 }
 
@@ -1278,7 +1295,7 @@ TMQ_EXPORT int tmq_linear_kernel_choice(int64_t M, int64_t N, int64_t K, int64_t
     case 26: bm = 32, bn = 64, waves = 8; break;
     case 27: bm = 64, bn = 64, waves = 8; break;
     case 8: bm = 16 * static_cast<int>(ceil_div(M, 16)), bn = 16, waves = kDecodeWaves; break;
-    case 28: bm = 16 * static_cast<int>(ceil_div(M, 16)), bn = 16, waves = kResidentWaves; break;
+    case 28: bm = 16 * static_cast<int>(ceil_div(M, 16)), bn = 16, waves = resident_pair(M, N, K, compute_units) ? 8 : kResidentWaves; break;
     default: break;  // 9: one thread per four outputs
   }
   out->kernel = c.cfg + 1;
@@ -1293,7 +1310,7 @@ TMQ_EXPORT int tmq_linear_kernel_choice(int64_t M, int64_t N, int64_t K, int64_t
     out->tiles = ceil_div(M, bm) * ceil_div(N, bn) * c.split.splits;
     out->blocks = out->tiles;
     if (c.cfg == 20 && out->tiles > compute_units) out->blocks = compute_units / 8 * 8;
-    if (c.cfg == 28 && out->tiles > compute_units) out->blocks = compute_units;
+    if (c.cfg == 28) out->blocks = std::min<int64_t>(out->tiles, (waves == 8 ? 2 : 1) * static_cast<int64_t>(compute_units));
   }
   return TMQ_OK;
 }

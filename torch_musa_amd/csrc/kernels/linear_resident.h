@@ -31,7 +31,7 @@ namespace tmq {
 constexpr int kResidentWaves = 16;
 constexpr int kResidentThreads = kResidentWaves * kWave;
 constexpr int kResidentDepth = 8;                 // k-blocks in flight per wave: 128 KB per block (12 and 16: no faster)
-constexpr int kResidentMaxGroups = 64;            // channel groups a block can own (their constants sit in LDS)
+constexpr int kResidentMaxGroups = 64;            // channel groups a block of 16 waves can own (their constants sit in LDS)
 constexpr int kResidentXBytes = 128 * 1024;       // 16 MG x K activation bytes
 
 // LDS barrier of the block without a fence: every wave's LDS operations so far are
@@ -42,14 +42,17 @@ __device__ __forceinline__ void resident_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <int MODE, int MG>
-__global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmArgs a, XLinear xs) {
+template <int MODE, int MG, int W = kResidentWaves>
+__global__ __launch_bounds__(W * kWave, 4) void linear_resident_kernel(GemmArgs a, XLinear xs) {
   constexpr int D = kResidentDepth;
-  __shared__ __attribute__((aligned(16))) uint8_t s_x[kResidentXBytes];
+  constexpr int kXBytes = kResidentXBytes / kResidentWaves * W;  // (eight waves: two blocks share a CU)
+  constexpr int kThreads = W * kWave;
+  constexpr int kGroups = kThreads / 16;       // channel groups a block can own: a thread per channel stages the constants
+  __shared__ __attribute__((aligned(16))) uint8_t s_x[kXBytes];
   __shared__ __attribute__((aligned(16))) int s_sum[2][MG][4][kWave];
-  __shared__ __attribute__((aligned(16))) int s_acc0[kResidentMaxGroups * 16];
-  __shared__ __attribute__((aligned(16))) float s_mult[kResidentMaxGroups * 16];
-  __shared__ __attribute__((aligned(16))) float s_bdiv[kResidentMaxGroups * 16];
+  __shared__ __attribute__((aligned(16))) int s_acc0[kGroups * 16];
+  __shared__ __attribute__((aligned(16))) float s_mult[kGroups * 16];
+  __shared__ __attribute__((aligned(16))) float s_bdiv[kGroups * 16];
   __shared__ float s_bmul;
 
   const int t = threadIdx.x, lane = t % kWave;
@@ -61,20 +64,20 @@ __global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmA
   const int NG = (N + 15) >> 4;                    // channel groups
   const int G = static_cast<int>(gridDim.x), b = static_cast<int>(blockIdx.x);
   const int ngb = (NG - b + G - 1) / G;            // groups of this block (G <= NG: at least one)
-  const int U = (KB + kResidentWaves - 1) / kResidentWaves;  // k-blocks of a group per wave
-  const int KBP = U * kResidentWaves;              // k-blocks in LDS: those past K hold zeros
+  const int U = (KB + W - 1) / W;  // k-blocks of a group per wave
+  const int KBP = U * W;              // k-blocks in LDS: those past K hold zeros
   const int Q = ngb * U;                           // this wave's stream of (group, k-block) units
   const int64_t slab = a.w_kchunks * 256;          // packed bytes of one channel group
 
   // ---- requests, oldest first: the activations (L2) ...
   // piece (mg, kb) = 16 rows x 64 bytes: lane -> row lane / 4, 16-byte chunk lane % 4
   // (four lanes ask for one cache line); pieces are dealt round-robin to the waves
-  constexpr int kXPieces = kResidentXBytes / 1024 / kResidentWaves;  // per wave, at most
+  constexpr int kXPieces = kXBytes / 1024 / W;  // per wave, at most
   v4i xr[kXPieces];
   const int sr = lane >> 2, sp = lane & 3;
 #pragma unroll
   for (int j = 0; j < kXPieces; ++j) {
-    const int p = wave + kResidentWaves * j;
+    const int p = wave + W * j;
     if (p < MG * KBP) {
       const int kb = p / MG, mg = p - kb * MG;
       const int row = mg * 16 + sr, c = kb * 4 + sp;
@@ -102,7 +105,7 @@ __global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmA
   const uint8_t* const wlane = a.w_packed + lane * 16;
   int li = 0, lu = 0;
   auto next_weights = [&]() {
-    const int kb = wave + kResidentWaves * lu;
+    const int kb = wave + W * lu;
     const int kbc = kb < KB ? kb : KB - 1;         // (slots past K: any k-block, it meets zeros)
     const v4i w = __builtin_nontemporal_load(
         reinterpret_cast<const v4i*>(wlane + static_cast<int64_t>(b + li * G) * slab + static_cast<int64_t>(kbc) * 1024));
@@ -118,13 +121,13 @@ __global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmA
     if (j < Q) wf[j] = next_weights();
 
   // ---- activations into LDS: piece (mg, kb), chunk c of row r -> ((4 kb + c) * 16 MG + 16 mg + r) * 16
-  for (int i = t; i < 2 * MG * 4 * kWave; i += kResidentThreads) (&s_sum[0][0][0][0])[i] = 0;
+  for (int i = t; i < 2 * MG * 4 * kWave; i += kThreads) (&s_sum[0][0][0][0])[i] = 0;
   {
     const int xor_word = static_cast<int>(a.x_xor);
     const v4i xmask = {xor_word, xor_word, xor_word, xor_word};
 #pragma unroll
     for (int j = 0; j < kXPieces; ++j) {
-      const int p = wave + kResidentWaves * j;
+      const int p = wave + W * j;
       if (p < MG * KBP) {
         const int kb = p / MG, mg = p - kb * MG;
         const bool ok = mg * 16 + sr < M && kb * 4 + sp < KC;
@@ -146,11 +149,9 @@ __global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmA
       bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, c_b, atw) : 0.f;
       bmul = bias_mul(a.w_scale_stride == 0, atw);  // (per tensor: the same for every channel)
     }
-    if (cslot < kResidentMaxGroups) {
-      s_acc0[t] = xq.coef * c_cs;
-      s_mult[t] = mult;
-      s_bdiv[t] = bdiv;
-    }
+    s_acc0[t] = xq.coef * c_cs;
+    s_mult[t] = mult;
+    s_bdiv[t] = bdiv;
     if (t == 0) s_bmul = bmul;
   }
   resident_barrier();
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmA
     resident_barrier();
     // One wave finishes the group and clears the slot.  The slot is next added to after
     // the following group's barrier, which this wave reaches only after its clears.
-    if (wave != (gi & (kResidentWaves - 1))) return;
+    if (wave != (gi & (W - 1))) return;
     const int64_t n = static_cast<int64_t>(b + gi * G) * 16 + 4 * fg;
     const v4i add = *reinterpret_cast<const v4i*>(&s_acc0[gi * 16 + 4 * fg]);
     const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[gi * 16 + 4 * fg]);
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(kResidentThreads) void linear_resident_kernel(GemmA
   int ci = 0, cu = 0;  // multiply cursor: group, k-block slot
   // unit j of a run of kDepth: multiply with wf[j], refill it with the unit kDepth further on
   auto unit = [&](int j, bool refill) {
-    const int kb = wave + kResidentWaves * cu;
+    const int kb = wave + W * cu;
 #pragma unroll
     for (int mg = 0; mg < MG; ++mg) {
       const v4i xv = ld16(xop + kb * (MG * 1024) + mg * 256);
