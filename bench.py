@@ -171,7 +171,7 @@ def main():
                     help="do not start the child process that samples the socket power (for runs under a profiler, "
                          "whose library has initialised the GPU before this program starts)")
     ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
-                                       "dequantize_pc", "decode", "rows64", "rows256", "c1", "conv", "conv_add_relu", "probe", "choice"],
+                                       "dequantize_pc", "decode", "rows64", "rows256", "c1", "decode16_proj", "conv", "conv_add_relu", "probe", "choice"],
                     help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
                          "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
                          "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
@@ -340,20 +340,22 @@ def main():
         print(json.dumps({"only": args.only, "launches": args.steps, "shape": [11008, 4096], "axis": 0}))
         return
 
-    if args.only in ("decode", "rows64", "rows256", "c1"):
+    if args.only in ("decode", "rows64", "rows256", "c1", "decode16_proj"):
         # config 4 at M = 1, or 64 / 256 rows against the same weights: 40 packed weights in turn
-        # (cold); config 1 (M = 128, K = N = 1024) likewise; plain launches
-        Mo, Ko = {"decode": (1, 4096), "rows64": (64, 4096), "rows256": (256, 4096), "c1": (128, 1024)}[args.only]
-        pws = [cabi.PackedLinear(torch.randint(-127, 128, (Ko, Ko), dtype=torch.int8, device=dev))
-               for _ in range(40)]
-        wsd = torch.rand(Ko, device=dev) * 0.002 + 0.001
-        bd = torch.randn(Ko, device=dev)
+        # (cold); config 1 (M = 128, K = N = 1024) likewise; 16 rows against an output projection
+        # (K = 4096, N = 32000, nine weights in turn); plain launches
+        Mo, No, Ko, nsets = {"decode": (1, 4096, 4096, 40), "rows64": (64, 4096, 4096, 40), "rows256": (256, 4096, 4096, 40),
+                             "c1": (128, 1024, 1024, 40), "decode16_proj": (16, 32000, 4096, 9)}[args.only]
+        pws = [cabi.PackedLinear(torch.randint(-127, 128, (No, Ko), dtype=torch.int8, device=dev))
+               for _ in range(nsets)]
+        wsd = torch.rand(No, device=dev) * 0.002 + 0.001
+        bd = torch.randn(No, device=dev)
         xd = torch.randint(0, 256, (Mo, Ko), dtype=torch.uint8, device=dev)
-        yd = torch.empty((Mo, Ko), dtype=torch.uint8, device=dev)
+        yd = torch.empty((Mo, No), dtype=torch.uint8, device=dev)
         for i in range(args.steps):
-            cabi.linear(xd, pws[i % 40], 0.02, 128, wsd, bd, 0.05, 128, out=yd)
+            cabi.linear(xd, pws[i % nsets], 0.02, 128, wsd, bd, 0.05, 128, out=yd)
         torch.cuda.synchronize()
-        print(json.dumps({"only": args.only, "launches": args.steps, "M": Mo, "K": Ko, "N": Ko}))
+        print(json.dumps({"only": args.only, "launches": args.steps, "M": Mo, "K": Ko, "N": No}))
         return
 
     if args.only in ("conv", "conv_add_relu"):

@@ -165,7 +165,7 @@ def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256
     elif cfg == 21:                                 # 64 x 64, four phases of 256 bytes of K in LDS: all of K <= 1024,
         assert (bm, bn) == (64, 64) and 64 * ldx <= 2 ** 29, what      # a longer K as a ring of phases
         if forced == 0:                             # one round; the ring only beyond the kernels with weights in registers
-            assert tiles <= 256 and (k <= 1024 or (k > 4096 and m <= 128)), what
+            assert tiles <= 256 and (k <= 1024 or (k >= 4096 and m <= 128)), what
     elif cfg == 24:                                 # all of K in LDS, 32 x 32, a quarter of K per wave
         assert k <= 1024 and (bm, bn) == (32, 32) and 64 * ldx <= 2 ** 29, what
         if forced == 0:
@@ -192,7 +192,7 @@ def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256
             assert mg == 1 and 16 * _ceil(k, 512) * 512 <= 64 * 1024 and 2 * cus <= _ceil(n, 16) <= 64 * cus, what
             assert c["blocks"] == min(tiles, 2 * cus), what
         if forced == 0:                             # rows that share the streamed weights, or a short K
-            assert k >= 1024 and ((m <= 16 and (k <= 2048 or m >= 12 or (m >= 5 and n >= 16384))) or n >= 98304), what
+            assert k >= 1024 and ((m <= 16 and (k <= 2048 or m >= 14 or (m >= 5 and n >= 10240))) or n >= 98304), what
         return
     else:                                           # register-staged tiles take any aligned shape
         assert cfg in (0, 1, 2, 3, 4, 5, 22, 23), what

@@ -178,7 +178,8 @@ def test_weights_through_registers_kernel(cabi, shape, x_signed, cfg):
 # choice is the kernel that walks K through LDS as a ring of 256-byte phases (K that ends inside
 # a phase and on an odd 16-byte chunk, ragged channels, both activation types)
 @pytest.mark.parametrize("shape, x_signed", [((64, 4500, 8208), False), ((128, 1000, 5136), True),
-                                             ((48, 4200, 4112), False), ((113, 130, 4112), True)])
+                                             ((48, 4200, 4112), False), ((113, 130, 4112), True),
+                                             ((64, 10300, 4096), False)])
 def test_long_k_as_a_ring_of_phases(cabi, shape, x_signed):
     say("ring of phases", shape, x_signed)
     M, N, K = shape

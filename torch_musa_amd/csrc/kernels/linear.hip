@@ -727,8 +727,11 @@ int wstream_tile(int64_t M, int64_t N, int64_t K) {
 // 26.5 us at 64 rows), while two wave groups slow down as the tiles fill (20.9 us and 29.3 us
 // at 64 rows; N = 4096, K = 11008, M = 64: 32.2 against 37.3 us).  With a tile half empty, or
 // from 192 rows on, the wave groups are ahead (N = 4096, K = 14336, M = 256: 42.4 against 45.6 us).
+// (K = 4096 against N >= 10240, where the tiles of 32 rows no longer fit one round: M = 64, N = 11008: 16.2 against
+// 17.5 us; N = 14336: 17.3 against 18.1 us; at 128 rows the wave groups are ahead, N = 8192: 15.7 against 16.2 us)
 bool phased_ring_preferred(int64_t M, int64_t N, int64_t K) {
-  return K > 4096 && K % 16 == 0 && ceil_div(M, 64) * ceil_div(N, 64) <= 256 && M <= 128 && (M - 1) % 64 >= 47;
+  if (K % 16 != 0 || ceil_div(M, 64) * ceil_div(N, 64) > 256 || (M - 1) % 64 < 47) return false;
+  return K > 4096 ? M <= 128 : (K == 4096 && M <= 64 && N >= 10240);
 }
 
 SmallRows small_rows_path(int64_t M, int64_t N, int64_t K, bool workspace) {
@@ -954,17 +957,19 @@ bool stream_limits_ok(const LinearQuery& q) {
 // (cold weights, us, resident | streaming; neither depends on N beyond what is shown):
 //   K <= 2048, from N = 4096 on, any M <= 16:  N = 4096, K = 1024: 3.9 | 4.2 ... 4.5;  N = 8192, K = 1024:
 //     4.8 ... 5.0 | 5.8 ... 6.3;  N = 4096, K = 2048: 4.5 | 4.7 ... 5.0;  N = 65536, K = 2048: 24.5 | 35 ... 42
-//   longer K, 12 rows and more (the streaming blocks re-read the rows from the L2s), from N = 5120 on:
+//   longer K, 14 rows and more (the streaming blocks re-read the rows from the L2s), from N = 5120 on:
 //     K = 4096, M = 16: N = 5120 7.7 | 8.6, N = 11008 10.6 | 12.3, N = 32000 25.4 | 32.2, N = 128256 97 | 122;
-//     M = 12: N = 49152 38.2 | 39.6, N = 65536 50.3 | 54.4;  N = K = 8192, M = 16: 14.7 | 16.1
-//   5 ... 11 rows at K = 4096 from N = 16384 on, as two blocks per CU: M = 8: N = 32000 24.0 | 25.6, N = 128256 91.7 | 95.7
+//     N = K = 8192, M = 16: 14.7 | 16.1  (M = 12: N = 5120 7.6 | 7.8, N = 8192 9.1 | 8.6: one full round of
+//     streaming blocks, two per CU, is that kernel's best case)
+//   5 ... 13 rows at K = 4096 beyond that round, N >= 10240: M = 8: N = 11008 10.8 | 11.3 ... 12.2, N = 32000
+//     24.0 | 25.6, N = 128256 91.7 | 95.7;  M = 12: N = 49152 38.2 | 39.6, N = 65536 50.3 | 54.4
 //   (fewer rows: level up to N = 32000, then the independent blocks stream faster: N = 128256, M = 1: 89 | 85;
 //   N = 4096 at K >= 4096: level or behind, 6.1 | 5.9 at M = 16)
 //   17 ... 32 rows against the largest N only (N = 128256, K = 4096: 104 against 111 us for 128 x 128 tiles;
 //   N = 32000: 27 against 25.4 us for 64 x 128 tiles).
 bool resident_preferred(const LinearQuery& q) {
   if (!q.vec_ok || q.K < 1024 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
-  if (q.M <= 16) return q.K <= 2048 ? q.N >= 4096 : ((q.M >= 12 && q.N >= 5120) || (q.M >= 5 && q.N >= 16384));
+  if (q.M <= 16) return q.K <= 2048 ? q.N >= 4096 : ((q.M >= 14 && q.N >= 5120) || (q.M >= 5 && q.N >= 10240));
   return q.M <= 32 && q.N >= 98304;
 }
 
