@@ -298,12 +298,18 @@ int tmq_linear_f32(const tmq_linear_desc* desc, const tmq_qparams* x_qparams_dev
                    int64_t ldy, tmq_stream_t stream);
 
 /* The whole dynamically quantized linear for a handful of rows in one launch:
- * fp32 x [M, ldx] -> fp32 y [M, ldy] with M <= 16, M * K <= 16384, K a multiple
- * of 16, x 16-byte aligned, ldx a multiple of 4 (TMQ_ERR_UNSUPPORTED otherwise:
- * use tmq_quantize_per_tensor_dynamic_dev + tmq_linear_f32, which give the same
- * results).  Every block of the weight-streaming kernel derives the activation
- * range, parameters and codes itself while its weights are on their way.  Uses
- * M, N, K, w_*, relu, bias of `desc`.  Same reference note as tmq_linear_f32. */
+ * fp32 x [M, ldx] -> fp32 y [M, ldy] with M <= 16, K a multiple of 16, x 16-byte
+ * aligned, ldx a multiple of 4, and either M * K <= 16384 (every block of the
+ * weight-streaming kernel derives the activation range, parameters and codes
+ * itself while its weights are on their way) or M * K <= 32768 with
+ * 64 <= K <= 8192 (one block per CU does so once, keeps the codes in LDS and
+ * streams the channel groups it owns; the library picks between the two where
+ * both apply).  TMQ_ERR_UNSUPPORTED otherwise: use
+ * tmq_quantize_per_tensor_dynamic_dev + tmq_linear_f32, which give the same
+ * results; tmq_linear_dynamic_small_takes says beforehand (1 / 0, alignment
+ * aside).  Uses M, N, K, w_*, relu, bias of `desc`; desc->kernel = 9 / 29 pins
+ * the first / second kernel for tests.  Same reference note as tmq_linear_f32. */
+int tmq_linear_dynamic_small_takes(int64_t M, int64_t N, int64_t K);
 int tmq_linear_dynamic_small(const tmq_linear_desc* desc, const float* x, int64_t ldx, int reduce_range,
                              float* y, int64_t ldy, tmq_stream_t stream);
 

@@ -612,10 +612,14 @@ def test_linear_dynamic_cases(cabi, golden, c):
                                                    ((16, 1024, 300), False, False, True, True),
                                                    ((3, 48, 17), False, True, True, False),
                                                    ((1, 16384, 64), True, True, True, False),
-                                                   ((5, 1040, 130), False, True, False, True)])
+                                                   ((5, 1040, 130), False, True, False, True),
+                                                   ((8, 4096, 1000), False, True, True, False),
+                                                   ((4, 8192, 130), True, False, False, True),
+                                                   ((11, 2064, 9000), False, True, True, False)])
 def test_linear_dynamic_one_launch(cabi, shape, relu, bias, pc, rr):
     # a handful of rows: range, parameters, codes and product inside the weight-streaming
-    # kernel; bit for bit the oracle and the two-launch path
+    # kernel or the kernel that keeps the rows in LDS (each pinned where it takes the shape,
+    # and the library's choice); bit for bit the oracle and the two-launch path
     say("linear_dynamic one launch", shape, relu, bias, pc, rr)
     M, K, N = shape
     rng = np.random.default_rng(M * 7 + K)
@@ -628,6 +632,13 @@ def test_linear_dynamic_one_launch(cabi, shape, relu, bias, pc, rr):
     assert cabi.fused_small_dynamic
     y = host(cabi.linear_dynamic(*args, relu=relu, reduce_range=rr))
     np.testing.assert_array_equal(y, oracle.linear_dynamic(x, wq, wsc, b, relu=relu, reduce_range=rr))
+    for pin in ([9] if M * K <= 16384 else []) + ([29] if 64 <= K <= 8192 and M * K <= 32768 else []):
+        cabi.dynamic_small_kernel = pin
+        try:
+            yp = host(cabi.linear_dynamic(*args, relu=relu, reduce_range=rr))
+        finally:
+            cabi.dynamic_small_kernel = 0
+        np.testing.assert_array_equal(yp, y)
     cabi.fused_small_dynamic = False
     try:
         y2 = host(cabi.linear_dynamic(*args, relu=relu, reduce_range=rr))

@@ -24,7 +24,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel", "tmq_dequantize_per_channel",
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
-    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_kernel_choice", "tmq_linear_static_workspace", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_quantize_per_tensor_dynamic_dev",
+    "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_kernel_choice", "tmq_linear_static_workspace", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_linear_dynamic_small_takes", "tmq_quantize_per_tensor_dynamic_dev",
     "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
@@ -134,6 +134,7 @@ def lib() -> C.CDLL:
         l.tmq_linear_acc32.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, v]
         l.tmq_linear_f32.argtypes = [C.POINTER(LinearDesc), v, v, C.c_int64, v]
         l.tmq_linear_dynamic_small.argtypes = [C.POINTER(LinearDesc), v, C.c_int64, C.c_int, v, C.c_int64, v]
+        l.tmq_linear_dynamic_small_takes.argtypes = [C.c_int64, C.c_int64, C.c_int64]
         l.tmq_quantize_per_tensor_dynamic_dev.argtypes = [v, v, C.c_int64, C.c_int, C.c_int, C.c_int, v, v, C.c_size_t, v]
         l.tmq_conv2d_prepack.argtypes = [v, C.POINTER(Conv2dGeom), v, v, v]
         l.tmq_conv2d_out_hw.argtypes = [C.POINTER(Conv2dGeom), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
@@ -313,6 +314,7 @@ class PackedLinear:
 use_linear_workspace = True
 # False: linear_dynamic always takes the two-launch path (quantize, then multiply)
 fused_small_dynamic = True
+dynamic_small_kernel = 0     # tmq_linear_dynamic_small: 0 the library's choice, 9 / 29 pin one of its two kernels
 # a preallocated uint8 tensor that every call on its device shares instead (calls
 # on one stream run in order, so one buffer serves them all); None: per call
 linear_workspace = None
@@ -406,7 +408,12 @@ def linear_dynamic(x, pw: PackedLinear, w_scales, bias, relu=False, reduce_range
     assert x.dtype == torch.float32 and x.is_contiguous()
     x2 = x.reshape(-1, x.shape[-1])
     m, k = x2.shape
-    if fused_small_dynamic and 0 < m <= 16 and m * k <= 16384 and k % 16 == 0 and x2.data_ptr() % 16 == 0:
+    takes = 0 < m <= 16 and k % 16 == 0 and lib().tmq_linear_dynamic_small_takes(m, pw.N, k) != 0
+    if dynamic_small_kernel == 9:                               # a block per 16 channels quantizes the rows itself
+        takes = takes and m * k <= 16384
+    elif dynamic_small_kernel == 29:                            # one block per CU does, once
+        takes = takes and 64 <= k <= 8192 and m * k <= 32768
+    if fused_small_dynamic and takes and x2.data_ptr() % 16 == 0:
         # a handful of rows: range, parameters, codes and product in one launch
         y = torch.empty((m, pw.N), dtype=torch.float32, device=x.device)
         assert k == pw.K and w_scales.dtype == torch.float32
@@ -414,6 +421,7 @@ def linear_dynamic(x, pw: PackedLinear, w_scales, bias, relu=False, reduce_range
         d.M, d.K, d.N = m, k, pw.N
         d.w_packed, d.w_colsum, d.w_scales = pw.packed.data_ptr(), pw.colsum.data_ptr(), w_scales.data_ptr()
         d.w_per_channel, d.relu, d.bias = int(w_scales.numel() > 1), int(relu), _ptr(bias)
+        d.kernel = dynamic_small_kernel
         check(lib().tmq_linear_dynamic_small(C.byref(d), x2.data_ptr(), x2.stride(0), int(reduce_range),
                                              y.data_ptr(), y.stride(0), stream_ptr()), "tmq_linear_dynamic_small")
         return y.reshape(tuple(x.shape[:-1]) + (pw.N,))

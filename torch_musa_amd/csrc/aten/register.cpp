@@ -382,7 +382,7 @@ struct PackedLinearWeightTmq final : public LinearPackedParamsBase {
     }
     const auto stream = current_stream(x);
     const auto bytes = x.options().dtype(at::kByte);
-    if (M <= 16 && M * K_ <= 16384 && K_ % 16 == 0 && reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0) {
+    if (tmq_linear_dynamic_small_takes(M, N_, K_) != 0 && reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0) {
       // a handful of rows: range, parameters, codes and product in one launch
       tmq_linear_desc d{};
       d.M = M;

@@ -646,15 +646,15 @@ int launch_linear_resident(const GemmArgs& a, const XLinear& xs, hipStream_t s) 
   const int64_t groups = ceil_div(a.N, 16);
   if (resident_pair(a.M, a.N, a.K, cus)) {
     const dim3 grid(static_cast<unsigned>(groups < 2 * cus ? groups : 2 * cus)), block(8 * kWave);
-    linear_resident_kernel<MODE, 1, 8><<<grid, block, 0, s>>>(a, xs);
+    linear_resident_kernel<MODE, 1, 8><<<grid, block, 0, s>>>(a, xs, nullptr, 0, 0);
     return launch_status();
   }
   const dim3 grid(static_cast<unsigned>(groups < cus ? groups : cus)), block(kResidentThreads);
   switch ((a.M + 15) / 16) {
-    case 1: linear_resident_kernel<MODE, 1><<<grid, block, 0, s>>>(a, xs); break;
-    case 2: linear_resident_kernel<MODE, 2><<<grid, block, 0, s>>>(a, xs); break;
-    case 3: linear_resident_kernel<MODE, 3><<<grid, block, 0, s>>>(a, xs); break;
-    default: linear_resident_kernel<MODE, 4><<<grid, block, 0, s>>>(a, xs); break;
+    case 1: linear_resident_kernel<MODE, 1><<<grid, block, 0, s>>>(a, xs, nullptr, 0, 0); break;
+    case 2: linear_resident_kernel<MODE, 2><<<grid, block, 0, s>>>(a, xs, nullptr, 0, 0); break;
+    case 3: linear_resident_kernel<MODE, 3><<<grid, block, 0, s>>>(a, xs, nullptr, 0, 0); break;
+    default: linear_resident_kernel<MODE, 4><<<grid, block, 0, s>>>(a, xs, nullptr, 0, 0); break;
   }
   return launch_status();
 }
@@ -971,6 +971,16 @@ bool resident_preferred(const LinearQuery& q) {
   if (!q.vec_ok || q.K < 1024 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
   if (q.M <= 16) return q.K <= 2048 ? q.N >= 4096 : ((q.M >= 14 && q.N >= 5120) || (q.M >= 5 && q.N >= 10240));
   return q.M <= 32 && q.N >= 98304;
+}
+
+// The one-launch dynamic linear: which of its two kernels, where both take the shape.  The block per CU
+// that quantizes the rows once is ahead almost everywhere (cold weights, us, it | a block per 16 channels
+// each quantizing the rows: K = N = 4096, M = 4: 7.7 | 8.1; N = 11008, M = 4: 12.3 | 15.2; N = 32000, M = 4:
+// 26.3 | 35.2; N = 4096, K = 1024, M = 16: 6.1 | 7.0; N = 16384, K = 1024, M = 1: 6.7 | 10.3; N = 4096,
+// K = 8192, M = 1: 9.8 | 10.1), except one or two rows against a single round of blocks at K = 4096
+// (K = N = 4096, M = 1: 6.6 | 6.1).
+bool dynamic_resident_preferred(int64_t M, int64_t N, int64_t K) {
+  return !(M <= 2 && N <= 4096 && K > 2048 && K <= 4096);
 }
 
 // forced: tmq_linear_desc::kernel - 1 (-1 = automatic choice).
@@ -1455,12 +1465,24 @@ TMQ_EXPORT int tmq_linear_f32(const tmq_linear_desc* d, const tmq_qparams* x_qpa
                                   d->workspace_bytes);
 }
 
+// The float rows of the one-launch dynamic linear as the resident kernel holds them: 16 waves x 64
+// lanes x up to 8 groups of four values (16 groups -- M = 16 at K = 4096 -- spill registers and every
+// CU then reads 256 KB of rows: 14.2 us against 11.0 us for the two launches at N = 4096).
+constexpr int64_t kDynResidentMaxValues = 32768;
+
+TMQ_EXPORT int tmq_linear_dynamic_small_takes(int64_t M, int64_t N, int64_t K) {
+  if (M < 1 || M > 16 || N < 1 || K < 16 || K % 16 != 0 || ceil_div(N, 16) > 0x7fffffff) return 0;
+  if (M * K <= kDynSmallMaxValues) return 1;
+  const int cus = cu_count();
+  return M * K <= kDynResidentMaxValues && resident_limits_ok(M, N, K, K, cus > 0 ? cus : 256) ? 1 : 0;
+}
+
 TMQ_EXPORT int tmq_linear_dynamic_small(const tmq_linear_desc* d, const float* x, int64_t ldx, int reduce_range,
                                         float* y, int64_t ldy, tmq_stream_t stream) {
   if (d == nullptr) return TMQ_ERR_INVALID_ARGUMENT;
   if (d->M < 0 || d->N < 0 || d->K < 0) return TMQ_ERR_INVALID_ARGUMENT;
   if (d->M == 0 || d->N == 0) return TMQ_OK;
-  if (d->M > 16 || d->K < 16 || d->K % 16 != 0 || d->M * d->K > kDynSmallMaxValues) return TMQ_ERR_UNSUPPORTED;
+  if (d->M > 16 || d->K < 16 || d->K % 16 != 0) return TMQ_ERR_UNSUPPORTED;
   if (x == nullptr || y == nullptr || d->w_packed == nullptr || d->w_colsum == nullptr || d->w_scales == nullptr)
     return TMQ_ERR_INVALID_ARGUMENT;
   if (ldx < d->K || ldy < d->N) return TMQ_ERR_INVALID_ARGUMENT;
@@ -1480,9 +1502,31 @@ TMQ_EXPORT int tmq_linear_dynamic_small(const tmq_linear_desc* d, const float* x
   a.lo_f = d->relu ? 0.f : -__builtin_inff();
   a.y = y;
   a.ldy = ldy;
+  hipStream_t s = as_stream(stream);
+  // Two kernels: a block per 16 channels that repeats the work on the input (up to 16384 values), and
+  // one block per CU that does it once for all its channel groups (up to 32768 values, K <= 8192).
+  // desc->kernel pins one for tests: 9 the first, 29 the second.
+  const int cus = cu_count();
+  const bool resident_ok = d->M * d->K <= kDynResidentMaxValues && resident_limits_ok(d->M, d->N, d->K, d->K, cus);
+  const bool small_ok = d->M * d->K <= kDynSmallMaxValues;
+  if ((d->kernel == 9 && !small_ok) || (d->kernel == 29 && !resident_ok) || (!small_ok && !resident_ok))
+    return TMQ_ERR_UNSUPPORTED;
+  const bool resident =
+      resident_ok && (d->kernel == 29 || (d->kernel != 9 && (!small_ok || dynamic_resident_preferred(d->M, d->N, d->K))));
+  if (resident) {
+    const XLinear none{nullptr, 0};
+    const dim3 grid(static_cast<unsigned>(blocks < cus ? blocks : cus)), block(kResidentThreads);
+    const int64_t held = ceil_div(d->M * d->K / 4, kResidentThreads);  // float4 per thread
+    if (held <= 2)
+      linear_resident_kernel<kOutF32, 1, kResidentWaves, 2><<<grid, block, 0, s>>>(a, none, x, ldx, reduce_range);
+    else if (held <= 4)
+      linear_resident_kernel<kOutF32, 1, kResidentWaves, 4><<<grid, block, 0, s>>>(a, none, x, ldx, reduce_range);
+    else
+      linear_resident_kernel<kOutF32, 1, kResidentWaves, 8><<<grid, block, 0, s>>>(a, none, x, ldx, reduce_range);
+    return launch_status();
+  }
   const size_t lds = static_cast<size_t>(d->M) * static_cast<size_t>(d->K + 16);
   const dim3 grid(static_cast<unsigned>(blocks)), block(kDecodeWaves * kWave);
-  hipStream_t s = as_stream(stream);
   const int64_t groups = ceil_div(d->M * d->K / 4, kDecodeWaves * kWave);  // float4 per thread
   if (groups <= 1)
     linear_decode_dynamic_kernel<1><<<grid, block, lds, s>>>(a, x, ldx, reduce_range);

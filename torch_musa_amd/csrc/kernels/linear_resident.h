@@ -22,9 +22,18 @@
 //     flight stay in flight.
 // D[i][j] of v_mfma_i32_16x16x64_i8: lane l, register r -> i = 4 (l / 16) + r (channel),
 // j = l % 16 (activation row).
+//
+// HELD > 0: the dynamically quantized linear in one launch (float rows in, float out, up to
+// 16 rows and HELD x 4096 values): the block reads the float rows instead of codes -- every
+// thread holds HELD groups of four values in registers --, reduces their range, one thread
+// derives the parameters (ChooseQuantizationParams), and the held values are quantized into
+// the same LDS operand layout, product and zero point rounded once, as PyTorch's CPU
+// quantized::linear_dynamic does while packing.  All of it runs under the latency of the
+// first weight requests; the stream that follows is the same.
 #pragma once
 
 #include "gemm_i8_core.h"
+#include "qparams.h"
 
 namespace tmq {
 
@@ -42,8 +51,10 @@ __device__ __forceinline__ void resident_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <int MODE, int MG, int W = kResidentWaves>
-__global__ __launch_bounds__(W * kWave, 4) void linear_resident_kernel(GemmArgs a, XLinear xs) {
+template <int MODE, int MG, int W = kResidentWaves, int HELD = 0>
+__global__ __launch_bounds__(W * kWave, 4) void linear_resident_kernel(GemmArgs a, XLinear xs, const float* __restrict__ xf,
+                                                                       int64_t ldxf, int reduce_range) {
+  static_assert(HELD == 0 || (MODE == kOutF32 && MG == 1 && W == kResidentWaves), "the dynamic form: float output, 16 rows");
   constexpr int D = kResidentDepth;
   constexpr int kXBytes = kResidentXBytes / kResidentWaves * W;  // (eight waves: two blocks share a CU)
   constexpr int kThreads = W * kWave;
@@ -54,6 +65,8 @@ __global__ __launch_bounds__(W * kWave, 4) void linear_resident_kernel(GemmArgs 
   __shared__ __attribute__((aligned(16))) float s_mult[kGroups * 16];
   __shared__ __attribute__((aligned(16))) float s_bdiv[kGroups * 16];
   __shared__ float s_bmul;
+  __shared__ float s_mn[W], s_mx[W];
+  __shared__ float s_scale, s_inv, s_zp;
 
   const int t = threadIdx.x, lane = t % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(t / kWave);
@@ -72,17 +85,30 @@ __global__ __launch_bounds__(W * kWave, 4) void linear_resident_kernel(GemmArgs 
   // ---- requests, oldest first: the activations (L2) ...
   // piece (mg, kb) = 16 rows x 64 bytes: lane -> row lane / 4, 16-byte chunk lane % 4
   // (four lanes ask for one cache line); pieces are dealt round-robin to the waves
-  constexpr int kXPieces = kXBytes / 1024 / W;  // per wave, at most
+  constexpr int kXPieces = HELD > 0 ? 1 : kXBytes / 1024 / W;  // per wave, at most
   v4i xr[kXPieces];
+  constexpr int kHeldN = HELD > 0 ? HELD : 1;
+  v4f held[kHeldN];
   const int sr = lane >> 2, sp = lane & 3;
+  const int k4 = K >> 2, total4 = M * k4;          // (dynamic form) groups of four float values
+  if constexpr (HELD > 0) {
 #pragma unroll
-  for (int j = 0; j < kXPieces; ++j) {
-    const int p = wave + W * j;
-    if (p < MG * KBP) {
-      const int kb = p / MG, mg = p - kb * MG;
-      const int row = mg * 16 + sr, c = kb * 4 + sp;
-      const bool ok = row < M && c < KC;
-      xr[j] = ld16(xs.x + (ok ? static_cast<int64_t>(row) * xs.ldx + c * 16 : 0));
+    for (int u = 0; u < HELD; ++u) {
+      const int e = t + u * kThreads;
+      const int ec = e < total4 ? e : 0;           // unconditional loads keep the load counter exact
+      const int row = ec / k4, c4 = ec - row * k4;
+      held[u] = *reinterpret_cast<const v4f*>(xf + row * ldxf + c4 * 4);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kXPieces; ++j) {
+      const int p = wave + W * j;
+      if (p < MG * KBP) {
+        const int kb = p / MG, mg = p - kb * MG;
+        const int row = mg * 16 + sr, c = kb * 4 + sp;
+        const bool ok = row < M && c < KC;
+        xr[j] = ld16(xs.x + (ok ? static_cast<int64_t>(row) * xs.ldx + c * 16 : 0));
+      }
     }
   }
   // ... the constants of this block's channels (cold): thread -> group slot t / 16, channel t % 16
@@ -122,7 +148,65 @@ __global__ __launch_bounds__(W * kWave, 4) void linear_resident_kernel(GemmArgs 
 
   // ---- activations into LDS: piece (mg, kb), chunk c of row r -> ((4 kb + c) * 16 MG + 16 mg + r) * 16
   for (int i = t; i < 2 * MG * 4 * kWave; i += kThreads) (&s_sum[0][0][0][0])[i] = 0;
-  {
+  XQuant xq;
+  if constexpr (HELD > 0) {
+    // rows past M and bytes past K stay zero: clear the area, then write the codes over it
+    for (int i = t; i < KBP * 64; i += kThreads) *reinterpret_cast<v4i*>(&s_x[i * 16]) = v4i{0, 0, 0, 0};
+    float mn = __builtin_inff(), mx = -__builtin_inff();
+#pragma unroll
+    for (int u = 0; u < HELD; ++u) {
+      if (t + u * kThreads < total4) {
+        const v4f v = held[u];
+        mn = fminf(fminf(mn, v.x), fminf(v.y, fminf(v.z, v.w)));
+        mx = fmaxf(fmaxf(mx, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
+      }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      mn = fminf(mn, __shfl_xor(mn, off, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+    }
+    if (lane == 0) {
+      s_mn[wave] = mn;
+      s_mx[wave] = mx;
+    }
+    resident_barrier();
+    if (t == 0) {
+#pragma unroll
+      for (int w = 1; w < W; ++w) {
+        mn = fminf(mn, s_mn[w]);
+        mx = fmaxf(mx, s_mx[w]);
+      }
+      double sc;
+      int32_t zp;
+      choose_qparams(mn, mx, 0, 255, reduce_range != 0, &sc, &zp);
+      const float scf = static_cast<float>(sc);
+      s_scale = scf;
+      s_inv = 1.0f / scf;  // IEEE division, as the separate quantize kernels
+      s_zp = static_cast<float>(zp);
+    }
+    resident_barrier();
+    const float inv = s_inv, zp_f = s_zp;
+#pragma unroll
+    for (int u = 0; u < HELD; ++u) {
+      const int e = t + u * kThreads;
+      if (e < total4) {
+        const int row = e / k4, c4 = e - row * k4;
+        const v4f v = held[u];
+        uint32_t q = 0;
+        const float f[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float r = __builtin_rintf(__builtin_fmaf(f[j], inv, zp_f));
+          r = fminf(fmaxf(r, 0.f), 255.f);
+          q |= static_cast<uint32_t>(static_cast<int>(r)) << (8 * j);
+        }
+        // bytes 4 c4 .. 4 c4 + 3 of the row: k-block c4 / 16, chunk (c4 / 4) % 4, byte 4 (c4 % 4) of the chunk
+        *reinterpret_cast<uint32_t*>(&s_x[((c4 >> 2) * 16 + row) * 16 + (c4 & 3) * 4]) = q ^ 0x80808080u;
+      }
+    }
+    xq = XQuant{s_scale, 128 - static_cast<int>(zp_f)};
+  } else {
     const int xor_word = static_cast<int>(a.x_xor);
     const v4i xmask = {xor_word, xor_word, xor_word, xor_word};
 #pragma unroll
@@ -135,10 +219,10 @@ __global__ __launch_bounds__(W * kWave, 4) void linear_resident_kernel(GemmArgs 
         *reinterpret_cast<v4i*>(&s_x[(((kb * 4 + sp) * MG + mg) * 16 + sr) * 16]) = v;
       }
     }
+    xq = x_quant(a);
   }
   // ---- the channels' constants, ready for the epilogue
   {
-    const XQuant xq = x_quant(a);
     float mult = 0.f, bdiv = 0.f, bmul = 1.f;
     if constexpr (MODE == kOutF32) {
       mult = xq.scale * c_ws;
