@@ -196,6 +196,21 @@ def test_long_k_as_a_ring_of_phases(cabi, shape, x_signed):
     np.testing.assert_array_equal(acc2, acc)
 
 
+# up to 64 rows against the very largest N: the automatic choice is the pipelined 64 x 128 tile over
+# several rounds (rows mostly padding, ragged channels, K that ends inside a stage)
+@pytest.mark.parametrize("shape, x_signed", [((9, 65600, 2064), False), ((40, 66000, 1040), True)])
+def test_few_rows_against_the_largest_n(cabi, shape, x_signed):
+    say("largest N", shape, x_signed)
+    M, N, K = shape
+    assert cabi.linear_kernel_choice(M, N, K)["kernel"] - 1 == 23
+    c = _tile_case(M, N, K, seed=6500 + M, x_signed=x_signed, relu=M % 2 == 1, bias=True, per_channel=M % 2 == 0)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(acc, oracle.linear_acc32(c["xq"], c["wq"], nthreads=8))
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], c["out_zp"], relu=c["relu"], nthreads=8)
+    _check(y, want, "64 x 128 tiles over several rounds")
+
+
 # up to 64 rows with the activations resident in LDS, one block per CU walking its channel groups:
 # one group and several per block (ragged last round), K that ends inside a k-block / inside the
 # padding to 16 k-blocks, every number of row groups, a single row, both activation types; the last

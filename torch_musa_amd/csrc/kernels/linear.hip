@@ -965,12 +965,21 @@ bool stream_limits_ok(const LinearQuery& q) {
 //     24.0 | 25.6, N = 128256 91.7 | 95.7;  M = 12: N = 49152 38.2 | 39.6, N = 65536 50.3 | 54.4
 //   (fewer rows: level up to N = 32000, then the independent blocks stream faster: N = 128256, M = 1: 89 | 85;
 //   N = 4096 at K >= 4096: level or behind, 6.1 | 5.9 at M = 16)
-//   17 ... 32 rows against the largest N only (N = 128256, K = 4096: 104 against 111 us for 128 x 128 tiles;
-//   N = 32000: 27 against 25.4 us for 64 x 128 tiles).
+//   17 ... 32 rows: never ahead of the tiles (N = 32000: 27 against 25.4 us for 64 x 128 tiles; N = 128256: 104
+//   against 87.7 us).
 bool resident_preferred(const LinearQuery& q) {
-  if (!q.vec_ok || q.K < 1024 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
-  if (q.M <= 16) return q.K <= 2048 ? q.N >= 4096 : ((q.M >= 14 && q.N >= 5120) || (q.M >= 5 && q.N >= 10240));
-  return q.M <= 32 && q.N >= 98304;
+  if (!q.vec_ok || q.K < 1024 || q.M > 16 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
+  return q.K <= 2048 ? q.N >= 4096 : ((q.M >= 14 && q.N >= 5120) || (q.M >= 5 && q.N >= 10240));
+}
+
+// Five rows and more against the very largest N at K > 2048: the pipelined 64 x 128 tiles, mostly padding
+// in their rows, stream such a weight faster than either kernel above -- two and more long-running blocks
+// per CU, each with its own ring of stages (cold weights, K = 4096, us, tiles | rows resident | a block per 16
+// channels: N = 128256: M = 16 85.0 | 93.5 | 118, M = 8 87.3 | 93.5 | 97.2, M = 1 87.4 | 88 | 85.0;
+// N = 65536: M = 16 47.6 | 51.4 | 63.8, M = 8 47.6 | 48.9 | 51.2; below, the resident rows are ahead:
+// N = 49152, M = 16: 40.1 | 38.7; N = 32000: 26.8 | 25.8; at K = 2048 the two are level up to N = 128256).
+bool huge_n_tiles_preferred(const LinearQuery& q) {
+  return q.vec_ok && q.M >= 5 && q.M <= 16 && q.K > 2048 && q.N >= 65536;
 }
 
 // The one-launch dynamic linear: which of its two kernels, where both take the shape.  The block per CU
@@ -988,6 +997,10 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
   LinearChoice c;
   if (!q.vec_ok || forced == 9) {
     c.cfg = 9;
+    return c;
+  }
+  if (forced < 0 && huge_n_tiles_preferred(q)) {
+    c.cfg = 23;
     return c;
   }
   if (forced < 0 && resident_preferred(q)) {
@@ -1064,12 +1077,15 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
       // all resident at once: M = 640, N = K = 8192: 53.9 against 59.7 us; N = 8192, K = 4096:
       // 30.2 against 31.6 us; at K = 2048 the 128x256 tiles stay ahead)
       cfg = K >= 4096 && nblk(128, 128) <= 320 ? 7 : cfg128x256;
-    else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && nblk(64, 128) <= 256)
+    else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && (nblk(64, 128) <= 256 || M <= 64))
       // a few hundred rows whose 128 x 128 tiles would leave half the chip idle and whose
       // 64 x 64 tiles need a second round: 64 rows x 128 channels, one round (K = N = 4096,
       // cold weights: M = 448: 24.6 -> 19.1 us, M = 512: 24.8 -> 19.3 us; K = 2048: 14.7 -> 11.7 us;
       // N = 8192, M = 192: 25.9 -> 19.9 us; against N = 1024 the 128 x 128 tiles stay ahead:
-      // M = 1536, K = 4096: 17.4 against 20.2 us, and at K = N = 2048, M = 1024: 11.5 against 12.2 us)
+      // M = 1536, K = 4096: 17.4 against 20.2 us, and at K = N = 2048, M = 1024: 11.5 against 12.2 us);
+      // up to 64 rows also over several rounds, ahead of 128 x 128 tiles that are three quarters padding
+      // (M = 32, K = 4096: N = 65536 48.2 against 53.4 us, N = 128256 87.7 against 95 us; K = 2048, N = 65536:
+      // 26.5 against 30.8 us; N = 49152: level)
       cfg = cfg_half;
     else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
       cfg = 22;
