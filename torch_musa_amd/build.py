@@ -50,7 +50,12 @@ DEVICE_FLAGS = [
 # compiler moved to scratch memory would be copied before its load has landed, so the
 # build fails if any of them uses scratch (the compiler reports each kernel's resources).
 NO_SCRATCH_KERNELS = ("gemm_i8_wring_kernel",)
-RESOURCE_REMARKS = ["-Rpass-analysis=kernel-resource-usage"]
+RESOURCE_REMARKS = ["-Rpass-analysis=kernel-resource-usage", "-save-temps=obj"]
+# The same kernels, on the assembly of the same compilation: besides the request itself and the
+# matrix instruction that consumes a fragment, nothing in the generated code may touch a fragment's
+# registers once the request for them is out (a copy the register allocator placed between a
+# request and its wait would move stale data).
+IN_FLIGHT_KERNELS = ("gemm_i8_wring_kernel",)
 
 
 def _needs_register_check(obj):
@@ -73,6 +78,75 @@ def _check_no_scratch(remarks, kernels):
     missing = set(kernels) - seen
     if missing:
         raise RuntimeError(f"no resource report for {sorted(missing)}: the register check did not run")
+
+
+def _vgprs(operand_text):
+    """VGPR numbers named in an operand list: v7, v[8:11]."""
+    import re
+    regs = set()
+    for m in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", operand_text):
+        if m.group(3) is not None:
+            regs.add(int(m.group(3)))
+        else:
+            regs.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    return regs
+
+
+def _check_in_flight_registers(asm_path, kernels):
+    import re
+    request = re.compile(r"^\s*global_load_dwordx4\s+(v\[\d+:\d+\]),\s*v\d+,\s*s\[\d+:\d+\]")
+    text = open(asm_path).read().split("\n")
+    seen = set()
+    name, body = None, []
+    def check(name, body):
+        pending = {}                                # register -> line of the request that is on its way
+        requests = 0
+        for i, line in enumerate(body):
+            code = line.split(";")[0].strip()
+            if not code or code.endswith(":") or code.startswith("."):
+                continue
+            m = request.match(line)
+            if m:
+                requests += 1
+                for r in _vgprs(m.group(1)):
+                    pending[r] = i
+                continue
+            touched = _vgprs(code) & pending.keys()
+            if not touched:
+                continue
+            if code.startswith("v_mfma_"):
+                ops = code.split(None, 1)[1].split(",")
+                # a fragment is consumed as the first source operand, behind a wait for the requests;
+                # its registers are free again from there on
+                if touched - _vgprs(ops[1]):
+                    raise RuntimeError(f"{name}: a v_mfma touches a fragment on its way other than as its first "
+                                       f"source (registers {sorted(touched - _vgprs(ops[1]))}): {code}")
+                if not any("s_waitcnt vmcnt" in b for b in body[max(pending[r] for r in touched):i]):
+                    raise RuntimeError(f"{name}: no wait between a fragment's request and {code}")
+                for r in touched:
+                    del pending[r]
+                continue
+            raise RuntimeError(f"{name}: an instruction other than the request and the consuming v_mfma touches a "
+                               f"fragment on its way (registers {sorted(touched)}, requested at line "
+                               f"{min(pending[r] for r in touched)} of the kernel): {code}")
+        if requests == 0:
+            raise RuntimeError(f"{name}: no fragment requests found: the in-flight register check did not run")
+    for line in text:
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            name, body = m.group(1), []
+            continue
+        if name is not None:
+            body.append(line)
+            if "s_endpgm" in line:
+                for k in kernels:
+                    if k in name:
+                        check(name, body)
+                        seen.add(k)
+                name = None
+    missing = set(kernels) - seen
+    if missing:
+        raise RuntimeError(f"no assembly for {sorted(missing)}: the in-flight register check did not run")
 
 
 def _run(cmd, verbose):
@@ -120,6 +194,16 @@ def _build_hip_library(sources, lib_path, verbose):
     for (obj, _), out in zip(jobs, outs):
         if _needs_register_check(obj):
             _check_no_scratch(out, NO_SCRATCH_KERNELS)
+            stem = os.path.basename(obj).split(".")[0]
+            temps = [f for f in os.listdir(OBJ) if f.startswith(stem + "-") or f.startswith(stem + ".hip-")]
+            asm = [f for f in temps if f.endswith(f"{ARCH}.s")]
+            if len(asm) != 1:
+                raise RuntimeError(f"expected one device assembly file for {stem}, found {asm}")
+            try:
+                _check_in_flight_registers(os.path.join(OBJ, asm[0]), IN_FLIGHT_KERNELS)
+            finally:
+                for f in temps:                      # tens of MB of intermediates: not part of the build's output
+                    os.remove(os.path.join(OBJ, f))
     _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", lib_path]
          + [j[0] for j in jobs], verbose)
     return lib_path
