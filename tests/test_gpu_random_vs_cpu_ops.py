@@ -80,6 +80,40 @@ def test_linear_ops(seed):
     assert done >= 25
 
 
+@pytest.mark.parametrize("seed", list(range(1, 7)))
+def test_linear_ops_few_rows_many_channels(seed):
+    """Decode-sized batches against wide layers: the kernels that stream the weights (a block per 16
+    channels, rows resident in LDS as one or two blocks per CU, their float-input forms, tiles over several
+    rounds) against PyTorch's CPU ops, static and dynamic."""
+    rng = np.random.default_rng(900 + seed)
+    for it in range(14):
+        M = int(rng.choice([1, 2, 4, 5, 8, 12, 14, 16, 17, 32]))
+        K = int(rng.choice([1024, 1040, 2048, 3072, 4096, 8192]))
+        N = int(rng.choice([4096, 5120, 8200, 11008, 16400, 33000, 66000]))
+        pc, relu, bias = (bool(rng.integers(2)) for _ in range(3))
+        if K * N > 1.4e8:
+            continue
+        say("random decode-sized linear", seed, it, (M, K, N), pc, relu, bias)
+        torch.manual_seed(7000 * seed + it)
+        x, w = torch.randn(M, K) * float(rng.uniform(0.5, 3)), torch.randn(N, K) * 0.05
+        b = torch.randn(N) * 2 if bias else None
+        xq = torch.quantize_per_tensor_dynamic(x, torch.quint8, False)
+        if pc:
+            s = (w.abs().amax(dim=1) / 127).clamp_min(1e-4).double()
+            wq = torch.quantize_per_channel(w, s, torch.zeros(N, dtype=torch.int64), 0, torch.qint8)
+        else:
+            wq = torch.quantize_per_tensor(w, float(w.abs().max() / 127), 0, torch.qint8)
+        cpu_packed = torch.ops.quantized.linear_prepack(wq, b)
+        gpu_packed = torch.ops.quantized.linear_prepack(wq.cuda(), None if b is None else b.cuda())
+        out_scale = max(float((x @ w.t()).std()) / 40, 1e-3)
+        op = torch.ops.quantized.linear_relu if relu else torch.ops.quantized.linear
+        _same_q(op(xq.cuda(), gpu_packed, out_scale, 100), op(xq, cpu_packed, out_scale, 100),
+                f"linear {(M, K, N)} pc={pc} relu={relu} bias={bias}")
+        dyn = torch.ops.quantized.linear_relu_dynamic if relu else torch.ops.quantized.linear_dynamic
+        assert torch.equal(dyn(x.cuda(), gpu_packed, False).cpu(), dyn(x, cpu_packed, False)), \
+            f"linear_dynamic {(M, K, N)} pc={pc} relu={relu} bias={bias}"
+
+
 @pytest.mark.parametrize("seed", list(range(1, 13)))
 def test_conv_and_glue_ops(seed):
     rng = np.random.default_rng(100 + seed)
