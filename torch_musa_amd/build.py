@@ -56,6 +56,8 @@ RESOURCE_REMARKS = ["-Rpass-analysis=kernel-resource-usage", "-save-temps=obj"]
 # registers once the request for them is out (a copy the register allocator placed between a
 # request and its wait would move stale data).
 IN_FLIGHT_KERNELS = ("gemm_i8_wring_kernel",)
+# Kernels that wait for their copies into LDS with a literal count of the weight loads issued after them.
+COUNTED_LOAD_KERNELS = ("gemm_i8_wstream_kernel",)
 
 
 def _needs_register_check(obj):
@@ -149,6 +151,46 @@ def _check_in_flight_registers(asm_path, kernels):
         raise RuntimeError(f"no assembly for {sorted(missing)}: the in-flight register check did not run")
 
 
+def _check_counted_loads(asm_path, kernels):
+    """Kernels whose copies into LDS are waited for with a literal `s_waitcnt vmcnt(N)` that counts on N
+    younger weight loads: the compiler must have emitted at least N loads between the last copy and the wait."""
+    import re
+    text = open(asm_path).read().split("\n")
+    seen = set()
+    name, body = None, []
+    for line in text:
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            name, body = m.group(1), []
+            continue
+        if name is None:
+            continue
+        body.append(line)
+        if "s_endpgm" not in line:
+            continue
+        for k in kernels:
+            if k not in name:
+                continue
+            copies = [i for i, b in enumerate(body) if "global_load_lds_dwordx4" in b]
+            waits = [(i, int(re.search(r"vmcnt\((\d+)\)", b).group(1))) for i, b in enumerate(body)
+                     if i > 0 and "#ASMSTART" in body[i - 1] and re.search(r"s_waitcnt vmcnt\(\d+\)", b)]
+            if not copies or not waits:
+                raise RuntimeError(f"{name}: copies or their wait not found: the load count check did not run")
+            wait_line, counted = next(((i, n) for i, n in waits if i > copies[-1]), (None, None))
+            if wait_line is None:
+                raise RuntimeError(f"{name}: no wait behind the last copy into LDS")
+            loads = sum(1 for b in body[copies[-1]:wait_line]
+                        if re.match(r"^\s*global_load_dwordx4\s", b) and "lds" not in b)
+            if loads < counted:
+                raise RuntimeError(f"{name}: vmcnt({counted}) behind the copies counts on {counted} younger loads, "
+                                   f"the compiler emitted {loads}")
+            seen.add(k)
+        name = None
+    missing = set(kernels) - seen
+    if missing:
+        raise RuntimeError(f"no assembly for {sorted(missing)}: the load count check did not run")
+
+
 def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -201,6 +243,7 @@ def _build_hip_library(sources, lib_path, verbose):
                 raise RuntimeError(f"expected one device assembly file for {stem}, found {asm}")
             try:
                 _check_in_flight_registers(os.path.join(OBJ, asm[0]), IN_FLIGHT_KERNELS)
+                _check_counted_loads(os.path.join(OBJ, asm[0]), COUNTED_LOAD_KERNELS)
             finally:
                 for f in temps:                      # tens of MB of intermediates: not part of the build's output
                     os.remove(os.path.join(OBJ, f))
