@@ -192,7 +192,7 @@ def _check_choice(c, m, n, k, ldx, out, workspace, misaligned, forced=0, cus=256
             assert mg == 1 and 16 * _ceil(k, 512) * 512 <= 64 * 1024 and 2 * cus <= _ceil(n, 16) <= 64 * cus, what
             assert c["blocks"] == min(tiles, 2 * cus), what
         if forced == 0:                             # rows that share the streamed weights, or a short K
-            assert k >= 1024 and m <= 16 and (k <= 2048 or m >= 14 or (m >= 5 and n >= 10240)), what
+            assert k >= 1024 and m <= 32 and (m <= 16 or 10240 <= n <= 20480), what
         return
     else:                                           # register-staged tiles take any aligned shape
         assert cfg in (0, 1, 2, 3, 4, 5, 22, 23), what

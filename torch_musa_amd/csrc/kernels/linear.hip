@@ -955,7 +955,7 @@ bool stream_limits_ok(const LinearQuery& q) {
 
 // Where the kernel that keeps the activations in LDS is ahead of a block per 16 channels
 // (cold weights, us, resident | streaming; neither depends on N beyond what is shown):
-//   K <= 2048, from N = 4096 on, any M <= 16:  N = 4096, K = 1024: 3.9 | 4.2 ... 4.5;  N = 8192, K = 1024:
+//   K <= 2048, from N = 2048 on, any M <= 16:  K = N = 2048: 4.0 ... 4.2 | 4.2 ... 4.7;  N = 4096, K = 1024: 3.9 | 4.2 ... 4.5;  N = 8192, K = 1024:
 //     4.8 ... 5.0 | 5.8 ... 6.3;  N = 4096, K = 2048: 4.5 | 4.7 ... 5.0;  N = 65536, K = 2048: 24.5 | 35 ... 42
 //   longer K, 14 rows and more (the streaming blocks re-read the rows from the L2s), from N = 5120 on:
 //     K = 4096, M = 16: N = 5120 7.7 | 8.6, N = 11008 10.6 | 12.3, N = 32000 25.4 | 32.2, N = 128256 97 | 122;
@@ -965,11 +965,16 @@ bool stream_limits_ok(const LinearQuery& q) {
 //     24.0 | 25.6, N = 128256 91.7 | 95.7;  M = 12: N = 49152 38.2 | 39.6, N = 65536 50.3 | 54.4
 //   (fewer rows: level up to N = 32000, then the independent blocks stream faster: N = 128256, M = 1: 89 | 85;
 //   N = 4096 at K >= 4096: level or behind, 6.1 | 5.9 at M = 16)
-//   17 ... 32 rows: never ahead of the tiles (N = 32000: 27 against 25.4 us for 64 x 128 tiles; N = 128256: 104
-//   against 87.7 us).
+//   a K that leaves the streaming blocks a short last pass (K = N = 5120: 8.4 ... 8.7 | 9.2 ... 11.3 at M = 1 ... 12)
+//   17 ... 32 rows: a narrow band between the tiles of 32 rows, which no longer fit one round, and the 64 x 128
+//   tiles (K = 4096, M = 24 / 32: N = 11008 11.9 / 12.2 against 12.5 / 12.7 us, N = 16384 15.5 / 15.7 against
+//   16.4 / 16.7 us; N = 8192: level with 32 x 32 tiles; N = 32000: 26.6 against 24.5 us for 64 x 128 tiles).
 bool resident_preferred(const LinearQuery& q) {
-  if (!q.vec_ok || q.K < 1024 || q.M > 16 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
-  return q.K <= 2048 ? q.N >= 4096 : ((q.M >= 14 && q.N >= 5120) || (q.M >= 5 && q.N >= 10240));
+  if (!q.vec_ok || q.K < 1024 || q.M > 32 || !resident_limits_ok(q.M, q.N, q.K, q.ldx, 256)) return false;
+  if (q.M > 16) return q.K > 2048 && q.N >= 10240 && q.N <= 20480;
+  if (q.K <= 2048) return q.N >= 2048;
+  if (q.K > 4096 && q.K % 4096 != 0 && q.K % 4096 <= 2048 && q.N >= 5120) return true;
+  return (q.M >= 14 && q.N >= 5120) || (q.M >= 5 && q.N >= 10240);
 }
 
 // Five rows and more against the very largest N at K > 2048: the pipelined 64 x 128 tiles, mostly padding
@@ -1089,7 +1094,9 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
       cfg = cfg_half;
     else if (N >= 2048 && (N >= 4096 || K >= 4096) && nblk(64, 64) > 256 && nblk(128, 64) <= 256)
       cfg = 22;
-    else if (nblk(128, 128) >= 128)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096)
+    else if (nblk(128, 128) >= 128 && M > 64)  // (64 tiles: 64x64 wins, 15.2 against 17.9 us at M = 256, K = N = 4096;
+                                               // up to 64 rows half of every tile is padding: M = 64, N = 16384, K = 4096:
+                                               // 27.5 us against 17.5 us for the 64 x 64 tiles that walk K in phases)
       cfg = 7;
     else if (onepass_ok && K >= 3072 && K <= kWringMaxK && nblk(64, 64) <= 256 && N * K <= (int64_t{1} << 24))
       // one round of 64 x 64 tiles against a long K: eight waves split K, weights through
