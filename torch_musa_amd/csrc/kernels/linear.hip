@@ -1073,8 +1073,11 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
     const int cfg128x256 = t128x256 <= 256 ? 19 : 17;
     // equal tile counts: the 64 x 128 tile; more row tiles than its mirror image has fewer
     // blocks and idle CUs (M = 192: N = 6144, K = 3072: 17.1 against 15.3 us with 128 x 64;
-    // N = 4096, K = 11008: 46.8 against 43.4 us)
-    const int cfg_half = nblk(128, 64) <= 256 && nblk(128, 64) > nblk(64, 128) ? 22 : 23;
+    // N = 4096, K = 11008: 46.8 against 43.4 us); up to 96 rows fill three of the 128 x 64 tile's
+    // four row strips and it is ahead at equal counts too (M = 96, N = 13824, K = 5120: 28.4
+    // against 31.0 us; N = 11008, K = 4096: 20.2 against 21.2 us)
+    const int cfg_half =
+        nblk(128, 64) <= 256 && (nblk(128, 64) > nblk(64, 128) || (M <= 96 && nblk(128, 64) == nblk(64, 128))) ? 22 : 23;
     if (t128x256 > 256 && rows_used(256))
       cfg = t256 > 256 && t256 <= 400 ? 17 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
     else if (t128x256 >= 160 && rows_used(128))
@@ -1098,13 +1101,14 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
                                                // up to 64 rows half of every tile is padding: M = 64, N = 16384, K = 4096:
                                                // 27.5 us against 17.5 us for the 64 x 64 tiles that walk K in phases)
       cfg = 7;
-    else if (onepass_ok && K >= 3072 && K <= kWringMaxK && nblk(64, 64) <= 256 && N * K <= (int64_t{1} << 24))
+    else if (onepass_ok && K >= 3072 && K <= kWringMaxK && nblk(64, 64) <= 256 && N * K <= (int64_t{3} << 23))
       // one round of 64 x 64 tiles against a long K: eight waves split K, weights through
       // registers, activations through a ring per wave, no barrier before the partial tiles
       // meet (cold weights, K = N = 4096: M = 130 12.1 -> 11.8 us, M = 192 14.0 -> 12.8 us,
       // M = 256 14.3 -> 13.6 us; N = 2048: M = 512 14.0 -> 13.0 us; K = 3072: M = 192
       // 13.0 -> 12.1 us; behind the two wave groups at K = 2560 (12.3 against 11.7 us) and
-      // against 32 MB of weights, N = 8192: 15.3 against 14.6 us)
+      // against 32 MB of weights, N = 8192: 15.3 against 14.6 us; 24 MB, N = 6144, K = 4096,
+      // M = 128: 13.7 against 15.0 us)
       cfg = 27;
     else if (onepass_ok && phased_ring_preferred(M, N, K))
       cfg = 21;
