@@ -389,3 +389,23 @@ def test_qunary_unaligned_and_large(cabi):
     np.testing.assert_array_equal(y, oracle.qunary(x[3:], "gelu", 0.05, 120, 0.05, 120))
     y = host(cabi.qunary(xd, "sigmoid", 0.05, 120, 1 / 256, 0))
     np.testing.assert_array_equal(y, oracle.qunary(x, "sigmoid", 0.05, 120, 1 / 256, 0))
+
+
+def test_qunary_several_sweeps_of_the_grid(cabi):
+    # more 16-byte groups than the largest grid has threads (4096 blocks), a partial last sweep
+    # and a few stray bytes: every thread walks the array several times.  The output is a
+    # function of the code alone, so the oracle's 256 answers check all of it.
+    say("qunary several sweeps of the grid")
+    import torch
+    n = 2048 * 16384 * 2 + 16 * 700 + 7
+    g = torch.Generator(device="cuda").manual_seed(5)
+    xd = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    codes = np.arange(256, dtype=np.uint8)
+    for kind, (os_, oz) in (("gelu", (0.05, 120)), ("sigmoid", (1 / 256, 0))):
+        table = torch.from_numpy(oracle.qunary(codes, kind, 0.05, 120, os_, oz)).cuda()
+        y = cabi.qunary(xd, kind, 0.05, 120, os_, oz)
+        assert torch.equal(y, table[xd.long()])
+        xs = xd.view(torch.int8)
+        table_s = torch.from_numpy(oracle.qunary(codes.view(np.int8), kind, 0.05, -8, os_, oz - 128)).cuda()
+        ys = cabi.qunary(xs, kind, 0.05, -8, os_, oz - 128)
+        assert torch.equal(ys.view(torch.uint8), table_s.view(torch.uint8)[xd.long()])
