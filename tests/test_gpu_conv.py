@@ -128,6 +128,68 @@ def test_conv_auto_path_shapes(cabi, spec):
     _check(y, want, "auto conv")
 
 
+@pytest.mark.parametrize("spec", [
+    (2, 64, 64, 3, 64, 7, 2, 3, 1, 1),       # an image network's first layer: 7 x 7 stride 2, 3 -> 64
+    (2, 33, 33, 3, 32, 3, 2, 1, 1, 1),       # 3 x 3 stride 2, 3 -> 32; image rows of 99 bytes: byte copies
+    (1, 36, 36, 3, 48, 6, 2, 2, 1, 1),       # 6 x 6 stride 2
+    (3, 28, 28, 24, 144, 1, 1, 0, 1, 1),     # pointwise, 24 channels in, three 64-channel blocks out
+    (2, 14, 14, 40, 100, 1, 1, 0, 1, 1),     # pointwise, nothing a multiple of 16
+    (2, 30, 30, 1, 16, 5, 1, 2, 1, 1),       # one input channel
+    (1, 20, 20, 4, 20, 3, 1, 1, 1, 1),       # four input channels, 20 out: byte stores
+    (1, 8, 600, 3, 16, 3, 2, 1, 1, 1),       # 300 output columns: three tile columns
+    (1, 300, 9, 3, 8, 3, 1, 1, 1, 1),        # narrow and tall
+    (2, 19, 23, 8, 64, 3, 1, 0, 1, 1),       # eight channels, 3 x 3: runs of 24 bytes
+    (1, 9, 9, 5, 7, 4, 3, 0, 1, 1),          # 4 x 4 stride 3, 5 -> 7 channels
+    (2, 12, 12, 48, 32, 1, 2, 0, 1, 1),      # a multiple of 16 (pinned only): one run of 48 bytes
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_few_channels_as_byte_runs(cabi, spec, x_signed):
+    say("conv byte runs", spec, x_signed)
+    c = _conv_case(*spec, seed=sum(spec) + 7, x_signed=x_signed, relu=not x_signed)
+    want_acc = oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                   c["groups"], c["x_zp"], nthreads=8)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    for path in (4, -1):
+        cabi.force_conv_path(path)
+        try:
+            y, acc, _ = _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+        np.testing.assert_array_equal(acc, want_acc)
+        _check(y, want, f"path {path}")
+
+
+def test_conv_byte_runs_limits(cabi):
+    """groups, dilation and kernel rows beyond 256 padded bytes are not this kernel's."""
+    say("conv byte runs limits")
+    for spec in [(1, 12, 12, 6, 6, 3, 1, 1, 1, 2), (1, 12, 12, 3, 8, 3, 1, 2, 2, 1), (1, 24, 24, 3, 8, 11, 1, 0, 1, 1)]:
+        c = _conv_case(*spec, seed=3)
+        cabi.force_conv_path(4)
+        try:
+            with pytest.raises(cabi.TmqError):
+                _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+        y, acc, _ = _run(cabi, c)   # the direct kernel takes them
+        np.testing.assert_array_equal(
+            acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"], c["groups"], c["x_zp"]))
+
+
+def test_conv_first_layer_full_size(cabi):
+    """[32, 224, 224, 3] (x) [64, 7, 7, 3], stride 2, pad 3, with ReLU: the first layer of a ResNet at batch 32."""
+    say("conv first layer full size")
+    c = _conv_case(32, 224, 224, 3, 64, 7, 2, 3, 1, 1, seed=77, relu=True)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"], c["groups"], c["x_zp"],
+                                 nthreads=8))
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], c["stride"],
+                         c["padding"], c["dilation"], c["groups"], c["out_scale"], c["out_zp"], relu=True, nthreads=8)
+    _check(y, want, "first layer")
+
+
 def test_c5_full_size(cabi):
     """benchmark configuration 5: [32,56,56,64] (x) [64,3,3,64], stride 1, pad 1."""
     say("C5 full size")
@@ -167,12 +229,16 @@ def _run_fused(cabi, c):
     return host(y)
 
 
-@pytest.mark.parametrize("path", [-1, 2, 3], ids=["auto", "gemm", "direct"])
+@pytest.mark.parametrize("path", [-1, 2, 3, 4], ids=["auto", "gemm", "direct", "runs"])
 @pytest.mark.parametrize("c", cases.conv_fused_cases(), ids=lambda c: c["name"])
 def test_conv_fused(cabi, golden, c, path):
     say("conv fused", c["name"], path)
     if path == 2 and (c["xq"].shape[3] // c["groups"]) % 16 != 0:
         pytest.skip("the MFMA kernels need 16-channel blocks")
+    if path == 4:
+        oc_, kh_, kw_, ic_ = c["wq"].shape
+        if c["groups"] != 1 or kh_ * (-(-kw_ * ic_ // 16) * 16) > 256:
+            pytest.skip("the byte-run kernel takes one group and kernel rows of at most 256 padded bytes in all")
     cabi.force_conv_path(path)
     try:
         y = _run_fused(cabi, c)

@@ -9,6 +9,7 @@
 #include <atomic>
 #include <type_traits>
 
+#include "conv_runs.h"
 #include "conv_tile.h"
 #include "gemm_i8_core.h"
 
@@ -343,6 +344,88 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
   }
 }
 
+// Tile shape and LDS use of the few-channel kernel (conv_runs.h) for one problem; false
+// when the kernel does not take it: groups, dilation, kernel rows of more than 256 padded bytes.
+struct RunPlan {
+  int RL, RP, KS, TR, TW, mtw, rows_in, pitch, lds;
+};
+bool plan_runs(const ConvShape& s, RunPlan* p) {
+  if (s.groups != 1 || s.dh != 1 || s.dw != 1) return false;
+  const int64_t RL = s.KW * s.IC, RP = round_up(RL, 16);
+  if (s.KH * RP > 64 * kCrMaxKS) return false;
+  const int64_t KS = ceil_div(s.KH * RP, 64);
+  int64_t TW = s.OW < 128 ? s.OW : 128;
+  int64_t TR = ceil_div(8, ceil_div(TW, 16));  // eight 16-pixel pieces per tile: two turns per wave
+  TR = TR > s.OH ? s.OH : TR;
+  for (;;) {
+    const int64_t rows_in = (TR - 1) * s.sh + s.KH;
+    const int64_t pitch = round_up((TW - 1) * s.sw * s.IC + RP + 8, 4);
+    const int64_t lds = KS * 4096 + rows_in * pitch;
+    if (lds <= 48 * 1024) {
+      p->RL = static_cast<int>(RL); p->RP = static_cast<int>(RP); p->KS = static_cast<int>(KS);
+      p->TR = static_cast<int>(TR); p->TW = static_cast<int>(TW); p->mtw = static_cast<int>(ceil_div(TW, 16));
+      p->rows_in = static_cast<int>(rows_in); p->pitch = static_cast<int>(pitch); p->lds = static_cast<int>(lds);
+      return true;
+    }
+    if (TR > 1)
+      TR = (TR + 1) / 2;
+    else if (TW > 16)
+      TW = round_up(TW / 2, 16);
+    else
+      return false;
+  }
+}
+
+template <int MODE>
+int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan& p, const PostOps& po, float zp_f,
+                     float lo_f, float hi_f, void* out, hipStream_t stream) {
+  ConvRunArgs a{};
+  a.x = static_cast<const uint8_t*>(d->x);
+  a.w_packed = static_cast<const uint8_t*>(d->w_packed);
+  a.colsum = d->w_colsum;
+  a.w_scales = d->w_scales;
+  a.bias = d->bias;
+  a.y = out;
+  a.w_kchunks = s.KC;
+  a.H = static_cast<int>(s.H); a.W = static_cast<int>(s.W); a.IC = static_cast<int>(s.IC);
+  a.OH = static_cast<int>(s.OH); a.OW = static_cast<int>(s.OW); a.OC = static_cast<int>(s.OC);
+  a.KH = static_cast<int>(s.KH); a.KW = static_cast<int>(s.KW);
+  a.sh = static_cast<int>(s.sh); a.sw = static_cast<int>(s.sw);
+  a.ph = static_cast<int>(s.ph); a.pw = static_cast<int>(s.pw);
+  a.ICp = static_cast<int>(s.ICgp);
+  a.RL = p.RL; a.RP = p.RP; a.KS = p.KS;
+  a.TR = p.TR; a.TW = p.TW; a.mtw = p.mtw;
+  a.rows_in = p.rows_in; a.pitch = p.pitch;
+  a.uniform_rows = (s.W * s.IC) % 4 == 0 ? 1 : 0;
+  a.tiles_h = static_cast<int>(ceil_div(s.OH, p.TR));
+  a.tiles_w = static_cast<int>(ceil_div(s.OW, p.TW));
+  a.tiles = s.B * a.tiles_h * a.tiles_w;
+  a.vec = aligned(out, 16) && s.OC % (MODE == kOutAcc32 ? 4 : 16) == 0 ? 1 : 0;
+  a.w_scale_stride = d->w_per_channel ? 1 : 0;
+  a.x_xor = d->x_signed ? 0u : 0x80808080u;
+  a.pad_word = 0x01010101u * static_cast<uint32_t>(static_cast<uint8_t>(d->x_zero_point));
+  a.acc_coef = (d->x_signed ? 0 : 128) - d->x_zero_point;
+  a.x_scale = d->x_scale;
+  a.out_scale = d->out_scale;
+  a.zp_f = zp_f; a.lo_f = lo_f; a.hi_f = hi_f;
+  a.rcp_p4 = 4.0f / static_cast<float>(p.pitch);
+  a.post = po;
+  const int64_t by = ceil_div(s.OC, kCrBN);
+  if (by > 65535) return TMQ_ERR_UNSUPPORTED;
+  // three blocks per CU (their registers), each with its weights in registers for every tile it walks
+  const int64_t bx = a.tiles < 768 ? a.tiles : 768;
+  const dim3 grid(static_cast<unsigned>(bx), static_cast<unsigned>(by)), block(kCrThreads);
+  if constexpr (MODE == kOutAcc32) {
+    conv_runs_kernel<MODE, false><<<grid, block, p.lds, stream>>>(a);
+  } else {
+    if (po.any())
+      conv_runs_kernel<MODE, true><<<grid, block, p.lds, stream>>>(a);
+    else
+      conv_runs_kernel<MODE, false><<<grid, block, p.lds, stream>>>(a);
+  }
+  return launch_status();
+}
+
 template <int MODE>
 int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, hipStream_t stream) {
   ConvShape s;
@@ -387,6 +470,13 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   const int forced = d->kernel > 0 ? d->kernel : -1;
   const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
   if ((forced == 1 || forced == 2) && !mfma_ok) return TMQ_ERR_UNSUPPORTED;
+  // channel counts (or an address) the 16-byte chunks of the kernels below cannot take:
+  // kernel rows as runs of bytes where they are short enough
+  if (forced == 4 || (forced < 0 && !mfma_ok)) {
+    RunPlan rp;
+    if (plan_runs(s, &rp)) return launch_conv_runs<MODE>(d, s, rp, po, zp_f, lo_f, hi_f, out, stream);
+    if (forced == 4) return TMQ_ERR_UNSUPPORTED;
+  }
   if (!mfma_ok || forced == 3) {
     PlainArgs p{};
     p.x = static_cast<const uint8_t*>(d->x);
