@@ -349,31 +349,38 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
 struct RunPlan {
   int RL, RP, KS, TR, TW, mtw, rows_in, pitch, lds;
 };
-bool plan_runs(const ConvShape& s, RunPlan* p) {
+bool plan_runs(const ConvShape& s, int forced_rows, RunPlan* p) {
   if (s.groups != 1 || s.dh != 1 || s.dw != 1) return false;
   const int64_t RL = s.KW * s.IC, RP = round_up(RL, 16);
   if (s.KH * RP > 64 * kCrMaxKS) return false;
   const int64_t KS = ceil_div(s.KH * RP, 64);
-  int64_t TW = s.OW < 128 ? s.OW : 128;
-  int64_t TR = ceil_div(8, ceil_div(TW, 16));  // eight 16-pixel pieces per tile: two turns per wave
-  TR = TR > s.OH ? s.OH : TR;
-  for (;;) {
-    const int64_t rows_in = (TR - 1) * s.sh + s.KH;
+  // Tile = TR output rows x TW columns.  The staged image rows of a tile pass through
+  // kCrStage registers per thread; among the shapes that fit, the one with the shortest
+  // schedule: rounds of tiles over the blocks the chip holds (three per CU) times the
+  // turns its four waves need for the tile's 16-pixel pieces.
+  constexpr int64_t kSlots = 3 * 256, kStageBytes = int64_t{kCrStage} * kCrThreads * 4;
+  int64_t best = -1;
+  for (int64_t TW = s.OW < 128 ? s.OW : 128;; TW = round_up(TW / 2, 16)) {
+    const int64_t mtw = ceil_div(TW, 16);
     const int64_t pitch = round_up((TW - 1) * s.sw * s.IC + RP + 8, 4);
-    const int64_t lds = KS * 4096 + rows_in * pitch;
-    if (lds <= 48 * 1024) {
-      p->RL = static_cast<int>(RL); p->RP = static_cast<int>(RP); p->KS = static_cast<int>(KS);
-      p->TR = static_cast<int>(TR); p->TW = static_cast<int>(TW); p->mtw = static_cast<int>(ceil_div(TW, 16));
-      p->rows_in = static_cast<int>(rows_in); p->pitch = static_cast<int>(pitch); p->lds = static_cast<int>(lds);
-      return true;
+    for (int64_t TR = 1; TR <= s.OH && TR <= 8; ++TR) {
+      const int64_t rows_in = (TR - 1) * s.sh + s.KH;
+      if (rows_in * pitch > kStageBytes) break;
+      if (forced_rows > 0 && TR != forced_rows) continue;
+      const int64_t tiles = s.B * ceil_div(s.OH, TR) * ceil_div(s.OW, TW);
+      if (tiles > 0x7fffffff) continue;
+      const int64_t cost = ceil_div(tiles, kSlots) * (ceil_div(TR * mtw, kCrWaves) * 10 + 5);
+      if (best < 0 || cost < best) {
+        best = cost;
+        p->RL = static_cast<int>(RL); p->RP = static_cast<int>(RP); p->KS = static_cast<int>(KS);
+        p->TR = static_cast<int>(TR); p->TW = static_cast<int>(TW); p->mtw = static_cast<int>(mtw);
+        p->rows_in = static_cast<int>(rows_in); p->pitch = static_cast<int>(pitch);
+        p->lds = static_cast<int>(KS * 4096 + rows_in * pitch);
+      }
     }
-    if (TR > 1)
-      TR = (TR + 1) / 2;
-    else if (TW > 16)
-      TW = round_up(TW / 2, 16);
-    else
-      return false;
+    if (TW <= 16) break;
   }
+  return best >= 0;
 }
 
 template <int MODE>
@@ -387,6 +394,7 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   a.bias = d->bias;
   a.y = out;
   a.w_kchunks = s.KC;
+  a.B = static_cast<int>(s.B);
   a.H = static_cast<int>(s.H); a.W = static_cast<int>(s.W); a.IC = static_cast<int>(s.IC);
   a.OH = static_cast<int>(s.OH); a.OW = static_cast<int>(s.OW); a.OC = static_cast<int>(s.OC);
   a.KH = static_cast<int>(s.KH); a.KW = static_cast<int>(s.KW);
@@ -396,10 +404,9 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   a.RL = p.RL; a.RP = p.RP; a.KS = p.KS;
   a.TR = p.TR; a.TW = p.TW; a.mtw = p.mtw;
   a.rows_in = p.rows_in; a.pitch = p.pitch;
-  a.uniform_rows = (s.W * s.IC) % 4 == 0 ? 1 : 0;
   a.tiles_h = static_cast<int>(ceil_div(s.OH, p.TR));
   a.tiles_w = static_cast<int>(ceil_div(s.OW, p.TW));
-  a.tiles = s.B * a.tiles_h * a.tiles_w;
+  a.tiles = static_cast<int32_t>(s.B * a.tiles_h * a.tiles_w);
   a.vec = aligned(out, 16) && s.OC % (MODE == kOutAcc32 ? 4 : 16) == 0 ? 1 : 0;
   a.w_scale_stride = d->w_per_channel ? 1 : 0;
   a.x_xor = d->x_signed ? 0u : 0x80808080u;
@@ -413,7 +420,7 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   const int64_t by = ceil_div(s.OC, kCrBN);
   if (by > 65535) return TMQ_ERR_UNSUPPORTED;
   // three blocks per CU (their registers), each with its weights in registers for every tile it walks
-  const int64_t bx = a.tiles < 768 ? a.tiles : 768;
+  const int64_t bx = a.tiles < 768 ? a.tiles : 768;  // (plan_runs: kSlots)
   const dim3 grid(static_cast<unsigned>(bx), static_cast<unsigned>(by)), block(kCrThreads);
   if constexpr (MODE == kOutAcc32) {
     conv_runs_kernel<MODE, false><<<grid, block, p.lds, stream>>>(a);
@@ -474,7 +481,7 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   // kernel rows as runs of bytes where they are short enough
   if (forced == 4 || (forced < 0 && !mfma_ok)) {
     RunPlan rp;
-    if (plan_runs(s, &rp)) return launch_conv_runs<MODE>(d, s, rp, po, zp_f, lo_f, hi_f, out, stream);
+    if (plan_runs(s, forced == 4 ? d->tile_rows : 0, &rp)) return launch_conv_runs<MODE>(d, s, rp, po, zp_f, lo_f, hi_f, out, stream);
     if (forced == 4) return TMQ_ERR_UNSUPPORTED;
   }
   if (!mfma_ok || forced == 3) {

@@ -13,8 +13,8 @@
 // A block of four waves walks tiles of TR x TW output pixels of one image:
 //   * it stages the (TR - 1) * stride + KH image rows the tile needs, as bytes, positions
 //     outside the image as the activation zero point, sign flip of unsigned activations
-//     applied; when every image row starts at the same address modulo 4 the copy runs
-//     in aligned words and the LDS row starts `shift` bytes before the tile's first byte;
+//     applied.  The copy runs in aligned words of memory whatever the address of an image
+//     row: each staged row starts 0 ... 3 bytes before the tile's first byte of its row;
 //   * a wave takes 16 output pixels of one output row at a time: the operand of pixel
 //     p, kernel row kh, 16-byte piece c of the run is the 16 bytes at
 //       row (orow * stride + kh), byte p * stride * IC + 16 c
@@ -36,6 +36,7 @@ constexpr int kCrThreads = 256;
 constexpr int kCrWaves = kCrThreads / kWave;
 constexpr int kCrBN = 64;      // output channels per block (grid y)
 constexpr int kCrMaxKS = 4;    // k-steps of 64 bytes
+constexpr int kCrStage = 8;    // staged words per thread and tile: 8 KB of image rows
 
 struct ConvRunArgs {
   const uint8_t* x;          // NHWC
@@ -45,14 +46,13 @@ struct ConvRunArgs {
   const float* bias;
   void* y;
   int64_t w_kchunks;
-  int64_t tiles;             // B * tiles_h * tiles_w
-  int H, W, IC, OH, OW, OC, KH, KW;
+  int32_t tiles;             // B * tiles_h * tiles_w
+  int B, H, W, IC, OH, OW, OC, KH, KW;
   int sh, sw, ph, pw;
   int ICp;                   // bytes of one tap in the packed weight (IC rounded up to 16)
   int RL, RP, KS;            // run bytes, padded run bytes, k-steps (KH * RP <= 64 KS)
   int TR, TW, mtw;           // output rows and columns per tile, 16-pixel pieces per tile row
   int rows_in, pitch;        // staged image rows, LDS bytes per staged row (multiple of 4)
-  int uniform_rows;          // W * IC is a multiple of 4
   int tiles_h, tiles_w;
   int vec;                   // 16-byte (int32 mode: per 4 channels) stores are aligned
   int32_t w_scale_stride;
@@ -64,7 +64,7 @@ struct ConvRunArgs {
 };
 
 template <int MODE, bool POST>
-__global__ __launch_bounds__(kCrThreads) void conv_runs_kernel(ConvRunArgs a) {
+__global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ __attribute__((aligned(16))) int s_acc0[kCrBN];
   __shared__ __attribute__((aligned(16))) float s_mult[kCrBN];
@@ -84,21 +84,30 @@ __global__ __launch_bounds__(kCrThreads) void conv_runs_kernel(ConvRunArgs a) {
     const int n = n0 + nl;
     const int koff = kc * 16;
     const int kh = koff / a.RP, ro = koff - kh * a.RP;
-    uint32_t words[4] = {0, 0, 0, 0};
-    if (n < a.OC && kh < a.KH) {
-      const uint8_t* const wrow = a.w_packed + static_cast<int64_t>(n >> 4) * a.w_kchunks * 256 + (n & 15) * 16;
+    // sixteen byte loads without a condition (invalid positions read the row's first byte
+    // and are masked): all of them are in flight together
+    const bool row_ok = n < a.OC && kh < a.KH;
+    const uint8_t* const wrow =
+        a.w_packed + (row_ok ? static_cast<int64_t>(n >> 4) * a.w_kchunks * 256 + (n & 15) * 16 : 0);
+    uint32_t bytes[16];
+    {
       int kw = ro / a.IC, ic = ro - kw * a.IC;
+#pragma unroll
       for (int bb = 0; bb < 16; ++bb) {
-        if (ro + bb < a.RL) {
-          const int kp = (kh * a.KW + kw) * a.ICp + ic;
-          words[bb >> 2] |= static_cast<uint32_t>(wrow[(kp >> 4) * 256 + (kp & 15)]) << (8 * (bb & 3));
-        }
+        const bool ok = row_ok && ro + bb < a.RL;
+        const int kp = ok ? (kh * a.KW + kw) * a.ICp + ic : 0;
+        const uint32_t v = wrow[(kp >> 4) * 256 + (kp & 15)];
+        bytes[bb] = ok ? v : 0u;
         if (++ic == a.IC) {
           ic = 0;
           ++kw;
         }
       }
     }
+    uint32_t words[4];
+#pragma unroll
+    for (int w4 = 0; w4 < 4; ++w4)
+      words[w4] = bytes[4 * w4] | (bytes[4 * w4 + 1] << 8) | (bytes[4 * w4 + 2] << 16) | (bytes[4 * w4 + 3] << 24);
     const int i = 4 * (nl >> 4) + (nl & 3), nt = (nl & 15) >> 2;
     *reinterpret_cast<v4i*>(sW + (((nt * KS + (kc >> 2)) * kWave) + (kc & 3) * 16 + i) * 16) =
         v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
@@ -128,7 +137,7 @@ __global__ __launch_bounds__(kCrThreads) void conv_runs_kernel(ConvRunArgs a) {
     for (int ks = 0; ks < kCrMaxKS; ++ks)
       wreg[nt][ks] = ks < KS ? ld16(sW + ((nt * KS + ks) * kWave + lane) * 16) : v4i{0, 0, 0, 0};
   // this lane's piece of every k-step: staged row and byte inside the run
-  int lk[kCrMaxKS];
+  int lk[kCrMaxKS];  // (a multiple of 4) | the row's share of the alignment shift, (kh * (row bytes % 4)) % 4
 #pragma unroll
   for (int ks = 0; ks < kCrMaxKS; ++ks) {
     const int koff = ks * 64 + pq * 16;
@@ -137,7 +146,7 @@ __global__ __launch_bounds__(kCrThreads) void conv_runs_kernel(ConvRunArgs a) {
       kh = a.KH - 1;
       ro = 0;
     }
-    lk[ks] = kh * a.pitch + ro;
+    lk[ks] = (kh * a.pitch + ro) | ((kh * (a.W * a.IC)) & 3);
   }
   float bmul = 1.0f;
   if constexpr (MODE != kOutAcc32) bmul = bias_mul(a.w_scale_stride == 0, a.x_scale * a.w_scales[0]);
@@ -145,61 +154,140 @@ __global__ __launch_bounds__(kCrThreads) void conv_runs_kernel(ConvRunArgs a) {
   const int row_bytes = a.W * a.IC;
   const int P4 = a.pitch >> 2, stage_words = a.rows_in * P4;
   const int tile_mt = a.TR * a.mtw;
-  for (int64_t tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
-    const int tcol = static_cast<int>(tile % a.tiles_w);
-    const int64_t trb = tile / a.tiles_w;
-    const int trow = static_cast<int>(trb % a.tiles_h), b = static_cast<int>(trb / a.tiles_h);
-    const int oh0 = trow * a.TR, ow0 = tcol * a.TW;
-    const int ih0 = oh0 * a.sh - a.ph, iwb0 = (ow0 * a.sw - a.pw) * a.IC;
-    const uint8_t* const img = a.x + static_cast<int64_t>(b) * a.H * row_bytes;
-    // LDS byte q of a staged row is image-row byte iwb0 - shift + q
-    const int shift =
-        a.uniform_rows ? static_cast<int>((reinterpret_cast<uintptr_t>(img) + static_cast<uintptr_t>(iwb0 & 3)) & 3) : 0;
-
-    // ---- stage the image rows
-    for (int idx = t; idx < stage_words; idx += kCrThreads) {
-      int r = static_cast<int>(static_cast<float>(idx) * a.rcp_p4);
-      int p4 = idx - r * P4;
-      if (p4 < 0) {
-        --r;
-        p4 += P4;
-      } else if (p4 >= P4) {
-        ++r;
-        p4 -= P4;
-      }
-      const int ih = ih0 + r, colb = iwb0 - shift + 4 * p4;
-      uint32_t word = a.pad_word;
-      if (static_cast<unsigned>(ih) < static_cast<unsigned>(a.H)) {
-        const uint8_t* const src = img + static_cast<int64_t>(ih) * row_bytes + colb;
-        if (a.uniform_rows && colb >= 0 && colb + 3 < row_bytes) {
-          word = *reinterpret_cast<const uint32_t*>(src);
+  // The staged rows of a tile pass through registers: kCrStage words per thread (the host
+  // sizes the tiles for that), requested one tile ahead, so that they arrive while the
+  // tile in hand is multiplied.  Word u of thread t is word t + 256 u of the staged rows:
+  // its row and place in the row are the same for every tile.
+  int spos[kCrStage];  // row << 16 | byte in the row; -1: no such word
+#pragma unroll
+  for (int u = 0; u < kCrStage; ++u) {
+    const int idx = t + u * kCrThreads;
+    int r = static_cast<int>(static_cast<float>(idx) * a.rcp_p4);
+    int p4 = idx - r * P4;
+    if (p4 < 0) {
+      --r;
+      p4 += P4;
+    } else if (p4 >= P4) {
+      ++r;
+      p4 -= P4;
+    }
+    spos[u] = idx < stage_words ? (r << 16 | 4 * p4) : -1;
+  }
+  uint32_t pre[kCrStage];
+  // Staged row r of a tile starts shift(r) = (c0 + r * (row bytes % 4)) % 4 bytes before the
+  // tile's first byte of that image row, so that every staged word is an aligned word of
+  // memory: LDS byte q of the row is image-row byte iwb0 - shift(r) + q.
+  struct TilePos {
+    int b, oh0, ow0, c0;
+    int ih0, iwb0;        // image row and byte in the row of the tile's first staged byte (before the shift)
+    int64_t first;        // the same as a byte offset into the tensor
+    int edge;             // some staged word may reach outside the tensor
+  };
+  const int rb3 = row_bytes & 3;
+  const int64_t x_bytes = static_cast<int64_t>(a.B) * a.H * row_bytes;
+  auto tile_pos = [&](uint32_t tile) {
+    TilePos tp;
+    const uint32_t trb = tile / static_cast<uint32_t>(a.tiles_w);
+    const int tcol = static_cast<int>(tile - trb * static_cast<uint32_t>(a.tiles_w));
+    tp.b = static_cast<int>(trb / static_cast<uint32_t>(a.tiles_h));
+    const int trow = static_cast<int>(trb) - tp.b * a.tiles_h;
+    tp.oh0 = trow * a.TR;
+    tp.ow0 = tcol * a.TW;
+    tp.ih0 = tp.oh0 * a.sh - a.ph;
+    tp.iwb0 = (tp.ow0 * a.sw - a.pw) * a.IC;
+    tp.first = (static_cast<int64_t>(tp.b) * a.H + tp.ih0) * row_bytes + tp.iwb0;
+    tp.c0 = static_cast<int>((reinterpret_cast<uintptr_t>(a.x) + static_cast<uintptr_t>(tp.first)) & 3);
+    tp.edge = tp.first < 4 || tp.first + static_cast<int64_t>(a.rows_in) * row_bytes + a.pitch + 4 > x_bytes;
+    return tp;
+  };
+  // The loads only: whole aligned words, also where a word hangs over the end of its image
+  // row into the next one (store_tile masks those bytes); nothing here uses a loaded value,
+  // so nothing waits.  Only in the first and the last tiles of the tensor can a word reach
+  // outside it; those tiles check every byte.
+  auto request = [&](const TilePos& tp) {
+    const uint8_t* const base = a.x + (tp.first - 4);  // (an address to count from, not one to load from)
+#pragma unroll
+    for (int u = 0; u < kCrStage; ++u) {
+      pre[u] = 0;
+      if (u * kCrThreads >= stage_words) continue;  // (the same for the whole block)
+      const int r = spos[u] >> 16, q = spos[u] & 0xffff;
+      const int shift = (tp.c0 + r * rb3) & 3;
+      const int colb = tp.iwb0 - shift + q;
+      const bool ok = spos[u] >= 0 && static_cast<unsigned>(tp.ih0 + r) < static_cast<unsigned>(a.H) &&
+                      static_cast<unsigned>(colb + 3) < static_cast<unsigned>(row_bytes + 3);
+      const uint32_t off = static_cast<uint32_t>(r * row_bytes + q - shift + 4);
+      if (ok) {
+        if (!tp.edge) {
+          pre[u] = *reinterpret_cast<const uint32_t*>(base + off);
         } else {
+          const int64_t rel = tp.first - 4 + static_cast<int64_t>(off);
+          uint32_t word = 0;
 #pragma unroll
           for (int jj = 0; jj < 4; ++jj)
-            if (static_cast<unsigned>(colb + jj) < static_cast<unsigned>(row_bytes))
-              word = (word & ~(0xffu << (8 * jj))) | (static_cast<uint32_t>(src[jj]) << (8 * jj));
+            if (rel + jj >= 0 && rel + jj < x_bytes) word |= static_cast<uint32_t>(a.x[rel + jj]) << (8 * jj);
+          pre[u] = word;
         }
       }
-      *reinterpret_cast<uint32_t*>(sX + r * a.pitch + 4 * p4) = word ^ a.x_xor;
     }
+  };
+  // Bytes outside the image (rows above and below, columns left and right of the row) become
+  // the activation zero point; then the sign flip, and into LDS.
+  auto store_tile = [&](const TilePos& tp) {
+#pragma unroll
+    for (int u = 0; u < kCrStage; ++u) {
+      if (u * kCrThreads >= stage_words || spos[u] < 0) continue;
+      const int r = spos[u] >> 16, q = spos[u] & 0xffff;
+      const int colb = tp.iwb0 - ((tp.c0 + r * rb3) & 3) + q;
+      uint32_t word = pre[u];
+      const bool row_in = static_cast<unsigned>(tp.ih0 + r) < static_cast<unsigned>(a.H);
+      if (!(row_in && colb >= 0 && colb + 3 < row_bytes)) {  // (the few words at the image's edges)
+        uint32_t keep = 0;
+        if (row_in) {
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj)
+            if (static_cast<unsigned>(colb + jj) < static_cast<unsigned>(row_bytes)) keep |= 0xffu << (8 * jj);
+        }
+        word = (word & keep) | (a.pad_word & ~keep);
+      }
+      *reinterpret_cast<uint32_t*>(sX + r * a.pitch + q) = word ^ a.x_xor;
+    }
+  };
+  TilePos cur{};
+  if (static_cast<int>(blockIdx.x) < a.tiles) {
+    cur = tile_pos(blockIdx.x);
+    request(cur);
+  }
+  for (int tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+    const int b = cur.b, oh0 = cur.oh0, ow0 = cur.ow0, c0 = cur.c0;
+    // ---- the staged rows of this tile into LDS, the next tile's on their way
+    store_tile(cur);
     __syncthreads();
+    if (tile + static_cast<int>(gridDim.x) < a.tiles) {
+      cur = tile_pos(static_cast<uint32_t>(tile) + gridDim.x);
+      request(cur);
+    }
 
     // ---- multiply: 16 pixels of one output row per wave and turn
     const int tw_valid = a.OW - ow0 < a.TW ? a.OW - ow0 : a.TW;
     const int th_valid = a.OH - oh0 < a.TR ? a.OH - oh0 : a.TR;
-    for (int mt = wave; mt < tile_mt; mt += kCrWaves) {
-      const int orow = mt / a.mtw, mcol = mt - orow * a.mtw;
+    int orow = 0, mcol = wave;  // this wave's piece: row of the tile, 16-pixel piece of the row
+    for (int mt = wave; mt < tile_mt; mt += kCrWaves, mcol += kCrWaves) {
+      while (mcol >= a.mtw) {
+        mcol -= a.mtw;
+        ++orow;
+      }
       if (orow >= th_valid || mcol * 16 >= tw_valid) continue;  // (the same for the whole wave)
       const int pcol = mcol * 16 + pj;
       const int pc = pcol < tw_valid ? pcol : tw_valid - 1;
-      const int base = orow * a.sh * a.pitch + pc * a.sw * a.IC + shift;
-      v4i acc[4];
+      const int base = orow * a.sh * a.pitch + pc * a.sw * a.IC;
+      const int c0r = c0 + orow * a.sh * rb3;  // alignment shift of staged row orow * stride, before the % 4
+      v4i acc[4];  // start: the zero point's share, acc_coef * colsum
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) acc[nt] = v4i{0, 0, 0, 0};
+      for (int nt = 0; nt < 4; ++nt) acc[nt] = *reinterpret_cast<const v4i*>(&s_acc0[16 * pq + 4 * nt]);
 #pragma unroll
       for (int ks = 0; ks < kCrMaxKS; ++ks) {
         if (ks < KS) {
-          const int addr = base + lk[ks];
+          const int addr = base + (lk[ks] & ~3) + ((c0r + lk[ks]) & 3);
           const uint32_t* const src = reinterpret_cast<const uint32_t*>(sX + (addr & ~3));
           const uint32_t sb = static_cast<uint32_t>(addr & 3);
           const uint32_t d0 = src[0], d1 = src[1], d2 = src[2], d3 = src[3], d4 = src[4];
@@ -222,10 +310,7 @@ __global__ __launch_bounds__(kCrThreads) void conv_runs_kernel(ConvRunArgs a) {
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const int cl = 16 * pq + 4 * nt;
-        const v4i add = *reinterpret_cast<const v4i*>(&s_acc0[cl]);
-        int raw[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) raw[r] = acc[nt][r] + add[r];
+        const int raw[4] = {acc[nt][0], acc[nt][1], acc[nt][2], acc[nt][3]};
         if constexpr (MODE == kOutAcc32) {
           int32_t* const dst = static_cast<int32_t*>(a.y) + off + 4 * nt;
           if (a.vec && cb + 4 * nt + 4 <= a.OC) {
