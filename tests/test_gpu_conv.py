@@ -101,7 +101,7 @@ def test_conv_mfma_shapes(cabi, spec, x_signed, path):
 @pytest.mark.parametrize("spec", [
     (1, 9, 300, 16, 16, 3, 1, 1, 1, 1),      # wide rows: patches split the width
     (2, 33, 21, 32, 72, 3, 2, 1, 2, 1),      # stride 2 with dilation 2, OC over two 64-channel tiles
-    (1, 12, 12, 96, 48, 3, 1, 1, 1, 4),      # four groups of 24 in, 12 out -> direct kernel
+    (1, 12, 12, 96, 48, 3, 1, 1, 1, 4),      # four groups of 24 in, 12 out: merged in pairs
     (3, 10, 10, 64, 48, 3, 1, 1, 1, 2),      # groups whose 24 channels break 16-byte stores
     (1, 14, 14, 128, 64, 3, 1, 1, 1, 1),     # 72 KB weight slice in LDS
     (1, 14, 14, 256, 64, 3, 1, 1, 1, 1),     # weight slice too large for LDS: implicit GEMM
@@ -158,6 +158,43 @@ def test_conv_few_channels_as_byte_runs(cabi, spec, x_signed):
         finally:
             cabi.force_conv_path(-1)
         np.testing.assert_array_equal(acc, want_acc)
+        _check(y, want, f"path {path}")
+
+
+@pytest.mark.parametrize("spec", [
+    (2, 20, 20, 32, 32, 3, 1, 1, 1, 32),     # depthwise, 32 channels: one merged group
+    (1, 29, 29, 144, 144, 3, 2, 1, 1, 144),  # depthwise stride 2, 144 channels: three merged groups of 48
+    (1, 15, 15, 96, 96, 5, 1, 2, 1, 96),     # depthwise 5 x 5
+    (1, 14, 14, 384, 384, 3, 1, 1, 1, 384),  # depthwise, six merged groups of 64
+    (2, 16, 16, 128, 128, 3, 1, 1, 1, 32),   # 32 groups of 4 -> 4: two merged groups of 64
+    (1, 12, 12, 32, 64, 3, 1, 1, 1, 4),      # groups of 8 in, 16 out: two of them make 16 / 32
+    (1, 10, 10, 16, 32, 3, 1, 1, 1, 16),     # depthwise with two output channels per input channel
+    (1, 12, 12, 96, 48, 3, 1, 1, 1, 4),      # groups of 24 in, 12 out: pairs
+    (1, 9, 9, 40, 40, 3, 1, 1, 1, 40),       # depthwise, 40 channels: no multiple of 16 divides it, direct kernel
+    (1, 9, 9, 48, 48, 3, 1, 1, 2, 48),       # depthwise with dilation
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_narrow_groups_merged(cabi, spec, x_signed):
+    say("conv narrow groups", spec, x_signed)
+    c = _conv_case(*spec, seed=sum(spec) + 11, x_signed=x_signed, relu=x_signed)
+    want_acc = oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                   c["groups"], c["x_zp"], nthreads=8)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    merged = spec[3] != 40
+    for path in (-1, 1, 2, 3):
+        cabi.force_conv_path(path)
+        try:
+            if path in (1, 2) and not merged:
+                with pytest.raises(cabi.TmqError):
+                    _run(cabi, c)
+                continue
+            y, acc, pw = _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+        np.testing.assert_array_equal(acc, want_acc)
+        np.testing.assert_array_equal(host(pw.colsum), c["wq"].reshape(c["wq"].shape[0], -1).astype(np.int64).sum(1))
         _check(y, want, f"path {path}")
 
 

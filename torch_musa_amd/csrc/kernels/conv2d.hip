@@ -27,6 +27,7 @@ struct ConvShape {
   int64_t B, H, W, IC, OC, KH, KW, OH, OW;
   int64_t sh, sw, ph, pw, dh, dw, groups;
   int64_t ICg, OCg, ICgp, Kp, KC, group_bytes;
+  int64_t ICgo, OCgo;  // channels per group as the caller states them (see make_shape)
 };
 
 int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
@@ -42,8 +43,29 @@ int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
   s->OH = (g->H + 2 * g->pad_h - g->dil_h * (g->KH - 1) - 1) / g->stride_h + 1;
   s->OW = (g->W + 2 * g->pad_w - g->dil_w * (g->KW - 1) - 1) / g->stride_w + 1;
   if (s->OH <= 0 || s->OW <= 0) return TMQ_ERR_INVALID_ARGUMENT;
-  s->ICg = g->IC / g->groups;
-  s->OCg = g->OC / g->groups;
+  // Groups whose input channels are no multiple of 16 (depthwise and other narrow groups)
+  // are merged: `merge` neighbouring groups become one group with a block-diagonal weight --
+  // zeros where an output channel meets another group's input channels -- so that a 16-byte
+  // k-chunk is again 16 channels of one pixel and the MFMA kernels take the problem.  The
+  // matrix pipe multiplies the zeros at no cost that matters: these layers move bytes.
+  // The merged group has as many channels as a tile of the kernels is wide (64) where the
+  // group count allows.  groups / ICg / OCg below are the merged ones; the packed weight
+  // is laid out for them.
+  s->ICgo = g->IC / g->groups;
+  s->OCgo = g->OC / g->groups;
+  int64_t merge = 1;
+  if (g->groups > 1 && s->ICgo % 16 != 0) {
+    const int64_t low = s->ICgo & -s->ICgo;             // largest power of two in ICgo
+    const int64_t v0 = 16 / (low < 16 ? low : 16);      // fewest groups that make a multiple of 16
+    for (int64_t v = v0; v <= g->groups; v += v0) {
+      if (v > v0 && (v * s->OCgo > 64 || v * s->ICgo > 64)) break;
+      if (g->groups % v == 0) merge = v;
+    }
+    if ((merge * s->ICgo) % 16 != 0) merge = 1;         // (no such divisor of the group count)
+  }
+  s->groups = g->groups / merge;
+  s->ICg = merge * s->ICgo;
+  s->OCg = merge * s->OCgo;
   s->ICgp = round_up(s->ICg, 16);
   s->Kp = g->KH * g->KW * s->ICgp;
   s->KC = packed_kchunks(s->Kp);
@@ -70,10 +92,12 @@ __global__ __launch_bounds__(256) void conv_prepack_kernel(const int8_t* __restr
   const int64_t tap = k0 / s.ICgp, ic0 = k0 % s.ICgp;
   uint32_t words[4] = {0, 0, 0, 0};
   if (n < s.OCg && tap < s.KH * s.KW) {
-    const int8_t* src = w + ((g * s.OCg + n) * s.KH * s.KW + tap) * s.ICg;
+    // the output channel's own group inside a merged one: its input channels lo .. lo + ICgo - 1
+    const int64_t lo = n / s.OCgo * s.ICgo;
+    const int8_t* src = w + ((g * s.OCg + n) * s.KH * s.KW + tap) * s.ICgo;
     for (int b = 0; b < 16; ++b)
-      if (ic0 + b < s.ICg)
-        words[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(src[ic0 + b])) << (8 * (b & 3));
+      if (ic0 + b >= lo && ic0 + b < lo + s.ICgo)
+        words[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(src[ic0 + b - lo])) << (8 * (b & 3));
   }
   *reinterpret_cast<v4i*>(packed + id * 16) =
       v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
@@ -115,6 +139,7 @@ __global__ __launch_bounds__(256) void conv_plain_kernel(ConvShape s, PlainArgs 
   const int64_t g = oc / s.OCg, n = oc % s.OCg;
   const int64_t ow = m % s.OW, oh = (m / s.OW) % s.OH, b = m / (s.OW * s.OH);
   const uint8_t* wp = a.w_packed + g * s.group_bytes;
+  const int64_t sub = n / s.OCgo * s.ICgo;  // first input channel of the channel's own group inside a merged one
   int acc = 0;
   for (int64_t kh = 0; kh < s.KH; ++kh) {
     const int64_t ih = oh * s.sh - s.ph + kh * s.dh;
@@ -122,9 +147,9 @@ __global__ __launch_bounds__(256) void conv_plain_kernel(ConvShape s, PlainArgs 
     for (int64_t kw = 0; kw < s.KW; ++kw) {
       const int64_t iw = ow * s.sw - s.pw + kw * s.dw;
       if (iw < 0 || iw >= s.W) continue;
-      const uint8_t* xp = a.x + ((b * s.H + ih) * s.W + iw) * s.IC + g * s.ICg;
-      const int64_t kbase = (kh * s.KW + kw) * s.ICgp;
-      for (int64_t ic = 0; ic < s.ICg; ++ic) {
+      const uint8_t* xp = a.x + ((b * s.H + ih) * s.W + iw) * s.IC + g * s.ICg + sub;
+      const int64_t kbase = (kh * s.KW + kw) * s.ICgp + sub;
+      for (int64_t ic = 0; ic < s.ICgo; ++ic) {
         const int xv = a.x_signed ? static_cast<int>(static_cast<int8_t>(xp[ic])) : static_cast<int>(xp[ic]);
         const int64_t k = kbase + ic;
         const int wv = static_cast<int8_t>(wp[(((n >> 4) * s.KC + (k >> 4)) * 16 + (n & 15)) * 16 + (k & 15)]);
@@ -631,7 +656,7 @@ TMQ_EXPORT int tmq_conv2d_prepack(const int8_t* w_ohwi, const tmq_conv2d_geom* g
   if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
   blocks = ceil_div(s.OC, 256 / kWave);
   conv_colsum_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, hs>>>(
-      w_ohwi, s.OC, s.KH * s.KW * s.ICg, colsum);
+      w_ohwi, s.OC, s.KH * s.KW * s.ICgo, colsum);
   return launch_status();
 }
 
