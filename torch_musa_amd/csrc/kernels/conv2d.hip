@@ -28,6 +28,9 @@ struct ConvShape {
   int64_t sh, sw, ph, pw, dh, dw, groups;
   int64_t ICg, OCg, ICgp, Kp, KC, group_bytes;
   int64_t ICgo, OCgo;  // channels per group as the caller states them (see make_shape)
+  // the second weight layout, behind the first, for the kernel of conv_runs.h: k-steps
+  // (0: the shape is not that kernel's), run bytes, padded run bytes, offset and size in bytes
+  int64_t runs_KS, runs_RL, runs_RP, runs_off, runs_bytes;
 };
 
 int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
@@ -70,6 +73,17 @@ int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
   s->Kp = g->KH * g->KW * s->ICgp;
   s->KC = packed_kchunks(s->Kp);
   s->group_bytes = ceil_div(s->OCg, 16) * s->KC * 256;
+  s->runs_KS = s->runs_RL = s->runs_RP = s->runs_bytes = 0;
+  s->runs_off = s->groups * s->group_bytes;
+  if (g->groups == 1 && g->dil_h == 1 && g->dil_w == 1) {
+    const int64_t RL = g->KW * g->IC, RP = round_up(RL, 16);
+    if (g->KH * RP <= 64 * kCrMaxKS) {
+      s->runs_RL = RL;
+      s->runs_RP = RP;
+      s->runs_KS = ceil_div(g->KH * RP, 64);
+      s->runs_bytes = ceil_div(g->OC, kCrBN) * 4 * s->runs_KS * kWave * 16;
+    }
+  }
   // 32-bit index arithmetic inside the kernels
   if (g->H > (1 << 24) || g->W > (1 << 24) || g->IC > (1 << 24) || s->Kp > (1 << 30) ||
       g->B * s->OH * s->OW > 0x7fffffff || g->H * g->W * g->IC > 0x3fffffff)
@@ -102,6 +116,16 @@ __global__ __launch_bounds__(256) void conv_prepack_kernel(const int8_t* __restr
   *reinterpret_cast<v4i*>(packed + id * 16) =
       v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
           static_cast<int>(words[3])};
+}
+
+// One thread per 16-byte slot of the per-lane layout of conv_runs.h.
+__global__ __launch_bounds__(256) void conv_prepack_runs_kernel(const int8_t* __restrict__ w, ConvShape s,
+                                                                int64_t total, uint8_t* __restrict__ dst) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  *reinterpret_cast<v4i*>(dst + id * 16) =
+      conv_runs_slot(w, id, static_cast<int>(s.OC), static_cast<int>(s.KH), static_cast<int>(s.runs_RL),
+                     static_cast<int>(s.runs_RP), static_cast<int>(s.runs_KS));
 }
 
 __global__ __launch_bounds__(256) void conv_colsum_kernel(const int8_t* __restrict__ w, int64_t OC,
@@ -375,22 +399,20 @@ struct RunPlan {
   int RL, RP, KS, TR, TW, mtw, rows_in, pitch, lds;
 };
 bool plan_runs(const ConvShape& s, int forced_rows, RunPlan* p) {
-  if (s.groups != 1 || s.dh != 1 || s.dw != 1) return false;
-  const int64_t RL = s.KW * s.IC, RP = round_up(RL, 16);
-  if (s.KH * RP > 64 * kCrMaxKS) return false;
-  const int64_t KS = ceil_div(s.KH * RP, 64);
+  if (s.runs_KS == 0) return false;
+  const int64_t RL = s.runs_RL, RP = s.runs_RP, KS = s.runs_KS;
   // Tile = TR output rows x TW columns.  The staged image rows of a tile pass through
-  // kCrStage registers per thread; among the shapes that fit, the one with the shortest
-  // schedule: rounds of tiles over the blocks the chip holds (three per CU) times the
-  // turns its four waves need for the tile's 16-pixel pieces.
-  constexpr int64_t kSlots = 3 * 256, kStageBytes = int64_t{kCrStage} * kCrThreads * 4;
+  // registers in units of 1 KB of a row, at most kCrUnits per wave; among the shapes that
+  // fit, the one with the shortest schedule: rounds of tiles over the blocks the chip holds
+  // (three per CU) times the turns its four waves need for the tile's 16-pixel pieces.
+  constexpr int64_t kSlots = 3 * 256, kMaxUnits = int64_t{kCrUnits} * kCrWaves;
   int64_t best = -1;
   for (int64_t TW = s.OW < 128 ? s.OW : 128;; TW = round_up(TW / 2, 16)) {
     const int64_t mtw = ceil_div(TW, 16);
-    const int64_t pitch = round_up((TW - 1) * s.sw * s.IC + RP + 8, 4);
+    const int64_t pitch = round_up((TW - 1) * s.sw * s.IC + RP + 20, 16);
     for (int64_t TR = 1; TR <= s.OH && TR <= 8; ++TR) {
       const int64_t rows_in = (TR - 1) * s.sh + s.KH;
-      if (rows_in * pitch > kStageBytes) break;
+      if (rows_in * ceil_div(pitch, 1024) > kMaxUnits) break;
       if (forced_rows > 0 && TR != forced_rows) continue;
       const int64_t tiles = s.B * ceil_div(s.OH, TR) * ceil_div(s.OW, TW);
       if (tiles > 0x7fffffff) continue;
@@ -400,7 +422,7 @@ bool plan_runs(const ConvShape& s, int forced_rows, RunPlan* p) {
         p->RL = static_cast<int>(RL); p->RP = static_cast<int>(RP); p->KS = static_cast<int>(KS);
         p->TR = static_cast<int>(TR); p->TW = static_cast<int>(TW); p->mtw = static_cast<int>(mtw);
         p->rows_in = static_cast<int>(rows_in); p->pitch = static_cast<int>(pitch);
-        p->lds = static_cast<int>(KS * 4096 + rows_in * pitch);
+        p->lds = static_cast<int>(rows_in * pitch);
       }
     }
     if (TW <= 16) break;
@@ -413,19 +435,17 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
                      float lo_f, float hi_f, void* out, hipStream_t stream) {
   ConvRunArgs a{};
   a.x = static_cast<const uint8_t*>(d->x);
-  a.w_packed = static_cast<const uint8_t*>(d->w_packed);
+  a.w_runs = static_cast<const uint8_t*>(d->w_packed) + s.runs_off;
   a.colsum = d->w_colsum;
   a.w_scales = d->w_scales;
   a.bias = d->bias;
   a.y = out;
-  a.w_kchunks = s.KC;
   a.B = static_cast<int>(s.B);
   a.H = static_cast<int>(s.H); a.W = static_cast<int>(s.W); a.IC = static_cast<int>(s.IC);
   a.OH = static_cast<int>(s.OH); a.OW = static_cast<int>(s.OW); a.OC = static_cast<int>(s.OC);
   a.KH = static_cast<int>(s.KH); a.KW = static_cast<int>(s.KW);
   a.sh = static_cast<int>(s.sh); a.sw = static_cast<int>(s.sw);
   a.ph = static_cast<int>(s.ph); a.pw = static_cast<int>(s.pw);
-  a.ICp = static_cast<int>(s.ICgp);
   a.RL = p.RL; a.RP = p.RP; a.KS = p.KS;
   a.TR = p.TR; a.TW = p.TW; a.mtw = p.mtw;
   a.rows_in = p.rows_in; a.pitch = p.pitch;
@@ -440,7 +460,6 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   a.x_scale = d->x_scale;
   a.out_scale = d->out_scale;
   a.zp_f = zp_f; a.lo_f = lo_f; a.hi_f = hi_f;
-  a.rcp_p4 = 4.0f / static_cast<float>(p.pitch);
   a.post = po;
   const int64_t by = ceil_div(s.OC, kCrBN);
   if (by > 65535) return TMQ_ERR_UNSUPPORTED;
@@ -628,7 +647,7 @@ using namespace tmq;
 TMQ_EXPORT int64_t tmq_conv2d_packed_bytes(const tmq_conv2d_geom* g) {
   ConvShape s;
   if (make_shape(g, &s) != TMQ_OK) return 0;
-  return s.groups * s.group_bytes;
+  return s.groups * s.group_bytes + s.runs_bytes;
 }
 
 TMQ_EXPORT int tmq_conv2d_out_hw(const tmq_conv2d_geom* g, int64_t* OH, int64_t* OW) {
@@ -654,6 +673,12 @@ TMQ_EXPORT int tmq_conv2d_prepack(const int8_t* w_ohwi, const tmq_conv2d_geom* g
   conv_prepack_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, hs>>>(
       w_ohwi, s, total, static_cast<uint8_t*>(packed));
   if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  if (s.runs_bytes > 0) {
+    const int64_t slots = s.runs_bytes / 16;
+    conv_prepack_runs_kernel<<<dim3(static_cast<unsigned>(ceil_div(slots, 256))), dim3(256), 0, hs>>>(
+        w_ohwi, s, slots, static_cast<uint8_t*>(packed) + s.runs_off);
+    if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  }
   blocks = ceil_div(s.OC, 256 / kWave);
   conv_colsum_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, hs>>>(
       w_ohwi, s.OC, s.KH * s.KW * s.ICgo, colsum);

@@ -8,13 +8,14 @@
 // row, padded to RP = a multiple of 16 with zero weights: the bytes an operand picks
 // up past the run's end are multiplied by zero.  K = KH * RP is at most 256 here, the
 // weights of 64 output channels stay in registers (16 operands of
-// v_mfma_i32_16x16x64_i8) for the whole launch.
+// v_mfma_i32_16x16x64_i8) for the whole launch; prepack lays them out per lane
+// (conv_runs_slot) behind the packed weight of the other kernels.
 //
 // A block of four waves walks tiles of TR x TW output pixels of one image:
 //   * it stages the (TR - 1) * stride + KH image rows the tile needs, as bytes, positions
 //     outside the image as the activation zero point, sign flip of unsigned activations
-//     applied.  The copy runs in aligned words of memory whatever the address of an image
-//     row: each staged row starts 0 ... 3 bytes before the tile's first byte of its row;
+//     applied.  The copy runs in aligned 16-byte loads whatever the address of an image
+//     row: each staged row starts 0 ... 15 bytes before the tile's first byte of its row;
 //   * a wave takes 16 output pixels of one output row at a time: the operand of pixel
 //     p, kernel row kh, 16-byte piece c of the run is the 16 bytes at
 //       row (orow * stride + kh), byte p * stride * IC + 16 c
@@ -36,32 +37,55 @@ constexpr int kCrThreads = 256;
 constexpr int kCrWaves = kCrThreads / kWave;
 constexpr int kCrBN = 64;      // output channels per block (grid y)
 constexpr int kCrMaxKS = 4;    // k-steps of 64 bytes
-constexpr int kCrStage = 8;    // staged words per thread and tile: 8 KB of image rows
+constexpr int kCrUnits = 4;    // 1 KB units of staged image rows per wave and tile: 16 KB per block
 
 struct ConvRunArgs {
   const uint8_t* x;          // NHWC
-  const uint8_t* w_packed;   // the packed layout of conv2d.hip: [16 channels][k-chunk][channel][16 B], taps of ICp bytes
+  const uint8_t* w_runs;     // [64-channel block][channel tile nt][k-step][lane][16 B]: conv_runs_slot below
   const int32_t* colsum;
   const float* w_scales;
   const float* bias;
   void* y;
-  int64_t w_kchunks;
   int32_t tiles;             // B * tiles_h * tiles_w
   int B, H, W, IC, OH, OW, OC, KH, KW;
   int sh, sw, ph, pw;
-  int ICp;                   // bytes of one tap in the packed weight (IC rounded up to 16)
   int RL, RP, KS;            // run bytes, padded run bytes, k-steps (KH * RP <= 64 KS)
   int TR, TW, mtw;           // output rows and columns per tile, 16-pixel pieces per tile row
-  int rows_in, pitch;        // staged image rows, LDS bytes per staged row (multiple of 4)
+  int rows_in, pitch;        // staged image rows, LDS bytes per staged row (multiple of 16)
   int tiles_h, tiles_w;
   int vec;                   // 16-byte (int32 mode: per 4 channels) stores are aligned
   int32_t w_scale_stride;
   uint32_t x_xor, pad_word;  // pad_word: the activation zero point in 4 bytes, before the xor
   int32_t acc_coef;
   float x_scale, out_scale, zp_f, lo_f, hi_f;
-  float rcp_p4;              // 4 / pitch
   PostOps post;
 };
+
+// One 16-byte slot of the per-lane weight layout: slot index ->
+// (64-channel block cb, channel tile nt, k-step ks, lane).  The lane's row i = lane % 16 of
+// tile nt is channel 64 cb + 16 (i / 4) + 4 nt + i % 4; its bytes are k = 64 ks + 16 (lane / 16)
+// ... + 15 in (kh, run) order: kernel row kh = k / RP, byte k % RP of the run, which in OHWI
+// weights is byte (kw, ic) = k % RP of the contiguous row w[n][kh][.][.]; zeros past the
+// run's RL bytes, past the last kernel row and for channels that do not exist.
+__device__ __forceinline__ v4i conv_runs_slot(const int8_t* __restrict__ w, int64_t slot, int OC, int KH, int RL,
+                                              int RP, int KS) {
+  const int lane = static_cast<int>(slot & 63);
+  const int64_t op = slot >> 6;
+  const int ks = static_cast<int>(op % KS), nt = static_cast<int>((op / KS) & 3);
+  const int64_t cb = op / (4 * KS);
+  const int i = lane & 15;
+  const int64_t n = cb * 64 + 16 * (i >> 2) + 4 * nt + (i & 3);
+  const int k = 64 * ks + 16 * (lane >> 4);
+  const int kh = k / RP, ro = k - kh * RP;
+  uint32_t words[4] = {0, 0, 0, 0};
+  if (n < OC && kh < KH) {
+    const int8_t* const src = w + (n * KH + kh) * RL;
+    for (int b = 0; b < 16; ++b)
+      if (ro + b < RL) words[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(src[ro + b])) << (8 * (b & 3));
+  }
+  return v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
+             static_cast<int>(words[3])};
+}
 
 template <int MODE, bool POST>
 __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a) {
@@ -75,44 +99,8 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
   const int pj = lane & 15, pq = lane >> 4;
   const int n0 = static_cast<int>(blockIdx.y) * kCrBN;
   const int KS = a.KS;
-  uint8_t* const sW = lds;                  // [channel tile nt][k-step][lane][16 B]
-  uint8_t* const sX = lds + KS * 4096;      // staged image rows
+  uint8_t* const sX = lds;                  // staged image rows
 
-  // ---- the weight operands of this block's 64 channels, once
-  for (int item = t; item < kCrBN * 4 * KS; item += kCrThreads) {
-    const int nl = item & 63, kc = item >> 6;      // channel of the tile, 16-byte piece of k
-    const int n = n0 + nl;
-    const int koff = kc * 16;
-    const int kh = koff / a.RP, ro = koff - kh * a.RP;
-    // sixteen byte loads without a condition (invalid positions read the row's first byte
-    // and are masked): all of them are in flight together
-    const bool row_ok = n < a.OC && kh < a.KH;
-    const uint8_t* const wrow =
-        a.w_packed + (row_ok ? static_cast<int64_t>(n >> 4) * a.w_kchunks * 256 + (n & 15) * 16 : 0);
-    uint32_t bytes[16];
-    {
-      int kw = ro / a.IC, ic = ro - kw * a.IC;
-#pragma unroll
-      for (int bb = 0; bb < 16; ++bb) {
-        const bool ok = row_ok && ro + bb < a.RL;
-        const int kp = ok ? (kh * a.KW + kw) * a.ICp + ic : 0;
-        const uint32_t v = wrow[(kp >> 4) * 256 + (kp & 15)];
-        bytes[bb] = ok ? v : 0u;
-        if (++ic == a.IC) {
-          ic = 0;
-          ++kw;
-        }
-      }
-    }
-    uint32_t words[4];
-#pragma unroll
-    for (int w4 = 0; w4 < 4; ++w4)
-      words[w4] = bytes[4 * w4] | (bytes[4 * w4 + 1] << 8) | (bytes[4 * w4 + 2] << 16) | (bytes[4 * w4 + 3] << 24);
-    const int i = 4 * (nl >> 4) + (nl & 3), nt = (nl & 15) >> 2;
-    *reinterpret_cast<v4i*>(sW + (((nt * KS + (kc >> 2)) * kWave) + (kc & 3) * 16 + i) * 16) =
-        v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]),
-            static_cast<int>(words[3])};
-  }
   if (t < kCrBN) {
     const int n = n0 + t;
     int acc0 = 0;
@@ -129,15 +117,19 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
     s_mult[t] = mult;
     s_bdiv[t] = bdiv;
   }
-  __syncthreads();
+  // the weight operands of this block's 64 channels, laid out per lane at prepack
   v4i wreg[4][kCrMaxKS];
+  {
+    const uint8_t* const wsrc = a.w_runs + (static_cast<int64_t>(blockIdx.y) * 4 * KS * kWave + lane) * 16;
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt)
+    for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-    for (int ks = 0; ks < kCrMaxKS; ++ks)
-      wreg[nt][ks] = ks < KS ? ld16(sW + ((nt * KS + ks) * kWave + lane) * 16) : v4i{0, 0, 0, 0};
+      for (int ks = 0; ks < kCrMaxKS; ++ks)
+        wreg[nt][ks] = ks < KS ? ld16(wsrc + (nt * KS + ks) * (kWave * 16)) : v4i{0, 0, 0, 0};
+  }
+  __syncthreads();
   // this lane's piece of every k-step: staged row and byte inside the run
-  int lk[kCrMaxKS];  // (a multiple of 4) | the row's share of the alignment shift, (kh * (row bytes % 4)) % 4
+  int lk[kCrMaxKS];  // (a multiple of 16) | the row's share of the alignment shift, (kh * (row bytes % 16)) % 16
 #pragma unroll
   for (int ks = 0; ks < kCrMaxKS; ++ks) {
     const int koff = ks * 64 + pq * 16;
@@ -146,44 +138,29 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
       kh = a.KH - 1;
       ro = 0;
     }
-    lk[ks] = (kh * a.pitch + ro) | ((kh * (a.W * a.IC)) & 3);
+    lk[ks] = (kh * a.pitch + ro) | ((kh * (a.W * a.IC)) & 15);
   }
   float bmul = 1.0f;
   if constexpr (MODE != kOutAcc32) bmul = bias_mul(a.w_scale_stride == 0, a.x_scale * a.w_scales[0]);
 
   const int row_bytes = a.W * a.IC;
-  const int P4 = a.pitch >> 2, stage_words = a.rows_in * P4;
   const int tile_mt = a.TR * a.mtw;
-  // The staged rows of a tile pass through registers: kCrStage words per thread (the host
-  // sizes the tiles for that), requested one tile ahead, so that they arrive while the
-  // tile in hand is multiplied.  Word u of thread t is word t + 256 u of the staged rows:
-  // its row and place in the row are the same for every tile.
-  int spos[kCrStage];  // row << 16 | byte in the row; -1: no such word
-#pragma unroll
-  for (int u = 0; u < kCrStage; ++u) {
-    const int idx = t + u * kCrThreads;
-    int r = static_cast<int>(static_cast<float>(idx) * a.rcp_p4);
-    int p4 = idx - r * P4;
-    if (p4 < 0) {
-      --r;
-      p4 += P4;
-    } else if (p4 >= P4) {
-      ++r;
-      p4 -= P4;
-    }
-    spos[u] = idx < stage_words ? (r << 16 | 4 * p4) : -1;
-  }
-  uint32_t pre[kCrStage];
-  // Staged row r of a tile starts shift(r) = (c0 + r * (row bytes % 4)) % 4 bytes before the
-  // tile's first byte of that image row, so that every staged word is an aligned word of
-  // memory: LDS byte q of the row is image-row byte iwb0 - shift(r) + q.
+  // The staged rows of a tile pass through registers, requested one tile ahead, so that they
+  // arrive while the tile in hand is multiplied.  The unit of the copy is 1 KB of one staged
+  // row, one 16-byte load per lane; unit u belongs to wave u % 4 (the host sizes the tiles
+  // for at most kCrUnits units per wave).  Staged row r starts
+  //   shift(r) = (c0 + r * (row bytes % 16)) % 16
+  // bytes before the tile's first byte of that image row, so that every load is an aligned
+  // 16 bytes of memory: LDS byte q of the row is image-row byte iwb0 - shift(r) + q.
+  const int segs = (a.pitch + 1023) >> 10, units = a.rows_in * segs;
+  v4i pre[kCrUnits];
   struct TilePos {
     int b, oh0, ow0, c0;
     int ih0, iwb0;        // image row and byte in the row of the tile's first staged byte (before the shift)
     int64_t first;        // the same as a byte offset into the tensor
-    int edge;             // some staged word may reach outside the tensor
+    int edge;             // some load may reach outside the tensor
   };
-  const int rb3 = row_bytes & 3;
+  const int rb15 = row_bytes & 15;
   const int64_t x_bytes = static_cast<int64_t>(a.B) * a.H * row_bytes;
   auto tile_pos = [&](uint32_t tile) {
     TilePos tp;
@@ -196,60 +173,64 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
     tp.ih0 = tp.oh0 * a.sh - a.ph;
     tp.iwb0 = (tp.ow0 * a.sw - a.pw) * a.IC;
     tp.first = (static_cast<int64_t>(tp.b) * a.H + tp.ih0) * row_bytes + tp.iwb0;
-    tp.c0 = static_cast<int>((reinterpret_cast<uintptr_t>(a.x) + static_cast<uintptr_t>(tp.first)) & 3);
-    tp.edge = tp.first < 4 || tp.first + static_cast<int64_t>(a.rows_in) * row_bytes + a.pitch + 4 > x_bytes;
+    tp.c0 = static_cast<int>((reinterpret_cast<uintptr_t>(a.x) + static_cast<uintptr_t>(tp.first)) & 15);
+    tp.edge = tp.first < 16 || tp.first + static_cast<int64_t>(a.rows_in) * row_bytes + a.pitch + 16 > x_bytes;
     return tp;
   };
-  // The loads only: whole aligned words, also where a word hangs over the end of its image
-  // row into the next one (store_tile masks those bytes); nothing here uses a loaded value,
-  // so nothing waits.  Only in the first and the last tiles of the tensor can a word reach
-  // outside it; those tiles check every byte.
+  // Unit `slot` of this wave: staged row, first LDS byte of the unit in that row (-1: none).
+  auto unit_pos = [&](int slot, int* r, int* q0) {
+    const int u = wave + kCrWaves * slot;
+    *r = segs == 1 ? u : u / segs;
+    *q0 = u < units ? (u - *r * segs) << 10 : -1;
+  };
+  // The loads only.  A load may hang over either end of its image row into the neighbouring
+  // rows (store_tile overwrites those bytes); nothing here uses a loaded value, so nothing
+  // waits.  Only in the first and the last tiles of the tensor can a load reach outside it;
+  // those tiles check every byte.
   auto request = [&](const TilePos& tp) {
-    const uint8_t* const base = a.x + (tp.first - 4);  // (an address to count from, not one to load from)
 #pragma unroll
-    for (int u = 0; u < kCrStage; ++u) {
-      pre[u] = 0;
-      if (u * kCrThreads >= stage_words) continue;  // (the same for the whole block)
-      const int r = spos[u] >> 16, q = spos[u] & 0xffff;
-      const int shift = (tp.c0 + r * rb3) & 3;
-      const int colb = tp.iwb0 - shift + q;
-      const bool ok = spos[u] >= 0 && static_cast<unsigned>(tp.ih0 + r) < static_cast<unsigned>(a.H) &&
-                      static_cast<unsigned>(colb + 3) < static_cast<unsigned>(row_bytes + 3);
-      const uint32_t off = static_cast<uint32_t>(r * row_bytes + q - shift + 4);
-      if (ok) {
-        if (!tp.edge) {
-          pre[u] = *reinterpret_cast<const uint32_t*>(base + off);
-        } else {
-          const int64_t rel = tp.first - 4 + static_cast<int64_t>(off);
-          uint32_t word = 0;
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj)
-            if (rel + jj >= 0 && rel + jj < x_bytes) word |= static_cast<uint32_t>(a.x[rel + jj]) << (8 * jj);
-          pre[u] = word;
+    for (int slot = 0; slot < kCrUnits; ++slot) {
+      int r, q0;
+      unit_pos(slot, &r, &q0);
+      if (q0 < 0 || static_cast<unsigned>(tp.ih0 + r) >= static_cast<unsigned>(a.H)) continue;  // (wave-uniform)
+      const int q = q0 + 16 * lane;
+      const int64_t rel = tp.first + static_cast<int64_t>(r) * row_bytes - ((tp.c0 + r * rb15) & 15) + q0;
+      if (q >= a.pitch) continue;
+      if (!tp.edge) {
+        pre[slot] = *reinterpret_cast<const v4i*>(a.x + rel + 16 * lane);
+      } else {
+        uint32_t w4[4] = {0, 0, 0, 0};
+        for (int jj = 0; jj < 16; ++jj) {
+          const int64_t o = rel + 16 * lane + jj;
+          if (o >= 0 && o < x_bytes) w4[jj >> 2] |= static_cast<uint32_t>(a.x[o]) << (8 * (jj & 3));
         }
+        pre[slot] = v4i{static_cast<int>(w4[0]), static_cast<int>(w4[1]), static_cast<int>(w4[2]), static_cast<int>(w4[3])};
       }
     }
   };
-  // Bytes outside the image (rows above and below, columns left and right of the row) become
-  // the activation zero point; then the sign flip, and into LDS.
+  // Into LDS with the sign flip; then the bytes outside the image -- whole rows above and
+  // below it, the ends of a row left and right of it -- become the activation zero point.
+  // A wave pads its own units, after its own stores to them.
   auto store_tile = [&](const TilePos& tp) {
+    const int xw = static_cast<int>(a.x_xor), pw4 = static_cast<int>(a.pad_word ^ a.x_xor);
+    const v4i xmask = {xw, xw, xw, xw}, padv = {pw4, pw4, pw4, pw4};
 #pragma unroll
-    for (int u = 0; u < kCrStage; ++u) {
-      if (u * kCrThreads >= stage_words || spos[u] < 0) continue;
-      const int r = spos[u] >> 16, q = spos[u] & 0xffff;
-      const int colb = tp.iwb0 - ((tp.c0 + r * rb3) & 3) + q;
-      uint32_t word = pre[u];
+    for (int slot = 0; slot < kCrUnits; ++slot) {
+      int r, q0;
+      unit_pos(slot, &r, &q0);
+      if (q0 < 0) continue;
       const bool row_in = static_cast<unsigned>(tp.ih0 + r) < static_cast<unsigned>(a.H);
-      if (!(row_in && colb >= 0 && colb + 3 < row_bytes)) {  // (the few words at the image's edges)
-        uint32_t keep = 0;
-        if (row_in) {
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj)
-            if (static_cast<unsigned>(colb + jj) < static_cast<unsigned>(row_bytes)) keep |= 0xffu << (8 * jj);
-        }
-        word = (word & keep) | (a.pad_word & ~keep);
-      }
-      *reinterpret_cast<uint32_t*>(sX + r * a.pitch + q) = word ^ a.x_xor;
+      uint8_t* const row = sX + r * a.pitch;
+      const int q = q0 + 16 * lane;
+      if (q < a.pitch) *reinterpret_cast<v4i*>(row + q) = row_in ? (pre[slot] ^ xmask) : padv;
+      if (!row_in) continue;
+      const int shift = (tp.c0 + r * rb15) & 15;
+      const int qend = q0 + 1024 < a.pitch ? q0 + 1024 : a.pitch;
+      // left of the image row: LDS bytes [0, shift - iwb0); right of it: [shift + row bytes - iwb0, pitch)
+      const int left = shift - tp.iwb0 < qend ? shift - tp.iwb0 : qend;
+      for (int i = q0 + lane; i < left; i += kWave) row[i] = static_cast<uint8_t>(pw4);
+      const int right = shift + row_bytes - tp.iwb0 > q0 ? shift + row_bytes - tp.iwb0 : q0;
+      for (int i = right + lane; i < qend; i += kWave) row[i] = static_cast<uint8_t>(pw4);
     }
   };
   TilePos cur{};
@@ -280,14 +261,14 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
       const int pcol = mcol * 16 + pj;
       const int pc = pcol < tw_valid ? pcol : tw_valid - 1;
       const int base = orow * a.sh * a.pitch + pc * a.sw * a.IC;
-      const int c0r = c0 + orow * a.sh * rb3;  // alignment shift of staged row orow * stride, before the % 4
+      const int c0r = c0 + orow * a.sh * rb15;  // alignment shift of staged row orow * stride, before the % 16
       v4i acc[4];  // start: the zero point's share, acc_coef * colsum
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) acc[nt] = *reinterpret_cast<const v4i*>(&s_acc0[16 * pq + 4 * nt]);
 #pragma unroll
       for (int ks = 0; ks < kCrMaxKS; ++ks) {
         if (ks < KS) {
-          const int addr = base + (lk[ks] & ~3) + ((c0r + lk[ks]) & 3);
+          const int addr = base + (lk[ks] & ~15) + ((c0r + lk[ks]) & 15);
           const uint32_t* const src = reinterpret_cast<const uint32_t*>(sX + (addr & ~3));
           const uint32_t sb = static_cast<uint32_t>(addr & 3);
           const uint32_t d0 = src[0], d1 = src[1], d2 = src[2], d3 = src[3], d4 = src[4];
