@@ -361,8 +361,8 @@ typedef struct tmq_conv2d_desc {
   void* y;
   /* 0: the library chooses.  Otherwise, for tests of every kernel family at any
    * shape: 1 halo tiles, 2 implicit GEMM, 3 direct, 4 kernel rows as byte runs
-   * (few input channels) (TMQ_ERR_UNSUPPORTED when the family cannot run the
-   * problem).  tile_rows / tile_cols > 0 pin the halo
+   * (few input channels), 5 a pointwise layer as tmq_linear (TMQ_ERR_UNSUPPORTED
+   * when the family cannot run the problem).  tile_rows / tile_cols > 0 pin the halo
    * kernel's patch height / bound its patch width. */
   int32_t kernel;
   int32_t tile_rows, tile_cols;

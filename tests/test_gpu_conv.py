@@ -198,6 +198,38 @@ def test_conv_narrow_groups_merged(cabi, spec, x_signed):
         _check(y, want, f"path {path}")
 
 
+@pytest.mark.parametrize("spec", [
+    (2, 14, 14, 256, 64, 1, 1, 0, 1, 1),
+    (32, 7, 7, 512, 200, 1, 1, 0, 1, 1),     # 1568 pixels, channels off the 16 grid on the output side
+    (1, 5, 5, 16, 24, 1, 1, 0, 1, 1),
+    (3, 56, 56, 64, 48, 1, 1, 0, 1, 1),      # more pixels than the automatic choice sends this way
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_pointwise_as_linear(cabi, spec, x_signed):
+    say("conv pointwise as linear", spec, x_signed)
+    c = _conv_case(*spec, seed=sum(spec) + 13, x_signed=x_signed, relu=not x_signed)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    for path in (5, 1, -1):
+        cabi.force_conv_path(path)
+        try:
+            y, _, _ = _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+        _check(y, want, f"path {path}")
+    # not a pointwise layer: stride, padding, kernel size, groups
+    for bad in [(1, 8, 8, 16, 16, 1, 2, 0, 1, 1), (1, 8, 8, 16, 16, 1, 1, 1, 1, 1), (1, 8, 8, 16, 16, 3, 1, 1, 1, 1),
+                (1, 8, 8, 32, 32, 1, 1, 0, 1, 2)]:
+        cb = _conv_case(*bad, seed=5)
+        cabi.force_conv_path(5)
+        try:
+            with pytest.raises(cabi.TmqError):
+                _run(cabi, cb)
+        finally:
+            cabi.force_conv_path(-1)
+
+
 def test_conv_byte_runs_limits(cabi):
     """groups, dilation and kernel rows beyond 256 padded bytes are not this kernel's."""
     say("conv byte runs limits")
