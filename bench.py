@@ -1140,6 +1140,60 @@ def main():
             "algorithmic_bytes_per_launch": pbytes}
         del pxs
 
+        # ------------------------- convolutions off the 16-channel grid: an image network's first
+        # layer (3 -> 64 channels, 7 x 7, stride 2, 224 x 224) and a depthwise layer (32 channels,
+        # 3 x 3, 112 x 112), batch 32, through torch.ops.quantized.conv2d_relu
+        def conv_line(name, ic, oc, k, stride, pad, groups, hw, what):
+            wf_ = torch.randn(oc, ic // groups, k, k) * 0.05
+            wq_ = torch.quantize_per_channel(wf_, wf_.abs().amax(dim=(1, 2, 3)) / 127, torch.zeros(oc, dtype=torch.long),
+                                             0, torch.qint8).to(dev)
+            packed_ = torch.ops.quantized.conv2d_prepack(wq_, torch.randn(oc, device=dev), [stride, stride], [pad, pad],
+                                                         [1, 1], groups)
+            nsets = 6
+            xqs_ = []
+            for _ in range(nsets):
+                xf_ = torch.relu(torch.randn(32, ic, hw, hw, device=dev)).contiguous(memory_format=torch.channels_last)
+                xqs_.append(torch.quantize_per_tensor(xf_, 0.03, 0, torch.quint8))
+                del xf_
+            cnt = [0]
+
+            def one():
+                cnt[0] += 1
+                return torch.ops.quantized.conv2d_relu(xqs_[cnt[0] % nsets], packed_, 0.05, 0)
+
+            for _ in range(3):
+                y_ = one()
+            oh_ = y_.shape[2]
+            g_ = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                one()
+                side.synchronize()
+                with torch.cuda.graph(g_, stream=side):
+                    for _ in range(2 * nsets):
+                        one()
+            torch.cuda.synchronize()
+            for _ in range(3):
+                g_.replay()
+            ts_ = events_ms(g_.replay, 10)
+            avg_ = sum(ts_) / len(ts_) / (2 * nsets)
+            nbytes_ = 32 * hw * hw * ic + 32 * oh_ * oh_ * oc + oc * (ic // groups) * k * k
+            ops_ = 2 * 32 * oh_ * oh_ * oc * (ic // groups) * k * k
+            log(f"[bench] {what}: {avg_*1e3:.1f} us/launch in a replayed graph, {nbytes_/(avg_*1e-3)/1e9:.0f} GB/s, "
+                f"{ops_/(avg_*1e-3)/1e12:.1f} TOP/s")
+            secondary[name] = {
+                "avg_launch_us": round(avg_ * 1e3, 2), "value": round(nbytes_ / (avg_ * 1e-3) / 1e9, 1), "unit": "GB/s",
+                "roofline": {"bound": "hbm", "achieved": round(nbytes_ / (avg_ * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                             "unit": "GB/s", "frac": round(nbytes_ / (avg_ * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                             "traffic": None},
+                "tops": round(ops_ / (avg_ * 1e-3) / 1e12, 2),
+                "method": f"{what}; {2 * nsets} launches over {nsets} rotating inputs replayed in one HIP graph",
+                "algorithmic_bytes_per_launch": nbytes_, "ops_per_launch": ops_}
+
+        conv_line("conv2d_relu_first_layer_7x7_s2_3to64", 3, 64, 7, 2, 3, 1, 224,
+                  "conv2d_relu 7x7 stride 2, 3 -> 64 channels, [32,3,224,224]")
+        conv_line("conv2d_relu_depthwise_3x3_32ch", 32, 32, 3, 1, 1, 32, 112,
+                  "conv2d_relu depthwise 3x3, 32 channels, [32,32,112,112]")
+
     # ------------------------------------------------------------ CPU baseline
     # The reference CPU path = PyTorch's own quantized CPU ops (fbgemm engine), timed on
     # this host's cores on bounded samples of the same workloads; the scalar C port of the

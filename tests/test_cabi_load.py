@@ -69,6 +69,20 @@ def test_packed_size_arithmetic():
     assert lib.tmq_conv2d_packed_bytes(g) == 4 * 40 * 256  # K = 576 -> 640 padded
     g2 = cabi.conv_geom((8, 32, 32, 3), (32, 7, 7), (2, 2), (3, 3), (1, 1), 1)
     assert cabi.conv_out_hw(g2) == (16, 16)
+    # few input channels: 49 taps of 16 padded bytes (784 -> 896) for two blocks of 16 channels, then the
+    # per-lane layout of the byte-run kernel: one 64-channel block x 4 channel tiles x 4 k-steps x 1 KB
+    assert lib.tmq_conv2d_packed_bytes(g2) == 2 * 56 * 256 + 4 * 4 * 1024
+    # kernel rows beyond 256 padded bytes in all (11 rows of 48): no second layout
+    g3 = cabi.conv_geom((1, 64, 64, 3), (16, 11, 11), (4, 4), (0, 0), (1, 1), 1)
+    assert lib.tmq_conv2d_packed_bytes(g3) == 1 * (121 * 16 + 127) // 128 * 8 * 256
+    # depthwise, 32 channels: the 32 groups are packed as one block-diagonal group, K = 9 taps x 32 channels
+    g4 = cabi.conv_geom((1, 20, 20, 32), (32, 3, 3), (1, 1), (1, 1), (1, 1), 32)
+    assert lib.tmq_conv2d_packed_bytes(g4) == 2 * 24 * 256
+    # 144 channels: three merged groups of 48; 40 channels: no multiple of 16 divides them, 40 groups of one
+    g5 = cabi.conv_geom((1, 20, 20, 144), (144, 3, 3), (1, 1), (1, 1), (1, 1), 144)
+    assert lib.tmq_conv2d_packed_bytes(g5) == 3 * 3 * 32 * 256
+    g6 = cabi.conv_geom((1, 20, 20, 40), (40, 3, 3), (1, 1), (1, 1), (1, 1), 40)
+    assert lib.tmq_conv2d_packed_bytes(g6) == 40 * 1 * 16 * 256
 
 
 def test_split_k_workspace_arithmetic():
