@@ -361,15 +361,29 @@ typedef struct tmq_conv2d_desc {
   void* y;
   /* 0: the library chooses.  Otherwise, for tests of every kernel family at any
    * shape: 1 halo tiles, 2 implicit GEMM, 3 direct, 4 kernel rows as byte runs
-   * (few input channels), 5 a pointwise layer as tmq_linear (TMQ_ERR_UNSUPPORTED
-   * when the family cannot run the problem).  tile_rows / tile_cols > 0 pin the halo
+   * (few input channels), 5 a pointwise layer as tmq_linear, 6 patch rows in the
+   * workspace, then tmq_linear (TMQ_ERR_UNSUPPORTED when the family cannot run
+   * the problem).  tile_rows / tile_cols > 0 pin the halo
    * kernel's patch height / bound its patch width. */
   int32_t kernel;
   int32_t tile_rows, tile_cols;
   int32_t reserved;
+  /* Optional scratch device memory, owned by the caller like every other buffer
+   * (16-byte aligned; contents undefined before and after the call).  With at
+   * least tmq_conv2d_workspace_bytes(&geom) bytes, layers with few output pixels
+   * against a long K (3 x 3 over hundreds of channels on a 14 x 14 or 7 x 7
+   * image) write their patch rows there and run as one quantized::linear over
+   * them.  NULL / too small: the single-launch kernels, same results. */
+  void* workspace;
+  int64_t workspace_bytes;
 } tmq_conv2d_desc;
 
 int tmq_conv2d(const tmq_conv2d_desc* desc, tmq_stream_t stream);
+/* Bytes of workspace that tmq_conv2d can use for this geometry (B, H, W included);
+ * 0 when the single-launch kernels are chosen anyway.  No counterpart in the
+ * reference: muDNN allocates its own scratch through the InternalMemAlloc
+ * callback (torch_musa/csrc/aten/utils/Utils.cpp:79-153). */
+int64_t tmq_conv2d_workspace_bytes(const tmq_conv2d_geom* g);
 /* Zero-point-corrected accumulators, [B,OH,OW,OC] int32:
  * acc = sum over in-image taps of (x - x_zp) * w. */
 int tmq_conv2d_acc32(const tmq_conv2d_desc* desc, int32_t* acc, tmq_stream_t stream);

@@ -53,7 +53,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(cabi.LinearDesc) == 144
     assert C.sizeof(cabi.LinearChoice) == 48
     assert C.sizeof(cabi.Conv2dGeom) == 14 * 8
-    assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8 + 16
+    assert C.sizeof(cabi.Conv2dDesc) == 14 * 8 + 8 + 16 + 32 + 16 + 8 + 16 + 16
     assert C.sizeof(cabi.Conv2dPost) == 24
 
 
@@ -83,6 +83,13 @@ def test_packed_size_arithmetic():
     assert lib.tmq_conv2d_packed_bytes(g5) == 3 * 3 * 32 * 256
     g6 = cabi.conv_geom((1, 20, 20, 40), (40, 3, 3), (1, 1), (1, 1), (1, 1), 40)
     assert lib.tmq_conv2d_packed_bytes(g6) == 40 * 1 * 16 * 256
+    # scratch for layers that run on their patch rows: few pixels against a long K that the halo tiles do not hold
+    wsb = lib.tmq_conv2d_workspace_bytes
+    assert wsb(cabi.conv_geom((1, 7, 7, 512), (512, 3, 3), (1, 1), (1, 1), (1, 1), 1)) == 49 * 4608
+    assert wsb(cabi.conv_geom((2, 14, 14, 256), (256, 3, 3), (1, 1), (1, 1), (1, 1), 1)) == 392 * 2304
+    assert wsb(cabi.conv_geom((8, 14, 14, 256), (256, 3, 3), (1, 1), (1, 1), (1, 1), 1)) == 0    # 1568 pixels
+    assert wsb(g) == 0 and wsb(g2) == 0 and wsb(g4) == 0                                       # C5, few channels, depthwise
+    assert wsb(cabi.conv_geom((1, 14, 14, 2048), (512, 1, 1), (1, 1), (0, 0), (1, 1), 1)) == 0    # pointwise: rows already
 
 
 def test_split_k_workspace_arithmetic():

@@ -230,6 +230,121 @@ def test_conv_pointwise_as_linear(cabi, spec, x_signed):
             cabi.force_conv_path(-1)
 
 
+@pytest.mark.parametrize("spec", [
+    (1, 14, 14, 256, 64, 3, 1, 1, 1, 1),     # 36 stages of 64 bytes: 18 per wave group
+    (2, 7, 7, 512, 96, 3, 1, 1, 1, 1),       # 72 stages, channels over two tiles
+    (1, 9, 9, 128, 64, 3, 2, 1, 1, 1),       # 18 stages (pinned only), stride 2
+    (2, 10, 10, 256, 64, 3, 1, 1, 1, 2),     # two groups of 128 -> 32
+    (1, 6, 6, 48, 40, 5, 1, 2, 1, 1),        # 1200 bytes of K: 19 stages, odd: refused
+    (1, 8, 8, 128, 64, 3, 1, 1, 1, 1),       # 18 stages: two groups, not four
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+@pytest.mark.parametrize("wave_groups", [2, 4])
+def test_conv_gemm_wave_groups(cabi, spec, x_signed, wave_groups):
+    say("conv gemm wave groups", spec, x_signed, wave_groups)
+    c = _conv_case(*spec, seed=sum(spec) + 17, x_signed=x_signed, relu=x_signed)
+    kbytes = spec[5] * spec[5] * spec[3] // spec[9]
+    even = (-(-kbytes // 64)) % wave_groups == 0
+    cabi.force_conv_path(2)
+    cabi.force_conv_tile(0, wave_groups)
+    try:
+        if not even:
+            with pytest.raises(cabi.TmqError):
+                _run(cabi, c)
+            return
+        y, acc, _ = _run(cabi, c)
+    finally:
+        cabi.force_conv_path(-1)
+        cabi.force_conv_tile(0, 0)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"], c["groups"], c["x_zp"],
+                                 nthreads=8))
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], c["stride"],
+                         c["padding"], c["dilation"], c["groups"], c["out_scale"], c["out_zp"], relu=c["relu"],
+                         nthreads=8)
+    _check(y, want, "wave groups")
+    y2, _, _ = _run(cabi, c)   # the automatic choice
+    _check(y2, want, "auto")
+
+
+@pytest.mark.parametrize("activation", ["relu", "silu"])
+@pytest.mark.parametrize("wave_groups", [2, 4])
+def test_conv_gemm_wave_groups_fused(cabi, activation, wave_groups):
+    """residual and activation behind the wave groups' sum (256 -> 64 channels, 3 x 3, 14 x 14)."""
+    say("conv gemm wave groups fused", activation, wave_groups)
+    rng = np.random.default_rng(58)
+    xq = rng.integers(0, 256, (2, 14, 14, 256), dtype=np.uint8)
+    wq = rng.integers(-127, 128, (64, 3, 3, 256), dtype=np.int8)
+    accq = rng.integers(0, 256, (2, 14, 14, 64), dtype=np.uint8)
+    ws = (0.001 + 0.002 * rng.random(64)).astype(np.float32).astype(np.float64)
+    bias = rng.standard_normal(64).astype(np.float32)
+    c = dict(xq=xq, wq=wq, accq=accq, w_scales=ws, bias=bias, x_scale=0.02, x_zp=3, stride=(1, 1),
+             padding=(1, 1), dilation=(1, 1), groups=1, out_scale=1.8, out_zp=20, acc_scale=0.35,
+             acc_zp=110, activation=activation, signed=False)
+    cabi.force_conv_path(2)
+    cabi.force_conv_tile(0, wave_groups)
+    try:
+        y = _run_fused(cabi, c)
+    finally:
+        cabi.force_conv_path(-1)
+        cabi.force_conv_tile(0, 0)
+    want = oracle.conv2d_fused(xq, 0.02, 3, wq, ws, bias, (1, 1), (1, 1), (1, 1), 1, 1.8, 20, accum=accq,
+                               accum_scale=0.35, accum_zp=110, activation=activation, nthreads=8)
+    d = np.abs(y.astype(np.int32) - want.astype(np.int32))
+    if activation == "silu":
+        assert d.max() <= LSB_TOL and np.count_nonzero(d) <= 0.001 * d.size, (d.max(), np.count_nonzero(d))
+    else:
+        assert d.max() == 0, f"{np.count_nonzero(d)} of {d.size} bytes differ (max {d.max()})"
+
+
+@pytest.mark.parametrize("spec", [
+    (1, 7, 7, 512, 72, 3, 1, 1, 1, 1),       # one 7 x 7 image, K = 4608: the library asks for the workspace itself
+    (2, 14, 14, 256, 96, 3, 1, 1, 1, 1),     # 392 pixels, K = 2304
+    (3, 14, 14, 256, 64, 3, 2, 1, 1, 1),     # stride 2
+    (2, 9, 9, 32, 24, 3, 2, 1, 1, 1),        # small K: pinned only
+    (1, 10, 10, 16, 16, 3, 1, 2, 2, 1),      # dilation (pinned only)
+    (1, 5, 5, 48, 20, 1, 1, 0, 1, 1),        # pointwise (pinned only): the patch rows are the pixels
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_on_patch_rows(cabi, spec, x_signed):
+    say("conv on patch rows", spec, x_signed)
+    c = _conv_case(*spec, seed=sum(spec) + 19, x_signed=x_signed, relu=not x_signed)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], c["stride"],
+                         c["padding"], c["dilation"], c["groups"], c["out_scale"], c["out_zp"], relu=c["relu"],
+                         nthreads=8)
+    g = cabi.conv_geom(c["xq"].shape, c["wq"].shape, c["stride"], c["padding"], c["dilation"], c["groups"])
+    oh, ow = cabi.conv_out_hw(g)
+    kbytes = spec[5] * spec[5] * spec[3]
+    asked = cabi.lib().tmq_conv2d_workspace_bytes(g)
+    assert asked == (spec[0] * oh * ow * kbytes if kbytes >= 2048 else 0)
+    for path, ws in ((6, True), (-1, True), (-1, False)):
+        cabi.force_conv_path(path)
+        cabi.use_conv_workspace(ws)
+        try:
+            y, _, _ = _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+            cabi.use_conv_workspace(True)
+        _check(y, want, f"path {path} workspace {ws}")
+    # pinned without a workspace, or for a shape that has no patch rows of whole 16-channel blocks
+    cabi.force_conv_path(6)
+    cabi.use_conv_workspace(False)
+    try:
+        with pytest.raises(cabi.TmqError):
+            _run(cabi, c)
+    finally:
+        cabi.force_conv_path(-1)
+        cabi.use_conv_workspace(True)
+    for bad in [(1, 8, 8, 32, 32, 3, 1, 1, 1, 2), (1, 8, 8, 24, 16, 3, 1, 1, 1, 1)]:
+        cb = _conv_case(*bad, seed=5)
+        cabi.force_conv_path(6)
+        try:
+            with pytest.raises(cabi.TmqError):
+                _run(cabi, cb)
+        finally:
+            cabi.force_conv_path(-1)
+
+
 def test_conv_byte_runs_limits(cabi):
     """groups, dilation and kernel rows beyond 256 padded bytes are not this kernel's."""
     say("conv byte runs limits")

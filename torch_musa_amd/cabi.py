@@ -25,7 +25,7 @@ DECLARED_SYMBOLS = [
     "tmq_quantize_per_channel_float_qparams", "tmq_dequantize_per_channel_float_qparams",
     "tmq_linear_packed_kchunks", "tmq_linear_packed_bytes", "tmq_linear_prepack",
     "tmq_linear_unpack", "tmq_linear", "tmq_linear_workspace_bytes", "tmq_linear_split_plan", "tmq_linear_kernel_choice", "tmq_linear_static_workspace", "tmq_linear_acc32", "tmq_linear_f32", "tmq_linear_dynamic_small", "tmq_linear_dynamic_small_takes", "tmq_quantize_per_tensor_dynamic_dev",
-    "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw",
+    "tmq_conv2d_packed_bytes", "tmq_conv2d_prepack", "tmq_conv2d_out_hw", "tmq_conv2d_workspace_bytes",
     "tmq_conv2d", "tmq_conv2d_acc32", "tmq_conv2d_fused",
     "tmq_qadd", "tmq_qrelu", "tmq_qcat_rows", "tmq_qmaxpool2d", "tmq_qadaptive_avgpool2d", "tmq_qunary",
 ]
@@ -78,6 +78,7 @@ class Conv2dDesc(C.Structure):
         ("out_signed", C.c_int32), ("relu", C.c_int32),
         ("y", C.c_void_p),
         ("kernel", C.c_int32), ("tile_rows", C.c_int32), ("tile_cols", C.c_int32), ("reserved", C.c_int32),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
     ]
 
 
@@ -115,6 +116,8 @@ def lib() -> C.CDLL:
                                                C.c_int32, C.POINTER(LinearChoice)]
         l.tmq_conv2d_packed_bytes.restype = C.c_int64
         l.tmq_conv2d_packed_bytes.argtypes = [C.POINTER(Conv2dGeom)]
+        l.tmq_conv2d_workspace_bytes.restype = C.c_int64
+        l.tmq_conv2d_workspace_bytes.argtypes = [C.POINTER(Conv2dGeom)]
         v = C.c_void_p
         l.tmq_quantize_per_tensor.argtypes = [v, v, C.c_int64, C.c_double, C.c_int64, C.c_int, v]
         l.tmq_dequantize_per_tensor.argtypes = [v, v, C.c_int64, C.c_double, C.c_int64, C.c_int, v]
@@ -469,9 +472,19 @@ def force_linear_config(cfg: int) -> None:
 
 def force_conv_path(path: int) -> None:
     """Pin the conv2d kernel family of later calls through this binding
-    (-1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct, 4 byte runs, 5 pointwise as linear)."""
+    (-1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct, 4 byte runs, 5 pointwise as linear,
+    6 patch rows in a workspace + linear)."""
     global _conv_path
     _conv_path = int(path)
+
+
+_conv_workspace = True
+
+
+def use_conv_workspace(on: bool) -> None:
+    """Whether later conv2d calls through this binding pass the scratch memory the library asks for."""
+    global _conv_workspace
+    _conv_workspace = bool(on)
 
 
 def force_conv_tile(rows: int, cols: int) -> None:
@@ -549,6 +562,14 @@ def _conv_desc(x, pw, g, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_s
     d.y = _ptr(y)
     d.kernel = _conv_path if _conv_path > 0 else 0
     d.tile_rows, d.tile_cols = _conv_tile
+    # scratch for the layers that run on their patch rows (pinned for tests: whatever the size)
+    need = lib().tmq_conv2d_workspace_bytes(C.byref(g))
+    if _conv_path == 6 and g.groups == 1 and g.IC % 16 == 0:
+        oh, ow = conv_out_hw(g)
+        need = g.B * oh * ow * g.KH * g.KW * g.IC
+    if need > 0 and _conv_workspace:
+        d._ws = torch.empty(need, dtype=torch.uint8, device=x.device)   # (kept alive by the descriptor)
+        d.workspace, d.workspace_bytes = d._ws.data_ptr(), need
     return d
 
 

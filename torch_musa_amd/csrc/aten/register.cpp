@@ -631,6 +631,15 @@ struct PackedConvWeightTmq final : public ConvPackedParamsBase<2> {
     d.relu = activation == 1;
     d.y = y.data_ptr();
     if (!accum.has_value() && activation != 2) {
+      // scratch for the layers that run on their patch rows (from the caching allocator:
+      // safe under stream capture, freed for reuse in stream order)
+      at::Tensor workspace;
+      const int64_t ws_bytes = tmq_conv2d_workspace_bytes(&g);
+      if (ws_bytes > 0) {
+        workspace = at::empty({ws_bytes}, x.options().dtype(at::kByte));
+        d.workspace = workspace.data_ptr();
+        d.workspace_bytes = ws_bytes;
+      }
       check_status(tmq_conv2d(&d, current_stream(x)), "tmq_conv2d");
       return y;
     }
@@ -1413,6 +1422,13 @@ at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero
   d.relu = relu;
   d.y = y.data_ptr();
   if (!accum.has_value()) {
+    at::Tensor workspace;  // (as in PackedConvWeightTmq::apply)
+    const int64_t ws_bytes = tmq_conv2d_workspace_bytes(&g);
+    if (ws_bytes > 0) {
+      workspace = at::empty({ws_bytes}, act.options().dtype(at::kByte));
+      d.workspace = workspace.data_ptr();
+      d.workspace_bytes = ws_bytes;
+    }
     check_status(tmq_conv2d(&d, stream), "tmq_conv2d");
     return y;
   }

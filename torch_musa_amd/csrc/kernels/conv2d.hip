@@ -14,14 +14,18 @@
 #include "gemm_i8_core.h"
 
 static_assert(sizeof(tmq_conv2d_geom) == 112, "tmq_conv2d_geom layout changed");
-static_assert(sizeof(tmq_conv2d_desc) == 208, "tmq_conv2d_desc layout changed");
+static_assert(sizeof(tmq_conv2d_desc) == 224, "tmq_conv2d_desc layout changed");
 static_assert(sizeof(tmq_conv2d_post) == 24, "tmq_conv2d_post layout changed");
 
 namespace tmq {
 namespace {
 
 constexpr int64_t kKPad = 128;
-constexpr int64_t kPointwiseAsLinearRows = 8192;  // pixels up to which a pointwise layer runs as a linear layer
+constexpr int64_t kTwoGroupTiles = 512;          // 64 x 64 tiles up to which the implicit GEMM splits K over two wave groups
+constexpr int64_t kFourGroupTiles = 256;         // ... over four (K of 64 stages and more)
+constexpr int64_t kPointwiseAsLinearRows = 8192;
+constexpr int64_t kPatchRowsMax = 512;           // output pixels up to which a layer may run on its patch rows (workspace)
+constexpr int64_t kPatchRowsMinK = 2048;         // and the K from which on  // pixels up to which a pointwise layer runs as a linear layer
 inline int64_t packed_kchunks(int64_t K) { return (K + kKPad - 1) / kKPad * (kKPad / 16); }
 
 struct ConvShape {
@@ -141,6 +145,41 @@ __global__ __launch_bounds__(256) void conv_colsum_kernel(const int8_t* __restri
   if (lane == 0) colsum[n] = s;
 }
 
+// Patch rows (im2col) of a convolution over whole 16-channel blocks, one group: row m = output
+// pixel (b, oh, ow), k = (kh, kw, ic) as in the packed weight; one thread per 16-byte chunk.
+// Taps outside the image are the activation zero point.
+__global__ __launch_bounds__(256) void conv_patch_rows_kernel(const uint8_t* __restrict__ x, ConvShape s, int64_t total,
+                                                              uint32_t pad_word, uint8_t* __restrict__ rows) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const uint32_t kc = static_cast<uint32_t>(s.Kp / 16), icb = static_cast<uint32_t>(s.IC / 16);
+  const uint32_t m = static_cast<uint32_t>(id / kc), c = static_cast<uint32_t>(id - static_cast<int64_t>(m) * kc);
+  const uint32_t tap = c / icb, blk = c - tap * icb;
+  const uint32_t kh = tap / static_cast<uint32_t>(s.KW), kw = tap - kh * static_cast<uint32_t>(s.KW);
+  const uint32_t ow = m % static_cast<uint32_t>(s.OW), t = m / static_cast<uint32_t>(s.OW);
+  const uint32_t oh = t % static_cast<uint32_t>(s.OH), b = t / static_cast<uint32_t>(s.OH);
+  const int ih = static_cast<int>(oh * s.sh) - static_cast<int>(s.ph) + static_cast<int>(kh * s.dh);
+  const int iw = static_cast<int>(ow * s.sw) - static_cast<int>(s.pw) + static_cast<int>(kw * s.dw);
+  const int pw = static_cast<int>(pad_word);
+  v4i v = {pw, pw, pw, pw};
+  if (static_cast<unsigned>(ih) < static_cast<unsigned>(s.H) && static_cast<unsigned>(iw) < static_cast<unsigned>(s.W))
+    v = ld16(x + ((static_cast<int64_t>(b) * s.H + ih) * s.W + iw) * s.IC + blk * 16);
+  *reinterpret_cast<v4i*>(rows + id * 16) = v;
+}
+
+// Whether a layer may run on its patch rows, and the bytes they take: one group over whole
+// 16-channel blocks, few output pixels, a long K, and no halo tiles for it.
+int64_t patch_rows_bytes(const tmq_conv2d_geom& g, const ConvShape& s, bool pinned) {
+  if (g.groups != 1 || s.IC % 16 != 0) return 0;
+  const int64_t rows = s.B * s.OH * s.OW;
+  if (rows == 0 || rows * (s.Kp / 16) > 0x7fffffff) return 0;
+  if (!pinned) {
+    if (rows > kPatchRowsMax || s.Kp < kPatchRowsMinK) return 0;
+    if (s.KH == 1 && s.KW == 1 && s.sh == 1 && s.sw == 1 && s.ph == 0 && s.pw == 0) return 0;  // (already rows)
+  }
+  return rows * s.Kp;
+}
+
 struct PlainArgs {
   const uint8_t* x;
   const uint8_t* w_packed;
@@ -210,12 +249,12 @@ __global__ __launch_bounds__(256) void conv_plain_kernel(ConvShape s, PlainArgs 
   }
 }
 
-template <int BM, int BN, int WM, int WN, int MODE>
+template <int BM, int BN, int WM, int WN, int MODE, int KW = 1>
 int launch_conv_gemm(const GemmArgs& a, const XConv& xs, hipStream_t s) {
   const int64_t blocks = ceil_div(a.M, BM) * ceil_div(a.N, BN);
   if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
-  gemm_i8_kernel<BM, BN, WM, WN, MODE, XConv>
-      <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * kWave), 0, s>>>(a, xs);
+  gemm_i8_kernel<BM, BN, WM, WN, MODE, XConv, 4, false, KW>
+      <<<dim3(static_cast<unsigned>(blocks)), dim3(WM * WN * KW * kWave), 0, s>>>(a, xs);
   return launch_status();
 }
 
@@ -543,6 +582,38 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
       return tmq_linear(&l, reinterpret_cast<tmq_stream_t>(stream));
     }
   }
+  // Few output pixels against a long K and a weight slice the halo tiles cannot hold: with a
+  // workspace the patch rows are written out and the product runs on the linear kernels
+  // (3 x 3, 256 -> 256 channels, one 14 x 14 image: 13.1 -> 10.1 us; 512 -> 512, one 7 x 7 image:
+  // 19.8 -> 16.1 us, eight of them 19.7 -> 17.2 us; from about a thousand pixels on the implicit
+  // GEMM with its wave groups is ahead: 1568 pixels, 256 -> 256: 13.6 against 15.4 us).
+  if constexpr (MODE != kOutAcc32) {
+    if (forced == 6 || forced < 0) {
+      const int64_t need = po.any() || !aligned(d->x, 16) ? 0 : patch_rows_bytes(d->geom, s, forced == 6);
+      TilePlan tp;
+      const bool use = need > 0 && d->workspace != nullptr && d->workspace_bytes >= need && aligned(d->workspace, 16) &&
+                       (forced == 6 || !plan_tiles(s, false, 0, 0, &tp));
+      if (forced == 6 && !use) return TMQ_ERR_UNSUPPORTED;
+      if (use) {
+        const int64_t chunks = need / 16;
+        conv_patch_rows_kernel<<<dim3(static_cast<unsigned>(ceil_div(chunks, 256))), dim3(256), 0, stream>>>(
+            static_cast<const uint8_t*>(d->x), s, chunks,
+            0x01010101u * static_cast<uint32_t>(static_cast<uint8_t>(d->x_zero_point)), static_cast<uint8_t*>(d->workspace));
+        if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+        tmq_linear_desc l{};
+        l.M = rows; l.N = s.OC; l.K = s.Kp;
+        l.x = d->workspace; l.ldx = s.Kp;
+        l.x_signed = d->x_signed; l.x_zero_point = d->x_zero_point; l.x_scale = d->x_scale;
+        l.w_packed = d->w_packed; l.w_colsum = d->w_colsum; l.w_scales = d->w_scales;
+        l.w_per_channel = d->w_per_channel;
+        l.relu = relu ? 1 : 0;
+        l.bias = d->bias;
+        l.out_scale = d->out_scale; l.out_zero_point = d->out_zero_point; l.out_signed = d->out_signed;
+        l.y = out; l.ldy = s.OC;
+        return tmq_linear(&l, reinterpret_cast<tmq_stream_t>(stream));
+      }
+    }
+  }
   const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
   if ((forced == 1 || forced == 2) && !mfma_ok) return TMQ_ERR_UNSUPPORTED;
   // channel counts (or an address) the 16-byte chunks of the kernels below cannot take:
@@ -648,6 +719,25 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   a.y = out;
   a.ldy = s.OC;
   a.post = po;
+  // Few 64 x 64 tiles against a long K (3 x 3 layers over hundreds of channels on small images):
+  // two or four wave groups per block walk a half or a quarter of K each, as in quantized::linear.
+  // (pinned for tests: tile_cols = 1, 2 or 4 groups)
+  const int64_t stages = ceil_div(s.Kp, kBK);
+  const int64_t tiles64 = ceil_div(rows, 64) * ceil_div(s.OCg, 64) * s.groups;
+  const bool small_tiles = !(s.OCg > 64 && rows >= 128 * 128) && rows < 256 * 256;
+  int wave_groups = 1;
+  if (forced == 2 && d->tile_cols > 0) {
+    wave_groups = d->tile_cols;
+    if (wave_groups != 1 && ((wave_groups != 2 && wave_groups != 4) || !small_tiles || stages % wave_groups != 0))
+      return TMQ_ERR_UNSUPPORTED;
+  } else if (small_tiles && stages >= 32) {
+    // (four groups from 64 stages on: K = 4608, 200 tiles: 20.9 against 21.9 us with two, 56 tiles: 19.7 against
+    // 20.4 us; K = 2304: level at 100 tiles, 27 against 20.7 us at 392)
+    if (stages % 4 == 0 && stages >= 64 && tiles64 <= kFourGroupTiles)
+      wave_groups = 4;
+    else if (stages % 2 == 0 && tiles64 <= kTwoGroupTiles)
+      wave_groups = 2;
+  }
   for (int64_t g = 0; g < s.groups; ++g) {
     a.w_packed = static_cast<const uint8_t*>(d->w_packed) + g * s.group_bytes;
     a.n_off = static_cast<int32_t>(g * s.OCg);
@@ -656,6 +746,10 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
       rc = launch_conv_gemm<128, 128, 2, 2, MODE>(a, xs, stream);
     else if (rows >= 256 * 256)
       rc = launch_conv_gemm<256, 64, 4, 1, MODE>(a, xs, stream);
+    else if (wave_groups == 4)
+      rc = launch_conv_gemm<64, 64, 2, 2, MODE, 4>(a, xs, stream);
+    else if (wave_groups == 2)
+      rc = launch_conv_gemm<64, 64, 2, 2, MODE, 2>(a, xs, stream);
     else
       rc = launch_conv_gemm<64, 64, 2, 2, MODE>(a, xs, stream);
     if (rc != TMQ_OK) return rc;
@@ -672,6 +766,14 @@ TMQ_EXPORT int64_t tmq_conv2d_packed_bytes(const tmq_conv2d_geom* g) {
   ConvShape s;
   if (make_shape(g, &s) != TMQ_OK) return 0;
   return s.groups * s.group_bytes + s.runs_bytes;
+}
+
+TMQ_EXPORT int64_t tmq_conv2d_workspace_bytes(const tmq_conv2d_geom* g) {
+  ConvShape s;
+  if (make_shape(g, &s) != TMQ_OK) return 0;
+  TilePlan tp;
+  const int64_t need = patch_rows_bytes(*g, s, false);
+  return need > 0 && !(s.ICg % 16 == 0 && plan_tiles(s, false, 0, 0, &tp)) ? need : 0;
 }
 
 TMQ_EXPORT int tmq_conv2d_out_hw(const tmq_conv2d_geom* g, int64_t* OH, int64_t* OW) {

@@ -59,6 +59,7 @@ struct XConv {
   int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
   int ic_off;        // first input channel of this group
   uint32_t pad_word; // activation zero point replicated in 4 bytes
+  int kc0;           // first 16-byte k-chunk of this wave group's share of K (k-split groups), else 0
 };
 
 // Optional work between the requantisation's multiply and its rounding:
@@ -233,8 +234,8 @@ struct KCursor<XConv> {
   __device__ __forceinline__ void init(const XConv& s, int c_) {
     c = c_;
     kt_cur = 0;
-    const int tap = c_ / s.icb;
-    blk = c_ - tap * s.icb;
+    const int tap = (c_ + s.kc0) / s.icb;
+    blk = c_ + s.kc0 - tap * s.icb;
     kh = tap / s.KW;
     kw = tap - kh * s.KW;
     place(s);
@@ -383,7 +384,7 @@ __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv,
 // eight waves, mixed with their fragment reads, backs up the LDS queue and the
 // fragment reads behind it.
 //
-// KW > 1 (register staging of plain activation rows only): KW groups of WM x WN
+// KW > 1 (register staging only): KW groups of WM x WN
 // waves share one output tile and split its k loop into KW equal runs of
 // stages, each group with its own LDS stages and registers; after the loop the
 // groups' accumulators are added through LDS and group 0 runs the epilogue.
@@ -397,8 +398,7 @@ __global__ __launch_bounds__(WM* WN* KW* kWave, (WDMA && WM * WN == 4 && (BM / W
 void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
   constexpr int NT = WM * WN * kWave;   // threads of one group
   constexpr int NTB = NT * KW;          // threads of the block
-  static_assert(KW >= 1 && (KW == 1 || (!WDMA && std::is_same<XSRC, XLinear>::value)),
-                "k-split groups: register staging of plain rows only");
+  static_assert(KW >= 1 && (KW == 1 || !WDMA), "k-split groups: register staging only");
   const int kg = KW == 1 ? 0 : static_cast<int>(threadIdx.x) / NT;  // this thread's group
   if constexpr (KW > 1) {  // this group's share of K: move the operands, shorten K
     const int64_t per = ceil_div(a.K, kBK) / KW;
@@ -406,7 +406,10 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
     const int64_t left = a.K - k0;
     a.K = left < per * kBK ? left : per * kBK;
     a.w_packed += kg * per * (kChunks * 256);
-    xsrc.x += k0;
+    if constexpr (std::is_same<XSRC, XLinear>::value)
+      xsrc.x += k0;
+    else
+      xsrc.kc0 += static_cast<int>(k0 / 16);
   }
   constexpr bool kHasPost = XSRC::kPostOps;  // residual / activation epilogue compiled in
   if constexpr (MODE == kOutAcc32 && std::is_same<XSRC, XLinear>::value) {
