@@ -1189,6 +1189,48 @@ def main():
                 "method": f"{what}; {2 * nsets} launches over {nsets} rotating inputs replayed in one HIP graph",
                 "algorithmic_bytes_per_launch": nbytes_, "ops_per_launch": ops_}
 
+        # ------------------------- every convolution of a ResNet-50 (53 layers, 23 distinct shapes), per
+        # shape through the C ABI in a replayed graph over rotating inputs, summed with the shape's count:
+        # what the layers of the operator cost next to one another at batch 32 and on a single image
+        def resnet50_convs(batch):
+            shapes = [(3, 64, 7, 2, 224, 1), (64, 64, 1, 1, 56, 1), (64, 64, 3, 1, 56, 3), (64, 256, 1, 1, 56, 4),
+                      (256, 64, 1, 1, 56, 2), (256, 128, 1, 1, 56, 1), (128, 128, 3, 2, 56, 1), (128, 512, 1, 1, 28, 4),
+                      (256, 512, 1, 2, 56, 1), (512, 128, 1, 1, 28, 3), (128, 128, 3, 1, 28, 3), (512, 256, 1, 1, 28, 1),
+                      (256, 256, 3, 2, 28, 1), (256, 1024, 1, 1, 14, 6), (512, 1024, 1, 2, 28, 1), (1024, 256, 1, 1, 14, 5),
+                      (256, 256, 3, 1, 14, 5), (1024, 512, 1, 1, 14, 1), (512, 512, 3, 2, 14, 1), (512, 2048, 1, 1, 7, 3),
+                      (1024, 2048, 1, 2, 14, 1), (2048, 512, 1, 1, 7, 2), (512, 512, 3, 1, 7, 2)]
+            total_us, rows_, layers = 0.0, [], 0
+            for ic, oc, k, st, hw, count in shapes:
+                g_ = cabi.conv_geom((batch, hw, hw, ic), (oc, k, k), (st, st), (k // 2, k // 2), (1, 1), 1)
+                oh_, ow_ = cabi.conv_out_hw(g_)
+                nbytes_ = batch * hw * hw * ic + batch * oh_ * ow_ * oc
+                nsets = max(2, min(6, (600 << 20) // nbytes_))
+                xs_ = [torch.randint(0, 256, (batch, hw, hw, ic), dtype=torch.uint8, device=dev) for _ in range(nsets)]
+                pw_ = cabi.PackedConv2d(torch.randint(-127, 128, (oc, k, k, ic), dtype=torch.int8, device=dev), g_)
+                ws_, b_ = torch.rand(oc, device=dev) * 0.002 + 0.001, torch.randn(oc, device=dev)
+                ys_ = [torch.empty((batch, oh_, ow_, oc), dtype=torch.uint8, device=dev) for _ in range(nsets)]
+
+                def run_():
+                    for x_, y_ in zip(xs_, ys_):
+                        cabi.conv2d(x_, pw_, g_, 0.02, 128, ws_, b_, 0.05, 128, relu=True, out=y_)
+
+                us_ = graph_us(run_, nsets)
+                total_us += count * us_
+                layers += count
+                rows_.append({"ic": ic, "oc": oc, "k": k, "stride": st, "hw": hw, "count": count, "us": round(us_, 2)})
+                del xs_, ys_, pw_
+            return total_us, layers, rows_
+
+        for batch_ in (32, 1):
+            tot_, layers_, rows_ = resnet50_convs(batch_)
+            log(f"[bench] ResNet-50 convolutions, batch {batch_}: {layers_} layers, {tot_:.0f} us in all "
+                f"({tot_/layers_:.1f} us per layer)")
+            secondary[f"conv2d_relu_resnet50_stack_b{batch_}"] = {
+                "layers": layers_, "total_us": round(tot_, 1), "per_layer_us": round(tot_ / layers_, 2),
+                "images_per_s_convs_only": round(batch_ / (tot_ * 1e-6), 1), "shapes": rows_,
+                "method": "each distinct shape timed alone through tmq_conv2d (with ReLU) in a replayed HIP graph over "
+                          "rotating inputs, times its count; 224 x 224 images, NHWC"}
+
         conv_line("conv2d_relu_first_layer_7x7_s2_3to64", 3, 64, 7, 2, 3, 1, 224,
                   "conv2d_relu 7x7 stride 2, 3 -> 64 channels, [32,3,224,224]")
         conv_line("conv2d_relu_depthwise_3x3_32ch", 32, 32, 3, 1, 1, 32, 112,
