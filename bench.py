@@ -171,7 +171,8 @@ def main():
                     help="do not start the child process that samples the socket power (for runs under a profiler, "
                          "whose library has initialised the GPU before this program starts)")
     ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
-                                       "dequantize_pc", "decode", "rows64", "rows256", "c1", "decode16_proj", "conv", "conv_add_relu", "probe", "choice"],
+                                       "dequantize_pc", "decode", "rows64", "rows256", "c1", "decode16_proj", "conv", "conv_add_relu", "conv_first_layer", "conv_depthwise",
+                                       "probe", "choice"],
                     help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
                          "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
                          "1 GiB device copy used to calibrate the FETCH_SIZE / WRITE_SIZE counters")
@@ -378,6 +379,23 @@ def main():
                 torch.ops.quantized.conv2d_add_relu(xcqs[i % csets], accs[i % csets], pc, 0.05, 0)
         torch.cuda.synchronize()
         print(json.dumps({"only": args.only, "launches": args.steps, "x": [32, 56, 56, 64], "w": [64, 3, 3, 64]}))
+        return
+
+    if args.only in ("conv_first_layer", "conv_depthwise"):
+        # the two convolution lines off the 16-channel grid: 7 x 7 stride 2, 3 -> 64 on [32,3,224,224];
+        # depthwise 3 x 3 over 32 channels on [32,32,112,112]; twelve inputs in turn
+        ic, oc, k, st, pad, groups, hw = (3, 64, 7, 2, 3, 1, 224) if args.only == "conv_first_layer" else (32, 32, 3, 1, 1, 32, 112)
+        xs_ = [torch._make_per_tensor_quantized_tensor(
+            torch.randint(0, 120, (32, hw, hw, ic), dtype=torch.uint8, device=dev).permute(0, 3, 1, 2), 0.03, 0)
+            for _ in range(12)]
+        wf_ = torch.randn(oc, ic // groups, k, k, device=dev) * 0.05
+        wq_ = torch.quantize_per_channel(wf_, (wf_.abs().amax(dim=(1, 2, 3)) / 127.0).to(torch.float64),
+                                         torch.zeros(oc, dtype=torch.int64, device=dev), 0, torch.qint8)
+        pk_ = torch.ops.quantized.conv2d_prepack(wq_, torch.randn(oc, device=dev), [st, st], [pad, pad], [1, 1], groups)
+        for i in range(args.steps):
+            torch.ops.quantized.conv2d_relu(xs_[i % 12], pk_, 0.05, 0)
+        torch.cuda.synchronize()
+        print(json.dumps({"only": args.only, "launches": args.steps, "x": [32, hw, hw, ic], "w": [oc, k, k, ic // groups]}))
         return
 
     # ------------------------------------------------------------------ C3
