@@ -345,6 +345,56 @@ def test_conv_on_patch_rows(cabi, spec, x_signed):
             cabi.force_conv_path(-1)
 
 
+def _random_geometry(rng):
+    """A small convolution drawn so that every kernel family comes up: few channels, narrow groups
+    that merge (or cannot), whole 16-channel blocks, pointwise layers, long K."""
+    kind = rng.integers(0, 6)
+    k = int(rng.choice([1, 2, 3, 3, 5, 7]))
+    s = int(rng.choice([1, 1, 2, 3]))
+    p = int(rng.integers(0, k // 2 + 2))
+    d = int(rng.choice([1, 1, 1, 2]))
+    b = int(rng.integers(1, 4))
+    h, w = int(rng.integers(5, 34)), int(rng.integers(5, 34))
+    groups = 1
+    if kind == 0:      # few input channels
+        ic, oc = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 24, 40])), int(rng.integers(1, 80))
+    elif kind == 1:    # depthwise, with or without a channel multiplier
+        ic = int(rng.choice([16, 32, 40, 48, 96, 144]))
+        groups, oc = ic, ic * int(rng.choice([1, 1, 2]))
+    elif kind == 2:    # narrow groups
+        icg, ocg, groups = int(rng.choice([2, 4, 8, 24])), int(rng.choice([2, 4, 6, 16])), int(rng.choice([2, 4, 8, 16]))
+        ic, oc = icg * groups, ocg * groups
+    elif kind == 3:    # whole 16-channel blocks
+        ic, oc = 16 * int(rng.integers(1, 9)), int(rng.integers(1, 150))
+        groups = int(rng.choice([1, 1, 2])) if ic % 32 == 0 and oc % 2 == 0 else 1
+    elif kind == 4:    # pointwise
+        k, s, p, d = 1, int(rng.choice([1, 1, 2])), 0, 1
+        ic, oc = int(rng.choice([16, 24, 64, 200, 256])), int(rng.integers(1, 300))
+    else:              # long K on a small image
+        k, d = 3, 1
+        ic, oc, h, w = int(rng.choice([256, 512])), int(rng.choice([48, 64, 130])), int(rng.integers(5, 15)), int(rng.integers(5, 15))
+    if (h + 2 * p - d * (k - 1) - 1) // s + 1 <= 0 or (w + 2 * p - d * (k - 1) - 1) // s + 1 <= 0:
+        p = d * (k - 1)
+    return (b, h, w, ic, oc, k, s, p, d, groups)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_conv_random_geometries(cabi, seed):
+    rng = np.random.default_rng(7000 + seed)
+    spec = _random_geometry(rng)
+    say("conv random geometry", seed, spec)
+    c = _conv_case(*spec, seed=seed, x_signed=bool(seed & 1), relu=bool(seed & 2))
+    y, acc, pw = _run(cabi, c)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"], c["groups"], c["x_zp"],
+                                 nthreads=8))
+    np.testing.assert_array_equal(host(pw.colsum), c["wq"].reshape(c["wq"].shape[0], -1).astype(np.int64).sum(1))
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], c["stride"],
+                         c["padding"], c["dilation"], c["groups"], c["out_scale"], c["out_zp"], relu=c["relu"],
+                         nthreads=8)
+    _check(y, want, f"seed {seed} {spec}")
+
+
 def test_conv_byte_runs_limits(cabi):
     """groups, dilation and kernel rows beyond 256 padded bytes are not this kernel's."""
     say("conv byte runs limits")
