@@ -114,6 +114,8 @@ def test_conv_mfma_shapes(cabi, spec, x_signed, path):
     (4, 56, 56, 256, 96, 1, 2, 0, 1, 1),     # 1x1 stride 2: kernel smaller than the stride, implicit GEMM
     (4, 56, 56, 64, 128, 3, 2, 1, 1, 1),     # 3x3 stride 2: halo tiles
     (2, 38, 19, 16, 64, 2, 2, 0, 1, 1),      # 2x2 stride 2: every pixel used once
+    (1, 128, 128, 128, 512, 1, 1, 0, 1, 1),  # pointwise, 16384 pixels, a billion products: as a linear layer
+    (1, 128, 128, 128, 192, 1, 1, 0, 1, 1),  # fewer output channels: halo tiles
 ])
 def test_conv_auto_path_shapes(cabi, spec):
     say("conv auto", spec)
