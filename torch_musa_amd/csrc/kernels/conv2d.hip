@@ -517,6 +517,24 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   return launch_status();
 }
 
+// quantized::linear over `rows` rows of K bytes at `x` (the pixels of a pointwise layer, or patch
+// rows) with the layer's packed weight, which for one group over whole 16-channel blocks is the
+// linear layout: [OC, K] in 16-channel blocks, k = (kh, kw, ic).
+int run_as_linear(const tmq_conv2d_desc* d, int64_t rows, int64_t OC, int64_t K, const void* x, bool relu, void* out,
+                  hipStream_t stream) {
+  tmq_linear_desc l{};
+  l.M = rows; l.N = OC; l.K = K;
+  l.x = x; l.ldx = K;
+  l.x_signed = d->x_signed; l.x_zero_point = d->x_zero_point; l.x_scale = d->x_scale;
+  l.w_packed = d->w_packed; l.w_colsum = d->w_colsum; l.w_scales = d->w_scales;
+  l.w_per_channel = d->w_per_channel;
+  l.relu = relu ? 1 : 0;
+  l.bias = d->bias;
+  l.out_scale = d->out_scale; l.out_zero_point = d->out_zero_point; l.out_signed = d->out_signed;
+  l.y = out; l.ldy = OC;
+  return tmq_linear(&l, reinterpret_cast<tmq_stream_t>(stream));
+}
+
 template <int MODE>
 int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, hipStream_t stream) {
   ConvShape s;
@@ -574,17 +592,7 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
     // 28 x 28 14.3 against 18.0 us)
     const bool wide = s.IC >= 128 && s.OC >= 256 && rows * s.IC * s.OC >= 1000000000;
     if (forced == 5 || (forced < 0 && pointwise && (rows <= kPointwiseAsLinearRows || wide))) {
-      tmq_linear_desc l{};
-      l.M = rows; l.N = s.OC; l.K = s.IC;
-      l.x = d->x; l.ldx = s.IC;
-      l.x_signed = d->x_signed; l.x_zero_point = d->x_zero_point; l.x_scale = d->x_scale;
-      l.w_packed = d->w_packed; l.w_colsum = d->w_colsum; l.w_scales = d->w_scales;
-      l.w_per_channel = d->w_per_channel;
-      l.relu = relu ? 1 : 0;
-      l.bias = d->bias;
-      l.out_scale = d->out_scale; l.out_zero_point = d->out_zero_point; l.out_signed = d->out_signed;
-      l.y = out; l.ldy = s.OC;
-      return tmq_linear(&l, reinterpret_cast<tmq_stream_t>(stream));
+      return run_as_linear(d, rows, s.OC, s.IC, d->x, relu, out, stream);
     }
   }
   // Few output pixels against a long K and a weight slice the halo tiles cannot hold: with a
@@ -605,17 +613,7 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
             static_cast<const uint8_t*>(d->x), s, chunks,
             0x01010101u * static_cast<uint32_t>(static_cast<uint8_t>(d->x_zero_point)), static_cast<uint8_t*>(d->workspace));
         if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
-        tmq_linear_desc l{};
-        l.M = rows; l.N = s.OC; l.K = s.Kp;
-        l.x = d->workspace; l.ldx = s.Kp;
-        l.x_signed = d->x_signed; l.x_zero_point = d->x_zero_point; l.x_scale = d->x_scale;
-        l.w_packed = d->w_packed; l.w_colsum = d->w_colsum; l.w_scales = d->w_scales;
-        l.w_per_channel = d->w_per_channel;
-        l.relu = relu ? 1 : 0;
-        l.bias = d->bias;
-        l.out_scale = d->out_scale; l.out_zero_point = d->out_zero_point; l.out_signed = d->out_signed;
-        l.y = out; l.ldy = s.OC;
-        return tmq_linear(&l, reinterpret_cast<tmq_stream_t>(stream));
+        return run_as_linear(d, rows, s.OC, s.Kp, d->workspace, relu, out, stream);
       }
     }
   }
