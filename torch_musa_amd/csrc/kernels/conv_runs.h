@@ -317,9 +317,12 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
       }
       if constexpr (MODE != kOutAcc32) {
         uint8_t* const dst = static_cast<uint8_t*>(a.y) + off;
+        const v4i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1]), static_cast<int>(packed[2]),
+                         static_cast<int>(packed[3])};
         if (a.vec && cb + 16 <= a.OC) {
-          *reinterpret_cast<v4i*>(dst) = v4i{static_cast<int>(packed[0]), static_cast<int>(packed[1]),
-                                             static_cast<int>(packed[2]), static_cast<int>(packed[3])};
+          *reinterpret_cast<v4i*>(dst) = all;
+        } else if (cb + 16 <= a.OC) {
+          st16_any(dst, all);
         } else {
 #pragma unroll
           for (int c = 0; c < 16; ++c)

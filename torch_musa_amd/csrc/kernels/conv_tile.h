@@ -405,6 +405,8 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
             uint8_t* dst = y + static_cast<int64_t>(op) * a.OC + ch0 + cq * 16;
             if (vec_ok) {
               *reinterpret_cast<v4i*>(dst) = v;
+            } else if (n + 16 <= a.OCg) {
+              st16_any(dst, v);
             } else {
               const uint32_t w[4] = {static_cast<uint32_t>(v.x), static_cast<uint32_t>(v.y),
                                      static_cast<uint32_t>(v.z), static_cast<uint32_t>(v.w)};

@@ -133,6 +133,12 @@ __device__ __forceinline__ void store_f32x4(const GemmArgs& a, int64_t m, int64_
 }
 
 __device__ __forceinline__ v4i ld16(const void* p) { return *reinterpret_cast<const v4i*>(p); }
+// 16 bytes to an address of any alignment (output rows whose channel count is no multiple of 16):
+// still one store instruction, where byte stores would be sixteen.
+struct __attribute__((packed, aligned(1))) V4iAnyAlignment {
+  v4i v;
+};
+__device__ __forceinline__ void st16_any(void* p, v4i v) { reinterpret_cast<V4iAnyAlignment*>(p)->v = v; }
 // Streaming load: data that this CU reads exactly once (packed weight tiles)
 // should not push reusable lines out of the vector L1.
 __device__ __forceinline__ v4i ld16_stream(const void* p) {
@@ -1086,6 +1092,8 @@ void gemm_i8_kernel(GemmArgs a, XSRC xsrc) {
       uint8_t* dst = y + m * a.ldy + n;
       if (vec_ok && n + 16 <= a.N) {
         *reinterpret_cast<v4i*>(dst) = v;
+      } else if (n + 16 <= a.N) {
+        st16_any(dst, v);  // (a row pitch or pointer off the 16-byte grid)
       } else {
         const uint32_t w[4] = {static_cast<uint32_t>(v.x), static_cast<uint32_t>(v.y),
                                static_cast<uint32_t>(v.z), static_cast<uint32_t>(v.w)};

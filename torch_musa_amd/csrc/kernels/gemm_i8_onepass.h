@@ -263,6 +263,8 @@ __global__ __launch_bounds__(256) void gemm_i8_onepass_kernel(GemmArgs a, XLinea
       uint8_t* dst = y + m * a.ldy + n;
       if (vec_ok && n + 16 <= a.N) {
         *reinterpret_cast<v4i*>(dst) = v;
+      } else if (n + 16 <= a.N) {
+        st16_any(dst, v);  // (a row pitch or pointer off the 16-byte grid)
       } else {
         const uint32_t w[4] = {static_cast<uint32_t>(v.x), static_cast<uint32_t>(v.y), static_cast<uint32_t>(v.z),
                                static_cast<uint32_t>(v.w)};
