@@ -236,13 +236,7 @@ __global__ __launch_bounds__(256) void conv_plain_kernel(ConvShape s, PlainArgs 
       const float ad = static_cast<float>(qa - a.post.accum_zp) * a.post.amult;
       ab = ab + ad;
     }
-    if (a.post.silu) {
-      const float rv = ab * a.post.out_scale;
-      const float e = expf(-rv);
-      const float dd = 1.0f + e;
-      const float sl = rv / dd;
-      ab = sl / a.post.out_scale;
-    }
+    if (a.post.silu) ab = silu_in_output_units(ab, a.post.silu_c, a.post.silu_c_tail);
     float r = __builtin_rintf(ab) + a.zp_f;
     r = __builtin_amdgcn_fmed3f(r, a.lo_f, a.hi_f);
     static_cast<uint8_t*>(a.y)[id] = static_cast<uint8_t>(static_cast<int>(r));
@@ -562,6 +556,11 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
     relu = relu || post->activation == 1;
     po.silu = post->activation == 2;
     po.out_scale = d->out_scale;
+    {
+      const double exact = -static_cast<double>(d->out_scale) * 1.4426950408889634074;  // -s log2(e)
+      po.silu_c = static_cast<float>(exact);
+      po.silu_c_tail = static_cast<float>(exact - static_cast<double>(po.silu_c));
+    }
     if (post->accum != nullptr) {
       const int amin = post->accum_signed ? -128 : 0, amax = post->accum_signed ? 127 : 255;
       if (!(post->accum_scale > 0.f) || post->accum_zero_point < amin || post->accum_zero_point > amax)

@@ -425,7 +425,8 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
   // residual rows and the stores of the first tile then run under the k loop of
   // the second, and the two waves of a SIMD drift out of phase (C5 with a residual
   // and ReLU: 14.3 -> 13.5 us per launch; without a residual it changes nothing).
-  while (!kPost && count >= 2) {
+  // (SiLU without a residual has nothing to overlap: two at a time as well)
+  while ((!kPost || (KIND == 3 && a.post.accum == nullptr)) && count >= 2) {
     run(std::integral_constant<int, 2>{}, first);
     first += 2;
     count -= 2;
