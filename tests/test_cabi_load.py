@@ -70,8 +70,11 @@ def test_packed_size_arithmetic():
     g2 = cabi.conv_geom((8, 32, 32, 3), (32, 7, 7), (2, 2), (3, 3), (1, 1), 1)
     assert cabi.conv_out_hw(g2) == (16, 16)
     # few input channels: 49 taps of 16 padded bytes (784 -> 896) for two blocks of 16 channels, then the
-    # per-lane layout of the byte-run kernel: one 64-channel block x 4 channel tiles x 4 k-steps x 1 KB
-    assert lib.tmq_conv2d_packed_bytes(g2) == 2 * 56 * 256 + 4 * 4 * 1024
+    # per-lane layout of the byte-run kernel: one 32-channel block x 2 channel tiles x 4 k-steps x 1 KB
+    assert lib.tmq_conv2d_packed_bytes(g2) == 2 * 56 * 256 + 2 * 4 * 1024
+    # (64 output channels: one block of four tiles)
+    g2b = cabi.conv_geom((8, 32, 32, 3), (64, 7, 7), (2, 2), (3, 3), (1, 1), 1)
+    assert lib.tmq_conv2d_packed_bytes(g2b) == 4 * 56 * 256 + 4 * 4 * 1024
     # kernel rows beyond 256 padded bytes in all (11 rows of 48): no second layout
     g3 = cabi.conv_geom((1, 64, 64, 3), (16, 11, 11), (4, 4), (0, 0), (1, 1), 1)
     assert lib.tmq_conv2d_packed_bytes(g3) == 1 * (121 * 16 + 127) // 128 * 8 * 256

@@ -86,7 +86,8 @@ int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
       s->runs_RL = RL;
       s->runs_RP = RP;
       s->runs_KS = ceil_div(g->KH * RP, 64);
-      s->runs_bytes = ceil_div(g->OC, kCrBN) * 4 * s->runs_KS * kWave * 16;
+      const int64_t tiles = conv_runs_tiles(g->OC);  // 16-channel tiles per block
+      s->runs_bytes = ceil_div(g->OC, 16 * tiles) * tiles * s->runs_KS * kWave * 16;
     }
   }
   // 32-bit index arithmetic inside the kernels
@@ -495,19 +496,25 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   a.out_scale = d->out_scale;
   a.zp_f = zp_f; a.lo_f = lo_f; a.hi_f = hi_f;
   a.post = po;
-  const int64_t by = ceil_div(s.OC, kCrBN);
+  const int nt = conv_runs_tiles(s.OC);
+  const int64_t by = ceil_div(s.OC, 16 * nt);
   if (by > 65535) return TMQ_ERR_UNSUPPORTED;
   // three blocks per CU (their registers), each with its weights in registers for every tile it walks
   const int64_t bx = a.tiles < 768 ? a.tiles : 768;  // (plan_runs: kSlots)
   const dim3 grid(static_cast<unsigned>(bx), static_cast<unsigned>(by)), block(kCrThreads);
-  if constexpr (MODE == kOutAcc32) {
-    conv_runs_kernel<MODE, false><<<grid, block, p.lds, stream>>>(a);
-  } else {
-    if (po.any())
-      conv_runs_kernel<MODE, true><<<grid, block, p.lds, stream>>>(a);
-    else
-      conv_runs_kernel<MODE, false><<<grid, block, p.lds, stream>>>(a);
-  }
+  const auto launch = [&](auto post_tag, auto nt_tag) {
+    conv_runs_kernel<MODE, decltype(post_tag)::value, decltype(nt_tag)::value><<<grid, block, p.lds, stream>>>(a);
+  };
+  const auto launch_tiles = [&](auto nt_tag) {
+    if constexpr (MODE != kOutAcc32) {
+      if (po.any()) return launch(std::true_type{}, nt_tag);
+    }
+    launch(std::false_type{}, nt_tag);
+  };
+  if (nt == 2)
+    launch_tiles(std::integral_constant<int, 2>{});
+  else
+    launch_tiles(std::integral_constant<int, 4>{});
   return launch_status();
 }
 

@@ -7,7 +7,7 @@
 // image row, so k is ordered (kh, run) with run = the RL = KW * IC bytes of a kernel
 // row, padded to RP = a multiple of 16 with zero weights: the bytes an operand picks
 // up past the run's end are multiplied by zero.  K = KH * RP is at most 256 here, the
-// weights of 64 output channels stay in registers (16 operands of
+// weights of 64 (32) output channels stay in registers (16 operands of
 // v_mfma_i32_16x16x64_i8) for the whole launch; prepack lays them out per lane
 // (conv_runs_slot) behind the packed weight of the other kernels.
 //
@@ -23,8 +23,9 @@
 //     words with v_alignbyte_b32;
 //   * operand roles: weights are the rows (i), pixels the columns (j) of the MFMA,
 //     D[i][j]: lane l, register r -> i = 4 (l / 16) + r, j = l % 16.  Row i of channel
-//     tile nt is channel 16 (i / 4) + 4 nt + i % 4, so that a lane ends up with 16
-//     consecutive channels of one pixel: one 16-byte store.
+//     tile nt (of NT = 4, or 2 for at most 32 output channels) is channel
+//     4 NT (i / 4) + 4 nt + i % 4, so that a lane ends up with 4 NT consecutive channels of
+//     one pixel: one 16-byte (8-byte) store.
 // The x ^ 0x80 trick, the accumulator start value and the requantisation are those of
 // gemm_i8_core.h.
 #pragma once
@@ -35,13 +36,12 @@ namespace tmq {
 
 constexpr int kCrThreads = 256;
 constexpr int kCrWaves = kCrThreads / kWave;
-constexpr int kCrBN = 64;      // output channels per block (grid y)
 constexpr int kCrMaxKS = 4;    // k-steps of 64 bytes
 constexpr int kCrUnits = 4;    // 1 KB units of staged image rows per wave and tile: 16 KB per block
 
 struct ConvRunArgs {
   const uint8_t* x;          // NHWC
-  const uint8_t* w_runs;     // [64-channel block][channel tile nt][k-step][lane][16 B]: conv_runs_slot below
+  const uint8_t* w_runs;     // [channel block of 16 NT][channel tile nt][k-step][lane][16 B]: conv_runs_slot below
   const int32_t* colsum;
   const float* w_scales;
   const float* bias;
@@ -62,19 +62,23 @@ struct ConvRunArgs {
 };
 
 // One 16-byte slot of the per-lane weight layout: slot index ->
-// (64-channel block cb, channel tile nt, k-step ks, lane).  The lane's row i = lane % 16 of
-// tile nt is channel 64 cb + 16 (i / 4) + 4 nt + i % 4; its bytes are k = 64 ks + 16 (lane / 16)
-// ... + 15 in (kh, run) order: kernel row kh = k / RP, byte k % RP of the run, which in OHWI
-// weights is byte (kw, ic) = k % RP of the contiguous row w[n][kh][.][.]; zeros past the
-// run's RL bytes, past the last kernel row and for channels that do not exist.
+// (channel block cb of 16 NT channels, channel tile nt, k-step ks, lane).  NT = 4 tiles per block,
+// 2 for layers of at most 32 output channels.  The lane's row i = lane % 16 of tile nt is channel
+// 16 NT cb + 4 NT (i / 4) + 4 nt + i % 4 (a lane of the kernel then holds 4 NT consecutive
+// channels); its bytes are k = 64 ks + 16 (lane / 16) ... + 15 in (kh, run) order: kernel row
+// kh = k / RP, byte k % RP of the run, which in OHWI weights is byte (kw, ic) = k % RP of the
+// contiguous row w[n][kh][.][.]; zeros past the run's RL bytes, past the last kernel row and for
+// channels that do not exist.
+__host__ __device__ inline int conv_runs_tiles(int64_t OC) { return OC <= 32 ? 2 : 4; }
 __device__ __forceinline__ v4i conv_runs_slot(const int8_t* __restrict__ w, int64_t slot, int OC, int KH, int RL,
                                               int RP, int KS) {
+  const int NT = conv_runs_tiles(OC);
   const int lane = static_cast<int>(slot & 63);
   const int64_t op = slot >> 6;
-  const int ks = static_cast<int>(op % KS), nt = static_cast<int>((op / KS) & 3);
-  const int64_t cb = op / (4 * KS);
+  const int ks = static_cast<int>(op % KS), nt = static_cast<int>((op / KS) % NT);
+  const int64_t cb = op / (NT * KS);
   const int i = lane & 15;
-  const int64_t n = cb * 64 + 16 * (i >> 2) + 4 * nt + (i & 3);
+  const int64_t n = cb * 16 * NT + 4 * NT * (i >> 2) + 4 * nt + (i & 3);
   const int k = 64 * ks + 16 * (lane >> 4);
   const int kh = k / RP, ro = k - kh * RP;
   uint32_t words[4] = {0, 0, 0, 0};
@@ -87,8 +91,10 @@ __device__ __forceinline__ v4i conv_runs_slot(const int8_t* __restrict__ w, int6
              static_cast<int>(words[3])};
 }
 
-template <int MODE, bool POST>
+template <int MODE, bool POST, int NT>
 __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a) {
+  constexpr int kCrBN = 16 * NT;  // output channels per block (grid y)
+  constexpr int kLaneCh = 4 * NT; // consecutive channels of one pixel in a lane
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ __attribute__((aligned(16))) int s_acc0[kCrBN];
   __shared__ __attribute__((aligned(16))) float s_mult[kCrBN];
@@ -118,11 +124,11 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
     s_bdiv[t] = bdiv;
   }
   // the weight operands of this block's 64 channels, laid out per lane at prepack
-  v4i wreg[4][kCrMaxKS];
+  v4i wreg[NT][kCrMaxKS];
   {
-    const uint8_t* const wsrc = a.w_runs + (static_cast<int64_t>(blockIdx.y) * 4 * KS * kWave + lane) * 16;
+    const uint8_t* const wsrc = a.w_runs + (static_cast<int64_t>(blockIdx.y) * NT * KS * kWave + lane) * 16;
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int ks = 0; ks < kCrMaxKS; ++ks)
         wreg[nt][ks] = ks < KS ? ld16(wsrc + (nt * KS + ks) * (kWave * 16)) : v4i{0, 0, 0, 0};
@@ -262,9 +268,9 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
       const int pc = pcol < tw_valid ? pcol : tw_valid - 1;
       const int base = orow * a.sh * a.pitch + pc * a.sw * a.IC;
       const int c0r = c0 + orow * a.sh * rb15;  // alignment shift of staged row orow * stride, before the % 16
-      v4i acc[4];  // start: the zero point's share, acc_coef * colsum
+      v4i acc[NT];  // start: the zero point's share, acc_coef * colsum
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) acc[nt] = *reinterpret_cast<const v4i*>(&s_acc0[16 * pq + 4 * nt]);
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = *reinterpret_cast<const v4i*>(&s_acc0[kLaneCh * pq + 4 * nt]);
 #pragma unroll
       for (int ks = 0; ks < kCrMaxKS; ++ks) {
         if (ks < KS) {
@@ -277,20 +283,20 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
                           static_cast<int>(__builtin_amdgcn_alignbyte(d3, d2, sb)),
                           static_cast<int>(__builtin_amdgcn_alignbyte(d4, d3, sb))};
 #pragma unroll
-          for (int nt = 0; nt < 4; ++nt)
+          for (int nt = 0; nt < NT; ++nt)
             acc[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wreg[nt][ks], xv, acc[nt], 0, 0, 0);
         }
       }
-      // ---- requantise and store: this lane has channels n0 + 16 pq .. + 15 of pixel pj
+      // ---- requantise and store: this lane has channels n0 + 4 NT pq .. + 4 NT - 1 of pixel pj
       if (pcol >= tw_valid) continue;
       const int64_t opix = (static_cast<int64_t>(b) * a.OH + oh0 + orow) * a.OW + ow0 + pcol;
-      const int cb = n0 + 16 * pq;
+      const int cb = n0 + kLaneCh * pq;
       if (cb >= a.OC) continue;
       const int64_t off = opix * a.OC + cb;
-      uint32_t packed[4];
+      uint32_t packed[NT];
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const int cl = 16 * pq + 4 * nt;
+      for (int nt = 0; nt < NT; ++nt) {
+        const int cl = kLaneCh * pq + 4 * nt;
         const int raw[4] = {acc[nt][0], acc[nt][1], acc[nt][2], acc[nt][3]};
         if constexpr (MODE == kOutAcc32) {
           int32_t* const dst = static_cast<int32_t*>(a.y) + off + 4 * nt;
@@ -317,15 +323,24 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
       }
       if constexpr (MODE != kOutAcc32) {
         uint8_t* const dst = static_cast<uint8_t*>(a.y) + off;
-        const v4i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1]), static_cast<int>(packed[2]),
-                         static_cast<int>(packed[3])};
-        if (a.vec && cb + 16 <= a.OC) {
-          *reinterpret_cast<v4i*>(dst) = all;
-        } else if (cb + 16 <= a.OC) {
-          st16_any(dst, all);
+        if (cb + kLaneCh <= a.OC) {  // one store of 4 NT bytes; any alignment unless the host found the rows aligned
+          if constexpr (NT == 4) {
+            const v4i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1]), static_cast<int>(packed[2]),
+                             static_cast<int>(packed[3])};
+            if (a.vec)
+              *reinterpret_cast<v4i*>(dst) = all;
+            else
+              st16_any(dst, all);
+          } else {
+            const v2i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1])};
+            if (a.vec)
+              *reinterpret_cast<v2i*>(dst) = all;
+            else
+              st8_any(dst, all);
+          }
         } else {
 #pragma unroll
-          for (int c = 0; c < 16; ++c)
+          for (int c = 0; c < kLaneCh; ++c)
             if (cb + c < a.OC) dst[c] = static_cast<uint8_t>(packed[c >> 2] >> (8 * (c & 3)));
         }
       }

@@ -160,6 +160,11 @@ struct __attribute__((packed, aligned(1))) V4iAnyAlignment {
   v4i v;
 };
 __device__ __forceinline__ void st16_any(void* p, v4i v) { reinterpret_cast<V4iAnyAlignment*>(p)->v = v; }
+typedef int v2i __attribute__((ext_vector_type(2)));
+struct __attribute__((packed, aligned(1))) V2iAnyAlignment {
+  v2i v;
+};
+__device__ __forceinline__ void st8_any(void* p, v2i v) { reinterpret_cast<V2iAnyAlignment*>(p)->v = v; }
 // Streaming load: data that this CU reads exactly once (packed weight tiles)
 // should not push reusable lines out of the vector L1.
 __device__ __forceinline__ v4i ld16_stream(const void* p) {
