@@ -1161,7 +1161,7 @@ def main():
         # ------------------------- convolutions off the 16-channel grid: an image network's first
         # layer (3 -> 64 channels, 7 x 7, stride 2, 224 x 224) and a depthwise layer (32 channels,
         # 3 x 3, 112 x 112), batch 32, through torch.ops.quantized.conv2d_relu
-        def conv_line(name, ic, oc, k, stride, pad, groups, hw, what):
+        def conv_line(name, ic, oc, k, stride, pad, groups, hw, what, op="conv2d_relu", batch=32):
             wf_ = torch.randn(oc, ic // groups, k, k) * 0.05
             wq_ = torch.quantize_per_channel(wf_, wf_.abs().amax(dim=(1, 2, 3)) / 127, torch.zeros(oc, dtype=torch.long),
                                              0, torch.qint8).to(dev)
@@ -1170,14 +1170,14 @@ def main():
             nsets = 6
             xqs_ = []
             for _ in range(nsets):
-                xf_ = torch.relu(torch.randn(32, ic, hw, hw, device=dev)).contiguous(memory_format=torch.channels_last)
+                xf_ = torch.relu(torch.randn(batch, ic, hw, hw, device=dev)).contiguous(memory_format=torch.channels_last)
                 xqs_.append(torch.quantize_per_tensor(xf_, 0.03, 0, torch.quint8))
                 del xf_
             cnt = [0]
 
             def one():
                 cnt[0] += 1
-                return torch.ops.quantized.conv2d_relu(xqs_[cnt[0] % nsets], packed_, 0.05, 0)
+                return getattr(torch.ops.quantized, op)(xqs_[cnt[0] % nsets], packed_, 0.05, 0)
 
             for _ in range(3):
                 y_ = one()
@@ -1194,8 +1194,8 @@ def main():
                 g_.replay()
             ts_ = events_ms(g_.replay, 10)
             avg_ = sum(ts_) / len(ts_) / (2 * nsets)
-            nbytes_ = 32 * hw * hw * ic + 32 * oh_ * oh_ * oc + oc * (ic // groups) * k * k
-            ops_ = 2 * 32 * oh_ * oh_ * oc * (ic // groups) * k * k
+            nbytes_ = batch * hw * hw * ic + batch * oh_ * oh_ * oc + oc * (ic // groups) * k * k
+            ops_ = 2 * batch * oh_ * oh_ * oc * (ic // groups) * k * k
             log(f"[bench] {what}: {avg_*1e3:.1f} us/launch in a replayed graph, {nbytes_/(avg_*1e-3)/1e9:.0f} GB/s, "
                 f"{ops_/(avg_*1e-3)/1e12:.1f} TOP/s")
             secondary[name] = {
@@ -1253,6 +1253,9 @@ def main():
                   "conv2d_relu 7x7 stride 2, 3 -> 64 channels, [32,3,224,224]")
         conv_line("conv2d_relu_depthwise_3x3_32ch", 32, 32, 3, 1, 1, 32, 112,
                   "conv2d_relu depthwise 3x3, 32 channels, [32,32,112,112]")
+        # the fused SiLU form the reference adds for detectors: 32 -> 64 channels, 3 x 3 stride 2 on 320 x 320, batch 8
+        conv_line("conv2d_silu_3x3_s2_32to64_320", 32, 64, 3, 2, 1, 1, 320,
+                  "conv2d_silu 3x3 stride 2, 32 -> 64 channels, [8,32,320,320]", op="conv2d_silu", batch=8)
 
     # ------------------------------------------------------------ CPU baseline
     # The reference CPU path = PyTorch's own quantized CPU ops (fbgemm engine), timed on
