@@ -362,8 +362,8 @@ typedef struct tmq_conv2d_desc {
   /* 0: the library chooses.  Otherwise, for tests of every kernel family at any
    * shape: 1 halo tiles, 2 implicit GEMM, 3 direct, 4 kernel rows as byte runs
    * (few input channels), 5 a pointwise layer as tmq_linear, 6 patch rows in the
-   * workspace, then tmq_linear (TMQ_ERR_UNSUPPORTED when the family cannot run
-   * the problem).  tile_rows / tile_cols > 0 pin the halo
+   * workspace, then tmq_linear, 7 a depthwise layer four channels per lane on the
+   * vector ALU (TMQ_ERR_UNSUPPORTED when the family cannot run the problem).  tile_rows / tile_cols > 0 pin the halo
    * kernel's patch height / bound its patch width. */
   int32_t kernel;
   int32_t tile_rows, tile_cols;

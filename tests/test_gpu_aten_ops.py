@@ -240,10 +240,13 @@ CONV_CONFIGS = [
     dict(shape=(2, 64, 16, 16), oc=32, k=3, s=2, p=1, d=1, g=32, bias=False, relu=True),
     dict(shape=(8, 3, 32, 32), oc=32, k=7, s=2, p=3, d=1, g=1, bias=True, relu=False),
     dict(shape=(4, 64, 28, 28), oc=64, k=3, s=1, p=1, d=1, g=1, bias=True, relu=False),
-    # the layers of a mobile network: depthwise (merged groups), pointwise off the 16-channel grid (byte runs),
-    # pointwise over few pixels (as a linear layer); and a long K on one small image (patch rows in a workspace)
+    # the layers of a mobile network: depthwise (four channels per lane; 5 x 5 at stride 2 on 144 channels: merged
+    # groups on the matrix pipe), pointwise off the 16-channel grid (byte runs), pointwise over few pixels (as a
+    # linear layer); and a long K on one small image (patch rows in a workspace)
     dict(shape=(2, 32, 20, 20), oc=32, k=3, s=1, p=1, d=1, g=32, bias=True, relu=True),
     dict(shape=(1, 144, 14, 14), oc=144, k=3, s=2, p=1, d=1, g=144, bias=False, relu=False),
+    dict(shape=(2, 72, 15, 15), oc=72, k=5, s=1, p=2, d=1, g=72, bias=True, relu=True),
+    dict(shape=(1, 144, 14, 14), oc=144, k=5, s=2, p=2, d=1, g=144, bias=True, relu=False),
     dict(shape=(2, 24, 14, 14), oc=144, k=1, s=1, p=0, d=1, g=1, bias=True, relu=False),
     dict(shape=(2, 256, 6, 6), oc=48, k=1, s=1, p=0, d=1, g=1, bias=True, relu=True),
     dict(shape=(1, 256, 7, 7), oc=64, k=3, s=1, p=1, d=1, g=1, bias=True, relu=False),

@@ -201,6 +201,89 @@ def test_conv_narrow_groups_merged(cabi, spec, x_signed):
 
 
 @pytest.mark.parametrize("spec", [
+    (2, 19, 23, 72, 72, 3, 1, 1, 1, 72),     # 72 channels: no whole 16-channel blocks to merge into
+    (1, 9, 9, 40, 40, 3, 2, 1, 1, 40),       # stride 2
+    (3, 17, 13, 24, 24, 5, 1, 2, 1, 24),     # 5 x 5: whole weight dwords in registers
+    (2, 21, 21, 120, 120, 5, 2, 2, 1, 120),
+    (1, 15, 15, 12, 12, 7, 1, 3, 1, 12),     # any other kernel size: weights read at use
+    (2, 11, 14, 20, 20, 3, 1, 2, 2, 20),     # dilation
+    (1, 6, 6, 4, 4, 3, 1, 0, 1, 4),          # one lane per pixel, no padding
+    (2, 3, 40, 36, 36, 3, 1, 1, 1, 36),      # fewer output rows than a strip
+    (2, 30, 30, 96, 96, 3, 2, 1, 1, 96),     # channels that would also merge
+    (1, 12, 12, 8, 8, (1, 3), 1, 0, 1, 8),   # a kernel that is not square
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_depthwise_on_the_vector_alu(cabi, spec, x_signed):
+    """Depthwise layers, four channels per lane: every strip length against the oracle, with
+    the integer sums, plain and fused requantisation."""
+    say("conv depthwise lanes", spec, x_signed)
+    b, h, w, ic, oc, k, st, p, dl, g = spec
+    kh, kw = (k, k) if isinstance(k, int) else k
+    c = _conv_case(b, h, w, ic, oc, kh, st, p, dl, g, seed=sum(spec[:5]) + 17, x_signed=x_signed, relu=x_signed)
+    if kh != kw:
+        rng = np.random.default_rng(5)
+        c["wq"] = rng.integers(-127, 128, (oc, kh, kw, 1), dtype=np.int8)
+    want_acc = oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                   c["groups"], c["x_zp"], nthreads=8)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    for strip in (0, 1, 3, 8):
+        cabi.force_conv_path(7)
+        cabi.force_conv_tile(strip, 0)
+        try:
+            y, acc, pw = _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+            cabi.force_conv_tile(0, 0)
+        np.testing.assert_array_equal(acc, want_acc)
+        _check(y, want, f"strip {strip}")
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(acc, want_acc)
+    _check(y, want, "automatic")
+    # fused: residual + ReLU into a signed output, and SiLU
+    rng = np.random.default_rng(sum(spec[:5]))
+    for activation, signed in (("relu", True), ("silu", False)):
+        f = dict(c, accq=(rng.integers(-128, 128, want.shape, dtype=np.int8) if activation == "relu" else None),
+                 acc_scale=0.35, acc_zp=-7, activation=activation, signed=signed, relu=False,
+                 out_zp=-20 if signed else 30)
+        want_f = oracle.conv2d_fused(f["xq"], f["x_scale"], f["x_zp"], f["wq"], f["w_scales"], f["bias"],
+                                     f["stride"], f["padding"], f["dilation"], f["groups"], f["out_scale"],
+                                     f["out_zp"], accum=f["accq"], accum_scale=f["acc_scale"],
+                                     accum_zp=f["acc_zp"], activation=activation, out_signed=signed, nthreads=8)
+        cabi.force_conv_path(7)
+        try:
+            yf = _run_fused(cabi, f)
+        finally:
+            cabi.force_conv_path(-1)
+        d = np.abs(yf.astype(np.int32) - want_f.astype(np.int32))
+        if activation == "silu":
+            assert d.max() <= LSB_TOL and np.count_nonzero(d) <= max(2, 0.001 * d.size), (d.max(), np.count_nonzero(d))
+        else:
+            assert d.max() == 0, f"{np.count_nonzero(d)} of {d.size} bytes differ (max {d.max()})"
+
+
+def test_conv_depthwise_lanes_limits(cabi):
+    """What the four-channels-per-lane kernel refuses: groups that are not single channels, channel
+    counts off the dword grid, more output channels than input channels."""
+    say("conv depthwise lanes limits")
+    for spec in [(1, 8, 8, 32, 32, 3, 1, 1, 1, 1), (1, 8, 8, 32, 32, 3, 1, 1, 1, 16), (1, 8, 8, 10, 10, 3, 1, 1, 1, 10),
+                 (1, 8, 8, 8, 16, 3, 1, 1, 1, 8)]:
+        c = _conv_case(*spec, seed=3)
+        cabi.force_conv_path(7)
+        try:
+            with pytest.raises(cabi.TmqError):
+                _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+        y, _, _ = _run(cabi, c)   # ... and the automatic choice still serves
+        want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                             c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                             c["out_zp"], relu=c["relu"], nthreads=8)
+        _check(y, want, "automatic")
+
+
+@pytest.mark.parametrize("spec", [
     (2, 14, 14, 256, 64, 1, 1, 0, 1, 1),
     (32, 7, 7, 512, 200, 1, 1, 0, 1, 1),     # 1568 pixels, channels off the 16 grid on the output side
     (1, 5, 5, 16, 24, 1, 1, 0, 1, 1),

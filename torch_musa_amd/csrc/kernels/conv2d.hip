@@ -10,6 +10,7 @@
 #include <type_traits>
 
 #include "conv_runs.h"
+#include "conv_depthwise.h"
 #include "conv_tile.h"
 #include "gemm_i8_core.h"
 
@@ -36,6 +37,9 @@ struct ConvShape {
   // the second weight layout, behind the first, for the kernel of conv_runs.h: k-steps
   // (0: the shape is not that kernel's), run bytes, padded run bytes, offset and size in bytes
   int64_t runs_KS, runs_RL, runs_RP, runs_off, runs_bytes;
+  // depthwise layers over a multiple of 4 channels: a [tap][channel] copy of the weight for the
+  // kernel of conv_depthwise.h in the same place (0: not such a layer)
+  int64_t taps_bytes;
 };
 
 int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
@@ -90,6 +94,9 @@ int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
       s->runs_bytes = ceil_div(g->OC, 16 * tiles) * tiles * s->runs_KS * kWave * 16;
     }
   }
+  s->taps_bytes = 0;
+  if (g->groups > 1 && g->groups == g->IC && g->IC == g->OC && g->IC % 4 == 0)
+    s->taps_bytes = round_up(g->KH * g->KW * g->IC, 16);
   // 32-bit index arithmetic inside the kernels
   if (g->H > (1 << 24) || g->W > (1 << 24) || g->IC > (1 << 24) || s->Kp > (1 << 30) ||
       g->B * s->OH * s->OW > 0x7fffffff || g->H * g->W * g->IC > 0x3fffffff)
@@ -132,6 +139,15 @@ __global__ __launch_bounds__(256) void conv_prepack_runs_kernel(const int8_t* __
   *reinterpret_cast<v4i*>(dst + id * 16) =
       conv_runs_slot(w, id, static_cast<int>(s.OC), static_cast<int>(s.KH), static_cast<int>(s.runs_RL),
                      static_cast<int>(s.runs_RP), static_cast<int>(s.runs_KS));
+}
+
+// One thread per byte of the [tap][channel] layout of conv_depthwise.h (the caller's weight is [channel][tap]).
+__global__ __launch_bounds__(256) void conv_prepack_taps_kernel(const int8_t* __restrict__ w, int64_t C, int64_t taps,
+                                                                int64_t total, uint8_t* __restrict__ dst) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const int64_t tp = id / C, c = id % C;
+  dst[id] = tp < taps ? static_cast<uint8_t>(w[c * taps + tp]) : uint8_t{0};
 }
 
 __global__ __launch_bounds__(256) void conv_colsum_kernel(const int8_t* __restrict__ w, int64_t OC,
@@ -518,6 +534,65 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   return launch_status();
 }
 
+// Depthwise layers on the vector ALU (conv_depthwise.h).
+template <int MODE>
+int launch_conv_depthwise(const tmq_conv2d_desc* d, const ConvShape& s, const PostOps& po, float zp_f, float lo_f,
+                          float hi_f, void* out, hipStream_t stream) {
+  DepthwiseArgs a{};
+  a.x = static_cast<const uint8_t*>(d->x);
+  a.w_taps = static_cast<const uint8_t*>(d->w_packed) + s.runs_off;
+  a.colsum = d->w_colsum;
+  a.w_scales = d->w_scales;
+  a.bias = d->bias;
+  a.y = out;
+  a.B = static_cast<int>(s.B);
+  a.H = static_cast<int>(s.H); a.W = static_cast<int>(s.W); a.C = static_cast<int>(s.IC);
+  a.OH = static_cast<int>(s.OH); a.OW = static_cast<int>(s.OW);
+  a.KH = static_cast<int>(s.KH); a.KW = static_cast<int>(s.KW);
+  a.sh = static_cast<int>(s.sh); a.sw = static_cast<int>(s.sw);
+  a.ph = static_cast<int>(s.ph); a.pw = static_cast<int>(s.pw);
+  a.dh = static_cast<int>(s.dh); a.dw = static_cast<int>(s.dw);
+  // Output rows per lane: long strips amortise the lane's weights and constants, short ones put
+  // more waves in flight; the longest with a wave per SIMD.
+  int64_t strip = d->kernel == 7 && d->tile_rows > 0 ? d->tile_rows : kDwStripMax;
+  if (!(d->kernel == 7 && d->tile_rows > 0))
+    while (strip > 1 && s.B * ceil_div(s.OH, strip) * s.OW * (s.IC / 4) < (int64_t{1} << 16)) strip /= 2;
+  if (strip > s.OH) strip = s.OH;
+  a.strip = static_cast<int>(strip);
+  const int64_t per_image = ceil_div(s.OH, strip) * s.OW * (s.IC / 4);
+  const int64_t blocks_per_image = ceil_div(per_image, kDwThreads);
+  a.per_image = static_cast<uint32_t>(per_image);
+  a.blocks_per_image = static_cast<uint32_t>(blocks_per_image);
+  a.w_scale_stride = d->w_per_channel ? 1 : 0;
+  a.x_xor = d->x_signed ? 0u : 0x80808080u;
+  a.pad_word = 0x01010101u * static_cast<uint32_t>(static_cast<uint8_t>(d->x_zero_point));
+  a.acc_coef = (d->x_signed ? 0 : 128) - d->x_zero_point;
+  a.x_scale = d->x_scale;
+  a.out_scale = d->out_scale;
+  a.zp_f = zp_f; a.lo_f = lo_f; a.hi_f = hi_f;
+  a.post = po;
+  const int64_t blocks = s.B * blocks_per_image;
+  if (blocks > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kDwThreads);
+  const auto launch = [&](auto post_tag) {
+    constexpr bool kP = decltype(post_tag)::value;
+    if (s.KH == 3 && s.KW == 3)
+      conv_depthwise_kernel<MODE, kP, 9><<<grid, block, 0, stream>>>(a);
+    else if (s.KH == 5 && s.KW == 5)
+      conv_depthwise_kernel<MODE, kP, 25><<<grid, block, 0, stream>>>(a);
+    else
+      conv_depthwise_kernel<MODE, kP, 0><<<grid, block, 0, stream>>>(a);
+  };
+  if constexpr (MODE != kOutAcc32) {
+    if (po.any()) {
+      launch(std::true_type{});
+      return launch_status();
+    }
+  }
+  launch(std::false_type{});
+  return launch_status();
+}
+
 // quantized::linear over `rows` rows of K bytes at `x` (the pixels of a pointwise layer, or patch
 // rows) with the layer's packed weight, which for one group over whole 16-channel blocks is the
 // linear layout: [OC, K] in 16-channel blocks, k = (kh, kw, ic).
@@ -625,6 +700,21 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   }
   const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
   if ((forced == 1 || forced == 2) && !mfma_ok) return TMQ_ERR_UNSUPPORTED;
+  // depthwise layers: four channels per lane on the vector ALU
+  {
+    // (32-bit byte offsets into the input and the output)
+    const bool lanes_ok = s.taps_bytes > 0 && s.B * s.H * s.W * s.IC < (int64_t{1} << 31) &&
+                          s.B * s.OH * s.OW * s.OC < (int64_t{1} << (MODE == kOutAcc32 ? 29 : 31)) && aligned(d->x, 4) && aligned(out, MODE == kOutAcc32 ? 16 : 4) &&
+                          (po.accum == nullptr || aligned(po.accum, 4));
+    if (forced == 7 && !lanes_ok) return TMQ_ERR_UNSUPPORTED;
+    // Also where the groups would merge into 16-channel blocks for the matrix pipe, for 3 x 3 kernels and for
+    // 5 x 5 at stride 1 (batch 32, against the merged groups on the halo tiles: 32 channels on 112 x 112 14.7
+    // against 17.3 us; 96 channels, 112 x 112 -> 56 x 56: 13.6 against 26.0 us; 960 channels on 7 x 7: 4.6 against
+    // 5.8 us; 384 on 14 x 14 level at 6 us); other kernel sizes stay with the matrix pipe where they can.
+    const bool lanes_first = (s.KH == 3 && s.KW == 3) || (s.KH == 5 && s.KW == 5 && s.sh == 1 && s.dh == 1);
+    if (forced == 7 || (forced < 0 && lanes_ok && (!mfma_ok || lanes_first)))
+      return launch_conv_depthwise<MODE>(d, s, po, zp_f, lo_f, hi_f, out, stream);
+  }
   // channel counts (or an address) the 16-byte chunks of the kernels below cannot take:
   // kernel rows as runs of bytes where they are short enough
   if (forced == 4 || (forced < 0 && !mfma_ok)) {
@@ -774,7 +864,7 @@ using namespace tmq;
 TMQ_EXPORT int64_t tmq_conv2d_packed_bytes(const tmq_conv2d_geom* g) {
   ConvShape s;
   if (make_shape(g, &s) != TMQ_OK) return 0;
-  return s.groups * s.group_bytes + s.runs_bytes;
+  return s.groups * s.group_bytes + s.runs_bytes + s.taps_bytes;
 }
 
 TMQ_EXPORT int64_t tmq_conv2d_workspace_bytes(const tmq_conv2d_geom* g) {
@@ -812,6 +902,11 @@ TMQ_EXPORT int tmq_conv2d_prepack(const int8_t* w_ohwi, const tmq_conv2d_geom* g
     const int64_t slots = s.runs_bytes / 16;
     conv_prepack_runs_kernel<<<dim3(static_cast<unsigned>(ceil_div(slots, 256))), dim3(256), 0, hs>>>(
         w_ohwi, s, slots, static_cast<uint8_t*>(packed) + s.runs_off);
+    if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+  }
+  if (s.taps_bytes > 0) {
+    conv_prepack_taps_kernel<<<dim3(static_cast<unsigned>(ceil_div(s.taps_bytes, 256))), dim3(256), 0, hs>>>(
+        w_ohwi, s.IC, s.KH * s.KW, s.taps_bytes, static_cast<uint8_t*>(packed) + s.runs_off);
     if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
   }
   blocks = ceil_div(s.OC, 256 / kWave);
