@@ -363,7 +363,9 @@ typedef struct tmq_conv2d_desc {
    * shape: 1 halo tiles, 2 implicit GEMM, 3 direct, 4 kernel rows as byte runs
    * (few input channels), 5 a pointwise layer as tmq_linear, 6 patch rows in the
    * workspace, then tmq_linear, 7 a depthwise layer four channels per lane on the
-   * vector ALU (TMQ_ERR_UNSUPPORTED when the family cannot run the problem).  tile_rows / tile_cols > 0 pin the halo
+   * vector ALU, 8 the input copied into the workspace with its channels padded
+   * to a multiple of 16, then whatever the library chooses for that
+   * (TMQ_ERR_UNSUPPORTED when the family cannot run the problem).  tile_rows / tile_cols > 0 pin the halo
    * kernel's patch height / bound its patch width. */
   int32_t kernel;
   int32_t tile_rows, tile_cols;
@@ -373,7 +375,11 @@ typedef struct tmq_conv2d_desc {
    * least tmq_conv2d_workspace_bytes(&geom) bytes, layers with few output pixels
    * against a long K (3 x 3 over hundreds of channels on a 14 x 14 or 7 x 7
    * image) write their patch rows there and run as one quantized::linear over
-   * them.  NULL / too small: the single-launch kernels, same results. */
+   * them, and layers of one group whose channel count is no multiple of 16
+   * under kernel rows of more than 256 bytes (3 x 3 over 40 channels) run the
+   * matrix-core kernels on a copy of the input with padded channels instead of
+   * the slow direct kernel.  NULL / too small: the single-launch kernels, same
+   * results. */
   void* workspace;
   int64_t workspace_bytes;
 } tmq_conv2d_desc;

@@ -96,6 +96,11 @@ def test_packed_size_arithmetic():
     assert wsb(cabi.conv_geom((8, 14, 14, 256), (256, 3, 3), (1, 1), (1, 1), (1, 1), 1)) == 0    # 1568 pixels
     assert wsb(g) == 0 and wsb(g2) == 0 and wsb(g4) == 0                                       # C5, few channels, depthwise
     assert wsb(cabi.conv_geom((1, 14, 14, 2048), (512, 1, 1), (1, 1), (0, 0), (1, 1), 1)) == 0    # pointwise: rows already
+    # ... and for one group off the 16-channel grid under kernel rows too long for the byte-run kernel:
+    # the input once more with 48 channels per pixel
+    assert wsb(cabi.conv_geom((2, 20, 20, 40), (40, 3, 3), (1, 1), (1, 1), (1, 1), 1)) == 2 * 400 * 48
+    assert wsb(cabi.conv_geom((2, 20, 20, 24), (40, 3, 3), (1, 1), (1, 1), (1, 1), 1)) == 0      # 3 rows of 80 bytes: byte runs
+    assert wsb(cabi.conv_geom((2, 20, 20, 40), (40, 3, 3), (1, 1), (1, 1), (1, 1), 2)) == 0      # groups
 
 
 def test_split_k_workspace_arithmetic():

@@ -250,6 +250,8 @@ CONV_CONFIGS = [
     dict(shape=(2, 24, 14, 14), oc=144, k=1, s=1, p=0, d=1, g=1, bias=True, relu=False),
     dict(shape=(2, 256, 6, 6), oc=48, k=1, s=1, p=0, d=1, g=1, bias=True, relu=True),
     dict(shape=(1, 256, 7, 7), oc=64, k=3, s=1, p=1, d=1, g=1, bias=True, relu=False),
+    # 40 channels under a 3 x 3 kernel: the MFMA kernels on a channel-padded copy in a workspace
+    dict(shape=(2, 40, 14, 14), oc=24, k=3, s=1, p=1, d=1, g=1, bias=True, relu=True),
 ]
 
 

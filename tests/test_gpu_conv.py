@@ -263,6 +263,71 @@ def test_conv_depthwise_on_the_vector_alu(cabi, spec, x_signed):
             assert d.max() == 0, f"{np.count_nonzero(d)} of {d.size} bytes differ (max {d.max()})"
 
 
+@pytest.mark.parametrize("spec", [
+    (2, 14, 14, 40, 40, 3, 1, 1, 1, 1),      # 3 x 3 over 40 channels: kernel rows of 128 padded bytes, 384 in all
+    (1, 35, 35, 3, 16, 11, 4, 2, 1, 1),      # the 11 x 11 stride 4 first layer of an early image network
+    (2, 9, 9, 72, 24, 3, 2, 1, 1, 1),
+    (1, 10, 10, 300, 32, 1, 1, 0, 1, 1),     # a pointwise layer over 300 channels: then a linear layer over 304
+    (2, 12, 12, 24, 32, 5, 1, 2, 2, 1),      # dilation keeps the byte-run kernel away
+    (2, 12, 12, 3, 20, 3, 1, 1, 1, 1),       # a byte-run shape, pinned here
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_on_channel_padded_copy(cabi, spec, x_signed):
+    """One group off the 16-channel grid: the MFMA kernels on a copy of the input with padded
+    channels in the workspace, against the oracle and against the run without a workspace."""
+    say("conv padded channels", spec, x_signed)
+    c = _conv_case(*spec, seed=sum(spec) + 23, x_signed=x_signed, relu=not x_signed)
+    want_acc = oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                   c["groups"], c["x_zp"], nthreads=8)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    g = cabi.conv_geom(c["xq"].shape, c["wq"].shape, c["stride"], c["padding"], c["dilation"], c["groups"])
+    automatic = not (spec[3] == 3 and spec[5] == 3)   # (3 x 3 over 3 channels: the byte-run kernel's)
+    assert (cabi.lib().tmq_conv2d_workspace_bytes(g) > 0) == automatic
+    for path, workspace in ((8, True), (-1, True), (-1, False)):
+        cabi.force_conv_path(path)
+        cabi.use_conv_workspace(workspace)
+        try:
+            y, acc, _ = _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+            cabi.use_conv_workspace(True)
+        np.testing.assert_array_equal(acc, want_acc)
+        _check(y, want, f"path {path}, workspace {workspace}")
+    cabi.force_conv_path(8)
+    cabi.use_conv_workspace(False)
+    try:
+        with pytest.raises(cabi.TmqError):
+            _run(cabi, c)
+    finally:
+        cabi.force_conv_path(-1)
+        cabi.use_conv_workspace(True)
+    # fused: residual + ReLU
+    rng = np.random.default_rng(sum(spec))
+    f = dict(c, accq=rng.integers(0, 256, want.shape, dtype=np.uint8), acc_scale=0.35, acc_zp=110,
+             activation="relu", signed=False, relu=False, out_zp=20)
+    want_f = oracle.conv2d_fused(f["xq"], f["x_scale"], f["x_zp"], f["wq"], f["w_scales"], f["bias"],
+                                 f["stride"], f["padding"], f["dilation"], f["groups"], f["out_scale"],
+                                 f["out_zp"], accum=f["accq"], accum_scale=f["acc_scale"],
+                                 accum_zp=f["acc_zp"], activation="relu", out_signed=False, nthreads=8)
+    cabi.force_conv_path(8)
+    try:
+        yf = _run_fused(cabi, f)
+    finally:
+        cabi.force_conv_path(-1)
+    np.testing.assert_array_equal(yf, want_f)
+    # groups, or channels already on the grid: not this path's
+    for bad in [(1, 8, 8, 32, 16, 3, 1, 1, 1, 1), (1, 8, 8, 24, 24, 3, 1, 1, 1, 2)]:
+        cb = _conv_case(*bad, seed=1)
+        cabi.force_conv_path(8)
+        try:
+            with pytest.raises(cabi.TmqError):
+                _run(cabi, cb)
+        finally:
+            cabi.force_conv_path(-1)
+
+
 def test_conv_depthwise_lanes_limits(cabi):
     """What the four-channels-per-lane kernel refuses: groups that are not single channels, channel
     counts off the dword grid, more output channels than input channels."""

@@ -473,7 +473,8 @@ def force_linear_config(cfg: int) -> None:
 def force_conv_path(path: int) -> None:
     """Pin the conv2d kernel family of later calls through this binding
     (-1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct, 4 byte runs, 5 pointwise as linear,
-    6 patch rows in a workspace + linear, 7 depthwise on the vector ALU)."""
+    6 patch rows in a workspace + linear, 7 depthwise on the vector ALU, 8 channels padded to 16 in a
+    workspace, then the automatic choice for that)."""
     global _conv_path
     _conv_path = int(path)
 
@@ -562,11 +563,14 @@ def _conv_desc(x, pw, g, x_scale, x_zp, w_scales, bias, out_scale, out_zp, out_s
     d.y = _ptr(y)
     d.kernel = _conv_path if _conv_path > 0 else 0
     d.tile_rows, d.tile_cols = _conv_tile
-    # scratch for the layers that run on their patch rows (pinned for tests: whatever the size)
+    # scratch for the layers that run on their patch rows or on a channel-padded copy of the input
+    # (pinned for tests: whatever the size)
     need = lib().tmq_conv2d_workspace_bytes(C.byref(g))
     if _conv_path == 6 and g.groups == 1 and g.IC % 16 == 0:
         oh, ow = conv_out_hw(g)
         need = g.B * oh * ow * g.KH * g.KW * g.IC
+    if _conv_path == 8 and g.groups == 1 and g.IC % 16 != 0:
+        need = g.B * g.H * g.W * ((g.IC + 15) // 16 * 16)
     if need > 0 and _conv_workspace:
         d._ws = torch.empty(need, dtype=torch.uint8, device=x.device)   # (kept alive by the descriptor)
         d.workspace, d.workspace_bytes = d._ws.data_ptr(), need

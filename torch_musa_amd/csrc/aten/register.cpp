@@ -630,16 +630,16 @@ struct PackedConvWeightTmq final : public ConvPackedParamsBase<2> {
     d.out_signed = x_signed;
     d.relu = activation == 1;
     d.y = y.data_ptr();
+    // scratch for the layers that run on their patch rows or on a channel-padded copy of the
+    // input (from the caching allocator: safe under stream capture, freed for reuse in stream order)
+    at::Tensor workspace;
+    const int64_t ws_bytes = tmq_conv2d_workspace_bytes(&g);
+    if (ws_bytes > 0) {
+      workspace = at::empty({ws_bytes}, x.options().dtype(at::kByte));
+      d.workspace = workspace.data_ptr();
+      d.workspace_bytes = ws_bytes;
+    }
     if (!accum.has_value() && activation != 2) {
-      // scratch for the layers that run on their patch rows (from the caching allocator:
-      // safe under stream capture, freed for reuse in stream order)
-      at::Tensor workspace;
-      const int64_t ws_bytes = tmq_conv2d_workspace_bytes(&g);
-      if (ws_bytes > 0) {
-        workspace = at::empty({ws_bytes}, x.options().dtype(at::kByte));
-        d.workspace = workspace.data_ptr();
-        d.workspace_bytes = ws_bytes;
-      }
       check_status(tmq_conv2d(&d, current_stream(x)), "tmq_conv2d");
       return y;
     }
@@ -1402,6 +1402,13 @@ at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero
   if (accum.has_value())
     TORCH_CHECK(accum->sizes() == c10::IntArrayRef(out_shape) && accum->device() == act.device(), what,
                 ": accum must have the output's shape ", c10::IntArrayRef(out_shape), " and device");
+  at::Tensor workspace;  // (as in PackedConvWeightTmq::apply)
+  const int64_t ws_bytes = tmq_conv2d_workspace_bytes(&g);
+  if (ws_bytes > 0) {
+    workspace = at::empty({ws_bytes}, act.options().dtype(at::kByte));
+    d.workspace = workspace.data_ptr();
+    d.workspace_bytes = ws_bytes;
+  }
   if (!o.is_int) {
     // float output: exact int32 accumulators from the MFMA kernel, scaled here
     TORCH_CHECK(!accum.has_value() || accum_scale == 1.0, "fp32 or bf16 output, accum_scale must be 1.0.");
@@ -1422,13 +1429,6 @@ at::Tensor qconv_plain(const at::Tensor& act, double act_scale, int64_t act_zero
   d.relu = relu;
   d.y = y.data_ptr();
   if (!accum.has_value()) {
-    at::Tensor workspace;  // (as in PackedConvWeightTmq::apply)
-    const int64_t ws_bytes = tmq_conv2d_workspace_bytes(&g);
-    if (ws_bytes > 0) {
-      workspace = at::empty({ws_bytes}, act.options().dtype(at::kByte));
-      d.workspace = workspace.data_ptr();
-      d.workspace_bytes = ws_bytes;
-    }
     check_status(tmq_conv2d(&d, stream), "tmq_conv2d");
     return y;
   }

@@ -197,6 +197,36 @@ int64_t patch_rows_bytes(const tmq_conv2d_geom& g, const ConvShape& s, bool pinn
   return rows * s.Kp;
 }
 
+// One group whose channel count is no multiple of 16 and whose kernel rows are too long for the
+// byte-run kernel (3 x 3 over 40 channels, 11 x 11 over 3): with scratch memory the input is
+// copied once with every pixel's channels padded to whole 16-channel blocks, and the MFMA kernels
+// run on the copy -- the packed weight already holds zeros at the padded positions of K, so what
+// the padding bytes are does not matter.  The bytes of that copy, 0 when the layer is not such a one.
+int64_t padded_input_bytes(const tmq_conv2d_geom& g, const ConvShape& s, bool pinned) {
+  if (g.groups != 1 || s.IC % 16 == 0) return 0;
+  if (!pinned && s.runs_KS != 0) return 0;
+  const int64_t pixels = s.B * s.H * s.W, blocks = ceil_div(s.IC, 16);
+  if (pixels == 0 || pixels * blocks > 0x7fffffff) return 0;
+  return pixels * blocks * 16;
+}
+
+// One thread per 16-byte block of the padded copy.
+__global__ __launch_bounds__(256) void conv_pad_channels_kernel(const uint8_t* __restrict__ x, int IC, int blocks,
+                                                                int64_t total, uint8_t* __restrict__ dst) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const int64_t pixel = id / blocks;
+  const int c0 = static_cast<int>(id - pixel * blocks) * 16;
+  const uint8_t* src = x + pixel * IC + c0;
+  const int n = IC - c0 < 16 ? IC - c0 : 16;
+  uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int b = 0; b < 16; ++b)
+    if (b < n) words[b >> 2] |= static_cast<uint32_t>(src[b]) << (8 * (b & 3));
+  *reinterpret_cast<v4i*>(dst + id * 16) = v4i{static_cast<int>(words[0]), static_cast<int>(words[1]),
+                                               static_cast<int>(words[2]), static_cast<int>(words[3])};
+}
+
 struct PlainArgs {
   const uint8_t* x;
   const uint8_t* w_packed;
@@ -698,6 +728,33 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
       }
     }
   }
+  // Channel counts off the 16-channel grid under kernel rows too long for the byte runs: the MFMA kernels on a
+  // padded copy of the input in the caller's scratch memory (3 x 3, 40 -> 40 channels on 56 x 56 at batch 32 and
+  // the 11 x 11 stride 4 first layer of an early image network, 3 -> 64 on 224 x 224, otherwise on the direct kernel).
+  if (forced == 8 || forced < 0) {
+    const int64_t need = padded_input_bytes(d->geom, s, forced == 8);
+    tmq_conv2d_geom padded_geom = d->geom;
+    padded_geom.IC = round_up(s.IC, 16);
+    ConvShape padded_shape;
+    const bool use = need > 0 && d->workspace != nullptr && d->workspace_bytes >= need && aligned(d->workspace, 16) &&
+                     make_shape(&padded_geom, &padded_shape) == TMQ_OK;
+    if (forced == 8 && !use) return TMQ_ERR_UNSUPPORTED;
+    if (use) {
+      const int64_t chunks = need / 16;
+      conv_pad_channels_kernel<<<dim3(static_cast<unsigned>(ceil_div(chunks, 256))), dim3(256), 0, stream>>>(
+          static_cast<const uint8_t*>(d->x), static_cast<int>(s.IC), static_cast<int>(ceil_div(s.IC, 16)), chunks,
+          static_cast<uint8_t*>(d->workspace));
+      if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
+      tmq_conv2d_desc padded = *d;
+      padded.x = d->workspace;
+      padded.geom = padded_geom;
+      padded.workspace = nullptr;
+      padded.workspace_bytes = 0;
+      padded.kernel = 0;
+      padded.tile_rows = padded.tile_cols = 0;
+      return run_conv<MODE>(&padded, post, out, stream);
+    }
+  }
   const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
   if ((forced == 1 || forced == 2) && !mfma_ok) return TMQ_ERR_UNSUPPORTED;
   // depthwise layers: four channels per lane on the vector ALU
@@ -872,7 +929,8 @@ TMQ_EXPORT int64_t tmq_conv2d_workspace_bytes(const tmq_conv2d_geom* g) {
   if (make_shape(g, &s) != TMQ_OK) return 0;
   TilePlan tp;
   const int64_t need = patch_rows_bytes(*g, s, false);
-  return need > 0 && !(s.ICg % 16 == 0 && plan_tiles(s, false, 0, 0, &tp)) ? need : 0;
+  if (need > 0 && !(s.ICg % 16 == 0 && plan_tiles(s, false, 0, 0, &tp))) return need;
+  return padded_input_bytes(*g, s, false);
 }
 
 TMQ_EXPORT int tmq_conv2d_out_hw(const tmq_conv2d_geom* g, int64_t* OH, int64_t* OW) {
