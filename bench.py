@@ -1253,6 +1253,9 @@ def main():
                   "conv2d_relu 7x7 stride 2, 3 -> 64 channels, [32,3,224,224]")
         conv_line("conv2d_relu_depthwise_3x3_32ch", 32, 32, 3, 1, 1, 32, 112,
                   "conv2d_relu depthwise 3x3, 32 channels, [32,32,112,112]")
+        # the depthwise 7 x 7 of a ConvNeXt stage: 96 channels on 56 x 56
+        conv_line("conv2d_depthwise_7x7_96ch", 96, 96, 7, 1, 3, 96, 56,
+                  "conv2d depthwise 7x7, 96 channels, [32,96,56,56]", op="conv2d")
         # the fused SiLU form the reference adds for detectors: 32 -> 64 channels, 3 x 3 stride 2 on 320 x 320, batch 8
         conv_line("conv2d_silu_3x3_s2_32to64_320", 32, 64, 3, 2, 1, 1, 320,
                   "conv2d_silu 3x3 stride 2, 32 -> 64 channels, [8,32,320,320]", op="conv2d_silu", batch=8)

@@ -79,14 +79,14 @@ def test_packed_size_arithmetic():
     g3 = cabi.conv_geom((1, 64, 64, 3), (16, 11, 11), (4, 4), (0, 0), (1, 1), 1)
     assert lib.tmq_conv2d_packed_bytes(g3) == 1 * (121 * 16 + 127) // 128 * 8 * 256
     # depthwise, 32 channels: the 32 groups are packed as one block-diagonal group, K = 9 taps x 32 channels;
-    # behind it, for channel counts on the dword grid, the weight once more as [tap][channel] bytes
+    # behind it, for channel counts on the dword grid, the weight once more as [channel][3 rows][4 bytes]
     g4 = cabi.conv_geom((1, 20, 20, 32), (32, 3, 3), (1, 1), (1, 1), (1, 1), 32)
-    assert lib.tmq_conv2d_packed_bytes(g4) == 2 * 24 * 256 + 9 * 32
+    assert lib.tmq_conv2d_packed_bytes(g4) == 2 * 24 * 256 + 12 * 32
     # 144 channels: three merged groups of 48; 40 channels: no multiple of 16 divides them, 40 groups of one
     g5 = cabi.conv_geom((1, 20, 20, 144), (144, 3, 3), (1, 1), (1, 1), (1, 1), 144)
-    assert lib.tmq_conv2d_packed_bytes(g5) == 3 * 3 * 32 * 256 + 9 * 144
+    assert lib.tmq_conv2d_packed_bytes(g5) == 3 * 3 * 32 * 256 + 12 * 144
     g6 = cabi.conv_geom((1, 20, 20, 40), (40, 3, 3), (1, 1), (1, 1), (1, 1), 40)
-    assert lib.tmq_conv2d_packed_bytes(g6) == 40 * 1 * 16 * 256 + 368   # (9 * 40 bytes in whole 16-byte pieces)
+    assert lib.tmq_conv2d_packed_bytes(g6) == 40 * 1 * 16 * 256 + 12 * 40
     g7 = cabi.conv_geom((1, 20, 20, 10), (10, 3, 3), (1, 1), (1, 1), (1, 1), 10)                  # off the dword grid: no copy
     assert lib.tmq_conv2d_packed_bytes(g7) == 10 * 1 * 16 * 256
     # scratch for layers that run on their patch rows: few pixels against a long K that the halo tiles do not hold

@@ -205,7 +205,9 @@ def test_conv_narrow_groups_merged(cabi, spec, x_signed):
     (1, 9, 9, 40, 40, 3, 2, 1, 1, 40),       # stride 2
     (3, 17, 13, 24, 24, 5, 1, 2, 1, 24),     # 5 x 5: whole weight dwords in registers
     (2, 21, 21, 120, 120, 5, 2, 2, 1, 120),
-    (1, 15, 15, 12, 12, 7, 1, 3, 1, 12),     # any other kernel size: weights read at use
+    (1, 15, 15, 12, 12, 7, 1, 3, 1, 12),     # 7 x 7: two dwords of taps per kernel row
+    (2, 20, 9, 96, 96, 7, 2, 3, 1, 96),      # ... at stride 2: the whole window per output row
+    (1, 13, 13, 8, 8, 9, 1, 4, 1, 8),        # any other kernel size: a plain loop over the taps
     (2, 11, 14, 20, 20, 3, 1, 2, 2, 20),     # dilation
     (1, 6, 6, 4, 4, 3, 1, 0, 1, 4),          # one lane per pixel, no padding
     (2, 3, 40, 36, 36, 3, 1, 1, 1, 36),      # fewer output rows than a strip

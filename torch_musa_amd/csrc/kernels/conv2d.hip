@@ -37,8 +37,8 @@ struct ConvShape {
   // the second weight layout, behind the first, for the kernel of conv_runs.h: k-steps
   // (0: the shape is not that kernel's), run bytes, padded run bytes, offset and size in bytes
   int64_t runs_KS, runs_RL, runs_RP, runs_off, runs_bytes;
-  // depthwise layers over a multiple of 4 channels: a [tap][channel] copy of the weight for the
-  // kernel of conv_depthwise.h in the same place (0: not such a layer)
+  // depthwise layers over a multiple of 4 channels: a [channel][kernel row][taps padded to a multiple
+  // of 4] copy of the weight for the kernel of conv_depthwise.h in the same place (0: not such a layer)
   int64_t taps_bytes;
 };
 
@@ -96,7 +96,7 @@ int make_shape(const tmq_conv2d_geom* g, ConvShape* s) {
   }
   s->taps_bytes = 0;
   if (g->groups > 1 && g->groups == g->IC && g->IC == g->OC && g->IC % 4 == 0)
-    s->taps_bytes = round_up(g->KH * g->KW * g->IC, 16);
+    s->taps_bytes = round_up(g->IC * g->KH * round_up(g->KW, 4), 16);
   // 32-bit index arithmetic inside the kernels
   if (g->H > (1 << 24) || g->W > (1 << 24) || g->IC > (1 << 24) || s->Kp > (1 << 30) ||
       g->B * s->OH * s->OW > 0x7fffffff || g->H * g->W * g->IC > 0x3fffffff)
@@ -141,13 +141,15 @@ __global__ __launch_bounds__(256) void conv_prepack_runs_kernel(const int8_t* __
                      static_cast<int>(s.runs_RP), static_cast<int>(s.runs_KS));
 }
 
-// One thread per byte of the [tap][channel] layout of conv_depthwise.h (the caller's weight is [channel][tap]).
-__global__ __launch_bounds__(256) void conv_prepack_taps_kernel(const int8_t* __restrict__ w, int64_t C, int64_t taps,
-                                                                int64_t total, uint8_t* __restrict__ dst) {
+// One thread per byte of the [channel][kernel row][padded taps] layout of conv_depthwise.h (the
+// caller's weight is [channel][kernel row][tap]).
+__global__ __launch_bounds__(256) void conv_prepack_taps_kernel(const int8_t* __restrict__ w, int64_t C, int64_t KH,
+                                                                int64_t KW, int64_t total, uint8_t* __restrict__ dst) {
   const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (id >= total) return;
-  const int64_t tp = id / C, c = id % C;
-  dst[id] = tp < taps ? static_cast<uint8_t>(w[c * taps + tp]) : uint8_t{0};
+  const int64_t kwp = (KW + 3) / 4 * 4;
+  const int64_t kw = id % kwp, kh = id / kwp % KH, c = id / (kwp * KH);
+  dst[id] = c < C && kw < KW ? static_cast<uint8_t>(w[(c * KH + kh) * KW + kw]) : uint8_t{0};
 }
 
 __global__ __launch_bounds__(256) void conv_colsum_kernel(const int8_t* __restrict__ w, int64_t OC,
@@ -583,10 +585,12 @@ int launch_conv_depthwise(const tmq_conv2d_desc* d, const ConvShape& s, const Po
   a.ph = static_cast<int>(s.ph); a.pw = static_cast<int>(s.pw);
   a.dh = static_cast<int>(s.dh); a.dw = static_cast<int>(s.dw);
   // Output rows per lane: long strips amortise the lane's weights and constants, short ones put
-  // more waves in flight; the longest with a wave per SIMD.
+  // more waves in flight; the longest with a wave per SIMD (half a wave under a 7 x 7 kernel, whose
+  // window of 49 taps is the larger part of a short strip's work).
   int64_t strip = d->kernel == 7 && d->tile_rows > 0 ? d->tile_rows : kDwStripMax;
+  const int64_t lanes_wanted = int64_t{1} << (s.KH == 7 && s.KW == 7 ? 15 : 16);
   if (!(d->kernel == 7 && d->tile_rows > 0))
-    while (strip > 1 && s.B * ceil_div(s.OH, strip) * s.OW * (s.IC / 4) < (int64_t{1} << 16)) strip /= 2;
+    while (strip > 1 && s.B * ceil_div(s.OH, strip) * s.OW * (s.IC / 4) < lanes_wanted) strip /= 2;
   if (strip > s.OH) strip = s.OH;
   a.strip = static_cast<int>(strip);
   const int64_t per_image = ceil_div(s.OH, strip) * s.OW * (s.IC / 4);
@@ -607,9 +611,11 @@ int launch_conv_depthwise(const tmq_conv2d_desc* d, const ConvShape& s, const Po
   const auto launch = [&](auto post_tag) {
     constexpr bool kP = decltype(post_tag)::value;
     if (s.KH == 3 && s.KW == 3)
-      conv_depthwise_kernel<MODE, kP, 9><<<grid, block, 0, stream>>>(a);
+      conv_depthwise_kernel<MODE, kP, 3><<<grid, block, 0, stream>>>(a);
     else if (s.KH == 5 && s.KW == 5)
-      conv_depthwise_kernel<MODE, kP, 25><<<grid, block, 0, stream>>>(a);
+      conv_depthwise_kernel<MODE, kP, 5><<<grid, block, 0, stream>>>(a);
+    else if (s.KH == 7 && s.KW == 7)
+      conv_depthwise_kernel<MODE, kP, 7><<<grid, block, 0, stream>>>(a);
     else
       conv_depthwise_kernel<MODE, kP, 0><<<grid, block, 0, stream>>>(a);
   };
@@ -764,11 +770,12 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
                           s.B * s.OH * s.OW * s.OC < (int64_t{1} << (MODE == kOutAcc32 ? 29 : 31)) && aligned(d->x, 4) && aligned(out, MODE == kOutAcc32 ? 16 : 4) &&
                           (po.accum == nullptr || aligned(po.accum, 4));
     if (forced == 7 && !lanes_ok) return TMQ_ERR_UNSUPPORTED;
-    // Also where the groups would merge into 16-channel blocks for the matrix pipe, for 3 x 3 kernels and for
-    // 5 x 5 at stride 1 (batch 32, against the merged groups on the halo tiles: 32 channels on 112 x 112 14.7
-    // against 17.3 us; 96 channels, 112 x 112 -> 56 x 56: 13.6 against 26.0 us; 960 channels on 7 x 7: 4.6 against
-    // 5.8 us; 384 on 14 x 14 level at 6 us); other kernel sizes stay with the matrix pipe where they can.
-    const bool lanes_first = (s.KH == 3 && s.KW == 3) || (s.KH == 5 && s.KW == 5 && s.sh == 1 && s.dh == 1);
+    // Also where the groups would merge into 16-channel blocks for the matrix pipe, for the kernel sizes with a
+    // register window (batch 32, against the merged groups on the halo tiles or the implicit GEMM: 3 x 3, 32
+    // channels on 112 x 112 12.6 against 16.7 us; 96 channels, 112 x 112 -> 56 x 56: 13.9 against 25.2 us; 5 x 5, 240
+    // channels on 28 x 28: 13.0 against 17.1 us; 7 x 7, 96 channels on 56 x 56: 22 against 72 us, 768 on 7 x 7: 6.7
+    // against 242 us); other kernel sizes stay with the matrix pipe where they can.
+    const bool lanes_first = s.KH == s.KW && (s.KH == 3 || s.KH == 5 || s.KH == 7);
     if (forced == 7 || (forced < 0 && lanes_ok && (!mfma_ok || lanes_first)))
       return launch_conv_depthwise<MODE>(d, s, po, zp_f, lo_f, hi_f, out, stream);
   }
@@ -964,7 +971,7 @@ TMQ_EXPORT int tmq_conv2d_prepack(const int8_t* w_ohwi, const tmq_conv2d_geom* g
   }
   if (s.taps_bytes > 0) {
     conv_prepack_taps_kernel<<<dim3(static_cast<unsigned>(ceil_div(s.taps_bytes, 256))), dim3(256), 0, hs>>>(
-        w_ohwi, s.IC, s.KH * s.KW, s.taps_bytes, static_cast<uint8_t*>(packed) + s.runs_off);
+        w_ohwi, s.IC, s.KH, s.KW, s.taps_bytes, static_cast<uint8_t*>(packed) + s.runs_off);
     if (launch_status() != TMQ_OK) return TMQ_ERR_LAUNCH;
   }
   blocks = ceil_div(s.OC, 256 / kWave);

@@ -4,24 +4,26 @@
 // A depthwise layer has no sum over channels: per output value KH * KW products.  The matrix
 // pipe can only take it as a block-diagonal product that is mostly zeros (conv2d.hip merges
 // the groups for that, where the channel count allows); here a lane owns four consecutive
-// channels of one output column and walks a strip of output rows:
-//   * the four channels' weights, one dword per tap from a [tap][channel] copy of the weight
-//     that prepack appends to the packed one, stay in registers for the strip (3 x 3 and
-//     5 x 5 kernels) -- for 3 x 3 already split into the four words (w & 0xff << 8 j) that
-//     let v_dot4_i32_i8 deliver one channel's product each (the larger kernels split the
-//     activation dword instead: one register per tap);
-//   * per output value and tap one aligned dword of the NHWC input (the same four channels
-//     of the tap's pixel; neighbouring lanes read neighbouring channels, then neighbouring
-//     pixels: whole cache lines per wave), the activation zero point for taps outside the
-//     image, the sign flip of unsigned activations, four dot products;
+// channels of one output column and walks a strip of output rows.  For 3 x 3, 5 x 5 and 7 x 7
+// kernels:
+//   * per window row the lane loads one aligned dword per tap of the NHWC input (the same four
+//     channels of the tap's pixel; neighbouring lanes read neighbouring channels, then
+//     neighbouring pixels: whole cache lines per wave), puts the activation zero point where
+//     the tap is outside the image, flips the sign of unsigned activations, and transposes
+//     four pixels x four channels of bytes with eight v_perm_b32, so that a dword holds one
+//     channel's bytes of four neighbouring taps;
+//   * the weights come from a [channel][kernel row][taps padded to a multiple of 4] copy that
+//     prepack appends to the packed weight, in the same shape, and stay in registers for the
+//     strip: one v_dot4_i32_i8 then multiplies four taps of one channel -- a quarter of the
+//     dot products that a dword of four channels against one tap would take;
+//   * at stride 1 the window's rows stay in registers from one output row to the next (the
+//     loop is unrolled over the kernel's height so that they never move), and the row that
+//     enters is asked for before the current output row's arithmetic and looked at after it;
 //   * requantisation of the four values as everywhere else, one dword store.
-// The vector ALU is what the kernel runs on (some 100 instructions per 3 x 3 output dword, a
-// third of them the dot products), then the latency of its loads: the strips are short where
-// the problem is small (more waves in flight), at stride 1 the window keeps its rows in
-// registers from one output row to the next, and the 3 x 3 and stride-1 loops ask for the next
-// output row's taps before they work on the current one's.
-// The x ^ 0x80 trick, the accumulator start value and the requantisation are those of
-// gemm_i8_core.h.
+// Other kernel sizes take a plain loop over the taps.  What the kernel waits for besides the
+// vector ALU is the latency of its loads: the strips are short where the problem is small
+// (more waves in flight).  The x ^ 0x80 trick, the accumulator start value and the
+// requantisation are those of gemm_i8_core.h.
 #pragma once
 
 #include "gemm_i8_core.h"
@@ -33,7 +35,7 @@ constexpr int kDwStripMax = 8;  // output rows per lane, at most
 
 struct DepthwiseArgs {
   const uint8_t* x;        // NHWC, less than 2^31 bytes
-  const uint8_t* w_taps;   // [KH * KW][C] bytes
+  const uint8_t* w_taps;   // [C][KH][roundup(KW, 4)] bytes
   const int32_t* colsum;
   const float* w_scales;
   const float* bias;
@@ -50,14 +52,27 @@ struct DepthwiseArgs {
   PostOps post;
 };
 
-// TAPS = KH * KW for the kernel sizes whose weights stay in registers (9: split, 25: whole
-// dwords), 0: any kernel size, weights read at use.
+// Four dwords of four bytes each, transposed: t[j] byte i = a[i] byte j.
+__device__ __forceinline__ void transpose_4x4_bytes(uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t (&t)[4]) {
+  // v_perm_b32 D, S0, S1, sel: byte i of D = byte sel[i] of {S0, S1} (S1 the low dword)
+  const uint32_t lo01 = __builtin_amdgcn_perm(a1, a0, 0x05010400u);  // a0.0 a1.0 a0.1 a1.1
+  const uint32_t hi01 = __builtin_amdgcn_perm(a1, a0, 0x07030602u);  // a0.2 a1.2 a0.3 a1.3
+  const uint32_t lo23 = __builtin_amdgcn_perm(a3, a2, 0x05010400u);
+  const uint32_t hi23 = __builtin_amdgcn_perm(a3, a2, 0x07030602u);
+  t[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+  t[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+  t[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+  t[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+// KS = the side of a square 3 x 3 / 5 x 5 / 7 x 7 kernel, 0: any kernel size.
 //
 // Addresses are 32-bit offsets from the tensors' bases and advance by additions.  A tap outside
 // the image still loads -- from row 0 / column 0 of the lane's image in its place, so that no
-// load sits behind a branch -- and the zero point replaces what came back.
-template <int MODE, bool POST, int TAPS>
-__global__ __launch_bounds__(kDwThreads) void conv_depthwise_kernel(DepthwiseArgs a) {
+// load sits behind a branch -- and the zero point replaces what came back, chosen by bits (a
+// select would let the compiler move the load behind a branch again).
+template <int MODE, bool POST, int KS>
+__global__ __launch_bounds__(kDwThreads, KS == 7 && !POST ? 3 : 1) void conv_depthwise_kernel(DepthwiseArgs a) {
   const uint32_t b = blockIdx.x / a.blocks_per_image;
   const uint32_t q = (blockIdx.x - b * a.blocks_per_image) * kDwThreads + threadIdx.x;
   if (q >= a.per_image) return;
@@ -65,26 +80,22 @@ __global__ __launch_bounds__(kDwThreads) void conv_depthwise_kernel(DepthwiseArg
   const uint32_t rest = q / C4, cg = q - rest * C4;
   const uint32_t strip = rest / static_cast<uint32_t>(a.OW), ow = rest - strip * static_cast<uint32_t>(a.OW);
   const uint32_t c = cg * 4;
-  constexpr int kSide = TAPS == 9 ? 3 : TAPS == 25 ? 5 : 0;
-  constexpr int kRegTaps = TAPS > 0 ? TAPS : 1;
+  constexpr int kSide = KS > 0 ? KS : 1;
+  constexpr int kGroups = (kSide + 3) / 4;  // dwords of four taps per kernel row
 
   // ---- this lane's four channels: weights and constants
-  uint32_t wsplit[TAPS == 9 ? 9 : 1][4];
-  uint32_t wraw[TAPS == 25 ? 25 : 1];
-  if constexpr (TAPS > 0) {
-#pragma unroll
-    for (int tp = 0; tp < TAPS; ++tp) {
-      const uint32_t w4 = *reinterpret_cast<const uint32_t*>(a.w_taps + static_cast<uint32_t>(tp * a.C) + c);
-      if constexpr (TAPS == 9) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) wsplit[tp][j] = w4 & (0xffu << (8 * j));
-      } else {
-        wraw[tp] = w4;
-      }
-    }
-  }
   // (every load unconditional and independent of the others, so that they are in flight together:
   // without a bias the column sums stand in as something to read)
+  uint32_t wreg[kSide][4][kGroups];
+  if constexpr (KS > 0) {
+    const uint32_t* const wl = reinterpret_cast<const uint32_t*>(a.w_taps) + c * (KS * kGroups);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) wreg[kh][j][g] = wl[(j * KS + kh) * kGroups + g];
+  }
   int acc0[4];
   v4f mult = {0.f, 0.f, 0.f, 0.f}, bdiv = {0.f, 0.f, 0.f, 0.f};
   float bmul = 1.0f;
@@ -120,18 +131,6 @@ __global__ __launch_bounds__(kDwThreads) void conv_depthwise_kernel(DepthwiseArg
   const int oh_end = oh_first + a.strip < a.OH ? oh_first + a.strip : a.OH;
   uint32_t yoff = ((b * static_cast<uint32_t>(a.OH) + oh_first) * static_cast<uint32_t>(a.OW) + ow) * static_cast<uint32_t>(a.C) + c;
   const uint32_t ystep = static_cast<uint32_t>(a.OW * a.C);
-  const auto mac = [&](int (&acc)[4], uint32_t x4, const uint32_t (&ws)[4]) {
-    const int xs = static_cast<int>(x4 ^ a.x_xor);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_sdot4(xs, static_cast<int>(ws[j]), acc[j], false);
-  };
-  // (one weight dword against the activation's bytes one at a time: no per-tap weight words to keep)
-  const auto mac_whole = [&](int (&acc)[4], uint32_t x4, uint32_t w4) {
-    const uint32_t xs = x4 ^ a.x_xor;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      acc[j] = __builtin_amdgcn_sdot4(static_cast<int>(xs & (0xffu << (8 * j))), static_cast<int>(w4), acc[j], false);
-  };
   const auto finish = [&](const int (&acc)[4]) {
     if constexpr (MODE == kOutAcc32) {
       *reinterpret_cast<v4i*>(static_cast<int32_t*>(a.y) + yoff) = v4i{acc[0], acc[1], acc[2], acc[3]};
@@ -148,129 +147,138 @@ __global__ __launch_bounds__(kDwThreads) void conv_depthwise_kernel(DepthwiseArg
     yoff += ystep;
   };
 
-  if constexpr (TAPS > 0) {
-    // the window's columns: fixed for the lane
-    // (the masks, all ones where the tap is inside the image, choose by bits between what was
-    // loaded and the zero point: a select would let the compiler move the load behind a branch)
-    uint32_t col[kSide], col_in[kSide];
+  if constexpr (KS > 0) {
+    // the window's columns: fixed for the lane (masks: all ones where the tap is inside the image)
+    uint32_t col[KS], col_in[KS];
 #pragma unroll
-    for (int kw = 0; kw < kSide; ++kw) {
+    for (int kw = 0; kw < KS; ++kw) {
       const int iw = iw0 + kw * a.dw;
       col_in[kw] = static_cast<unsigned>(iw) < static_cast<unsigned>(a.W) ? ~0u : 0u;
       col[kw] = lane_base + (static_cast<uint32_t>(iw * a.C) & col_in[kw]);
     }
-    // its rows: image row and byte position of that row, both advancing with the output row
-    int ih[kSide], row_pos[kSide];
+    // loads of one window row (what comes back is not looked at here) ...
+    const auto request_row = [&](int ih, int pos, uint32_t (&raw)[KS], uint32_t& row_in) {
+      row_in = static_cast<unsigned>(ih) < static_cast<unsigned>(a.H) ? ~0u : 0u;
+      const uint32_t rp = static_cast<uint32_t>(pos) & row_in;
 #pragma unroll
-    for (int kh = 0; kh < kSide; ++kh) {
-      ih[kh] = oh_first * a.sh - a.ph + kh * a.dh;
-      row_pos[kh] = ih[kh] * static_cast<int>(row_bytes);
-    }
-    const int row_step = a.sh * static_cast<int>(row_bytes);
-    // loads of one window (what comes back is not looked at here) ...
-    uint32_t row_in[kSide];
-    const auto request_window = [&](uint32_t (&raw)[kRegTaps]) {
+      for (int kw = 0; kw < KS; ++kw) raw[kw] = *reinterpret_cast<const uint32_t*>(a.x + (rp + col[kw]));
+    };
+    // ... and the row they make: [channel][group of four taps]
+    const auto settle_row = [&](const uint32_t (&raw)[KS], uint32_t row_in, uint32_t (&row)[4][kGroups]) {
+      uint32_t v[4 * kGroups];
 #pragma unroll
-      for (int kh = 0; kh < kSide; ++kh) {
-        row_in[kh] = static_cast<unsigned>(ih[kh]) < static_cast<unsigned>(a.H) ? ~0u : 0u;
-        const uint32_t rp = static_cast<uint32_t>(row_pos[kh]) & row_in[kh];
+      for (int kw = 0; kw < 4 * kGroups; ++kw) {
+        if (kw < KS) {
+          const uint32_t in = row_in & col_in[kw];
+          v[kw] = ((raw[kw] & in) | (a.pad_word & ~in)) ^ a.x_xor;
+        } else {
+          v[kw] = 0u;  // (against zero weights)
+        }
+      }
 #pragma unroll
-        for (int kw = 0; kw < kSide; ++kw) raw[kh * kSide + kw] = *reinterpret_cast<const uint32_t*>(a.x + (rp + col[kw]));
-        ih[kh] += a.sh;
-        row_pos[kh] += row_step;
+      for (int g = 0; g < kGroups; ++g) {
+        uint32_t t[4];
+        transpose_4x4_bytes(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], t);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) row[j][g] = t[j];
       }
     };
-    // ... and the window they make
-    const auto settle_window = [&](const uint32_t (&raw)[kRegTaps], uint32_t (&xv)[kRegTaps]) {
+    uint32_t win[KS][4][kGroups];
+    // window row kh of the current output row is win[(kh + ROT) % KS]
+    const auto window_sums = [&](auto rot_tag, int (&acc)[4]) {
+      constexpr int ROT = decltype(rot_tag)::value;
 #pragma unroll
-      for (int kh = 0; kh < kSide; ++kh)
+      for (int kh = 0; kh < KS; ++kh)
 #pragma unroll
-        for (int kw = 0; kw < kSide; ++kw) {
-          const uint32_t in = row_in[kh] & col_in[kw];
-          xv[kh * kSide + kw] = (raw[kh * kSide + kw] & in) | (a.pad_word & ~in);
-        }
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int g = 0; g < kGroups; ++g)
+            acc[j] = __builtin_amdgcn_sdot4(static_cast<int>(win[(kh + ROT) % KS][j][g]), static_cast<int>(wreg[kh][j][g]), acc[j], false);
     };
-    uint32_t xv[kRegTaps] = {}, raw[kRegTaps] = {};
+    const int ih_first = oh_first * a.sh - a.ph;
     if (a.sh == 1 && a.dh == 1) {
-      // Stride 1: the window moves down one image row per output row.  All but one of its rows
-      // stay in registers (sign flip applied); the row that enters is asked for before the
-      // current output row's arithmetic and looked at after it, also behind the strip's last row
-      // (rows outside the image read row 0, and nothing uses them).  The fences keep the
-      // compiler's scheduler from moving the loads down to their use.
-      request_window(raw);
-      settle_window(raw, xv);
+      // Stride 1: the window moves down one image row per output row.  The fences keep the
+      // compiler's scheduler from moving the entering row's loads down to their use.
+      {
+        uint32_t raw[KS][KS], row_in[KS];
 #pragma unroll
-      for (int tp = 0; tp < TAPS; ++tp) xv[tp] ^= a.x_xor;
-      int ih_next = ih[kSide - 1], pos_next = row_pos[kSide - 1];  // (request_window advanced them by one row)
-      uint32_t next[kSide] = {};
-      for (int oh = oh_first; oh < oh_end; ++oh) {
-        const uint32_t next_in = static_cast<unsigned>(ih_next) < static_cast<unsigned>(a.H) ? ~0u : 0u;
-        const uint32_t rp = static_cast<uint32_t>(pos_next) & next_in;
+        for (int kh = 0; kh < KS; ++kh) request_row(ih_first + kh, (ih_first + kh) * static_cast<int>(row_bytes), raw[kh], row_in[kh]);
 #pragma unroll
-        for (int kw = 0; kw < kSide; ++kw) next[kw] = *reinterpret_cast<const uint32_t*>(a.x + (rp + col[kw]));
+        for (int kh = 0; kh < KS; ++kh) settle_row(raw[kh], row_in[kh], win[kh]);
+      }
+      int ih_next = ih_first + KS, pos_next = ih_next * static_cast<int>(row_bytes);
+      int oh = oh_first;
+      // one output row; the entering row (also asked for behind the strip's last row: rows outside the
+      // image read row 0, and nothing uses them) takes the place of the window's row 0
+      const auto step = [&](auto rot_tag) {
+        constexpr int ROT = decltype(rot_tag)::value;
+        uint32_t raw[KS], row_in;
+        request_row(ih_next, pos_next, raw, row_in);
         ih_next += 1;
         pos_next += static_cast<int>(row_bytes);
         __builtin_amdgcn_sched_barrier(0);
         int acc[4] = {acc0[0], acc0[1], acc0[2], acc0[3]};
-#pragma unroll
-        for (int tp = 0; tp < TAPS; ++tp)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if constexpr (TAPS == 9)
-              acc[j] = __builtin_amdgcn_sdot4(static_cast<int>(xv[tp]), static_cast<int>(wsplit[tp][j]), acc[j], false);
-            else
-              acc[j] = __builtin_amdgcn_sdot4(static_cast<int>(xv[tp] & (0xffu << (8 * j))), static_cast<int>(wraw[tp]), acc[j], false);
-          }
+        window_sums(rot_tag, acc);
         finish(acc);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int tp = 0; tp < TAPS - kSide; ++tp) xv[tp] = xv[tp + kSide];
-#pragma unroll
-        for (int kw = 0; kw < kSide; ++kw) {
-          const uint32_t in = next_in & col_in[kw];
-          xv[TAPS - kSide + kw] = ((next[kw] & in) | (a.pad_word & ~in)) ^ a.x_xor;
+        settle_row(raw, row_in, win[ROT]);
+        ++oh;
+      };
+      while (true) {
+        if (oh >= oh_end) return;
+        step(std::integral_constant<int, 0>{});
+        if (oh >= oh_end) return;
+        step(std::integral_constant<int, 1 % KS>{});
+        if (oh >= oh_end) return;
+        step(std::integral_constant<int, 2 % KS>{});
+        if constexpr (KS >= 5) {
+          if (oh >= oh_end) return;
+          step(std::integral_constant<int, 3 % KS>{});
+          if (oh >= oh_end) return;
+          step(std::integral_constant<int, 4 % KS>{});
+        }
+        if constexpr (KS >= 7) {
+          if (oh >= oh_end) return;
+          step(std::integral_constant<int, 5 % KS>{});
+          if (oh >= oh_end) return;
+          step(std::integral_constant<int, 6 % KS>{});
         }
       }
-      return;
-    }
-    if constexpr (TAPS == 9) {
-      request_window(raw);
-      settle_window(raw, xv);
-    }
-    for (int oh = oh_first; oh < oh_end; ++oh) {
-      int acc[4] = {acc0[0], acc0[1], acc0[2], acc0[3]};
-      if constexpr (TAPS == 9) {
-        // (the whole next window ahead, as above)
-        request_window(raw);
-        __builtin_amdgcn_sched_barrier(0);
+    } else {
+      // any stride and dilation: the whole window per output row
+      for (int oh = oh_first; oh < oh_end; ++oh) {
+        const int ih0 = oh * a.sh - a.ph;
+        uint32_t raw[KS][KS], row_in[KS];
 #pragma unroll
-        for (int tp = 0; tp < 9; ++tp) mac(acc, xv[tp], wsplit[tp]);
-        finish(acc);
-        __builtin_amdgcn_sched_barrier(0);
-        settle_window(raw, xv);
-      } else {
-        request_window(raw);
-        settle_window(raw, xv);
+        for (int kh = 0; kh < KS; ++kh) request_row(ih0 + kh * a.dh, (ih0 + kh * a.dh) * static_cast<int>(row_bytes), raw[kh], row_in[kh]);
 #pragma unroll
-        for (int tp = 0; tp < 25; ++tp) mac_whole(acc, xv[tp], wraw[tp]);
+        for (int kh = 0; kh < KS; ++kh) settle_row(raw[kh], row_in[kh], win[kh]);
+        int acc[4] = {acc0[0], acc0[1], acc0[2], acc0[3]};
+        window_sums(std::integral_constant<int, 0>{}, acc);
         finish(acc);
       }
     }
   } else {
+    const int kwp = (a.KW + 3) & ~3;
     for (int oh = oh_first; oh < oh_end; ++oh) {
       int acc[4] = {acc0[0], acc0[1], acc0[2], acc0[3]};
       const int ih0 = oh * a.sh - a.ph;
-      uint32_t wpos = c;
       for (int kh = 0; kh < a.KH; ++kh) {
         const int ihh = ih0 + kh * a.dh;
         const bool row_ok = static_cast<unsigned>(ihh) < static_cast<unsigned>(a.H);
         const uint32_t rp = lane_base + (row_ok ? static_cast<uint32_t>(ihh) * row_bytes : 0u);
-        for (int kw = 0; kw < a.KW; ++kw, wpos += static_cast<uint32_t>(a.C)) {
+        for (int kw = 0; kw < a.KW; ++kw) {
           const int iw = iw0 + kw * a.dw;
           const uint32_t in = row_ok && static_cast<unsigned>(iw) < static_cast<unsigned>(a.W) ? ~0u : 0u;
           const uint32_t got = *reinterpret_cast<const uint32_t*>(a.x + (rp + (static_cast<uint32_t>(iw * a.C) & in)));
-          const uint32_t w4 = *reinterpret_cast<const uint32_t*>(a.w_taps + wpos);
-          mac_whole(acc, (got & in) | (a.pad_word & ~in), w4);
+          const uint32_t xs = ((got & in) | (a.pad_word & ~in)) ^ a.x_xor;
+          const uint8_t* const wt = a.w_taps + static_cast<uint32_t>((static_cast<int>(c) * a.KH + kh) * kwp + kw);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            // (one channel's byte of the activation dword against that channel's weight, both in byte j)
+            const uint32_t wj = static_cast<uint32_t>(wt[static_cast<uint32_t>(j * a.KH * kwp)]) << (8 * j);
+            acc[j] = __builtin_amdgcn_sdot4(static_cast<int>(xs & (0xffu << (8 * j))), static_cast<int>(wj), acc[j], false);
+          }
         }
       }
       finish(acc);
