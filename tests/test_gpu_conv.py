@@ -509,9 +509,9 @@ def _random_geometry(rng):
     h, w = int(rng.integers(5, 34)), int(rng.integers(5, 34))
     groups = 1
     if kind == 0:      # few input channels
-        ic, oc = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 24, 40])), int(rng.integers(1, 80))
+        ic, oc = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 24, 40, 72, 100])), int(rng.integers(1, 80))
     elif kind == 1:    # depthwise, with or without a channel multiplier
-        ic = int(rng.choice([16, 32, 40, 48, 96, 144]))
+        ic = int(rng.choice([8, 16, 20, 32, 40, 48, 72, 96, 120, 144]))
         groups, oc = ic, ic * int(rng.choice([1, 1, 2]))
     elif kind == 2:    # narrow groups
         icg, ocg, groups = int(rng.choice([2, 4, 8, 24])), int(rng.choice([2, 4, 6, 16])), int(rng.choice([2, 4, 8, 16]))
