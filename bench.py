@@ -171,7 +171,7 @@ def main():
                     help="do not start the child process that samples the socket power (for runs under a profiler, "
                          "whose library has initialised the GPU before this program starts)")
     ap.add_argument("--only", choices=["linear", "quantize", "dequantize", "minmax", "copy", "quantize_pc",
-                                       "dequantize_pc", "decode", "rows64", "rows256", "c1", "decode16_proj", "conv", "conv_add_relu", "conv_first_layer", "conv_depthwise",
+                                       "dequantize_pc", "decode", "rows64", "rows256", "c1", "decode16_proj", "conv", "conv_add_relu", "conv_first_layer", "conv_depthwise", "conv_depthwise7",
                                        "probe", "choice"],
                     help="run just this kernel --steps times (for rocprofv3 --kernel-trace / --pmc runs, so that "
                          "every launch of the kernel in the trace has the benchmark size); 'copy' is a plain "
@@ -381,10 +381,12 @@ def main():
         print(json.dumps({"only": args.only, "launches": args.steps, "x": [32, 56, 56, 64], "w": [64, 3, 3, 64]}))
         return
 
-    if args.only in ("conv_first_layer", "conv_depthwise"):
-        # the two convolution lines off the 16-channel grid: 7 x 7 stride 2, 3 -> 64 on [32,3,224,224];
-        # depthwise 3 x 3 over 32 channels on [32,32,112,112]; twelve inputs in turn
-        ic, oc, k, st, pad, groups, hw = (3, 64, 7, 2, 3, 1, 224) if args.only == "conv_first_layer" else (32, 32, 3, 1, 1, 32, 112)
+    if args.only in ("conv_first_layer", "conv_depthwise", "conv_depthwise7"):
+        # the convolution lines off the 16-channel grid: 7 x 7 stride 2, 3 -> 64 on [32,3,224,224];
+        # depthwise 3 x 3 over 32 channels on [32,32,112,112] and 7 x 7 over 96 channels on [32,96,56,56];
+        # twelve inputs in turn
+        ic, oc, k, st, pad, groups, hw = {"conv_first_layer": (3, 64, 7, 2, 3, 1, 224), "conv_depthwise": (32, 32, 3, 1, 1, 32, 112),
+                                          "conv_depthwise7": (96, 96, 7, 1, 3, 96, 56)}[args.only]
         xs_ = [torch._make_per_tensor_quantized_tensor(
             torch.randint(0, 120, (32, hw, hw, ic), dtype=torch.uint8, device=dev).permute(0, 3, 1, 2), 0.03, 0)
             for _ in range(12)]
@@ -1210,21 +1212,15 @@ def main():
         # ------------------------- every convolution of a ResNet-50 (53 layers, 23 distinct shapes), per
         # shape through the C ABI in a replayed graph over rotating inputs, summed with the shape's count:
         # what the layers of the operator cost next to one another at batch 32 and on a single image
-        def resnet50_convs(batch):
-            shapes = [(3, 64, 7, 2, 224, 1), (64, 64, 1, 1, 56, 1), (64, 64, 3, 1, 56, 3), (64, 256, 1, 1, 56, 4),
-                      (256, 64, 1, 1, 56, 2), (256, 128, 1, 1, 56, 1), (128, 128, 3, 2, 56, 1), (128, 512, 1, 1, 28, 4),
-                      (256, 512, 1, 2, 56, 1), (512, 128, 1, 1, 28, 3), (128, 128, 3, 1, 28, 3), (512, 256, 1, 1, 28, 1),
-                      (256, 256, 3, 2, 28, 1), (256, 1024, 1, 1, 14, 6), (512, 1024, 1, 2, 28, 1), (1024, 256, 1, 1, 14, 5),
-                      (256, 256, 3, 1, 14, 5), (1024, 512, 1, 1, 14, 1), (512, 512, 3, 2, 14, 1), (512, 2048, 1, 1, 7, 3),
-                      (1024, 2048, 1, 2, 14, 1), (2048, 512, 1, 1, 7, 2), (512, 512, 3, 1, 7, 2)]
+        def conv_stack(shapes, batch):
             total_us, rows_, layers = 0.0, [], 0
-            for ic, oc, k, st, hw, count in shapes:
-                g_ = cabi.conv_geom((batch, hw, hw, ic), (oc, k, k), (st, st), (k // 2, k // 2), (1, 1), 1)
+            for ic, oc, k, st, hw, count, groups in shapes:
+                g_ = cabi.conv_geom((batch, hw, hw, ic), (oc, k, k), (st, st), (k // 2, k // 2), (1, 1), groups)
                 oh_, ow_ = cabi.conv_out_hw(g_)
                 nbytes_ = batch * hw * hw * ic + batch * oh_ * ow_ * oc
                 nsets = max(2, min(6, (600 << 20) // nbytes_))
                 xs_ = [torch.randint(0, 256, (batch, hw, hw, ic), dtype=torch.uint8, device=dev) for _ in range(nsets)]
-                pw_ = cabi.PackedConv2d(torch.randint(-127, 128, (oc, k, k, ic), dtype=torch.int8, device=dev), g_)
+                pw_ = cabi.PackedConv2d(torch.randint(-127, 128, (oc, k, k, ic // groups), dtype=torch.int8, device=dev), g_)
                 ws_, b_ = torch.rand(oc, device=dev) * 0.002 + 0.001, torch.randn(oc, device=dev)
                 ys_ = [torch.empty((batch, oh_, ow_, oc), dtype=torch.uint8, device=dev) for _ in range(nsets)]
 
@@ -1235,12 +1231,20 @@ def main():
                 us_ = graph_us(run_, nsets)
                 total_us += count * us_
                 layers += count
-                rows_.append({"ic": ic, "oc": oc, "k": k, "stride": st, "hw": hw, "count": count, "us": round(us_, 2)})
+                rows_.append({"ic": ic, "oc": oc, "k": k, "stride": st, "hw": hw, "groups": groups, "count": count,
+                              "us": round(us_, 2)})
                 del xs_, ys_, pw_
             return total_us, layers, rows_
 
+        # (input channels, output channels, kernel, stride, image side, count, groups)
+        resnet50 = [(3, 64, 7, 2, 224, 1), (64, 64, 1, 1, 56, 1), (64, 64, 3, 1, 56, 3), (64, 256, 1, 1, 56, 4),
+                    (256, 64, 1, 1, 56, 2), (256, 128, 1, 1, 56, 1), (128, 128, 3, 2, 56, 1), (128, 512, 1, 1, 28, 4),
+                    (256, 512, 1, 2, 56, 1), (512, 128, 1, 1, 28, 3), (128, 128, 3, 1, 28, 3), (512, 256, 1, 1, 28, 1),
+                    (256, 256, 3, 2, 28, 1), (256, 1024, 1, 1, 14, 6), (512, 1024, 1, 2, 28, 1), (1024, 256, 1, 1, 14, 5),
+                    (256, 256, 3, 1, 14, 5), (1024, 512, 1, 1, 14, 1), (512, 512, 3, 2, 14, 1), (512, 2048, 1, 1, 7, 3),
+                    (1024, 2048, 1, 2, 14, 1), (2048, 512, 1, 1, 7, 2), (512, 512, 3, 1, 7, 2)]
         for batch_ in (32, 1):
-            tot_, layers_, rows_ = resnet50_convs(batch_)
+            tot_, layers_, rows_ = conv_stack([sh + (1,) for sh in resnet50], batch_)
             log(f"[bench] ResNet-50 convolutions, batch {batch_}: {layers_} layers, {tot_:.0f} us in all "
                 f"({tot_/layers_:.1f} us per layer)")
             secondary[f"conv2d_relu_resnet50_stack_b{batch_}"] = {
@@ -1248,6 +1252,26 @@ def main():
                 "images_per_s_convs_only": round(batch_ / (tot_ * 1e-6), 1), "shapes": rows_,
                 "method": "each distinct shape timed alone through tmq_conv2d (with ReLU) in a replayed HIP graph over "
                           "rotating inputs, times its count; 224 x 224 images, NHWC"}
+
+        # ... and of a MobileNetV2 (52 layers, 30 distinct shapes: a 3-channel first layer, depthwise 3 x 3 layers
+        # at both strides, pointwise layers whose channel counts -- 24, 144, 160, 320 -- are mostly off the 64 grid)
+        dwl = lambda c, st, hw, count: (c, c, 3, st, hw, count, c)
+        pwl = lambda ic, oc, hw, count: (ic, oc, 1, 1, hw, count, 1)
+        mobilenet_v2 = [(3, 32, 3, 2, 224, 1, 1), dwl(32, 1, 112, 1), pwl(32, 16, 112, 1), pwl(16, 96, 112, 1),
+                        dwl(96, 2, 112, 1), pwl(96, 24, 56, 1), pwl(24, 144, 56, 2), dwl(144, 1, 56, 1), pwl(144, 24, 56, 1),
+                        dwl(144, 2, 56, 1), pwl(144, 32, 28, 1), pwl(32, 192, 28, 3), dwl(192, 1, 28, 2), pwl(192, 32, 28, 2),
+                        dwl(192, 2, 28, 1), pwl(192, 64, 14, 1), pwl(64, 384, 14, 4), dwl(384, 1, 14, 4), pwl(384, 64, 14, 3),
+                        pwl(384, 96, 14, 1), pwl(96, 576, 14, 3), dwl(576, 1, 14, 2), pwl(576, 96, 14, 2), dwl(576, 2, 14, 1),
+                        pwl(576, 160, 7, 1), pwl(160, 960, 7, 3), dwl(960, 1, 7, 3), pwl(960, 160, 7, 2), pwl(960, 320, 7, 1),
+                        pwl(320, 1280, 7, 1)]
+        for batch_ in (32, 1):
+            tot_, layers_, rows_ = conv_stack(mobilenet_v2, batch_)
+            log(f"[bench] MobileNetV2 convolutions, batch {batch_}: {layers_} layers, {tot_:.0f} us in all "
+                f"({tot_/layers_:.1f} us per layer)")
+            secondary[f"conv2d_relu_mobilenet_v2_stack_b{batch_}"] = {
+                "layers": layers_, "total_us": round(tot_, 1), "per_layer_us": round(tot_ / layers_, 2),
+                "images_per_s_convs_only": round(batch_ / (tot_ * 1e-6), 1), "shapes": rows_,
+                "method": "as the ResNet-50 stack"}
 
         conv_line("conv2d_relu_first_layer_7x7_s2_3to64", 3, 64, 7, 2, 3, 1, 224,
                   "conv2d_relu 7x7 stride 2, 3 -> 64 channels, [32,3,224,224]")

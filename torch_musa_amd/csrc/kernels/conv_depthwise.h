@@ -74,8 +74,7 @@ __device__ __forceinline__ void transpose_4x4_bytes(uint32_t a0, uint32_t a1, ui
 template <int MODE, bool POST, int KS>
 __global__ __launch_bounds__(kDwThreads, KS == 7 && !POST ? 3 : 1) void conv_depthwise_kernel(DepthwiseArgs a) {
   const uint32_t b = blockIdx.x / a.blocks_per_image;
-  const uint32_t q = (blockIdx.x - b * a.blocks_per_image) * kDwThreads + threadIdx.x;
-  if (q >= a.per_image) return;
+  const uint32_t q0 = (blockIdx.x - b * a.blocks_per_image) * kDwThreads, q = q0 + threadIdx.x;
   const uint32_t C4 = static_cast<uint32_t>(a.C) >> 2;
   const uint32_t rest = q / C4, cg = q - rest * C4;
   const uint32_t strip = rest / static_cast<uint32_t>(a.OW), ow = rest - strip * static_cast<uint32_t>(a.OW);
@@ -83,33 +82,20 @@ __global__ __launch_bounds__(kDwThreads, KS == 7 && !POST ? 3 : 1) void conv_dep
   constexpr int kSide = KS > 0 ? KS : 1;
   constexpr int kGroups = (kSide + 3) / 4;  // dwords of four taps per kernel row
 
-  // ---- this lane's four channels: weights and constants
+  // ---- the channels' constants: accumulator start value, requantisation multiplier, bias term.
   // (every load unconditional and independent of the others, so that they are in flight together:
   // without a bias the column sums stand in as something to read)
-  uint32_t wreg[kSide][4][kGroups];
-  if constexpr (KS > 0) {
-    const uint32_t* const wl = reinterpret_cast<const uint32_t*>(a.w_taps) + c * (KS * kGroups);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int kh = 0; kh < KS; ++kh)
-#pragma unroll
-        for (int g = 0; g < kGroups; ++g) wreg[kh][j][g] = wl[(j * KS + kh) * kGroups + g];
-  }
-  int acc0[4];
-  v4f mult = {0.f, 0.f, 0.f, 0.f}, bdiv = {0.f, 0.f, 0.f, 0.f};
-  float bmul = 1.0f;
-  {
+  const auto channel_constants = [&](uint32_t ch, int (&acc0)[4], v4f& mult, v4f& bdiv) {
     const bool has_bias = a.bias != nullptr;
     const float* const bias_src = has_bias ? a.bias : reinterpret_cast<const float*>(a.colsum);
     int cs[4];
-    float wsc[4], bs[4];
+    float wsc[4] = {0.f, 0.f, 0.f, 0.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      cs[j] = a.colsum[c + j];
+      cs[j] = a.colsum[ch + j];
       if constexpr (MODE != kOutAcc32) {
-        wsc[j] = a.w_scales[(c + j) * a.w_scale_stride];
-        bs[j] = bias_src[c + j];
+        wsc[j] = a.w_scales[(ch + j) * a.w_scale_stride];
+        bs[j] = bias_src[ch + j];
       }
     }
 #pragma unroll
@@ -121,7 +107,46 @@ __global__ __launch_bounds__(kDwThreads, KS == 7 && !POST ? 3 : 1) void conv_dep
         bdiv[j] = has_bias ? bias_term(a.w_scale_stride == 0, bs[j], atw) : 0.f;
       }
     }
-    if constexpr (MODE != kOutAcc32) bmul = bias_mul(a.w_scale_stride == 0, a.x_scale * a.w_scales[0]);
+  };
+  int acc0[4];
+  v4f mult = {0.f, 0.f, 0.f, 0.f}, bdiv = {0.f, 0.f, 0.f, 0.f};
+  // With at most a block's worth of channel groups, the lanes of a block share few of them: the
+  // first C / 4 lanes work the constants out (a dozen divisions per group), the others read them.
+  __shared__ int s_acc0[kDwThreads * 4];
+  __shared__ float s_mult[kDwThreads * 4], s_bdiv[kDwThreads * 4];
+  if (C4 <= kDwThreads) {
+    if (threadIdx.x < C4) {
+      const uint32_t g = (q0 + threadIdx.x) % C4;
+      int a0[4];
+      v4f m = {0.f, 0.f, 0.f, 0.f}, bd = {0.f, 0.f, 0.f, 0.f};
+      channel_constants(g * 4, a0, m, bd);
+      *reinterpret_cast<v4i*>(&s_acc0[g * 4]) = v4i{a0[0], a0[1], a0[2], a0[3]};
+      *reinterpret_cast<v4f*>(&s_mult[g * 4]) = m;
+      *reinterpret_cast<v4f*>(&s_bdiv[g * 4]) = bd;
+    }
+    __syncthreads();
+    if (q >= a.per_image) return;
+    const v4i a0 = *reinterpret_cast<const v4i*>(&s_acc0[cg * 4]);
+    acc0[0] = a0[0]; acc0[1] = a0[1]; acc0[2] = a0[2]; acc0[3] = a0[3];
+    mult = *reinterpret_cast<const v4f*>(&s_mult[cg * 4]);
+    bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[cg * 4]);
+  } else {
+    if (q >= a.per_image) return;
+    channel_constants(c, acc0, mult, bdiv);
+  }
+  float bmul = 1.0f;
+  if constexpr (MODE != kOutAcc32) bmul = bias_mul(a.w_scale_stride == 0, a.x_scale * a.w_scales[0]);
+
+  // ---- this lane's four channels' weights
+  uint32_t wreg[kSide][4][kGroups];
+  if constexpr (KS > 0) {
+    const uint32_t* const wl = reinterpret_cast<const uint32_t*>(a.w_taps) + c * (KS * kGroups);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) wreg[kh][j][g] = wl[(j * KS + kh) * kGroups + g];
   }
 
   const uint32_t row_bytes = static_cast<uint32_t>(a.W * a.C);
