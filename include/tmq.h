@@ -364,7 +364,8 @@ typedef struct tmq_conv2d_desc {
    * (few input channels), 5 a pointwise layer as tmq_linear, 6 patch rows in the
    * workspace, then tmq_linear, 7 a depthwise layer four channels per lane on the
    * vector ALU, 8 the input copied into the workspace with its channels padded
-   * to a multiple of 16, then whatever the library chooses for that
+   * to a multiple of 16, then whatever the library chooses for that, 9 a pointwise
+   * layer over at most 256 input channels with its pixels straight from memory
    * (TMQ_ERR_UNSUPPORTED when the family cannot run the problem).  tile_rows / tile_cols > 0 pin the halo
    * kernel's patch height / bound its patch width. */
   int32_t kernel;

@@ -330,6 +330,71 @@ def test_conv_on_channel_padded_copy(cabi, spec, x_signed):
             cabi.force_conv_path(-1)
 
 
+@pytest.mark.parametrize("spec", [
+    (2, 14, 14, 24, 144, 1, 1, 0, 1, 1),     # 24 channels in: pixels at 8-byte addresses
+    (1, 9, 9, 3, 5, 1, 1, 0, 1, 1),          # 3 in, 5 out: any address, two channel tiles, byte stores
+    (2, 7, 7, 64, 256, 1, 1, 0, 1, 1),       # one whole k-step, four channel blocks
+    (1, 5, 5, 256, 64, 1, 1, 0, 1, 1),       # four k-steps
+    (3, 10, 10, 100, 40, 1, 1, 0, 1, 1),     # 100 in: the second k-step's last operand reaches into the next pixel
+    (1, 20, 20, 16, 16, 1, 1, 0, 1, 1),
+    (1, 3, 3, 32, 300, 1, 1, 0, 1, 1),       # fewer pixels than a piece, five channel blocks, the last one ragged
+    (1, 33, 31, 32, 16, 1, 1, 0, 1, 1),      # more pieces than one round of the waves
+])
+@pytest.mark.parametrize("x_signed", [False, True])
+def test_conv_pointwise_rows_from_memory(cabi, spec, x_signed):
+    """Pointwise layers over at most 256 input channels: MFMA operands straight from the NHWC input."""
+    say("conv pointwise rows", spec, x_signed)
+    c = _conv_case(*spec, seed=sum(spec) + 29, x_signed=x_signed, relu=x_signed)
+    want_acc = oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"],
+                                   c["groups"], c["x_zp"], nthreads=8)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["stride"], c["padding"], c["dilation"], c["groups"], c["out_scale"],
+                         c["out_zp"], relu=c["relu"], nthreads=8)
+    cabi.force_conv_path(9)
+    try:
+        y, acc, _ = _run(cabi, c)
+    finally:
+        cabi.force_conv_path(-1)
+    np.testing.assert_array_equal(acc, want_acc)
+    _check(y, want, "pinned")
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(acc, want_acc)
+    _check(y, want, "automatic")
+    rng = np.random.default_rng(sum(spec))
+    for activation, signed in (("relu", True), ("silu", False)):
+        f = dict(c, accq=(rng.integers(-128, 128, want.shape, dtype=np.int8) if activation == "relu" else None),
+                 acc_scale=0.35, acc_zp=-7, activation=activation, signed=signed, relu=False,
+                 out_zp=-20 if signed else 30)
+        want_f = oracle.conv2d_fused(f["xq"], f["x_scale"], f["x_zp"], f["wq"], f["w_scales"], f["bias"],
+                                     f["stride"], f["padding"], f["dilation"], f["groups"], f["out_scale"],
+                                     f["out_zp"], accum=f["accq"], accum_scale=f["acc_scale"],
+                                     accum_zp=f["acc_zp"], activation=activation, out_signed=signed, nthreads=8)
+        cabi.force_conv_path(9)
+        try:
+            yf = _run_fused(cabi, f)
+        finally:
+            cabi.force_conv_path(-1)
+        d = np.abs(yf.astype(np.int32) - want_f.astype(np.int32))
+        if activation == "silu":
+            assert d.max() <= LSB_TOL and np.count_nonzero(d) <= max(2, 0.001 * d.size), (d.max(), np.count_nonzero(d))
+        else:
+            assert d.max() == 0, f"{np.count_nonzero(d)} of {d.size} bytes differ (max {d.max()})"
+
+
+def test_conv_pointwise_rows_limits(cabi):
+    """Not that kernel's: a 3 x 3 kernel, a stride, padding, groups, more than 256 input channels."""
+    say("conv pointwise rows limits")
+    for spec in [(1, 8, 8, 16, 16, 3, 1, 1, 1, 1), (1, 8, 8, 16, 16, 1, 2, 0, 1, 1), (1, 8, 8, 16, 16, 1, 1, 1, 1, 1),
+                 (1, 8, 8, 32, 32, 1, 1, 0, 1, 2), (1, 4, 4, 272, 16, 1, 1, 0, 1, 1)]:
+        c = _conv_case(*spec, seed=5)
+        cabi.force_conv_path(9)
+        try:
+            with pytest.raises(cabi.TmqError):
+                _run(cabi, c)
+        finally:
+            cabi.force_conv_path(-1)
+
+
 def test_conv_depthwise_lanes_limits(cabi):
     """What the four-channels-per-lane kernel refuses: groups that are not single channels, channel
     counts off the dword grid, more output channels than input channels."""

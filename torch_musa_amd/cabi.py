@@ -474,7 +474,7 @@ def force_conv_path(path: int) -> None:
     """Pin the conv2d kernel family of later calls through this binding
     (-1 automatic, 1 halo tiles, 2 implicit GEMM, 3 direct, 4 byte runs, 5 pointwise as linear,
     6 patch rows in a workspace + linear, 7 depthwise on the vector ALU, 8 channels padded to 16 in a
-    workspace, then the automatic choice for that)."""
+    workspace, then the automatic choice for that, 9 pointwise with the pixels straight from memory)."""
     global _conv_path
     _conv_path = int(path)
 

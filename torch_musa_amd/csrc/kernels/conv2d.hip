@@ -566,6 +566,74 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   return launch_status();
 }
 
+// Pointwise layers over at most 256 input channels with their pixels straight from memory
+// (conv_runs_pointwise_kernel); false when the layer is not one of them.
+bool pointwise_rows_ok(const tmq_conv2d_geom& g, const ConvShape& s) {
+  return g.groups == 1 && s.KH == 1 && s.KW == 1 && s.sh == 1 && s.sw == 1 && s.ph == 0 && s.pw == 0 && s.runs_KS > 0 &&
+         conv_runs_pointwise_lds(s.OC, s.runs_KS) <= kCrPointwiseLdsMax;
+}
+
+template <int MODE>
+int launch_conv_pointwise_rows(const tmq_conv2d_desc* d, const ConvShape& s, const PostOps& po, float zp_f, float lo_f,
+                               float hi_f, void* out, hipStream_t stream) {
+  ConvRunArgs a{};
+  a.x = static_cast<const uint8_t*>(d->x);
+  a.w_runs = static_cast<const uint8_t*>(d->w_packed) + s.runs_off;
+  a.colsum = d->w_colsum;
+  a.w_scales = d->w_scales;
+  a.bias = d->bias;
+  a.y = out;
+  a.B = static_cast<int>(s.B);
+  a.H = static_cast<int>(s.H); a.W = static_cast<int>(s.W); a.IC = static_cast<int>(s.IC);
+  a.OH = static_cast<int>(s.OH); a.OW = static_cast<int>(s.OW); a.OC = static_cast<int>(s.OC);
+  a.KH = a.KW = 1;
+  a.sh = a.sw = 1;
+  a.RL = static_cast<int>(s.runs_RL); a.RP = static_cast<int>(s.runs_RP); a.KS = static_cast<int>(s.runs_KS);
+  const int64_t pieces = ceil_div(s.B * s.H * s.W, 16);
+  if (pieces > 0x7fffffff) return TMQ_ERR_UNSUPPORTED;
+  a.tiles = static_cast<int32_t>(pieces);
+  a.vec = aligned(out, 16) && s.OC % (MODE == kOutAcc32 ? 4 : 16) == 0 ? 1 : 0;
+  a.w_scale_stride = d->w_per_channel ? 1 : 0;
+  a.x_xor = d->x_signed ? 0u : 0x80808080u;
+  a.acc_coef = (d->x_signed ? 0 : 128) - d->x_zero_point;
+  a.x_scale = d->x_scale;
+  a.out_scale = d->out_scale;
+  a.zp_f = zp_f; a.lo_f = lo_f; a.hi_f = hi_f;
+  a.post = po;
+  const int nt = conv_runs_tiles(s.OC);
+  const int64_t lds = conv_runs_pointwise_lds(s.OC, s.runs_KS);
+  // as many blocks per CU as their registers and weights allow (three),
+  // each walking the pieces its waves are dealt
+  int64_t per_cu = (160 * 1024) / (lds + 512);
+  const int64_t by_registers = 3;
+  per_cu = per_cu < 1 ? 1 : per_cu > by_registers ? by_registers : per_cu;
+  const int64_t want = ceil_div(pieces, kCrWaves), cap = 256 * per_cu;
+  const dim3 grid(static_cast<unsigned>(want < cap ? want : cap)), block(kCrThreads);
+  const auto launch = [&](auto post_tag, auto nt_tag) {
+    auto* const kernel = conv_runs_pointwise_kernel<MODE, decltype(post_tag)::value, decltype(nt_tag)::value>;
+    // the kernel's LDS allowance is a per-device attribute: set once per device (and kernel)
+    static std::atomic<uint64_t> done{0};
+    const int dev = current_device();
+    if (dev < 0) return false;
+    if ((done.load(std::memory_order_acquire) >> dev & 1) == 0) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kCrPointwiseLdsMax) != hipSuccess)
+        return false;
+      done.fetch_or(uint64_t{1} << dev, std::memory_order_release);
+    }
+    kernel<<<grid, block, static_cast<size_t>(lds), stream>>>(a);
+    return true;
+  };
+  const auto launch_tiles = [&](auto nt_tag) {
+    if constexpr (MODE != kOutAcc32) {
+      if (po.any()) return launch(std::true_type{}, nt_tag);
+    }
+    return launch(std::false_type{}, nt_tag);
+  };
+  const bool ok = nt == 2 ? launch_tiles(std::integral_constant<int, 2>{}) : launch_tiles(std::integral_constant<int, 4>{});
+  return ok ? launch_status() : TMQ_ERR_LAUNCH;
+}
+
 // Depthwise layers on the vector ALU (conv_depthwise.h).
 template <int MODE>
 int launch_conv_depthwise(const tmq_conv2d_desc* d, const ConvShape& s, const PostOps& po, float zp_f, float lo_f,
@@ -763,6 +831,20 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   }
   const bool mfma_ok = s.ICg % 16 == 0 && aligned(d->x, 16);
   if ((forced == 1 || forced == 2) && !mfma_ok) return TMQ_ERR_UNSUPPORTED;
+  // pointwise layers over few input channels: pixels straight from memory against weights in LDS
+  {
+    const bool rows_ok = pointwise_rows_ok(d->geom, s) && (MODE != kOutAcc32 || aligned(out, 4));
+    if (forced == 9 && !rows_ok) return TMQ_ERR_UNSUPPORTED;
+    // Automatic where the image offers enough 16-pixel pieces for the chip's waves and few enough channel blocks
+    // for a wave to run them all (batch 32, against the halo tiles or the byte-run kernel: 32 -> 16 channels on
+    // 112 x 112 19.3 -> 10 us, 24 -> 144 on 56 x 56 21.5 -> 11.5 us, 16 -> 96 on 112 x 112 31 -> 25 us, 256 -> 128 on
+    // 56 x 56 18.6 -> 15.6 us, 192 -> 32 on 28 x 28 4.7 -> 4.0 us; 128 -> 512 on 28 x 28 10.5 against 12.5 us and
+    // 96 -> 576 on 14 x 14 5.8 against 11.4 us stay where they were).
+    const int64_t pieces = ceil_div(s.B * s.H * s.W, 16), blocks = ceil_div(s.OC, 16 * conv_runs_tiles(s.OC));
+    const bool worth = pieces >= 1024 && (blocks <= 3 || (pieces >= 4096 && blocks <= 4));
+    if (forced == 9 || (forced < 0 && rows_ok && worth))
+      return launch_conv_pointwise_rows<MODE>(d, s, po, zp_f, lo_f, hi_f, out, stream);
+  }
   // depthwise layers: four channels per lane on the vector ALU
   {
     // (32-bit byte offsets into the input and the output)

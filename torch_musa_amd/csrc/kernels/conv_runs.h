@@ -91,6 +91,66 @@ __device__ __forceinline__ v4i conv_runs_slot(const int8_t* __restrict__ w, int6
              static_cast<int>(words[3])};
 }
 
+// Requantise (or pass on) the 4 NT consecutive channels cb ... of one pixel that a lane holds after the
+// MFMAs of its NT channel tiles, and store them at element offset `off` of the output: one store of 4 NT
+// bytes where all the channels exist.  mult / bdiv: the constants of channel cb onwards.
+template <int MODE, bool POST, int NT>
+__device__ __forceinline__ void runs_requant_store(const ConvRunArgs& a, const v4i (&acc)[NT], int64_t off, int cb,
+                                                   const float* mult_cb, const float* bdiv_cb, float bmul) {
+  constexpr int kLaneCh = 4 * NT;
+  uint32_t packed[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int raw[4] = {acc[nt][0], acc[nt][1], acc[nt][2], acc[nt][3]};
+    if constexpr (MODE == kOutAcc32) {
+      int32_t* const dst = static_cast<int32_t*>(a.y) + off + 4 * nt;
+      if (a.vec && cb + 4 * nt + 4 <= a.OC) {
+        *reinterpret_cast<v4i*>(dst) = v4i{raw[0], raw[1], raw[2], raw[3]};
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (cb + 4 * nt + r < a.OC) dst[r] = raw[r];
+      }
+    } else {
+      const v4f mult = *reinterpret_cast<const v4f*>(mult_cb + 4 * nt);
+      const v4f bdiv = *reinterpret_cast<const v4f*>(bdiv_cb + 4 * nt);
+      if constexpr (POST) {
+        const int left = a.OC - (cb + 4 * nt);
+        const int nvalid = left < 0 ? 0 : (left < 4 ? left : 4);
+        const uint32_t accw =
+            a.post.accum != nullptr && nvalid > 0 ? load_accum4(a.post, off + 4 * nt, nvalid) : 0u;
+        packed[nt] = requant4_post<MODE>(raw, bdiv, bmul, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
+      } else {
+        packed[nt] = requant4<MODE>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+      }
+    }
+  }
+  if constexpr (MODE != kOutAcc32) {
+    uint8_t* const dst = static_cast<uint8_t*>(a.y) + off;
+    if (cb + kLaneCh <= a.OC) {  // one store of 4 NT bytes; any alignment unless the host found the rows aligned
+      if constexpr (NT == 4) {
+        const v4i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1]), static_cast<int>(packed[2]),
+                         static_cast<int>(packed[3])};
+        if (a.vec)
+          *reinterpret_cast<v4i*>(dst) = all;
+        else
+          st16_any(dst, all);
+      } else {
+        static_assert(NT == 2, "channel tiles per block: 2 or 4");
+        const v2i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1])};
+        if (a.vec)
+          *reinterpret_cast<v2i*>(dst) = all;
+        else
+          st8_any(dst, all);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < kLaneCh; ++c)
+        if (cb + c < a.OC) dst[c] = static_cast<uint8_t>(packed[c >> 2] >> (8 * (c & 3)));
+    }
+  }
+}
+
 template <int MODE, bool POST, int NT>
 __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a) {
   constexpr int kCrBN = 16 * NT;  // output channels per block (grid y)
@@ -293,59 +353,149 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
       const int cb = n0 + kLaneCh * pq;
       if (cb >= a.OC) continue;
       const int64_t off = opix * a.OC + cb;
-      uint32_t packed[NT];
+      runs_requant_store<MODE, POST, NT>(a, acc, off, cb, &s_mult[kLaneCh * pq], &s_bdiv[kLaneCh * pq], bmul);
+    }
+    __syncthreads();  // the staged rows are overwritten by the next tile
+  }
+}
+
+// Pointwise layers (1 x 1, stride 1, no padding, one group) over at most 256 input channels,
+// on the same per-lane weight layout: here a pixel's IC bytes *are* the run, a lane's MFMA
+// operand for pixel p and k-step ks is the 16 bytes at p * IC + 64 ks + 16 (lane / 16) of the
+// input -- straight from memory, any alignment, no staging -- and what it picks up past the
+// pixel's last channel (the next pixel's bytes) meets zero weights.  The weights of all output
+// channels sit in LDS as MFMA operands; a wave walks 16-pixel pieces of the image on its own
+// (no barrier after set-up), asks for the next piece's bytes before it works on the current
+// one's, and runs every 16 NT-channel block of the output over the piece in hand: the input is
+// read once whatever OC is.  a.tiles: the number of 16-pixel pieces.
+constexpr int kCrPointwiseLdsMax = 144 * 1024;
+__host__ __device__ inline int64_t conv_runs_pointwise_lds(int64_t OC, int64_t KS) {
+  const int64_t nt = conv_runs_tiles(OC), nblk = (OC + 16 * nt - 1) / (16 * nt);
+  return nblk * nt * KS * 1024 + nblk * 16 * nt * 12;
+}
+
+template <int MODE, bool POST, int NT>
+__global__ __launch_bounds__(kCrThreads, 3) void conv_runs_pointwise_kernel(ConvRunArgs a) {
+  constexpr int kCrBN = 16 * NT;   // output channels per channel block
+  constexpr int kLaneCh = 4 * NT;  // consecutive channels of one pixel in a lane
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int t = threadIdx.x, lane = t % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(t / kWave);
+  const int pj = lane & 15, pq = lane >> 4;
+  const int KS = a.KS;
+  const int nblk = (a.OC + kCrBN - 1) / kCrBN;
+  const int wslots = nblk * NT * KS * kWave;  // 16-byte operands
+  int* const s_acc0 = reinterpret_cast<int*>(lds + wslots * 16);
+  float* const s_mult = reinterpret_cast<float*>(s_acc0 + nblk * kCrBN);
+  float* const s_bdiv = s_mult + nblk * kCrBN;
+  const int64_t npix = static_cast<int64_t>(a.B) * a.H * a.W, x_bytes = npix * a.IC;
+  // this lane's 16 bytes of every k-step for the pixel pj of a piece (zeros where the piece has no such pixel or the
+  // k-step no such bytes; the tensor's last few bytes one by one)
+  const auto fetch = [&](int64_t piece, v4i (&xv)[kCrMaxKS]) {
+    const int64_t pix = piece * 16 + pj;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const int cl = kLaneCh * pq + 4 * nt;
-        const int raw[4] = {acc[nt][0], acc[nt][1], acc[nt][2], acc[nt][3]};
-        if constexpr (MODE == kOutAcc32) {
-          int32_t* const dst = static_cast<int32_t*>(a.y) + off + 4 * nt;
-          if (a.vec && cb + 4 * nt + 4 <= a.OC) {
-            *reinterpret_cast<v4i*>(dst) = v4i{raw[0], raw[1], raw[2], raw[3]};
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (cb + 4 * nt + r < a.OC) dst[r] = raw[r];
-          }
+    for (int ks = 0; ks < kCrMaxKS; ++ks) {
+      xv[ks] = v4i{0, 0, 0, 0};
+      const int k0 = ks * 64 + pq * 16;
+      if (ks < KS && pix < npix && k0 < a.RP) {
+        const int64_t o = pix * a.IC + k0;
+        if (o + 16 <= x_bytes) {
+          xv[ks] = ld16_any(a.x + o);
         } else {
-          const v4f mult = *reinterpret_cast<const v4f*>(&s_mult[cl]);
-          const v4f bdiv = *reinterpret_cast<const v4f*>(&s_bdiv[cl]);
-          if constexpr (POST) {
-            const int left = a.OC - (cb + 4 * nt);
-            const int nvalid = left < 0 ? 0 : (left < 4 ? left : 4);
-            const uint32_t accw =
-                a.post.accum != nullptr && nvalid > 0 ? load_accum4(a.post, off + 4 * nt, nvalid) : 0u;
-            packed[nt] = requant4_post<MODE>(raw, bdiv, bmul, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
-          } else {
-            packed[nt] = requant4<MODE>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
-          }
-        }
-      }
-      if constexpr (MODE != kOutAcc32) {
-        uint8_t* const dst = static_cast<uint8_t*>(a.y) + off;
-        if (cb + kLaneCh <= a.OC) {  // one store of 4 NT bytes; any alignment unless the host found the rows aligned
-          if constexpr (NT == 4) {
-            const v4i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1]), static_cast<int>(packed[2]),
-                             static_cast<int>(packed[3])};
-            if (a.vec)
-              *reinterpret_cast<v4i*>(dst) = all;
-            else
-              st16_any(dst, all);
-          } else {
-            const v2i all = {static_cast<int>(packed[0]), static_cast<int>(packed[1])};
-            if (a.vec)
-              *reinterpret_cast<v2i*>(dst) = all;
-            else
-              st8_any(dst, all);
-          }
-        } else {
-#pragma unroll
-          for (int c = 0; c < kLaneCh; ++c)
-            if (cb + c < a.OC) dst[c] = static_cast<uint8_t>(packed[c >> 2] >> (8 * (c & 3)));
+          uint32_t words[4] = {0, 0, 0, 0};
+          for (int b = 0; b < 16; ++b)
+            if (o + b < x_bytes) words[b >> 2] |= static_cast<uint32_t>(a.x[o + b]) << (8 * (b & 3));
+          xv[ks] = v4i{static_cast<int>(words[0]), static_cast<int>(words[1]), static_cast<int>(words[2]), static_cast<int>(words[3])};
         }
       }
     }
-    __syncthreads();  // the staged rows are overwritten by the next tile
+  };
+  // the first pieces' bytes are asked for before the weights and constants are set up: their latencies overlap
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kCrWaves;
+  int64_t piece = static_cast<int64_t>(blockIdx.x) * kCrWaves + wave;
+  // (KS == 1: pre[i] is the one k-step of the i-th piece ahead, four pieces in flight; otherwise the next piece's k-steps)
+  static_assert(kCrMaxKS == 4, "the ring of four pieces shares the registers of one piece's four k-steps");
+  v4i pre[kCrMaxKS] = {};
+  if (KS == 1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (piece + i * stride < a.tiles) {
+        v4i tmp[kCrMaxKS];
+        fetch(piece + i * stride, tmp);
+        pre[i] = tmp[0];
+      }
+  } else if (piece < a.tiles) {
+    fetch(piece, pre);
+  }
+  for (int i = t; i < wslots; i += kCrThreads) *reinterpret_cast<v4i*>(lds + i * 16) = ld16(a.w_runs + static_cast<int64_t>(i) * 16);
+  for (int n = t; n < nblk * kCrBN; n += kCrThreads) {
+    int acc0 = 0;
+    float mult = 0.f, bdiv = 0.f;
+    if (n < a.OC) {
+      acc0 = a.acc_coef * a.colsum[n];
+      if constexpr (MODE != kOutAcc32) {
+        const float atw = a.x_scale * a.w_scales[n * a.w_scale_stride];
+        mult = atw / a.out_scale;
+        bdiv = a.bias != nullptr ? bias_term(a.w_scale_stride == 0, a.bias[n], atw) : 0.f;
+      }
+    }
+    s_acc0[n] = acc0;
+    s_mult[n] = mult;
+    s_bdiv[n] = bdiv;
+  }
+  __syncthreads();
+  float bmul = 1.0f;
+  if constexpr (MODE != kOutAcc32) bmul = bias_mul(a.w_scale_stride == 0, a.x_scale * a.w_scales[0]);
+
+  // every channel block over the piece in hand (xv: its bytes, sign flip applied)
+  const auto multiply = [&](int64_t piece, const v4i (&xv)[kCrMaxKS]) {
+    const int64_t pix = piece * 16 + pj;
+    for (int cbi = 0; cbi < nblk; ++cbi) {
+      const int cl = cbi * kCrBN + kLaneCh * pq;  // this lane's first channel of the block
+      v4i acc[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = *reinterpret_cast<const v4i*>(&s_acc0[cl + 4 * nt]);
+#pragma unroll
+      for (int ks = 0; ks < kCrMaxKS; ++ks) {
+        if (ks < KS) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const v4i w = *reinterpret_cast<const v4i*>(lds + ((((cbi * NT + nt) * KS + ks) * kWave + lane) << 4));
+            acc[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, xv[ks], acc[nt], 0, 0, 0);
+          }
+        }
+      }
+      if (pix < npix && cl < a.OC)
+        runs_requant_store<MODE, POST, NT>(a, acc, pix * a.OC + cl, cl, &s_mult[cl], &s_bdiv[cl], bmul);
+    }
+  };
+  const int xo = static_cast<int>(a.x_xor);
+  const v4i flip = {xo, xo, xo, xo};
+  if (KS == 1) {
+    // At most 64 input channels: one load per piece, four pieces' loads in flight per wave.
+    while (piece < a.tiles) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (piece < a.tiles) {
+          const v4i xv[kCrMaxKS] = {pre[i] ^ flip, v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}};
+          if (piece + 4 * stride < a.tiles) {
+            v4i tmp[kCrMaxKS];
+            fetch(piece + 4 * stride, tmp);
+            pre[i] = tmp[0];
+          }
+          multiply(piece, xv);
+          piece += stride;
+        }
+      }
+    }
+    return;
+  }
+  for (; piece < a.tiles; piece += stride) {
+    v4i xv[kCrMaxKS];
+#pragma unroll
+    for (int ks = 0; ks < kCrMaxKS; ++ks) xv[ks] = pre[ks] ^ flip;
+    if (piece + stride < a.tiles) fetch(piece + stride, pre);
+    multiply(piece, xv);
   }
 }
 

@@ -160,6 +160,7 @@ struct __attribute__((packed, aligned(1))) V4iAnyAlignment {
   v4i v;
 };
 __device__ __forceinline__ void st16_any(void* p, v4i v) { reinterpret_cast<V4iAnyAlignment*>(p)->v = v; }
+__device__ __forceinline__ v4i ld16_any(const void* p) { return reinterpret_cast<const V4iAnyAlignment*>(p)->v; }
 typedef int v2i __attribute__((ext_vector_type(2)));
 struct __attribute__((packed, aligned(1))) V2iAnyAlignment {
   v2i v;
