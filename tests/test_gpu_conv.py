@@ -454,16 +454,18 @@ def test_conv_pointwise_as_linear(cabi, spec, x_signed):
     (2, 10, 10, 256, 64, 3, 1, 1, 1, 2),     # two groups of 128 -> 32
     (1, 6, 6, 48, 40, 5, 1, 2, 1, 1),        # 1200 bytes of K: 19 stages, odd: refused
     (1, 8, 8, 128, 64, 3, 1, 1, 1, 1),       # 18 stages: two groups, not four
+    (17, 14, 14, 256, 200, 3, 1, 1, 1, 1),   # 53 x 4 tiles of 64 x 64: tiles of 128 rows by themselves
 ])
 @pytest.mark.parametrize("x_signed", [False, True])
-@pytest.mark.parametrize("wave_groups", [2, 4])
-def test_conv_gemm_wave_groups(cabi, spec, x_signed, wave_groups):
-    say("conv gemm wave groups", spec, x_signed, wave_groups)
+@pytest.mark.parametrize("wave_groups,tile_rows", [(2, 0), (4, 0), (2, 128), (1, 128)],
+                         ids=["two", "four", "two-128-rows", "one-128-rows"])
+def test_conv_gemm_wave_groups(cabi, spec, x_signed, wave_groups, tile_rows):
+    say("conv gemm wave groups", spec, x_signed, wave_groups, tile_rows)
     c = _conv_case(*spec, seed=sum(spec) + 17, x_signed=x_signed, relu=x_signed)
     kbytes = spec[5] * spec[5] * spec[3] // spec[9]
     even = (-(-kbytes // 64)) % wave_groups == 0
     cabi.force_conv_path(2)
-    cabi.force_conv_tile(0, wave_groups)
+    cabi.force_conv_tile(tile_rows, wave_groups)
     try:
         if not even:
             with pytest.raises(cabi.TmqError):
