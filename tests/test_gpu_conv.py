@@ -381,6 +381,30 @@ def test_conv_pointwise_rows_from_memory(cabi, spec, x_signed):
             assert d.max() == 0, f"{np.count_nonzero(d)} of {d.size} bytes differ (max {d.max()})"
 
 
+@pytest.mark.parametrize("spec", [
+    (8, 56, 56, 24, 144, 1, 1, 0, 1, 1),     # 1568 pieces, three channel blocks: the automatic choice at size
+    (4, 112, 112, 32, 16, 1, 1, 0, 1, 1),    # 3136 pieces, two channel tiles
+    (6, 56, 56, 256, 128, 1, 1, 0, 1, 1),    # four k-steps
+    (4, 56, 56, 96, 96, 7, 1, 3, 1, 96),     # depthwise 7 x 7, whole strips and several blocks per image
+    (3, 112, 112, 32, 32, 3, 1, 1, 1, 32),   # depthwise 3 x 3
+    (2, 112, 112, 96, 96, 3, 2, 1, 1, 96),   # ... at stride 2
+    (2, 56, 56, 40, 40, 3, 1, 1, 1, 1),      # channel-padded copy, then halo tiles
+])
+def test_conv_layers_of_mobile_networks_at_size(cabi, spec):
+    """The kernels for pointwise, depthwise and off-grid layers as the library picks them at sizes where
+    every lane, strip and block of theirs has work, against the oracle."""
+    say("conv mobile layers at size", spec)
+    c = _conv_case(*spec, seed=sum(spec) + 31, x_signed=False, relu=True)
+    y, acc, _ = _run(cabi, c)
+    np.testing.assert_array_equal(
+        acc, oracle.conv2d_acc32(c["xq"], c["wq"], c["stride"], c["padding"], c["dilation"], c["groups"], c["x_zp"],
+                                 nthreads=8))
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], c["stride"],
+                         c["padding"], c["dilation"], c["groups"], c["out_scale"], c["out_zp"], relu=c["relu"],
+                         nthreads=8)
+    _check(y, want, "at size")
+
+
 def test_conv_pointwise_rows_limits(cabi):
     """Not that kernel's: a 3 x 3 kernel, a stride, padding, groups, more than 256 input channels."""
     say("conv pointwise rows limits")

@@ -847,8 +847,9 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   }
   // depthwise layers: four channels per lane on the vector ALU
   {
-    // (32-bit byte offsets into the input and the output)
+    // (32-bit byte offsets into the input and the output, also for the rows a window reaches past the image)
     const bool lanes_ok = s.taps_bytes > 0 && s.B * s.H * s.W * s.IC < (int64_t{1} << 31) &&
+                          (s.H + s.KH * s.dh + s.sh + 8) * s.W * s.IC < (int64_t{1} << 31) &&
                           s.B * s.OH * s.OW * s.OC < (int64_t{1} << (MODE == kOutAcc32 ? 29 : 31)) && aligned(d->x, 4) && aligned(out, MODE == kOutAcc32 ? 16 : 4) &&
                           (po.accum == nullptr || aligned(po.accum, 4));
     if (forced == 7 && !lanes_ok) return TMQ_ERR_UNSUPPORTED;
