@@ -947,6 +947,8 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
   xs.pad_h = static_cast<int>(s.ph); xs.pad_w = static_cast<int>(s.pw);
   xs.dil_h = static_cast<int>(s.dh); xs.dil_w = static_cast<int>(s.dw);
   xs.pad_word = 0x01010101u * static_cast<uint32_t>(static_cast<uint8_t>(d->x_zero_point));
+  xs.step_w = static_cast<int>(s.dw * s.IC - 16 * (s.ICgp / 16));
+  xs.step_h = static_cast<int>(s.dh * s.W * s.IC - s.KW * s.dw * s.IC);
 
   GemmArgs a{};
   a.M = rows;

@@ -60,6 +60,10 @@ struct XConv {
   int ic_off;        // first input channel of this group
   uint32_t pad_word; // activation zero point replicated in 4 bytes
   int kc0;           // first 16-byte k-chunk of this wave group's share of K (k-split groups), else 0
+  // byte offset gained, beyond a block's 16 bytes, when the k order wraps from a tap's last 16-channel block into the
+  // next tap (dil_w * IC - 16 icb), and on top of that from a kernel row's last tap into the next row
+  // (dil_h * W * IC - KW * dil_w * IC)
+  int step_w, step_h;
 };
 
 // Optional work between the requantisation's multiply and its rounding:
@@ -257,43 +261,48 @@ struct KCursor<XLinear> {
 template <>
 struct KCursor<XConv> {
   int kt_cur, c;
-  int kh, kw, blk;      // tap (kh, kw) and 16-channel block of the current chunk
-  int dh, dw, tapoff;   // the tap's input displacement and its byte offset
-  __device__ __forceinline__ void place(const XConv& s) {
-    dh = kh * s.dil_h;
-    dw = kw * s.dil_w;
-    tapoff = (dh * s.W + dw) * s.IC + blk * 16;
-  }
+  int kw, blk;          // tap column and 16-channel block of the current chunk
+  int dh, dw, tapoff;   // the tap's input displacement and the chunk's byte offset from the window's corner
   __device__ __forceinline__ void init(const XConv& s, int c_) {
     c = c_;
     kt_cur = 0;
     const int tap = (c_ + s.kc0) / s.icb;
     blk = c_ + s.kc0 - tap * s.icb;
-    kh = tap / s.KW;
+    const int kh = tap / s.KW;
     kw = tap - kh * s.KW;
-    place(s);
+    dh = kh * s.dil_h;
+    dw = kw * s.dil_w;
+    tapoff = (dh * s.W + dw) * s.IC + blk * 16;
+  }
+  // `n` blocks on (fewer than a tap holds: one wrap into the next tap at most), by additions only:
+  // s.step_w / s.step_h are what the offset gains at the wrap into the next tap / next kernel row
+  // beyond the blocks' own 16 bytes each.
+  __device__ __forceinline__ void advance(const XConv& s, int n) {
+    int b = blk + n, off = tapoff + 16 * n;
+    const bool wrap = b >= s.icb;
+    b -= wrap ? s.icb : 0;
+    off += wrap ? s.step_w : 0;
+    const int w = kw + (wrap ? 1 : 0), x = dw + (wrap ? s.dil_w : 0);
+    const bool row = w == s.KW;
+    kw = row ? 0 : w;
+    dw = row ? 0 : x;
+    dh += row ? s.dil_h : 0;
+    tapoff = off + (row ? s.step_h : 0);
+    blk = b;
   }
   // Advances by at most one stage per call (stages are requested in order, the
-  // last one repeatedly).  Written with selects only: a branch between the
-  // global loads would make the compiler drain all outstanding loads.
+  // last one repeatedly).  Written with selects only where lanes differ: a divergent branch
+  // between the global loads would make the compiler drain all outstanding loads.  (The
+  // branch on the layer's channel count is the same for every lane and holds no load.)
   __device__ __forceinline__ void seek(const XConv& s, int kt) {
     const bool adv = kt > kt_cur;
     kt_cur = adv ? kt_cur + 1 : kt_cur;
-    int b = blk + (adv ? kChunks : 0);
-    int w = kw, h = kh;
+    if (s.icb >= kChunks) {
+      advance(s, adv ? kChunks : 0);
+    } else {
 #pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-      const bool wrap = b >= s.icb;
-      b -= wrap ? s.icb : 0;
-      w += wrap ? 1 : 0;
-      const bool row = w == s.KW;
-      w = row ? 0 : w;
-      h += row ? 1 : 0;
+      for (int i = 0; i < kChunks; ++i) advance(s, adv ? 1 : 0);
     }
-    blk = b;
-    kw = w;
-    kh = h;
-    place(s);
   }
   // Out-of-image taps read as the activation zero point, i.e. real value 0;
   // chunks past K land on taps past the kernel window: any in-bounds address
