@@ -375,7 +375,8 @@ typedef struct tmq_conv2d_desc {
    * (16-byte aligned; contents undefined before and after the call).  With at
    * least tmq_conv2d_workspace_bytes(&geom) bytes, layers with few output pixels
    * against a long K (3 x 3 over hundreds of channels on a 14 x 14 or 7 x 7
-   * image) write their patch rows there and run as one quantized::linear over
+   * image) and pointwise layers with a stride over 512 input channels and more
+   * write their patch rows there and run as one quantized::linear over
    * them, and layers of one group whose channel count is no multiple of 16
    * under kernel rows of more than 256 bytes (3 x 3 over 40 channels) run the
    * matrix-core kernels on a copy of the input with padded channels instead of

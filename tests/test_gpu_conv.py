@@ -547,6 +547,8 @@ def test_conv_gemm_wave_groups_fused(cabi, activation, wave_groups):
     (2, 9, 9, 32, 24, 3, 2, 1, 1, 1),        # small K: pinned only
     (1, 10, 10, 16, 16, 3, 1, 2, 2, 1),      # dilation (pinned only)
     (1, 5, 5, 48, 20, 1, 1, 0, 1, 1),        # pointwise (pinned only): the patch rows are the pixels
+    (8, 14, 14, 1024, 1280, 1, 2, 0, 1, 1),  # pointwise at stride 2 over many channels: its pixels gathered, by itself
+    (1, 14, 14, 1024, 64, 1, 2, 0, 1, 1),    # ... over few pixels: halo tiles by themselves
 ])
 @pytest.mark.parametrize("x_signed", [False, True])
 def test_conv_on_patch_rows(cabi, spec, x_signed):
@@ -559,7 +561,10 @@ def test_conv_on_patch_rows(cabi, spec, x_signed):
     oh, ow = cabi.conv_out_hw(g)
     kbytes = spec[5] * spec[5] * spec[3]
     asked = cabi.lib().tmq_conv2d_workspace_bytes(g)
-    assert asked == (spec[0] * oh * ow * kbytes if kbytes >= 2048 else 0)
+    if spec[5] == 1 and spec[6] == 2:
+        assert asked == (spec[0] * oh * ow * kbytes if spec[0] == 8 else 0)
+    else:
+        assert asked == (spec[0] * oh * ow * kbytes if kbytes >= 2048 else 0)
     for path, ws in ((6, True), (-1, True), (-1, False)):
         cabi.force_conv_path(path)
         cabi.use_conv_workspace(ws)

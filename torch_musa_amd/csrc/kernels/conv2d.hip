@@ -193,8 +193,16 @@ int64_t patch_rows_bytes(const tmq_conv2d_geom& g, const ConvShape& s, bool pinn
   const int64_t rows = s.B * s.OH * s.OW;
   if (rows == 0 || rows * (s.Kp / 16) > 0x7fffffff) return 0;
   if (!pinned) {
-    if (rows > kPatchRowsMax || s.Kp < kPatchRowsMinK) return 0;
-    if (s.KH == 1 && s.KW == 1 && s.sh == 1 && s.sw == 1 && s.ph == 0 && s.pw == 0) return 0;  // (already rows)
+    const bool pointwise = s.KH == 1 && s.KW == 1 && s.ph == 0 && s.pw == 0;
+    if (pointwise && s.sh == 1 && s.sw == 1) return 0;  // (already rows)
+    if (pointwise) {
+      // A pointwise layer with a stride: its patch rows are the pixels it reads, gathered.  From 512 input
+      // channels on (batch 32: 512 -> 1024 on 28 x 28 19.5 -> 13.1 us, 1024 -> 2048 on 14 x 14 16.9 -> 12.8 us; batch 8,
+      // 1024 -> 2048: 9.9 -> 8.8 us; 256 -> 512 on 56 x 56 level at batch 32 and behind at batch 8, 8.8 against 9.4 us).
+      if (s.IC < 512 || rows * s.IC * s.OC < 500000000) return 0;
+    } else if (rows > kPatchRowsMax || s.Kp < kPatchRowsMinK) {
+      return 0;
+    }
   }
   return rows * s.Kp;
 }
@@ -348,8 +356,12 @@ bool plan_tiles(const ConvShape& s, bool forced, int forced_rows, int forced_col
   // implicit GEMM, which gathers only what it multiplies.  Everything else that
   // fits is faster here, measured over ResNet-50's layer shapes at batch 32:
   // 3x3 stride 1 and 7x7 stride 2 by 1.8x, 3x3 stride 2 by 1.2-1.7x, 1x1 stride 1
-  // by 1.05-1.8x.
-  if (!forced && s.KH * s.KW < s.sh * s.sw) return false;
+  // by 1.05-1.8x.  With few output pixels and one round of blocks the wasted pixels cost
+  // less than the implicit GEMM's long k loop on a handful of tiles (one image, 1x1 stride 2:
+  // 256 -> 512 on 56 x 56 4.6 against 5.7 us, 1024 -> 2048 on 14 x 14 5.8 against 9.4 us; eight
+  // images, 1024 -> 2048: 512 blocks, 17.6 against 9.7 us).
+  const bool wasteful = !forced && s.KH * s.KW < s.sh * s.sw;
+  if (wasteful && s.B * s.OH * s.OW > 1024) return false;
   const int64_t icb = s.ICg / 16;
   const int64_t chunks = s.KH * s.KW * icb;
   const int64_t KS = round_up(ceil_div(chunks, 2), 2);  // <= packed k-chunks / 2 (padded to 8)
@@ -415,6 +427,7 @@ bool plan_tiles(const ConvShape& s, bool forced, int forced_rows, int forced_col
       const double overlapped = simd > copy ? simd : copy;
       const double group = 3000.0 + mfma + copy + epilogue + static_cast<double>(together - 1) * overlapped;
       const double cost = static_cast<double>(ceil_div(per_cu, together)) * group;
+      if (wasteful && blocks > 256) continue;
       if (best_cost < 0 || cost < best_cost) {
         best_cost = cost;
         best->TH = static_cast<int>(TH); best->TW = static_cast<int>(TW);
