@@ -199,7 +199,8 @@ int64_t patch_rows_bytes(const tmq_conv2d_geom& g, const ConvShape& s, bool pinn
       // A pointwise layer with a stride: its patch rows are the pixels it reads, gathered.  From 512 input
       // channels on (batch 32: 512 -> 1024 on 28 x 28 19.5 -> 13.1 us, 1024 -> 2048 on 14 x 14 16.9 -> 12.8 us; batch 8,
       // 1024 -> 2048: 9.9 -> 8.8 us; 256 -> 512 on 56 x 56 level at batch 32 and behind at batch 8, 8.8 against 9.4 us).
-      if (s.IC < 512 || rows * s.IC * s.OC < 500000000) return 0;
+      // (eight images, 512 -> 1024 on 28 x 28: 9.0 against 7.9 us on the implicit GEMM)
+      if (s.IC < 512 || rows * s.IC * s.OC < (s.IC >= 1024 ? 500000000 : 2000000000)) return 0;
     } else if (rows > kPatchRowsMax || s.Kp < kPatchRowsMinK) {
       return 0;
     }
@@ -854,7 +855,10 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
     // 56 x 56 18.6 -> 15.6 us, 192 -> 32 on 28 x 28 4.7 -> 4.0 us; 128 -> 512 on 28 x 28 10.5 against 12.5 us and
     // 96 -> 576 on 14 x 14 5.8 against 11.4 us stay where they were).
     const int64_t pieces = ceil_div(s.B * s.H * s.W, 16), blocks = ceil_div(s.OC, 16 * conv_runs_tiles(s.OC));
-    const bool worth = pieces >= 1024 && (blocks <= 3 || (pieces >= 4096 && blocks <= 4));
+    // (one channel block: from 128 pieces on -- one image, 32 -> 16 channels on 112 x 112 4.3 -> 3.7 us; and whenever the
+    // channel count leaves only the byte-run kernel: one image, 24 -> 144 on 56 x 56 6.6 -> 5.0 us)
+    const bool worth = (pieces >= 1024 && (blocks <= 3 || (pieces >= 4096 && blocks <= 4))) ||
+                       (pieces >= 128 && blocks == 1) || !mfma_ok;
     if (forced == 9 || (forced < 0 && rows_ok && worth))
       return launch_conv_pointwise_rows<MODE>(d, s, po, zp_f, lo_f, hi_f, out, stream);
   }
