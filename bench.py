@@ -1226,7 +1226,7 @@ def main():
 
                 def run_():
                     for x_, y_ in zip(xs_, ys_):
-                        cabi.conv2d(x_, pw_, g_, 0.02, 128, ws_, b_, 0.05, 128, relu=True, out=y_)
+                        cabi.conv2d(x_, pw_, g_, 0.02, 0, ws_, b_, 0.05, 0, relu=True, out=y_)
 
                 us_ = graph_us(run_, nsets)
                 total_us += count * us_
@@ -1250,8 +1250,9 @@ def main():
             secondary[f"conv2d_relu_resnet50_stack_b{batch_}"] = {
                 "layers": layers_, "total_us": round(tot_, 1), "per_layer_us": round(tot_ / layers_, 2),
                 "images_per_s_convs_only": round(batch_ / (tot_ * 1e-6), 1), "shapes": rows_,
-                "method": "each distinct shape timed alone through tmq_conv2d (with ReLU) in a replayed HIP graph over "
-                          "rotating inputs, times its count; 224 x 224 images, NHWC"}
+                "method": "each distinct shape timed alone through tmq_conv2d (with ReLU; input and output zero point 0, "
+                          "as tensors behind a ReLU have it) in a replayed HIP graph over rotating inputs, times its "
+                          "count; 224 x 224 images, NHWC"}
 
         # ... and of a MobileNetV2 (52 layers, 30 distinct shapes: a 3-channel first layer, depthwise 3 x 3 layers
         # at both strides, pointwise layers whose channel counts -- 24, 144, 160, 320 -- are mostly off the 64 grid)

@@ -257,11 +257,11 @@ CONV_CONFIGS = [
 
 @pytest.mark.parametrize("cfg", CONV_CONFIGS, ids=lambda c: f"{c['shape']}-{c['oc']}-k{c['k']}g{c['g']}")
 @pytest.mark.parametrize("per_channel", [False, True])
-@pytest.mark.parametrize("channels_last_input", [False, True])
-def test_qconv2d_matches_cpu_op(cfg, per_channel, channels_last_input):
+@pytest.mark.parametrize("channels_last_input,out_zp", [(False, 90), (True, 90), (True, 0)])
+def test_qconv2d_matches_cpu_op(cfg, per_channel, channels_last_input, out_zp):
     """Configurations of the reference's test_qconv2d, through nnq.Conv2d with
     weights set from outside (test_quantized_conv.py:83-150), against the CPU op."""
-    say("aten qconv", cfg, per_channel, channels_last_input)
+    say("aten qconv", cfg, per_channel, channels_last_input, out_zp)
     torch.manual_seed(41)
     ic = cfg["shape"][1]
     x = torch.randn(cfg["shape"])
@@ -280,7 +280,7 @@ def test_qconv2d_matches_cpu_op(cfg, per_channel, channels_last_input):
     for dev in ("cpu", "cuda"):
         m = cls(ic, cfg["oc"], cfg["k"], cfg["s"], cfg["p"], cfg["d"], cfg["g"], cfg["bias"])
         m.set_weight_bias(wq.to(dev), None if b is None else b.to(dev))
-        m.scale, m.zero_point = 0.25, 90
+        m.scale, m.zero_point = 0.25, out_zp
         mods.append(m)
     ref = mods[0](xq)
     got = mods[1](xq.cuda())
@@ -291,7 +291,7 @@ def test_qconv2d_matches_cpu_op(cfg, per_channel, channels_last_input):
         # 7056 outputs on a CPU-only machine.  The float pipeline judges instead, as in the reference's own tests
         # (test_quantized_conv.py:83-150): quantize(conv(dequantized operands)) within one LSB.
         rf = torch.nn.functional.conv2d(xq.dequantize(), wq.dequantize(), b, cfg["s"], cfg["p"], cfg["d"], cfg["g"])
-        ref = torch.quantize_per_tensor(torch.relu(rf) if cfg["relu"] else rf, 0.25, 90, torch.quint8)
+        ref = torch.quantize_per_tensor(torch.relu(rf) if cfg["relu"] else rf, 0.25, out_zp, torch.quint8)
     assert_q_equal(got, ref, abs_diff=LSB_TOL)
     n_off = (got.int_repr().cpu() != ref.int_repr()).sum().item()
     if cfg["g"] == ic and per_channel:

@@ -405,6 +405,46 @@ def test_conv_layers_of_mobile_networks_at_size(cabi, spec):
     _check(y, want, "at size")
 
 
+@pytest.mark.parametrize("spec,path", [
+    ((2, 20, 20, 64, 64, 3, 1, 1, 1, 1), 1), ((2, 20, 20, 64, 64, 3, 1, 1, 1, 1), 2), ((1, 14, 14, 256, 64, 3, 1, 1, 1, 1), 2),
+    ((2, 19, 19, 3, 40, 7, 2, 3, 1, 1), 4), ((2, 14, 14, 24, 144, 1, 1, 0, 1, 1), 9), ((2, 14, 14, 256, 64, 1, 1, 0, 1, 1), 5),
+    ((2, 19, 23, 72, 72, 3, 1, 1, 1, 72), 7), ((2, 15, 15, 96, 96, 7, 1, 3, 1, 96), 7), ((1, 9, 9, 40, 40, 3, 2, 1, 1, 40), 3),
+    ((2, 14, 14, 40, 40, 3, 1, 1, 1, 1), 8), ((1, 7, 7, 512, 72, 3, 1, 1, 1, 1), 6), ((2, 12, 12, 96, 48, 3, 1, 1, 1, 4), -1),
+])
+@pytest.mark.parametrize("relu", [False, True])
+def test_conv_unsigned_output_with_zero_point_0(cabi, spec, path, relu):
+    """quint8 output with zero point 0 (what follows a ReLU) through every kernel family, plain and fused: the
+    packing conversion alone rounds and saturates there."""
+    say("conv zero point 0", spec, path, relu)
+    c = _conv_case(*spec, seed=sum(spec) + 37, x_signed=False, relu=relu)
+    c["out_zp"] = 0
+    c["out_scale"] /= 3     # (255 at two standard deviations of the sums: the upper bound is met too)
+    want = oracle.conv2d(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"], c["stride"],
+                         c["padding"], c["dilation"], c["groups"], c["out_scale"], 0, relu=relu, nthreads=8)
+    assert 0.25 < np.mean(want == 0) < 0.75 and np.any(want == 255)
+    cabi.force_conv_path(path)
+    try:
+        y, _, _ = _run(cabi, c)
+        _check(y, want, f"path {path}")
+        if path not in (5, 6):   # (the linear kernels take no residual)
+            rng = np.random.default_rng(3)
+            for activation in ("relu", "silu"):
+                f = dict(c, accq=rng.integers(0, 256, want.shape, dtype=np.uint8), acc_scale=0.35, acc_zp=110,
+                         activation=activation, signed=False, relu=False)
+                want_f = oracle.conv2d_fused(f["xq"], f["x_scale"], f["x_zp"], f["wq"], f["w_scales"], f["bias"],
+                                             f["stride"], f["padding"], f["dilation"], f["groups"], f["out_scale"], 0,
+                                             accum=f["accq"], accum_scale=0.35, accum_zp=110, activation=activation,
+                                             out_signed=False, nthreads=8)
+                yf = _run_fused(cabi, f)
+                d = np.abs(yf.astype(np.int32) - want_f.astype(np.int32))
+                if activation == "silu":
+                    assert d.max() <= LSB_TOL and np.count_nonzero(d) <= max(2, 0.001 * d.size), (d.max(), np.count_nonzero(d))
+                else:
+                    assert d.max() == 0, f"{np.count_nonzero(d)} of {d.size} bytes differ (max {d.max()})"
+    finally:
+        cabi.force_conv_path(-1)
+
+
 def test_conv_pointwise_rows_limits(cabi):
     """Not that kernel's: a 3 x 3 kernel, a stride, padding, groups, more than 256 input channels."""
     say("conv pointwise rows limits")

@@ -679,6 +679,26 @@ def test_linear_dynamic_prefill_sized(cabi):
     np.testing.assert_array_equal(y, want)
 
 
+@pytest.mark.parametrize("cfg,shape", [(-1, (130, 260, 448)), (0, (130, 260, 448)), (2, (300, 520, 448)), (7, (300, 520, 448)),
+                                       (9, (40, 70, 784)), (17, (270, 300, 400)), (20, (1300, 1100, 704)), (21, (64, 1040, 1168)),
+                                       (24, (40, 70, 784)), (25, (64, 1040, 1168)), (26, (64, 1040, 1168)), (27, (130, 260, 1168)),
+                                       (8, (3, 300, 448)), (28, (16, 300, 448)), (-1, (1, 4096, 256)), (-1, (256, 300, 4608))])
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_unsigned_output_with_zero_point_0(cabi, cfg, shape, relu, per_channel):
+    """quint8 output with zero point 0 (what follows a ReLU): the packing conversion alone rounds and
+    saturates in the kernels; half of the sums are negative and must come out as 0, ties go to even."""
+    say("zero point 0", cfg, shape, relu, per_channel)
+    c = _tile_case(*shape, seed=cfg * 7 + shape[1], relu=relu, per_channel=per_channel)
+    c["out_zp"] = 0
+    c["out_scale"] /= 3     # (255 at two standard deviations of the sums: the upper bound is met too)
+    y, _, _ = _run(cabi, c, cfg)
+    want = oracle.linear(c["xq"], c["x_scale"], c["x_zp"], c["wq"], c["w_scales"], c["bias"],
+                         c["out_scale"], 0, relu=relu)
+    assert 0.3 < np.mean(want == 0) < 0.7 and np.any(want == 255)
+    _check(y, want, f"cfg {cfg}")
+
+
 def _random_shapes(seed, count):
     rng = np.random.default_rng(seed)
     out = []
