@@ -351,6 +351,12 @@ __device__ __forceinline__ bool requant_plain_u8(float zp_f, float lo_f, float h
 template <int MODE, bool CLAMP = true>
 __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, float bmul, v4f mult, float zp_f,
                                              float lo_f, float hi_f) {
+  // Signed bytes are the unsigned ones of the same sequence with zero point and bounds 128 higher, sign bits flipped
+  // at the end (clamp(r + zp, lo, hi) = clamp(r + zp + 128, lo + 128, hi + 128) - 128, every term a small integer in
+  // fp32): the packing conversion serves them too, where a signed byte took a float-to-int conversion, a mask, a shift
+  // and an or.
+  if constexpr (MODE == kOutS8)
+    return requant4<kOutU8, CLAMP>(raw, bdiv, bmul, mult, zp_f + 128.f, lo_f + 128.f, hi_f + 128.f) ^ 0x80808080u;
   uint32_t packed = 0;
   if constexpr (MODE == kOutU8) {
     if (requant_plain_u8(zp_f, lo_f, hi_f)) {
@@ -397,6 +403,9 @@ template <int MODE, int POST = 0>
 __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv, float bmul, v4f mult,
                                                   const PostOps& p, uint32_t accw, float zp_f,
                                                   float lo_f, float hi_f) {
+  if constexpr (MODE == kOutS8)  // (see requant4)
+    return requant4_post<kOutU8, POST>(raw, bdiv, bmul, mult, p, accw, zp_f + 128.f, lo_f + 128.f, hi_f + 128.f) ^
+           0x80808080u;
   uint32_t packed = 0;
   // The residual bytes are taken as unsigned values (one conversion instruction
   // per byte): a signed byte s equals (s ^ 0x80) - 128, so the word is flipped
