@@ -49,13 +49,26 @@ __device__ __forceinline__ int quantize_one(float x, float inv, float zp_f) {
   return static_cast<int>(r);
 }
 
+// Four values into one word.  v_cvt_pk_u8_f32 rounds to nearest even, saturates to [0, 255] (NaN -> 0,
+// as the clamp of quantize_one has it) and writes its byte into the word: it stands for the clamp, the
+// conversion and the packing -- and, where product and zero point are rounded together, for the rounding
+// as well.  Signed bytes are the unsigned ones for a zero point 128 higher with the sign bits flipped.
 template <bool SIGNED, bool FUSED = false>
 __device__ __forceinline__ uint32_t quantize_four(v4f v, float inv, float zp_f) {
-  uint32_t a = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.x, inv, zp_f)) & 0xffu;
-  uint32_t b = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.y, inv, zp_f)) & 0xffu;
-  uint32_t c = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.z, inv, zp_f)) & 0xffu;
-  uint32_t d = static_cast<uint32_t>(quantize_one<SIGNED, FUSED>(v.w, inv, zp_f)) & 0xffu;
-  return a | (b << 8) | (c << 16) | (d << 24);
+  const float zp_u = SIGNED ? zp_f + 128.f : zp_f;
+  uint32_t packed = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float r;
+    if constexpr (FUSED && SIGNED)  // (the one rounding of product and zero point is that of the signed zero point)
+      r = __builtin_rintf(__builtin_fmaf(v[j], inv, zp_f)) + 128.f;
+    else if constexpr (FUSED)
+      r = __builtin_fmaf(v[j], inv, zp_u);
+    else
+      r = __builtin_rintf(v[j] * inv) + zp_u;
+    packed = __builtin_amdgcn_cvt_pk_u8_f32(r, j, packed);
+  }
+  return SIGNED ? packed ^ 0x80808080u : packed;
 }
 
 template <bool SIGNED>
@@ -64,13 +77,18 @@ __device__ __forceinline__ float dequantize_one(uint32_t byte, int zp, float sca
   return scale * static_cast<float>(v - zp);
 }
 
+// Four bytes of one word.  Byte to float is one instruction (v_cvt_f32_ubyte0..3); the zero point is
+// subtracted in fp32, where both terms are small integers and the difference is the exact float(q - zp);
+// signed bytes are read as unsigned with the sign bits flipped, against a zero point 128 higher.
 template <bool SIGNED>
 __device__ __forceinline__ v4f dequantize_four(uint32_t w, int zp, float scale) {
+  const uint32_t u = SIGNED ? w ^ 0x80808080u : w;
+  const float zp_f = static_cast<float>(SIGNED ? zp + 128 : zp);
   v4f r;
-  r.x = dequantize_one<SIGNED>(w & 0xffu, zp, scale);
-  r.y = dequantize_one<SIGNED>((w >> 8) & 0xffu, zp, scale);
-  r.z = dequantize_one<SIGNED>((w >> 16) & 0xffu, zp, scale);
-  r.w = dequantize_one<SIGNED>(w >> 24, zp, scale);
+  r.x = scale * (static_cast<float>(u & 0xffu) - zp_f);
+  r.y = scale * (static_cast<float>((u >> 8) & 0xffu) - zp_f);
+  r.z = scale * (static_cast<float>((u >> 16) & 0xffu) - zp_f);
+  r.w = scale * (static_cast<float>(u >> 24) - zp_f);
   return r;
 }
 
