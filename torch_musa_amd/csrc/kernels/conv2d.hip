@@ -490,6 +490,14 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
   }
 }
 
+// Whether the packing conversion alone requantises this call's outputs (requant_plain_u8 of gemm_i8_core.h): zero
+// point 0 and no bounds inside [0, 255] for unsigned bytes, the same 128 lower for signed ones.
+template <int MODE>
+bool plain_bytes(float zp_f, float lo_f, float hi_f) {
+  const float shift = MODE == kOutS8 ? 128.f : 0.f;
+  return requant_plain_u8(zp_f + shift, lo_f + shift, hi_f + shift);
+}
+
 // Tile shape and LDS use of the few-channel kernel (conv_runs.h) for one problem; false
 // when the kernel does not take it: groups, dilation, kernel rows of more than 256 padded bytes.
 struct RunPlan {
@@ -564,14 +572,16 @@ int launch_conv_runs(const tmq_conv2d_desc* d, const ConvShape& s, const RunPlan
   // three blocks per CU (their registers), each with its weights in registers for every tile it walks
   const int64_t bx = a.tiles < 768 ? a.tiles : 768;  // (plan_runs: kSlots)
   const dim3 grid(static_cast<unsigned>(bx), static_cast<unsigned>(by)), block(kCrThreads);
-  const auto launch = [&](auto post_tag, auto nt_tag) {
-    conv_runs_kernel<MODE, decltype(post_tag)::value, decltype(nt_tag)::value><<<grid, block, p.lds, stream>>>(a);
+  const auto launch = [&](auto post_tag, auto nt_tag, auto plain_tag) {
+    conv_runs_kernel<MODE, decltype(post_tag)::value, decltype(nt_tag)::value, decltype(plain_tag)::value>
+        <<<grid, block, p.lds, stream>>>(a);
   };
   const auto launch_tiles = [&](auto nt_tag) {
     if constexpr (MODE != kOutAcc32) {
-      if (po.any()) return launch(std::true_type{}, nt_tag);
+      if (po.any()) return launch(std::true_type{}, nt_tag, std::false_type{});
+      if (plain_bytes<MODE>(zp_f, lo_f, hi_f)) return launch(std::false_type{}, nt_tag, std::true_type{});
     }
-    launch(std::false_type{}, nt_tag);
+    launch(std::false_type{}, nt_tag, std::false_type{});
   };
   if (nt == 2)
     launch_tiles(std::integral_constant<int, 2>{});
@@ -623,8 +633,9 @@ int launch_conv_pointwise_rows(const tmq_conv2d_desc* d, const ConvShape& s, con
   per_cu = per_cu < 1 ? 1 : per_cu > by_registers ? by_registers : per_cu;
   const int64_t want = ceil_div(pieces, kCrWaves), cap = 256 * per_cu;
   const dim3 grid(static_cast<unsigned>(want < cap ? want : cap)), block(kCrThreads);
-  const auto launch = [&](auto post_tag, auto nt_tag) {
-    auto* const kernel = conv_runs_pointwise_kernel<MODE, decltype(post_tag)::value, decltype(nt_tag)::value>;
+  const auto launch = [&](auto post_tag, auto nt_tag, auto plain_tag) {
+    auto* const kernel = conv_runs_pointwise_kernel<MODE, decltype(post_tag)::value, decltype(nt_tag)::value,
+                                                    decltype(plain_tag)::value>;
     // the kernel's LDS allowance is a per-device attribute: set once per device (and kernel)
     static std::atomic<uint64_t> done{0};
     const int dev = current_device();
@@ -640,9 +651,10 @@ int launch_conv_pointwise_rows(const tmq_conv2d_desc* d, const ConvShape& s, con
   };
   const auto launch_tiles = [&](auto nt_tag) {
     if constexpr (MODE != kOutAcc32) {
-      if (po.any()) return launch(std::true_type{}, nt_tag);
+      if (po.any()) return launch(std::true_type{}, nt_tag, std::false_type{});
+      if (plain_bytes<MODE>(zp_f, lo_f, hi_f)) return launch(std::false_type{}, nt_tag, std::true_type{});
     }
-    return launch(std::false_type{}, nt_tag);
+    return launch(std::false_type{}, nt_tag, std::false_type{});
   };
   const bool ok = nt == 2 ? launch_tiles(std::integral_constant<int, 2>{}) : launch_tiles(std::integral_constant<int, 4>{});
   return ok ? launch_status() : TMQ_ERR_LAUNCH;

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kDwThreads, KS == 7 && !POST ? 3 : 1) void conv_dep
         const uint32_t accw = a.post.accum != nullptr ? *reinterpret_cast<const uint32_t*>(a.post.accum + yoff) : 0u;
         packed = requant4_post<MODE>(acc, bdiv, bmul, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
       } else {
-        packed = requant4<MODE>(acc, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+        packed = requant4<MODE, true, 2>(acc, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);  // (tested here: 11.8 -> 10.8 us where it holds, level where not)
       }
       *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(a.y) + yoff) = packed;
     }

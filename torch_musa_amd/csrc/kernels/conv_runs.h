@@ -93,8 +93,9 @@ __device__ __forceinline__ v4i conv_runs_slot(const int8_t* __restrict__ w, int6
 
 // Requantise (or pass on) the 4 NT consecutive channels cb ... of one pixel that a lane holds after the
 // MFMAs of its NT channel tiles, and store them at element offset `off` of the output: one store of 4 NT
-// bytes where all the channels exist.  mult / bdiv: the constants of channel cb onwards.
-template <int MODE, bool POST, int NT>
+// bytes where all the channels exist.  mult / bdiv: the constants of channel cb onwards.  PLAIN: the host found
+// requant_plain_u8 to hold (zero point 0 for unsigned bytes, -128 for signed ones, no bounds inside the range).
+template <int MODE, bool POST, int NT, bool PLAIN = false>
 __device__ __forceinline__ void runs_requant_store(const ConvRunArgs& a, const v4i (&acc)[NT], int64_t off, int cb,
                                                    const float* mult_cb, const float* bdiv_cb, float bmul) {
   constexpr int kLaneCh = 4 * NT;
@@ -121,7 +122,7 @@ __device__ __forceinline__ void runs_requant_store(const ConvRunArgs& a, const v
             a.post.accum != nullptr && nvalid > 0 ? load_accum4(a.post, off + 4 * nt, nvalid) : 0u;
         packed[nt] = requant4_post<MODE>(raw, bdiv, bmul, mult, a.post, accw, a.zp_f, a.lo_f, a.hi_f);
       } else {
-        packed[nt] = requant4<MODE>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+        packed[nt] = requant4<MODE, true, PLAIN ? 1 : 0>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
       }
     }
   }
@@ -151,7 +152,7 @@ __device__ __forceinline__ void runs_requant_store(const ConvRunArgs& a, const v
   }
 }
 
-template <int MODE, bool POST, int NT>
+template <int MODE, bool POST, int NT, bool PLAIN = false>
 __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a) {
   constexpr int kCrBN = 16 * NT;  // output channels per block (grid y)
   constexpr int kLaneCh = 4 * NT; // consecutive channels of one pixel in a lane
@@ -353,7 +354,7 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_kernel(ConvRunArgs a)
       const int cb = n0 + kLaneCh * pq;
       if (cb >= a.OC) continue;
       const int64_t off = opix * a.OC + cb;
-      runs_requant_store<MODE, POST, NT>(a, acc, off, cb, &s_mult[kLaneCh * pq], &s_bdiv[kLaneCh * pq], bmul);
+      runs_requant_store<MODE, POST, NT, PLAIN>(a, acc, off, cb, &s_mult[kLaneCh * pq], &s_bdiv[kLaneCh * pq], bmul);
     }
     __syncthreads();  // the staged rows are overwritten by the next tile
   }
@@ -374,7 +375,7 @@ __host__ __device__ inline int64_t conv_runs_pointwise_lds(int64_t OC, int64_t K
   return nblk * nt * KS * 1024 + nblk * 16 * nt * 12;
 }
 
-template <int MODE, bool POST, int NT>
+template <int MODE, bool POST, int NT, bool PLAIN = false>
 __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_pointwise_kernel(ConvRunArgs a) {
   constexpr int kCrBN = 16 * NT;   // output channels per channel block
   constexpr int kLaneCh = 4 * NT;  // consecutive channels of one pixel in a lane
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(kCrThreads, 3) void conv_runs_pointwise_kernel(Conv
         }
       }
       if (pix < npix && cl < a.OC)
-        runs_requant_store<MODE, POST, NT>(a, acc, pix * a.OC + cl, cl, &s_mult[cl], &s_bdiv[cl], bmul);
+        runs_requant_store<MODE, POST, NT, PLAIN>(a, acc, pix * a.OC + cl, cl, &s_mult[cl], &s_bdiv[cl], bmul);
     }
   };
   const int xo = static_cast<int>(a.x_xor);

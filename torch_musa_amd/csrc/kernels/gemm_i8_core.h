@@ -342,13 +342,16 @@ __host__ __device__ __forceinline__ float bias_mul(bool per_tensor, float atw) {
 // and no bounds inside [0, 255]: v_cvt_pk_u8_f32 itself rounds to nearest even and saturates, so it
 // stands for rint, + zero point, clamp and pack at once -- the same byte for every input (checked on
 // the device against nearbyintf + clamp over a million values between -2 and 258 and the special
-// ones), four vector instructions per value for seven.  The test is on kernel arguments: one scalar
-// branch per call.
-__device__ __forceinline__ bool requant_plain_u8(float zp_f, float lo_f, float hi_f) {
-  return zp_f == 0.f && lo_f <= 0.f && hi_f >= 255.f;
+// ones), four vector instructions per value for seven.  PLAIN says who decides: 0 never (the kernels
+// bound by the matrix pipe or by latencies, where a second epilogue in the code only costs), 1 the
+// host has checked requant_plain_u8 and launched the variant, 2 the kernel tests it per call (a branch
+// on kernel arguments; their bit patterns are compared as integers, which the scalar unit can do).
+__host__ __device__ __forceinline__ bool requant_plain_u8(float zp_f, float lo_f, float hi_f) {
+  return __builtin_bit_cast(int, zp_f) == 0 && __builtin_bit_cast(int, lo_f) <= 0 &&
+         __builtin_bit_cast(int, hi_f) >= 0x437f0000;
 }
 
-template <int MODE, bool CLAMP = true>
+template <int MODE, bool CLAMP = true, int PLAIN = 0>
 __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, float bmul, v4f mult, float zp_f,
                                              float lo_f, float hi_f) {
   // Signed bytes are the unsigned ones of the same sequence with zero point and bounds 128 higher, sign bits flipped
@@ -356,10 +359,10 @@ __device__ __forceinline__ uint32_t requant4(const int (&raw)[4], v4f bdiv, floa
   // fp32): the packing conversion serves them too, where a signed byte took a float-to-int conversion, a mask, a shift
   // and an or.
   if constexpr (MODE == kOutS8)
-    return requant4<kOutU8, CLAMP>(raw, bdiv, bmul, mult, zp_f + 128.f, lo_f + 128.f, hi_f + 128.f) ^ 0x80808080u;
+    return requant4<kOutU8, CLAMP, PLAIN>(raw, bdiv, bmul, mult, zp_f + 128.f, lo_f + 128.f, hi_f + 128.f) ^ 0x80808080u;
   uint32_t packed = 0;
-  if constexpr (MODE == kOutU8) {
-    if (requant_plain_u8(zp_f, lo_f, hi_f)) {
+  if constexpr (MODE == kOutU8 && PLAIN != 0) {
+    if (PLAIN == 1 || requant_plain_u8(zp_f, lo_f, hi_f)) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float v = __builtin_fmaf(bdiv[j], bmul, static_cast<float>(raw[j]));
@@ -424,12 +427,6 @@ __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv,
       t = t + a;
     }
     if (POST == 2 || (POST == 0 && p.silu)) t = silu_in_output_units(t, p.silu_c, p.silu_c_tail);
-    if constexpr (MODE == kOutU8) {
-      if (requant_plain_u8(zp_f, lo_f, hi_f)) {  // (see requant4)
-        packed = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed);
-        continue;
-      }
-    }
     float r = __builtin_rintf(t) + zp_f;
     r = __builtin_amdgcn_fmed3f(r, lo_f, hi_f);
     if constexpr (MODE == kOutU8) {
