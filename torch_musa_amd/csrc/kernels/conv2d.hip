@@ -464,6 +464,14 @@ int launch_conv_tiles_variant(const ConvShape& s, const TilePlan& p, const ConvT
   return launch_status();
 }
 
+// Whether the packing conversion alone requantises this call's outputs (requant_plain_u8 of gemm_i8_core.h): zero
+// point 0 and no bounds inside [0, 255] for unsigned bytes, the same 128 lower for signed ones.
+template <int MODE>
+bool plain_bytes(float zp_f, float lo_f, float hi_f) {
+  const float shift = MODE == kOutS8 ? 128.f : 0.f;
+  return requant_plain_u8(zp_f + shift, lo_f + shift, hi_f + shift);
+}
+
 // Which epilogue the launch needs (see conv_tile_kernel) is known on the host.
 template <int MODE>
 int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs& a, hipStream_t stream) {
@@ -476,6 +484,7 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
     const bool vec = (a.OC & 15) == 0 && (a.OCg & 15) == 0 && aligned16;
     const int kind = a.post.silu ? 3
                      : a.post.accum != nullptr ? 0
+                     : plain_bytes<MODE>(a.zp_f, a.lo_f, a.hi_f) ? 4
                      : ((MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f) ? 2 : 1);
     switch (kind * 2 + (vec ? 1 : 0)) {
       case 0: return launch_conv_tiles_variant<MODE, 0, false>(s, p, a, stream);
@@ -485,17 +494,11 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
       case 4: return launch_conv_tiles_variant<MODE, 2, false>(s, p, a, stream);
       case 5: return launch_conv_tiles_variant<MODE, 2, true>(s, p, a, stream);
       case 6: return launch_conv_tiles_variant<MODE, 3, false>(s, p, a, stream);
-      default: return launch_conv_tiles_variant<MODE, 3, true>(s, p, a, stream);
+      case 7: return launch_conv_tiles_variant<MODE, 3, true>(s, p, a, stream);
+      case 8: return launch_conv_tiles_variant<MODE, 4, false>(s, p, a, stream);
+      default: return launch_conv_tiles_variant<MODE, 4, true>(s, p, a, stream);
     }
   }
-}
-
-// Whether the packing conversion alone requantises this call's outputs (requant_plain_u8 of gemm_i8_core.h): zero
-// point 0 and no bounds inside [0, 255] for unsigned bytes, the same 128 lower for signed ones.
-template <int MODE>
-bool plain_bytes(float zp_f, float lo_f, float hi_f) {
-  const float shift = MODE == kOutS8 ? 128.f : 0.f;
-  return requant_plain_u8(zp_f + shift, lo_f + shift, hi_f + shift);
 }
 
 // Tile shape and LDS use of the few-channel kernel (conv_runs.h) for one problem; false

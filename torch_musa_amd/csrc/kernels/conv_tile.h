@@ -76,7 +76,8 @@ __device__ __forceinline__ uint32_t small_div(uint32_t n, uint32_t d, float rcp)
 
 // KIND selects the requantisation compiled in: 0 a residual and no SiLU, 3 SiLU
 // (with a residual if there is one), 1 plain with clamp, 2 plain for unsigned
-// output without ReLU (the saturating pack conversion is the clamp).  VEC: output rows take aligned 16-byte (int32 mode:
+// output without ReLU (the saturating pack conversion is the clamp), 4 plain for bytes with zero point 0 (-128 for
+// signed ones) and no bounds inside the range (the pack conversion is rounding, zero point and clamp).  VEC: output rows take aligned 16-byte (int32 mode:
 // 4-channel) stores.  One variant per launch keeps the straight-line code that
 // every wave runs exactly once small: the kernel with all variants inside was
 // five times longer and spent a quarter of its time fetching instructions.
@@ -389,7 +390,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
                 q4 = requant4_post<MODE, KIND == 0 ? 1 : 2>(raw, bdiv, bmul, mult, a.post, accw[tm][tn * 4 + gq],
                                                             a.zp_f, a.lo_f, a.hi_f);
               else
-                q4 = requant4<MODE, KIND == 1>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
+                q4 = requant4<MODE, KIND == 1, KIND == 4 ? 1 : 0>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);
               *reinterpret_cast<uint32_t*>(sT + li * kCtTPitch + nl) = q4;
             }
         }
