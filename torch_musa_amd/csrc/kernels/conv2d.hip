@@ -804,7 +804,8 @@ int run_conv(const tmq_conv2d_desc* d, const tmq_conv2d_post* post, void* out, h
     // 56 x 56 at batch 32 35.9 -> 25.8 us, 512 -> 512 on 28 x 28 25.0 -> 16.1 us, 128 -> 512 13.7 -> 11.6 us; fewer
     // channels on either side stay with the tiles: 256 -> 64 on 56 x 56 11.7 against 19.9 us, 96 -> 576 on
     // 28 x 28 14.3 against 18.0 us)
-    const bool wide = s.IC >= 128 && s.OC >= 256 && rows * s.IC * s.OC >= 1000000000;
+    // (a detection head's 255 channels count as wide: 128 -> 255 on 80 x 80 at batch 8 18.0 -> 15.2 us)
+    const bool wide = s.IC >= 128 && s.OC >= 224 && rows * s.IC * s.OC >= 1000000000;
     if (forced == 5 || (forced < 0 && pointwise && (rows <= kPointwiseAsLinearRows || wide))) {
       return run_as_linear(d, rows, s.OC, s.IC, d->x, relu, out, stream);
     }
