@@ -1078,7 +1078,14 @@ LinearChoice choose_linear(const LinearQuery& q, int forced) {
     // against 31.0 us; N = 11008, K = 4096: 20.2 against 21.2 us)
     const int cfg_half =
         nblk(128, 64) <= 256 && (nblk(128, 64) > nblk(64, 128) || (M <= 96 && nblk(128, 64) == nblk(64, 128))) ? 22 : 23;
-    if (t128x256 > 256 && rows_used(256))
+    // Many rows against a short K are bound by the epilogue, and 256-channel tiles requantise the padding behind
+    // N as well: 128 x 128 tiles where those pad a quarter less (M = 100352 pixels of a 56 x 56 feature map at batch
+    // 32: N = 384, K = 96: 35.1 -> 27 us; N = 96, K = 384: 20.9 -> 15.7 us; N = 512, K = 128 has nothing to gain and
+    // stays: 10.4 against 12.5 us).
+    const bool padding_bound = K <= 512 && round_up(N, 256) * 4 >= round_up(N, 128) * 5;
+    if (t128x256 > 256 && rows_used(256) && padding_bound)
+      cfg = 7;
+    else if (t128x256 > 256 && rows_used(256))
       cfg = t256 > 256 && t256 <= 400 ? 17 : 6;  // 6: 8 waves of 128x64, operands copied straight into LDS
     else if (t128x256 >= 160 && rows_used(128))
       // (barely more than half a round of them, against a long K: 128x128 tiles, at most 320,
