@@ -31,7 +31,7 @@
 namespace tmq {
 
 constexpr int kDwThreads = 256;
-constexpr int kDwStripMax = 8;  // output rows per lane, at most
+constexpr int kDwStripMax = 8;  // output rows per lane under 3 x 3 windows, at most (the host gives larger windows up to 14)
 
 struct DepthwiseArgs {
   const uint8_t* x;        // NHWC, less than 2^31 bytes
