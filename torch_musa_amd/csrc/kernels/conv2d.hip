@@ -483,7 +483,7 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
   } else {
     const bool vec = (a.OC & 15) == 0 && (a.OCg & 15) == 0 && aligned16;
     const int kind = a.post.silu ? 3
-                     : a.post.accum != nullptr ? 0
+                     : a.post.accum != nullptr ? (plain_bytes<MODE>(a.zp_f, a.lo_f, a.hi_f) ? 5 : 0)
                      : plain_bytes<MODE>(a.zp_f, a.lo_f, a.hi_f) ? 4
                      : ((MODE == kOutU8 && a.lo_f <= 0.f && a.hi_f >= 255.f) ? 2 : 1);
     switch (kind * 2 + (vec ? 1 : 0)) {
@@ -496,7 +496,9 @@ int launch_conv_tiles(const ConvShape& s, const TilePlan& p, const ConvTileArgs&
       case 6: return launch_conv_tiles_variant<MODE, 3, false>(s, p, a, stream);
       case 7: return launch_conv_tiles_variant<MODE, 3, true>(s, p, a, stream);
       case 8: return launch_conv_tiles_variant<MODE, 4, false>(s, p, a, stream);
-      default: return launch_conv_tiles_variant<MODE, 4, true>(s, p, a, stream);
+      case 9: return launch_conv_tiles_variant<MODE, 4, true>(s, p, a, stream);
+      case 10: return launch_conv_tiles_variant<MODE, 5, false>(s, p, a, stream);
+      default: return launch_conv_tiles_variant<MODE, 5, true>(s, p, a, stream);
     }
   }
 }

@@ -77,13 +77,14 @@ __device__ __forceinline__ uint32_t small_div(uint32_t n, uint32_t d, float rcp)
 // KIND selects the requantisation compiled in: 0 a residual and no SiLU, 3 SiLU
 // (with a residual if there is one), 1 plain with clamp, 2 plain for unsigned
 // output without ReLU (the saturating pack conversion is the clamp), 4 plain for bytes with zero point 0 (-128 for
-// signed ones) and no bounds inside the range (the pack conversion is rounding, zero point and clamp).  VEC: output rows take aligned 16-byte (int32 mode:
+// signed ones) and no bounds inside the range (the pack conversion is rounding, zero point and clamp), 5 a residual
+// and no SiLU into such bytes.  VEC: output rows take aligned 16-byte (int32 mode:
 // 4-channel) stores.  One variant per launch keeps the straight-line code that
 // every wave runs exactly once small: the kernel with all variants inside was
 // five times longer and spent a quarter of its time fetching instructions.
 template <int MODE, int KIND, bool VEC>
 __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
-  constexpr bool kPost = KIND == 0 || KIND == 3;  // the epilogue with post operations
+  constexpr bool kPost = KIND == 0 || KIND == 3 || KIND == 5;  // the epilogue with post operations
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ __attribute__((aligned(16))) int s_acc0[kCtBN];
   __shared__ __attribute__((aligned(16))) float s_mult[kCtBN];
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(kCtThreads) void conv_tile_kernel(ConvTileArgs a) {
               for (int j = 0; j < 4; ++j) raw[j] = acc[tn][tm][4 * gq + j];
               uint32_t q4;
               if constexpr (kPost)
-                q4 = requant4_post<MODE, KIND == 0 ? 1 : 2>(raw, bdiv, bmul, mult, a.post, accw[tm][tn * 4 + gq],
+                q4 = requant4_post<MODE, KIND == 3 ? 2 : 1, KIND == 5>(raw, bdiv, bmul, mult, a.post, accw[tm][tn * 4 + gq],
                                                             a.zp_f, a.lo_f, a.hi_f);
               else
                 q4 = requant4<MODE, KIND == 1, KIND == 4 ? 1 : 0>(raw, bdiv, bmul, mult, a.zp_f, a.lo_f, a.hi_f);

@@ -401,13 +401,14 @@ __device__ __forceinline__ uint32_t load_accum4(const PostOps& p, int64_t off, i
 
 // requant4 with the post operations (see PostOps) before the rounding.  POST says
 // what the caller knows at compile time: 0 nothing (both operations are looked up
-// in `p`), 1 a residual and no SiLU, 2 SiLU (a residual if `p` has one).
-template <int MODE, int POST = 0>
+// in `p`), 1 a residual and no SiLU, 2 SiLU (a residual if `p` has one).  PLAIN: as in requant4.
+template <int MODE, int POST = 0, bool PLAIN = false>
 __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv, float bmul, v4f mult,
                                                   const PostOps& p, uint32_t accw, float zp_f,
                                                   float lo_f, float hi_f) {
   if constexpr (MODE == kOutS8)  // (see requant4)
-    return requant4_post<kOutU8, POST>(raw, bdiv, bmul, mult, p, accw, zp_f + 128.f, lo_f + 128.f, hi_f + 128.f) ^
+    return requant4_post<kOutU8, POST, PLAIN>(raw, bdiv, bmul, mult, p, accw, zp_f + 128.f, lo_f + 128.f,
+                                              hi_f + 128.f) ^
            0x80808080u;
   uint32_t packed = 0;
   // The residual bytes are taken as unsigned values (one conversion instruction
@@ -427,6 +428,10 @@ __device__ __forceinline__ uint32_t requant4_post(const int (&raw)[4], v4f bdiv,
       t = t + a;
     }
     if (POST == 2 || (POST == 0 && p.silu)) t = silu_in_output_units(t, p.silu_c, p.silu_c_tail);
+    if constexpr (PLAIN && MODE == kOutU8) {  // (the host has checked requant_plain_u8: see requant4)
+      packed = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed);
+      continue;
+    }
     float r = __builtin_rintf(t) + zp_f;
     r = __builtin_amdgcn_fmed3f(r, lo_f, hi_f);
     if constexpr (MODE == kOutU8) {
